@@ -1,0 +1,344 @@
+"""Whole-model oracle: the operator namespace of ``folx_amd.numpy`` on numpy arrays with
+dense Jacobians (test infrastructure; also the CPU baseline timed by ``bench.py``).
+
+A model written against the namespace (``xp.dot``, ``xp.tanh``, ``xp.slogdet`` ...) runs
+unchanged on this backend.  Values are ``OArr`` triplets in the package layout
+``x (B, *s)``, ``J (P, B, *s)``, ``lap (B, *s)``; walker-varying constants are ``OConst``
+(data ``(B, *s)``); walker-invariant constants are plain numpy arrays / scalars of the
+logical shape ``s``.  Every op applies the rule from ``oracle.rules``.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+from . import rules
+
+
+class OConst:
+    """A constant that differs per walker: data (B, *s)."""
+
+    def __init__(self, data):
+        self.data = np.asarray(data)
+
+    @property
+    def shape(self):
+        return self.data.shape[1:]
+
+
+class OArr:
+    def __init__(self, x, J, lap):
+        self.x, self.J, self.lap = x, J, lap
+
+    @property
+    def shape(self):
+        return self.x.shape[1:]
+
+    @property
+    def ndim(self):
+        return self.x.ndim - 1
+
+    @property
+    def B(self):
+        return self.x.shape[0]
+
+    @property
+    def P(self):
+        return self.J.shape[0]
+
+    # operator sugar -----------------------------------------------------------------
+    def __add__(self, o):
+        return add(self, o)
+
+    __radd__ = __add__
+
+    def __sub__(self, o):
+        return subtract(self, o)
+
+    def __rsub__(self, o):
+        return subtract(o, self)
+
+    def __mul__(self, o):
+        return multiply(self, o)
+
+    __rmul__ = __mul__
+
+    def __truediv__(self, o):
+        return divide(self, o)
+
+    def __neg__(self):
+        return negative(self)
+
+    def __getitem__(self, idx):
+        return getitem(self, idx)
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        return reshape(self, shape)
+
+    def sum(self, axis=None, keepdims=False):
+        return sum(self, axis, keepdims)
+
+
+def init_state(x, weights=None, dtype=None) -> OArr:
+    """x (B, *s) -> J = identity rows (folx/interpreter.py:295), lap = 0 (:297)."""
+    x = np.asarray(x, dtype=dtype)
+    B = x.shape[0]
+    n = int(np.prod(x.shape[1:], dtype=int))
+    eye = np.eye(n, dtype=x.dtype)
+    if weights is not None:
+        eye = eye * np.broadcast_to(np.asarray(weights, dtype=x.dtype), x.shape[1:]).reshape(-1)
+    J = np.broadcast_to(eye.reshape(n, 1, *x.shape[1:]), (n, B, *x.shape[1:])).copy()
+    return OArr(x, J, np.zeros_like(x))
+
+
+def _is(a):
+    return isinstance(a, OArr)
+
+
+def _const(c, like: OArr):
+    """Constant as (array (B or 1, *s_c), logical ndim)."""
+    dt = like.x.dtype
+    if isinstance(c, OConst):
+        d = c.data.astype(dt)
+        return d, d.ndim - 1
+    c = np.asarray(c, dtype=dt)
+    return c[None], c.ndim
+
+
+def _pad(t: OArr, nd: int) -> OArr:
+    """Prepend size-1 logical axes so the triplet has ``nd`` logical dims."""
+    ex = nd - t.ndim
+    if ex <= 0:
+        return t
+    B, P = t.B, t.P
+    one = [1] * ex
+    return OArr(
+        t.x.reshape(B, *one, *t.shape),
+        t.J.reshape(P, B, *one, *t.shape),
+        t.lap.reshape(B, *one, *t.shape),
+    )
+
+
+def _padJ(a: OArr, b: OArr):
+    """Dense Jacobians of different row counts are zero-extended (folx/utils.py:432-450)."""
+    P = max(a.P, b.P)
+
+    def ext(J):
+        if J.shape[0] == P:
+            return J
+        z = np.zeros((P - J.shape[0], *J.shape[1:]), dtype=J.dtype)
+        return np.concatenate([J, z], 0)
+
+    return ext(a.J), ext(b.J)
+
+
+def _bcast3(a: OArr, b: OArr):
+    nd = max(a.ndim, b.ndim)
+    a, b = _pad(a, nd), _pad(b, nd)
+    Ja, Jb = _padJ(a, b)
+    xa, xb = np.broadcast_arrays(a.x, b.x)
+    Ja, Jb = np.broadcast_arrays(Ja, Jb)
+    La, Lb = np.broadcast_arrays(a.lap, b.lap)
+    return (xa, Ja, La), (xb, Jb, Lb)
+
+
+def _with_const(a: OArr, c):
+    """Align a triplet and a constant: returns (padded triplet, constant (B|1, *s))."""
+    c, cn = _const(c, a)
+    nd = max(a.ndim, cn)
+    a = _pad(a, nd)
+    c = c.reshape(c.shape[0], *([1] * (nd - cn)), *c.shape[1:])
+    return a, c
+
+
+def add(a, b, sign=1.0):
+    if _is(a) and _is(b):
+        ta, tb = _bcast3(a, b)
+        return OArr(*rules.add_rule(*ta, *tb, sign=sign))
+    if _is(a):
+        a, c = _with_const(a, b)
+        x = a.x + sign * c
+        return OArr(
+            x,
+            np.broadcast_to(a.J, (a.P, *x.shape)).copy(),
+            np.broadcast_to(a.lap, x.shape).copy(),
+        )
+    # constant +- triplet
+    return add(multiply(b, sign), a, 1.0)
+
+
+def subtract(a, b):
+    return add(a, b, sign=-1.0)
+
+
+def multiply(a, b):
+    if _is(a) and _is(b):
+        ta, tb = _bcast3(a, b)
+        return OArr(*rules.mul_rule(*ta, *tb))
+    if _is(b):
+        a, b = b, a
+    a, c = _with_const(a, b)
+    return OArr(a.x * c, a.J * c[None], a.lap * c)
+
+
+def divide(a, b):
+    if _is(a) and _is(b):
+        ta, tb = _bcast3(a, b)
+        return OArr(*rules.div_rule(*ta, *tb))
+    if _is(a):
+        if isinstance(b, OConst):
+            return multiply(a, OConst(1.0 / b.data))
+        return multiply(a, 1.0 / np.asarray(b, dtype=a.x.dtype))
+    return multiply(reciprocal(b), a)
+
+
+def _unary(name, param=None):
+    def fn(a):
+        if not _is(a):
+            raise TypeError('oracle unary ops take triplets')
+        return OArr(*rules.elementwise_rule(name, a.x, a.J, a.lap, param))
+
+    fn.__name__ = name
+    return fn
+
+
+tanh = _unary('tanh')
+silu = _unary('silu')
+exp = _unary('exp')
+log = _unary('log')
+sqrt = _unary('sqrt')
+rsqrt = _unary('rsqrt')
+square = _unary('square')
+sigmoid = _unary('logistic')
+logistic = sigmoid
+softplus = _unary('softplus')
+sin = _unary('sin')
+cos = _unary('cos')
+abs = _unary('abs')
+negative = _unary('neg')
+log1p = _unary('log1p')
+reciprocal = _unary('reciprocal')
+expm1 = _unary('expm1')
+
+
+def integer_pow(a, n):
+    return OArr(*rules.elementwise_rule('integer_pow', a.x, a.J, a.lap, n))
+
+
+def dot(h: OArr, W, b=None):
+    W = np.asarray(W, dtype=h.x.dtype)
+    bb = None if b is None else np.asarray(b, dtype=h.x.dtype)
+    return OArr(*rules.dense_rule(h.x, h.J, h.lap, W, bb))
+
+
+def sum(a: OArr, axis=None, keepdims=False):
+    if axis is None:
+        axis = tuple(range(a.ndim))
+    return OArr(*rules.sum_rule(a.x, a.J, a.lap, axis, keepdims))
+
+
+def mean(a: OArr, axis=None, keepdims=False):
+    if axis is None:
+        axis = tuple(range(a.ndim))
+    n = int(np.prod([a.shape[i] for i in np.atleast_1d(axis)]))
+    return multiply(sum(a, axis, keepdims), 1.0 / n)
+
+
+def reshape(a: OArr, shape):
+    shape = tuple(shape)
+    return OArr(
+        a.x.reshape(a.B, *shape), a.J.reshape(a.P, a.B, *shape), a.lap.reshape(a.B, *shape)
+    )
+
+
+def transpose(a: OArr, axes):
+    axes = tuple(ax % a.ndim for ax in axes)
+    xa = (0, *[ax + 1 for ax in axes])
+    ja = (0, 1, *[ax + 2 for ax in axes])
+    return OArr(a.x.transpose(xa), a.J.transpose(ja), a.lap.transpose(xa))
+
+
+def swapaxes(a: OArr, i, j):
+    axes = list(range(a.ndim))
+    axes[i], axes[j] = axes[j], axes[i]
+    return transpose(a, axes)
+
+
+def expand_dims(a: OArr, axis):
+    axis = axis % (a.ndim + 1)
+    return OArr(
+        np.expand_dims(a.x, axis + 1), np.expand_dims(a.J, axis + 2), np.expand_dims(a.lap, axis + 1)
+    )
+
+
+def broadcast_to(a: OArr, shape):
+    shape = tuple(shape)
+    ex = len(shape) - a.ndim
+    x = a.x.reshape(a.B, *([1] * ex), *a.shape)
+    J = a.J.reshape(a.P, a.B, *([1] * ex), *a.shape)
+    L = a.lap.reshape(a.B, *([1] * ex), *a.shape)
+    return OArr(
+        np.broadcast_to(x, (a.B, *shape)).copy(),
+        np.broadcast_to(J, (a.P, a.B, *shape)).copy(),
+        np.broadcast_to(L, (a.B, *shape)).copy(),
+    )
+
+
+def getitem(a: OArr, idx):
+    if not isinstance(idx, tuple):
+        idx = (idx,)
+    return OArr(
+        a.x[(slice(None), *idx)], a.J[(slice(None), slice(None), *idx)], a.lap[(slice(None), *idx)]
+    )
+
+
+def concatenate(arrs, axis=-1):
+    first = [t for t in arrs if _is(t)][0]
+    nd = first.ndim
+    axis = axis % nd
+    P = max(t.P for t in arrs if _is(t))
+    xs, Js, Ls = [], [], []
+    for t in arrs:
+        if _is(t):
+            J = t.J
+            if J.shape[0] < P:
+                J = np.concatenate([J, np.zeros((P - J.shape[0], *J.shape[1:]), J.dtype)], 0)
+            xs.append(t.x), Js.append(J), Ls.append(t.lap)
+        else:
+            c = np.asarray(t, dtype=first.x.dtype)
+            c = np.broadcast_to(c[None], (first.B, *c.shape))
+            xs.append(c)
+            Js.append(np.zeros((P, *c.shape), c.dtype))
+            Ls.append(np.zeros_like(c))
+    return OArr(
+        np.concatenate(xs, axis + 1), np.concatenate(Js, axis + 2), np.concatenate(Ls, axis + 1)
+    )
+
+
+def stop_gradient(a):
+    return OConst(a.x) if _is(a) else a
+
+
+def amax_const(a, axis, keepdims=False):
+    """max over ``axis`` of the values only, as a walker-varying constant."""
+    x = a.x if _is(a) else a.data
+    ax = tuple(i % (x.ndim - 1) + 1 for i in np.atleast_1d(axis))
+    return OConst(x.max(ax, keepdims=keepdims))
+
+
+def slogdet(A: OArr):
+    sign, (ld, J, L) = rules.slogdet_rule(A.x, A.J, A.lap)
+    return OConst(sign), OArr(ld, J, L)
+
+
+def multi_head_self_attention(q: OArr, k: OArr, v: OArr, mask=None, input_mask=None):
+    o, oJ, oL = rules.mhsa_rule(
+        q.x, q.J, q.lap, k.x, k.J, k.lap, v.x, v.J, v.lap, mask, input_mask
+    )
+    return OArr(o, oJ, oL)
+
+
+def to_numpy(a):
+    return a

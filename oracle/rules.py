@@ -1,0 +1,326 @@
+"""Numpy restatement of the forward-Laplacian propagation rules (test infrastructure).
+
+Every rule maps input triplets ``(x, J, lap)`` to the output triplet following
+
+    y     = f(x)
+    J_y   = J_f . J                              (folx/jvp.py:676-711)
+    lap_y = J_f . lap + tr(J^T H_f J)            (folx/wrapper.py:120-125)
+
+Arrays use the layout ``x (B, *s)``, ``J (P, B, *s)``, ``lap (B, *s)``.  All functions
+work in the dtype of their inputs (float64 for pinning, float32 for the CPU baseline).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# --------------------------------------------------------------------------------------
+# Elementwise activations: (f, f', f'') in closed form.
+# Reference: f'(x) comes from a vjp with ones (folx/jvp.py:687-697, :262-272), f''(x)
+# from jvp-of-jvp (folx/hessian.py:87-112); the closed forms below are what those AD
+# calls evaluate to for each registered primitive (folx/wrapped_functions.py:385-415,
+# :552-560, :622-625).
+# --------------------------------------------------------------------------------------
+
+
+def _sigmoid(x):
+    # numerically stable logistic
+    out = np.empty_like(x)
+    pos = x >= 0
+    out[pos] = 1.0 / (1.0 + np.exp(-x[pos]))
+    e = np.exp(x[~pos])
+    out[~pos] = e / (1.0 + e)
+    return out
+
+
+def _tanh(x):
+    t = np.tanh(x)
+    return t, 1 - t * t, -2 * t * (1 - t * t)
+
+
+def _silu(x):
+    s = _sigmoid(x)
+    return x * s, s * (1 + x * (1 - s)), s * (1 - s) * (2 + x * (1 - 2 * s))
+
+
+def _exp(x):
+    e = np.exp(x)
+    return e, e, e
+
+
+def _log(x):
+    return np.log(x), 1 / x, -1 / (x * x)
+
+
+def _sqrt(x):
+    r = np.sqrt(x)
+    return r, 0.5 / r, -0.25 / (r * x)
+
+
+def _rsqrt(x):
+    r = 1 / np.sqrt(x)
+    return r, -0.5 * r / x, 0.75 * r / (x * x)
+
+
+def _square(x):
+    return x * x, 2 * x, np.full_like(x, 2.0)
+
+
+def _logistic(x):
+    s = _sigmoid(x)
+    return s, s * (1 - s), s * (1 - s) * (1 - 2 * s)
+
+
+def _softplus(x):
+    s = _sigmoid(x)
+    return np.logaddexp(x, 0), s, s * (1 - s)
+
+
+def _sin(x):
+    return np.sin(x), np.cos(x), -np.sin(x)
+
+
+def _cos(x):
+    return np.cos(x), -np.sin(x), -np.cos(x)
+
+
+def _abs(x):
+    # registered LINEAR (folx/wrapped_functions.py:349-352): no Hessian term
+    return np.abs(x), np.sign(x), np.zeros_like(x)
+
+
+def _neg(x):
+    return -x, np.full_like(x, -1.0), np.zeros_like(x)
+
+
+def _log1p(x):
+    return np.log1p(x), 1 / (1 + x), -1 / ((1 + x) * (1 + x))
+
+
+def _reciprocal(x):
+    r = 1 / x
+    return r, -r * r, 2 * r * r * r
+
+
+def _expm1(x):
+    e = np.exp(x)
+    return np.expm1(x), e, e
+
+
+def _identity(x):
+    return x, np.ones_like(x), np.zeros_like(x)
+
+
+ACTIVATIONS = {
+    'tanh': _tanh,
+    'silu': _silu,
+    'exp': _exp,
+    'log': _log,
+    'sqrt': _sqrt,
+    'rsqrt': _rsqrt,
+    'square': _square,
+    'logistic': _logistic,
+    'sigmoid': _logistic,
+    'softplus': _softplus,
+    'sin': _sin,
+    'cos': _cos,
+    'abs': _abs,
+    'neg': _neg,
+    'log1p': _log1p,
+    'reciprocal': _reciprocal,
+    'expm1': _expm1,
+    'identity': _identity,
+}
+
+
+def integer_pow(x, n: int):
+    """``lax.integer_pow`` closed forms (folx/wrapped_functions.py:385)."""
+    return x**n, n * x ** (n - 1), n * (n - 1) * x ** (n - 2)
+
+
+def elementwise_rule(name, x, J, lap, param=None):
+    """y = f(x); J_y = f'(x) * J; lap_y = f'(x) * lap + f''(x) * sum_p J_p^2.
+
+    folx/jvp.py:687-697 (dense), folx/jvp.py:262-272 (sparse rows, mask unchanged),
+    folx/hessian.py:87-112 (sum over the Jacobian axis of J*J, valid for sparse storage
+    when no index repeats per position), combined at folx/wrapper.py:120-125.
+    """
+    if name == 'integer_pow':
+        y, d1, d2 = integer_pow(x, int(param))
+    elif name == 'scale':  # y = param * x, linear
+        y, d1, d2 = param * x, np.full_like(x, param), np.zeros_like(x)
+    else:
+        y, d1, d2 = ACTIVATIONS[name](x)
+    Jy = d1[None] * J
+    lapy = d1 * lap + d2 * (J * J).sum(0)
+    return y, Jy, lapy
+
+
+# --------------------------------------------------------------------------------------
+# Dense layer: one operand carries derivatives, the other is constant.
+# --------------------------------------------------------------------------------------
+
+
+def dense_rule(x, J, lap, W, b=None):
+    """y = x @ W (+ b) along the last axis; the op is linear so the same product is
+    applied to x, to every Jacobian row and to the Laplacian
+    (folx/wrapped_functions.py:167-169).  A constant bias shifts x only
+    (``add`` is LINEAR, folx/wrapped_functions.py:365-367)."""
+    y = x @ W
+    if b is not None:
+        y = y + b
+    return y, J @ W, lap @ W
+
+
+# --------------------------------------------------------------------------------------
+# Binary elementwise rules with both operands carrying derivatives (dense Jacobians).
+# --------------------------------------------------------------------------------------
+
+
+def _bc(*arrs):
+    return np.broadcast_arrays(*arrs)
+
+
+def mul_rule(a, Ja, La, b, Jb, Lb):
+    """y = a * b.  JVP by linearity in each argument (folx/jvp.py:676-684); the Hessian
+    is the off-diagonal identity so tr(J^T H J) = 2 sum_p Ja_p * Jb_p
+    (folx/hessian.py:177-188, MULTIPLICATION flag folx/wrapped_functions.py:377-379)."""
+    y = a * b
+    Jy = a[None] * Jb + b[None] * Ja
+    lap = a * Lb + b * La + 2 * (Ja * Jb).sum(0)
+    return y, Jy, lap
+
+
+def div_rule(a, Ja, La, b, Jb, Lb):
+    """y = a / b with the custom Hessian of folx/custom_hessian.py:35-59:
+    H_lr = -2 / b^2 (counted once for the symmetric pair), H_rr = 2 a / b^3."""
+    y = a / b
+    rb2 = 1 / (b * b)
+    Jy = Ja / b[None] - (a * rb2)[None] * Jb
+    lap = La / b - a * rb2 * Lb
+    lap = lap + (-2 * rb2) * (Ja * Jb).sum(0) + (2 * a * rb2 / b) * (Jb * Jb).sum(0)
+    return y, Jy, lap
+
+
+def add_rule(a, Ja, La, b, Jb, Lb, sign=1.0):
+    """y = a +- b (LINEAR, folx/wrapped_functions.py:365-370)."""
+    return a + sign * b, Ja + sign * Jb, La + sign * Lb
+
+
+def sum_rule(x, J, lap, axes, keepdims=False):
+    """reduce_sum is linear (SUMMATION flag, folx/wrapped_functions.py:388-392): the same
+    reduction is applied to x, J rows and lap (folx/jvp.py:104-106)."""
+    ax = tuple(a % (x.ndim - 1) for a in np.atleast_1d(axes))
+    xa = tuple(a + 1 for a in ax)
+    ja = tuple(a + 2 for a in ax)
+    return (
+        x.sum(xa, keepdims=keepdims),
+        J.sum(ja, keepdims=keepdims),
+        lap.sum(xa, keepdims=keepdims),
+    )
+
+
+# --------------------------------------------------------------------------------------
+# slogdet
+# --------------------------------------------------------------------------------------
+
+
+def slogdet_rule(A, J, lap):
+    """Forward Laplacian of ``log|det A|`` from the dense Jacobian
+    (folx/slogdet.py:296-317):
+
+        M_c = A^-1 dA/dx_c,  d_c log|det A| = tr M_c,
+        lap = tr(A^-1 lap_A) - sum_c tr(M_c M_c).
+
+    A: (B, ..., n, n); J: (P, B, ..., n, n); lap: (B, ..., n, n).
+    Returns sign (plain array), (logdet, J_logdet, lap_logdet).
+    """
+    sign, logdet = np.linalg.slogdet(A)
+    Ainv = np.linalg.inv(A)
+    M = np.einsum('...ij,p...jd->p...id', Ainv, J)
+    jac = np.einsum('p...ii->p...', M)
+    lap_out = np.einsum('...ji,...ij->...', Ainv, lap) - np.einsum(
+        'p...id,p...di->...', M, M
+    )
+    return sign.astype(A.dtype), (logdet.astype(A.dtype), jac, lap_out)
+
+
+# --------------------------------------------------------------------------------------
+# Multi-head self attention
+# --------------------------------------------------------------------------------------
+
+
+def big_number(dtype) -> float:
+    """Mask fill value (folx/experimental/pallas/attention/utils.py:210-220)."""
+    return 1e40 if np.dtype(dtype) == np.float64 else 1e20
+
+
+def mhsa_forward(q, k, v, mask=None):
+    """softmax(q k^T) v with padded-sequence masking and no 1/sqrt(d) inside
+    (folx/experimental/pallas/attention/mhsa.py:79-94).  q, k, v: (B, n, H, d)."""
+    B, n, H, d = q.shape
+    if mask is None:
+        mask = np.ones((B, n), dtype=bool)
+    sq = mask[:, :, None, None] & mask[:, None, None, :]
+    s = np.einsum('bihd,bjhd->bihj', q, k)
+    s = np.where(sq, s, -big_number(s.dtype))
+    s = s - s.max(-1, keepdims=True)
+    e = np.exp(s)
+    p = e / e.sum(-1, keepdims=True)
+    return np.einsum('bihj,bjhd->bihd', p, v), p
+
+
+def mhsa_rule(q, qJ, qL, k, kJ, kL, v, vJ, vL, mask=None, input_mask=None):
+    """Forward Laplacian of masked multi-head self attention.
+
+    Specification: folx/experimental/pallas/attention/forward_laplacian.py:212-346 (einsum
+    form) and :349-487 (kernel form); the algebra below is the factored form the same
+    file uses for the edge-bias variant (:663-704) with the edge term removed:
+
+        s'_c = q'_c k^T + q k'_c^T          p'_c = p * (s'_c - rowsum(p * s'_c))
+        o'_c = p v'_c + p'_c v
+        lap_o = [same with the Laplacians in place of the c-derivatives]
+              + ( sum_c p'_c * (s'_c - rowsum(p s'_c))
+                  + p * (S - sum_c rowsum(p'_c s'_c) - rowsum(p S)) ) v
+              + 2 sum_c p'_c v'_c,           S = 2 sum_c q'_c k'_c^T
+
+    Masking (:231-241): Jacobian rows are zeroed where the coordinate is inactive
+    (``input_mask[p, b]`` False) or the electron is padding (``mask[b, i]`` False);
+    Laplacians are zeroed for padding electrons; scores of padded pairs are set to
+    ``-big_number`` before the softmax.  Rows of padding queries carry no meaning (the
+    reference's tests mask them out before comparing, test_attention.py:80-100).
+
+    Shapes: q/k/v (B, n, H, d); *J (P, B, n, H, d); *L (B, n, H, d);
+    mask (B, n) bool; input_mask (P, B) bool.
+    """
+    B, n, H, d = q.shape
+    P = qJ.shape[0]
+    if mask is None:
+        mask = np.ones((B, n), dtype=bool)
+    if input_mask is None:
+        input_mask = np.ones((P, B), dtype=bool)
+    mask = mask.astype(bool)
+    input_mask = input_mask.astype(bool)
+    cm = input_mask[:, :, None, None, None] & mask[None, :, :, None, None]
+    em = mask[:, :, None, None]
+    qJ, kJ, vJ = (np.where(cm, a, 0.0) for a in (qJ, kJ, vJ))
+    qL, kL, vL = (np.where(em, a, 0.0) for a in (qL, kL, vL))
+
+    o, p = mhsa_forward(q, k, v, mask)
+
+    sJ = np.einsum('pbihd,bjhd->pbihj', qJ, k) + np.einsum('bihd,pbjhd->pbihj', q, kJ)
+    rJ = (p[None] * sJ).sum(-1, keepdims=True)
+    pJ = p[None] * (sJ - rJ)
+    oJ = np.einsum('bihj,pbjhd->pbihd', p, vJ) + np.einsum('pbihj,bjhd->pbihd', pJ, v)
+
+    sL = np.einsum('bihd,bjhd->bihj', qL, k) + np.einsum('bihd,bjhd->bihj', q, kL)
+    pL = p * (sL - (p * sL).sum(-1, keepdims=True))
+    oL = np.einsum('bihj,bjhd->bihd', p, vL) + np.einsum('bihj,bjhd->bihd', pL, v)
+
+    S = 2 * np.einsum('pbihd,pbjhd->bihj', qJ, kJ)
+    pI = (pJ * (sJ - rJ)).sum(0) + p * (
+        S - (pJ * sJ).sum((0, -1))[..., None] - (p * S).sum(-1, keepdims=True)
+    )
+    oL = oL + np.einsum('bihj,bjhd->bihd', pI, v)
+    oL = oL + 2 * np.einsum('pbihj,pbjhd->bihd', pJ, vJ)
+    return o, oJ, oL

@@ -1,0 +1,172 @@
+"""Brute-force fp64 oracle: value, Jacobian and trace of the Hessian by torch autograd.
+
+Same method as the reference's own test base class (test/laplacian_testcase.py:22-49:
+Jacobian by AD, Laplacian as the trace of the full AD Hessian in float64).  A model
+written against the operator namespace runs here on plain fp64 torch tensors of ONE
+walker; ``brute_force`` loops over walkers.
+"""
+
+import math
+
+import numpy as np
+import torch
+
+
+class plain:
+    """Operator namespace on plain torch tensors (single walker, no derivatives)."""
+
+    float64 = torch.float64
+
+    @staticmethod
+    def _c(c, like):
+        if isinstance(c, torch.Tensor):
+            return c.to(like.dtype)
+        return torch.as_tensor(np.asarray(c), dtype=like.dtype)
+
+    @staticmethod
+    def dot(h, W, b=None):
+        y = h @ plain._c(W, h)
+        return y if b is None else y + plain._c(b, h)
+
+    tanh = staticmethod(torch.tanh)
+    exp = staticmethod(torch.exp)
+    log = staticmethod(torch.log)
+    sqrt = staticmethod(torch.sqrt)
+    rsqrt = staticmethod(torch.rsqrt)
+    square = staticmethod(torch.square)
+    sigmoid = staticmethod(torch.sigmoid)
+    logistic = staticmethod(torch.sigmoid)
+    softplus = staticmethod(torch.nn.functional.softplus)
+    silu = staticmethod(torch.nn.functional.silu)
+    sin = staticmethod(torch.sin)
+    cos = staticmethod(torch.cos)
+    abs = staticmethod(torch.abs)
+    negative = staticmethod(torch.neg)
+    log1p = staticmethod(torch.log1p)
+    reciprocal = staticmethod(torch.reciprocal)
+    expm1 = staticmethod(torch.expm1)
+
+    @staticmethod
+    def integer_pow(a, n):
+        return a**n
+
+    @staticmethod
+    def _b(a, b):
+        if isinstance(a, torch.Tensor) and not isinstance(b, torch.Tensor):
+            b = plain._c(b, a)
+        elif isinstance(b, torch.Tensor) and not isinstance(a, torch.Tensor):
+            a = plain._c(a, b)
+        return a, b
+
+    @staticmethod
+    def add(a, b):
+        a, b = plain._b(a, b)
+        return a + b
+
+    @staticmethod
+    def subtract(a, b):
+        a, b = plain._b(a, b)
+        return a - b
+
+    @staticmethod
+    def multiply(a, b):
+        a, b = plain._b(a, b)
+        return a * b
+
+    @staticmethod
+    def divide(a, b):
+        a, b = plain._b(a, b)
+        return a / b
+
+    @staticmethod
+    def sum(a, axis=None, keepdims=False):
+        if axis is None:
+            return a.sum()
+        return a.sum(dim=axis, keepdim=keepdims)
+
+    @staticmethod
+    def mean(a, axis=None, keepdims=False):
+        if axis is None:
+            return a.mean()
+        return a.mean(dim=axis, keepdim=keepdims)
+
+    @staticmethod
+    def reshape(a, shape):
+        return a.reshape(tuple(shape))
+
+    @staticmethod
+    def transpose(a, axes):
+        return a.permute(tuple(axes))
+
+    @staticmethod
+    def swapaxes(a, i, j):
+        return a.transpose(i, j)
+
+    @staticmethod
+    def expand_dims(a, axis):
+        return a.unsqueeze(axis)
+
+    @staticmethod
+    def broadcast_to(a, shape):
+        return a.expand(tuple(shape))
+
+    @staticmethod
+    def getitem(a, idx):
+        return a[idx]
+
+    @staticmethod
+    def concatenate(arrs, axis=-1):
+        like = [t for t in arrs if isinstance(t, torch.Tensor)][0]
+        return torch.cat([plain._c(t, like) for t in arrs], dim=axis)
+
+    @staticmethod
+    def stop_gradient(a):
+        return a.detach()
+
+    @staticmethod
+    def amax_const(a, axis, keepdims=False):
+        return a.detach().amax(dim=axis, keepdim=keepdims)
+
+    @staticmethod
+    def slogdet(A):
+        sign, ld = torch.linalg.slogdet(A)
+        return sign.detach(), ld
+
+    @staticmethod
+    def multi_head_self_attention(q, k, v, mask=None, input_mask=None):
+        # q, k, v: (n, H, d); softmax(q k^T) v, no 1/sqrt(d) inside
+        s = torch.einsum('ihd,jhd->ihj', q, k)
+        if mask is not None:
+            m = torch.as_tensor(np.asarray(mask), dtype=torch.bool)
+            sq = m[:, None, None] & m[None, None, :]
+            s = torch.where(sq, s, torch.full_like(s, -1e40))
+        p = torch.softmax(s, dim=-1)
+        return torch.einsum('ihj,jhd->ihd', p, v)
+
+
+def brute_force_single(fn, x):
+    """fn: tensor (s) -> tensor (out).  Returns (y, J (n_in, *out), lap (*out)) in fp64."""
+    x = torch.as_tensor(np.asarray(x), dtype=torch.float64)
+    flat = x.reshape(-1)
+
+    def f(z):
+        return fn(z.reshape(x.shape))
+
+    y = f(flat)
+    J = torch.func.jacrev(f)(flat)  # (*out, n)
+    # forward-over-reverse: torch's forward-over-forward through linalg.det / slogdet
+    # returns wrong second derivatives (checked against an explicit cofactor expansion in
+    # tests/test_oracle_rules.py), so the Hessian is never taken that way here.
+    H = torch.func.jacfwd(torch.func.jacrev(f))(flat)  # (*out, n, n)
+    lap = torch.diagonal(H, dim1=-2, dim2=-1).sum(-1)
+    J = torch.movedim(J, -1, 0)
+    return y.detach().numpy(), J.detach().numpy(), lap.detach().numpy()
+
+
+def brute_force(fn, x):
+    """x: (B, *s) numpy.  Returns x (B, *out), J (n_in, B, *out), lap (B, *out)."""
+    ys, Js, Ls = [], [], []
+    for b in range(x.shape[0]):
+        y, J, L = brute_force_single(fn, x[b])
+        ys.append(y), Js.append(J), Ls.append(L)
+    return np.stack(ys, 0), np.stack(Js, 1), np.stack(Ls, 0)

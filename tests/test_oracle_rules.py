@@ -1,0 +1,253 @@
+"""Pins oracle.rules against checks that do not retype its formulas: torch fp64 autograd
+(jvp-of-jvp for activations, full Hessian traces for the composite rules), numpy.linalg
+closed forms for slogdet, and the masked-attention cases of the reference's own test
+(test/experimental/pallas/test_attention.py:320-326)."""
+
+import numpy as np
+import pytest
+import torch
+
+from bruteforce import brute_force, plain
+from oracle import backend as ob
+from oracle import rules
+
+RTOL, ATOL = 2e-5, 1e-10  # the reference's own bar (test/laplacian_testcase.py:16-20)
+
+
+def _close(a, b, rtol=RTOL, atol=ATOL):
+    np.testing.assert_allclose(a, b, rtol=rtol, atol=atol)
+
+
+POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal'}
+
+
+@pytest.mark.parametrize('name', sorted(rules.ACTIVATIONS))
+def test_activation_closed_forms_vs_autograd(name):
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=64) * 2
+    if name in POSITIVE:
+        x = np.abs(x) + 0.1
+    tname = {'neg': 'negative', 'identity': None}.get(name, name)
+    f = (lambda t: t) if tname is None else getattr(plain, tname)
+    xt = torch.tensor(x, dtype=torch.float64)
+    ones = torch.ones_like(xt)
+    df = lambda t: torch.func.jvp(f, (t,), (ones,))[1]
+    d1 = df(xt)
+    d2 = torch.func.jvp(df, (xt,), (ones,))[1]
+    y, g1, g2 = rules.ACTIVATIONS[name](x)
+    _close(y, f(xt).numpy())
+    _close(g1, d1.numpy())
+    _close(g2, d2.numpy(), atol=1e-9)
+
+
+def test_integer_pow():
+    x = np.linspace(0.5, 2, 7)
+    for n in (2, 3, -1, -2):
+        y, d1, d2 = rules.integer_pow(x, n)
+        _close(y, x**n)
+        _close(d1, n * x ** (n - 1))
+        _close(d2, n * (n - 1) * x ** (n - 2))
+
+
+def _run_oracle(fn, x):
+    out = fn(ob, ob.init_state(x, dtype=np.float64))
+    return out.x, out.J, out.lap
+
+
+def _check(fn, x, rtol=RTOL, atol=1e-9):
+    y, J, L = _run_oracle(fn, x)
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x)
+    _close(y, by, rtol, atol)
+    _close(J, bJ, rtol, atol)
+    _close(L, bL, rtol, atol)
+
+
+def test_mlp_vs_bruteforce():
+    # same structure as test/test_composite.py:13-43 (tanh MLP, summed)
+    rng = np.random.default_rng(1)
+    Ws = [(rng.normal(size=(12, 12)) / 3, rng.normal(size=12)) for _ in range(3)]
+
+    def mlp(xp, x):
+        for W, b in Ws:
+            x = xp.tanh(xp.dot(x, W, b))
+        return xp.sum(x)
+
+    _check(mlp, rng.normal(size=(3, 12)))
+
+
+def test_silu_mlp_nodewise_vs_bruteforce():
+    # README example shape in miniature: nodes pass through the MLP independently
+    rng = np.random.default_rng(2)
+    Ws = [rng.normal(size=(4, 6)) / 2, rng.normal(size=(6, 6)) / 2, rng.normal(size=(6, 1))]
+
+    def f(xp, x):
+        for W in Ws[:-1]:
+            x = xp.silu(xp.dot(x, W))
+        return xp.sum(xp.dot(x, Ws[-1]))
+
+    _check(f, rng.normal(size=(2, 5, 4)))
+
+
+@pytest.mark.parametrize('op', ['multiply', 'divide', 'add', 'subtract'])
+def test_binary_rules_vs_bruteforce(op):
+    rng = np.random.default_rng(3)
+    W1, W2 = rng.normal(size=(6, 5)), rng.normal(size=(6, 5))
+
+    def f(xp, x):
+        a = xp.tanh(xp.dot(x, W1))
+        b = xp.add(xp.exp(xp.dot(x, W2) * 0.3 if xp is plain else xp.multiply(xp.dot(x, W2), 0.3)), 0.5)
+        return getattr(xp, op)(a, b)
+
+    _check(f, rng.normal(size=(2, 6)))
+
+
+def test_binary_broadcast_and_reductions_vs_bruteforce():
+    # layer-norm built from primitives: mean / sub / square / rsqrt / mul with broadcasting
+    rng = np.random.default_rng(4)
+    g = rng.normal(size=8)
+
+    def ln(xp, x):
+        mu = xp.mean(x, axis=-1, keepdims=True)
+        c = xp.subtract(x, mu)
+        var = xp.mean(xp.square(c), axis=-1, keepdims=True)
+        y = xp.multiply(c, xp.rsqrt(xp.add(var, 1e-5)))
+        return xp.multiply(y, g)
+
+    _check(ln, rng.normal(size=(2, 3, 8)))
+
+
+def test_indexing_ops_vs_bruteforce():
+    rng = np.random.default_rng(5)
+    R = rng.normal(size=(2, 3))
+
+    def feats(xp, r):  # r (4, 3): electron-nucleus vectors and distances
+        d = xp.subtract(xp.expand_dims(r, 1), R)  # (4, 2, 3)
+        dist = xp.sqrt(xp.sum(xp.square(d), axis=-1))  # (4, 2)
+        f = xp.concatenate([xp.reshape(d, (4, 6)), dist], axis=-1)  # (4, 8)
+        f = xp.transpose(f, (1, 0))
+        return xp.getitem(f, (slice(1, 7),))
+
+    _check(feats, rng.normal(size=(2, 4, 3)))
+
+
+@pytest.mark.parametrize('n', [1, 2, 4, 6])
+def test_slogdet_vs_bruteforce(n):
+    # shapes of test/test_layers.py:341-396 (small matrices through a tanh layer)
+    rng = np.random.default_rng(6)
+    W = rng.normal(size=(5, n * n))
+
+    def f(xp, x):
+        A = xp.reshape(xp.tanh(xp.dot(x, W)), (n, n))
+        return xp.slogdet(A)[1]
+
+    _check(f, rng.normal(size=(3, 5)), rtol=1e-4 if n == 6 else RTOL, atol=1e-8)
+
+
+@pytest.mark.parametrize('n', [2, 3])
+def test_slogdet_vs_cofactor_expansion(n):
+    """log|det| written as an explicit polynomial (no linalg call in the brute force), so
+    the check does not lean on torch's derivative formulas for det / slogdet."""
+    rng = np.random.default_rng(16)
+    W = rng.normal(size=(4, n * n))
+
+    def det_poly(A):
+        if n == 2:
+            return A[0, 0] * A[1, 1] - A[0, 1] * A[1, 0]
+        return (
+            A[0, 0] * (A[1, 1] * A[2, 2] - A[1, 2] * A[2, 1])
+            - A[0, 1] * (A[1, 0] * A[2, 2] - A[1, 2] * A[2, 0])
+            + A[0, 2] * (A[1, 0] * A[2, 1] - A[1, 1] * A[2, 0])
+        )
+
+    def f(xp, x):
+        A = xp.reshape(xp.tanh(xp.dot(x, W)), (n, n))
+        if xp is plain:
+            return torch.log(torch.abs(det_poly(A)))
+        return xp.slogdet(A)[1]
+
+    _check(f, rng.normal(size=(3, 4)), atol=1e-8)
+
+
+def test_slogdet_closed_forms():
+    rng = np.random.default_rng(7)
+    B, n, P = 4, 5, 3
+    # diagonal A(x): log|det| = sum log|a_ii|, derivative rows only on the diagonal
+    a = rng.uniform(0.5, 2.0, size=(B, n)) * rng.choice([-1, 1], size=(B, n))
+    A = np.zeros((B, n, n))
+    A[:, range(n), range(n)] = a
+    Jd = rng.normal(size=(P, B, n))
+    J = np.zeros((P, B, n, n))
+    J[:, :, range(n), range(n)] = Jd
+    Ld = rng.normal(size=(B, n))
+    L = np.zeros((B, n, n))
+    L[:, range(n), range(n)] = Ld
+    sign, (ld, Jo, Lo) = rules.slogdet_rule(A, J, L)
+    _close(sign, np.prod(np.sign(a), -1))
+    _close(ld, np.log(np.abs(a)).sum(-1))
+    _close(Jo, (Jd / a[None]).sum(-1))
+    _close(Lo, (Ld / a).sum(-1) - ((Jd / a[None]) ** 2).sum((0, -1)))
+    # swapping two rows flips the sign and nothing else
+    A2 = rng.normal(size=(B, n, n))
+    J2, L2 = rng.normal(size=(P, B, n, n)), rng.normal(size=(B, n, n))
+    perm = [1, 0, 2, 3, 4]
+    s1, (l1, j1, p1) = rules.slogdet_rule(A2, J2, L2)
+    s2, (l2, j2, p2) = rules.slogdet_rule(A2[:, perm], J2[:, :, perm], L2[:, perm])
+    _close(s2, -s1), _close(l2, l1), _close(j2, j1), _close(p2, p1, atol=1e-9)
+
+
+@pytest.mark.parametrize('n,H,d,valid', [(1, 1, 1, 1), (4, 2, 3, 4), (5, 2, 3, 2)])
+def test_mhsa_vs_bruteforce(n, H, d, valid):
+    """softmax(q k^T) v where q, k, v are random linear maps of the 3n inputs; the last
+    case pads the sequence as test_attention.py:323-326 does (max_sequence < n)."""
+    rng = np.random.default_rng(8)
+    n_in = 3 * n
+    Wq, Wk, Wv = (rng.normal(size=(n_in, n * H * d)) / np.sqrt(n_in) for _ in range(3))
+    mask = np.zeros(n, dtype=bool)
+    mask[:valid] = True
+    in_mask = np.zeros(n_in, dtype=bool)
+    in_mask[: 3 * valid] = True
+
+    def f(xp, x):
+        x = xp.reshape(x, (n_in,))
+        q, k, v = (xp.reshape(xp.tanh(xp.dot(x, W)), (n, H, d)) for W in (Wq, Wk, Wv))
+        if xp is plain:
+            return xp.multi_head_self_attention(q, k, v, mask)
+        B = q.B
+        return xp.multi_head_self_attention(
+            q, k, v, np.broadcast_to(mask, (B, n)), np.broadcast_to(in_mask[:, None], (n_in, B))
+        )
+
+    x = rng.normal(size=(2, n_in))
+    # padded electrons' coordinates are inactive inputs: zero weights in the forward
+    # Laplacian (folx/interpreter.py:319 ``weights=``), frozen in the brute force
+    w = np.broadcast_to(in_mask.astype(np.float64), (n_in,))
+    out = f(ob, ob.init_state(x, weights=w, dtype=np.float64))
+    y, J, L = out.x, out.J, out.lap
+
+    def f_plain(t):
+        t = torch.where(torch.as_tensor(in_mask), t, t.detach())
+        return f(plain, t)
+
+    by, bJ, bL = brute_force(f_plain, x)
+    m = mask
+    _close(y[:, m], by[:, m], atol=1e-9)
+    _close(J[:, :, m], bJ[:, :, m], atol=1e-9)
+    _close(L[:, m], bL[:, m], rtol=1e-5, atol=1e-8)
+
+
+def test_mhsa_masking_zeroes_inactive_rows():
+    rng = np.random.default_rng(9)
+    P, B, n, H, d = 6, 2, 4, 1, 2
+    t = lambda *s: rng.normal(size=s)
+    args = [t(B, n, H, d), t(P, B, n, H, d), t(B, n, H, d)] * 3
+    in_mask = np.ones((P, B), dtype=bool)
+    in_mask[3:] = False
+    o, oJ, oL = rules.mhsa_rule(*args, None, in_mask)
+    assert np.all(oJ[3:] == 0)
+    # inactive coordinates do not contribute to the Laplacian either
+    args2 = [a.copy() for a in args]
+    for i in (1, 4, 7):
+        args2[i][3:] = 123.0
+    o2, oJ2, oL2 = rules.mhsa_rule(*args2, None, in_mask)
+    _close(oL, oL2)
+    _close(oJ, oJ2)
