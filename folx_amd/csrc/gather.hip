@@ -1,0 +1,81 @@
+// Re-indexing of sparse Jacobian rows between row frames.  The index masks are static and
+// live on the host; the device only sees small int32 tables.  Both kernels stream the
+// Jacobian once and are bound by HBM bandwidth.
+#include "common.h"
+
+namespace {
+
+// out[t][b][so][si] = sum_s data[take[t][s][so]][b][so][si]   (take < 0: no source)
+// Threads run along (so, si) so reads and writes are coalesced; the table entry is shared
+// by the S_inner consecutive threads of one `so` and by all walkers b (blockIdx.y).
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ data,
+                                                          const int32_t* __restrict__ take,
+                                                          float* __restrict__ out, int32_t k_out,
+                                                          int32_t n_slots, int64_t B, int64_t S_outer,
+                                                          int64_t S_inner) {
+  const int64_t S = S_outer * S_inner;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= S) return;
+  const int64_t so = e / S_inner;
+  const int32_t t = blockIdx.z;
+  int32_t src[8];
+  const int32_t ns = n_slots < 8 ? n_slots : 8;
+  for (int s = 0; s < ns; ++s) src[s] = take[((int64_t)t * n_slots + s) * S_outer + so];
+  for (int64_t b = blockIdx.y; b < B; b += gridDim.y) {
+    float acc = 0.0f;
+    for (int s = 0; s < n_slots; ++s) {
+      const int32_t r = s < 8 ? src[s] : take[((int64_t)t * n_slots + s) * S_outer + so];
+      if (r >= 0) acc += data[((int64_t)r * B + b) * S + e];
+    }
+    out[((int64_t)t * B + b) * S + e] = acc;
+  }
+}
+
+__global__ __launch_bounds__(256) void scatter_add_rows_kernel(const float* __restrict__ data,
+                                                               const int32_t* __restrict__ idx,
+                                                               float* __restrict__ out, int64_t B,
+                                                               int64_t S_outer, int64_t S_inner) {
+  const int64_t S = S_outer * S_inner;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= S) return;
+  const int64_t so = e / S_inner;
+  const int32_t r = blockIdx.z;
+  const int32_t t = idx[(int64_t)r * S_outer + so];
+  if (t < 0) return;
+  for (int64_t b = blockIdx.y; b < B; b += gridDim.y)
+    atomicAdd(&out[((int64_t)t * B + b) * S + e], data[((int64_t)r * B + b) * S + e]);
+}
+
+}  // namespace
+
+extern "C" int folx_hip_gather_rows(void* stream, const float* data, const int32_t* take, float* out,
+                                    int32_t k_in, int32_t k_out, int32_t n_slots, int64_t B,
+                                    int64_t S_outer, int64_t S_inner) {
+  if (k_in < 0 || k_out < 0 || n_slots < 0 || B < 0 || S_outer < 0 || S_inner < 0) return FOLX_HIP_EINVAL;
+  const int64_t S = S_outer * S_inner;
+  if (k_out == 0 || B == 0 || S == 0) return FOLX_HIP_OK;
+  if (!out || (n_slots > 0 && (!take || (k_in > 0 && !data)))) return FOLX_HIP_EINVAL;
+  if (k_out > 65535) return FOLX_HIP_ENOTSUP;
+  const int64_t blocks = (S + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  const unsigned gy = (unsigned)(B < 4096 ? B : 4096);
+  gather_rows_kernel<<<dim3((unsigned)blocks, gy, (unsigned)k_out), dim3(256), 0, (hipStream_t)stream>>>(
+      data, take, out, k_out, n_slots, B, S_outer, S_inner);
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_scatter_add_rows(void* stream, const float* data, const int32_t* idx,
+                                         float* out, int32_t k_in, int32_t k_out, int64_t B,
+                                         int64_t S_outer, int64_t S_inner) {
+  if (k_in < 0 || k_out < 0 || B < 0 || S_outer < 0 || S_inner < 0) return FOLX_HIP_EINVAL;
+  const int64_t S = S_outer * S_inner;
+  if (k_in == 0 || B == 0 || S == 0) return FOLX_HIP_OK;
+  if (!data || !idx || !out) return FOLX_HIP_EINVAL;
+  if (k_in > 65535) return FOLX_HIP_ENOTSUP;
+  const int64_t blocks = (S + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  const unsigned gy = (unsigned)(B < 4096 ? B : 4096);
+  scatter_add_rows_kernel<<<dim3((unsigned)blocks, gy, (unsigned)k_in), dim3(256), 0, (hipStream_t)stream>>>(
+      data, idx, out, B, S_outer, S_inner);
+  return folx_launch_status();
+}

@@ -1,0 +1,138 @@
+// Broadcasting elementwise rules on a shared Jacobian row frame: the binary rule
+// (mul / div / add / sub of two triplets) and the affine map against constants.
+// Both are single streaming passes bound by HBM bandwidth.
+#include "common.h"
+
+namespace {
+
+constexpr int PSPLIT = 4;
+
+// Binary rule.  A workgroup is 4 wavefronts over the same 64 output elements; wavefront
+// w handles Jacobian rows p = w, w + 4, ...; the sums over p meet in LDS.
+template <int OP>
+__global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
+    const float* __restrict__ a, const float* __restrict__ aj, const float* __restrict__ al,
+    const float* __restrict__ b, const float* __restrict__ bj, const float* __restrict__ bl,
+    float* __restrict__ y, float* __restrict__ yj, float* __restrict__ yl, int64_t S, Bcast3 ia,
+    Bcast3 ib, int64_t a_S, int64_t b_S, int32_t P) {
+  __shared__ float red[2][PSPLIT][FOLX_WAVE];
+  const int lane = threadIdx.x % FOLX_WAVE;
+  const int w = threadIdx.x / FOLX_WAVE;
+  const int64_t i = (int64_t)blockIdx.x * FOLX_WAVE + lane;
+  const bool active = i < S;
+  float sab = 0.0f, sbb = 0.0f;
+  float av = 0.f, bv = 1.f, ca = 0.f, cb = 0.f;
+  int64_t oa = 0, ob = 0;
+  if (active) {
+    oa = ia.off(i);
+    ob = ib.off(i);
+    av = a[oa];
+    bv = b[ob];
+    // y_jac = ca * a_jac + cb * b_jac
+    if constexpr (OP == FOLX_BIN_MUL) { ca = bv; cb = av; }
+    else if constexpr (OP == FOLX_BIN_DIV) { ca = 1.0f / bv; cb = -av * ca * ca; }
+    else if constexpr (OP == FOLX_BIN_ADD) { ca = 1.0f; cb = 1.0f; }
+    else { ca = 1.0f; cb = -1.0f; }
+    for (int p = w; p < P; p += PSPLIT) {
+      const float ja = aj[(int64_t)p * a_S + oa];
+      const float jb = bj[(int64_t)p * b_S + ob];
+      yj[(int64_t)p * S + i] = ca * ja + cb * jb;
+      if constexpr (OP == FOLX_BIN_MUL || OP == FOLX_BIN_DIV) sab += ja * jb;
+      if constexpr (OP == FOLX_BIN_DIV) sbb += jb * jb;
+    }
+  }
+  if constexpr (OP == FOLX_BIN_MUL || OP == FOLX_BIN_DIV) {
+    red[0][w][lane] = sab;
+    red[1][w][lane] = sbb;
+    __syncthreads();
+  }
+  if (w == 0 && active) {
+    float l = ca * al[oa] + cb * bl[ob];
+    if constexpr (OP == FOLX_BIN_MUL) {
+      float s = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
+      y[i] = av * bv;
+      l += 2.0f * s;
+    } else if constexpr (OP == FOLX_BIN_DIV) {
+      float s = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
+      float t = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+      const float rb = 1.0f / bv;
+      y[i] = av * rb;
+      // H_lr = -2 / b^2 (counted once for the pair), H_rr = 2 a / b^3
+      l += -2.0f * rb * rb * s + 2.0f * av * rb * rb * rb * t;
+    } else if constexpr (OP == FOLX_BIN_ADD) {
+      y[i] = av + bv;
+    } else {
+      y[i] = av - bv;
+    }
+    yl[i] = l;
+  }
+}
+
+__global__ __launch_bounds__(256) void rows_affine_kernel(const float* __restrict__ in,
+                                                          float* __restrict__ out, int64_t rows,
+                                                          int64_t in_S, int64_t S,
+                                                          const float* __restrict__ c,
+                                                          const float* __restrict__ d, float alpha,
+                                                          float beta, Bcast3 iin, Bcast3 ic,
+                                                          Bcast3 id) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= S) return;
+  const int64_t oi = iin.off(i);
+  const float cv = c ? alpha * c[ic.off(i)] : alpha;
+  const float dv = d ? beta * d[id.off(i)] : 0.0f;
+  // blockIdx.y strides over rows so that very tall stacks need no 64-bit grid
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) out[r * S + i] = in[r * in_S + oi] * cv + dv;
+}
+
+Bcast3 mk(const int64_t* dims, int k) {
+  Bcast3 b;
+  b.n1 = dims[1]; b.n2 = dims[2];
+  b.s0 = dims[3 * k + 0]; b.s1 = dims[3 * k + 1]; b.s2 = dims[3 * k + 2];
+  return b;
+}
+
+}  // namespace
+
+extern "C" int folx_hip_binary_fwdlap(void* stream, int32_t op, const float* a, const float* a_jac,
+                                      const float* a_lap, const float* b, const float* b_jac,
+                                      const float* b_lap, float* y, float* y_jac, float* y_lap,
+                                      const int64_t* dims, int64_t a_S, int64_t b_S, int32_t P) {
+  if (!dims || op < 0 || op >= FOLX_BIN_COUNT || P < 0) return FOLX_HIP_EINVAL;
+  if (dims[0] < 0 || dims[1] < 0 || dims[2] < 0) return FOLX_HIP_EINVAL;
+  const int64_t S = dims[0] * dims[1] * dims[2];
+  if (S == 0) return FOLX_HIP_OK;
+  if (!a || !a_lap || !b || !b_lap || !y || !y_lap || (P > 0 && (!a_jac || !b_jac || !y_jac)))
+    return FOLX_HIP_EINVAL;
+  const int64_t blocks = (S + FOLX_WAVE - 1) / FOLX_WAVE;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  Bcast3 ia = mk(dims, 1), ib = mk(dims, 2);
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)blocks), block(FOLX_WAVE * PSPLIT);
+#define FOLX_CASE(OP)                                                                         \
+  case OP:                                                                                    \
+    binary_kernel<OP><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, y, y_jac,    \
+                                               y_lap, S, ia, ib, a_S, b_S, P);                \
+    break;
+  switch (op) {
+    FOLX_CASE(FOLX_BIN_MUL) FOLX_CASE(FOLX_BIN_DIV) FOLX_CASE(FOLX_BIN_ADD) FOLX_CASE(FOLX_BIN_SUB)
+  }
+#undef FOLX_CASE
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_rows_affine(void* stream, const float* in, float* out, int64_t rows,
+                                    int64_t in_S, const float* c, const float* d, float alpha,
+                                    float beta, const int64_t* dims) {
+  if (!dims || rows < 0 || in_S < 0) return FOLX_HIP_EINVAL;
+  if (dims[0] < 0 || dims[1] < 0 || dims[2] < 0) return FOLX_HIP_EINVAL;
+  const int64_t S = dims[0] * dims[1] * dims[2];
+  if (S == 0 || rows == 0) return FOLX_HIP_OK;
+  if (!in || !out) return FOLX_HIP_EINVAL;
+  const int64_t blocks = (S + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  Bcast3 iin = mk(dims, 1), ic = mk(dims, 2), id = mk(dims, 3);
+  const unsigned gy = (unsigned)(rows < 1024 ? rows : 1024);
+  rows_affine_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
+      in, out, rows, in_S, S, c, d, alpha, beta, iin, ic, id);
+  return folx_launch_status();
+}

@@ -1,0 +1,77 @@
+// Reductions over a middle axis: in [rows][outer][red][inner] -> out [rows][outer][inner].
+// The sum rule is linear, so the same kernel serves x, the Jacobian rows and lap.
+#include "common.h"
+
+namespace {
+
+// inner >= 2: one thread per output element, consecutive threads on consecutive `inner`
+// positions so every step of the loop over `red` is a coalesced read.
+template <bool MAX>
+__global__ __launch_bounds__(256) void reduce_mid_kernel(const float* __restrict__ in,
+                                                         float* __restrict__ out, int64_t total,
+                                                         int64_t red, int64_t inner, float alpha) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= total) return;
+  const int64_t ii = o % inner;
+  const int64_t ro = o / inner;  // (row, outer) flattened
+  const float* src = in + ro * red * inner + ii;
+  float acc = MAX ? -INFINITY : 0.0f;
+  for (int64_t r = 0; r < red; ++r) {
+    const float v = src[r * inner];
+    acc = MAX ? fmaxf(acc, v) : acc + v;
+  }
+  out[o] = MAX ? acc : alpha * acc;
+}
+
+// inner == 1: one wavefront per output element, lanes stride over the reduced axis.
+template <bool MAX>
+__global__ __launch_bounds__(256) void reduce_last_kernel(const float* __restrict__ in,
+                                                          float* __restrict__ out, int64_t total,
+                                                          int64_t red, float alpha) {
+  const int lane = threadIdx.x % FOLX_WAVE;
+  const int64_t o = (int64_t)blockIdx.x * (256 / FOLX_WAVE) + threadIdx.x / FOLX_WAVE;
+  if (o >= total) return;
+  const float* src = in + o * red;
+  float acc = MAX ? -INFINITY : 0.0f;
+  for (int64_t r = lane; r < red; r += FOLX_WAVE) {
+    const float v = src[r];
+    acc = MAX ? fmaxf(acc, v) : acc + v;
+  }
+#pragma unroll
+  for (int off = FOLX_WAVE / 2; off > 0; off >>= 1) {
+    const float v = __shfl_xor(acc, off, FOLX_WAVE);
+    acc = MAX ? fmaxf(acc, v) : acc + v;
+  }
+  if (lane == 0) out[o] = MAX ? acc : alpha * acc;
+}
+
+template <bool MAX>
+int launch_reduce(hipStream_t st, const float* in, float* out, int64_t rows, int64_t outer,
+                  int64_t red, int64_t inner, float alpha) {
+  if (rows < 0 || outer < 0 || red < 0 || inner < 0) return FOLX_HIP_EINVAL;
+  const int64_t total = rows * outer * inner;
+  if (total == 0) return FOLX_HIP_OK;
+  if (!in || !out) return FOLX_HIP_EINVAL;
+  if (inner == 1 && red >= 16) {
+    const int64_t blocks = (total + 3) / 4;
+    if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+    reduce_last_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, alpha);
+  } else {
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+    reduce_mid_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, inner, alpha);
+  }
+  return folx_launch_status();
+}
+
+}  // namespace
+
+extern "C" int folx_hip_reduce_sum(void* stream, const float* in, float* out, int64_t rows,
+                                   int64_t outer, int64_t red, int64_t inner, float alpha) {
+  return launch_reduce<false>((hipStream_t)stream, in, out, rows, outer, red, inner, alpha);
+}
+
+extern "C" int folx_hip_reduce_max(void* stream, const float* in, float* out, int64_t outer,
+                                   int64_t red, int64_t inner) {
+  return launch_reduce<true>((hipStream_t)stream, in, out, 1, outer, red, inner, 1.0f);
+}

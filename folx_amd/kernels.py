@@ -1,0 +1,239 @@
+"""Thin tensor-level wrappers over the C ABI: torch tensors in, torch tensors out.
+
+torch is used only to own device memory and to name the current HIP stream; every
+arithmetic operation happens inside ``libfolx_hip.so``.  All tensors must be float32,
+contiguous and on the GPU.  Layout: x (B, *s), jac (P, B, *s), lap (B, *s).
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import ACT, BINOP, check
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    if t is None:
+        return None
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _chk(*ts):
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise _lib.FolxHipError('folx_amd kernels need GPU tensors (no CPU fallback)')
+        if not t.is_contiguous():
+            raise ValueError('non-contiguous tensor passed to a folx_amd kernel')
+        if t.dtype not in (torch.float32, torch.int32, torch.uint8):
+            raise TypeError(f'unsupported dtype {t.dtype}')
+
+
+def _dims(*vals):
+    return (ctypes.c_int64 * len(vals))(*[int(v) for v in vals])
+
+
+def dense(x, jac, lap, W, bias=None):
+    """x (.., K), jac (P, .., K), lap (.., K), W (K, N) -> triplet with last dim N."""
+    _chk(x, jac, lap, W, bias)
+    K, N = W.shape
+    P = jac.shape[0]
+    R = x.numel() // K
+    y = torch.empty((*x.shape[:-1], N), device=x.device, dtype=torch.float32)
+    yj = torch.empty((P, *x.shape[:-1], N), device=x.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    check(
+        _lib.load().folx_hip_dense_fwdlap(
+            _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(y), _p(yj), _p(yl), R, P, K, N
+        ),
+        'dense_fwdlap',
+    )
+    return y, yj, yl
+
+
+def elementwise(name, x, jac, lap, param=0.0, inplace=False):
+    _chk(x, jac, lap)
+    P = jac.shape[0]
+    S = x.numel()
+    if inplace:
+        y, yj, yl = x, jac, lap
+    else:
+        y, yj, yl = torch.empty_like(x), torch.empty_like(jac), torch.empty_like(lap)
+    check(
+        _lib.load().folx_hip_elementwise_fwdlap(
+            _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(y), _p(yj), _p(yl), S, P
+        ),
+        f'elementwise_fwdlap[{name}]',
+    )
+    return y, yj, yl
+
+
+def collapse3(out_shape, *strides_list):
+    """Collapse a broadcast index space to <= 3 dims.  ``strides_list``: per operand, the
+    element strides over ``out_shape`` (0 where broadcast).  Returns (n, [s, ...]) with
+    len(n) == 3, or None if more than 3 dims remain."""
+    dims = [(int(n), tuple(int(s[i]) for s in strides_list)) for i, n in enumerate(out_shape) if n != 1]
+    merged = []
+    for n, st in dims:
+        if merged:
+            pn, pst = merged[-1]
+            if all(ps == s * n for ps, s in zip(pst, st)):
+                merged[-1] = (pn * n, st)
+                continue
+        merged.append((n, st))
+    if len(merged) > 3:
+        return None
+    while len(merged) < 3:
+        merged.insert(0, (1, tuple(0 for _ in strides_list)))
+    n = [m[0] for m in merged]
+    per_op = [[m[1][k] for m in merged] for k in range(len(strides_list))]
+    return n, per_op
+
+
+def bstrides(shape, out_shape):
+    """Element strides of a contiguous array of ``shape`` broadcast to ``out_shape``."""
+    shape = (1,) * (len(out_shape) - len(shape)) + tuple(shape)
+    st, acc = [], 1
+    for n in reversed(shape):
+        st.append(acc)
+        acc *= n
+    st = st[::-1]
+    return [0 if n == 1 and o != 1 else s for n, s, o in zip(shape, st, out_shape)]
+
+
+def binary(op, a, aj, al, b, bj, bl):
+    """Same-frame binary rule with numpy-style broadcasting of the (B, *s) shapes."""
+    _chk(a, aj, al, b, bj, bl)
+    P = aj.shape[0]
+    assert bj.shape[0] == P
+    out_shape = torch.broadcast_shapes(a.shape, b.shape)
+    col = collapse3(out_shape, bstrides(a.shape, out_shape), bstrides(b.shape, out_shape))
+    if col is None:
+        a, aj, al = (t.expand(*t.shape[: t.dim() - a.dim()], *out_shape).contiguous() for t in (a, aj, al))
+        b, bj, bl = (t.expand(*t.shape[: t.dim() - b.dim()], *out_shape).contiguous() for t in (b, bj, bl))
+        col = collapse3(out_shape, bstrides(a.shape, out_shape), bstrides(b.shape, out_shape))
+    n, (sa, sb) = col
+    y = torch.empty(out_shape, device=a.device, dtype=torch.float32)
+    yj = torch.empty((P, *out_shape), device=a.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    check(
+        _lib.load().folx_hip_binary_fwdlap(
+            _stream(), BINOP[op], _p(a), _p(aj), _p(al), _p(b), _p(bj), _p(bl), _p(y), _p(yj), _p(yl),
+            _dims(*n, *sa, *sb), a.numel(), b.numel(), P,
+        ),
+        f'binary_fwdlap[{op}]',
+    )
+    return y, yj, yl
+
+
+def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta=1.0):
+    """out[r] = alpha * in[r] * c + beta * d with broadcasting to ``out_shape``.
+    ``inp`` holds ``rows`` rows of shape ``row_shape``; c / d are arrays broadcastable to
+    ``out_shape``.  Returns a tensor (rows, *out_shape)."""
+    _chk(inp, c, d)
+    sin = bstrides(row_shape, out_shape)
+    sc = bstrides(c.shape, out_shape) if c is not None else [0] * len(out_shape)
+    sd = bstrides(d.shape, out_shape) if d is not None else [0] * len(out_shape)
+    col = collapse3(out_shape, sin, sc, sd)
+    if col is None:
+        raise ValueError('rows_affine: more than 3 broadcast dims after collapsing')
+    n, (s_in, s_c, s_d) = col
+    out = torch.empty((rows, *out_shape), device=inp.device, dtype=torch.float32)
+    in_S = int(np.prod(row_shape, dtype=np.int64))
+    check(
+        _lib.load().folx_hip_rows_affine(
+            _stream(), _p(inp), _p(out), rows, in_S, _p(c), _p(d), float(alpha), float(beta),
+            _dims(*n, *s_in, *s_c, *s_d),
+        ),
+        'rows_affine',
+    )
+    return out
+
+
+def reduce_sum(inp, rows, outer, red, inner, alpha=1.0):
+    _chk(inp)
+    out = torch.empty((rows, outer, inner), device=inp.device, dtype=torch.float32)
+    check(
+        _lib.load().folx_hip_reduce_sum(_stream(), _p(inp), _p(out), rows, outer, red, inner, float(alpha)),
+        'reduce_sum',
+    )
+    return out
+
+
+def reduce_max(inp, outer, red, inner):
+    _chk(inp)
+    out = torch.empty((outer, inner), device=inp.device, dtype=torch.float32)
+    check(_lib.load().folx_hip_reduce_max(_stream(), _p(inp), _p(out), outer, red, inner), 'reduce_max')
+    return out
+
+
+def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
+    """data (k_in, B, S_outer * S_inner); take int32 (k_out, n_slots, S_outer) on device."""
+    _chk(data, take)
+    k_in = data.shape[0]
+    out = torch.empty((k_out, B, S_outer * S_inner), device=data.device, dtype=torch.float32)
+    check(
+        _lib.load().folx_hip_gather_rows(
+            _stream(), _p(data), _p(take), _p(out), k_in, k_out, n_slots, B, S_outer, S_inner
+        ),
+        'gather_rows',
+    )
+    return out
+
+
+def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
+    _chk(data, idx)
+    k_in = data.shape[0]
+    out = torch.zeros((k_out, B, S_outer * S_inner), device=data.device, dtype=torch.float32)
+    check(
+        _lib.load().folx_hip_scatter_add_rows(
+            _stream(), _p(data), _p(idx), _p(out), k_in, k_out, B, S_outer, S_inner
+        ),
+        'scatter_add_rows',
+    )
+    return out
+
+
+def slogdet(A, AJ, AL):
+    """A (.., n, n), AJ (P, .., n, n), AL (.., n, n) -> sign, logdet (..), jac (P, ..), lap (..)."""
+    _chk(A, AJ, AL)
+    n = A.shape[-1]
+    P = AJ.shape[0]
+    lead = A.shape[:-2]
+    NM = int(np.prod(lead, dtype=np.int64)) if len(lead) else 1
+    sign = torch.empty(lead, device=A.device, dtype=torch.float32)
+    ld = torch.empty_like(sign)
+    ldj = torch.empty((P, *lead), device=A.device, dtype=torch.float32)
+    ldl = torch.empty_like(sign)
+    check(
+        _lib.load().folx_hip_slogdet_fwdlap(
+            _stream(), _p(A), _p(AJ), _p(AL), _p(sign), _p(ld), _p(ldj), _p(ldl), NM, n, P
+        ),
+        'slogdet_fwdlap',
+    )
+    return sign, ld, ldj, ldl
+
+
+def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None):
+    """q/k/v (B, n, H, d) triplets; mask uint8 (B, n); input_mask uint8 (P, B)."""
+    _chk(q, qj, ql, k, kj, kl, v, vj, vl, mask, input_mask)
+    B, n, H, d = q.shape
+    P = qj.shape[0]
+    o, oj, ol = torch.empty_like(q), torch.empty_like(qj), torch.empty_like(q)
+    check(
+        _lib.load().folx_hip_mhsa_fwdlap(
+            _stream(), _p(q), _p(qj), _p(ql), _p(k), _p(kj), _p(kl), _p(v), _p(vj), _p(vl),
+            _p(mask), _p(input_mask), _p(o), _p(oj), _p(ol), B, n, H, d, P,
+        ),
+        'mhsa_fwdlap',
+    )
+    return o, oj, ol

@@ -1,0 +1,188 @@
+/*
+ * folx_hip.h -- C ABI of the MI355X (gfx950) forward-Laplacian kernel library.
+ *
+ * Every entry point propagates the triplet (x, jacobian, laplacian) of microsoft/folx
+ * through one rule.  Conventions shared by all calls:
+ *
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls are
+ *     asynchronous on that stream, allocate nothing and never synchronise.
+ *   - All data pointers are DEVICE pointers to contiguous float32 (index tables: int32).
+ *   - Layout: value x[S], Jacobian jac[P][S] (Jacobian axis leading, reference JAC_DIM = 0,
+ *     folx/api.py:16), Laplacian lap[S], where S flattens (walker, *shape) with the walker
+ *     axis outermost.  For a sparse Jacobian P is the number of stored rows k; the int
+ *     index mask lives on the host and never reaches the library except as gather tables.
+ *   - Return value: FOLX_HIP_OK (0) or a negative FOLX_HIP_E* code; nothing is launched
+ *     when an argument check fails.  folx_hip_strerror() names the code.
+ *   - Unless stated, outputs must not alias inputs.
+ */
+#ifndef FOLX_HIP_H
+#define FOLX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FOLX_HIP_OK 0
+#define FOLX_HIP_EINVAL (-1)   /* null pointer, negative size, inconsistent shape      */
+#define FOLX_HIP_ENOTSUP (-2)  /* size outside what the kernels are built for          */
+#define FOLX_HIP_ELAUNCH (-3)  /* hipGetLastError() != hipSuccess after the launch     */
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int folx_hip_version(void);
+/* Static description of a return code. */
+const char* folx_hip_strerror(int code);
+
+/* Elementwise functions of folx_hip_elementwise_fwdlap; the rule needs f, f', f''.
+ * Replaces the per-primitive entries of folx/wrapped_functions.py:400-415, :552-556. */
+enum folx_hip_act {
+  FOLX_ACT_TANH = 0,
+  FOLX_ACT_SILU = 1,
+  FOLX_ACT_EXP = 2,
+  FOLX_ACT_LOG = 3,
+  FOLX_ACT_SQRT = 4,
+  FOLX_ACT_RSQRT = 5,
+  FOLX_ACT_SQUARE = 6,
+  FOLX_ACT_LOGISTIC = 7,
+  FOLX_ACT_SOFTPLUS = 8,
+  FOLX_ACT_SIN = 9,
+  FOLX_ACT_COS = 10,
+  FOLX_ACT_ABS = 11,
+  FOLX_ACT_LOG1P = 12,
+  FOLX_ACT_RECIPROCAL = 13,
+  FOLX_ACT_EXPM1 = 14,
+  FOLX_ACT_INTEGER_POW = 15, /* param = exponent (integer value) */
+  FOLX_ACT_COUNT = 16
+};
+
+/* Binary functions of folx_hip_binary_fwdlap. */
+enum folx_hip_binop {
+  FOLX_BIN_MUL = 0, /* jax.lax.mul, MULTIPLICATION rule (folx/hessian.py:177-188)   */
+  FOLX_BIN_DIV = 1, /* jax.lax.div, custom Hessian (folx/custom_hessian.py:35-59)   */
+  FOLX_BIN_ADD = 2, /* jax.lax.add, LINEAR                                          */
+  FOLX_BIN_SUB = 3, /* jax.lax.sub, LINEAR                                          */
+  FOLX_BIN_COUNT = 4
+};
+
+/*
+ * Dense layer y = h @ W (+ bias) applied to the stacked operand [x; J; lap].
+ * Replaces _dot_general_one_constant, folx/wrapped_functions.py:71-171 (the three
+ * dot_generals at :167-169) for a constant right operand contracted with the last axis.
+ *   x   [R][K]      jac [P][R][K]     lap [R][K]       R = walkers * positions
+ *   W   [K][N] row-major, shared by all rows;  bias [N] or NULL (added to y only)
+ *   y   [R][N]      y_jac [P][R][N]   y_lap [R][N]
+ * One launch covers all (P + 2) * R rows (FP32 MFMA, fp32 accumulate).
+ */
+int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac, const float* lap,
+                          const float* W, const float* bias, float* y, float* y_jac,
+                          float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N);
+
+/*
+ * Elementwise activation rule  y = f(x), y_jac[p] = f'(x) * jac[p],
+ * y_lap = f'(x) * lap + f''(x) * sum_p jac[p]^2   in one pass over the Jacobian.
+ * Replaces dense_elementwise_jvp (folx/jvp.py:687-697), the single-argument branch of
+ * sparse_diag_jvp (folx/jvp.py:262-272) and elementwise_jhj_trace (folx/hessian.py:87-112),
+ * combined as in folx/wrapper.py:120-125.  In-place use (y == x, y_jac == jac,
+ * y_lap == lap) is allowed.
+ */
+int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float param, const float* x,
+                                const float* jac, const float* lap, float* y, float* y_jac,
+                                float* y_lap, int64_t S, int32_t P);
+
+/*
+ * Binary elementwise rule for two operands whose Jacobians live on the same row frame
+ * (both dense with P rows, or sparse with identical index masks).  The output index
+ * space is (n0, n1, n2), row-major; each operand addresses it with element strides
+ * sa / sb (0 = broadcast).  dims = {n0, n1, n2, sa0, sa1, sa2, sb0, sb1, sb2} is a HOST
+ * array.  a_S / b_S are the element counts of one Jacobian row of a / b.
+ * MUL: y = a b, y_jac = a b_jac + b a_jac, y_lap = a b_lap + b a_lap + 2 sum_p a_jac b_jac
+ * Replaces dense_split_jvp (folx/jvp.py:676-684) + dot_product_jac_hessian_jac
+ * (folx/hessian.py:177-188) / div_jac_hessian_jac (folx/custom_hessian.py:35-59).
+ */
+int folx_hip_binary_fwdlap(void* stream, int32_t op, const float* a, const float* a_jac,
+                           const float* a_lap, const float* b, const float* b_jac,
+                           const float* b_lap, float* y, float* y_jac, float* y_lap,
+                           const int64_t* dims, int64_t a_S, int64_t b_S, int32_t P);
+
+/*
+ * Row-stack affine map with broadcast coefficient arrays:
+ *   out[r][i] = alpha * in[r][ia(i)] * (c ? c[ic(i)] : 1) + (d ? beta * d[id(i)] : 0)
+ * over rows r < rows and the index space (n0, n1, n2).  dims = {n0, n1, n2, sin0..2,
+ * sc0..2, sd0..2} is a HOST array of element strides; in_S is the element count of one
+ * input row.  Used for every LINEAR rule against constants (add, sub, neg, scaling by a
+ * constant, folx/wrapped_functions.py:361-376) on x, on the Jacobian rows and on lap.
+ */
+int folx_hip_rows_affine(void* stream, const float* in, float* out, int64_t rows,
+                         int64_t in_S, const float* c, const float* d, float alpha,
+                         float beta, const int64_t* dims);
+
+/*
+ * Sum over the middle axis: in [rows][outer][red][inner] -> out [rows][outer][inner],
+ * scaled by alpha.  The reduce_sum rule is linear and is applied to x, jac and lap alike
+ * (SUMMATION, folx/wrapped_functions.py:388-392; folx/jvp.py:104-106).
+ */
+int folx_hip_reduce_sum(void* stream, const float* in, float* out, int64_t rows,
+                        int64_t outer, int64_t red, int64_t inner, float alpha);
+
+/* max over the middle axis of a value array (no derivatives): [outer][red][inner] ->
+ * [outer][inner].  Used for the stop-gradient shift of logsumexp. */
+int folx_hip_reduce_max(void* stream, const float* in, float* out, int64_t outer,
+                        int64_t red, int64_t inner);
+
+/*
+ * Re-index sparse Jacobian rows into another row frame by a static gather table:
+ *   out[t][b][so][si] = sum_{s < n_slots} ( r = take[(t * n_slots + s) * S_outer + so];
+ *                                           r >= 0 ? data[r][b][so][si] : 0 )
+ * data [k_in][B][S_outer][S_inner], take int32 [k_out][n_slots][S_outer] with values in
+ * [-1, k_in).  Replaces materialize_by_gather (folx/utils.py:71-114) as used by
+ * FwdJacobian.materialize_for_idx (folx/api.py:58-118), get_jacobian_for_reduction
+ * (folx/utils.py:499-588) and sparse_sum_jvp (folx/jvp.py:163-171).
+ */
+int folx_hip_gather_rows(void* stream, const float* data, const int32_t* take, float* out,
+                         int32_t k_in, int32_t k_out, int32_t n_slots, int64_t B,
+                         int64_t S_outer, int64_t S_inner);
+
+/*
+ * Scatter-add form of the same re-indexing (the reference's segment_sum fallback,
+ * folx/api.py:110-114, folx/jvp.py:170-171): out must be zero-filled by the caller;
+ *   out[idx[r][so]][b][so][si] += data[r][b][so][si]   for idx >= 0.
+ * idx int32 [k_in][S_outer] with values in [-1, k_out).
+ */
+int folx_hip_scatter_add_rows(void* stream, const float* data, const int32_t* idx,
+                              float* out, int32_t k_in, int32_t k_out, int64_t B,
+                              int64_t S_outer, int64_t S_inner);
+
+/*
+ * slogdet rule for NM matrices of size n x n (n <= 32) with dense Jacobians.
+ *   A [NM][n][n]   A_jac [P][NM][n][n]   A_lap [NM][n][n]
+ *   sign [NM]   logdet [NM]   ld_jac [P][NM]   ld_lap [NM]
+ * sign/logdet by LU with partial pivoting; M_p = A^-1 A_jac[p]; ld_jac[p] = tr M_p;
+ * ld_lap = tr(A^-1 A_lap) - sum_p tr(M_p M_p).
+ * Replaces _dense_log_det / dense_slogdet (folx/slogdet.py:296-344).
+ */
+int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
+                            const float* A_lap, float* sign, float* logdet, float* ld_jac,
+                            float* ld_lap, int64_t NM, int32_t n, int32_t P);
+
+/*
+ * Multi-head self attention with Laplacian, o = softmax(q k^T) v (no 1/sqrt(d) inside).
+ *   q, k, v, their lap and o, o_lap: [B][n][H][d];  *_jac, o_jac: [P][B][n][H][d]
+ *   mask uint8 [B][n] (1 = real electron) or NULL; input_mask uint8 [P][B]
+ *   (1 = active coordinate) or NULL.
+ * Replaces mhsa_forward_laplacian and its Pallas kernel
+ * (folx/experimental/pallas/attention/forward_laplacian.py:27-179, :349-487).
+ * Supported: n <= 64, d <= 64, d % 4 == 0.
+ */
+int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q_jac, const float* q_lap,
+                         const float* k, const float* k_jac, const float* k_lap,
+                         const float* v, const float* v_jac, const float* v_lap,
+                         const uint8_t* mask, const uint8_t* input_mask, float* o,
+                         float* o_jac, float* o_lap, int64_t B, int32_t n, int32_t H,
+                         int32_t d, int32_t P);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FOLX_HIP_H */

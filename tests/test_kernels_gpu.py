@@ -1,0 +1,274 @@
+"""GPU parity of every C-ABI entry point against the fp64 oracle on the same seeded fp32
+inputs.  All calls go through libfolx_hip.so (folx_amd.kernels -> ctypes)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import index_algebra as ia
+from oracle import rules
+from tolerances import assert_lap, assert_triplet, assert_val
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype).cuda()
+
+
+def f64(*arrs):
+    return [np.asarray(a, dtype=np.float64) for a in arrs]
+
+
+def rand(rng, *shape):
+    return rng.normal(size=shape).astype(np.float32)
+
+
+POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal'}
+ACTS = ['tanh', 'silu', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'softplus', 'sin', 'cos',
+        'abs', 'log1p', 'reciprocal', 'expm1']
+
+
+@pytest.mark.parametrize('name', ACTS)
+@pytest.mark.parametrize('shape,P', [((3, 5, 8), 7), ((2, 13), 1), ((4, 100, 100), 40)])
+def test_elementwise(name, shape, P):
+    from folx_amd import kernels as K
+
+    print(f'case elementwise {name} {shape} P={P}', flush=True)
+    rng = np.random.default_rng(0)
+    x, J, L = rand(rng, *shape), rand(rng, P, *shape), rand(rng, *shape)
+    if name in POSITIVE:
+        x = np.abs(x) + 0.2
+    ref = rules.elementwise_rule(name, *f64(x, J, L))
+    got = K.elementwise(name, dev(x), dev(J), dev(L))
+    assert_triplet(got, ref, name)
+    # in-place use is part of the contract
+    tx, tJ, tL = dev(x), dev(J), dev(L)
+    got2 = K.elementwise(name, tx, tJ, tL, inplace=True)
+    assert got2[0].data_ptr() == tx.data_ptr()
+    assert_triplet(got2, ref, name + ' in-place')
+
+
+@pytest.mark.parametrize('n', [2, 3, -1, -2, 5])
+def test_integer_pow(n):
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(1)
+    x, J, L = np.abs(rand(rng, 6, 9)) + 0.5, rand(rng, 5, 6, 9), rand(rng, 6, 9)
+    ref = rules.elementwise_rule('integer_pow', *f64(x, J, L), n)
+    got = K.elementwise('integer_pow', dev(x), dev(J), dev(L), param=n)
+    assert_triplet(got, ref, f'integer_pow {n}')
+
+
+DENSE_CASES = [
+    # (rows shape, P, K, N, bias)
+    ((20, 100), 8, 4, 100, True),      # first layer of the README MLP (K = 4)
+    ((3, 100), 40, 100, 100, True),    # hidden layer (K = N = 100, not a tile multiple)
+    ((3, 100), 12, 100, 1, False),     # output layer (N = 1)
+    ((5, 32), 9, 256, 256, True),      # PsiFormer width
+    ((2, 7), 3, 17, 33, True),         # odd sizes: scalar load paths
+    ((1, 1), 1, 1, 1, False),
+    ((2, 64), 6, 512, 512, False),     # large-config width
+    ((4, 16), 5, 64, 48, True),        # BN = 64 variant
+]
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,bias', DENSE_CASES)
+def test_dense(rows, P, Kd, N, bias):
+    from folx_amd import kernels as K
+
+    print(f'case dense rows={rows} P={P} K={Kd} N={N}', flush=True)
+    rng = np.random.default_rng(2)
+    x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    ref = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
+    got = K.dense(dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
+    assert_triplet(got, ref, 'dense')
+
+
+def test_dense_linearity_large():
+    """Size-independent property at full PsiFormer row counts: the rule is linear, so
+    f(a h1 + h2) = a f(h1) + f(h2) row by row, and zero rows map to zero."""
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(3)
+    R, P, Kd, N = 4096 * 8, 10, 256, 256
+    g = torch.Generator(device='cuda').manual_seed(0)
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.zeros(R, Kd, device='cuda')
+    W = dev(rand(rng, Kd, N) / 16)
+    y1, J1, L1 = K.dense(x, J, L, W)
+    assert float(L1.abs().max()) == 0.0
+    # rows of J are just more rows of the same GEMM: J1[0] must equal dense(J[0]) as x
+    y2, _, _ = K.dense(J[0].contiguous(), J[:1].contiguous(), L, W)
+    assert torch.equal(y2, J1[0])
+    # against an fp64 product on a row sample
+    idx = torch.randint(0, R, (64,), device='cuda')
+    ref = (x[idx].double() @ W.double()).cpu().numpy()
+    assert_val(y1[idx], ref, 'dense sample')
+
+
+@pytest.mark.parametrize('op', ['mul', 'div', 'add', 'sub'])
+@pytest.mark.parametrize('sa,sb', [((3, 4, 6), (3, 4, 6)), ((3, 4, 6), (3, 4, 1)), ((3, 1, 6), (3, 4, 6)),
+                                   ((2, 5, 1, 7), (2, 1, 3, 7))])
+def test_binary(op, sa, sb):
+    from folx_amd import kernels as K
+
+    print(f'case binary {op} {sa} {sb}', flush=True)
+    rng = np.random.default_rng(4)
+    P = 6
+    a, aj, al = rand(rng, *sa), rand(rng, P, *sa), rand(rng, *sa)
+    b, bj, bl = rand(rng, *sb), rand(rng, P, *sb), rand(rng, *sb)
+    if op == 'div':
+        b = np.abs(b) + 0.5
+    rule = {'mul': rules.mul_rule, 'div': rules.div_rule, 'add': rules.add_rule,
+            'sub': lambda *t: rules.add_rule(*t, sign=-1.0)}[op]
+    A = [np.broadcast_to(t, np.broadcast_shapes(t.shape, u.shape)) for t, u in
+         zip(f64(a, aj, al), f64(b, bj, bl))]
+    Bb = [np.broadcast_to(u, np.broadcast_shapes(t.shape, u.shape)) for t, u in
+          zip(f64(a, aj, al), f64(b, bj, bl))]
+    ref = rule(*A, *Bb)
+    got = K.binary(op, dev(a), dev(aj), dev(al), dev(b), dev(bj), dev(bl))
+    assert_triplet(got, ref, op)
+
+
+def test_rows_affine():
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(5)
+    rows, shape = 5, (3, 4, 6)
+    inp = rand(rng, rows, *shape)
+    c, d = rand(rng, 3, 1, 6), rand(rng, 1, 4, 1)
+    got = K.rows_affine(dev(inp), rows, shape, shape, dev(c), dev(d), alpha=0.5, beta=-2.0)
+    assert_val(got, 0.5 * inp.astype(np.float64) * c + (-2.0) * d)
+    got = K.rows_affine(dev(inp[:, :, :1]), rows, (3, 1, 6), shape, None, None, alpha=-1.0)
+    assert_val(got, -np.broadcast_to(inp[:, :, :1], (rows, *shape)))
+
+
+@pytest.mark.parametrize('outer,red,inner', [(7, 5, 9), (6, 100, 1), (3, 4, 1), (1, 33, 70)])
+def test_reduce(outer, red, inner):
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(6)
+    rows = 4
+    inp = rand(rng, rows, outer, red, inner)
+    got = K.reduce_sum(dev(inp), rows, outer, red, inner, alpha=0.25)
+    assert_val(got, 0.25 * inp.astype(np.float64).sum(2))
+    got = K.reduce_max(dev(inp[0]), outer, red, inner)
+    assert_val(got, inp[0].max(1))
+
+
+def test_gather_and_scatter_rows():
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(7)
+    k_in, B, So, Si, k_out = 3, 4, 5, 6, 7
+    mask = rng.integers(-1, k_out, size=(k_in, So))
+    data = rand(rng, k_in, B, So, Si)
+    ref = ia.materialize(data.astype(np.float64), np.broadcast_to(mask[:, :, None], (k_in, So, Si)), k_out)
+    # static gather table: slot s of (t, so) = s-th row r with mask[r, so] == t
+    n_slots = max(1, int(max((mask[:, so] == t).sum() for so in range(So) for t in range(k_out))))
+    take = np.full((k_out, n_slots, So), -1, dtype=np.int32)
+    for so in range(So):
+        for t in range(k_out):
+            rows = np.nonzero(mask[:, so] == t)[0]
+            take[t, : len(rows), so] = rows
+    got = K.gather_rows(dev(data).reshape(k_in, B, So * Si), dev(take, torch.int32), k_out, n_slots, B, So, Si)
+    assert_val(got.reshape(k_out, B, So, Si), ref)
+    got = K.scatter_add_rows(dev(data).reshape(k_in, B, So * Si), dev(mask, torch.int32), k_out, B, So, Si)
+    assert_val(got.reshape(k_out, B, So, Si), ref)
+
+
+@pytest.mark.parametrize('n,P,lead', [(1, 3, (4,)), (2, 5, (3, 2)), (5, 7, (6,)), (8, 24, (4, 3)),
+                                      (16, 96, (5, 4)), (32, 20, (3, 2)), (11, 4, (7,))])
+def test_slogdet(n, P, lead):
+    from folx_amd import kernels as K
+
+    print(f'case slogdet n={n} P={P} lead={lead}', flush=True)
+    rng = np.random.default_rng(8)
+    A = rand(rng, *lead, n, n)
+    J = rand(rng, P, *lead, n, n)
+    L = rand(rng, *lead, n, n)
+    sign, (ld, jac, lap) = rules.slogdet_rule(*f64(A, J, L))
+    gs, gld, gj, gl = K.slogdet(dev(A), dev(J), dev(L))
+    np.testing.assert_array_equal(gs.cpu().numpy(), sign)
+    # A^-1 amplifies rounding by the condition number: scale the bar with it
+    cond = float(np.linalg.cond(A.astype(np.float64)).max())
+    amp = max(1.0, cond / 50)
+    np.testing.assert_allclose(gld.cpu().numpy(), ld, rtol=1e-5 * amp, atol=1e-6 * amp)
+    sc = float(np.abs(jac).max())
+    np.testing.assert_allclose(gj.cpu().numpy(), jac, rtol=1e-5 * amp, atol=2e-6 * amp * sc)
+    sl = float(np.abs(lap).max())
+    np.testing.assert_allclose(gl.cpu().numpy(), lap, rtol=1e-4 * amp, atol=1e-5 * amp * sl)
+
+
+def test_slogdet_closed_forms_gpu():
+    """Well-conditioned closed forms at the strict bar: diagonal matrices and a row swap."""
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(9)
+    B, n, P = 64, 16, 12
+    a = (rng.uniform(0.5, 2.0, size=(B, n)) * rng.choice([-1, 1], size=(B, n))).astype(np.float32)
+    A = np.zeros((B, n, n), np.float32)
+    A[:, range(n), range(n)] = a
+    Jd = rand(rng, P, B, n)
+    J = np.zeros((P, B, n, n), np.float32)
+    J[:, :, range(n), range(n)] = Jd
+    Ld = rand(rng, B, n)
+    L = np.zeros((B, n, n), np.float32)
+    L[:, range(n), range(n)] = Ld
+    perm = rng.permutation(n)
+    gs, gld, gj, gl = K.slogdet(dev(A[:, perm]), dev(J[:, :, perm]), dev(L[:, perm]))
+    a64, Jd64, Ld64 = f64(a, Jd, Ld)
+    from math import prod  # noqa: F401
+
+    # sign of the permutation
+    inv = sum(1 for i in range(n) for j in range(i + 1, n) if perm[i] > perm[j])
+    psign = -1.0 if inv % 2 else 1.0
+    np.testing.assert_array_equal(gs.cpu().numpy(), psign * np.prod(np.sign(a64), -1))
+    assert_val(gld, np.log(np.abs(a64)).sum(-1), 'logdet')
+    assert_val(gj, (Jd64 / a64[None]).sum(-1), 'jac')
+    assert_lap(gl, (Ld64 / a64).sum(-1) - ((Jd64 / a64[None]) ** 2).sum((0, -1)), 'lap')
+
+
+MHSA_CASES = [
+    # B, n, H, d, P, valid electrons (None = all)
+    (2, 1, 1, 4, 3, None),
+    (1, 16, 4, 32, 48, None),    # shape of test_attention.py:320-326
+    (1, 16, 4, 32, 48, 4),       # padded sequence (max_sequence = 4)
+    (3, 32, 4, 64, 12, None),    # PsiFormer-style tile
+    (2, 20, 2, 24, 9, 13),       # sizes that are no multiple of 16
+    (1, 64, 2, 64, 6, None),     # large-config tile
+]
+
+
+@pytest.mark.parametrize('B,n,H,d,P,valid', MHSA_CASES)
+def test_mhsa(B, n, H, d, P, valid):
+    from folx_amd import kernels as K
+
+    print(f'case mhsa B={B} n={n} H={H} d={d} P={P} valid={valid}', flush=True)
+    rng = np.random.default_rng(10)
+    sig = [1 / np.sqrt(d), 1.0, 1.0]  # q pre-scaled by the caller (test_attention.py:38)
+    args = []
+    for s in sig:
+        args += [s * rand(rng, B, n, H, d), s * rand(rng, P, B, n, H, d), s * rand(rng, B, n, H, d)]
+    mask = np.ones((B, n), dtype=bool)
+    imask = np.ones((P, B), dtype=bool)
+    if valid is not None:
+        mask[:, valid:] = False
+        imask[min(P, 3 * valid):] = False
+    ref = rules.mhsa_rule(*f64(*args), mask, imask)
+    got = K.mhsa(*[dev(t) for t in args], dev(mask, torch.uint8), dev(imask, torch.uint8))
+    m = mask[0]
+    # rows of padding queries carry no meaning (the reference masks them before comparing)
+    assert_val(got[0][:, m], ref[0][:, m], 'o')
+    assert_val(got[1][:, :, m], ref[1][:, :, m], 'o_jac')
+    assert_lap(got[2][:, m], ref[2][:, m], 'o_lap')
+    for t in got:
+        assert torch.isfinite(t).all()
+    if valid is None:
+        got2 = K.mhsa(*[dev(t) for t in args], None, None)
+        for g1, g2 in zip(got, got2):
+            assert torch.equal(g1, g2)
