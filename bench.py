@@ -1,0 +1,170 @@
+"""Benchmark of the forward-Laplacian hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload psiformer32]
+
+A step is one full forward Laplacian (value, 96-row Jacobian, Laplacian per walker) of the
+PsiFormer-style 32-electron wavefunction over a batch of 4096 synthetic walkers that are
+resident in HBM before the timed region starts.  Prints ONE JSON line with walkers/s, the
+roofline of the dominant kernel (per-launch durations taken with HIP events on the launch
+stream inside the timed region) and the CPU baseline (the numpy oracle on a bounded
+sample of the same workload, timed on this host).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense FP32 matrix peak
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=5)
+    ap.add_argument('--warmup', type=int, default=2)
+    ap.add_argument('--workload', default='psiformer32')
+    ap.add_argument('--walkers', type=int, default=0, help='override the batch (0 = the configuration default)')
+    ap.add_argument('--chunk', type=int, default=1024, help='walkers per batched_vmap chunk')
+    ap.add_argument('--cpu-seconds', type=float, default=20.0, help='budget of the CPU baseline sample')
+    ap.add_argument('--no-cpu', action='store_true')
+    return ap.parse_args()
+
+
+def cpu_baseline(workload, budget_s):
+    """The numpy oracle (fp32, dense Jacobians) on a bounded sample of the same workload."""
+    from oracle import backend as ob
+
+    from folx_amd import workloads as wl
+
+    cfg, _, sigma, _ = wl.CONFIGS[workload]
+    p = wl.psiformer_params(cfg)
+    try:
+        from threadpoolctl import threadpool_info
+
+        threads = max([i.get('num_threads', 1) for i in threadpool_info()] or [1])
+    except Exception:
+        threads = 1
+
+    def run(n):
+        x = wl.sample_electrons(n, cfg.n_elec, sigma, seed=2)
+        t0 = time.perf_counter()
+        out = wl.psiformer_forward(p, ob.init_state(x, dtype=np.float32), ob)
+        dt = time.perf_counter() - t0
+        assert np.isfinite(out.lap).all()
+        return dt
+
+    t1 = run(1)
+    n = int(max(1, min(16, budget_s / max(t1, 1e-3))))
+    dt = run(n) if n > 1 else t1
+    return {
+        'value': n / dt,
+        'unit': 'walkers/s',
+        'cores': threads,
+        'kind': 'port',
+        'sample': f'{n} walkers of {workload}, numpy fp32 oracle with dense Jacobians, {dt:.1f} s',
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py measures one GPU: walkers are independent, every GPU would run this same '
+              'path on its share of the batch; run with --gpus 1', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import folx_amd
+    from folx_amd import kernels as K
+    from folx_amd import workloads as wl
+
+    cfg, B, sigma, thr = wl.CONFIGS[args.workload]
+    if args.walkers:
+        B = args.walkers
+    dev = torch.device('cuda', 0)
+    torch.cuda.set_device(dev)
+    params = wl.to_device(wl.psiformer_params(cfg), dev)
+    x = torch.as_tensor(wl.sample_electrons(B, cfg.n_elec, sigma, seed=2)).to(dev)
+    fl = folx_amd.forward_laplacian(lambda r: wl.psiformer_forward(params, r), thr)
+    step = folx_amd.batched_vmap(fl, args.chunk)
+
+    for _ in range(args.warmup):
+        out = step(x)
+    torch.cuda.synchronize()
+
+    with K.LaunchTimer() as lt:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = step(x)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    assert torch.isfinite(out.x).all() and torch.isfinite(out.laplacian).all()
+    ms_per_step = 1e3 * dt / args.steps
+    value = B * args.steps / dt
+
+    # dominant kernel: the launch shape with the largest total time inside the timed region
+    summ = lt.summary()
+    per_kernel = {}
+    for (name, key), (n, ms) in summ.items():
+        per_kernel[name] = per_kernel.get(name, 0.0) + ms
+    (dname, dkey), (dn, dms) = max(summ.items(), key=lambda kv: kv[1][1])
+    roof = None
+    if dname == 'dense_fwdlap':
+        R, P, Kd, N = dkey
+        flops = 2.0 * (P + 2) * R * Kd * N
+        achieved = flops / (dms / dn * 1e-3) / 1e12
+        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
+                'kernel': f'dense_kernel R={R} P={P} K={Kd} N={N}', 'launches': dn,
+                'avg_launch_ms': dms / dn}
+    elif dname == 'mhsa_fwdlap':
+        Bc, n, H, d, P = dkey
+        flops = (7.0 * P + 6) * 2 * n * n * d * Bc * H
+        achieved = flops / (dms / dn * 1e-3) / 1e12
+        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
+                'kernel': f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}', 'launches': dn,
+                'avg_launch_ms': dms / dn}
+    else:
+        roof = {'bound': 'hbm', 'achieved': None, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': None,
+                'traffic': None, 'kernel': f'{dname} {dkey}', 'launches': dn, 'avg_launch_ms': dms / dn}
+
+    line = {
+        'metric': 'walkers/s of full forward Laplacian at 1 GPU',
+        'value': value,
+        'unit': 'walkers/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': ms_per_step,
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'f32',
+        'data': 'synthetic',
+        'config': {
+            'workload': f'{args.workload}: PsiFormer-style, {cfg.n_elec} electrons, {cfg.n_nuc} nuclei, '
+                        f'{cfg.n_layers} layers x {cfg.n_heads} heads x {cfg.head_dim}, width {cfg.width}, '
+                        f'{cfg.n_det} determinants, ForwardLaplacianOperator({thr})',
+            'walkers': B,
+            'chunk': args.chunk,
+            'jacobian_rows': 3 * cfg.n_elec,
+        },
+        'roofline': roof,
+        'kernel_ms_per_step': {k: v / args.steps for k, v in sorted(per_kernel.items(), key=lambda kv: -kv[1])},
+    }
+    if not args.no_cpu:
+        line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds)
+    print(json.dumps(line))
+
+
+if __name__ == '__main__':
+    main()

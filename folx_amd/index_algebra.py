@@ -1,0 +1,247 @@
+"""Static sparsity algebra on the host (numpy, integers only).
+
+Sparse Jacobians carry a compile-time mask ``x0_idx (k, *shape)``; every rule has to say
+what the mask of its output is and how input rows map to output rows.  The functions here
+compute those maps, vectorised over positions, and turn them into the small int32 tables
+the gather kernel consumes.  They mirror the reference's host-side helpers; each cites the
+lines it follows.  Nothing here touches the GPU.
+"""
+
+from __future__ import annotations
+
+from typing import Sequence
+
+import numpy as np
+
+INT = np.int64
+
+
+# --------------------------------------------------------------------------------------
+# small helpers
+# --------------------------------------------------------------------------------------
+
+
+def init_mask(shape) -> np.ndarray:
+    """Initial sparse mask: one row, entry i <- flat input i (folx/interpreter.py:283-293)."""
+    n = int(np.prod(shape, dtype=int))
+    return np.arange(n, dtype=np.int32).reshape(1, *shape)
+
+
+def has_duplicates(mask: np.ndarray | None) -> bool:
+    """True iff a position lists a valid index twice (folx/hessian.py:71-84)."""
+    if mask is None or mask.shape[0] <= 1:
+        return False
+    s = np.sort(mask, axis=0)
+    return bool(((s[1:] == s[:-1]) & (s[:-1] >= 0)).any())
+
+
+def split_inner(idx: np.ndarray) -> int:
+    """Number of trailing position axes along which ``idx (k, *s)`` is constant.  Tables
+    are stored without those axes, so consecutive threads share one table entry."""
+    n_inner = 0
+    for ax in range(idx.ndim - 1, 0, -1):
+        first = np.take(idx, [0], axis=ax)
+        if idx.shape[ax] == 1 or (idx == first).all():
+            idx = first
+            n_inner += 1
+        else:
+            break
+    return n_inner
+
+
+def per_position_sorted_unique(arr: np.ndarray) -> np.ndarray:
+    """Sorted unique non-negative values along the last axis, ``-1`` padded at the end;
+    width = the largest per-position count (folx/hessian.py:234-258)."""
+    lead = arr.shape[:-1]
+    if arr.shape[-1] == 0:
+        return np.full((*lead, 0), -1, dtype=arr.dtype)
+    s = np.sort(arr, axis=-1)
+    prev = np.concatenate([np.full((*lead, 1), -2, dtype=arr.dtype), s[..., :-1]], axis=-1)
+    first = (s != prev) & (s >= 0)
+    big = np.iinfo(arr.dtype).max
+    packed = np.sort(np.where(first, s, big), axis=-1)
+    width = int(first.sum(-1).max()) if first.size else 0
+    out = packed[..., :width]
+    return np.where(out == big, -1, out)
+
+
+def per_position_intersection(masks: Sequence[np.ndarray]) -> np.ndarray:
+    """Values present in every operand's set, per position (folx/hessian.py:261-285)."""
+    n = len(masks)
+    per = [per_position_sorted_unique(m) for m in masks]
+    comb = np.concatenate(per, axis=-1)
+    lead, total = comb.shape[:-1], comb.shape[-1]
+    if total < n:
+        return np.full((*lead, 0), -1, dtype=comb.dtype)
+    s = np.sort(comb, axis=-1)
+    first, last = s[..., : total - n + 1], s[..., n - 1 :]
+    hit = (first == last) & (first >= 0)
+    big = np.iinfo(comb.dtype).max
+    packed = np.sort(np.where(hit, first, big), axis=-1)
+    width = int(hit.sum(-1).max()) if hit.size else 0
+    out = packed[..., :width]
+    return np.where(out == big, -1, out)
+
+
+# --------------------------------------------------------------------------------------
+# row re-indexing
+# --------------------------------------------------------------------------------------
+
+
+def get_index_mask(mask: np.ndarray, outputs: np.ndarray) -> np.ndarray:
+    """Slot of ``outputs`` (axis 0) holding the same input index as each sparse entry, or
+    ``-1``; first match wins (folx/api.py:120-159)."""
+    s = np.broadcast_shapes(mask.shape[1:], outputs.shape[1:])
+    m = np.broadcast_to(mask, (mask.shape[0], *s))
+    o = np.broadcast_to(outputs, (outputs.shape[0], *s))
+    match = m[:, None] == o[None]  # (k, T, *s)
+    idx = match.argmax(1)
+    return np.where(match.any(1), idx, -1).astype(INT)
+
+
+def gather_table(idx: np.ndarray, n_out: int):
+    """Static gather table of ``materialize_by_gather`` (folx/utils.py:71-114).
+
+    idx (k, *s): target row of every source entry, ``-1`` = none.
+    Returns ``take (n_out, n_slots, *s)`` int32: the source rows summed into target row t
+    at each position, ``-1`` padded; sources keep their original order within a target
+    (stable sort), which fixes the floating-point summation order.
+    """
+    k = idx.shape[0]
+    s = idx.shape[1:]
+    S = int(np.prod(s, dtype=int))
+    flat = idx.reshape(k, S).T  # (S, k)
+    if k == 0 or S == 0:
+        return np.full((n_out, 1, *s), -1, dtype=np.int32)
+    order = np.argsort(flat, axis=1, kind='stable')
+    st = np.take_along_axis(flat, order, axis=1)
+    first = np.concatenate([np.ones((S, 1), dtype=bool), st[:, 1:] != st[:, :-1]], axis=1)
+    ar = np.arange(k)[None, :]
+    run_start = np.maximum.accumulate(np.where(first, ar, 0), axis=1)
+    slot = ar - run_start
+    valid = st >= 0
+    n_slots = int(slot[valid].max()) + 1 if valid.any() else 1
+    take = np.full((S, n_out, n_slots), -1, dtype=np.int32)
+    pos = np.broadcast_to(np.arange(S)[:, None], (S, k))
+    take[pos[valid], st[valid], slot[valid]] = order[valid]
+    return np.ascontiguousarray(np.moveaxis(take, 0, -1)).reshape(n_out, n_slots, *s)
+
+
+def reduction_frame(masks: Sequence[np.ndarray], axes) -> np.ndarray:
+    """Index part of ``get_jacobian_for_reduction`` (folx/utils.py:499-588): per kept
+    position, the ascending union of valid indices over all operands, rows and reduced
+    axes, ``-1`` padded at the END.  Returns ``(m, *kept_shape)``."""
+    s = np.broadcast_shapes(*[m.shape[1:] for m in masks])
+    nd = len(s)
+    axes = tuple(sorted(a % nd for a in np.atleast_1d(axes)))
+    kept = [a for a in range(nd) if a not in axes]
+    cols = []
+    for m in masks:
+        m = np.broadcast_to(m, (m.shape[0], *s))
+        m = np.transpose(m, [a + 1 for a in kept] + [0] + [a + 1 for a in axes])
+        cols.append(m.reshape(*[s[a] for a in kept], -1))
+    allv = np.concatenate(cols, axis=-1).astype(INT)
+    out = per_position_sorted_unique(allv)
+    return np.moveaxis(out, -1, 0)
+
+
+def sum_out_mask(mask: np.ndarray, axes):
+    """Index part of ``sparse_sum_jvp`` (folx/jvp.py:108-146).
+
+    Per output position the distinct values over rows and reduced axes, ascending, with
+    ``-1`` treated as a value (so it sorts FIRST, :116-126), ``-1`` filled at the end.
+    Returns ``(idx_out (m, *kept), slot (k, *s))``; ``slot`` is the output row each input
+    entry is summed into (first match, :144).
+    """
+    k, *s = mask.shape
+    nd = len(s)
+    axes = tuple(sorted(a % nd for a in np.atleast_1d(axes)))
+    kept = [a for a in range(nd) if a not in axes]
+    perm = [a + 1 for a in kept] + [0] + [a + 1 for a in axes]
+    m = np.transpose(mask, perm).astype(INT)
+    kept_shape = [s[a] for a in kept]
+    flat = m.reshape(*kept_shape, -1)  # (*kept, k * red)
+    srt = np.sort(flat, axis=-1)
+    prev = np.concatenate(
+        [np.full((*kept_shape, 1), np.iinfo(INT).min, dtype=INT), srt[..., :-1]], axis=-1
+    )
+    first = srt != prev
+    width = int(first.sum(-1).max())
+    big = np.iinfo(INT).max
+    packed = np.sort(np.where(first, srt, big), axis=-1)[..., :width]
+    idx_out = np.where(packed == big, -1, packed)  # (*kept, width)
+    match = flat[..., :, None] == idx_out[..., None, :]  # (*kept, k*red, width)
+    slot_flat = match.argmax(-1)
+    slot = slot_flat.reshape(*kept_shape, k, *[s[a] for a in axes])
+    slot = np.transpose(slot, np.argsort(perm))
+    return np.moveaxis(idx_out, -1, 0), slot
+
+
+def merge_rows(masks: Sequence[np.ndarray]):
+    """Row merge of a multi-operand elementwise op (folx/jvp.py:294-317): broadcast and
+    concatenate the masks along the row axis, merge identical rows with
+    ``np.unique(axis=0)``.  Returns ``(result_mask, inverse)``."""
+    s = np.broadcast_shapes(*[m.shape[1:] for m in masks])
+    cat = np.concatenate([np.broadcast_to(m, (m.shape[0], *s)) for m in masks], axis=0)
+    res, inv = np.unique(cat, axis=0, return_inverse=True)
+    return res, np.asarray(inv).reshape(-1)
+
+
+def find_out_idx(masks, x_shapes, in_axes, linear_in_one: bool, threshold: int):
+    """``hessian.find_out_idx`` (folx/hessian.py:288-340).
+
+    masks[i] is ``(k_i, *x_shapes[i])`` (pass ``FwdJacobian.mask`` for dense operands) or
+    None for all-dense calls.  ``in_axes[i]`` are the axes operand i is consumed along.
+    The position frame is the broadcast of the operands' remaining axes with the axes that
+    have size 1 in every operand dropped (folx/utils.py:271-327).  Returns
+    ``(idx (M, *frame), dense_out)``.
+    """
+    if all(m is None for m in masks):
+        return None, True
+    n_args = len(masks)
+    pos_shapes, perms = [], []
+    for m, xs, ax in zip(masks, x_shapes, in_axes):
+        nd = len(xs)
+        axn = tuple(a % nd for a in ax) if nd else ()
+        mapped = [a for a in range(nd) if a not in axn]
+        pos_shapes.append([xs[a] for a in mapped])
+        perms.append((mapped, [a for a in range(nd) if a in axn]))
+    nfr = max(len(p) for p in pos_shapes)
+    padded = [[1] * (nfr - len(p)) + list(p) for p in pos_shapes]
+    keep = [d for d in range(nfr) if any(p[d] != 1 for p in padded)]
+    frame = [max(p[d] for p in padded) for d in keep]
+
+    aligned = []
+    for m, xs, (mapped, red), pp in zip(masks, x_shapes, perms, padded):
+        m = np.asarray(m).astype(INT)
+        # (mapped axes..., row axis, consumed axes...) -> (*padded frame, K_flat)
+        t = np.transpose(m, [a + 1 for a in mapped] + [0] + [a + 1 for a in red])
+        t = t.reshape(*pp, -1)
+        t = t.reshape(*[pp[d] for d in keep], t.shape[-1])  # dropped dims have size 1
+        aligned.append(np.broadcast_to(t, (*frame, t.shape[-1])))
+
+    max_size = max(int((np.unique(np.asarray(m)) >= 0).sum()) for m in masks)
+    if linear_in_one:
+        idx = per_position_intersection(aligned)
+    else:
+        idx = per_position_sorted_unique(np.concatenate(aligned, axis=-1))
+    idx = np.moveaxis(idx, -1, 0)
+    dense_out = bool(idx.shape[0] >= max_size or idx.shape[0] > threshold)
+    return idx, dense_out
+
+
+def dot_projection(mask: np.ndarray, contract_axis: int, threshold: int):
+    """Mask of ``h @ W`` for sparse ``h`` with one contracted axis
+    (folx/wrapped_functions.py:113-157).  Returns ``(proj, aligned)``: ``proj`` is
+    ``(k', *s_without_contract, 1)`` -- rows unchanged when the mask is constant along the
+    contracted axis (:131-133), else the union frame (``aligned`` True), or None when
+    that union exceeds the threshold (:129-130)."""
+    nd = mask.ndim - 1
+    ca = contract_axis % nd
+    first = np.take(mask, [0], axis=ca + 1)
+    if (mask == first).all():
+        return np.take(mask, 0, axis=ca + 1)[..., None], False
+    proj = reduction_frame([mask], (ca,))
+    if proj.shape[0] > threshold:
+        return None, True
+    return proj[..., None], True

@@ -20,6 +20,56 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+class LaunchTimer:
+    """Optional per-launch timing with HIP events recorded on the launch stream.
+
+        with LaunchTimer() as lt:
+            ...                       # kernels.dense / kernels.mhsa / ... calls
+        lt.summary()                  # {(kernel, key): (launches, total_ms)}
+
+    Events bracket each launch on the stream it is issued to, so the elapsed time is the
+    kernel's own duration (plus launch gaps of a few microseconds)."""
+
+    active = None
+
+    def __init__(self):
+        self.records = []
+
+    def __enter__(self):
+        LaunchTimer.active = self
+        return self
+
+    def __exit__(self, *exc):
+        LaunchTimer.active = None
+
+    def summary(self):
+        torch.cuda.synchronize()
+        out = {}
+        for name, key, e0, e1 in self.records:
+            n, ms = out.get((name, key), (0, 0.0))
+            out[(name, key)] = (n + 1, ms + e0.elapsed_time(e1))
+        return out
+
+
+class _timed:
+    __slots__ = ('name', 'key', 'e0')
+
+    def __init__(self, name, key):
+        self.name, self.key = name, key
+
+    def __enter__(self):
+        if LaunchTimer.active is not None:
+            self.e0 = torch.cuda.Event(enable_timing=True)
+            self.e0.record()
+
+    def __exit__(self, *exc):
+        lt = LaunchTimer.active
+        if lt is not None:
+            e1 = torch.cuda.Event(enable_timing=True)
+            e1.record()
+            lt.records.append((self.name, self.key, self.e0, e1))
+
+
 def _p(t):
     if t is None:
         return None
@@ -51,12 +101,13 @@ def dense(x, jac, lap, W, bias=None):
     y = torch.empty((*x.shape[:-1], N), device=x.device, dtype=torch.float32)
     yj = torch.empty((P, *x.shape[:-1], N), device=x.device, dtype=torch.float32)
     yl = torch.empty_like(y)
-    check(
-        _lib.load().folx_hip_dense_fwdlap(
-            _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(y), _p(yj), _p(yl), R, P, K, N
-        ),
-        'dense_fwdlap',
-    )
+    with _timed('dense_fwdlap', (R, P, K, N)):
+        check(
+            _lib.load().folx_hip_dense_fwdlap(
+                _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(y), _p(yj), _p(yl), R, P, K, N
+            ),
+            'dense_fwdlap',
+        )
     return y, yj, yl
 
 
@@ -68,12 +119,13 @@ def elementwise(name, x, jac, lap, param=0.0, inplace=False):
         y, yj, yl = x, jac, lap
     else:
         y, yj, yl = torch.empty_like(x), torch.empty_like(jac), torch.empty_like(lap)
-    check(
-        _lib.load().folx_hip_elementwise_fwdlap(
-            _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(y), _p(yj), _p(yl), S, P
-        ),
-        f'elementwise_fwdlap[{name}]',
-    )
+    with _timed('elementwise_fwdlap', (name, S, P)):
+        check(
+            _lib.load().folx_hip_elementwise_fwdlap(
+                _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(y), _p(yj), _p(yl), S, P
+            ),
+            f'elementwise_fwdlap[{name}]',
+        )
     return y, yj, yl
 
 
@@ -125,13 +177,14 @@ def binary(op, a, aj, al, b, bj, bl):
     y = torch.empty(out_shape, device=a.device, dtype=torch.float32)
     yj = torch.empty((P, *out_shape), device=a.device, dtype=torch.float32)
     yl = torch.empty_like(y)
-    check(
-        _lib.load().folx_hip_binary_fwdlap(
-            _stream(), BINOP[op], _p(a), _p(aj), _p(al), _p(b), _p(bj), _p(bl), _p(y), _p(yj), _p(yl),
-            _dims(*n, *sa, *sb), a.numel(), b.numel(), P,
-        ),
-        f'binary_fwdlap[{op}]',
-    )
+    with _timed('binary_fwdlap', (op, int(y.numel()), P)):
+        check(
+            _lib.load().folx_hip_binary_fwdlap(
+                _stream(), BINOP[op], _p(a), _p(aj), _p(al), _p(b), _p(bj), _p(bl), _p(y), _p(yj), _p(yl),
+                _dims(*n, *sa, *sb), a.numel(), b.numel(), P,
+            ),
+            f'binary_fwdlap[{op}]',
+        )
     return y, yj, yl
 
 
@@ -149,23 +202,25 @@ def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta
     n, (s_in, s_c, s_d) = col
     out = torch.empty((rows, *out_shape), device=inp.device, dtype=torch.float32)
     in_S = int(np.prod(row_shape, dtype=np.int64))
-    check(
-        _lib.load().folx_hip_rows_affine(
-            _stream(), _p(inp), _p(out), rows, in_S, _p(c), _p(d), float(alpha), float(beta),
-            _dims(*n, *s_in, *s_c, *s_d),
-        ),
-        'rows_affine',
-    )
+    with _timed('rows_affine', (rows, int(np.prod(out_shape, dtype=np.int64)))):
+        check(
+            _lib.load().folx_hip_rows_affine(
+                _stream(), _p(inp), _p(out), rows, in_S, _p(c), _p(d), float(alpha), float(beta),
+                _dims(*n, *s_in, *s_c, *s_d),
+            ),
+            'rows_affine',
+        )
     return out
 
 
 def reduce_sum(inp, rows, outer, red, inner, alpha=1.0):
     _chk(inp)
     out = torch.empty((rows, outer, inner), device=inp.device, dtype=torch.float32)
-    check(
-        _lib.load().folx_hip_reduce_sum(_stream(), _p(inp), _p(out), rows, outer, red, inner, float(alpha)),
-        'reduce_sum',
-    )
+    with _timed('reduce_sum', (rows, outer, red, inner)):
+        check(
+            _lib.load().folx_hip_reduce_sum(_stream(), _p(inp), _p(out), rows, outer, red, inner, float(alpha)),
+            'reduce_sum',
+        )
     return out
 
 
@@ -181,12 +236,13 @@ def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
     _chk(data, take)
     k_in = data.shape[0]
     out = torch.empty((k_out, B, S_outer * S_inner), device=data.device, dtype=torch.float32)
-    check(
-        _lib.load().folx_hip_gather_rows(
-            _stream(), _p(data), _p(take), _p(out), k_in, k_out, n_slots, B, S_outer, S_inner
-        ),
-        'gather_rows',
-    )
+    with _timed('gather_rows', (k_in, k_out, n_slots, B, S_outer, S_inner)):
+        check(
+            _lib.load().folx_hip_gather_rows(
+                _stream(), _p(data), _p(take), _p(out), k_in, k_out, n_slots, B, S_outer, S_inner
+            ),
+            'gather_rows',
+        )
     return out
 
 
@@ -214,12 +270,13 @@ def slogdet(A, AJ, AL):
     ld = torch.empty_like(sign)
     ldj = torch.empty((P, *lead), device=A.device, dtype=torch.float32)
     ldl = torch.empty_like(sign)
-    check(
-        _lib.load().folx_hip_slogdet_fwdlap(
-            _stream(), _p(A), _p(AJ), _p(AL), _p(sign), _p(ld), _p(ldj), _p(ldl), NM, n, P
-        ),
-        'slogdet_fwdlap',
-    )
+    with _timed('slogdet_fwdlap', (NM, n, P)):
+        check(
+            _lib.load().folx_hip_slogdet_fwdlap(
+                _stream(), _p(A), _p(AJ), _p(AL), _p(sign), _p(ld), _p(ldj), _p(ldl), NM, n, P
+            ),
+            'slogdet_fwdlap',
+        )
     return sign, ld, ldj, ldl
 
 
@@ -229,11 +286,12 @@ def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None):
     B, n, H, d = q.shape
     P = qj.shape[0]
     o, oj, ol = torch.empty_like(q), torch.empty_like(qj), torch.empty_like(q)
-    check(
-        _lib.load().folx_hip_mhsa_fwdlap(
-            _stream(), _p(q), _p(qj), _p(ql), _p(k), _p(kj), _p(kl), _p(v), _p(vj), _p(vl),
-            _p(mask), _p(input_mask), _p(o), _p(oj), _p(ol), B, n, H, d, P,
-        ),
-        'mhsa_fwdlap',
-    )
+    with _timed('mhsa_fwdlap', (B, n, H, d, P)):
+        check(
+            _lib.load().folx_hip_mhsa_fwdlap(
+                _stream(), _p(q), _p(qj), _p(ql), _p(k), _p(kj), _p(kl), _p(v), _p(vj), _p(vl),
+                _p(mask), _p(input_mask), _p(o), _p(oj), _p(ol), B, n, H, d, P,
+            ),
+            'mhsa_fwdlap',
+        )
     return o, oj, ol

@@ -1,0 +1,197 @@
+"""``jax.numpy``-shaped front end: the functions a model calls, each dispatched through the
+rule registry under the primitive name the reference uses.
+
+The reference traces ``jnp`` code into a jaxpr and interprets it (folx/interpreter.py:
+127-264); here the same dispatch happens define-by-run: every function below looks up
+``get_laplacian(<primitive>)`` and calls the rule with ``(args, kwargs,
+sparsity_threshold)``.  Shapes and axes are per walker, as inside ``jax.vmap``.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import threading
+
+import numpy as np
+
+from .api import BatchedArray, FwdLaplArray
+from .wrapped_functions import get_laplacian
+
+_state = threading.local()
+
+
+def current_threshold() -> int:
+    return getattr(_state, 'threshold', 0)
+
+
+@contextlib.contextmanager
+def sparsity_threshold(value: int):
+    old = current_threshold()
+    _state.threshold = int(value)
+    try:
+        yield
+    finally:
+        _state.threshold = old
+
+
+def _call(name, args, kwargs=None):
+    return get_laplacian(name, wrap_if_missing=True)(tuple(args), kwargs or {}, current_threshold())
+
+
+def _shape(a):
+    if isinstance(a, (FwdLaplArray, BatchedArray)):
+        return tuple(a.shape)
+    return tuple(np.shape(a))
+
+
+# elementwise -------------------------------------------------------------------------------
+def _u(name):
+    def fn(a):
+        return _call(name, (a,))
+
+    fn.__name__ = name
+    return fn
+
+
+tanh, exp, log, sqrt, rsqrt, square = _u('tanh'), _u('exp'), _u('log'), _u('sqrt'), _u('rsqrt'), _u('square')
+sin, cos, abs, log1p, expm1 = _u('sin'), _u('cos'), _u('abs'), _u('log1p'), _u('expm1')
+silu, softplus, sigmoid, logistic = _u('silu'), _u('softplus'), _u('sigmoid'), _u('logistic')
+reciprocal, negative, sign, stop_gradient = _u('reciprocal'), _u('neg'), _u('sign'), _u('stop_gradient')
+
+
+def integer_pow(a, n: int):
+    return _call('integer_pow', (a,), {'y': int(n)})
+
+
+def add(a, b):
+    return _call('add', (a, b))
+
+
+def subtract(a, b):
+    return _call('sub', (a, b))
+
+
+def multiply(a, b):
+    return _call('mul', (a, b))
+
+
+def divide(a, b):
+    return _call('div', (a, b))
+
+
+# linear algebra ----------------------------------------------------------------------------
+def dot(h, W, b=None):
+    """``h @ W (+ b)``: last axis of ``h`` against the first axis of the constant ``W``."""
+    return _call('dot_general', (h, W), {'bias': b})
+
+
+def slogdet(A):
+    return _call('slogdet', (A,))
+
+
+def multi_head_self_attention(q, k, v, mask=None, input_mask=None, **kwargs):
+    """softmax(q k^T) v over per-walker arrays (n, H, d); no 1/sqrt(d) inside.  Same
+    registry key as the reference's jitted wrapper
+    (folx/experimental/pallas/attention/__init__.py:17-45)."""
+    return _call('_multi_head_self_attention', (q, k, v, mask, input_mask), kwargs)
+
+
+# reductions --------------------------------------------------------------------------------
+def _axes(axis, nd):
+    if axis is None:
+        return tuple(range(nd))
+    if isinstance(axis, int):
+        axis = (axis,)
+    return tuple(a % nd for a in axis)
+
+
+def sum(a, axis=None, keepdims=False):
+    shape = _shape(a)
+    axes = _axes(axis, len(shape))
+    out = _call('reduce_sum', (a,), {'axes': axes})
+    if keepdims:
+        out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
+    return out
+
+
+def mean(a, axis=None, keepdims=False):
+    shape = _shape(a)
+    axes = _axes(axis, len(shape))
+    n = int(np.prod([shape[i] for i in axes], dtype=int))
+    return multiply(sum(a, axis, keepdims), 1.0 / n)
+
+
+def amax_const(a, axis, keepdims=False):
+    """max of the values as a derivative-free array (``stop_gradient(max(a))``)."""
+    shape = _shape(a)
+    axes = _axes(axis, len(shape))
+    out = _call('reduce_max_values', (a,), {'axes': axes})
+    if keepdims:
+        out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
+    return out
+
+
+def logsumexp(a, axis=-1, b=None):
+    """``jax.nn.logsumexp(a, axis, b=b, return_sign=True)``: the same primitive sequence
+    (max shift under stop_gradient, exp, weighted sum, log|.|).  Returns (value, sign)."""
+    m = amax_const(a, axis, keepdims=True)
+    e = exp(subtract(a, m))
+    if b is not None:
+        e = multiply(e, b)
+    s = sum(e, axis)
+    sg = sign(s)
+    val = add(log(abs(s)), reshape(m, _shape(s)))
+    return val, sg
+
+
+# indexing ----------------------------------------------------------------------------------
+def reshape(a, shape):
+    shape = tuple(int(s) for s in shape)
+    if -1 in shape:
+        tot = int(np.prod(_shape(a), dtype=int))
+        rest = -int(np.prod(shape, dtype=int))
+        shape = tuple(tot // rest if s == -1 else s for s in shape)
+    return _call('reshape', (a,), {'new_sizes': shape})
+
+
+def transpose(a, axes=None):
+    nd = len(_shape(a))
+    axes = tuple(range(nd))[::-1] if axes is None else tuple(ax % nd for ax in axes)
+    return _call('transpose', (a,), {'permutation': axes})
+
+
+def swapaxes(a, i, j):
+    nd = len(_shape(a))
+    axes = list(range(nd))
+    axes[i % nd], axes[j % nd] = axes[j % nd], axes[i % nd]
+    return transpose(a, axes)
+
+
+def expand_dims(a, axis):
+    shape = list(_shape(a))
+    axis = axis % (len(shape) + 1)
+    shape.insert(axis, 1)
+    return reshape(a, shape)
+
+
+def squeeze(a, axis):
+    shape = list(_shape(a))
+    axis = axis % len(shape)
+    assert shape[axis] == 1
+    del shape[axis]
+    return reshape(a, shape)
+
+
+def broadcast_to(a, shape):
+    shape = tuple(shape)
+    src = _shape(a)
+    off = len(shape) - len(src)
+    return _call('broadcast_in_dim', (a,), {'shape': shape, 'broadcast_dimensions': tuple(range(off, len(shape)))})
+
+
+def getitem(a, idx):
+    return _call('slice', (a,), {'idx': idx})
+
+
+def concatenate(arrs, axis=-1):
+    return _call('concatenate', tuple(arrs), {'dimension': axis})

@@ -1,0 +1,130 @@
+"""Device side of the sparse-Jacobian bookkeeping: host masks in, gather-kernel launches out.
+
+The index tables built by ``index_algebra`` are uploaded once and cached by content, so a
+model that is evaluated repeatedly (or replayed from a HIP graph) never re-uploads them.
+"""
+
+from __future__ import annotations
+
+import hashlib
+
+import numpy as np
+import torch
+
+from . import index_algebra as ia
+from . import kernels as K
+from .api import FwdJacobian
+
+_TABLE_CACHE: dict = {}
+_CONST_CACHE: dict = {}
+_MAX_TABLE_ENTRIES = 1 << 27  # beyond this the scatter-add kernel is used instead
+
+
+def _key(arr: np.ndarray, *extra):
+    a = np.ascontiguousarray(arr)
+    return (hashlib.blake2b(a.tobytes(), digest_size=16).digest(), a.shape, str(a.dtype), *extra)
+
+
+def device_table(arr: np.ndarray, device) -> torch.Tensor:
+    """int32 table on the device, cached by content."""
+    key = _key(arr, 'i32', str(device))
+    t = _TABLE_CACHE.get(key)
+    if t is None:
+        t = torch.as_tensor(np.ascontiguousarray(arr, dtype=np.int32)).to(device)
+        _TABLE_CACHE[key] = t
+    return t
+
+
+def device_const(arr, device) -> torch.Tensor:
+    """float32 constant on the device; numpy inputs are cached by content."""
+    if isinstance(arr, torch.Tensor):
+        if arr.device != device or arr.dtype != torch.float32:
+            arr = arr.to(device=device, dtype=torch.float32)
+        return arr.contiguous()
+    a = np.array(arr, dtype=np.float32, order='C', copy=True)
+    key = _key(a, 'f32', str(device))
+    t = _CONST_CACHE.get(key)
+    if t is None:
+        t = torch.as_tensor(a).to(device)
+        _CONST_CACHE[key] = t
+    return t
+
+
+def clear_caches():
+    _TABLE_CACHE.clear()
+    _CONST_CACHE.clear()
+
+
+def zeros(shape, device) -> torch.Tensor:
+    """Zero tensor produced by a fill kernel (never by a memset node, so that the call can
+    sit inside a captured HIP graph)."""
+    return torch.empty(shape, device=device, dtype=torch.float32).zero_()
+
+
+def materialize(data: torch.Tensor, idx: np.ndarray, n_out: int) -> torch.Tensor:
+    """out[t, b, pos] = sum of data[r, b, pos] over rows r with idx[r, pos] == t.
+
+    data (k, B, *s) on the device, idx (k, *s) host slot map (``-1`` = drop).  Static
+    gather (folx/utils.py:71-114) through ``folx_hip_gather_rows``; the table is stored
+    without the trailing axes along which ``idx`` is constant.
+    """
+    k, B = data.shape[0], data.shape[1]
+    s = tuple(data.shape[2:])
+    idx = np.broadcast_to(idx, (k, *s))
+    if n_out == 0 or k == 0:
+        return zeros((n_out, B, *s), data.device)
+    n_inner = ia.split_inner(idx)
+    n_outer_axes = len(s) - n_inner
+    s_outer, s_inner = s[:n_outer_axes], s[n_outer_axes:]
+    S_outer = int(np.prod(s_outer, dtype=np.int64))
+    S_inner = int(np.prod(s_inner, dtype=np.int64))
+    idx_c = idx[(slice(None), *([slice(None)] * n_outer_axes), *([0] * n_inner))]
+    data = data.contiguous().reshape(k, B, S_outer * S_inner)
+    key = _key(idx_c, 'take', n_out)
+    cached = _TABLE_CACHE.get((key, str(data.device)))
+    if cached is None:
+        take = ia.gather_table(idx_c, n_out)
+        n_slots = take.shape[1]
+        if take.size > _MAX_TABLE_ENTRIES:
+            cached = ('scatter', device_table(idx_c.reshape(k, S_outer), data.device), 0)
+        else:
+            cached = ('gather', device_table(take.reshape(n_out, n_slots, S_outer), data.device), n_slots)
+        _TABLE_CACHE[(key, str(data.device))] = cached
+    kind, table, n_slots = cached
+    if kind == 'gather':
+        out = K.gather_rows(data, table, n_out, n_slots, B, S_outer, S_inner)
+    else:
+        out = K.scatter_add_rows(data, table, n_out, B, S_outer, S_inner)
+    return out.reshape(n_out, B, *s)
+
+
+def pad_rows(data: torch.Tensor, P: int) -> torch.Tensor:
+    """Zero-extend a dense Jacobian to P rows (folx/utils.py:432-450)."""
+    if data.shape[0] == P:
+        return data
+    out = torch.empty((P, *data.shape[1:]), device=data.device, dtype=data.dtype)
+    out[: data.shape[0]].copy_(data)
+    out[data.shape[0] :].zero_()
+    return out
+
+
+def add_rowstacks(a: torch.Tensor, b: torch.Tensor, sign: float = 1.0) -> torch.Tensor:
+    """a + sign * b for two equally shaped row stacks (one flat affine launch)."""
+    n = a.numel()
+    out = K.rows_affine(a.contiguous(), 1, (n,), (n,), None, b.contiguous().reshape(n), 1.0, sign)
+    return out.reshape(a.shape)
+
+
+def add_jacobians(a: FwdJacobian, b: FwdJacobian) -> FwdJacobian:
+    """``FwdJacobian.__add__`` (folx/api.py:230-249)."""
+    if not a.weak or not b.weak:
+        da, db = a.dense_array, b.dense_array
+        P = max(da.shape[0], db.shape[0])
+        return FwdJacobian(add_rowstacks(pad_rows(da, P), pad_rows(db, P)), None)
+    if a.x0_idx.shape[0] == b.x0_idx.shape[0] and np.array_equal(
+        *np.broadcast_arrays(a.x0_idx, b.x0_idx)
+    ):
+        return FwdJacobian(add_rowstacks(a.data, b.data), np.broadcast_arrays(a.x0_idx, b.x0_idx)[0])
+    return FwdJacobian(
+        torch.cat([a.data, b.data], dim=0), np.concatenate([a.x0_idx, b.x0_idx], axis=0)
+    )

@@ -1,0 +1,781 @@
+"""Rule registry and the forward-Laplacian rules, each one a launch (or a few) of the HIP
+kernel library.
+
+Mirrors folx/wrapped_functions.py: ``_LAPLACE_FN_REGISTRY`` (:355-561) keyed by primitive
+name, ``register_function`` / ``deregister_function`` / ``is_registered`` /
+``get_laplacian`` (:564-618).  A rule has the reference's signature
+``rule(args, kwargs, sparsity_threshold) -> FwdLaplArray | tuple`` (folx/api.py:444-450).
+Keys are the jax primitive / jitted-function names the reference registers under
+(``'dot_general'``, ``'tanh'``, ``'reduce_sum'``, ``'slogdet'``,
+``'_multi_head_self_attention'`` ...), so a rule written for folx's registry plugs in
+under the same name.
+
+Unlike the reference there is no generic autodiff fallback: a primitive without a kernel
+rule raises ``KeyError`` in ``get_laplacian``.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Any, Callable
+
+import numpy as np
+import torch
+
+from . import index_algebra as ia
+from . import kernels as K
+from . import sparse_ops as so
+from .api import BatchedArray, FwdJacobian, FwdLaplArray
+
+ForwardLaplacian = Callable[[tuple, dict, int], Any]
+
+_LAPLACE_FN_REGISTRY: dict[str, ForwardLaplacian] = {}
+
+
+def register_function(primitive_or_name: str, laplacian: ForwardLaplacian):
+    """Register a rule under a primitive / function name (folx/wrapped_functions.py:564)."""
+    _LAPLACE_FN_REGISTRY[primitive_or_name] = laplacian
+
+
+def deregister_function(primitive_or_name: str):
+    del _LAPLACE_FN_REGISTRY[primitive_or_name]
+
+
+def is_registered(primitive_or_name: str) -> bool:
+    return primitive_or_name in _LAPLACE_FN_REGISTRY
+
+
+def get_laplacian(primitive_or_name: str, wrap_if_missing: bool = False) -> ForwardLaplacian | None:
+    """folx/wrapped_functions.py:597-618.  ``wrap_if_missing`` cannot be honoured (there
+    is no autodiff to derive a rule from) and raises instead."""
+    if primitive_or_name in _LAPLACE_FN_REGISTRY:
+        return _LAPLACE_FN_REGISTRY[primitive_or_name]
+    if wrap_if_missing:
+        raise KeyError(
+            f'{primitive_or_name!r} has no forward-Laplacian rule; register one with '
+            'folx_amd.register_function'
+        )
+    return None
+
+
+# --------------------------------------------------------------------------------------
+# helpers
+# --------------------------------------------------------------------------------------
+
+
+def _is(a):
+    return isinstance(a, FwdLaplArray)
+
+
+def _logical_shape(c) -> tuple:
+    if isinstance(c, (FwdLaplArray, BatchedArray)):
+        return tuple(c.shape)
+    if isinstance(c, torch.Tensor):
+        return tuple(c.shape)
+    return tuple(np.shape(c))
+
+
+def _pad_logical(t: FwdLaplArray, nd: int) -> FwdLaplArray:
+    """Prepend size-1 logical axes (numpy broadcasting aligns shapes on the right)."""
+    ex = nd - t.ndim
+    if ex <= 0:
+        return t
+    one = (1,) * ex
+    B, k = t.B, t.jacobian.data.shape[0]
+    mask = t.jacobian.x0_idx
+    if mask is not None:
+        mask = mask.reshape(mask.shape[0], *one, *mask.shape[1:])
+    return FwdLaplArray(
+        t.x.reshape(B, *one, *t.shape),
+        FwdJacobian(t.jacobian.data.reshape(k, B, *one, *t.shape), mask),
+        t.laplacian.reshape(B, *one, *t.shape),
+    )
+
+
+def _const_tensor(c, nd: int, device) -> torch.Tensor:
+    """Constant as a device tensor of shape (B or 1, *logical padded to nd dims)."""
+    if isinstance(c, BatchedArray):
+        d = c.data
+        return d.reshape(d.shape[0], *((1,) * (nd - c.ndim)), *c.shape).contiguous()
+    t = so.device_const(c, device)
+    return t.reshape(1, *((1,) * (nd - t.dim())), *t.shape)
+
+
+def _empty_jac(like: torch.Tensor) -> torch.Tensor:
+    return torch.empty((0, *like.shape), device=like.device, dtype=torch.float32)
+
+
+def _values_binary(op: str, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Binary op on derivative-free device arrays (the P = 0 case of the binary kernel)."""
+    a, b = a.contiguous(), b.contiguous()
+    y, _, _ = K.binary(op, a, _empty_jac(a), a, b, _empty_jac(b), b)
+    return y
+
+
+def _values_unary(name: str, a: torch.Tensor, param=0.0) -> torch.Tensor:
+    a = a.contiguous()
+    y, _, _ = K.elementwise(name, a, _empty_jac(a), a, param)
+    return y
+
+
+def _bmask(mask, k, out_shape):
+    return None if mask is None else np.broadcast_to(mask, (k, *out_shape))
+
+
+# --------------------------------------------------------------------------------------
+# unary elementwise rules (kernel family 2)
+# --------------------------------------------------------------------------------------
+
+_NP_UNARY = {
+    'tanh': np.tanh, 'exp': np.exp, 'log': np.log, 'sqrt': np.sqrt, 'square': np.square,
+    'sin': np.sin, 'cos': np.cos, 'abs': np.abs, 'log1p': np.log1p, 'expm1': np.expm1,
+    'rsqrt': lambda x: 1 / np.sqrt(x), 'reciprocal': lambda x: 1 / x,
+    'logistic': lambda x: 1 / (1 + np.exp(-x)), 'silu': lambda x: x / (1 + np.exp(-x)),
+    'softplus': lambda x: np.logaddexp(x, 0), 'neg': np.negative,
+}
+
+
+def _unary_rule(name: str) -> ForwardLaplacian:
+    """``wrap_forward_laplacian(f, in_axes=())`` for a scalar function
+    (folx/wrapped_functions.py:400-415): one fused pass ``y = f(x)``, ``J_y = f'(x) J``,
+    ``lap_y = f'(x) lap + f''(x) sum_p J_p^2`` for dense and sparse storage alike
+    (folx/jvp.py:687-697, :262-272; folx/hessian.py:87-112, gate :460-470)."""
+
+    def rule(args, kwargs, sparsity_threshold):
+        (a,) = args
+        param = kwargs.get('y', kwargs.get('param', 0.0))
+        if isinstance(a, BatchedArray):
+            return BatchedArray(_values_unary(name, a.data, param))
+        if not _is(a):
+            if name == 'integer_pow':
+                return np.asarray(a) ** int(param)
+            return _NP_UNARY[name](np.asarray(a))
+        mask = a.jacobian.x0_idx
+        x, J, lap = a.x, a.jacobian.data, a.laplacian
+        if mask is not None and ia.has_duplicates(mask):
+            # An index listed twice at one position breaks sum_k J_k^2 = |grad|^2, so the
+            # reference leaves its fast path (folx/hessian.py:460-470): the Jacobian rows
+            # keep their layout (folx/jvp.py:262-272) while the Hessian term is taken on
+            # the per-position unique frame (folx/hessian.py:288-340).
+            y, Jy, _ = K.elementwise(name, x, J, lap, param)
+            frame, _ = ia.find_out_idx([mask], [list(a.shape)], [()], False, sparsity_threshold)
+            frame = frame.reshape(frame.shape[0], *a.shape)
+            Jm = so.materialize(J, ia.get_index_mask(mask, frame), frame.shape[0])
+            _, _, lapy = K.elementwise(name, x, Jm, lap, param)
+            return FwdLaplArray(y, FwdJacobian(Jy, mask), lapy)
+        y, Jy, lapy = K.elementwise(name, x, J, lap, param)
+        return FwdLaplArray(y, FwdJacobian(Jy, mask), lapy)
+
+    rule.__name__ = name
+    return rule
+
+
+def neg_rule(args, kwargs, sparsity_threshold):
+    """``lax.neg`` is LINEAR (folx/wrapped_functions.py:361-363)."""
+    (a,) = args
+    if isinstance(a, BatchedArray):
+        return BatchedArray(_scale_rows(a.data, 1, -1.0))
+    if not _is(a):
+        return -np.asarray(a)
+    k = a.jacobian.data.shape[0]
+    return FwdLaplArray(
+        _scale_rows(a.x, 1, -1.0),
+        FwdJacobian(_scale_rows(a.jacobian.data, k, -1.0), a.jacobian.x0_idx),
+        _scale_rows(a.laplacian, 1, -1.0),
+    )
+
+
+def _scale_rows(t: torch.Tensor, rows: int, alpha: float) -> torch.Tensor:
+    n = t.numel() // max(rows, 1)
+    if t.numel() == 0:
+        return t.clone()
+    out = K.rows_affine(t.contiguous(), rows, (n,), (n,), None, None, alpha, 0.0)
+    return out.reshape(t.shape)
+
+
+# --------------------------------------------------------------------------------------
+# binary elementwise rules
+# --------------------------------------------------------------------------------------
+
+
+def _affine_const(t: FwdLaplArray, c, *, mul: bool, alpha: float, beta: float) -> FwdLaplArray:
+    """Triplet against a constant: ``y = alpha * x (* c) (+ beta * c)``; the Jacobian rows
+    and the Laplacian are scaled the same way and never shifted (LINEAR rules,
+    folx/wrapped_functions.py:361-376; mul by a constant is the one-argument case of
+    MULTIPLICATION, folx/hessian.py:561-570 -> zero Hessian term)."""
+    scalar = isinstance(c, (int, float)) or (not isinstance(c, (BatchedArray, torch.Tensor)) and np.ndim(c) == 0)
+    cshape = () if scalar else _logical_shape(c)
+    nd = max(t.ndim, len(cshape))
+    t = _pad_logical(t, nd)
+    out_shape = tuple(np.broadcast_shapes(t.shape, cshape))
+    B, k = t.B, t.jacobian.data.shape[0]
+    dev = t.x.device
+    if scalar:
+        cval = float(c)
+        ct = None
+        if mul:
+            a_x = a_j = alpha * cval
+            d_t, b_x = None, 0.0
+        else:
+            a_x = a_j = alpha
+            d_t = so.device_const(np.full((1,) * (nd + 1), cval, dtype=np.float32), dev)
+            b_x = beta
+    else:
+        ct = _const_tensor(c, nd, dev)
+        a_x = a_j = alpha
+        d_t, b_x = (None, 0.0) if mul else (ct, beta)
+        if not mul:
+            ct = None
+    full = (B, *out_shape)
+    x = K.rows_affine(t.x, 1, (B, *t.shape), full, ct, d_t, a_x, b_x).reshape(full)
+    same = out_shape == t.shape and ct is None and a_j == 1.0
+    if same:
+        J, lap = t.jacobian.data, t.laplacian
+    else:
+        J = K.rows_affine(t.jacobian.data, k, (B, *t.shape), full, ct, None, a_j, 0.0).reshape(k, *full)
+        lap = K.rows_affine(t.laplacian, 1, (B, *t.shape), full, ct, None, a_j, 0.0).reshape(full)
+    return FwdLaplArray(x, FwdJacobian(J, _bmask(t.jacobian.x0_idx, k, out_shape)), lap)
+
+
+def _binary_const(op: str, t: FwdLaplArray, c, t_is_left: bool) -> FwdLaplArray:
+    if op == 'add':
+        return _affine_const(t, c, mul=False, alpha=1.0, beta=1.0)
+    if op == 'sub':
+        if t_is_left:
+            return _affine_const(t, c, mul=False, alpha=1.0, beta=-1.0)
+        return _affine_const(t, c, mul=False, alpha=-1.0, beta=1.0)
+    if op == 'mul':
+        return _affine_const(t, c, mul=True, alpha=1.0, beta=0.0)
+    if op == 'div':
+        if t_is_left:
+            if isinstance(c, BatchedArray):
+                rc = BatchedArray(_values_unary('reciprocal', c.data))
+            elif isinstance(c, torch.Tensor):
+                rc = 1.0 / c.detach().cpu().numpy().astype(np.float64)
+            else:
+                rc = 1.0 / np.asarray(c, dtype=np.float64)
+            return _affine_const(t, rc, mul=True, alpha=1.0, beta=0.0)
+        r = _LAPLACE_FN_REGISTRY['reciprocal']((t,), {}, 0)
+        return _affine_const(r, c, mul=True, alpha=1.0, beta=0.0)
+    raise ValueError(op)
+
+
+def _expand_rows(J: torch.Tensor, k: int, src_shape, full) -> torch.Tensor:
+    """Materialise the broadcast of Jacobian rows (k, *src_shape) to (k, *full)."""
+    if tuple(src_shape) == tuple(full):
+        return J
+    return K.rows_affine(J, k, tuple(src_shape), tuple(full), None, None, 1.0, 0.0).reshape(k, *full)
+
+
+def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLaplArray:
+    nd = max(a.ndim, b.ndim)
+    a, b = _pad_logical(a, nd), _pad_logical(b, nd)
+    out_shape = tuple(np.broadcast_shapes(a.shape, b.shape))
+    B = a.B
+
+    def fused(Ja, Jb, mask):
+        y, J, lap = K.binary(op, a.x, Ja, a.laplacian, b.x, Jb, b.laplacian)
+        return FwdLaplArray(y, FwdJacobian(J, mask), lap)
+
+    if not (a.jacobian.weak and b.jacobian.weak):
+        # Any dense operand: the reference adds the per-operand results through
+        # FwdJacobian.__add__, which densifies (folx/jvp.py:742-796, folx/api.py:233-236).
+        Ja, Jb = a.jacobian.dense_array, b.jacobian.dense_array
+        P = max(Ja.shape[0], Jb.shape[0])
+        return fused(so.pad_rows(Ja, P), so.pad_rows(Jb, P), None)
+
+    ma = np.broadcast_to(a.jacobian.x0_idx, (a.jacobian.x0_idx.shape[0], *out_shape))
+    mb = np.broadcast_to(b.jacobian.x0_idx, (b.jacobian.x0_idx.shape[0], *out_shape))
+    ka, kb = ma.shape[0], mb.shape[0]
+    if ka == kb and np.array_equal(ma, mb) and not ia.has_duplicates(ma) and (
+        ka == 1 or np.unique(ma.reshape(ka, -1), axis=0).shape[0] == ka
+    ):
+        # identical masks: merged rows = the rows themselves, and the intersection /
+        # union frame is the mask itself, so one fused launch on k rows is the rule
+        return fused(a.jacobian.data, b.jacobian.data, ma)
+
+    # ---- general sparse case: merged one-hot rows (folx/jvp.py:273-317) -----------------
+    res_mask, inv = ia.merge_rows([ma, mb])
+    full = (B, *out_shape)
+    if op in ('add', 'sub'):
+        ca = cb = None
+        sa, sb = 1.0, (1.0 if op == 'add' else -1.0)
+    elif op == 'mul':
+        ca, cb, sa, sb = b.x, a.x, 1.0, 1.0
+    else:  # div: d/da = 1/b, d/db = -a/b^2
+        rb = _values_unary('reciprocal', b.x)
+        q = _values_binary('mul', a.x, rb)
+        ca, cb, sa, sb = rb, _values_binary('mul', q, rb), 1.0, -1.0
+
+    def scaled_row(J, r, src_shape, c, alpha):
+        row = J[r : r + 1].contiguous()
+        return K.rows_affine(row, 1, (B, *src_shape), full, c, None, alpha, 0.0).reshape(1, *full)
+
+    rows = [scaled_row(a.jacobian.data, r, a.shape, ca, sa) for r in range(ka)]
+    rows += [scaled_row(b.jacobian.data, r, b.shape, cb, sb) for r in range(kb)]
+    merged = []
+    for o in range(res_mask.shape[0]):
+        members = np.nonzero(inv == o)[0]
+        acc = rows[members[0]]
+        for m in members[1:]:
+            acc = so.add_rowstacks(acc, rows[m])
+        merged.append(acc)
+    J_out = torch.cat(merged, dim=0) if len(merged) > 1 else merged[0]
+
+    if op in ('add', 'sub'):
+        y = K.rows_affine(a.x, 1, (B, *a.shape), full, None,
+                          _expand_rows(b.x, 1, (B, *b.shape), full).reshape(full), 1.0, sb).reshape(full)
+        lap = K.rows_affine(a.laplacian, 1, (B, *a.shape), full, None,
+                            _expand_rows(b.laplacian, 1, (B, *b.shape), full).reshape(full), 1.0, sb).reshape(full)
+        return FwdLaplArray(y, FwdJacobian(J_out, res_mask), lap)
+
+    # Hessian term on the static index frame (folx/hessian.py:288-340, :379-428):
+    # intersection for mul (LINEAR_IN_ONE), union for div; dense when the frame says so.
+    frame, dense_out = ia.find_out_idx(
+        [ma, mb], [list(out_shape), list(out_shape)], [(), ()], op == 'mul', thr
+    )
+    if dense_out:
+        Ja, Jb = a.jacobian.dense_array, b.jacobian.dense_array
+        P = max(Ja.shape[0], Jb.shape[0])
+        Ja, Jb = so.pad_rows(Ja, P), so.pad_rows(Jb, P)
+    else:
+        frame = frame.reshape(frame.shape[0], *out_shape)
+        M = frame.shape[0]
+        Ja = so.materialize(_expand_rows(a.jacobian.data, ka, (B, *a.shape), full), ia.get_index_mask(ma, frame), M)
+        Jb = so.materialize(_expand_rows(b.jacobian.data, kb, (B, *b.shape), full), ia.get_index_mask(mb, frame), M)
+    if Ja.shape[0] == 0:
+        Ja = Jb = _empty_jac(a.x.expand(full))
+    y, _, lap = K.binary(op, a.x, Ja, a.laplacian, b.x, Jb, b.laplacian)
+    return FwdLaplArray(y, FwdJacobian(J_out, res_mask), lap)
+
+
+_NP_BINARY = {'add': np.add, 'sub': np.subtract, 'mul': np.multiply, 'div': np.divide}
+
+
+def _binary_rule(op: str) -> ForwardLaplacian:
+    def rule(args, kwargs, sparsity_threshold):
+        a, b = args
+        if _is(a) and _is(b):
+            return _binary_both(op, a, b, sparsity_threshold)
+        if _is(a):
+            return _binary_const(op, a, b, True)
+        if _is(b):
+            return _binary_const(op, b, a, False)
+        if isinstance(a, BatchedArray) or isinstance(b, BatchedArray):
+            ref = a if isinstance(a, BatchedArray) else b
+            nd = max(len(_logical_shape(a)), len(_logical_shape(b)))
+            ta = _const_tensor(a, nd, ref.data.device)
+            tb = _const_tensor(b, nd, ref.data.device)
+            Bn = ref.B
+            ta = ta.expand(Bn, *ta.shape[1:]) if ta.shape[0] == 1 else ta
+            tb = tb.expand(Bn, *tb.shape[1:]) if tb.shape[0] == 1 else tb
+            return BatchedArray(_values_binary(op, ta.contiguous(), tb.contiguous()))
+        return _NP_BINARY[op](np.asarray(a), np.asarray(b))
+
+    rule.__name__ = op
+    return rule
+
+
+# --------------------------------------------------------------------------------------
+# dense layer (kernel family 1)
+# --------------------------------------------------------------------------------------
+
+
+def dot_general(args, kwargs, sparsity_threshold: int = 0):
+    """``h @ W`` with exactly one operand carrying derivatives and the last axis of ``h``
+    contracted with the first axis of a constant matrix ``W (K, N)``
+    (``_dot_general_one_constant``, folx/wrapped_functions.py:71-171): the product is
+    applied to x, to every Jacobian row and to the Laplacian in one GEMM launch.
+    ``kwargs['bias']`` (constant, shape (N,)) is added to x only.
+
+    Sparse ``h``: rows pass through when the mask is constant along the contracted axis;
+    otherwise they are first aligned to the per-position union frame over that axis
+    (:113-130); a union wider than the threshold falls back to the dense Jacobian, which
+    is what the reference's general path produces for this case (folx/jvp.py:224-230).
+    """
+    h, W = args
+    bias = kwargs.get('bias')
+    if not _is(h):
+        if _is(W):
+            raise NotImplementedError('dot_general: constant @ triplet is not supported; transpose the product')
+        if isinstance(h, BatchedArray):
+            raise NotImplementedError('dot_general on walker-varying constants')
+        y = np.asarray(h) @ np.asarray(W)
+        return y if bias is None else y + np.asarray(bias)
+    if _is(W):
+        raise NotImplementedError(
+            'dot_general with two derivative-carrying operands: use multiply + sum, or '
+            'multi_head_self_attention for attention'
+        )
+    dev = h.x.device
+    Wt = so.device_const(W, dev)
+    bt = None if bias is None else so.device_const(bias, dev)
+    Kd, N = Wt.shape
+    assert h.shape[-1] == Kd, f'dot: contracting {h.shape} with {tuple(Wt.shape)}'
+    J, mask = h.jacobian.data, h.jacobian.x0_idx
+    new_mask = None
+    if mask is not None:
+        proj, aligned = ia.dot_projection(mask, -1, sparsity_threshold)
+        if proj is None:
+            logging.info('dot_general: union over the contracted axis exceeds the sparsity threshold; densifying')
+            J = h.jacobian.dense_array
+        else:
+            if aligned:
+                J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
+            new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
+    y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt)
+    return FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
+
+
+# --------------------------------------------------------------------------------------
+# reductions
+# --------------------------------------------------------------------------------------
+
+
+def _norm_axes(axes, nd):
+    if axes is None:
+        return tuple(range(nd))
+    if isinstance(axes, int):
+        axes = (axes,)
+    return tuple(sorted(set(a % nd for a in axes)))
+
+
+def _reduce_tensor(t: torch.Tensor, lead: int, axes, alpha=1.0) -> torch.Tensor:
+    """Sum ``t`` over logical ``axes``; ``lead`` = number of leading non-logical axes."""
+    shape = list(t.shape)
+    for ax in sorted(axes, reverse=True):
+        full_ax = ax + lead
+        outer = int(np.prod(shape[:full_ax], dtype=np.int64))
+        red = shape[full_ax]
+        inner = int(np.prod(shape[full_ax + 1 :], dtype=np.int64))
+        t = K.reduce_sum(t.contiguous().reshape(-1), 1, outer, red, inner, alpha)
+        alpha = 1.0
+        del shape[full_ax]
+        t = t.reshape(shape)
+    return t
+
+
+def reduce_sum(args, kwargs, sparsity_threshold):
+    """``reduce_sum`` (SUMMATION, folx/wrapped_functions.py:388-392).  Dense: the same sum
+    on x, rows and lap.  Sparse (``sparse_sum_jvp``, folx/jvp.py:89-176): static output
+    mask, rows gathered into their output slots; past the threshold the rows are summed
+    straight into the dense Jacobian (:128-140)."""
+    (a,) = args
+    if not _is(a):
+        if isinstance(a, BatchedArray):
+            axes = _norm_axes(kwargs.get('axes'), a.ndim)
+            return BatchedArray(_reduce_tensor(a.data, 1, axes))
+        return np.sum(np.asarray(a), axis=kwargs.get('axes'))
+    axes = _norm_axes(kwargs.get('axes'), a.ndim)
+    if len(axes) == 0:
+        return a
+    x = _reduce_tensor(a.x, 1, axes)
+    lap = _reduce_tensor(a.laplacian, 1, axes)
+    J, mask = a.jacobian.data, a.jacobian.x0_idx
+    if mask is None:
+        return FwdLaplArray(x, FwdJacobian(_reduce_tensor(J, 2, axes), None), lap)
+
+    idx_out, slot = ia.sum_out_mask(mask, axes)
+    if idx_out.shape[0] > sparsity_threshold:
+        logging.info(
+            f'reduce_sum: output ({idx_out.shape[0]}) reaches sparsity threshold '
+            f'({sparsity_threshold}); switching to dense'
+        )
+        n_out = int(mask.max()) + 1
+        slot, out_mask = mask, None
+    else:
+        n_out, out_mask = idx_out.shape[0], idx_out
+    k = mask.shape[0]
+    red_ax = [ax + 1 for ax in axes]
+    first = slot
+    for ax in red_ax:
+        first = np.take(first, [0], axis=ax)
+    if (slot == first).all():
+        # every row keeps one slot along the reduced axes: reduce rows, then re-slot
+        Jr = _reduce_tensor(J, 2, axes)
+        slot_c = first.reshape(k, *[n for i, n in enumerate(a.shape) if i not in axes])
+        ident = n_out == k and (slot_c == np.arange(k).reshape(k, *([1] * (slot_c.ndim - 1)))).all()
+        Jo = Jr if ident else so.materialize(Jr, slot_c, n_out)
+    else:
+        # fold the reduced axes into the row axis, then gather (rows, reduced) -> slots
+        nd = a.ndim
+        kept = [i for i in range(nd) if i not in axes]
+        perm = [0] + [ax + 2 for ax in axes] + [1] + [i + 2 for i in kept]
+        R = int(np.prod([a.shape[ax] for ax in axes], dtype=np.int64))
+        Jp = J.permute(*perm).contiguous().reshape(k * R, a.B, *[a.shape[i] for i in kept])
+        sp = np.transpose(slot, [0] + [ax + 1 for ax in axes] + [i + 1 for i in kept])
+        sp = sp.reshape(k * R, *[a.shape[i] for i in kept])
+        Jo = so.materialize(Jp, sp, n_out)
+    return FwdLaplArray(x, FwdJacobian(Jo, out_mask), lap)
+
+
+# --------------------------------------------------------------------------------------
+# indexing rules: the op is applied to x, rows, lap and to the mask alike
+# (sparse_index_jvp, folx/jvp.py:330-413)
+# --------------------------------------------------------------------------------------
+
+
+def _index_rule(fn_t, fn_m):
+    """fn_t(tensor, lead) applies the op to a tensor with ``lead`` leading non-logical
+    axes; fn_m(mask) applies it to a host mask (one leading row axis)."""
+
+    def apply(a: FwdLaplArray) -> FwdLaplArray:
+        mask = a.jacobian.x0_idx
+        return FwdLaplArray(
+            fn_t(a.x, 1).contiguous(),
+            FwdJacobian(fn_t(a.jacobian.data, 2).contiguous(), None if mask is None else fn_m(mask)),
+            fn_t(a.laplacian, 1).contiguous(),
+        )
+
+    return apply
+
+
+def _const_index(a, fn_t):
+    if isinstance(a, BatchedArray):
+        return BatchedArray(fn_t(a.data, 1).contiguous())
+    t = torch.as_tensor(np.asarray(a))
+    return fn_t(t, 0).numpy()
+
+
+def reshape_rule(args, kwargs, sparsity_threshold):
+    (a,) = args
+    shape = tuple(kwargs['new_sizes'])
+    fn_t = lambda t, lead: t.reshape(*t.shape[:lead], *shape)
+    if not _is(a):
+        return _const_index(a, fn_t)
+    return _index_rule(fn_t, lambda m: m.reshape(m.shape[0], *shape))(a)
+
+
+def transpose_rule(args, kwargs, sparsity_threshold):
+    (a,) = args
+    perm = tuple(kwargs['permutation'])
+    fn_t = lambda t, lead: t.permute(*range(lead), *[p + lead for p in perm])
+    if not _is(a):
+        return _const_index(a, fn_t)
+    return _index_rule(fn_t, lambda m: np.transpose(m, (0, *[p + 1 for p in perm])))(a)
+
+
+def broadcast_in_dim_rule(args, kwargs, sparsity_threshold):
+    """``broadcast_in_dim(shape, broadcast_dimensions)`` as in lax."""
+    (a,) = args
+    shape = tuple(kwargs['shape'])
+    bdims = tuple(kwargs['broadcast_dimensions'])
+
+    def mid_shape(src):
+        mid = [1] * len(shape)
+        for i, d in enumerate(bdims):
+            mid[d] = src[i]
+        return mid
+
+    def fn_t(t, lead):
+        mid = mid_shape(t.shape[lead:])
+        return t.reshape(*t.shape[:lead], *mid).expand(*t.shape[:lead], *shape)
+
+    if not _is(a):
+        return _const_index(a, fn_t)
+    fn_m = lambda m: np.broadcast_to(m.reshape(m.shape[0], *mid_shape(m.shape[1:])), (m.shape[0], *shape))
+    return _index_rule(fn_t, fn_m)(a)
+
+
+def _canon_index(idx, nd):
+    if not isinstance(idx, tuple):
+        idx = (idx,)
+    if any(i is Ellipsis for i in idx):
+        pos = [n for n, i in enumerate(idx) if i is Ellipsis][0]
+        n_real = len([i for i in idx if i is not None and i is not Ellipsis])
+        idx = idx[:pos] + (slice(None),) * (nd - n_real) + idx[pos + 1 :]
+    for i in idx:
+        if not (isinstance(i, (int, np.integer, slice)) or i is None):
+            raise TypeError('only static basic indexing (ints, slices, None, ...) is supported')
+    return idx
+
+
+def getitem_rule(args, kwargs, sparsity_threshold):
+    """Static basic indexing (``slice`` / ``squeeze`` / ``expand_dims`` primitives)."""
+    (a,) = args
+    idx = _canon_index(kwargs['idx'], len(_logical_shape(a)))
+    fn_t = lambda t, lead: t[(*([slice(None)] * lead), *idx)]
+    if not _is(a):
+        return _const_index(a, fn_t)
+    return _index_rule(fn_t, lambda m: m[(slice(None), *idx)])(a)
+
+
+def concatenate_rule(args, kwargs, sparsity_threshold):
+    """``concatenate`` (INDEXING with every operand static-capable,
+    folx/wrapped_functions.py:461-466).  All operands sparse: row counts are padded with
+    (mask -1, data 0) (``broadcast_dim``, folx/utils.py:453-481) and constants enter as
+    all ``-1`` rows (folx/jvp.py:350-372).  Any dense operand: everything densified
+    (folx/jvp.py:340-341)."""
+    axis = kwargs.get('dimension', kwargs.get('axis', -1))
+    trip = [t for t in args if _is(t)]
+    if not trip:
+        return np.concatenate([np.asarray(t) for t in args], axis=axis)
+    first = trip[0]
+    nd, B, dev = first.ndim, first.B, first.x.device
+    axis = axis % nd
+    all_sparse = all(t.jacobian.weak for t in trip)
+    if all_sparse:
+        k = max(t.jacobian.data.shape[0] for t in trip)
+    else:
+        k = max(t.jacobian.dense_array.shape[0] if not t.jacobian.weak else t.jacobian.max_n + 1 for t in trip)
+    xs, Js, Ls, Ms = [], [], [], []
+    for t in args:
+        if _is(t):
+            J = t.jacobian.data if all_sparse else t.jacobian.dense_array
+            xs.append(t.x), Ls.append(t.laplacian), Js.append(so.pad_rows(J, k))
+            if all_sparse:
+                m = t.jacobian.x0_idx
+                if m.shape[0] < k:
+                    m = np.concatenate([m, np.full((k - m.shape[0], *m.shape[1:]), -1, dtype=m.dtype)], 0)
+                Ms.append(m)
+        else:
+            if isinstance(t, BatchedArray):
+                c = t.data
+            else:
+                c = so.device_const(t, dev)
+                c = c.reshape(1, *c.shape).expand(B, *c.shape)
+            xs.append(c)
+            Ls.append(so.zeros(c.shape, dev))
+            Js.append(so.zeros((k, *c.shape), dev))
+            if all_sparse:
+                Ms.append(np.full((k, *c.shape[1:]), -1, dtype=np.int32))
+    x = torch.cat(xs, dim=axis + 1)
+    J = torch.cat(Js, dim=axis + 2)
+    lap = torch.cat(Ls, dim=axis + 1)
+    mask = np.concatenate(Ms, axis=axis + 1) if all_sparse else None
+    return FwdLaplArray(x, FwdJacobian(J, mask), lap)
+
+
+# --------------------------------------------------------------------------------------
+# derivative-free outputs
+# --------------------------------------------------------------------------------------
+
+
+def stop_gradient_rule(args, kwargs, sparsity_threshold):
+    """``warp_without_fwd_laplacian`` (folx/wrapper.py:141-154): derivatives are dropped."""
+    (a,) = args
+    return BatchedArray(a.x) if _is(a) else a
+
+
+def sign_rule(args, kwargs, sparsity_threshold):
+    (a,) = args
+    data = a.x if _is(a) else (a.data if isinstance(a, BatchedArray) else None)
+    if data is None:
+        return np.sign(np.asarray(a))
+    # sign(x) = d|x|/dx, evaluated by the abs rule on a one-row Jacobian of ones
+    ones = torch.empty((1, *data.shape), device=data.device, dtype=torch.float32).fill_(1.0)
+    _, d1, _ = K.elementwise('abs', data.contiguous(), ones, data.contiguous())
+    return BatchedArray(d1[0])
+
+
+def reduce_max_values(args, kwargs, sparsity_threshold):
+    """max over ``axes`` of the values only, returned derivative-free (the
+    ``stop_gradient(max)`` shift of logsumexp / softmax)."""
+    (a,) = args
+    data = a.x if _is(a) else a.data
+    nd = data.dim() - 1
+    axes = _norm_axes(kwargs.get('axes'), nd)
+    shape = list(data.shape)
+    t = data
+    for ax in sorted(axes, reverse=True):
+        f = ax + 1
+        outer = int(np.prod(shape[:f], dtype=np.int64))
+        inner = int(np.prod(shape[f + 1 :], dtype=np.int64))
+        t = K.reduce_max(t.contiguous().reshape(-1), outer, shape[f], inner)
+        del shape[f]
+        t = t.reshape(shape)
+    return BatchedArray(t)
+
+
+# --------------------------------------------------------------------------------------
+# slogdet (kernel family 4) and attention (kernel family 5)
+# --------------------------------------------------------------------------------------
+
+
+def slogdet_wrapper(args, kwargs, sparsity_threshold):
+    """``slogdet_wrapper`` -> ``dense_slogdet`` (folx/slogdet.py:347-358, :320-344):
+    returns ``(sign, FwdLaplArray(logdet))`` with a dense Jacobian.  A sparse input
+    Jacobian is densified first (the reference's rank-one shortcut for sparse inputs,
+    folx/slogdet.py:251-293, is not implemented)."""
+    (A,) = args
+    if not _is(A):
+        raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
+    assert A.shape[-1] == A.shape[-2], 'slogdet needs square matrices'
+    J = A.jacobian.dense_array
+    sign, ld, ldj, ldl = K.slogdet(A.x, J, A.laplacian)
+    return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
+
+
+def _mask_tensor(m, shape, device):
+    if m is None:
+        return None
+    if isinstance(m, BatchedArray):
+        m = m.data
+    if isinstance(m, torch.Tensor):
+        t = m.to(device=device)
+        t = (t != 0).to(torch.uint8)
+    else:
+        t = torch.as_tensor(np.ascontiguousarray(np.asarray(m) != 0).astype(np.uint8)).to(device)
+    return t.expand(*shape).contiguous()
+
+
+def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
+    """Rule of ``multi_head_self_attention`` (``mhsa_forward_laplacian``,
+    folx/experimental/pallas/attention/forward_laplacian.py:27-179).
+
+    args = (q, k, v, mask, input_mask): q, k, v triplets of per-walker shape (n, H, d)
+    (the caller scales q by 1/sqrt(d)); ``mask`` (B, n) or (n,) marks real electrons,
+    ``input_mask`` (P, B) or (P,) marks active input coordinates; either may be None.
+    Jacobians are densified as in the reference (:166-178).
+    """
+    del sparsity_threshold
+    q, k, v, mask, input_mask = (tuple(args) + (None, None))[:5]
+    if not (_is(q) and _is(k) and _is(v)):
+        raise NotImplementedError('multi_head_self_attention needs derivative-carrying q, k, v')
+    B, dev = q.B, q.x.device
+    n = q.shape[0]
+    Js = [t.jacobian.dense_array for t in (q, k, v)]
+    P = max(J.shape[0] for J in Js)
+    Js = [so.pad_rows(J, P) for J in Js]
+    mt = _mask_tensor(mask, (B, n), dev)
+    it = None
+    if input_mask is not None:
+        im = input_mask.data if isinstance(input_mask, BatchedArray) else input_mask
+        if not isinstance(im, torch.Tensor):
+            im = np.asarray(im)
+            if im.ndim == 1:
+                im = im[:, None]
+        elif im.dim() == 1:
+            im = im[:, None]
+        assert im.shape[0] == P, 'input_mask must have one entry per Jacobian row'
+        it = _mask_tensor(im, (P, B), dev)
+    o, oj, ol = K.mhsa(q.x, Js[0], q.laplacian, k.x, Js[1], k.laplacian, v.x, Js[2], v.laplacian, mt, it)
+    return FwdLaplArray(o, FwdJacobian(oj, None), ol)
+
+
+# --------------------------------------------------------------------------------------
+# registry (names follow folx/wrapped_functions.py:355-561)
+# --------------------------------------------------------------------------------------
+
+for _n in ['tanh', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'sin', 'cos', 'abs', 'log1p',
+           'expm1', 'integer_pow', 'silu', 'softplus', 'reciprocal']:
+    register_function(_n, _unary_rule(_n))
+register_function('sigmoid', _unary_rule('logistic'))  # string key, folx/wrapped_functions.py:554
+register_function('neg', neg_rule)
+register_function('add', _binary_rule('add'))
+register_function('add_any', _binary_rule('add'))
+register_function('sub', _binary_rule('sub'))
+register_function('mul', _binary_rule('mul'))
+register_function('div', _binary_rule('div'))
+register_function('dot_general', dot_general)
+register_function('reduce_sum', reduce_sum)
+register_function('reshape', reshape_rule)
+register_function('transpose', transpose_rule)
+register_function('broadcast_in_dim', broadcast_in_dim_rule)
+register_function('slice', getitem_rule)
+register_function('concatenate', concatenate_rule)
+register_function('stop_gradient', stop_gradient_rule)
+register_function('sign', sign_rule)
+register_function('reduce_max_values', reduce_max_values)
+register_function('slogdet', slogdet_wrapper)
+register_function('_multi_head_self_attention', mhsa_forward_laplacian)

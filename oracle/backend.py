@@ -174,6 +174,10 @@ def subtract(a, b):
 
 
 def multiply(a, b):
+    if not _is(a) and not _is(b):
+        da = a.data if isinstance(a, OConst) else np.asarray(a)[None]
+        db = b.data if isinstance(b, OConst) else np.asarray(b)[None]
+        return OConst(da * db)
     if _is(a) and _is(b):
         ta, tb = _bcast3(a, b)
         return OArr(*rules.mul_rule(*ta, *tb))
@@ -326,6 +330,27 @@ def amax_const(a, axis, keepdims=False):
     x = a.x if _is(a) else a.data
     ax = tuple(i % (x.ndim - 1) + 1 for i in np.atleast_1d(axis))
     return OConst(x.max(ax, keepdims=keepdims))
+
+
+def sign(a):
+    return OConst(np.sign(a.x if _is(a) else a.data))
+
+
+def squeeze(a: OArr, axis):
+    shape = list(a.shape)
+    del shape[axis % a.ndim]
+    return reshape(a, shape)
+
+
+def logsumexp(a: OArr, axis=-1, b=None):
+    """Same primitive sequence as ``jax.nn.logsumexp(..., b=b, return_sign=True)``."""
+    m = amax_const(a, axis, keepdims=True)
+    e = exp(subtract(a, m))
+    if b is not None:
+        e = multiply(e, b)
+    s = sum(e, axis)
+    val = add(log(abs(s)), OConst(m.data.reshape(s.x.shape)))
+    return val, sign(s)
 
 
 def slogdet(A: OArr):

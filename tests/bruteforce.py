@@ -128,6 +128,23 @@ class plain:
         return a.detach().amax(dim=axis, keepdim=keepdims)
 
     @staticmethod
+    def sign(a):
+        return torch.sign(a.detach())
+
+    @staticmethod
+    def squeeze(a, axis):
+        return a.squeeze(axis)
+
+    @staticmethod
+    def logsumexp(a, axis=-1, b=None):
+        m = a.detach().amax(dim=axis, keepdim=True)
+        e = torch.exp(a - m)
+        if b is not None:
+            e = e * plain._c(b, a)
+        s = e.sum(dim=axis)
+        return torch.log(torch.abs(s)) + m.reshape(s.shape), torch.sign(s.detach())
+
+    @staticmethod
     def slogdet(A):
         sign, ld = torch.linalg.slogdet(A)
         return sign.detach(), ld

@@ -1,0 +1,106 @@
+"""CPU stand-ins for ``folx_amd.kernels`` -- TEST INFRASTRUCTURE, used only by the
+``not gpu`` tests to exercise the host logic (index algebra, rule composition, masks) in
+a container without a GPU.  Each stand-in evaluates the oracle's rule in float64 and
+returns float32 torch CPU tensors.  The product never imports this module; without a GPU
+and without this patch every rule raises.
+"""
+
+import numpy as np
+import torch
+
+from oracle import index_algebra as oia
+from oracle import rules
+
+
+def _n(t):
+    return t.detach().cpu().numpy().astype(np.float64)
+
+
+def _t(a):
+    return torch.as_tensor(np.ascontiguousarray(a, dtype=np.float32))
+
+
+def dense(x, jac, lap, W, bias=None):
+    return tuple(_t(a) for a in rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias)))
+
+
+def elementwise(name, x, jac, lap, param=0.0, inplace=False):
+    nm = {'sigmoid': 'logistic'}.get(name, name)
+    return tuple(_t(a) for a in rules.elementwise_rule(nm, _n(x), _n(jac), _n(lap), param))
+
+
+def binary(op, a, aj, al, b, bj, bl):
+    rule = {'mul': rules.mul_rule, 'div': rules.div_rule, 'add': rules.add_rule,
+            'sub': lambda *t: rules.add_rule(*t, sign=-1.0)}[op]
+    A = [_n(t) for t in (a, aj, al)]
+    Bb = [_n(t) for t in (b, bj, bl)]
+    shp = np.broadcast_shapes(A[0].shape, Bb[0].shape)
+    P = A[1].shape[0]
+    A = [np.broadcast_to(A[0], shp), np.broadcast_to(A[1], (P, *shp)), np.broadcast_to(A[2], shp)]
+    Bb = [np.broadcast_to(Bb[0], shp), np.broadcast_to(Bb[1], (P, *shp)), np.broadcast_to(Bb[2], shp)]
+    return tuple(_t(t) for t in rule(*A, *Bb))
+
+
+def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta=1.0):
+    a = _n(inp).reshape(rows, *row_shape)
+    nd = len(out_shape)
+    a = a.reshape(rows, *([1] * (nd - len(row_shape))), *row_shape)
+    out = alpha * np.broadcast_to(a, (rows, *out_shape))
+    if c is not None:
+        out = out * _n(c)
+    if d is not None:
+        out = out + beta * _n(d)
+    return _t(np.broadcast_to(out, (rows, *out_shape)))
+
+
+def reduce_sum(inp, rows, outer, red, inner, alpha=1.0):
+    return _t(alpha * _n(inp).reshape(rows, outer, red, inner).sum(2))
+
+
+def reduce_max(inp, outer, red, inner):
+    return _t(_n(inp).reshape(outer, red, inner).max(1))
+
+
+def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
+    d = _n(data).reshape(data.shape[0], B, S_outer, S_inner)
+    tk = take.cpu().numpy().reshape(k_out, n_slots, S_outer)
+    out = np.zeros((k_out, B, S_outer, S_inner))
+    for t in range(k_out):
+        for s in range(n_slots):
+            for so in range(S_outer):
+                r = tk[t, s, so]
+                if r >= 0:
+                    out[t, :, so] += d[r, :, so]
+    return _t(out.reshape(k_out, B, S_outer * S_inner))
+
+
+def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
+    d = _n(data).reshape(data.shape[0], B, S_outer, S_inner)
+    ix = idx.cpu().numpy()
+    out = np.zeros((k_out, B, S_outer, S_inner))
+    for r in range(d.shape[0]):
+        for so in range(S_outer):
+            if ix[r, so] >= 0:
+                out[ix[r, so], :, so] += d[r, :, so]
+    return _t(out.reshape(k_out, B, S_outer * S_inner))
+
+
+def slogdet(A, AJ, AL):
+    sign, (ld, jac, lap) = rules.slogdet_rule(_n(A), _n(AJ), _n(AL))
+    return _t(sign), _t(ld), _t(jac), _t(lap)
+
+
+def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None):
+    m = None if mask is None else mask.cpu().numpy().astype(bool)
+    im = None if input_mask is None else input_mask.cpu().numpy().astype(bool)
+    return tuple(_t(a) for a in rules.mhsa_rule(*[_n(t) for t in (q, qj, ql, k, kj, kl, v, vj, vl)], m, im))
+
+
+def install(monkeypatch):
+    import folx_amd.interpreter as interp
+    import folx_amd.kernels as K
+
+    for name in ('dense', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
+                 'gather_rows', 'scatter_add_rows', 'slogdet', 'mhsa'):
+        monkeypatch.setattr(K, name, globals()[name])
+    monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

@@ -1,0 +1,72 @@
+"""The C-ABI library loads and exports every symbol include/folx_hip.h declares; argument
+checks reject bad calls before anything is launched (no GPU needed: nothing computes)."""
+
+import ctypes
+import os
+
+import pytest
+
+import __graft_entry__ as entry
+from folx_amd import _lib
+
+
+@pytest.fixture(scope='module')
+def lib():
+    if not os.path.exists(_lib.LIBPATH):
+        from folx_amd import build
+
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def test_exports_every_declared_symbol(lib):
+    declared = entry.declared_symbols()
+    assert len(declared) >= 12
+    assert set(declared) == set(_lib.SIGNATURES)
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_version_and_strerror(lib):
+    assert lib.folx_hip_version() >= 100
+    assert lib.folx_hip_strerror(0) == b'ok'
+    for code in (-1, -2, -3, -99):
+        assert len(lib.folx_hip_strerror(code)) > 0
+
+
+def test_argument_checks_return_error_codes(lib):
+    null = ctypes.c_void_p(None)
+    # negative sizes / null pointers -> EINVAL, nothing launched
+    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, 4, 1, 8, 8) == _lib.EINVAL
+    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, -1, 1, 8, 8) == _lib.EINVAL
+    assert lib.folx_hip_elementwise_fwdlap(null, 99, 0.0, null, null, null, null, null, null, 4, 1) == _lib.EINVAL
+    assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 4, 1) == _lib.EINVAL
+    assert lib.folx_hip_binary_fwdlap(null, 0, null, null, null, null, null, null, null, null, null, null, 1, 1, 1) == _lib.EINVAL
+    assert lib.folx_hip_rows_affine(null, null, null, 1, 1, null, null, 1.0, 1.0, null) == _lib.EINVAL
+    assert lib.folx_hip_reduce_sum(null, null, null, 1, 1, -1, 1, 1.0) == _lib.EINVAL
+    assert lib.folx_hip_slogdet_fwdlap(null, null, null, null, null, null, null, null, 4, 0, 1) == _lib.EINVAL
+    assert lib.folx_hip_mhsa_fwdlap(*([null] * 15), 1, 8, 1, 8, 1) == _lib.EINVAL
+    # empty problems are fine and launch nothing
+    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, 0, 1, 8, 8) == _lib.OK
+    assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 0, 1) == _lib.OK
+    assert lib.folx_hip_gather_rows(null, null, null, null, 1, 0, 1, 4, 4, 4) == _lib.OK
+
+
+def test_unsupported_sizes(lib):
+    one = ctypes.c_void_p(16)  # non-null, never dereferenced: the size check comes first
+    assert lib.folx_hip_slogdet_fwdlap(None, one, one, one, one, one, one, one, 4, 33, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_mhsa_fwdlap(None, *([one] * 9), None, None, one, one, one, 1, 65, 1, 8, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_mhsa_fwdlap(None, *([one] * 9), None, None, one, one, one, 1, 8, 1, 6, 1) == _lib.ENOTSUP
+
+
+def test_product_fails_loudly_without_gpu():
+    import numpy as np
+    import torch
+
+    import folx_amd
+    from folx_amd import numpy as fnp
+
+    if torch.cuda.is_available():
+        pytest.skip('GPU present')
+    with pytest.raises(_lib.FolxHipError):
+        folx_amd.forward_laplacian(lambda x: fnp.tanh(x), 0)(np.zeros(3, np.float32))

@@ -1,0 +1,253 @@
+"""Host logic of the product (rule composition, mask propagation, index tables) on CPU
+stand-ins for the kernels: results must equal the dense oracle and brute-force AD, and
+sparse / dense runs of the same model must agree."""
+
+import numpy as np
+import pytest
+import torch
+
+import cpu_kernels
+from bruteforce import brute_force, plain
+from oracle import backend as ob
+
+import folx_amd
+from folx_amd import numpy as fnp
+from folx_amd import workloads as wl
+
+
+@pytest.fixture(autouse=True)
+def _cpu(monkeypatch):
+    cpu_kernels.install(monkeypatch)
+    from folx_amd import sparse_ops
+
+    sparse_ops.clear_caches()
+
+
+def run_product(fn, x, thr):
+    out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fn(fnp, t), thr))(x)
+    return out
+
+
+def triplet_np(out):
+    return (out.x.numpy().astype(np.float64), out.jacobian.dense_array.numpy().astype(np.float64),
+            out.laplacian.numpy().astype(np.float64))
+
+
+def check_against_oracle(fn, x, thr, rtol=2e-4, atol=2e-5):
+    got = triplet_np(run_product(fn, x, thr))
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    P = ref.J.shape[0]
+    J = got[1]
+    if J.shape[0] < P:  # trailing inputs nothing depends on (dense_array is max_n + 1 rows)
+        J = np.concatenate([J, np.zeros((P - J.shape[0], *J.shape[1:]))], 0)
+    np.testing.assert_allclose(got[0], ref.x, rtol=rtol, atol=atol)
+    np.testing.assert_allclose(J, ref.J, rtol=rtol, atol=atol)
+    np.testing.assert_allclose(got[2], ref.lap, rtol=rtol, atol=atol)
+    return got
+
+
+@pytest.mark.parametrize('thr', [0, 4, 3, 100])
+def test_nodewise_mlp(thr):
+    """README example in miniature; thr=4 keeps k=4 rows, thr=3 falls back to dense."""
+    params = wl.mlp_params(seed=0, in_dim=4, width=8, n_hidden=3)
+    x = np.random.default_rng(0).normal(size=(3, 6, 4)).astype(np.float32)
+    fn = lambda xp, t: wl.mlp_forward(params, t, xp)
+    check_against_oracle(fn, x, thr)
+
+
+def test_nodewise_mlp_sparsity_pattern():
+    """k stays 4 through the hidden layers (node-wise MLP, README.md:41-70) and the final
+    sum switches to the dense Jacobian (400 > threshold)."""
+    params = wl.mlp_params(seed=0, in_dim=4, width=8, n_hidden=2)
+    x = np.random.default_rng(0).normal(size=(2, 5, 4)).astype(np.float32)
+    seen = []
+
+    def fn(t):
+        h = t
+        for W, b in params[:-1]:
+            h = fnp.silu(fnp.dot(h, W, b))
+            seen.append(h.jacobian)
+        h = fnp.dot(h, *params[-1])
+        seen.append(h.jacobian)
+        return fnp.sum(h)
+
+    out = folx_amd.vmap(folx_amd.forward_laplacian(fn, 4))(x)
+    for jac in seen:
+        assert jac.weak and jac.data.shape[0] == 4
+        # node m depends on inputs 4m .. 4m+3, ascending, identical across features
+        want = (4 * np.arange(5)[None, :, None] + np.arange(4)[:, None, None])
+        np.testing.assert_array_equal(jac.x0_idx, np.broadcast_to(want, jac.x0_idx.shape))
+    assert not out.jacobian.weak and out.jacobian.data.shape[0] == 20
+
+
+BINARY_FNS = {
+    'same_mask_mul': lambda xp, x: xp.multiply(xp.tanh(x), xp.exp(x)),
+    'same_mask_div': lambda xp, x: xp.divide(xp.sin(x), xp.add(xp.square(x), 1.0)),
+    'diff_mask_sub': lambda xp, x: xp.subtract(xp.expand_dims(x, 1), xp.expand_dims(xp.tanh(x), 0)),
+    'diff_mask_mul': lambda xp, x: xp.multiply(xp.expand_dims(x, 1), xp.expand_dims(xp.sin(x), 0)),
+    'diff_mask_div': lambda xp, x: xp.divide(xp.expand_dims(x, 1), xp.add(xp.expand_dims(xp.square(x), 0), 1.0)),
+    'dup_then_unary': lambda xp, x: xp.tanh(xp.add(xp.expand_dims(x, 1), xp.expand_dims(x, 0))),
+    'const_ops': lambda xp, x: xp.divide(2.0, xp.add(xp.multiply(xp.subtract(1.5, x), np.arange(1, 4.0)), 7.0)),
+}
+
+
+@pytest.mark.parametrize('name', sorted(BINARY_FNS))
+@pytest.mark.parametrize('thr', [0, 2, 6, 100])
+def test_binary_rules(name, thr):
+    x = np.random.default_rng(1).normal(size=(2, 4, 3)).astype(np.float32)
+    got = check_against_oracle(BINARY_FNS[name], x, thr)
+    by, bJ, bL = brute_force(lambda t: BINARY_FNS[name](plain, t), x.astype(np.float64))
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-5)
+
+
+def test_duplicate_mask_layout_follows_reference():
+    """x[:, None] + x[None, :] concatenates the two one-row masks (folx/jvp.py:294-317):
+    k = 2 with the diagonal listing the same input twice; the following tanh keeps the
+    rows (folx/jvp.py:262-272) and takes its Hessian term on the unique frame."""
+    x = np.random.default_rng(2).normal(size=(1, 3)).astype(np.float32)
+
+    def fn(t):
+        s = fnp.add(fnp.expand_dims(t, 1), fnp.expand_dims(t, 0))
+        assert s.jacobian.x0_idx.shape == (2, 3, 3)
+        np.testing.assert_array_equal(s.jacobian.x0_idx[:, 1, 1], [1, 1])
+        return fnp.tanh(s)
+
+    out = folx_amd.vmap(folx_amd.forward_laplacian(fn, 4))(x)
+    assert out.jacobian.x0_idx.shape == (2, 3, 3)
+    xs = x[0].astype(np.float64)
+    s = xs[:, None] + xs[None, :]
+    t = np.tanh(s)
+    cnt = np.where(np.eye(3, dtype=bool), 4.0, 2.0)  # |grad s|^2: (2)^2 on the diagonal, 1 + 1 off it
+    np.testing.assert_allclose(out.laplacian[0].numpy(), -2 * t * (1 - t * t) * cnt, rtol=1e-5, atol=1e-6)
+
+
+REDUCE_FNS = {
+    'sum_all': lambda xp, x: xp.sum(xp.tanh(x)),
+    'sum_last': lambda xp, x: xp.sum(xp.square(x), axis=-1),
+    'sum_first_keep': lambda xp, x: xp.sum(xp.exp(x), axis=0, keepdims=True),
+    'mean_mid': lambda xp, x: xp.mean(xp.sin(xp.expand_dims(x, 1) * 1.0 if xp is plain else xp.multiply(xp.expand_dims(x, 1), 1.0)), axis=1),
+    'dist': lambda xp, x: xp.sqrt(xp.sum(xp.square(xp.subtract(xp.expand_dims(x, 1), np.arange(6.0).reshape(2, 3))), axis=-1)),
+}
+
+
+@pytest.mark.parametrize('name', sorted(REDUCE_FNS))
+@pytest.mark.parametrize('thr', [0, 3, 12])
+def test_reductions(name, thr):
+    x = np.random.default_rng(3).normal(size=(2, 4, 3)).astype(np.float32)
+    check_against_oracle(REDUCE_FNS[name], x, thr)
+
+
+def test_indexing_rules():
+    R = np.random.default_rng(4).normal(size=(2, 3))
+
+    def fn(xp, r):
+        d = xp.subtract(xp.expand_dims(r, 1), R)
+        dist = xp.sqrt(xp.sum(xp.square(d), axis=-1))
+        f = xp.concatenate([xp.reshape(d, (4, 6)), dist, np.ones((4, 1))], axis=-1)
+        f = xp.transpose(f, (1, 0))
+        return xp.getitem(f, (slice(1, 8),))
+
+    x = np.random.default_rng(5).normal(size=(2, 4, 3)).astype(np.float32)
+    for thr in (0, 3, 6):
+        check_against_oracle(fn, x, thr)
+    # constants keep sparsity (test/test_layers.py:763-776): k stays 3 after the concat
+    out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fn(fnp, t), 6))(x)
+    assert out.jacobian.weak and out.jacobian.data.shape[0] == 3
+
+
+def test_operator_and_single_sample_api():
+    """README.md:22-33: f(x) = sum x^2 at arange(3) -> 5, [0, 2, 4], 6."""
+    f = lambda x: fnp.sum(fnp.square(x))
+    for thr in (0, 3):
+        res = folx_amd.forward_laplacian(f, thr)(np.arange(3, dtype=np.float32))
+        assert float(res.x[0]) == 5.0
+        np.testing.assert_allclose(res.jacobian.dense_array[:, 0].numpy(), [0, 2, 4])
+        assert float(res.laplacian[0]) == 6.0
+        lap, jac = folx_amd.ForwardLaplacianOperator(thr)(f)(np.arange(3, dtype=np.float32))
+        assert float(lap) == 6.0 and jac.shape == (3,)
+
+
+def test_weights_argument():
+    f = lambda x: fnp.sum(fnp.exp(x))
+    x = np.array([[0.1, -0.3, 0.7]], dtype=np.float32)
+    w = np.array([1.0, 0.0, 2.0], dtype=np.float32)
+    for thr in (0, 3):
+        res = folx_amd.forward_laplacian(f, thr).batched(x, weights=w)
+        np.testing.assert_allclose(res.jacobian.dense_array[:, 0].numpy(), np.exp(x[0]) * w, rtol=1e-6)
+        np.testing.assert_allclose(float(res.laplacian[0]), (np.exp(x[0]) * w * w).sum(), rtol=1e-6)
+
+
+def test_batched_vmap_chunks():
+    f = lambda x: fnp.sum(fnp.tanh(x))
+    x = np.random.default_rng(6).normal(size=(7, 5)).astype(np.float32)
+    full = folx_amd.vmap(folx_amd.forward_laplacian(f, 0))(x)
+    for mb in (2, 3, 7, 10):
+        part = folx_amd.batched_vmap(folx_amd.forward_laplacian(f, 0), mb)(x)
+        np.testing.assert_allclose(part.x.numpy(), full.x.numpy())
+        np.testing.assert_allclose(part.laplacian.numpy(), full.laplacian.numpy())
+        np.testing.assert_allclose(part.jacobian.data.numpy(), full.jacobian.data.numpy())
+
+
+def test_register_function_plugs_in():
+    calls = []
+
+    def my_tanh(args, kwargs, sparsity_threshold):
+        calls.append(sparsity_threshold)
+        return folx_amd.wrapped_functions._unary_rule('tanh')(args, kwargs, sparsity_threshold)
+
+    old = folx_amd.get_laplacian('tanh')
+    folx_amd.register_function('tanh', my_tanh)
+    try:
+        folx_amd.forward_laplacian(lambda x: fnp.tanh(x), 5)(np.zeros(2, np.float32))
+    finally:
+        folx_amd.register_function('tanh', old)
+    assert calls == [5]
+    folx_amd.register_function('my_op', my_tanh)
+    assert folx_amd.is_registered('my_op')
+    folx_amd.deregister_function('my_op')
+    assert not folx_amd.is_registered('my_op')
+    with pytest.raises(KeyError):
+        folx_amd.get_laplacian('no_such_primitive', wrap_if_missing=True)
+
+
+SMALL_PSI = wl.PsiFormerConfig(n_elec=4, n_nuc=2, n_layers=2, n_heads=2, head_dim=4, width=8, mlp_width=8, n_det=2)
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_psiformer_small_vs_oracle_and_bruteforce(thr):
+    p = wl.psiformer_params(SMALL_PSI)
+    x = wl.sample_electrons(2, SMALL_PSI.n_elec, 1.0, seed=3)
+    fn = lambda xp, t: wl.psiformer_forward(p, t, xp)
+    got = check_against_oracle(fn, x, thr, rtol=5e-4, atol=5e-5)
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    np.testing.assert_allclose(ref.x, by, rtol=1e-8)
+    np.testing.assert_allclose(ref.J, bJ, rtol=1e-6, atol=1e-9)
+    np.testing.assert_allclose(ref.lap, bL, rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(got[2], bL, rtol=5e-4, atol=5e-5)
+
+
+def test_psiformer_sparse_stage_keeps_three_rows():
+    """Before the first attention layer every per-electron quantity depends on that
+    electron's three coordinates only: k = 3 with thr = 6 (README.md:72)."""
+    p = wl.psiformer_params(SMALL_PSI)
+    x = wl.sample_electrons(2, SMALL_PSI.n_elec, 1.0, seed=3)
+    seen = {}
+
+    def fn(r):
+        d, dist = wl.electron_nuclear_features(fnp, r, p.nuclei)
+        seen['d'], seen['dist'] = d.jacobian, dist.jacobian
+        feats = fnp.concatenate([fnp.reshape(d, (4, 6)), dist, p.spin], axis=-1)
+        h = fnp.dot(feats, p.w_in)
+        seen['h'] = h.jacobian
+        hn = wl.layer_norm(fnp, h, p.layers[0]['ln1_g'], p.layers[0]['ln1_b'], 1e-5)
+        seen['ln'] = hn.jacobian
+        return fnp.sum(hn)
+
+    folx_amd.vmap(folx_amd.forward_laplacian(fn, 6))(x)
+    assert seen['d'].x0_idx.shape[0] == 1 and seen['dist'].x0_idx.shape[0] == 3
+    for key in ('h', 'ln'):
+        jac = seen[key]
+        assert jac.weak and jac.x0_idx.shape[0] == 3
+        want = 3 * np.arange(4)[None, :, None] + np.arange(3)[:, None, None]
+        np.testing.assert_array_equal(jac.x0_idx, np.broadcast_to(want, jac.x0_idx.shape))
