@@ -34,6 +34,8 @@ def parse():
     ap.add_argument('--chunk', type=int, default=1024, help='walkers per batched_vmap chunk')
     ap.add_argument('--cpu-seconds', type=float, default=20.0, help='budget of the CPU baseline sample')
     ap.add_argument('--no-cpu', action='store_true')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also launch one plain copy (rows_affine, 1 GiB in, 1 GiB out) for scaling HBM counters')
     return ap.parse_args()
 
 
@@ -98,6 +100,12 @@ def main():
     for _ in range(args.warmup):
         out = step(x)
     torch.cuda.synchronize()
+    if args.calibrate_copy:
+        n = 1 << 28  # 2^28 floats = 1 GiB read + 1 GiB written by rows_affine_kernel
+        src = torch.empty(n, device=dev, dtype=torch.float32).fill_(1.0)
+        K.rows_affine(src, 1, (n,), (n,), None, None, 1.0, 0.0)
+        torch.cuda.synchronize()
+        del src
 
     with K.LaunchTimer() as lt:
         torch.cuda.synchronize()

@@ -27,6 +27,7 @@ SOURCES = [
     'gather.hip',
     'slogdet.hip',
     'mhsa.hip',
+    'layernorm.hip',
 ]
 
 # Packed FP32 instructions are switched off for all device code (-packed-fp32-ops).

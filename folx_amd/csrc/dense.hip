@@ -1,49 +1,61 @@
-// Dense-layer rule: y = h @ W (+ bias) over the stacked operand [x; J; lap].
+// Dense-layer rule: y = h @ W (+ bias) (+ residual) over the stacked operand [x; J; lap].
 //
 // All (P + 2) * R rows go through ONE launch of an LDS-tiled FP32-MFMA GEMM
 // (v_mfma_f32_32x32x2_f32).  The three operands are separate allocations, so the row
 // tiles are laid out per segment (x, jac, lap) and never straddle two of them.
 //
-// Tiling: a workgroup of 4 wavefronts owns BM = 128 rows x BN columns and walks K in
-// chunks of BK = 32 through double-buffered LDS tiles (global -> registers -> LDS, one
-// barrier per chunk).  A rows are stored [row][k] with a stride of 36 floats: a lane
-// fetches 4 consecutive k with one 128-bit LDS read, and the rows of 8 consecutive lanes
-// fall into distinct bank groups.  The MFMA only needs A and B to agree on which k a
-// lane holds, so the k order inside a chunk is permuted to fit that read:
+// Tiling: a workgroup owns BM rows x BN columns and walks K in chunks of BK = 16 through
+// double-buffered LDS tiles (global -> registers -> LDS, one barrier per chunk).  For
+// N > 128 the tile is 256 x 256 on 8 wavefronts (each 64 x 128), so a layer of width 256
+// reads its A rows from HBM exactly once; narrower layers use 128 x {128, 64, 32} tiles on
+// 4 wavefronts.  A rows are stored [row][k] with a stride of BK + 4 floats: a lane fetches
+// 4 consecutive k with one 128-bit LDS read and the rows of 8 consecutive lanes fall into
+// distinct bank groups.  The MFMA only needs A and B to agree on which k a lane holds, so
+// the k order inside a group of 8 is permuted to fit that read:
 //     lane l, register j of group t  <->  k = 8 t + 4 (l / 32) + j.
-// W rows are stored [k][n], read with consecutive n across lanes.
+// W rows are stored [k][n] and read with consecutive n across lanes.
+//
+// Global loads of the vector path are branch free: out-of-range rows / columns are clamped
+// to a valid address and zeroed by a select, so the loads of the next chunk issue
+// back to back ahead of the MFMAs of the current one.
 //
 // Workgroup ids are remapped so that the column tiles of one row tile run back to back
 // on the same XCD (ids are dealt round-robin to the 8 XCDs), which keeps the second
-// read of an A tile in that XCD's L2.
+// read of an A tile in that XCD's L2 when N needs more than one column tile.
 #include "common.h"
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128;
-constexpr int BK = 32;
+constexpr int BK = 16;
 constexpr int AS = BK + 4;  // LDS row stride of the A tile (floats)
 constexpr int NXCD = 8;
 
 struct Segs {
   const float* in[3];
+  const float* res[3];  // optional residual (same shape as out) added in the epilogue
   float* out[3];
   int64_t rows[3];
   int64_t tiles[3];
 };
 
-template <int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void dense_kernel(Segs sg, const float* __restrict__ W,
-                                                    const float* __restrict__ bias, int32_t K,
-                                                    int32_t N, int64_t row_tiles, int32_t col_tiles,
-                                                    int vecA, int vecW) {
+template <int BM, int BN, int WM, int WN, int MINB, bool VEC, bool HAS_RES>
+__global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, const float* __restrict__ W,
+                                                                   const float* __restrict__ bias,
+                                                                   int32_t K, int32_t N,
+                                                                   int64_t row_tiles,
+                                                                   int32_t col_tiles) {
+  constexpr int NT = 64 * WM * WN;
   constexpr int WROWS = BM / WM;  // rows per wavefront
   constexpr int WCOLS = BN / WN;  // columns per wavefront
   constexpr int TM = WROWS / 32;
   constexpr int TN = WCOLS / 32;
-  static_assert(WM * WN == 4, "4 wavefronts");
+  constexpr int TG = BK / 8;
+  constexpr int A_V4 = BM * BK / 4;                 // float4 of one A chunk
+  constexpr int W_V4 = BK * BN / 4;                 // float4 of one W chunk
+  constexpr int A_LD = (A_V4 + NT - 1) / NT;
+  constexpr int W_LD = (W_V4 + NT - 1) / NT;
 
   __shared__ __attribute__((aligned(16))) float As[2][BM * AS];
   __shared__ __attribute__((aligned(16))) float Ws[2][BK * BN];
@@ -81,72 +93,84 @@ __global__ __launch_bounds__(256) void dense_kernel(Segs sg, const float* __rest
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  constexpr int A_LD = BM * BK / 4 / 256;  // float4 loads per thread for the A tile
-  constexpr int W_LD = BK * BN / 4 / 256;  // float4 loads per thread for the W tile
-  float4 ra[A_LD];
-  float4 rw[W_LD];
+  float4 ra[A_LD], rw[W_LD];
+
+  // per-thread source rows / columns are fixed over the K loop
+  int a_r[A_LD], a_k[A_LD], w_k[W_LD], w_n[W_LD];
+  bool a_ok[A_LD], w_ok[W_LD];
+  const float* a_p[A_LD];
+  const float* w_p[W_LD];
+#pragma unroll
+  for (int i = 0; i < A_LD; ++i) {
+    const int idx = tid + NT * i;
+    a_r[i] = idx / (BK / 4);
+    a_k[i] = (idx % (BK / 4)) * 4;
+    int64_t gr = row0 + a_r[i];
+    a_ok[i] = (A_V4 % NT == 0 || idx < A_V4) && gr < rows;
+    if (gr >= rows) gr = rows - 1;
+    a_p[i] = A + gr * (int64_t)K;
+  }
+#pragma unroll
+  for (int i = 0; i < W_LD; ++i) {
+    const int idx = tid + NT * i;
+    w_k[i] = idx / (BN / 4);
+    w_n[i] = (idx % (BN / 4)) * 4;
+    w_ok[i] = (W_V4 % NT == 0 || idx < W_V4) && (col0 + w_n[i] < N);
+    w_p[i] = W + (w_ok[i] ? col0 + w_n[i] : 0);
+  }
 
   auto load_global = [&](int kt) {
     const int k0 = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
-      const int idx = tid + 256 * i;
-      const int r = idx / (BK / 4);
-      const int kq = (idx % (BK / 4)) * 4;
-      const int64_t gr = row0 + r;
-      const int gk = k0 + kq;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (gr < rows) {
-        const float* src = A + gr * (int64_t)K + gk;
-        if (vecA && gk + 3 < K) {
-          v = *reinterpret_cast<const float4*>(src);
-        } else {
+      const int gk = k0 + a_k[i];
+      if constexpr (VEC) {
+        const bool ok = a_ok[i] && gk < K;
+        const float4 v = *reinterpret_cast<const float4*>(a_p[i] + (gk < K ? gk : 0));
+        ra[i] = ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a_ok[i]) {
+          const float* src = a_p[i] + gk;
           if (gk + 0 < K) v.x = src[0];
           if (gk + 1 < K) v.y = src[1];
           if (gk + 2 < K) v.z = src[2];
           if (gk + 3 < K) v.w = src[3];
         }
+        ra[i] = v;
       }
-      ra[i] = v;
     }
 #pragma unroll
     for (int i = 0; i < W_LD; ++i) {
-      const int idx = tid + 256 * i;
-      const int kk = idx / (BN / 4);
-      const int nq = (idx % (BN / 4)) * 4;
-      const int gk = k0 + kk;
-      const int gn = col0 + nq;
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (gk < K) {
-        const float* src = W + (int64_t)gk * N + gn;
-        if (vecW && gn + 3 < N) {
-          v = *reinterpret_cast<const float4*>(src);
-        } else {
+      const int gk = k0 + w_k[i];
+      if constexpr (VEC) {
+        const bool ok = w_ok[i] && gk < K;
+        const float4 v = *reinterpret_cast<const float4*>(w_p[i] + (int64_t)(gk < K ? gk : 0) * N);
+        rw[i] = ok ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((W_V4 % NT == 0 || tid + NT * i < W_V4) && gk < K) {
+          const int gn = col0 + w_n[i];
+          const float* src = W + (int64_t)gk * N + gn;
           if (gn + 0 < N) v.x = src[0];
           if (gn + 1 < N) v.y = src[1];
           if (gn + 2 < N) v.z = src[2];
           if (gn + 3 < N) v.w = src[3];
         }
+        rw[i] = v;
       }
-      rw[i] = v;
     }
   };
 
   auto store_lds = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i) {
-      const int idx = tid + 256 * i;
-      const int r = idx / (BK / 4);
-      const int kq = (idx % (BK / 4)) * 4;
-      *reinterpret_cast<float4*>(&As[buf][r * AS + kq]) = ra[i];
-    }
+    for (int i = 0; i < A_LD; ++i)
+      if (A_V4 % NT == 0 || tid + NT * i < A_V4)
+        *reinterpret_cast<float4*>(&As[buf][a_r[i] * AS + a_k[i]]) = ra[i];
 #pragma unroll
-    for (int i = 0; i < W_LD; ++i) {
-      const int idx = tid + 256 * i;
-      const int kk = idx / (BN / 4);
-      const int nq = (idx % (BN / 4)) * 4;
-      *reinterpret_cast<float4*>(&Ws[buf][kk * BN + nq]) = rw[i];
-    }
+    for (int i = 0; i < W_LD; ++i)
+      if (W_V4 % NT == 0 || tid + NT * i < W_V4)
+        *reinterpret_cast<float4*>(&Ws[buf][w_k[i] * BN + w_n[i]]) = rw[i];
   };
 
   const int KT = (K + BK - 1) / BK;
@@ -159,7 +183,7 @@ __global__ __launch_bounds__(256) void dense_kernel(Segs sg, const float* __rest
     if (kt + 1 < KT) load_global(kt + 1);
 
 #pragma unroll
-    for (int tg = 0; tg < BK / 8; ++tg) {
+    for (int tg = 0; tg < TG; ++tg) {
       float4 a4[TM];
       float b[TN][4];
 #pragma unroll
@@ -186,53 +210,85 @@ __global__ __launch_bounds__(256) void dense_kernel(Segs sg, const float* __rest
   }
 
   // Epilogue: register r of a 32x32 tile holds row 8 (r / 4) + 4 (lane / 32) + r % 4,
-  // column lane % 32, so each store instruction writes two 128-byte row segments.
+  // column lane % 32, so each store instruction writes two 128-byte row segments.  The
+  // residual of a sub-tile is fetched as a block before that sub-tile is stored.
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int gc = col0 + wc + j * 32 + l32;
-      if (gc < N) {
-        const float bv = (seg == 0 && bias != nullptr) ? bias[gc] : 0.0f;
+      const bool cok = gc < N;
+      const float bv = (seg == 0 && bias != nullptr && cok) ? bias[gc] : 0.0f;
+      float rs[16];
+      if constexpr (HAS_RES) {
+        const float* __restrict__ Rs = sg.res[seg];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int64_t gr = row0 + wr + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+          const bool ok = cok && gr < rows;
+          if (gr >= rows) gr = rows - 1;
+          const float v = Rs[gr * (int64_t)N + (cok ? gc : 0)];
+          rs[r] = ok ? v : 0.0f;
+        }
+      }
+      if (cok) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int64_t gr = row0 + wr + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-          if (gr < rows) C[gr * (int64_t)N + gc] = acc[i][j][r] + bv;
+          float o = acc[i][j][r] + bv;
+          if constexpr (HAS_RES) o += rs[r];
+          if (gr < rows) C[gr * (int64_t)N + gc] = o;
         }
       }
     }
   }
 }
 
+template <int BM, int BN, int WM, int WN, int MINB>
+int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int32_t K, int32_t N,
+               bool vec, bool has_res) {
+  int64_t row_tiles = 0;
+  for (int s = 0; s < 3; ++s) { sg.tiles[s] = (sg.rows[s] + BM - 1) / BM; row_tiles += sg.tiles[s]; }
+  const int32_t col_tiles = (N + BN - 1) / BN;
+  const int64_t groups = (row_tiles + NXCD - 1) / NXCD;
+  const int64_t blocks = groups * NXCD * col_tiles;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  dim3 grid((unsigned)blocks), block(64 * WM * WN);
+  if (vec && has_res)
+    dense_kernel<BM, BN, WM, WN, MINB, true, true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+  else if (vec)
+    dense_kernel<BM, BN, WM, WN, MINB, true, false><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+  else if (has_res)
+    dense_kernel<BM, BN, WM, WN, MINB, false, true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+  else
+    dense_kernel<BM, BN, WM, WN, MINB, false, false><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+  return folx_launch_status();
+}
+
 }  // namespace
 
 extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac,
                                      const float* lap, const float* W, const float* bias,
+                                     const float* res, const float* res_jac, const float* res_lap,
                                      float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
                                      int32_t K, int32_t N) {
   if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
   if (R == 0) return FOLX_HIP_OK;
   if (!x || !lap || !W || !y || !y_lap || (P > 0 && (!jac || !y_jac))) return FOLX_HIP_EINVAL;
+  if ((res != nullptr) != (res_lap != nullptr) || (P > 0 && (res != nullptr) != (res_jac != nullptr)))
+    return FOLX_HIP_EINVAL;
   Segs sg;
+  sg.res[0] = res; sg.res[1] = res_jac; sg.res[2] = res_lap;
   sg.in[0] = x; sg.in[1] = jac; sg.in[2] = lap;
   sg.out[0] = y; sg.out[1] = y_jac; sg.out[2] = y_lap;
   sg.rows[0] = R; sg.rows[1] = (int64_t)P * R; sg.rows[2] = R;
-  int64_t row_tiles = 0;
-  for (int s = 0; s < 3; ++s) { sg.tiles[s] = (sg.rows[s] + BM - 1) / BM; row_tiles += sg.tiles[s]; }
-  const int vecA = (K % 4 == 0) && folx_aligned16(x) && folx_aligned16(jac) && folx_aligned16(lap);
-  const int vecW = (N % 4 == 0) && folx_aligned16(W);
-  const int BN = N > 64 ? 128 : (N > 32 ? 64 : 32);
-  const int32_t col_tiles = (N + BN - 1) / BN;
-  const int64_t groups = (row_tiles + NXCD - 1) / NXCD;
-  const int64_t blocks = groups * NXCD * col_tiles;
-  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  if (P == 0) { sg.in[1] = x; sg.out[1] = y; sg.res[1] = res; }  // never dereferenced: 0 tiles
+  const bool vec = (K % 4 == 0) && (N % 4 == 0) && folx_aligned16(x) && folx_aligned16(jac) &&
+                   folx_aligned16(lap) && folx_aligned16(W);
+  const bool has_res = res != nullptr;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)blocks), block(256);
-  if (BN == 128)
-    dense_kernel<128, 2, 2><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles, vecA, vecW);
-  else if (BN == 64)
-    dense_kernel<64, 4, 1><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles, vecA, vecW);
-  else
-    dense_kernel<32, 4, 1><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles, vecA, vecW);
-  return folx_launch_status();
+  if (N > 128) return launch_cfg<256, 256, 4, 2, 1>(st, sg, W, bias, K, N, vec, has_res);
+  if (N > 64) return launch_cfg<128, 128, 2, 2, 3>(st, sg, W, bias, K, N, vec, has_res);
+  if (N > 32) return launch_cfg<128, 64, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);
+  return launch_cfg<128, 32, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);
 }

@@ -92,9 +92,13 @@ def _dims(*vals):
     return (ctypes.c_int64 * len(vals))(*[int(v) for v in vals])
 
 
-def dense(x, jac, lap, W, bias=None):
-    """x (.., K), jac (P, .., K), lap (.., K), W (K, N) -> triplet with last dim N."""
+def dense(x, jac, lap, W, bias=None, res=None):
+    """x (.., K), jac (P, .., K), lap (.., K), W (K, N) -> triplet with last dim N.
+    ``res`` = optional (x, jac, lap) residual triplet of the output shape, added in the
+    GEMM epilogue."""
     _chk(x, jac, lap, W, bias)
+    rx, rj, rl = res if res is not None else (None, None, None)
+    _chk(rx, rj, rl)
     K, N = W.shape
     P = jac.shape[0]
     R = x.numel() // K
@@ -104,7 +108,8 @@ def dense(x, jac, lap, W, bias=None):
     with _timed('dense_fwdlap', (R, P, K, N)):
         check(
             _lib.load().folx_hip_dense_fwdlap(
-                _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(y), _p(yj), _p(yl), R, P, K, N
+                _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(rx), _p(rj), _p(rl),
+                _p(y), _p(yj), _p(yl), R, P, K, N
             ),
             'dense_fwdlap',
         )
@@ -125,6 +130,23 @@ def elementwise(name, x, jac, lap, param=0.0, inplace=False):
                 _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(y), _p(yj), _p(yl), S, P
             ),
             f'elementwise_fwdlap[{name}]',
+        )
+    return y, yj, yl
+
+
+def layernorm(x, jac, lap, gamma, beta, eps):
+    """Fused LayerNorm rule over the last axis."""
+    _chk(x, jac, lap, gamma, beta)
+    F = x.shape[-1]
+    R = x.numel() // F
+    P = jac.shape[0]
+    y, yj, yl = torch.empty_like(x), torch.empty_like(jac), torch.empty_like(lap)
+    with _timed('layernorm_fwdlap', (R, F, P)):
+        check(
+            _lib.load().folx_hip_layernorm_fwdlap(
+                _stream(), _p(x), _p(jac), _p(lap), _p(gamma), _p(beta), _p(y), _p(yj), _p(yl), R, F, P, float(eps)
+            ),
+            'layernorm_fwdlap',
         )
     return y, yj, yl
 

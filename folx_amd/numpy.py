@@ -80,9 +80,15 @@ def divide(a, b):
 
 
 # linear algebra ----------------------------------------------------------------------------
-def dot(h, W, b=None):
-    """``h @ W (+ b)``: last axis of ``h`` against the first axis of the constant ``W``."""
-    return _call('dot_general', (h, W), {'bias': b})
+def dot(h, W, b=None, residual=None):
+    """``h @ W (+ b) (+ residual)``: last axis of ``h`` against the first axis of the
+    constant ``W``; ``residual`` is a triplet of the output shape (skip connection)."""
+    return _call('dot_general', (h, W), {'bias': b, 'residual': residual})
+
+
+def layer_norm(h, gamma=None, beta=None, eps=1e-5):
+    """LayerNorm over the last axis (one fused rule; same result as the primitive chain)."""
+    return _call('layer_norm', (h, gamma, beta), {'eps': eps})
 
 
 def slogdet(A):

@@ -140,13 +140,17 @@ def to_device(params, device):
     return conv(params)
 
 
-def layer_norm(xp, h, g, b, eps):
+def layer_norm_primitives(xp, h, g, b, eps):
     """LayerNorm over the feature axis from primitives (what flax's LayerNorm lowers to)."""
     mu = xp.mean(h, axis=-1, keepdims=True)
     c = xp.subtract(h, mu)
     var = xp.mean(xp.square(c), axis=-1, keepdims=True)
     y = xp.multiply(c, xp.rsqrt(xp.add(var, eps)))
     return xp.add(xp.multiply(y, g), b)
+
+
+def layer_norm(xp, h, g, b, eps):
+    return xp.layer_norm(h, g, b, eps)
 
 
 def electron_nuclear_features(xp, r, nuclei):
@@ -172,9 +176,9 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         k = xp.reshape(xp.dot(hn, L['w_k']), (n, H, dh))
         v = xp.reshape(xp.dot(hn, L['w_v']), (n, H, dh))
         att = xp.multi_head_self_attention(q, k, v)
-        h = xp.add(h, xp.dot(xp.reshape(att, (n, H * dh)), L['w_o']))
+        h = xp.dot(xp.reshape(att, (n, H * dh)), L['w_o'], None, residual=h)
         hn = layer_norm(xp, h, L['ln2_g'], L['ln2_b'], cfg.ln_eps)
-        h = xp.add(h, xp.dot(xp.tanh(xp.dot(hn, L['w_1'], L['b_1'])), L['w_2'], L['b_2']))
+        h = xp.dot(xp.tanh(xp.dot(hn, L['w_1'], L['b_1'])), L['w_2'], L['b_2'], residual=h)
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, cfg.n_up), (cfg.n_up, n)]):
         m = hi - lo

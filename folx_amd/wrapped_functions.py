@@ -386,7 +386,9 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     contracted with the first axis of a constant matrix ``W (K, N)``
     (``_dot_general_one_constant``, folx/wrapped_functions.py:71-171): the product is
     applied to x, to every Jacobian row and to the Laplacian in one GEMM launch.
-    ``kwargs['bias']`` (constant, shape (N,)) is added to x only.
+    ``kwargs['bias']`` (constant, shape (N,)) is added to x only.  ``kwargs['residual']``
+    (a triplet of the output shape) is added to the result; with matching dense Jacobians
+    the addition happens in the GEMM epilogue, otherwise through the ``add`` rule.
 
     Sparse ``h``: rows pass through when the mask is constant along the contracted axis;
     otherwise they are first aligned to the per-position union frame over that axis
@@ -395,6 +397,7 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     """
     h, W = args
     bias = kwargs.get('bias')
+    residual = kwargs.get('residual')
     if not _is(h):
         if _is(W):
             raise NotImplementedError('dot_general: constant @ triplet is not supported; transpose the product')
@@ -423,8 +426,51 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
             if aligned:
                 J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
             new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
-    y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt)
-    return FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
+    res = None
+    if residual is not None and _is(residual):
+        rj = residual.jacobian
+        if (
+            new_mask is None and not rj.weak and rj.data.shape[0] == J.shape[0]
+            and tuple(residual.shape) == (*h.shape[:-1], N)
+        ):
+            res, residual = (residual.x, rj.data, residual.laplacian), None
+    y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt, res)
+    out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
+    if residual is not None:
+        out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)
+    return out
+
+
+def layer_norm_rule(args, kwargs, sparsity_threshold):
+    """Fused rule of ``layer_norm(h, gamma, beta, eps)`` over the last axis -- a custom
+    registered function in the way the reference registers its attention kernel
+    (folx/experimental/pallas/attention/__init__.py:45).  The fused kernel applies when the
+    Jacobian is dense, or sparse with a mask that is constant along the feature axis and
+    lists no index twice (every op of the chain then keeps the rows and the mask); other
+    inputs go through the chain of primitive rules."""
+    h, gamma, beta = args
+    eps = float(kwargs.get('eps', 1e-5))
+    F = h.shape[-1]
+    mask = h.jacobian.x0_idx
+    fusable = F % 4 == 0 and F <= 1024
+    if fusable and mask is not None:
+        first = np.take(mask, [0], axis=-1)
+        fusable = bool((mask == first).all()) and not ia.has_duplicates(mask)
+    if not fusable:
+        from . import numpy as fnp
+
+        mu = fnp.mean(h, axis=-1, keepdims=True)
+        c = fnp.subtract(h, mu)
+        var = fnp.mean(fnp.square(c), axis=-1, keepdims=True)
+        y = fnp.multiply(c, fnp.rsqrt(fnp.add(var, eps)))
+        if gamma is not None:
+            y = fnp.multiply(y, gamma)
+        return y if beta is None else fnp.add(y, beta)
+    dev = h.x.device
+    g = None if gamma is None else so.device_const(gamma, dev)
+    b = None if beta is None else so.device_const(beta, dev)
+    y, Jy, lapy = K.layernorm(h.x, h.jacobian.data, h.laplacian, g, b, eps)
+    return FwdLaplArray(y, FwdJacobian(Jy, mask), lapy)
 
 
 # --------------------------------------------------------------------------------------
@@ -768,6 +814,7 @@ register_function('sub', _binary_rule('sub'))
 register_function('mul', _binary_rule('mul'))
 register_function('div', _binary_rule('div'))
 register_function('dot_general', dot_general)
+register_function('layer_norm', layer_norm_rule)
 register_function('reduce_sum', reduce_sum)
 register_function('reshape', reshape_rule)
 register_function('transpose', transpose_rule)

@@ -72,11 +72,15 @@ enum folx_hip_binop {
  * dot_generals at :167-169) for a constant right operand contracted with the last axis.
  *   x   [R][K]      jac [P][R][K]     lap [R][K]       R = walkers * positions
  *   W   [K][N] row-major, shared by all rows;  bias [N] or NULL (added to y only)
+ *   res [R][N]      res_jac [P][R][N] res_lap [R][N]   optional residual triplet (all three
+ *       NULL or all three set) added in the epilogue: the `add` rule that follows a
+ *       residual branch (LINEAR, folx/wrapped_functions.py:365-367) fused into the GEMM
  *   y   [R][N]      y_jac [P][R][N]   y_lap [R][N]
  * One launch covers all (P + 2) * R rows (FP32 MFMA, fp32 accumulate).
  */
 int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac, const float* lap,
-                          const float* W, const float* bias, float* y, float* y_jac,
+                          const float* W, const float* bias, const float* res,
+                          const float* res_jac, const float* res_lap, float* y, float* y_jac,
                           float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N);
 
 /*
@@ -105,6 +109,20 @@ int folx_hip_binary_fwdlap(void* stream, int32_t op, const float* a, const float
                            const float* a_lap, const float* b, const float* b_jac,
                            const float* b_lap, float* y, float* y_jac, float* y_lap,
                            const int64_t* dims, int64_t a_S, int64_t b_S, int32_t P);
+
+/*
+ * Fused LayerNorm over the last axis, y = gamma * (x - mean) * rsqrt(var + eps) + beta,
+ * for R rows of F features (F % 4 == 0, F <= 1024); gamma / beta [F] or NULL.
+ *   x [R][F]   jac [P][R][F]   lap [R][F]   ->   y, y_jac, y_lap of the same shapes.
+ * The reference has no LayerNorm rule of its own: it interprets the primitive chain
+ * reduce_sum / sub / square / reduce_sum / rsqrt / mul / add with the LINEAR, elementwise
+ * and MULTIPLICATION rules (folx/wrapped_functions.py:361-415, folx/hessian.py:87-112,
+ * :177-188); this entry point evaluates that chain's closed form in one pass.  For a
+ * sparse Jacobian the mask must be constant along the feature axis (rows then keep it).
+ */
+int folx_hip_layernorm_fwdlap(void* stream, const float* x, const float* jac, const float* lap,
+                              const float* gamma, const float* beta, float* y, float* y_jac,
+                              float* y_lap, int64_t R, int32_t F, int32_t P, float eps);
 
 /*
  * Row-stack affine map with broadcast coefficient arrays:

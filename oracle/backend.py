@@ -231,10 +231,22 @@ def integer_pow(a, n):
     return OArr(*rules.elementwise_rule('integer_pow', a.x, a.J, a.lap, n))
 
 
-def dot(h: OArr, W, b=None):
+def dot(h: OArr, W, b=None, residual=None):
     W = np.asarray(W, dtype=h.x.dtype)
     bb = None if b is None else np.asarray(b, dtype=h.x.dtype)
-    return OArr(*rules.dense_rule(h.x, h.J, h.lap, W, bb))
+    out = OArr(*rules.dense_rule(h.x, h.J, h.lap, W, bb))
+    return out if residual is None else add(residual, out)
+
+
+def layer_norm(h: OArr, gamma=None, beta=None, eps=1e-5):
+    """LayerNorm as the chain of primitive rules the reference interprets it with."""
+    mu = mean(h, axis=-1, keepdims=True)
+    c = subtract(h, mu)
+    var = mean(square(c), axis=-1, keepdims=True)
+    y = multiply(c, rsqrt(add(var, eps)))
+    if gamma is not None:
+        y = multiply(y, gamma)
+    return y if beta is None else add(y, beta)
 
 
 def sum(a: OArr, axis=None, keepdims=False):

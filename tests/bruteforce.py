@@ -24,9 +24,19 @@ class plain:
         return torch.as_tensor(np.asarray(c), dtype=like.dtype)
 
     @staticmethod
-    def dot(h, W, b=None):
+    def dot(h, W, b=None, residual=None):
         y = h @ plain._c(W, h)
-        return y if b is None else y + plain._c(b, h)
+        y = y if b is None else y + plain._c(b, h)
+        return y if residual is None else residual + y
+
+    @staticmethod
+    def layer_norm(h, gamma=None, beta=None, eps=1e-5):
+        mu = h.mean(-1, keepdim=True)
+        c = h - mu
+        y = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps)
+        if gamma is not None:
+            y = y * plain._c(gamma, h)
+        return y if beta is None else y + plain._c(beta, h)
 
     tanh = staticmethod(torch.tanh)
     exp = staticmethod(torch.exp)

@@ -20,8 +20,19 @@ def _t(a):
     return torch.as_tensor(np.ascontiguousarray(a, dtype=np.float32))
 
 
-def dense(x, jac, lap, W, bias=None):
-    return tuple(_t(a) for a in rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias)))
+def dense(x, jac, lap, W, bias=None, res=None):
+    out = rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias))
+    if res is not None:
+        out = tuple(o + _n(r) for o, r in zip(out, res))
+    return tuple(_t(a) for a in out)
+
+
+def layernorm(x, jac, lap, gamma, beta, eps):
+    from oracle import backend as ob
+
+    out = ob.layer_norm(ob.OArr(_n(x), _n(jac), _n(lap)), None if gamma is None else _n(gamma),
+                        None if beta is None else _n(beta), eps)
+    return _t(out.x), _t(out.J), _t(out.lap)
 
 
 def elementwise(name, x, jac, lap, param=0.0, inplace=False):
@@ -100,7 +111,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'scatter_add_rows', 'slogdet', 'mhsa'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

@@ -37,17 +37,18 @@ def test_version_and_strerror(lib):
 def test_argument_checks_return_error_codes(lib):
     null = ctypes.c_void_p(None)
     # negative sizes / null pointers -> EINVAL, nothing launched
-    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, 4, 1, 8, 8) == _lib.EINVAL
-    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, -1, 1, 8, 8) == _lib.EINVAL
+    assert lib.folx_hip_dense_fwdlap(*([null] * 12), 4, 1, 8, 8) == _lib.EINVAL
+    assert lib.folx_hip_dense_fwdlap(*([null] * 12), -1, 1, 8, 8) == _lib.EINVAL
     assert lib.folx_hip_elementwise_fwdlap(null, 99, 0.0, null, null, null, null, null, null, 4, 1) == _lib.EINVAL
     assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 4, 1) == _lib.EINVAL
     assert lib.folx_hip_binary_fwdlap(null, 0, null, null, null, null, null, null, null, null, null, null, 1, 1, 1) == _lib.EINVAL
     assert lib.folx_hip_rows_affine(null, null, null, 1, 1, null, null, 1.0, 1.0, null) == _lib.EINVAL
     assert lib.folx_hip_reduce_sum(null, null, null, 1, 1, -1, 1, 1.0) == _lib.EINVAL
     assert lib.folx_hip_slogdet_fwdlap(null, null, null, null, null, null, null, null, 4, 0, 1) == _lib.EINVAL
+    assert lib.folx_hip_layernorm_fwdlap(*([null] * 9), 4, 8, 1, 1e-5) == _lib.EINVAL
     assert lib.folx_hip_mhsa_fwdlap(*([null] * 15), 1, 8, 1, 8, 1) == _lib.EINVAL
     # empty problems are fine and launch nothing
-    assert lib.folx_hip_dense_fwdlap(null, null, null, null, null, null, null, null, null, 0, 1, 8, 8) == _lib.OK
+    assert lib.folx_hip_dense_fwdlap(*([null] * 12), 0, 1, 8, 8) == _lib.OK
     assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 0, 1) == _lib.OK
     assert lib.folx_hip_gather_rows(null, null, null, null, 1, 0, 1, 4, 4, 4) == _lib.OK
 
@@ -57,6 +58,8 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_slogdet_fwdlap(None, one, one, one, one, one, one, one, 4, 33, 1) == _lib.ENOTSUP
     assert lib.folx_hip_mhsa_fwdlap(None, *([one] * 9), None, None, one, one, one, 1, 65, 1, 8, 1) == _lib.ENOTSUP
     assert lib.folx_hip_mhsa_fwdlap(None, *([one] * 9), None, None, one, one, one, 1, 8, 1, 6, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_layernorm_fwdlap(None, one, one, one, None, None, one, one, one, 4, 6, 1, 1e-5) == _lib.ENOTSUP
+    assert lib.folx_hip_layernorm_fwdlap(None, one, one, one, None, None, one, one, one, 4, 2048, 1, 1e-5) == _lib.ENOTSUP
 
 
 def test_product_fails_loudly_without_gpu():

@@ -251,3 +251,21 @@ def test_psiformer_sparse_stage_keeps_three_rows():
         assert jac.weak and jac.x0_idx.shape[0] == 3
         want = 3 * np.arange(4)[None, :, None] + np.arange(3)[:, None, None]
         np.testing.assert_array_equal(jac.x0_idx, np.broadcast_to(want, jac.x0_idx.shape))
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_layer_norm_rule_fused_equals_primitive_chain(thr):
+    g, b = np.linspace(0.5, 1.5, 8), np.linspace(-1, 1, 8)
+    W = np.random.default_rng(7).normal(size=(3, 8))
+    x = np.random.default_rng(8).normal(size=(2, 4, 3)).astype(np.float32)
+    fused = lambda xp, t: xp.layer_norm(xp.dot(t, W), g, b, 1e-5)
+    chain = lambda xp, t: wl.layer_norm_primitives(xp, xp.dot(t, W), g, b, 1e-5)
+    a = check_against_oracle(fused, x, thr)
+    c = triplet_np(run_product(chain, x, thr))
+    for u, v in zip(a, c):
+        np.testing.assert_allclose(u, v, rtol=2e-4, atol=2e-5)
+    # sparse input whose mask varies along the normalised axis: falls back to the chain
+    varying = lambda xp, t: xp.layer_norm(xp.reshape(t, (3, 4)), None, None, 1e-5)
+    check_against_oracle(varying, x, thr)
+    out = run_product(fused, x, 6)
+    assert out.jacobian.weak and out.jacobian.x0_idx.shape[0] == 3

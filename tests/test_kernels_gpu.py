@@ -272,3 +272,36 @@ def test_mhsa(B, n, H, d, P, valid):
         got2 = K.mhsa(*[dev(t) for t in args], None, None)
         for g1, g2 in zip(got, got2):
             assert torch.equal(g1, g2)
+
+
+@pytest.mark.parametrize('rows,F,P', [((3, 5), 8, 4), ((2, 32), 256, 9), ((7,), 512, 3), ((4, 3), 100, 5),
+                                      ((2, 2), 1024, 2), ((5,), 4, 1)])
+def test_layernorm(rows, F, P):
+    """Fused LayerNorm rule against the chain of primitive rules evaluated by the oracle."""
+    from folx_amd import kernels as K
+    from oracle import backend as ob
+
+    print(f'case layernorm rows={rows} F={F} P={P}', flush=True)
+    rng = np.random.default_rng(11)
+    x, J, L = rand(rng, *rows, F), rand(rng, P, *rows, F), rand(rng, *rows, F)
+    g, b = 1 + 0.1 * rand(rng, F), rand(rng, F)
+    ref = ob.layer_norm(ob.OArr(*f64(x, J, L)), g.astype(np.float64), b.astype(np.float64), 1e-5)
+    got = K.layernorm(dev(x), dev(J), dev(L), dev(g), dev(b), 1e-5)
+    assert_triplet(got, (ref.x, ref.J, ref.lap), 'layernorm')
+    got = K.layernorm(dev(x), dev(J), dev(L), None, None, 1e-5)
+    ref = ob.layer_norm(ob.OArr(*f64(x, J, L)), None, None, 1e-5)
+    assert_triplet(got, (ref.x, ref.J, ref.lap), 'layernorm no affine')
+
+
+def test_dense_residual_epilogue():
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(12)
+    rows, P, Kd, N = (3, 32), 7, 256, 256
+    x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    rx, rJ, rL = rand(rng, *rows, N), rand(rng, P, *rows, N), rand(rng, *rows, N)
+    W, b = rand(rng, Kd, N) / 16, rand(rng, N)
+    ref = rules.dense_rule(*f64(x, J, L, W), b.astype(np.float64))
+    ref = tuple(r + s for r, s in zip(ref, f64(rx, rJ, rL)))
+    got = K.dense(dev(x), dev(J), dev(L), dev(W), dev(b), (dev(rx), dev(rJ), dev(rL)))
+    assert_triplet(got, ref, 'dense + residual')
