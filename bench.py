@@ -23,6 +23,15 @@ import numpy as np
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense FP32 matrix peak
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
+# scaled by what the same counter reads for a plain 1 GiB copy: x2.000 and x1.000); the
+# figures and the commands are in profiles/psiformer32_forward_laplacian.txt.
+MEASURED_TRAFFIC_BYTES = {
+    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.692e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, True)): 10.029e9,
+    ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.153e9,
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -63,7 +72,7 @@ def cpu_baseline(workload, budget_s):
         return dt
 
     t1 = run(1)
-    n = int(max(1, min(16, budget_s / max(t1, 1e-3))))
+    n = int(max(1, min(64, budget_s / max(t1, 1e-3))))
     dt = run(n) if n > 1 else t1
     return {
         'value': n / dt,
@@ -125,20 +134,21 @@ def main():
         per_kernel[name] = per_kernel.get(name, 0.0) + ms
     (dname, dkey), (dn, dms) = max(summ.items(), key=lambda kv: kv[1][1])
     roof = None
+    traffic = MEASURED_TRAFFIC_BYTES.get((dname, dkey))
     if dname == 'dense_fwdlap':
-        R, P, Kd, N = dkey
+        R, P, Kd, N, has_res = dkey
         flops = 2.0 * (P + 2) * R * Kd * N
         achieved = flops / (dms / dn * 1e-3) / 1e12
         roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
-                'kernel': f'dense_kernel R={R} P={P} K={Kd} N={N}', 'launches': dn,
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
+                'kernel': f'dense_kernel R={R} P={P} K={Kd} N={N} residual={has_res}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
     elif dname == 'mhsa_fwdlap':
         Bc, n, H, d, P = dkey
         flops = (7.0 * P + 6) * 2 * n * n * d * Bc * H
         achieved = flops / (dms / dn * 1e-3) / 1e12
         roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': None,
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
                 'kernel': f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
     else:

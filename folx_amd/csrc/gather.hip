@@ -6,28 +6,45 @@
 namespace {
 
 // out[t][b][so][si] = sum_s data[take[t][s][so]][b][so][si]   (take < 0: no source)
-// Threads run along (so, si) so reads and writes are coalesced; the table entry is shared
-// by the S_inner consecutive threads of one `so` and by all walkers b (blockIdx.y).
+// Threads run along (so, si) in units of VEC floats so reads and writes are coalesced
+// 128-bit accesses when S_inner allows; the table entries are read once per thread and
+// reused for the WPT walkers the thread loops over (blockIdx.y selects the walker group).
+constexpr int GATHER_WPT = 8;
+
+template <int VEC>
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restrict__ data,
                                                           const int32_t* __restrict__ take,
-                                                          float* __restrict__ out, int32_t k_out,
-                                                          int32_t n_slots, int64_t B, int64_t S_outer,
-                                                          int64_t S_inner) {
+                                                          float* __restrict__ out, int32_t n_slots,
+                                                          int64_t B, int64_t S_outer, int64_t S_inner) {
   const int64_t S = S_outer * S_inner;
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
   if (e >= S) return;
   const int64_t so = e / S_inner;
   const int32_t t = blockIdx.z;
   int32_t src[8];
   const int32_t ns = n_slots < 8 ? n_slots : 8;
   for (int s = 0; s < ns; ++s) src[s] = take[((int64_t)t * n_slots + s) * S_outer + so];
-  for (int64_t b = blockIdx.y; b < B; b += gridDim.y) {
-    float acc = 0.0f;
+  const int64_t b0 = (int64_t)blockIdx.y * GATHER_WPT;
+  const int64_t b1 = b0 + GATHER_WPT < B ? b0 + GATHER_WPT : B;
+  for (int64_t b = b0; b < b1; ++b) {
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
     for (int s = 0; s < n_slots; ++s) {
       const int32_t r = s < 8 ? src[s] : take[((int64_t)t * n_slots + s) * S_outer + so];
-      if (r >= 0) acc += data[((int64_t)r * B + b) * S + e];
+      if (r >= 0) {
+        const float* p = data + ((int64_t)r * B + b) * S + e;
+        if constexpr (VEC == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(p);
+          acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+        } else {
+          acc[0] += *p;
+        }
+      }
     }
-    out[((int64_t)t * B + b) * S + e] = acc;
+    float* q = out + ((int64_t)t * B + b) * S + e;
+    if constexpr (VEC == 4) *reinterpret_cast<float4*>(q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    else *q = acc[0];
   }
 }
 
@@ -56,11 +73,16 @@ extern "C" int folx_hip_gather_rows(void* stream, const float* data, const int32
   if (k_out == 0 || B == 0 || S == 0) return FOLX_HIP_OK;
   if (!out || (n_slots > 0 && (!take || (k_in > 0 && !data)))) return FOLX_HIP_EINVAL;
   if (k_out > 65535) return FOLX_HIP_ENOTSUP;
-  const int64_t blocks = (S + 255) / 256;
+  const int64_t gy = (B + GATHER_WPT - 1) / GATHER_WPT;
+  if (gy > 65535) return FOLX_HIP_ENOTSUP;
+  const bool vec = (S_inner % 4 == 0) && folx_aligned16(data) && folx_aligned16(out);
+  const int64_t blocks = vec ? (S / 4 + 255) / 256 : (S + 255) / 256;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-  const unsigned gy = (unsigned)(B < 4096 ? B : 4096);
-  gather_rows_kernel<<<dim3((unsigned)blocks, gy, (unsigned)k_out), dim3(256), 0, (hipStream_t)stream>>>(
-      data, take, out, k_out, n_slots, B, S_outer, S_inner);
+  dim3 grid((unsigned)blocks, (unsigned)gy, (unsigned)k_out);
+  if (vec)
+    gather_rows_kernel<4><<<grid, dim3(256), 0, (hipStream_t)stream>>>(data, take, out, n_slots, B, S_outer, S_inner);
+  else
+    gather_rows_kernel<1><<<grid, dim3(256), 0, (hipStream_t)stream>>>(data, take, out, n_slots, B, S_outer, S_inner);
   return folx_launch_status();
 }
 

@@ -105,7 +105,7 @@ def dense(x, jac, lap, W, bias=None, res=None):
     y = torch.empty((*x.shape[:-1], N), device=x.device, dtype=torch.float32)
     yj = torch.empty((P, *x.shape[:-1], N), device=x.device, dtype=torch.float32)
     yl = torch.empty_like(y)
-    with _timed('dense_fwdlap', (R, P, K, N)):
+    with _timed('dense_fwdlap', (R, P, K, N, res is not None)):
         check(
             _lib.load().folx_hip_dense_fwdlap(
                 _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(rx), _p(rj), _p(rl),
