@@ -43,6 +43,8 @@ def parse():
     ap.add_argument('--chunk', type=int, default=1024, help='walkers per batched_vmap chunk')
     ap.add_argument('--cpu-seconds', type=float, default=20.0, help='budget of the CPU baseline sample')
     ap.add_argument('--no-cpu', action='store_true')
+    ap.add_argument('--graph', action='store_true',
+                    help='replay each chunk as a captured HIP graph (no per-kernel timing, no roofline)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also launch one plain copy (rows_affine, 1 GiB in, 1 GiB out) for scaling HBM counters')
     return ap.parse_args()
@@ -54,8 +56,7 @@ def cpu_baseline(workload, budget_s):
 
     from folx_amd import workloads as wl
 
-    cfg, _, sigma, _ = wl.CONFIGS[workload]
-    p = wl.psiformer_params(cfg)
+    forward, p, cfg, _, sigma, _ = wl.build(workload)
     try:
         from threadpoolctl import threadpool_info
 
@@ -66,7 +67,7 @@ def cpu_baseline(workload, budget_s):
     def run(n):
         x = wl.sample_electrons(n, cfg.n_elec, sigma, seed=2)
         t0 = time.perf_counter()
-        out = wl.psiformer_forward(p, ob.init_state(x, dtype=np.float32), ob)
+        out = forward(p, ob.init_state(x, dtype=np.float32), ob)
         dt = time.perf_counter() - t0
         assert np.isfinite(out.lap).all()
         return dt
@@ -83,6 +84,14 @@ def cpu_baseline(workload, budget_s):
     }
 
 
+def describe(cfg):
+    if hasattr(cfg, 'n_heads'):
+        return (f'PsiFormer-style, {cfg.n_elec} electrons, {cfg.n_nuc} nuclei, {cfg.n_layers} layers x '
+                f'{cfg.n_heads} heads x {cfg.head_dim}, width {cfg.width}, {cfg.n_det} determinants')
+    return (f'FermiNet-style, {cfg.n_elec} electrons, {cfg.n_nuc} nuclei, {cfg.n_layers} layers, one-electron '
+            f'width {cfg.w1}, two-electron width {cfg.w2}, {cfg.n_det} determinants')
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -96,15 +105,15 @@ def main():
     from folx_amd import kernels as K
     from folx_amd import workloads as wl
 
-    cfg, B, sigma, thr = wl.CONFIGS[args.workload]
+    forward, params_np, cfg, B, sigma, thr = wl.build(args.workload)
     if args.walkers:
         B = args.walkers
     dev = torch.device('cuda', 0)
     torch.cuda.set_device(dev)
-    params = wl.to_device(wl.psiformer_params(cfg), dev)
+    params = wl.to_device(params_np, dev)
     x = torch.as_tensor(wl.sample_electrons(B, cfg.n_elec, sigma, seed=2)).to(dev)
-    fl = folx_amd.forward_laplacian(lambda r: wl.psiformer_forward(params, r), thr)
-    step = folx_amd.batched_vmap(fl, args.chunk)
+    fl = folx_amd.forward_laplacian(lambda r: forward(params, r), thr)
+    step = folx_amd.batched_vmap(folx_amd.jit(folx_amd.vmap(fl)) if args.graph else fl, args.chunk)
 
     for _ in range(args.warmup):
         out = step(x)
@@ -129,6 +138,15 @@ def main():
 
     # dominant kernel: the launch shape with the largest total time inside the timed region
     summ = lt.summary()
+    if not summ:
+        line = {'metric': 'walkers/s of full forward Laplacian at 1 GPU', 'value': value, 'unit': 'walkers/s',
+                'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': ms_per_step,
+                'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
+                'data': 'synthetic', 'config': {'workload': f'{args.workload}: {describe(cfg)}', 'walkers': B,
+                                                'chunk': args.chunk, 'mode': 'hip graph replay'},
+                'roofline': None}
+        print(json.dumps(line))
+        return
     per_kernel = {}
     for (name, key), (n, ms) in summ.items():
         per_kernel[name] = per_kernel.get(name, 0.0) + ms
@@ -169,9 +187,7 @@ def main():
         'dtype': 'f32',
         'data': 'synthetic',
         'config': {
-            'workload': f'{args.workload}: PsiFormer-style, {cfg.n_elec} electrons, {cfg.n_nuc} nuclei, '
-                        f'{cfg.n_layers} layers x {cfg.n_heads} heads x {cfg.head_dim}, width {cfg.width}, '
-                        f'{cfg.n_det} determinants, ForwardLaplacianOperator({thr})',
+            'workload': f'{args.workload}: {describe(cfg)}, ForwardLaplacianOperator({thr})',
             'walkers': B,
             'chunk': args.chunk,
             'jacobian_rows': 3 * cfg.n_elec,

@@ -91,8 +91,27 @@ def layer_norm(h, gamma=None, beta=None, eps=1e-5):
     return _call('layer_norm', (h, gamma, beta), {'eps': eps})
 
 
+def matmul(a, b):
+    """``numpy.matmul`` for two operands of which at least one carries derivatives."""
+    from .api import FwdLaplArray as _F
+
+    if isinstance(a, _F) and not isinstance(b, _F) and len(_shape(b)) == 2:
+        return dot(a, b)
+    if isinstance(a, _F) and isinstance(b, _F):
+        return _call('dot_general', (a, b), {})
+    if isinstance(b, _F):  # constant @ triplet = (triplet^T @ constant^T)^T
+        bt = swapaxes(b, -1, -2) if len(_shape(b)) > 1 else b
+        out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
+        return swapaxes(out, -1, -2) if len(_shape(out)) > 1 else out
+    return np.matmul(a, b)
+
+
 def slogdet(A):
     return _call('slogdet', (A,))
+
+
+def det(A):
+    return _call('det', (A,))
 
 
 def multi_head_self_attention(q, k, v, mask=None, input_mask=None, **kwargs):

@@ -133,7 +133,7 @@ def to_device(params, device):
             return {k: conv(x) for k, x in v.items()}
         if isinstance(v, (list, tuple)):
             return type(v)(conv(x) for x in v)
-        if dataclasses.is_dataclass(v) and not isinstance(v, type) and not isinstance(v, PsiFormerConfig):
+        if dataclasses.is_dataclass(v) and not isinstance(v, type) and not type(v).__name__.endswith('Config'):
             return dataclasses.replace(v, **{f.name: conv(getattr(v, f.name)) for f in dataclasses.fields(v)})
         return v
 
@@ -198,12 +198,137 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
     return logpsi
 
 
+# --------------------------------------------------------------------------------------
+# FermiNet-style wavefunction: one-electron stream (width w1) and two-electron stream
+# (width w2), tanh layers with residual connections, determinants with exponential
+# envelopes.  The two-electron stream depends on six coordinates per pair, so it stays a
+# sparse Jacobian (k = 6) with ForwardLaplacianOperator(6); the one-electron stream turns
+# dense in the first layer through the spin-wise means over electrons.
+# --------------------------------------------------------------------------------------
+
+
+@dataclass
+class FermiNetConfig:
+    n_elec: int = 16
+    n_nuc: int = 4
+    n_layers: int = 4
+    w1: int = 256
+    w2: int = 32
+    n_det: int = 16
+    nuc_box: float = 2.0
+    seed: int = 0
+
+    @property
+    def n_up(self):
+        return self.n_elec // 2
+
+    @property
+    def n_down(self):
+        return self.n_elec - self.n_up
+
+
+@dataclass
+class FermiNetParams:
+    cfg: FermiNetConfig
+    nuclei: np.ndarray
+    eye: np.ndarray
+    layers: list = field(default_factory=list)
+    w_orb: tuple = ()
+    env_sigma: tuple = ()
+    env_pi: tuple = ()
+
+
+def ferminet_params(cfg: FermiNetConfig) -> FermiNetParams:
+    rng = np.random.default_rng(cfg.seed)
+    nuclei = np.random.default_rng(cfg.seed + 1).uniform(-cfg.nuc_box, cfg.nuc_box, size=(cfg.n_nuc, 3)).astype(np.float32)
+    p = FermiNetParams(cfg=cfg, nuclei=nuclei, eye=np.eye(cfg.n_elec, dtype=np.float32))
+    d1, d2 = 4 * cfg.n_nuc, 4
+    for layer in range(cfg.n_layers):
+        f_in = 3 * d1 + 2 * d2
+        L = dict(v=_dense_init(rng, f_in, cfg.w1), b=np.zeros(cfg.w1, np.float32))
+        if layer < cfg.n_layers - 1:  # the last layer does not update the pair stream
+            L['w'] = _dense_init(rng, d2, cfg.w2)
+            L['c'] = np.zeros(cfg.w2, np.float32)
+        p.layers.append(L)
+        d1, d2 = cfg.w1, cfg.w2
+    p.w_orb = (_dense_init(rng, cfg.w1, cfg.n_det * cfg.n_up), _dense_init(rng, cfg.w1, cfg.n_det * cfg.n_down))
+    p.env_sigma = tuple(
+        rng.uniform(0.5, 1.5, size=(cfg.n_nuc, cfg.n_det * m)).astype(np.float32) for m in (cfg.n_up, cfg.n_down)
+    )
+    p.env_pi = tuple(
+        rng.uniform(0.5, 1.5, size=(cfg.n_nuc, cfg.n_det * m)).astype(np.float32) for m in (cfg.n_up, cfg.n_down)
+    )
+    return p
+
+
+def ferminet_forward(p: FermiNetParams, r, xp=None):
+    """log|psi(r)| for one walker; r (n_elec, 3)."""
+    if xp is None:
+        from . import numpy as xp
+    cfg = p.cfg
+    n, nu = cfg.n_elec, cfg.n_up
+    d, dist = electron_nuclear_features(xp, r, p.nuclei)
+    h = xp.concatenate([xp.reshape(d, (n, 3 * cfg.n_nuc)), dist], axis=-1)  # (n, 4 nuc)
+    # pair features; the distance of an electron to itself is regularised as in FermiNet:
+    # |r_ij + eye| * (1 - eye), so the square root is never taken at zero
+    rij = xp.subtract(xp.expand_dims(r, 1), xp.expand_dims(r, 0))  # (n, n, 3)
+    r2 = xp.add(xp.sum(xp.square(rij), axis=-1), p.eye)
+    rn = xp.multiply(xp.sqrt(r2), 1.0 - p.eye)
+    g = xp.concatenate([rij, xp.expand_dims(rn, 2)], axis=-1)  # (n, n, 4)
+
+    def spin_means(t, axis_len):
+        up = xp.mean(xp.getitem(t, (slice(0, nu),)), axis=0) if nu > 0 else None
+        dn = xp.mean(xp.getitem(t, (slice(nu, n),)), axis=0) if n - nu > 0 else None
+        return up, dn
+
+    for li, L in enumerate(p.layers):
+        hu, hd = spin_means(h, n)  # (d1,) each
+        # means over the second electron of every pair: (n, d2)
+        gu = xp.mean(xp.getitem(g, (slice(None), slice(0, nu))), axis=1)
+        gd = xp.mean(xp.getitem(g, (slice(None), slice(nu, n))), axis=1)
+        d1 = h.shape[-1]
+        parts = [h, xp.broadcast_to(hu, (n, d1)), xp.broadcast_to(hd, (n, d1)), gu, gd]
+        f = xp.concatenate(parts, axis=-1)
+        hn = xp.tanh(xp.dot(f, L['v'], L['b']))
+        h = xp.add(h, hn) if hn.shape == h.shape else hn
+        if 'w' in L:
+            gn = xp.tanh(xp.dot(g, L['w'], L['c']))
+            g = xp.add(g, gn) if gn.shape == g.shape else gn
+    logdets, signs = [], []
+    for s, (lo, hi) in enumerate([(0, nu), (nu, n)]):
+        m = hi - lo
+        if m == 0:
+            continue
+        hs = xp.getitem(h, (slice(lo, hi),))
+        orb = xp.dot(hs, p.w_orb[s])
+        ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)
+        env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
+        orb = xp.multiply(orb, env)
+        mats = xp.transpose(xp.reshape(orb, (m, cfg.n_det, m)), (1, 0, 2))
+        sg, ld = xp.slogdet(mats)
+        logdets.append(ld), signs.append(sg)
+    total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
+    sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
+    logpsi, _ = xp.logsumexp(total, axis=0, b=sign)
+    return logpsi
+
+
 def sample_electrons(n_walkers, n_elec, sigma, seed):
     return (sigma * np.random.default_rng(seed).normal(size=(n_walkers, n_elec, 3))).astype(np.float32)
 
 
+def build(name):
+    """(forward(params, r, xp=None), params, config, walkers, sigma, threshold) of a named
+    benchmark configuration."""
+    cfg, walkers, sigma, thr = CONFIGS[name]
+    if isinstance(cfg, FermiNetConfig):
+        return ferminet_forward, ferminet_params(cfg), cfg, walkers, sigma, thr
+    return psiformer_forward, psiformer_params(cfg), cfg, walkers, sigma, thr
+
+
 CONFIGS = {
-    # name: (PsiFormerConfig, walkers, position sigma, sparsity threshold)
+    # name: (config, walkers, position sigma, sparsity threshold)
+    'ferminet16': (FermiNetConfig(), 4096, 1.5, 6),
     'psiformer32': (PsiFormerConfig(), 4096, 1.5, 6),
     'psiformer64': (
         PsiFormerConfig(n_elec=64, n_nuc=8, n_heads=8, head_dim=64, width=512, mlp_width=512, nuc_box=4.0),

@@ -406,10 +406,12 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
         y = np.asarray(h) @ np.asarray(W)
         return y if bias is None else y + np.asarray(bias)
     if _is(W):
-        raise NotImplementedError(
-            'dot_general with two derivative-carrying operands: use multiply + sum, or '
-            'multi_head_self_attention for attention'
-        )
+        out = _dot_two_operands(h, W, sparsity_threshold)
+        if bias is not None:
+            out = _LAPLACE_FN_REGISTRY['add']((out, bias), {}, sparsity_threshold)
+        if residual is not None:
+            out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)
+        return out
     dev = h.x.device
     Wt = so.device_const(W, dev)
     bt = None if bias is None else so.device_const(bias, dev)
@@ -438,6 +440,32 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
     if residual is not None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)
+    return out
+
+
+def _dot_two_operands(lhs: FwdLaplArray, rhs: FwdLaplArray, thr: int) -> FwdLaplArray:
+    """Matrix product of two derivative-carrying operands with ``numpy.matmul`` shapes,
+    ``lhs (..., i, k) @ rhs (..., k, j)`` (1-D operands as in matmul).  Both operands are
+    rearranged so that the contracted axis is last and broadcast against each other, then
+    multiplied and summed -- the decomposition the reference takes for this case
+    (``rearrange`` + ``mul_sum``, folx/wrapped_functions.py:47-68, :253-286); the rules of
+    ``mul`` (JVP both ways + 2 tr(J_l J_r^T), folx/hessian.py:177-188) and ``reduce_sum``
+    then give the triplet."""
+    from . import numpy as fnp
+
+    a, b = lhs, rhs
+    a_vec, b_vec = a.ndim == 1, b.ndim == 1
+    if a_vec:
+        a = fnp.expand_dims(a, 0)
+    if b_vec:
+        b = fnp.expand_dims(b, 1)
+    bt = fnp.swapaxes(b, -1, -2)  # (..., j, k)
+    prod = fnp.multiply(fnp.expand_dims(a, -2), fnp.expand_dims(bt, -3))  # (..., i, j, k)
+    out = fnp.sum(prod, axis=-1)
+    if b_vec:
+        out = fnp.squeeze(out, -1)
+    if a_vec:
+        out = fnp.squeeze(out, -1 if b_vec else -2)
     return out
 
 
@@ -752,6 +780,16 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
     return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
 
 
+def det_wrapper(args, kwargs, sparsity_threshold):
+    """``det`` from the log-determinant (``det_wrapper``, folx/slogdet.py:361-395):
+    det = sign exp(logdet), d_c det = det d_c logdet,
+    lap det = det (lap logdet + sum_c (d_c logdet)^2) -- which is the ``exp`` rule applied
+    to the logdet triplet, scaled by the sign."""
+    sign, ld = slogdet_wrapper(args, kwargs, sparsity_threshold)
+    e = _LAPLACE_FN_REGISTRY['exp']((ld,), {}, sparsity_threshold)
+    return _LAPLACE_FN_REGISTRY['mul']((e, sign), {}, sparsity_threshold)
+
+
 def _mask_tensor(m, shape, device):
     if m is None:
         return None
@@ -825,4 +863,5 @@ register_function('stop_gradient', stop_gradient_rule)
 register_function('sign', sign_rule)
 register_function('reduce_max_values', reduce_max_values)
 register_function('slogdet', slogdet_wrapper)
+register_function('det', det_wrapper)
 register_function('_multi_head_self_attention', mhsa_forward_laplacian)

@@ -365,6 +365,35 @@ def logsumexp(a: OArr, axis=-1, b=None):
     return val, sign(s)
 
 
+def matmul(a, b):
+    """numpy.matmul semantics; two triplets go through multiply + sum like the reference's
+    mul_sum decomposition (folx/wrapped_functions.py:253-286)."""
+    if _is(a) and not _is(b):
+        return dot(a, b)
+    if _is(a) and _is(b):
+        av, bv = a.ndim == 1, b.ndim == 1
+        if av:
+            a = expand_dims(a, 0)
+        if bv:
+            b = expand_dims(b, 1)
+        bt = swapaxes(b, -1, -2)
+        out = sum(multiply(expand_dims(a, -2), expand_dims(bt, -3)), axis=-1)
+        if bv:
+            out = squeeze(out, -1)
+        if av:
+            out = squeeze(out, -1 if bv else -2)
+        return out
+    bt = swapaxes(b, -1, -2) if b.ndim > 1 else b
+    out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
+    return swapaxes(out, -1, -2) if out.ndim > 1 else out
+
+
+def det(A: OArr):
+    """det = sign * exp(logdet) (folx/slogdet.py:361-395)."""
+    sg, ld = slogdet(A)
+    return multiply(exp(ld), sg)
+
+
 def slogdet(A: OArr):
     sign, (ld, J, L) = rules.slogdet_rule(A.x, A.J, A.lap)
     return OConst(sign), OArr(ld, J, L)

@@ -138,6 +138,23 @@ class plain:
         return a.detach().amax(dim=axis, keepdim=keepdims)
 
     @staticmethod
+    def matmul(a, b):
+        a, b = plain._b(a, b)
+        return a @ b
+
+    @staticmethod
+    def det(A):
+        n = A.shape[-1]
+        if n == 1:
+            return A[..., 0, 0]
+        # Laplace expansion along the first row: pure arithmetic, safe under any AD mode
+        out = 0
+        for j in range(n):
+            minor = torch.cat([A[..., 1:, :j], A[..., 1:, j + 1:]], dim=-1)
+            out = out + ((-1) ** j) * A[..., 0, j] * plain.det(minor)
+        return out
+
+    @staticmethod
     def sign(a):
         return torch.sign(a.detach())
 

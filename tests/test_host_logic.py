@@ -269,3 +269,79 @@ def test_layer_norm_rule_fused_equals_primitive_chain(thr):
     check_against_oracle(varying, x, thr)
     out = run_product(fused, x, 6)
     assert out.jacobian.weak and out.jacobian.x0_idx.shape[0] == 3
+
+
+MATMUL_FNS = {
+    'mat_mat': lambda xp, x: xp.matmul(xp.tanh(x), xp.swapaxes(xp.sin(x), -1, -2)),        # (4,3)@(3,4)
+    'attn_like': lambda xp, x: xp.matmul(xp.exp(xp.multiply(xp.matmul(x, xp.swapaxes(x, -1, -2)), 0.1)), x),
+    'vec_mat': lambda xp, x: xp.matmul(xp.getitem(x, (0,)), xp.swapaxes(xp.cos(x), -1, -2)),  # (3,)@(3,4)
+    'const_left': lambda xp, x: xp.matmul(np.arange(8.0).reshape(2, 4) / 8, xp.tanh(x)),      # (2,4)@(4,3)
+}
+
+
+@pytest.mark.parametrize('name', sorted(MATMUL_FNS))
+@pytest.mark.parametrize('thr', [0, 12])
+def test_two_operand_matmul(name, thr):
+    """test/test_layers.py:141-171 (matmul with both operands carrying Jacobians)."""
+    x = np.random.default_rng(9).normal(size=(2, 4, 3)).astype(np.float32)
+    got = check_against_oracle(MATMUL_FNS[name], x, thr)
+    by, bJ, bL = brute_force(lambda t: MATMUL_FNS[name](plain, t), x.astype(np.float64))
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize('thr', [0, 9])
+def test_det_rule(thr):
+    """test/test_layers.py:424-444."""
+    W = np.random.default_rng(10).normal(size=(5, 9)) / 2
+    fn = lambda xp, x: xp.det(xp.reshape(xp.tanh(xp.dot(x, W)), (3, 3)))
+    x = np.random.default_rng(11).normal(size=(3, 5)).astype(np.float32)
+    got = check_against_oracle(fn, x, thr)
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-5)
+
+
+SMALL_FERMI = wl.FermiNetConfig(n_elec=4, n_nuc=2, n_layers=3, w1=8, w2=4, n_det=2)
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_ferminet_small_vs_oracle_and_bruteforce(thr):
+    p = wl.ferminet_params(SMALL_FERMI)
+    x = wl.sample_electrons(2, SMALL_FERMI.n_elec, 1.0, seed=4)
+    fn = lambda xp, t: wl.ferminet_forward(p, t, xp)
+    got = check_against_oracle(fn, x, thr, rtol=5e-4, atol=5e-5)
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    np.testing.assert_allclose(ref.x, by, rtol=1e-8)
+    np.testing.assert_allclose(ref.J, bJ, rtol=1e-6, atol=1e-9)
+    np.testing.assert_allclose(ref.lap, bL, rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(got[2], bL, rtol=5e-4, atol=5e-5)
+
+
+def test_ferminet_pair_stream_stays_sparse():
+    """The pair stream depends on six coordinates per pair: k = 6 with thr = 6, through
+    the tanh layers and the residual adds (README.md:72)."""
+    p = wl.ferminet_params(SMALL_FERMI)
+    x = wl.sample_electrons(2, SMALL_FERMI.n_elec, 1.0, seed=4)
+    seen = {}
+
+    def fn(r):
+        rij = fnp.subtract(fnp.expand_dims(r, 1), fnp.expand_dims(r, 0))
+        seen['rij'] = rij.jacobian
+        r2 = fnp.add(fnp.sum(fnp.square(rij), axis=-1), p.eye)
+        seen['r2'] = r2.jacobian
+        rn = fnp.multiply(fnp.sqrt(r2), 1.0 - p.eye)
+        g = fnp.concatenate([rij, fnp.expand_dims(rn, 2)], axis=-1)
+        seen['g'] = g.jacobian
+        g2 = fnp.tanh(fnp.dot(g, p.layers[0]['w'], p.layers[0]['c']))
+        seen['g2'] = g2.jacobian
+        return fnp.sum(g2)
+
+    folx_amd.vmap(folx_amd.forward_laplacian(fn, 6))(x)
+    assert seen['rij'].x0_idx.shape[0] == 2          # rows of r_i and of r_j
+    assert seen['r2'].x0_idx.shape[0] == 6           # union over xyz of both electrons
+    assert seen['g'].x0_idx.shape[0] == 6 and seen['g2'].x0_idx.shape[0] == 6
+    i, j = 1, 3
+    assert sorted(int(v) for v in seen['g2'].x0_idx[:, i, j, 0]) == [3, 4, 5, 9, 10, 11]
+    # a diagonal pair depends on three coordinates only
+    assert sorted(set(int(v) for v in seen['g2'].x0_idx[:, 2, 2, 0] if v >= 0)) == [6, 7, 8]

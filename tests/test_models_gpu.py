@@ -69,7 +69,21 @@ def test_psiformer_small_vs_oracle_and_loop_laplacian(thr):
     assert_val(out.x, by), assert_val(out.jacobian.dense_array, bJ), assert_lap(out.laplacian, bL)
 
 
-@pytest.mark.parametrize('name', ['psiformer32', 'psiformer64'])
+SMALL_FERMI = wl.FermiNetConfig(n_elec=6, n_nuc=2, n_layers=3, w1=16, w2=8, n_det=3)
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_ferminet_small_vs_oracle_and_loop_laplacian(thr):
+    """BASELINE config 3 in miniature: sparse pair stream (k = 6), dense one-electron stream."""
+    p = wl.ferminet_params(SMALL_FERMI)
+    x = wl.sample_electrons(4, SMALL_FERMI.n_elec, 1.0, seed=3)
+    fn = lambda xp, t: wl.ferminet_forward(p, t, xp)
+    out, ref = check(fn, x, thr, 'ferminet small')
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    assert_val(out.x, by), assert_val(out.jacobian.dense_array, bJ), assert_lap(out.laplacian, bL)
+
+
+@pytest.mark.parametrize('name', ['ferminet16', 'psiformer32', 'psiformer64'])
 def test_psiformer_full_architecture_two_walkers(name):
     """The benchmark architectures at their real widths (P = 96 / 192), 2 walkers.
 
@@ -81,10 +95,9 @@ def test_psiformer_full_architecture_two_walkers(name):
     fp32 oracle is (factor 2 head-room).  The strict
     bars (values/Jacobians rtol 1e-5, Laplacians rtol 1e-4 + atol 1e-5) are enforced per
     kernel and on the well-conditioned models above."""
-    cfg, _, sigma, thr = wl.CONFIGS[name]
-    p = wl.psiformer_params(cfg)
+    forward, p, cfg, _, sigma, thr = wl.build(name)
     x = wl.sample_electrons(2, cfg.n_elec, sigma, seed=2)
-    fn = lambda xp, t: wl.psiformer_forward(p, t, xp)
+    fn = lambda xp, t: forward(p, t, xp)
     print(f'case {name} full architecture', flush=True)
     out = run(fn, x, thr)
     r64 = fn(ob, ob.init_state(x, dtype=np.float64))
