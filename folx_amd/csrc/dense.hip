@@ -6,9 +6,10 @@
 //
 // Tiling: a workgroup owns BM rows x BN columns and walks K in chunks of BK = 16 through
 // double-buffered LDS tiles (global -> registers -> LDS, one barrier per chunk).  For
-// N > 128 the tile is 256 x 256 on 8 wavefronts (each 64 x 128), so a layer of width 256
-// reads its A rows from HBM exactly once; narrower layers use 128 x {128, 64, 32} tiles on
-// 4 wavefronts.  A rows are stored [row][k] with a stride of BK + 4 floats: a lane fetches
+// N > 128 the tile is 128 x 256 on 8 wavefronts (each 64 x 64), so a layer of width 256
+// reads its A rows from HBM exactly once and two workgroups share a CU (the stores of one
+// overlap the MFMAs of the other); narrower layers use 128 x {128, 64, 32} tiles on 4
+// wavefronts.  A rows are stored [row][k] with a stride of BK + 4 floats: a lane fetches
 // 4 consecutive k with one 128-bit LDS read and the rows of 8 consecutive lanes fall into
 // distinct bank groups.  The MFMA only needs A and B to agree on which k a lane holds, so
 // the k order inside a group of 8 is permuted to fit that read:
@@ -287,7 +288,7 @@ extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* 
                    folx_aligned16(lap) && folx_aligned16(W);
   const bool has_res = res != nullptr;
   hipStream_t st = (hipStream_t)stream;
-  if (N > 128) return launch_cfg<256, 256, 4, 2, 1>(st, sg, W, bias, K, N, vec, has_res);
+  if (N > 128) return launch_cfg<128, 256, 2, 4, 2>(st, sg, W, bias, K, N, vec, has_res);
   if (N > 64) return launch_cfg<128, 128, 2, 2, 3>(st, sg, W, bias, K, N, vec, has_res);
   if (N > 32) return launch_cfg<128, 64, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);
   return launch_cfg<128, 32, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);

@@ -9,7 +9,7 @@
 // which is what the chain mean / sub / square / mean / rsqrt / mul of elementwise and
 // reduction rules evaluates to.  One wavefront owns one row of F features and streams the
 // Jacobian rows once (read once, written once: 8 (P + 2) F bytes per row, HBM bound); the
-// three per-row means are butterfly reductions inside the wavefront, two Jacobian rows
+// three per-row means are butterfly reductions inside the wavefront, four Jacobian rows
 // in flight at a time.
 #include "common.h"
 
@@ -114,19 +114,27 @@ __global__ __launch_bounds__(FOLX_WAVE * ROWS_PER_BLOCK) void layernorm_kernel(
   };
 
   int p = 0;
-  for (; p + 1 < P; p += 2) {
-    float4 u0[NV], u1[NV];
+  for (; p + 3 < P; p += 4) {  // four Jacobian rows in flight per wavefront
+    float4 u0[NV], u1[NV], u2[NV], u3[NV];
     load_row(p, u0);
     load_row(p + 1, u1);
-    float a1, a2, a3, b1, b2, b3;
+    load_row(p + 2, u2);
+    load_row(p + 3, u3);
+    float a1, a2, a3, b1, b2, b3, c1, c2, c3, e1, e2, e3;
     partial(u0, a1, a2, a3);
     partial(u1, b1, b2, b3);
+    partial(u2, c1, c2, c3);
+    partial(u3, e1, e2, e3);
     wave_sum3(a1, a2, a3);
     wave_sum3(b1, b2, b3);
+    wave_sum3(c1, c2, c3);
+    wave_sum3(e1, e2, e3);
     finish_row(p, u0, a1, a2, a3);
     finish_row(p + 1, u1, b1, b2, b3);
+    finish_row(p + 2, u2, c1, c2, c3);
+    finish_row(p + 3, u3, e1, e2, e3);
   }
-  if (p < P) {
+  for (; p < P; ++p) {
     float4 u0[NV];
     load_row(p, u0);
     float a1, a2, a3;

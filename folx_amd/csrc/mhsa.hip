@@ -163,10 +163,16 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
     for (int jt = 0; jt < NW; ++jt)
 #pragma unroll
       for (int r = 0; r < 4; ++r) st[(4 * lg + r) * NS + 16 * jt + l16] = c[jt][r];
-    __syncthreads();
+    // The tile is private to this wavefront, whose LDS accesses complete in issue order:
+    // a wavefront-scope fence (no reordering by the compiler) is all the exchange needs.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
     for (int t = 0; t < NW; ++t) areg[t] = *reinterpret_cast<const float4*>(&st[l16 * NS + 4 * lg + 16 * t]);
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   };
 
   floatx4 pc[NW];  // softmax probabilities, result layout
@@ -300,8 +306,6 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) z[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
       out_store(a.oj + (int64_t)c * slice, z);
-      __syncthreads();  // keep the barrier count of to_a_layout
-      __syncthreads();
     }
     if (nact) {
       tile_store(kjs[buf ^ 1], rk);
