@@ -31,6 +31,7 @@ SIGNATURES = {
     'folx_hip_scatter_add_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int64, c_int64, c_int64]),
     'folx_hip_slogdet_fwdlap': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int32, c_int32]),
     'folx_hip_mhsa_fwdlap': (c_int, [_P] * 15 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
+    'folx_hip_mhsea_fwdlap': (c_int, [_P] * 18 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 
 ACT = {

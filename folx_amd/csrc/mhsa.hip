@@ -7,7 +7,9 @@
 //   lap_o = p lap_v + pL v                                   (pL: same as p'_c with lap_q, lap_k)
 //         + [ X + p * (2 G - u - rowsum(p * 2 G)) ] v + 2 sum_c p'_c v'_c
 //   X = sum_c p'_c * (s'_c - rowsum(p s'_c)),  G = sum_c q'_c k'_c^T,  u = sum_c rowsum(p'_c s'_c)
-// i.e. six n x n x d matrix products per row, all on v_mfma_f32_16x16x4_f32.
+// i.e. six n x n x d matrix products per row, all on v_mfma_f32_16x16x4_f32.  With an edge
+// bias e (s = q k^T + e) the rows e'_c and lap_e are added to s'_c and to the Laplacian's
+// first-order part; they have no second-order contribution.
 //
 // Mapping: wavefront w owns query rows [16 w, 16 w + 16) and every key column, so all
 // row reductions stay inside 16-lane groups of one wavefront.  k, v and the current
@@ -38,13 +40,14 @@ __device__ __forceinline__ float f4get(const float4& v, int r) {
 
 struct MhsaArgs {
   const float *q, *qj, *ql, *k, *kj, *kl, *v, *vj, *vl;
+  const float *e, *ej, *el;  // optional edge bias [B][n][H][n] and its Jacobian rows / Laplacian
   const uint8_t *mask, *imask;
   float *o, *oj, *ol;
   int64_t B;
   int32_t n, H, d, P;
 };
 
-template <int NW, int DT>
+template <int NW, int DT, bool EDGE>
 __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   constexpr int NP = 16 * NW;   // padded sequence length
   constexpr int DP = 16 * DT;   // padded head dim
@@ -75,6 +78,19 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   const int64_t slice = B * n * tok;                  // stride between Jacobian rows
 
   auto valid = [&](int i) -> bool { return i < n && (a.mask == nullptr || a.mask[b * n + i] != 0); };
+  // edge-bias entries of this lane in result layout: row 16 w + 4 lg + r, column 16 jt + l16
+  const int64_t etok = (int64_t)H * n;
+  const int64_t ebase = (b * n) * etok + (int64_t)h * n;
+  const int64_t eslice = B * n * etok;
+  auto edge_add = [&](const float* src, floatx4* acc) {
+#pragma unroll
+    for (int jt = 0; jt < NW; ++jt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 16 * w + 4 * lg + r, col = 16 * jt + l16;
+        if (row < n && col < n) acc[jt][r] += src[ebase + (int64_t)row * etok + col];
+      }
+  };
 
   // cooperative load of an (n x d) tile into LDS, rows of padding electrons zeroed
   float4 rk[LD4], rv[LD4];
@@ -181,6 +197,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
     for (int jt = 0; jt < NW; ++jt) s[jt] = floatx4{0.f, 0.f, 0.f, 0.f};
     qk_product(qa, ks, s);
+    if constexpr (EDGE) edge_add(a.e, s);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float mx = -INFINITY;
@@ -266,6 +283,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       for (int jt = 0; jt < NW; ++jt) sj[jt] = floatx4{0.f, 0.f, 0.f, 0.f};
       qk_product(qja, ks, sj);
       qk_product(qa, kjs[buf], sj);
+      if constexpr (EDGE) edge_add(is_lap ? a.el : a.ej + (int64_t)c * eslice, sj);
       if (!is_lap) qk_product(qja, kjs[buf], G);
       // p'_c = p * (s'_c - rowsum(p s'_c))
       floatx4 pj[NW];
@@ -343,7 +361,10 @@ template <int NW, int DT>
 int launch_mhsa(hipStream_t st, const MhsaArgs& a) {
   const int64_t blocks = a.B * a.H;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-  mhsa_kernel<NW, DT><<<dim3((unsigned)blocks), dim3(FOLX_WAVE * NW), 0, st>>>(a);
+  if (a.e != nullptr)
+    mhsa_kernel<NW, DT, true><<<dim3((unsigned)blocks), dim3(FOLX_WAVE * NW), 0, st>>>(a);
+  else
+    mhsa_kernel<NW, DT, false><<<dim3((unsigned)blocks), dim3(FOLX_WAVE * NW), 0, st>>>(a);
   return folx_launch_status();
 }
 
@@ -360,21 +381,22 @@ int launch_mhsa_d(hipStream_t st, const MhsaArgs& a) {
 
 }  // namespace
 
-extern "C" int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q_jac,
-                                    const float* q_lap, const float* k, const float* k_jac,
-                                    const float* k_lap, const float* v, const float* v_jac,
-                                    const float* v_lap, const uint8_t* mask,
-                                    const uint8_t* input_mask, float* o, float* o_jac, float* o_lap,
-                                    int64_t B, int32_t n, int32_t H, int32_t d, int32_t P) {
+static int mhsa_entry(void* stream, const float* q, const float* q_jac, const float* q_lap,
+                      const float* k, const float* k_jac, const float* k_lap, const float* v,
+                      const float* v_jac, const float* v_lap, const float* e, const float* e_jac,
+                      const float* e_lap, const uint8_t* mask, const uint8_t* input_mask, float* o,
+                      float* o_jac, float* o_lap, int64_t B, int32_t n, int32_t H, int32_t d,
+                      int32_t P) {
   if (B < 0 || n <= 0 || H <= 0 || d <= 0 || P < 0) return FOLX_HIP_EINVAL;
   if (B == 0) return FOLX_HIP_OK;
   if (!q || !q_lap || !k || !k_lap || !v || !v_lap || !o || !o_lap) return FOLX_HIP_EINVAL;
   if (P > 0 && (!q_jac || !k_jac || !v_jac || !o_jac)) return FOLX_HIP_EINVAL;
+  if (e != nullptr && (!e_lap || (P > 0 && !e_jac))) return FOLX_HIP_EINVAL;
   if (n > 64 || d > 64 || d % 4 != 0) return FOLX_HIP_ENOTSUP;
   const float* ptrs[] = {q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap};
   for (const float* p : ptrs)
     if (p && !folx_aligned16(p)) return FOLX_HIP_ENOTSUP;
-  MhsaArgs a{q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, mask, input_mask,
+  MhsaArgs a{q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, e, e_jac, e_lap, mask, input_mask,
              o, o_jac, o_lap, B, n, H, d, P};
   hipStream_t st = (hipStream_t)stream;
   const int nw = (n + 15) / 16;
@@ -384,4 +406,26 @@ extern "C" int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q
     case 3: return launch_mhsa_d<3>(st, a);
     default: return launch_mhsa_d<4>(st, a);
   }
+}
+
+extern "C" int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q_jac,
+                                    const float* q_lap, const float* k, const float* k_jac,
+                                    const float* k_lap, const float* v, const float* v_jac,
+                                    const float* v_lap, const uint8_t* mask,
+                                    const uint8_t* input_mask, float* o, float* o_jac, float* o_lap,
+                                    int64_t B, int32_t n, int32_t H, int32_t d, int32_t P) {
+  return mhsa_entry(stream, q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, nullptr, nullptr, nullptr,
+                    mask, input_mask, o, o_jac, o_lap, B, n, H, d, P);
+}
+
+extern "C" int folx_hip_mhsea_fwdlap(void* stream, const float* q, const float* q_jac,
+                                     const float* q_lap, const float* k, const float* k_jac,
+                                     const float* k_lap, const float* e, const float* e_jac,
+                                     const float* e_lap, const float* v, const float* v_jac,
+                                     const float* v_lap, const uint8_t* mask,
+                                     const uint8_t* input_mask, float* o, float* o_jac, float* o_lap,
+                                     int64_t B, int32_t n, int32_t H, int32_t d, int32_t P) {
+  if (!e) return FOLX_HIP_EINVAL;
+  return mhsa_entry(stream, q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, e, e_jac, e_lap, mask,
+                    input_mask, o, o_jac, o_lap, B, n, H, d, P);
 }

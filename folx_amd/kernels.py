@@ -302,12 +302,26 @@ def slogdet(A, AJ, AL):
     return sign, ld, ldj, ldl
 
 
-def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None):
-    """q/k/v (B, n, H, d) triplets; mask uint8 (B, n); input_mask uint8 (P, B)."""
+def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None):
+    """q/k/v (B, n, H, d) triplets; mask uint8 (B, n); input_mask uint8 (P, B); ``edge`` =
+    optional (e, e_jac, e_lap) bias triplet with e (B, n, H, n)."""
     _chk(q, qj, ql, k, kj, kl, v, vj, vl, mask, input_mask)
     B, n, H, d = q.shape
     P = qj.shape[0]
     o, oj, ol = torch.empty_like(q), torch.empty_like(qj), torch.empty_like(q)
+    if edge is not None:
+        e, ej, el = edge
+        _chk(e, ej, el)
+        assert tuple(e.shape) == (B, n, H, n) and ej.shape[0] == P
+        with _timed('mhsea_fwdlap', (B, n, H, d, P)):
+            check(
+                _lib.load().folx_hip_mhsea_fwdlap(
+                    _stream(), _p(q), _p(qj), _p(ql), _p(k), _p(kj), _p(kl), _p(e), _p(ej), _p(el),
+                    _p(v), _p(vj), _p(vl), _p(mask), _p(input_mask), _p(o), _p(oj), _p(ol), B, n, H, d, P,
+                ),
+                'mhsea_fwdlap',
+            )
+        return o, oj, ol
     with _timed('mhsa_fwdlap', (B, n, H, d, P)):
         check(
             _lib.load().folx_hip_mhsa_fwdlap(

@@ -114,10 +114,12 @@ def det(A):
     return _call('det', (A,))
 
 
-def multi_head_self_attention(q, k, v, mask=None, input_mask=None, **kwargs):
-    """softmax(q k^T) v over per-walker arrays (n, H, d); no 1/sqrt(d) inside.  Same
-    registry key as the reference's jitted wrapper
-    (folx/experimental/pallas/attention/__init__.py:17-45)."""
+def multi_head_self_attention(q, k, v, mask=None, input_mask=None, bias=None, **kwargs):
+    """softmax(q k^T (+ bias)) v over per-walker arrays (n, H, d); no 1/sqrt(d) inside;
+    ``bias`` is an optional edge-bias triplet (n, H, n).  Same registry keys as the
+    reference's jitted wrappers (folx/experimental/pallas/attention/__init__.py:17-80)."""
+    if bias is not None:
+        return _call('_multi_head_self_edge_attention', (q, k, bias, v, mask, input_mask), kwargs)
     return _call('_multi_head_self_attention', (q, k, v, mask, input_mask), kwargs)
 
 

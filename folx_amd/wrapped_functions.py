@@ -814,11 +814,13 @@ def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
     """
     del sparsity_threshold
     q, k, v, mask, input_mask = (tuple(args) + (None, None))[:5]
+    bias = kwargs.get('bias')
     if not (_is(q) and _is(k) and _is(v)):
         raise NotImplementedError('multi_head_self_attention needs derivative-carrying q, k, v')
     B, dev = q.B, q.x.device
     n = q.shape[0]
-    Js = [t.jacobian.dense_array for t in (q, k, v)]
+    trip = (q, k, v) if bias is None else (q, k, v, bias)
+    Js = [t.jacobian.dense_array for t in trip]
     P = max(J.shape[0] for J in Js)
     Js = [so.pad_rows(J, P) for J in Js]
     mt = _mask_tensor(mask, (B, n), dev)
@@ -833,8 +835,20 @@ def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
             im = im[:, None]
         assert im.shape[0] == P, 'input_mask must have one entry per Jacobian row'
         it = _mask_tensor(im, (P, B), dev)
-    o, oj, ol = K.mhsa(q.x, Js[0], q.laplacian, k.x, Js[1], k.laplacian, v.x, Js[2], v.laplacian, mt, it)
+    edge = None if bias is None else (bias.x, Js[3], bias.laplacian)
+    o, oj, ol = K.mhsa(q.x, Js[0], q.laplacian, k.x, Js[1], k.laplacian, v.x, Js[2], v.laplacian, mt, it, edge)
     return FwdLaplArray(o, FwdJacobian(oj, None), ol)
+
+
+def mhsea_forward_laplacian(args, kwargs, sparsity_threshold):
+    """Rule of ``multi_head_self_edge_attention`` with the reference's argument order
+    ``(q, k, e, v, mask, input_mask)`` (``mhsea_forward_laplacian``,
+    folx/experimental/pallas/attention/forward_laplacian.py:495-614): scores
+    ``q k^T + e`` with an edge-bias triplet ``e`` of per-walker shape (n, H, n)."""
+    q, k, e, v, mask, input_mask = (tuple(args) + (None, None))[:6]
+    if not _is(e):
+        raise NotImplementedError('multi_head_self_edge_attention needs a derivative-carrying edge bias')
+    return mhsa_forward_laplacian((q, k, v, mask, input_mask), {**kwargs, 'bias': e}, sparsity_threshold)
 
 
 # --------------------------------------------------------------------------------------
@@ -865,3 +879,4 @@ register_function('reduce_max_values', reduce_max_values)
 register_function('slogdet', slogdet_wrapper)
 register_function('det', det_wrapper)
 register_function('_multi_head_self_attention', mhsa_forward_laplacian)
+register_function('_multi_head_self_edge_attention', mhsea_forward_laplacian)

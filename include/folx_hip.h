@@ -200,6 +200,20 @@ int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q_jac, const
                          float* o_jac, float* o_lap, int64_t B, int32_t n, int32_t H,
                          int32_t d, int32_t P);
 
+/*
+ * Edge-bias variant: o = softmax(q k^T + e) v with e, e_lap [B][n][H][n], e_jac [P][B][n][H][n]
+ * (argument order q, k, e, v as in the reference's rule).  Replaces mhsea_forward_laplacian
+ * and its Pallas kernel (folx/experimental/pallas/attention/forward_laplacian.py:495-614,
+ * :745-854).  Same size limits as folx_hip_mhsa_fwdlap.
+ */
+int folx_hip_mhsea_fwdlap(void* stream, const float* q, const float* q_jac, const float* q_lap,
+                          const float* k, const float* k_jac, const float* k_lap,
+                          const float* e, const float* e_jac, const float* e_lap,
+                          const float* v, const float* v_jac, const float* v_lap,
+                          const uint8_t* mask, const uint8_t* input_mask, float* o,
+                          float* o_jac, float* o_lap, int64_t B, int32_t n, int32_t H,
+                          int32_t d, int32_t P);
+
 #ifdef __cplusplus
 }
 #endif

@@ -399,10 +399,13 @@ def slogdet(A: OArr):
     return OConst(sign), OArr(ld, J, L)
 
 
-def multi_head_self_attention(q: OArr, k: OArr, v: OArr, mask=None, input_mask=None):
-    o, oJ, oL = rules.mhsa_rule(
-        q.x, q.J, q.lap, k.x, k.J, k.lap, v.x, v.J, v.lap, mask, input_mask
-    )
+def multi_head_self_attention(q: OArr, k: OArr, v: OArr, mask=None, input_mask=None, bias=None):
+    """``bias`` = optional edge-bias triplet of per-walker shape (n, H, n)."""
+    if bias is None:
+        o, oJ, oL = rules.mhsa_rule(q.x, q.J, q.lap, k.x, k.J, k.lap, v.x, v.J, v.lap, mask, input_mask)
+    else:
+        o, oJ, oL = rules.mhsa_rule(q.x, q.J, q.lap, k.x, k.J, k.lap, v.x, v.J, v.lap, mask, input_mask,
+                                    bias.x, bias.J, bias.lap)
     return OArr(o, oJ, oL)
 
 

@@ -255,14 +255,17 @@ def big_number(dtype) -> float:
     return 1e40 if np.dtype(dtype) == np.float64 else 1e20
 
 
-def mhsa_forward(q, k, v, mask=None):
-    """softmax(q k^T) v with padded-sequence masking and no 1/sqrt(d) inside
-    (folx/experimental/pallas/attention/mhsa.py:79-94).  q, k, v: (B, n, H, d)."""
+def mhsa_forward(q, k, v, mask=None, e=None):
+    """softmax(q k^T (+ e)) v with padded-sequence masking and no 1/sqrt(d) inside
+    (folx/experimental/pallas/attention/mhsa.py:79-94, mhsea.py:80-97).
+    q, k, v: (B, n, H, d); e: (B, n, H, n)."""
     B, n, H, d = q.shape
     if mask is None:
         mask = np.ones((B, n), dtype=bool)
     sq = mask[:, :, None, None] & mask[:, None, None, :]
     s = np.einsum('bihd,bjhd->bihj', q, k)
+    if e is not None:
+        s = s + e
     s = np.where(sq, s, -big_number(s.dtype))
     s = s - s.max(-1, keepdims=True)
     e = np.exp(s)
@@ -270,8 +273,13 @@ def mhsa_forward(q, k, v, mask=None):
     return np.einsum('bihj,bjhd->bihd', p, v), p
 
 
-def mhsa_rule(q, qJ, qL, k, kJ, kL, v, vJ, vL, mask=None, input_mask=None):
-    """Forward Laplacian of masked multi-head self attention.
+def mhsa_rule(q, qJ, qL, k, kJ, kL, v, vJ, vL, mask=None, input_mask=None, e=None, eJ=None, eL=None):
+    """Forward Laplacian of masked multi-head self attention, optionally with an additive
+    edge bias ``e (B, n, H, n)`` on the scores (``s = q k^T + e``): the edge term enters
+    ``s'_c`` and the direct Laplacian part linearly and has no second-order contribution
+    (folx/experimental/pallas/attention/forward_laplacian.py:663-704).  Its Jacobian rows
+    are zeroed for inactive coordinates only (:649).
+
 
     Specification: folx/experimental/pallas/attention/forward_laplacian.py:212-346 (einsum
     form) and :349-487 (kernel form); the algebra below is the factored form the same
@@ -306,14 +314,18 @@ def mhsa_rule(q, qJ, qL, k, kJ, kL, v, vJ, vL, mask=None, input_mask=None):
     qJ, kJ, vJ = (np.where(cm, a, 0.0) for a in (qJ, kJ, vJ))
     qL, kL, vL = (np.where(em, a, 0.0) for a in (qL, kL, vL))
 
-    o, p = mhsa_forward(q, k, v, mask)
+    o, p = mhsa_forward(q, k, v, mask, e)
 
     sJ = np.einsum('pbihd,bjhd->pbihj', qJ, k) + np.einsum('bihd,pbjhd->pbihj', q, kJ)
+    if e is not None:
+        sJ = sJ + np.where(input_mask[:, :, None, None, None], eJ, 0.0)
     rJ = (p[None] * sJ).sum(-1, keepdims=True)
     pJ = p[None] * (sJ - rJ)
     oJ = np.einsum('bihj,pbjhd->pbihd', p, vJ) + np.einsum('pbihj,bjhd->pbihd', pJ, v)
 
     sL = np.einsum('bihd,bjhd->bihj', qL, k) + np.einsum('bihd,bjhd->bihj', q, kL)
+    if e is not None:
+        sL = sL + eL
     pL = p * (sL - (p * sL).sum(-1, keepdims=True))
     oL = np.einsum('bihj,bjhd->bihd', p, vL) + np.einsum('bihj,bjhd->bihd', pL, v)
 

@@ -177,9 +177,11 @@ class plain:
         return sign.detach(), ld
 
     @staticmethod
-    def multi_head_self_attention(q, k, v, mask=None, input_mask=None):
-        # q, k, v: (n, H, d); softmax(q k^T) v, no 1/sqrt(d) inside
+    def multi_head_self_attention(q, k, v, mask=None, input_mask=None, bias=None):
+        # q, k, v: (n, H, d); softmax(q k^T (+ bias)) v, no 1/sqrt(d) inside
         s = torch.einsum('ihd,jhd->ihj', q, k)
+        if bias is not None:
+            s = s + bias
         if mask is not None:
             m = torch.as_tensor(np.asarray(mask), dtype=torch.bool)
             sq = m[:, None, None] & m[None, None, :]

@@ -101,10 +101,11 @@ def slogdet(A, AJ, AL):
     return _t(sign), _t(ld), _t(jac), _t(lap)
 
 
-def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None):
+def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None):
     m = None if mask is None else mask.cpu().numpy().astype(bool)
     im = None if input_mask is None else input_mask.cpu().numpy().astype(bool)
-    return tuple(_t(a) for a in rules.mhsa_rule(*[_n(t) for t in (q, qj, ql, k, kj, kl, v, vj, vl)], m, im))
+    ed = () if edge is None else tuple(_n(t) for t in edge)
+    return tuple(_t(a) for a in rules.mhsa_rule(*[_n(t) for t in (q, qj, ql, k, kj, kl, v, vj, vl)], m, im, *ed))
 
 
 def install(monkeypatch):

@@ -47,6 +47,7 @@ def test_argument_checks_return_error_codes(lib):
     assert lib.folx_hip_slogdet_fwdlap(null, null, null, null, null, null, null, null, 4, 0, 1) == _lib.EINVAL
     assert lib.folx_hip_layernorm_fwdlap(*([null] * 9), 4, 8, 1, 1e-5) == _lib.EINVAL
     assert lib.folx_hip_mhsa_fwdlap(*([null] * 15), 1, 8, 1, 8, 1) == _lib.EINVAL
+    assert lib.folx_hip_mhsea_fwdlap(*([null] * 18), 1, 8, 1, 8, 1) == _lib.EINVAL
     # empty problems are fine and launch nothing
     assert lib.folx_hip_dense_fwdlap(*([null] * 12), 0, 1, 8, 8) == _lib.OK
     assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 0, 1) == _lib.OK

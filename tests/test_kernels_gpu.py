@@ -305,3 +305,28 @@ def test_dense_residual_epilogue():
     ref = tuple(r + s for r, s in zip(ref, f64(rx, rJ, rL)))
     got = K.dense(dev(x), dev(J), dev(L), dev(W), dev(b), (dev(rx), dev(rJ), dev(rL)))
     assert_triplet(got, ref, 'dense + residual')
+
+
+@pytest.mark.parametrize('B,n,H,d,P,valid', [(2, 1, 1, 4, 3, None), (1, 16, 4, 32, 48, None), (1, 16, 4, 32, 48, 4),
+                                             (2, 32, 4, 64, 12, None), (2, 20, 2, 24, 9, 13)])
+def test_mhsea(B, n, H, d, P, valid):
+    """Edge-bias attention (shapes of test_attention.py:389-395)."""
+    from folx_amd import kernels as K
+
+    print(f'case mhsea B={B} n={n} H={H} d={d} P={P} valid={valid}', flush=True)
+    rng = np.random.default_rng(13)
+    args = []
+    for s in [1 / np.sqrt(d), 1.0, 1.0]:
+        args += [s * rand(rng, B, n, H, d), s * rand(rng, P, B, n, H, d), s * rand(rng, B, n, H, d)]
+    edge = [rand(rng, B, n, H, n), rand(rng, P, B, n, H, n), rand(rng, B, n, H, n)]
+    mask = np.ones((B, n), dtype=bool)
+    imask = np.ones((P, B), dtype=bool)
+    if valid is not None:
+        mask[:, valid:] = False
+        imask[min(P, 3 * valid):] = False
+    ref = rules.mhsa_rule(*f64(*args), mask, imask, *f64(*edge))
+    got = K.mhsa(*[dev(t) for t in args], dev(mask, torch.uint8), dev(imask, torch.uint8), tuple(dev(t) for t in edge))
+    m = mask[0]
+    assert_val(got[0][:, m], ref[0][:, m], 'o')
+    assert_val(got[1][:, :, m], ref[1][:, :, m], 'o_jac')
+    assert_lap(got[2][:, m], ref[2][:, m], 'o_lap')

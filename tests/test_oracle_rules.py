@@ -251,3 +251,39 @@ def test_mhsa_masking_zeroes_inactive_rows():
     o2, oJ2, oL2 = rules.mhsa_rule(*args2, None, in_mask)
     _close(oL, oL2)
     _close(oJ, oJ2)
+
+
+@pytest.mark.parametrize('n,H,d,valid', [(1, 1, 1, 1), (4, 2, 3, 4), (5, 2, 3, 3)])
+def test_mhsea_vs_bruteforce(n, H, d, valid):
+    """softmax(q k^T + e) v with an input-dependent edge bias, incl. a padded sequence
+    (test/experimental/pallas/test_attention.py:389-459)."""
+    rng = np.random.default_rng(18)
+    n_in = 3 * n
+    Wq, Wk, Wv = (rng.normal(size=(n_in, n * H * d)) / np.sqrt(n_in) for _ in range(3))
+    We = rng.normal(size=(n_in, n * H * n)) / np.sqrt(n_in)
+    mask = np.zeros(n, dtype=bool)
+    mask[:valid] = True
+    in_mask = np.zeros(n_in, dtype=bool)
+    in_mask[: 3 * valid] = True
+
+    def f(xp, x):
+        x = xp.reshape(x, (n_in,))
+        q, k, v = (xp.reshape(xp.tanh(xp.dot(x, W)), (n, H, d)) for W in (Wq, Wk, Wv))
+        e = xp.reshape(xp.sin(xp.dot(x, We)), (n, H, n))
+        if xp is plain:
+            return xp.multi_head_self_attention(q, k, v, mask, None, e)
+        B = q.B
+        return xp.multi_head_self_attention(
+            q, k, v, np.broadcast_to(mask, (B, n)), np.broadcast_to(in_mask[:, None], (n_in, B)), e)
+
+    x = rng.normal(size=(2, n_in))
+    out = f(ob, ob.init_state(x, weights=in_mask.astype(np.float64), dtype=np.float64))
+
+    def f_plain(t):
+        return f(plain, torch.where(torch.as_tensor(in_mask), t, t.detach()))
+
+    by, bJ, bL = brute_force(f_plain, x)
+    m = mask
+    _close(out.x[:, m], by[:, m], atol=1e-9)
+    _close(out.J[:, :, m], bJ[:, :, m], atol=1e-9)
+    _close(out.lap[:, m], bL[:, m], rtol=1e-5, atol=1e-8)
