@@ -27,8 +27,8 @@ PEAK_HBM_GBS = 8000.0
 # scaled by what the same counter reads for a plain 1 GiB copy: x2.000 and x1.000); the
 # figures and the commands are in profiles/psiformer32_forward_laplacian.txt.
 MEASURED_TRAFFIC_BYTES = {
-    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.692e9,
-    ('dense_fwdlap', (32768, 96, 256, 256, True)): 10.029e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.757e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, True)): 10.050e9,
     ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.153e9,
 }
 
@@ -65,7 +65,7 @@ def cpu_baseline(workload, budget_s):
         threads = 1
 
     def run(n):
-        x = wl.sample_electrons(n, cfg.n_elec, sigma, seed=2)
+        x = wl.sample_inputs(workload, n, seed=2)
         t0 = time.perf_counter()
         out = forward(p, ob.init_state(x, dtype=np.float32), ob)
         dt = time.perf_counter() - t0
@@ -85,6 +85,9 @@ def cpu_baseline(workload, budget_s):
 
 
 def describe(cfg):
+    if hasattr(cfg, 'n_nodes'):
+        return (f'node-wise MLP, {cfg.n_nodes} nodes x {cfg.in_dim} inputs, {cfg.n_hidden} x [Dense({cfg.width}) + SiLU] '
+                f'+ Dense(1), summed')
     if hasattr(cfg, 'n_heads'):
         return (f'PsiFormer-style, {cfg.n_elec} electrons, {cfg.n_nuc} nuclei, {cfg.n_layers} layers x '
                 f'{cfg.n_heads} heads x {cfg.head_dim}, width {cfg.width}, {cfg.n_det} determinants')
@@ -111,7 +114,7 @@ def main():
     dev = torch.device('cuda', 0)
     torch.cuda.set_device(dev)
     params = wl.to_device(params_np, dev)
-    x = torch.as_tensor(wl.sample_electrons(B, cfg.n_elec, sigma, seed=2)).to(dev)
+    x = torch.as_tensor(wl.sample_inputs(args.workload, B, seed=2)).to(dev)
     fl = folx_amd.forward_laplacian(lambda r: forward(params, r), thr)
     step = folx_amd.batched_vmap(folx_amd.jit(folx_amd.vmap(fl)) if args.graph else fl, args.chunk)
 
@@ -190,7 +193,7 @@ def main():
             'workload': f'{args.workload}: {describe(cfg)}, ForwardLaplacianOperator({thr})',
             'walkers': B,
             'chunk': args.chunk,
-            'jacobian_rows': 3 * cfg.n_elec,
+            'jacobian_rows': int(out.jacobian.dense_array.shape[0]),
         },
         'roofline': roof,
         'kernel_ms_per_step': {k: v / args.steps for k, v in sorted(per_kernel.items(), key=lambda kv: -kv[1])},

@@ -317,10 +317,32 @@ def sample_electrons(n_walkers, n_elec, sigma, seed):
     return (sigma * np.random.default_rng(seed).normal(size=(n_walkers, n_elec, 3))).astype(np.float32)
 
 
+@dataclass
+class MLPConfig:
+    """Node-wise MLP of the reference README: input (n_nodes, in_dim) per walker."""
+
+    n_nodes: int = 100
+    in_dim: int = 4
+    width: int = 100
+    n_hidden: int = 10
+    seed: int = 0
+
+
+def sample_inputs(name, n_walkers, seed=2):
+    """Seeded synthetic inputs (B, *shape) of a named configuration."""
+    cfg, _, sigma, _ = CONFIGS[name]
+    if isinstance(cfg, MLPConfig):
+        return np.random.default_rng(seed).normal(size=(n_walkers, cfg.n_nodes, cfg.in_dim)).astype(np.float32)
+    return sample_electrons(n_walkers, cfg.n_elec, sigma, seed)
+
+
 def build(name):
     """(forward(params, r, xp=None), params, config, walkers, sigma, threshold) of a named
     benchmark configuration."""
     cfg, walkers, sigma, thr = CONFIGS[name]
+    if isinstance(cfg, MLPConfig):
+        params = mlp_params(cfg.seed, cfg.in_dim, cfg.width, cfg.n_hidden)
+        return mlp_forward, params, cfg, walkers, sigma, thr
     if isinstance(cfg, FermiNetConfig):
         return ferminet_forward, ferminet_params(cfg), cfg, walkers, sigma, thr
     return psiformer_forward, psiformer_params(cfg), cfg, walkers, sigma, thr
@@ -328,6 +350,8 @@ def build(name):
 
 CONFIGS = {
     # name: (config, walkers, position sigma, sparsity threshold)
+    'mlp_dense': (MLPConfig(), 20, 1.0, 0),     # README.md:63-65, ForwardLaplacianOperator(0)
+    'mlp_sparse': (MLPConfig(), 256, 1.0, 4),   # README.md:68-70 model, ForwardLaplacianOperator(4)
     'ferminet16': (FermiNetConfig(), 4096, 1.5, 6),
     'psiformer32': (PsiFormerConfig(), 4096, 1.5, 6),
     'psiformer64': (
