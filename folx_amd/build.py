@@ -28,6 +28,7 @@ SOURCES = [
     'slogdet.hip',
     'mhsa.hip',
     'layernorm.hip',
+    'linsolve.hip',
 ]
 
 # Packed FP32 instructions are switched off for all device code (-packed-fp32-ops).

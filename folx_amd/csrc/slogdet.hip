@@ -9,22 +9,18 @@
 //      of A^-1 in registers, ld_jac[p] = tr M, and sum_p tr(M M) through an LDS transpose.
 // The Jacobian is read exactly once, so the kernel is bound by HBM bandwidth as long as
 // the 2 n^3 flops per row stay hidden (they do for n <= 32 on the vector ALUs).
-#include "common.h"
+#include "smallmat.h"
 
 namespace {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = FOLX_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, FOLX_WAVE);
-  return v;
-}
+using smallmat::wave_sum;
 
 template <int NP>
 __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P) {
-  constexpr int AUGS = 2 * NP + 1;     // row stride of the augmented matrix
+  constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
   constexpr int G = FOLX_WAVE / NP;    // lane groups per row
   constexpr int CPL = NP / G;          // columns of M per lane
   constexpr int MS = NP + 1;           // row stride of the M staging tile
@@ -38,76 +34,9 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   const int64_t nn = (int64_t)n * n;
   const float* a = A + m * nn;
 
-  // ---- stage [A | I], zero padded (padding rows get a unit diagonal on the A side so
-  // the elimination leaves them alone; their inverse block stays zero-coupled) ----------
-  for (int e = lane; e < NP * 2 * NP; e += FOLX_WAVE) {
-    const int i = e / (2 * NP), j = e % (2 * NP);
-    float v;
-    if (j < NP) v = (i < n && j < n) ? a[i * n + j] : (i == j ? 1.0f : 0.0f);
-    else v = (j - NP == i) ? 1.0f : 0.0f;
-    aug[i * AUGS + j] = v;
-  }
-  __syncthreads();
-
-  float logdet = 0.0f, sgn = 1.0f;
-  for (int k = 0; k < n; ++k) {
-    // pivot search over rows k..n-1 of column k (first maximum wins, as in idamax)
-    float best = -1.0f;
-    int bi = k;
-    if (lane >= k && lane < n) { best = fabsf(aug[lane * AUGS + k]); bi = lane; }
-#pragma unroll
-    for (int off = FOLX_WAVE / 2; off > 0; off >>= 1) {
-      const float ob = __shfl_xor(best, off, FOLX_WAVE);
-      const int oi = __shfl_xor(bi, off, FOLX_WAVE);
-      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
-    }
-    if (bi != k) {
-      for (int j = lane; j < 2 * NP; j += FOLX_WAVE) {
-        const float t = aug[k * AUGS + j];
-        aug[k * AUGS + j] = aug[bi * AUGS + j];
-        aug[bi * AUGS + j] = t;
-      }
-      sgn = -sgn;
-      __syncthreads();
-    }
-    const float pv = aug[k * AUGS + k];
-    logdet += logf(fabsf(pv));
-    if (pv < 0.0f) sgn = -sgn;
-    if (pv == 0.0f) sgn = 0.0f;
-    const float rp = 1.0f / pv;
-    __syncthreads();
-    float rowk[(2 * NP + FOLX_WAVE - 1) / FOLX_WAVE];
-#pragma unroll
-    for (int c = 0; c < (2 * NP + FOLX_WAVE - 1) / FOLX_WAVE; ++c) {
-      const int j = lane + c * FOLX_WAVE;
-      if (j < 2 * NP) {
-        rowk[c] = aug[k * AUGS + j] * rp;
-        aug[k * AUGS + j] = rowk[c];
-      }
-    }
-    __syncthreads();
-    for (int i = 0; i < n; ++i) {
-      if (i == k) continue;
-      const float f = aug[i * AUGS + k];
-      __syncthreads();  // everyone has read f before column k of row i is overwritten
-#pragma unroll
-      for (int c = 0; c < (2 * NP + FOLX_WAVE - 1) / FOLX_WAVE; ++c) {
-        const int j = lane + c * FOLX_WAVE;
-        if (j < 2 * NP) aug[i * AUGS + j] -= f * rowk[c];
-      }
-    }
-    __syncthreads();
-  }
-
-  // ---- tr(A^-1 lap_A) = sum_ij Ainv[j][i] lap[i][j] -----------------------------------
-  float tl = 0.0f;
-  {
-    const float* l = AL + m * nn;
-    for (int e = lane; e < nn; e += FOLX_WAVE) {
-      const int i = e / n, j = e % n;
-      tl += aug[j * AUGS + NP + i] * l[e];
-    }
-  }
+  float logdet, sgn;
+  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn);
+  float tl = smallmat::trace_inv_times<NP>(aug, AL + m * nn, n, lane);
 
   // ---- row i of A^-1 in registers -------------------------------------------------------
   const int i = lane % NP;
@@ -182,6 +111,86 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   }
 }
 
+// slogdet rule from rank-one factors of dA/dx_c (sparse Jacobian whose coordinate c touches
+// few rows, columns or entries of A).  For coordinate c, factor s collects `width` entries
+// dA[r_s][j_l]/dx_c (addresses in `take`, columns j_l in `cols`), `rows[c][t]` is the row of
+// factor t, and
+//     W_c[s][t] = sum_l dA[r_s][j_l]/dx_c * Ainv[j_l][r_t]
+// gives d_c log|det A| = tr W_c and lap = tr(Ainv lap_A) - sum_c sum_st W_c[s][t] W_c[t][s].
+// With `transposed` the tables describe A^T: addresses already point into A, and the
+// inverse is read transposed.  One wavefront per matrix, tables shared by all matrices.
+constexpr int SP_MAX_RANK = 64;       // W_c tile held in LDS: rank^2 floats
+constexpr int SP_MAX_FACTOR = 2048;   // staged factor entries per coordinate: rank * width
+
+template <int NP>
+__global__ __launch_bounds__(FOLX_WAVE) void sparse_slogdet_kernel(
+    const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
+    const int32_t* __restrict__ take, const int32_t* __restrict__ cols, const int32_t* __restrict__ rows,
+    float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
+    float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t n_coords, int32_t rank, int32_t width,
+    int32_t transposed) {
+  constexpr int AUGS = smallmat::Aug<NP>::stride;
+  __shared__ float aug[NP * AUGS];
+  __shared__ float wb[SP_MAX_RANK * SP_MAX_RANK];
+  __shared__ float vb[SP_MAX_FACTOR];
+  __shared__ int32_t cb[SP_MAX_FACTOR];
+  __shared__ int32_t rb[SP_MAX_RANK];
+
+  const int lane = threadIdx.x;
+  const int64_t m = blockIdx.x;
+  const int64_t nn = (int64_t)n * n;
+  float logdet, sgn;
+  smallmat::gauss_jordan<NP>(aug, A + m * nn, n, lane, logdet, sgn);
+  float tl = smallmat::trace_inv_times<NP>(aug, AL + m * nn, n, lane);
+
+  const int rw = rank * width;
+  float pair = 0.0f;
+  for (int c = 0; c < n_coords; ++c) {
+    // stage the factor entries of this coordinate
+    for (int e = lane; e < rw; e += FOLX_WAVE) {
+      const int32_t t = take[(int64_t)c * rw + e];
+      float v = 0.0f;
+      if (t >= 0) {
+        const int32_t row = t / (int32_t)nn, rem = t % (int32_t)nn;
+        v = AJ[((int64_t)row * NM + m) * nn + rem];
+      }
+      vb[e] = v;
+      cb[e] = cols[(int64_t)c * rw + e];
+    }
+    for (int e = lane; e < rank; e += FOLX_WAVE) rb[e] = rows[(int64_t)c * rank + e];
+    __syncthreads();
+    for (int e = lane; e < rank * rank; e += FOLX_WAVE) {
+      const int s = e / rank, t = e % rank;
+      const int rt = rb[t];
+      float w = 0.0f;
+      for (int l = 0; l < width; ++l) {
+        const int j = cb[s * width + l];
+        const float ai = transposed ? aug[rt * AUGS + NP + j] : aug[j * AUGS + NP + rt];
+        w += vb[s * width + l] * ai;
+      }
+      wb[e] = w;
+    }
+    __syncthreads();
+    float tr = 0.0f;
+    for (int e = lane; e < rank * rank; e += FOLX_WAVE) {
+      const int s = e / rank, t = e % rank;
+      const float w = wb[e];
+      if (s == t) tr += w;
+      pair += w * wb[t * rank + s];
+    }
+    tr = wave_sum(tr);
+    if (lane == 0) jac_out[(int64_t)c * NM + m] = tr;
+    __syncthreads();  // wb, vb, cb, rb are rewritten by the next coordinate
+  }
+  pair = wave_sum(pair);
+  tl = wave_sum(tl);
+  if (lane == 0) {
+    sign_out[m] = sgn;
+    logdet_out[m] = logdet;
+    lap_out[m] = tl - pair;
+  }
+}
+
 }  // namespace
 
 extern "C" int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
@@ -200,5 +209,30 @@ extern "C" int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float
     slogdet_kernel<16><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P);
   else
     slogdet_kernel<32><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P);
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_sparse_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
+                                              const float* A_lap, const int32_t* take, const int32_t* cols,
+                                              const int32_t* rows, float* sign, float* logdet, float* ld_jac,
+                                              float* ld_lap, int64_t NM, int32_t n, int32_t k,
+                                              int32_t n_coords, int32_t rank, int32_t width,
+                                              int32_t transposed) {
+  if (NM < 0 || n <= 0 || k <= 0 || n_coords <= 0 || rank <= 0 || width <= 0) return FOLX_HIP_EINVAL;
+  if (NM == 0) return FOLX_HIP_OK;
+  if (!A || !A_jac || !A_lap || !take || !cols || !rows || !sign || !logdet || !ld_jac || !ld_lap)
+    return FOLX_HIP_EINVAL;
+  if (n > 32 || NM > 0x7fffffffLL || rank > SP_MAX_RANK || (int64_t)rank * width > SP_MAX_FACTOR ||
+      (int64_t)k * n * n > 0x7fffffffLL)
+    return FOLX_HIP_ENOTSUP;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)NM), block(FOLX_WAVE);
+#define FOLX_SP_LAUNCH(NPV)                                                                          \
+  sparse_slogdet_kernel<NPV><<<grid, block, 0, st>>>(A, A_jac, A_lap, take, cols, rows, sign, logdet, \
+                                                     ld_jac, ld_lap, NM, n, n_coords, rank, width, transposed)
+  if (n <= 8) FOLX_SP_LAUNCH(8);
+  else if (n <= 16) FOLX_SP_LAUNCH(16);
+  else FOLX_SP_LAUNCH(32);
+#undef FOLX_SP_LAUNCH
   return folx_launch_status();
 }

@@ -245,3 +245,109 @@ def dot_projection(mask: np.ndarray, contract_axis: int, threshold: int):
     if proj.shape[0] > threshold:
         return None, True
     return proj[..., None], True
+
+
+# --------------------------------------------------------------------------------------
+# sparse slogdet planner (folx/slogdet.py:73-293)
+# --------------------------------------------------------------------------------------
+
+SLOGDET_MAX_MASK_ENTRIES = 2**24  # bound of the host-side mask analysis (folx/slogdet.py:73)
+
+
+def slogdet_entry_mask(x0_idx, k: int, x_shape, transposed: bool):
+    """Mask ``(k, n, m)`` naming the input coordinate of every (stored row, matrix row,
+    column) entry, if it is the same for every batch position; else None
+    (``_entry_mask``, folx/slogdet.py:94-125).  ``transposed`` describes A^T."""
+    if x0_idx is None:
+        return None
+    idx = np.asarray(x0_idx)
+    shape = tuple(int(d) for d in x_shape)
+    if transposed:
+        if idx.ndim != len(shape) + 1:
+            return None
+        idx = idx.swapaxes(-1, -2)
+        shape = shape[:-2] + (shape[-1], shape[-2])
+    if k * int(np.prod(shape, dtype=np.int64)) > SLOGDET_MAX_MASK_ENTRIES:
+        return None
+    n, m = shape[-2:]
+    full = np.broadcast_to(idx, (k, *shape)).reshape(k, -1, n, m)
+    if not (full == full[:, :1]).all():
+        return None
+    return np.ascontiguousarray(full[:, 0]).astype(INT)
+
+
+def _rank_in_group(sorted_keys: np.ndarray) -> np.ndarray:
+    """Position of every element inside its run of equal (sorted) keys."""
+    return np.arange(sorted_keys.size) - np.searchsorted(sorted_keys, sorted_keys, side='left')
+
+
+def slogdet_factor_tables(mask: np.ndarray, per_entry: bool):
+    """Static tables that split every ``dA/dx_c`` into rank-one factors: one per touched
+    row, or one per touched entry with ``per_entry`` (``_factor_tables``,
+    folx/slogdet.py:142-179).  Returns ``(cost, tables)`` or None when the tables would
+    be too large; ``tables``: ``take (C, rank, width)`` flat (stored row, row, column)
+    addresses with ``k n m`` for unused slots, ``cols`` likewise, ``rows (C, rank)``,
+    ``coords (C,)``, ``per_entry``."""
+    k, n, m = mask.shape
+    flat = mask.reshape(-1)
+    pos = np.flatnonzero(flat >= 0)
+    coords, ci = np.unique(flat[pos], return_inverse=True)
+    ci = ci.reshape(-1)
+    r, c = np.divmod(pos % (n * m), m)
+    fkey = (ci * n + r) * m + (c if per_entry else 0)
+    # entries ordered by factor, then column, then stored row (pos is ascending in the latter)
+    order = np.lexsort((pos, c, fkey))
+    pos, c, fkey = pos[order], c[order], fkey[order]
+    fkeys, f_of = np.unique(fkey, return_inverse=True)
+    f_of = f_of.reshape(-1)
+    f_coord = fkeys // (n * m)
+    slot = _rank_in_group(f_coord)
+    within = _rank_in_group(fkey)
+    rank, width = int(slot.max()) + 1, int(within.max()) + 1
+    C = coords.size
+    if C * rank * width > SLOGDET_MAX_MASK_ENTRIES:
+        return None
+    take = np.full((C, rank, width), k * n * m, dtype=INT)
+    cols = np.zeros((C, rank, width), dtype=INT)
+    rows = np.zeros((C, rank), dtype=INT)
+    take[f_coord[f_of], slot[f_of], within] = pos
+    cols[f_coord[f_of], slot[f_of], within] = c
+    rows[f_coord, slot] = (fkeys % (n * m)) // m
+    cost = C * rank * rank * (1 if per_entry else width)
+    return cost, dict(take=take, cols=cols, rows=rows, coords=coords.astype(INT), per_entry=per_entry)
+
+
+def slogdet_plan(x0_idx, k: int, x_shape, max_n: int):
+    """Cheapest of the four decompositions (rows or entries of A, rows of A^T; the first
+    of equal costs wins), if it beats contracting the dense Jacobian (``sparse_slogdet``,
+    folx/slogdet.py:249-293).  Returns ``(tables, transposed)`` or None."""
+    best = None
+    for transposed in (False, True):
+        mask = slogdet_entry_mask(x0_idx, k, x_shape, transposed)
+        if mask is None or not (mask >= 0).any():
+            continue
+        for per_entry in ((False,) if transposed else (False, True)):
+            plan = slogdet_factor_tables(mask, per_entry)
+            if plan is not None and (best is None or plan[0] < best[0]):
+                best = (plan[0], plan[1], transposed)
+    if best is None:
+        return None
+    cost, tables, transposed = best
+    n, m = x_shape[-2:]
+    tangents = max_n + 1
+    if 4 * cost > tangents * n * m * (n + 1) or cost > 2 * tangents * n * m:
+        return None
+    return tables, transposed
+
+
+def slogdet_kernel_tables(tables, transposed: bool, k: int, n: int):
+    """int32 tables in the kernel's convention: ``take`` addresses the Jacobian as stored
+    (for tables of A^T the row and column of every address are swapped back) and unused
+    slots are ``-1``."""
+    take = tables['take']
+    valid = take < k * n * n
+    t, rem = np.divmod(np.where(valid, take, 0), n * n)
+    r, c = np.divmod(rem, n)
+    addr = (t * n + c) * n + r if transposed else (t * n + r) * n + c
+    take32 = np.where(valid, addr, -1).astype(np.int32)
+    return take32, tables['cols'].astype(np.int32), tables['rows'].astype(np.int32)

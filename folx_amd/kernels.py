@@ -302,6 +302,65 @@ def slogdet(A, AJ, AL):
     return sign, ld, ldj, ldl
 
 
+def sparse_slogdet(A, AJ, AL, take, cols, rows, transposed):
+    """A (.., n, n), AJ (k, .., n, n) stored rows, AL (.., n, n); int32 device tables take /
+    cols (C, rank, width) and rows (C, rank) -> sign, logdet (..), jac (C, ..), lap (..)."""
+    _chk(A, AJ, AL, take, cols, rows)
+    n = A.shape[-1]
+    k = AJ.shape[0]
+    C, rank, width = take.shape
+    lead = A.shape[:-2]
+    NM = int(np.prod(lead, dtype=np.int64)) if len(lead) else 1
+    sign = torch.empty(lead, device=A.device, dtype=torch.float32)
+    ld = torch.empty_like(sign)
+    ldj = torch.empty((C, *lead), device=A.device, dtype=torch.float32)
+    ldl = torch.empty_like(sign)
+    with _timed('sparse_slogdet_fwdlap', (NM, n, k, C, rank, width)):
+        check(
+            _lib.load().folx_hip_sparse_slogdet_fwdlap(
+                _stream(), _p(A), _p(AJ), _p(AL), _p(take), _p(cols), _p(rows), _p(sign), _p(ld), _p(ldj),
+                _p(ldl), NM, n, k, C, rank, width, int(bool(transposed))
+            ),
+            'sparse_slogdet_fwdlap',
+        )
+    return sign, ld, ldj, ldl
+
+
+def inv(A, AJ, AL):
+    """A (.., n, n), AJ (P, .., n, n), AL (.., n, n) -> C, C_jac, C_lap of the same shapes."""
+    _chk(A, AJ, AL)
+    n = A.shape[-1]
+    P = AJ.shape[0]
+    lead = A.shape[:-2]
+    NM = int(np.prod(lead, dtype=np.int64)) if len(lead) else 1
+    C, CJ, CL = torch.empty_like(A), torch.empty_like(AJ), torch.empty_like(AL)
+    with _timed('inv_fwdlap', (NM, n, P)):
+        check(_lib.load().folx_hip_inv_fwdlap(_stream(), _p(A), _p(AJ), _p(AL), _p(C), _p(CJ), _p(CL), NM, n, P),
+              'inv_fwdlap')
+    return C, CJ, CL
+
+
+def solve(A, AJ, AL, b, bJ, bL, P):
+    """A (.., n, n), b (.., n, m) with equal leading shapes; AJ/AL or bJ/bL may be None for
+    a constant operand -> y, y_jac (P, .., n, m), y_lap."""
+    _chk(A, AJ, AL, b, bJ, bL)
+    n, m = b.shape[-2:]
+    lead = A.shape[:-2]
+    assert tuple(b.shape[:-2]) == tuple(lead) and A.shape[-1] == n and A.shape[-2] == n
+    NM = int(np.prod(lead, dtype=np.int64)) if len(lead) else 1
+    y = torch.empty_like(b)
+    yJ = torch.empty((P, *b.shape), device=b.device, dtype=torch.float32)
+    yL = torch.empty_like(b)
+    with _timed('solve_fwdlap', (NM, n, m, P, AJ is not None, bJ is not None)):
+        check(
+            _lib.load().folx_hip_solve_fwdlap(
+                _stream(), _p(A), _p(AJ), _p(AL), _p(b), _p(bJ), _p(bL), _p(y), _p(yJ), _p(yL), NM, n, m, P
+            ),
+            'solve_fwdlap',
+        )
+    return y, yJ, yL
+
+
 def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None):
     """q/k/v (B, n, H, d) triplets; mask uint8 (B, n); input_mask uint8 (P, B); ``edge`` =
     optional (e, e_jac, e_lap) bias triplet with e (B, n, H, n)."""

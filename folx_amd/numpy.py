@@ -114,6 +114,17 @@ def det(A):
     return _call('det', (A,))
 
 
+def inv(A):
+    """``numpy.linalg.inv`` of a stack of matrices carrying derivatives."""
+    return _call('inv', (A,))
+
+
+def solve(A, b):
+    """``numpy.linalg.solve``: ``b`` of rank 1 is a vector, else a stack of matrices; either
+    operand may be a constant."""
+    return _call('solve', (A, b))
+
+
 def multi_head_self_attention(q, k, v, mask=None, input_mask=None, bias=None, **kwargs):
     """softmax(q k^T (+ bias)) v over per-walker arrays (n, H, d); no 1/sqrt(d) inside;
     ``bias`` is an optional edge-bias triplet (n, H, n).  Same registry keys as the

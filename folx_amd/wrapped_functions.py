@@ -766,18 +766,117 @@ def reduce_max_values(args, kwargs, sparsity_threshold):
 # --------------------------------------------------------------------------------------
 
 
+_SPARSE_SLOGDET_MAX_RANK = 64        # limits of folx_hip_sparse_slogdet_fwdlap
+_SPARSE_SLOGDET_MAX_FACTOR = 2048
+
+
+def _sparse_slogdet(A):
+    """Rank-one-factor shortcut for a sparse Jacobian (``sparse_slogdet``,
+    folx/slogdet.py:249-293): returns ``(sign, FwdLaplArray)`` or None when the planner
+    declines (dense Jacobian, mask differing between batch positions, dense contraction
+    cheaper) or the tables exceed what the kernel holds in LDS."""
+    jac = A.jacobian
+    if not jac.weak:
+        return None
+    k = jac.data.shape[0]
+    n = A.shape[-1]
+    plan = ia.slogdet_plan(jac.x0_idx, k, A.shape, jac.max_n)
+    if plan is None:
+        return None
+    tables, transposed = plan
+    C, rank, width = tables['take'].shape
+    if n > 32 or rank > _SPARSE_SLOGDET_MAX_RANK or rank * width > _SPARSE_SLOGDET_MAX_FACTOR:
+        return None
+    dev = A.x.device
+    take, cols, rows = ia.slogdet_kernel_tables(tables, transposed, k, n)
+    take, cols, rows = (so.device_table(t, dev) for t in (take, cols, rows))
+    sign, ld, ldj, ldl = K.sparse_slogdet(A.x.contiguous(), jac.data.contiguous(), A.laplacian.contiguous(),
+                                          take, cols, rows, transposed)
+    # a determinant depends on every coordinate its matrix is sparse in: dense output
+    # (folx/slogdet.py:238-246)
+    out_idx = np.broadcast_to(tables['coords'].reshape(C, *([1] * (ld.dim() - 1))), (C, *ld.shape[1:]))
+    dense = FwdJacobian(ldj, out_idx.astype(np.int32)).dense_array
+    return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(dense, None), ldl)
+
+
 def slogdet_wrapper(args, kwargs, sparsity_threshold):
-    """``slogdet_wrapper`` -> ``dense_slogdet`` (folx/slogdet.py:347-358, :320-344):
-    returns ``(sign, FwdLaplArray(logdet))`` with a dense Jacobian.  A sparse input
-    Jacobian is densified first (the reference's rank-one shortcut for sparse inputs,
-    folx/slogdet.py:251-293, is not implemented)."""
+    """``slogdet_wrapper`` (folx/slogdet.py:347-358): returns ``(sign, FwdLaplArray(logdet))``
+    with a dense Jacobian, through the rank-one-factor shortcut when the Jacobian's
+    sparsity pays (``sparse_slogdet``, :249-293), else ``dense_slogdet`` (:320-344)."""
     (A,) = args
     if not _is(A):
         raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
     assert A.shape[-1] == A.shape[-2], 'slogdet needs square matrices'
+    fast = _sparse_slogdet(A)
+    if fast is not None:
+        return fast
     J = A.jacobian.dense_array
     sign, ld, ldj, ldl = K.slogdet(A.x, J, A.laplacian)
     return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
+
+
+def inv_wrapper(args, kwargs, sparsity_threshold):
+    """Matrix inverse (``inv_wrapper``, folx/linear_solve.py:114-145); dense output."""
+    (A,) = args
+    if not _is(A):
+        raise NotImplementedError('inverse of a constant: call numpy.linalg.inv')
+    assert A.shape[-1] == A.shape[-2], 'inv needs square matrices'
+    C, CJ, CL = K.inv(A.x.contiguous(), A.jacobian.dense_array.contiguous(), A.laplacian.contiguous())
+    return FwdLaplArray(C, FwdJacobian(CJ, None), CL)
+
+
+def solve_wrapper(args, kwargs, sparsity_threshold):
+    """``y = A^-1 b`` (``solve_wrapper``, folx/linear_solve.py:54-111).  ``b`` of rank 1 is a
+    vector, anything else a stack of matrices; batch axes broadcast from the right and an
+    operand with fewer batch axes gets them inserted behind the Jacobian axis (``_align``,
+    :36-51).  Either operand may be constant; Jacobians are densified and zero-extended to
+    a common row count (:93-94)."""
+    A, b = args
+    like = A if _is(A) else b
+    if not _is(like):
+        raise NotImplementedError('solve of two constants: call numpy.linalg.solve')
+    B, dev = like.B, like.x.device
+
+    def parts(v):
+        if _is(v):
+            return v.x, v.jacobian.dense_array, v.laplacian
+        if isinstance(v, BatchedArray):
+            return v.data.to(torch.float32), None, None
+        if not isinstance(v, torch.Tensor):
+            v = np.asarray(v, dtype=np.float32)
+        return so.device_const(v, dev)[None], None, None
+
+    Ax, AJ, AL = parts(A)
+    bx, bJ, bL = parts(b)
+    vector = bx.dim() - 1 == 1
+    if vector:
+        bx = bx.unsqueeze(-1)
+        bJ = None if bJ is None else bJ.unsqueeze(-1)
+        bL = None if bL is None else bL.unsqueeze(-1)
+    nb = max(Ax.dim() - 3, bx.dim() - 3)
+
+    def lift(t, lead):
+        if t is None:
+            return None
+        missing = nb - (t.dim() - lead - 2)
+        return t.reshape(*t.shape[:lead], *([1] * missing), *t.shape[lead:])
+
+    Ax, AL, bx, bL = lift(Ax, 1), lift(AL, 1), lift(bx, 1), lift(bL, 1)
+    AJ, bJ = lift(AJ, 2), lift(bJ, 2)
+    n, m = bx.shape[-2:]
+    assert Ax.shape[-1] == n and Ax.shape[-2] == n, 'solve: shapes of A and b do not match'
+    batch = tuple(np.broadcast_shapes(tuple(Ax.shape[1:-2]), tuple(bx.shape[1:-2])))
+    if AJ is not None and bJ is not None:
+        P = max(AJ.shape[0], bJ.shape[0])
+        AJ, bJ = so.pad_rows(AJ, P), so.pad_rows(bJ, P)
+    P = (AJ if AJ is not None else bJ).shape[0]
+    full_A, full_b = (B, *batch, n, n), (B, *batch, n, m)
+    ex = lambda t, shape: None if t is None else t.expand(*shape).contiguous()
+    y, yJ, yL = K.solve(ex(Ax, full_A), ex(AJ, (P, *full_A)), ex(AL, full_A),
+                        ex(bx, full_b), ex(bJ, (P, *full_b)), ex(bL, full_b), P)
+    if vector:
+        y, yJ, yL = y.squeeze(-1), yJ.squeeze(-1), yL.squeeze(-1)
+    return FwdLaplArray(y, FwdJacobian(yJ, None), yL)
 
 
 def det_wrapper(args, kwargs, sparsity_threshold):
@@ -878,5 +977,7 @@ register_function('sign', sign_rule)
 register_function('reduce_max_values', reduce_max_values)
 register_function('slogdet', slogdet_wrapper)
 register_function('det', det_wrapper)
+register_function('inv', inv_wrapper)      # string keys, folx/wrapped_functions.py:559-560
+register_function('solve', solve_wrapper)
 register_function('_multi_head_self_attention', mhsa_forward_laplacian)
 register_function('_multi_head_self_edge_attention', mhsea_forward_laplacian)

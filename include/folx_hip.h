@@ -185,6 +185,52 @@ int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
                             float* ld_lap, int64_t NM, int32_t n, int32_t P);
 
 /*
+ * slogdet rule for a sparse Jacobian whose coordinates touch few rows, columns or entries
+ * of A, from static rank-one factor tables shared by all NM matrices.
+ *   A [NM][n][n]   A_jac [k][NM][n][n] (k stored rows)   A_lap [NM][n][n]
+ *   take  int32 [n_coords][rank][width]: address t * n * n + r * n + c of a factor entry in
+ *         (stored row t, matrix row r, column c) of A_jac, or -1 for an unused slot
+ *   cols  int32 [n_coords][rank][width]: the column the entry contracts with
+ *   rows  int32 [n_coords][rank]: the matrix row of every factor
+ *   sign [NM]   logdet [NM]   ld_jac [n_coords][NM] (row c belongs to the c-th coordinate of
+ *   the tables)   ld_lap [NM]
+ * W_c[s][t] = sum_l A_jac[take[c][s][l]] * Ainv[cols[c][s][l]][rows[c][t]];
+ * ld_jac[c] = tr W_c;  ld_lap = tr(Ainv A_lap) - sum_c sum_st W_c[s][t] W_c[t][s].
+ * transposed != 0: the tables were built for A^T (cols are rows of A and vice versa; take
+ * still addresses A_jac as stored) and Ainv is read transposed.
+ * Limits: n <= 32, rank <= 64, rank * width <= 2048 (else FOLX_HIP_ENOTSUP).
+ * Replaces _sparse_slogdet / _pack_slogdet (folx/slogdet.py:182-246); the tables are the
+ * ones of _factor_tables (folx/slogdet.py:142-179).
+ */
+int folx_hip_sparse_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
+                                   const float* A_lap, const int32_t* take, const int32_t* cols,
+                                   const int32_t* rows, float* sign, float* logdet, float* ld_jac,
+                                   float* ld_lap, int64_t NM, int32_t n, int32_t k,
+                                   int32_t n_coords, int32_t rank, int32_t width, int32_t transposed);
+
+/*
+ * Inverse rule for NM matrices of size n x n (n <= 32) with dense Jacobians.
+ *   A, A_lap, C, C_lap [NM][n][n]   A_jac, C_jac [P][NM][n][n]
+ * C = A^-1;  M_p = C A_jac[p];  C_jac[p] = -M_p C;  C_lap = (2 sum_p M_p M_p - C A_lap) C.
+ * Replaces inv_wrapper (folx/linear_solve.py:114-145).
+ */
+int folx_hip_inv_fwdlap(void* stream, const float* A, const float* A_jac, const float* A_lap,
+                        float* C, float* C_jac, float* C_lap, int64_t NM, int32_t n, int32_t P);
+
+/*
+ * Linear-solve rule y = A^-1 b for NM systems, n <= 32 unknowns, m <= 32 right-hand sides.
+ *   A [NM][n][n]   b, y [NM][n][m]   *_jac [P][NM][...]   *_lap like the values
+ * A_jac/A_lap or b_jac/b_lap may both be NULL for a constant operand (not both operands);
+ * a NULL Laplacian is what marks an operand as constant (with P = 0 no Jacobian is read).
+ *   A y_jac[p] = b_jac[p] - A_jac[p] y
+ *   A y_lap    = b_lap - A_lap y - 2 sum_p A_jac[p] y_jac[p]
+ * Replaces solve_wrapper (folx/linear_solve.py:54-111).
+ */
+int folx_hip_solve_fwdlap(void* stream, const float* A, const float* A_jac, const float* A_lap,
+                          const float* b, const float* b_jac, const float* b_lap, float* y,
+                          float* y_jac, float* y_lap, int64_t NM, int32_t n, int32_t m, int32_t P);
+
+/*
  * Multi-head self attention with Laplacian, o = softmax(q k^T) v (no 1/sqrt(d) inside).
  *   q, k, v, their lap and o, o_lap: [B][n][H][d];  *_jac, o_jac: [P][B][n][H][d]
  *   mask uint8 [B][n] (1 = real electron) or NULL; input_mask uint8 [P][B]

@@ -17,6 +17,11 @@ Pinning status (what fixes each function independently of its own formula):
   rules.binary rules         brute-force fp64 Hessian trace
   rules.slogdet_rule         numpy.linalg fp64 + brute-force Hessian trace (n <= 6),
                              diagonal / triangular closed forms, row-swap sign
+  rules.inv_rule, solve_rule brute-force fp64 Hessian trace through an adjugate/determinant
+                             inverse (cases of test/test_layers.py:443-499), closed forms
+  rules.sparse_slogdet_rule, index_algebra.slogdet_*
+                             path choices and table shape the reference's tests expect
+                             (test/test_layers.py:341-421) + equality with slogdet_rule
   rules.mhsa_rule            brute-force fp64 Hessian trace of softmax(q k^T) v composed
                              with random linear maps, incl. the padded-sequence masks of
                              test/experimental/pallas/test_attention.py:320-326

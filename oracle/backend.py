@@ -399,6 +399,61 @@ def slogdet(A: OArr):
     return OConst(sign), OArr(ld, J, L)
 
 
+def inv(A: OArr):
+    """Matrix inverse (folx/linear_solve.py:114-145)."""
+    return OArr(*rules.inv_rule(A.x, A.J, A.lap))
+
+
+def solve(A, b):
+    """``numpy.linalg.solve`` semantics per walker (folx/linear_solve.py:54-111): ``b`` of
+    logical rank 1 is a vector, anything else a stack of matrices; batch axes broadcast
+    from the right, the solution carries the broadcast batch shape.  Either operand may
+    be a constant."""
+    like = A if _is(A) else b
+    assert _is(like), 'solve of two constants is not a forward-Laplacian rule'
+    B = like.B
+
+    def parts(v, tail):
+        # -> x (B|1, *batch, *tail axes), J or None, lap or None, logical batch ndim
+        if _is(v):
+            return v.x, v.J, v.lap
+        c, _ = _const(v, like)
+        return c, None, None
+
+    Ax, AJ, AL = parts(A, 2)
+    bx, bJ, bL = parts(b, None)
+    vector = bx.ndim - 1 == 1
+    if vector:
+        bx = bx[..., None]
+        bJ = None if bJ is None else bJ[..., None]
+        bL = None if bL is None else bL[..., None]
+    nb = max(Ax.ndim - 3, bx.ndim - 3)  # logical batch axes of the solution
+
+    def lift(x, lead):
+        # insert missing batch axes right behind the leading ``lead`` axes
+        if x is None:
+            return None
+        missing = nb - (x.ndim - lead - 2)
+        return x.reshape(*x.shape[:lead], *([1] * missing), *x.shape[lead:])
+
+    Ax, AL, bx, bL = lift(Ax, 1), lift(AL, 1), lift(bx, 1), lift(bL, 1)
+    AJ, bJ = lift(AJ, 2), lift(bJ, 2)
+    batch = np.broadcast_shapes(Ax.shape[1:-2], bx.shape[1:-2])
+    n, m = bx.shape[-2:]
+    full_A, full_b = (B, *batch, n, n), (B, *batch, n, m)
+    if AJ is not None and bJ is not None and AJ.shape[0] != bJ.shape[0]:
+        P = max(AJ.shape[0], bJ.shape[0])
+        AJ = np.concatenate([AJ, np.zeros((P - AJ.shape[0], *AJ.shape[1:]), AJ.dtype)], 0)
+        bJ = np.concatenate([bJ, np.zeros((P - bJ.shape[0], *bJ.shape[1:]), bJ.dtype)], 0)
+    bc = lambda x, shape: None if x is None else np.broadcast_to(x, shape)
+    P = (AJ if AJ is not None else bJ).shape[0]
+    y, yJ, yL = rules.solve_rule(bc(Ax, full_A), bc(AJ, (P, *full_A)), bc(AL, full_A),
+                                 bc(bx, full_b), bc(bJ, (P, *full_b)), bc(bL, full_b))
+    if vector:
+        y, yJ, yL = y[..., 0], yJ[..., 0], yL[..., 0]
+    return OArr(y, yJ, yL)
+
+
 def multi_head_self_attention(q: OArr, k: OArr, v: OArr, mask=None, input_mask=None, bias=None):
     """``bias`` = optional edge-bias triplet of per-walker shape (n, H, n)."""
     if bias is None:

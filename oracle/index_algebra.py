@@ -258,3 +258,103 @@ def dot_projection(mask: np.ndarray, contract_axis: int, threshold: int):
     if proj.shape[0] > threshold:
         return None, True
     return proj[..., None], True
+
+
+# --------------------------------------------------------------------------------------
+# Sparse slogdet planner (folx/slogdet.py:73-293)
+# --------------------------------------------------------------------------------------
+
+SLOGDET_MAX_MASK_ENTRIES = 2**24  # folx/slogdet.py:73
+
+
+def slogdet_entry_mask(x0_idx, k: int, x_shape, transposed: bool):
+    """Per-entry coordinate mask ``(k, n, m)`` shared by all batch positions, or None
+    (folx/slogdet.py:94-125).  ``x_shape`` is the per-walker shape ``(..., n, m)`` of the
+    matrix array, ``k`` the number of stored Jacobian rows."""
+    if x0_idx is None:
+        return None
+    idx = np.asarray(x0_idx)
+    shape = tuple(x_shape)
+    if transposed:
+        if idx.ndim != len(shape) + 1:
+            return None
+        idx = np.swapaxes(idx, -1, -2)
+        shape = (*shape[:-2], shape[-1], shape[-2])
+    if k * int(np.prod(shape, dtype=np.int64)) > SLOGDET_MAX_MASK_ENTRIES:
+        return None
+    full = np.broadcast_to(idx, (k, *shape))
+    n, m = shape[-2:]
+    first = None
+    for pos in itertools.product(*[range(d) for d in shape[:-2]]):
+        cur = full[(slice(None), *pos)]
+        if first is None:
+            first = cur
+        elif not np.array_equal(first, cur):
+            return None
+    return np.ascontiguousarray(first).astype(np.int64).reshape(k, n, m)
+
+
+def slogdet_factor_tables(mask: np.ndarray, per_entry: bool):
+    """Rank-one factor tables of every ``dA/dx_c`` (folx/slogdet.py:142-179).
+
+    A factor is one touched row of ``dA/dx_c`` (or one touched entry with ``per_entry``).
+    Returns ``(cost, tables)`` with ``tables`` a dict: ``take (C, rank, width)`` flat
+    ``(tangent, row, column)`` addresses (``k n m`` = unused), ``cols (C, rank, width)``,
+    ``rows (C, rank)``, ``coords (C,)``, ``per_entry``; None when the tables are too large.
+    """
+    k, n, m = mask.shape
+    by_coord: dict[int, list] = {}
+    for t in range(k):
+        for r in range(n):
+            for c in range(m):
+                v = int(mask[t, r, c])
+                if v >= 0:
+                    by_coord.setdefault(v, []).append((r, c, t))
+    coords = sorted(by_coord)
+    factor_lists = []
+    for v in coords:
+        entries = sorted(by_coord[v])  # by row, column, then tangent
+        factors: dict[tuple, list] = {}
+        for r, c, t in entries:
+            key = (r, c) if per_entry else (r,)
+            factors.setdefault(key, []).append((r, c, t))
+        factor_lists.append([factors[key] for key in sorted(factors)])
+    rank = max(len(f) for f in factor_lists)
+    width = max(len(e) for f in factor_lists for e in f)
+    C = len(coords)
+    if C * rank * width > SLOGDET_MAX_MASK_ENTRIES:
+        return None
+    take = np.full((C, rank, width), k * n * m, dtype=np.int64)
+    cols = np.zeros((C, rank, width), dtype=np.int64)
+    rows = np.zeros((C, rank), dtype=np.int64)
+    for ci, facs in enumerate(factor_lists):
+        for s, ents in enumerate(facs):
+            rows[ci, s] = ents[0][0]
+            for l, (r, c, t) in enumerate(ents):
+                take[ci, s, l] = (t * n + r) * m + c
+                cols[ci, s, l] = c
+    cost = C * rank * rank * (1 if per_entry else width)
+    return cost, dict(take=take, cols=cols, rows=rows, coords=np.asarray(coords, dtype=np.int64),
+                      per_entry=per_entry)
+
+
+def slogdet_plan(x0_idx, k: int, x_shape, max_n: int):
+    """Choice among the four decompositions and the gate against the dense contraction
+    (folx/slogdet.py:249-293).  Returns ``(tables, transposed)`` or None."""
+    best = None
+    for transposed in (False, True):
+        mask = slogdet_entry_mask(x0_idx, k, x_shape, transposed)
+        if mask is None or not (mask >= 0).any():
+            continue
+        for per_entry in ((False,) if transposed else (False, True)):
+            plan = slogdet_factor_tables(mask, per_entry)
+            if plan is not None and (best is None or plan[0] < best[0]):
+                best = (plan[0], plan[1], transposed)
+    if best is None:
+        return None
+    cost, tables, transposed = best
+    n, m = x_shape[-2:]
+    tangents = max_n + 1
+    if 4 * cost > tangents * n * m * (n + 1) or cost > 2 * tangents * n * m:
+        return None
+    return tables, transposed

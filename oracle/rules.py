@@ -245,6 +245,88 @@ def slogdet_rule(A, J, lap):
     return sign.astype(A.dtype), (logdet.astype(A.dtype), jac, lap_out)
 
 
+def sparse_slogdet_rule(A, Jdata, lap, tables):
+    """Forward Laplacian of ``log|det A|`` from rank-one factors of ``dA/dx_c``
+    (folx/slogdet.py:182-246).  With ``dA/dx_c = sum_s e_{i_s} w_s^T`` (row factors
+    restricted to the entries the coordinate touches) and
+    ``W_c[s, t] = sum_l w_s[j_l] A^-1[j_l, i_t]``:
+
+        d_c log|det A| = tr W_c,   lap = tr(A^-1 lap_A) - sum_c sum_st W_c[s,t] W_c[t,s].
+
+    A, lap: (B, ..., n, n); Jdata: (k, B, ..., n, n) sparse rows; ``tables`` from
+    ``oracle.index_algebra.slogdet_factor_tables``.  Returns sign and
+    ``(logdet, jac (n_coords, B, ...), lap_out)``; the Jacobian rows belong to
+    ``tables['coords']``.
+    """
+    take, cols, rows, per_entry = tables['take'], tables['cols'], tables['rows'], tables['per_entry']
+    k = Jdata.shape[0]
+    n, m = A.shape[-2:]
+    batch = A.shape[:-2]
+    sign, logdet = np.linalg.slogdet(A)
+    Ainv = np.linalg.inv(A)
+    C, R, Wd = take.shape
+    Jb = np.broadcast_to(Jdata, (k, *A.shape))
+    W = np.zeros((*batch, C, R, R), dtype=A.dtype)
+    for c in range(C):
+        for s in range(R):
+            for t in range(R):
+                acc = np.zeros(batch, dtype=A.dtype)
+                if per_entry:
+                    tot = np.zeros(batch, dtype=A.dtype)
+                    for l in range(Wd):
+                        pos = take[c, s, l]
+                        if pos < k * n * m:
+                            tt, rem = divmod(int(pos), n * m)
+                            tot = tot + Jb[tt][..., rem // m, rem % m]
+                    acc = tot * Ainv[..., cols[c, s, 0], rows[c, t]]
+                else:
+                    for l in range(Wd):
+                        pos = take[c, s, l]
+                        if pos < k * n * m:
+                            tt, rem = divmod(int(pos), n * m)
+                            acc = acc + Jb[tt][..., rem // m, rem % m] * Ainv[..., cols[c, s, l], rows[c, t]]
+                W[..., c, s, t] = acc
+    jac = np.moveaxis(np.einsum('...css->...c', W), -1, 0)
+    lap_out = np.einsum('...ji,...ij->...', Ainv, lap) - np.einsum('...cst,...cts->...', W, W)
+    return sign.astype(A.dtype), (logdet.astype(A.dtype), jac, lap_out)
+
+
+def inv_rule(A, J, lap):
+    """Forward Laplacian of ``C = A^-1`` (folx/linear_solve.py:114-145): with
+    ``M_c = C dA/dx_c``,  ``d_c C = -M_c C``  and
+    ``lap C = (2 sum_c M_c M_c - C lap_A) C``.
+    A, lap: (B, ..., n, n); J: (P, B, ..., n, n)."""
+    C = np.linalg.inv(A)
+    M = np.einsum('...il,p...lj->p...ij', C, J)
+    jac = -np.einsum('p...il,...lj->p...ij', M, C)
+    inner = 2.0 * np.einsum('p...il,p...lj->...ij', M, M) - np.einsum('...il,...lj->...ij', C, lap)
+    return C, jac, np.einsum('...il,...lj->...ij', inner, C)
+
+
+def solve_rule(A, AJ, AL, b, bJ, bL):
+    """Forward Laplacian of ``y = A^-1 b`` (folx/linear_solve.py:54-111):
+
+        A d_c y = d_c b - d_c A y,     A lap_y = lap_b - lap_A y - 2 sum_c d_c A d_c y.
+
+    A: (B, ..., n, n), b: (B, ..., n, m); either Jacobian/Laplacian pair may be None
+    (constant operand) but not both.  Jacobians: (P, B, ..., n, *)."""
+    assert AJ is not None or bJ is not None
+    y = np.linalg.solve(A, b)
+    P = (AJ if AJ is not None else bJ).shape[0]
+    rhsJ = np.zeros((P, *y.shape), dtype=y.dtype)
+    rhsL = np.zeros_like(y)
+    if bJ is not None:
+        rhsJ = rhsJ + bJ
+        rhsL = rhsL + bL
+    if AJ is not None:
+        rhsJ = rhsJ - np.einsum('p...il,...lm->p...im', AJ, y)
+        rhsL = rhsL - np.einsum('...il,...lm->...im', AL, y)
+    yJ = np.linalg.solve(np.broadcast_to(A, (P, *A.shape)), rhsJ)
+    if AJ is not None:
+        rhsL = rhsL - 2.0 * np.einsum('p...il,p...lm->...im', AJ, yJ)
+    return y, yJ, np.linalg.solve(A, rhsL)
+
+
 # --------------------------------------------------------------------------------------
 # Multi-head self attention
 # --------------------------------------------------------------------------------------

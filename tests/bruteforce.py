@@ -155,6 +155,30 @@ class plain:
         return out
 
     @staticmethod
+    def inv(A):
+        # adjugate / determinant by cofactor expansion: pure arithmetic under any AD mode
+        n = A.shape[-1]
+        if n == 1:
+            return 1.0 / A
+        rows = []
+        for i in range(n):
+            cols = []
+            for j in range(n):
+                # entry (i, j) of the inverse = cofactor (j, i) / det
+                minor = torch.cat([A[..., :j, :], A[..., j + 1:, :]], dim=-2)
+                minor = torch.cat([minor[..., :, :i], minor[..., :, i + 1:]], dim=-1)
+                cols.append(((-1) ** (i + j)) * plain.det(minor))
+            rows.append(torch.stack(cols, dim=-1))
+        return torch.stack(rows, dim=-2) / plain.det(A)[..., None, None]
+
+    @staticmethod
+    def solve(A, b):
+        A, b = plain._b(A, b)
+        if b.ndim == 1:
+            return (plain.inv(A) @ b[..., None])[..., 0]
+        return plain.inv(A) @ b
+
+    @staticmethod
     def sign(a):
         return torch.sign(a.detach())
 

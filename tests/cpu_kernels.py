@@ -101,6 +101,31 @@ def slogdet(A, AJ, AL):
     return _t(sign), _t(ld), _t(jac), _t(lap)
 
 
+def sparse_slogdet(A, AJ, AL, take, cols, rows, transposed):
+    take, cols, rows = (t.cpu().numpy().astype(np.int64) for t in (take, cols, rows))
+    a, aj, al = _n(A), _n(AJ), _n(AL)
+    k, n = aj.shape[0], a.shape[-1]
+    if transposed:
+        # the tables describe A^T and address A_jac as stored: run the oracle on A^T
+        t, rem = np.divmod(np.where(take >= 0, take, 0), n * n)
+        r, c = np.divmod(rem, n)
+        take = np.where(take >= 0, (t * n + c) * n + r, -1)
+        a, aj, al = (np.swapaxes(v, -1, -2) for v in (a, aj, al))
+    take = np.where(take >= 0, take, k * n * n)
+    sign, (ld, jac, lap) = rules.sparse_slogdet_rule(
+        a, aj, al, dict(take=take, cols=cols, rows=rows, per_entry=False))
+    return _t(sign), _t(ld), _t(jac), _t(lap)
+
+
+def inv(A, AJ, AL):
+    return tuple(_t(v) for v in rules.inv_rule(_n(A), _n(AJ), _n(AL)))
+
+
+def solve(A, AJ, AL, b, bJ, bL, P):
+    opt = lambda v: None if v is None else _n(v)
+    return tuple(_t(v) for v in rules.solve_rule(_n(A), opt(AJ), opt(AL), _n(b), opt(bJ), opt(bL)))
+
+
 def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None):
     m = None if mask is None else mask.cpu().numpy().astype(bool)
     im = None if input_mask is None else input_mask.cpu().numpy().astype(bool)
@@ -113,6 +138,6 @@ def install(monkeypatch):
     import folx_amd.kernels as K
 
     for name in ('dense', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
-                 'gather_rows', 'scatter_add_rows', 'slogdet', 'mhsa'):
+                 'gather_rows', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))
