@@ -28,6 +28,7 @@ SIGNATURES = {
     'folx_hip_reduce_sum': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_float]),
     'folx_hip_reduce_max': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64]),
     'folx_hip_gather_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64]),
+    'folx_hip_gather_cols': (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int32, c_int64]),
     'folx_hip_scatter_add_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int64, c_int64, c_int64]),
     'folx_hip_slogdet_fwdlap': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int32, c_int32]),
     'folx_hip_sparse_slogdet_fwdlap': (c_int, [_P] * 11 + [c_int64] + [c_int32] * 6),
@@ -42,7 +43,7 @@ ACT = {
     'logistic': 7, 'sigmoid': 7, 'softplus': 8, 'sin': 9, 'cos': 10, 'abs': 11,
     'log1p': 12, 'reciprocal': 13, 'expm1': 14, 'integer_pow': 15,
 }
-BINOP = {'mul': 0, 'div': 1, 'add': 2, 'sub': 3}
+BINOP = {'mul': 0, 'div': 1, 'add': 2, 'sub': 3, 'min': 4, 'max': 5}
 
 _lib = None
 

@@ -63,6 +63,33 @@ __global__ __launch_bounds__(256) void scatter_add_rows_kernel(const float* __re
     atomicAdd(&out[((int64_t)t * B + b) * S + e], data[((int64_t)r * B + b) * S + e]);
 }
 
+// Static gather along the position axis with a sum over slots (the transposed form of a
+// scatter with static indices: every output position lists the inputs that land on it):
+//   out[rb][po][si] = sum_s data[rb][table[po][s]][si]        (table < 0: no source)
+// Threads run along (po, si); blockIdx.y strides over the rb = (triplet row, walker) axis.
+__global__ __launch_bounds__(256) void gather_cols_kernel(const float* __restrict__ data,
+                                                          const int32_t* __restrict__ table,
+                                                          float* __restrict__ out, int64_t RB,
+                                                          int64_t S_in, int64_t S_out_outer,
+                                                          int32_t n_slots, int64_t S_inner) {
+  const int64_t S_out = S_out_outer * S_inner;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= S_out) return;
+  const int64_t po = e / S_inner, si = e % S_inner;
+  int32_t src[4];
+  const int32_t ns = n_slots < 4 ? n_slots : 4;
+  for (int s = 0; s < ns; ++s) src[s] = table[po * n_slots + s];
+  for (int64_t rb = blockIdx.y; rb < RB; rb += gridDim.y) {
+    const float* row = data + rb * S_in;
+    float acc = 0.0f;
+    for (int s = 0; s < n_slots; ++s) {
+      const int32_t t = s < 4 ? src[s] : table[po * n_slots + s];
+      if (t >= 0) acc += row[(int64_t)t * S_inner + si];
+    }
+    out[rb * S_out + e] = acc;
+  }
+}
+
 }  // namespace
 
 extern "C" int folx_hip_gather_rows(void* stream, const float* data, const int32_t* take, float* out,
@@ -99,5 +126,20 @@ extern "C" int folx_hip_scatter_add_rows(void* stream, const float* data, const 
   const unsigned gy = (unsigned)(B < 4096 ? B : 4096);
   scatter_add_rows_kernel<<<dim3((unsigned)blocks, gy, (unsigned)k_in), dim3(256), 0, (hipStream_t)stream>>>(
       data, idx, out, B, S_outer, S_inner);
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_gather_cols(void* stream, const float* data, const int32_t* table, float* out,
+                                    int64_t RB, int64_t S_in_outer, int64_t S_out_outer, int32_t n_slots,
+                                    int64_t S_inner) {
+  if (RB < 0 || S_in_outer < 0 || S_out_outer < 0 || n_slots < 0 || S_inner < 0) return FOLX_HIP_EINVAL;
+  const int64_t S_out = S_out_outer * S_inner;
+  if (RB == 0 || S_out == 0) return FOLX_HIP_OK;
+  if (!out || (n_slots > 0 && (!table || (S_in_outer > 0 && !data)))) return FOLX_HIP_EINVAL;
+  const int64_t blocks = (S_out + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  const unsigned gy = (unsigned)(RB < 4096 ? RB : 4096);
+  gather_cols_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
+      data, table, out, RB, S_in_outer * S_inner, S_out_outer, n_slots, S_inner);
   return folx_launch_status();
 }

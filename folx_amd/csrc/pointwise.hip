@@ -1,5 +1,5 @@
 // Broadcasting elementwise rules on a shared Jacobian row frame: the binary rule
-// (mul / div / add / sub of two triplets) and the affine map against constants.
+// (mul / div / add / sub / min / max of two triplets) and the affine map against constants.
 // Both are single streaming passes bound by HBM bandwidth.
 #include "common.h"
 
@@ -32,7 +32,9 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
     if constexpr (OP == FOLX_BIN_MUL) { ca = bv; cb = av; }
     else if constexpr (OP == FOLX_BIN_DIV) { ca = 1.0f / bv; cb = -av * ca * ca; }
     else if constexpr (OP == FOLX_BIN_ADD) { ca = 1.0f; cb = 1.0f; }
-    else { ca = 1.0f; cb = -1.0f; }
+    else if constexpr (OP == FOLX_BIN_SUB) { ca = 1.0f; cb = -1.0f; }
+    else if constexpr (OP == FOLX_BIN_MIN) { ca = av < bv ? 1.0f : (av == bv ? 0.5f : 0.0f); cb = 1.0f - ca; }
+    else { ca = av > bv ? 1.0f : (av == bv ? 0.5f : 0.0f); cb = 1.0f - ca; }
     for (int p = w; p < P; p += PSPLIT) {
       const float ja = aj[(int64_t)p * a_S + oa];
       const float jb = bj[(int64_t)p * b_S + ob];
@@ -61,8 +63,12 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
       l += -2.0f * rb * rb * s + 2.0f * av * rb * rb * rb * t;
     } else if constexpr (OP == FOLX_BIN_ADD) {
       y[i] = av + bv;
-    } else {
+    } else if constexpr (OP == FOLX_BIN_SUB) {
       y[i] = av - bv;
+    } else if constexpr (OP == FOLX_BIN_MIN) {
+      y[i] = fminf(av, bv);
+    } else {
+      y[i] = fmaxf(av, bv);
     }
     yl[i] = l;
   }
@@ -115,6 +121,7 @@ extern "C" int folx_hip_binary_fwdlap(void* stream, int32_t op, const float* a, 
     break;
   switch (op) {
     FOLX_CASE(FOLX_BIN_MUL) FOLX_CASE(FOLX_BIN_DIV) FOLX_CASE(FOLX_BIN_ADD) FOLX_CASE(FOLX_BIN_SUB)
+    FOLX_CASE(FOLX_BIN_MIN) FOLX_CASE(FOLX_BIN_MAX)
   }
 #undef FOLX_CASE
   return folx_launch_status();

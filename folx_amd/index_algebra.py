@@ -93,6 +93,8 @@ def get_index_mask(mask: np.ndarray, outputs: np.ndarray) -> np.ndarray:
     ``-1``; first match wins (folx/api.py:120-159)."""
     s = np.broadcast_shapes(mask.shape[1:], outputs.shape[1:])
     m = np.broadcast_to(mask, (mask.shape[0], *s))
+    if outputs.shape[0] == 0:
+        return np.full(m.shape, -1, dtype=INT)
     o = np.broadcast_to(outputs, (outputs.shape[0], *s))
     match = m[:, None] == o[None]  # (k, T, *s)
     idx = match.argmax(1)
@@ -351,3 +353,100 @@ def slogdet_kernel_tables(tables, transposed: bool, k: int, n: int):
     addr = (t * n + c) * n + r if transposed else (t * n + r) * n + c
     take32 = np.where(valid, addr, -1).astype(np.int32)
     return take32, tables['cols'].astype(np.int32), tables['rows'].astype(np.int32)
+
+
+# --------------------------------------------------------------------------------------
+# static positions of indexed reads and scatters (folx/jvp.py:416-471, :536-609)
+# --------------------------------------------------------------------------------------
+
+
+def index_positions(shape, idx) -> np.ndarray:
+    """Flat position in an array of ``shape`` that every element of ``array[idx]`` refers
+    to, for a static numpy index (ints, slices, ``None``, ``Ellipsis``, integer arrays).
+    Integer-array entries outside ``[-size, size)`` give ``-1`` (a scatter drops those
+    updates, folx/jvp.py:434-435); negative ones count from the end."""
+    shape = tuple(int(d) for d in shape)
+    idx = idx if isinstance(idx, tuple) else (idx,)
+    n_named = sum(1 for i in idx if i is not None and i is not Ellipsis)
+    assert n_named <= len(shape), 'too many indices'
+    # walk the index to find the axis every integer array applies to
+    axis, padded_axes, new_idx = 0, [], []
+    for i in idx:
+        if i is None:
+            new_idx.append(None)
+        elif i is Ellipsis:
+            axis += len(shape) - n_named
+            new_idx.append(Ellipsis)
+        elif isinstance(i, (slice, int, np.integer)):
+            new_idx.append(i)
+            axis += 1
+        else:
+            arr = np.asarray(i)
+            assert arr.dtype.kind in 'iu', 'only integer index arrays are static positions'
+            size = shape[axis]
+            arr = np.where(arr < 0, arr + size, arr)
+            # out-of-range entries point at an extra slot that holds -1
+            new_idx.append(np.where((arr < 0) | (arr >= size), size, arr))
+            padded_axes.append(axis)
+            axis += 1
+    pos = np.arange(int(np.prod(shape, dtype=np.int64)), dtype=INT).reshape(shape)
+    for ax in padded_axes:
+        pad = [(0, 0)] * len(shape)
+        pad[ax] = (0, 1)
+        pos = np.pad(pos, pad, constant_values=-1)
+    return np.asarray(pos[tuple(new_idx)])
+
+
+def scatter_source_table(tpos: np.ndarray, op_size: int, last_only: bool) -> np.ndarray:
+    """For every operand position the update elements that land on it, ascending, ``-1``
+    padded: ``(op_size, n_slots)`` int32 (at least one slot).  ``last_only`` keeps the last
+    element only (a 'set' is decided by the final write)."""
+    t = np.asarray(tpos).reshape(-1)
+    e = np.flatnonzero(t >= 0)
+    p = t[e]
+    order = np.argsort(p, kind='stable')
+    p, e = p[order], e[order]
+    slot = np.arange(p.size) - np.searchsorted(p, p, side='left')
+    if last_only and p.size:
+        count = np.bincount(p, minlength=op_size)
+        keep = slot == count[p] - 1
+        p, e, slot = p[keep], e[keep], np.zeros(int(keep.sum()), dtype=INT)
+    n_slots = int(slot.max()) + 1 if p.size else 1
+    table = np.full((op_size, n_slots), -1, dtype=np.int32)
+    table[p, slot] = e
+    return table
+
+
+def scatter_out_mask(op_mask, upd_mask, tpos: np.ndarray, op_shape, is_set: bool) -> np.ndarray:
+    """Mask of a scatter's output (folx/jvp.py:536-609): per operand position the ascending
+    union of the operand's dependencies (none where a 'set' overwrites the position) and of
+    those of the update elements landing there, ``-1`` padded at the end; at least one row."""
+    op_shape = tuple(int(d) for d in op_shape)
+    op_size = int(np.prod(op_shape, dtype=np.int64))
+    tflat = np.asarray(tpos).reshape(-1)
+    pos_parts, dep_parts = [], []
+    if upd_mask is not None:
+        um = np.broadcast_to(upd_mask, (upd_mask.shape[0], *np.shape(tpos))).reshape(upd_mask.shape[0], -1)
+        tp = np.broadcast_to(tflat, um.shape)
+        sel = (um >= 0) & (tp >= 0)
+        pos_parts.append(tp[sel]), dep_parts.append(um[sel])
+    if op_mask is not None:
+        om = np.broadcast_to(op_mask, (op_mask.shape[0], *op_shape)).reshape(op_mask.shape[0], -1)
+        keep = om >= 0
+        if is_set:
+            hit = np.zeros(op_size, dtype=bool)
+            hit[tflat[tflat >= 0]] = True
+            keep = keep & ~hit
+        pp = np.broadcast_to(np.arange(op_size), om.shape)
+        pos_parts.append(pp[keep]), dep_parts.append(om[keep])
+    pos = np.concatenate(pos_parts).astype(INT) if pos_parts else np.zeros(0, INT)
+    dep = np.concatenate(dep_parts).astype(INT) if dep_parts else np.zeros(0, INT)
+    if pos.size == 0:
+        return np.full((1, *op_shape), -1, dtype=np.int32)
+    span = int(dep.max()) + 1
+    keys = np.unique(pos * span + dep)   # sorted by position, then dependency
+    kp, kd = keys // span, keys % span
+    slot = np.arange(kp.size) - np.searchsorted(kp, kp, side='left')
+    out = np.full((int(slot.max()) + 1, op_size), -1, dtype=np.int32)
+    out[slot, kp] = kd
+    return out.reshape(out.shape[0], *op_shape)

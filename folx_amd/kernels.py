@@ -268,6 +268,24 @@ def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
     return out
 
 
+def gather_cols(data, table, S_inner=1):
+    """out[rb, po, si] = sum_s data[rb, table[po, s], si]: ``data`` (RB, S_in_outer * S_inner),
+    ``table`` int32 (S_out_outer, n_slots) on the device -> (RB, S_out_outer * S_inner)."""
+    _chk(data, table)
+    RB = data.shape[0]
+    S_in_outer = data.shape[1] // S_inner
+    S_out_outer, n_slots = table.shape
+    out = torch.empty((RB, S_out_outer * S_inner), device=data.device, dtype=torch.float32)
+    with _timed('gather_cols', (RB, S_in_outer, S_out_outer, n_slots, S_inner)):
+        check(
+            _lib.load().folx_hip_gather_cols(
+                _stream(), _p(data), _p(table), _p(out), RB, S_in_outer, S_out_outer, n_slots, S_inner
+            ),
+            'gather_cols',
+        )
+    return out
+
+
 def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
     _chk(data, idx)
     k_in = data.shape[0]

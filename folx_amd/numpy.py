@@ -114,6 +114,24 @@ def det(A):
     return _call('det', (A,))
 
 
+def minimum(a, b):
+    return _call('min', (a, b))
+
+
+def maximum(a, b):
+    return _call('max', (a, b))
+
+
+_SCATTER_KEYS = {'set': 'scatter', 'add': 'scatter-add', 'min': 'scatter_min', 'max': 'scatter_max'}
+
+
+def scatter(operand, idx, updates, mode='set'):
+    """``operand.at[idx].set / add / min / max(updates)`` (the ``mode``) for a static numpy
+    index; either argument may be a constant.  Out-of-range integer indices drop their
+    update."""
+    return _call(_SCATTER_KEYS[mode], (operand, updates), {'idx': idx})
+
+
 def inv(A):
     """``numpy.linalg.inv`` of a stack of matrices carrying derivatives."""
     return _call('inv', (A,))

@@ -257,7 +257,36 @@ def _binary_const(op: str, t: FwdLaplArray, c, t_is_left: bool) -> FwdLaplArray:
             return _affine_const(t, rc, mul=True, alpha=1.0, beta=0.0)
         r = _LAPLACE_FN_REGISTRY['reciprocal']((t,), {}, 0)
         return _affine_const(r, c, mul=True, alpha=1.0, beta=0.0)
+    if op in ('min', 'max'):
+        return _minmax_const(op, t, c)
     raise ValueError(op)
+
+
+def _selection_weights(op: str, ax: torch.Tensor, bx: torch.Tensor):
+    """``min`` / ``max`` of two value arrays and the weight of the first operand in the
+    result's derivatives (1 where it is selected, 1/2 at a tie, else 0): the binary kernel
+    applied to a Jacobian row of ones against a row of zeros."""
+    shape = torch.broadcast_shapes(ax.shape, bx.shape)
+    one = torch.empty((1, *ax.shape), device=ax.device, dtype=torch.float32).fill_(1.0)
+    zero = so.zeros((1, *bx.shape), ax.device)
+    y, w, _ = K.binary(op, ax.contiguous(), one, ax.contiguous(), bx.contiguous(), zero, bx.contiguous())
+    return y, w.reshape(shape)
+
+
+def _minmax_const(op: str, t: FwdLaplArray, c) -> FwdLaplArray:
+    """``min`` / ``max`` against a constant: where the constant wins the derivatives vanish;
+    the mask is unchanged."""
+    cshape = _logical_shape(c)
+    nd = max(t.ndim, len(cshape))
+    t = _pad_logical(t, nd)
+    out_shape = tuple(np.broadcast_shapes(t.shape, cshape))
+    B, k, dev = t.B, t.jacobian.data.shape[0], t.x.device
+    ct = _const_tensor(c, nd, dev)
+    full = (B, *out_shape)
+    y, w = _selection_weights(op, t.x, ct)
+    J = K.rows_affine(t.jacobian.data, k, (B, *t.shape), full, w, None, 1.0, 0.0).reshape(k, *full)
+    lap = K.rows_affine(t.laplacian, 1, (B, *t.shape), full, w, None, 1.0, 0.0).reshape(full)
+    return FwdLaplArray(y.reshape(full), FwdJacobian(J, _bmask(t.jacobian.x0_idx, k, out_shape)), lap)
 
 
 def _expand_rows(J: torch.Tensor, k: int, src_shape, full) -> torch.Tensor:
@@ -302,6 +331,13 @@ def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLapl
         sa, sb = 1.0, (1.0 if op == 'add' else -1.0)
     elif op == 'mul':
         ca, cb, sa, sb = b.x, a.x, 1.0, 1.0
+    elif op in ('min', 'max'):
+        # the selected operand's rows pass through (LINEAR, folx/wrapped_functions.py:508-513)
+        y, ca = _selection_weights(op, a.x, b.x)
+        cb = K.rows_affine(ca, 1, tuple(ca.shape), tuple(ca.shape), None,
+                           so.device_const(np.ones((1,) * ca.dim(), dtype=np.float32), ca.device),
+                           -1.0, 1.0).reshape(ca.shape)
+        sa = sb = 1.0
     else:  # div: d/da = 1/b, d/db = -a/b^2
         rb = _values_unary('reciprocal', b.x)
         q = _values_binary('mul', a.x, rb)
@@ -328,6 +364,9 @@ def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLapl
         lap = K.rows_affine(a.laplacian, 1, (B, *a.shape), full, None,
                             _expand_rows(b.laplacian, 1, (B, *b.shape), full).reshape(full), 1.0, sb).reshape(full)
         return FwdLaplArray(y, FwdJacobian(J_out, res_mask), lap)
+    if op in ('min', 'max'):
+        _, _, lap = K.binary(op, a.x, _empty_jac(a.x), a.laplacian, b.x, _empty_jac(b.x), b.laplacian)
+        return FwdLaplArray(y.reshape(full), FwdJacobian(J_out, res_mask), lap.reshape(full))
 
     # Hessian term on the static index frame (folx/hessian.py:288-340, :379-428):
     # intersection for mul (LINEAR_IN_ONE), union for div; dense when the frame says so.
@@ -349,7 +388,8 @@ def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLapl
     return FwdLaplArray(y, FwdJacobian(J_out, res_mask), lap)
 
 
-_NP_BINARY = {'add': np.add, 'sub': np.subtract, 'mul': np.multiply, 'div': np.divide}
+_NP_BINARY = {'add': np.add, 'sub': np.subtract, 'mul': np.multiply, 'div': np.divide,
+              'min': np.minimum, 'max': np.maximum}
 
 
 def _binary_rule(op: str) -> ForwardLaplacian:
@@ -664,14 +704,211 @@ def _canon_index(idx, nd):
     return idx
 
 
+def _has_index_arrays(idx) -> bool:
+    idx = idx if isinstance(idx, tuple) else (idx,)
+    return any(isinstance(i, (np.ndarray, list, torch.Tensor)) for i in idx)
+
+
+def _take_positions(a, idx):
+    """Indexing with static integer arrays (the ``gather`` primitive under
+    ``sparse_index_jvp``, folx/jvp.py:330-413): every output element reads one static
+    position, so values, Jacobian rows, Laplacian and mask are all re-indexed alike."""
+    shape = _logical_shape(a)
+    idx = tuple(np.asarray(i.cpu() if isinstance(i, torch.Tensor) else i) if isinstance(i, (list, torch.Tensor))
+                else i for i in (idx if isinstance(idx, tuple) else (idx,)))
+    pos = ia.index_positions(shape, idx)
+    if (pos < 0).any():
+        raise IndexError('index out of bounds in a static integer-array index')
+    if not _is(a):
+        if isinstance(a, BatchedArray):
+            flat = a.data.reshape(a.B, -1)
+            t = so.device_table(pos.reshape(-1, 1), flat.device)
+            return BatchedArray(K.gather_cols(flat.contiguous(), t).reshape(a.B, *pos.shape))
+        return np.asarray(a).reshape(-1)[pos]
+    B, dev = a.B, a.x.device
+    k = a.jacobian.data.shape[0]
+    S = int(np.prod(shape, dtype=np.int64))
+    t = so.device_table(pos.reshape(-1, 1), dev)
+    x = K.gather_cols(a.x.reshape(B, S), t).reshape(B, *pos.shape)
+    J = K.gather_cols(a.jacobian.data.reshape(k * B, S), t).reshape(k, B, *pos.shape)
+    L = K.gather_cols(a.laplacian.reshape(B, S), t).reshape(B, *pos.shape)
+    mask = a.jacobian.x0_idx
+    if mask is not None:
+        mask = np.broadcast_to(mask, (mask.shape[0], *shape)).reshape(mask.shape[0], S)[:, pos]
+    return FwdLaplArray(x, FwdJacobian(J, mask), L)
+
+
 def getitem_rule(args, kwargs, sparsity_threshold):
-    """Static basic indexing (``slice`` / ``squeeze`` / ``expand_dims`` primitives)."""
+    """Static indexing: basic (``slice`` / ``squeeze`` / ``expand_dims`` primitives) on
+    views, integer arrays (``gather``) through the position-gather kernel."""
     (a,) = args
+    if _has_index_arrays(kwargs['idx']):
+        return _take_positions(a, kwargs['idx'])
     idx = _canon_index(kwargs['idx'], len(_logical_shape(a)))
     fn_t = lambda t, lead: t[(*([slice(None)] * lead), *idx)]
     if not _is(a):
         return _const_index(a, fn_t)
     return _index_rule(fn_t, lambda m: m[(slice(None), *idx)])(a)
+
+
+# --------------------------------------------------------------------------------------
+# scatter rules (folx/jvp.py:416-673)
+# --------------------------------------------------------------------------------------
+
+_SCATTER_BIG = 3.0e38  # stands in for +-inf at positions no update lands on (min / max)
+
+
+def _scatter_rows(mode: str, op, upd, tpos: np.ndarray, op_size: int, dev):
+    """The scatter arithmetic on row stacks that share one row frame.
+
+    op = (x (B, S_op), J (P, B, S_op), lap (B, S_op)) with J possibly None (constant
+    operand), upd likewise over the update elements (J None = constant updates).  Every
+    operand position gathers the update elements that land on it through a static table
+    (``folx_hip_gather_cols``), so the result does not depend on any write order."""
+    ox, oJ, oL = op
+    ux, uJ, uL = upd
+    B = ox.shape[0]
+    withJ = [J for J in (oJ, uJ) if J is not None]
+    P = withJ[0].shape[0] if withJ else 0
+
+    def gather(table):
+        t = so.device_table(table, dev)
+        gx = K.gather_cols(ux.contiguous(), t)
+        if uJ is None:
+            return gx, None, None
+        gJ = K.gather_cols(uJ.reshape(P * B, -1), t).reshape(P, B, op_size)
+        return gx, gJ, K.gather_cols(uL.contiguous(), t)
+
+    def plus(a, b):
+        if a is None or b is None:
+            return a if b is None else b
+        return so.add_rowstacks(a.contiguous(), b.contiguous())
+
+    if mode == 'add':
+        gx, gJ, gL = gather(ia.scatter_source_table(tpos, op_size, last_only=False))
+        return plus(ox, gx), plus(oJ, gJ), plus(oL, gL)
+
+    if mode == 'set':
+        table = ia.scatter_source_table(tpos, op_size, last_only=True)
+        gx, gJ, gL = gather(table)
+        keep = so.device_const((table[:, 0] < 0).astype(np.float32).reshape(1, op_size), dev)
+        x = K.rows_affine(ox.contiguous(), 1, (B, op_size), (B, op_size), keep, gx, 1.0, 1.0).reshape(B, op_size)
+        if oJ is None:
+            return x, gJ, gL
+        J = K.rows_affine(oJ.contiguous(), P, (B, op_size), (B, op_size), keep, None, 1.0, 0.0)
+        L = K.rows_affine(oL.contiguous(), 1, (B, op_size), (B, op_size), keep, None, 1.0, 0.0).reshape(B, op_size)
+        return x, plus(J.reshape(P, B, op_size), gJ), plus(L, gL)
+
+    # min / max: fold the update elements in, one table slot at a time; a position without
+    # an element in the slot sees +-BIG there, so the running value wins
+    table = ia.scatter_source_table(tpos, op_size, last_only=False)
+    op_name = 'min' if mode == 'min' else 'max'
+    big = _SCATTER_BIG if mode == 'min' else -_SCATTER_BIG
+    zJ = lambda: so.zeros((P, B, op_size), dev)
+    cx, cJ, cL = ox.contiguous(), (oJ if oJ is not None else zJ()), (oL if oL is not None else so.zeros((B, op_size), dev))
+    for s_ in range(table.shape[1]):
+        col = table[:, s_ : s_ + 1]
+        gx, gJ, gL = gather(col)
+        valid = (col[:, 0] >= 0).astype(np.float32).reshape(1, op_size)
+        fill = so.device_const((1.0 - valid) * big, dev)
+        gx = K.rows_affine(gx, 1, (B, op_size), (B, op_size), so.device_const(valid, dev), fill, 1.0, 1.0)
+        gx = gx.reshape(B, op_size)
+        if gJ is None:
+            gJ, gL = zJ(), so.zeros((B, op_size), dev)
+        cx, cJ, cL = K.binary(op_name, cx, cJ.contiguous(), cL.contiguous(), gx, gJ, gL)
+    return cx, cJ, cL
+
+
+def _scatter_rule(mode: str) -> ForwardLaplacian:
+    """``operand.at[idx].set / add / min / max(updates)`` with a static index
+    (``sparse_scatter_jvp``, folx/jvp.py:474-673).  args = (operand, updates), kwargs
+    ``idx``.  The target position of every update element is computed on the host
+    (``index_positions``; out-of-range integer indices drop their update, :434-435).
+
+    Sparse Jacobians: the output mask is the per-position union of the operand's
+    dependencies (none where a 'set' overwrites, :549-553) and of the updates landing there
+    (:536-567); both arguments are re-indexed to that frame (:640-655) and scattered row by
+    row.  Past the threshold the rule densifies before or after the scatter, whichever
+    moves fewer elements (:582-598).  Adding constants passes the operand's derivatives
+    through (:505-509)."""
+
+    def rule(args, kwargs, sparsity_threshold):
+        operand, updates = args
+        op_shape = _logical_shape(operand)
+        tpos = ia.index_positions(op_shape, kwargs['idx'])
+        upd_shape = tuple(tpos.shape)
+        op_size = int(np.prod(op_shape, dtype=np.int64))
+        upd_size = int(np.prod(upd_shape, dtype=np.int64))
+        if not _is(operand) and not _is(updates):
+            raise NotImplementedError('scatter of constants into constants needs no derivative rule')
+        like = operand if _is(operand) else updates
+        B, dev = like.B, like.x.device
+
+        def const_rows(c, shape, size):
+            if isinstance(c, BatchedArray):
+                t = c.data.to(torch.float32)
+                return t.reshape(B, *([1] * (len(shape) - c.ndim)), *c.shape).expand(B, *shape).reshape(B, size)
+            t = so.device_const(np.broadcast_to(np.asarray(c, dtype=np.float32), shape), dev)
+            return t.reshape(1, size).expand(B, size)
+
+        if _is(updates) and tuple(updates.shape) != upd_shape:
+            nd = len(upd_shape)
+            updates = _pad_logical(updates, nd)
+            updates = broadcast_in_dim_rule((updates,), {'shape': upd_shape, 'broadcast_dimensions': range(nd)}, 0)
+
+        if not _is(updates) and mode == 'add':
+            x, _, _ = _scatter_rows('add', (operand.x.reshape(B, op_size), None, None),
+                                    (const_rows(updates, upd_shape, upd_size), None, None), tpos, op_size, dev)
+            return FwdLaplArray(x.reshape(B, *op_shape), operand.jacobian, operand.laplacian)
+
+        trip = [t for t in (operand, updates) if _is(t)]
+        sparse = all(t.jacobian.weak for t in trip)
+        out_mask, densify_after = None, False
+        if sparse:
+            out_mask = ia.scatter_out_mask(
+                operand.jacobian.x0_idx if _is(operand) else None,
+                updates.jacobian.x0_idx if _is(updates) else None, tpos, op_shape, mode == 'set')
+            max_out = out_mask.shape[0]
+            if max_out > sparsity_threshold:
+                n_dense = max(t.jacobian.max_n for t in trip) + 1
+                sparse_cost = (max_out + 1) * (upd_size + op_size) + n_dense * op_size
+                if sparse_cost >= n_dense * (upd_size + op_size):
+                    sparse = False
+                else:
+                    densify_after = True
+
+        def rows_of(t, shape, size, frame):
+            if not _is(t):
+                return const_rows(t, shape, size), None, None
+            if frame is None:
+                J = t.jacobian.dense_array
+            else:
+                M = frame.shape[0]
+                data = _expand_rows(t.jacobian.data, t.jacobian.data.shape[0], (B, *t.shape), (B, *shape))
+                J = so.materialize(data.reshape(-1, B, *shape), ia.get_index_mask(
+                    np.broadcast_to(t.jacobian.x0_idx, (t.jacobian.x0_idx.shape[0], *shape)), frame), M)
+            return t.x.reshape(B, size), J.reshape(J.shape[0], B, size), t.laplacian.reshape(B, size)
+
+        if sparse:
+            flat = out_mask.reshape(out_mask.shape[0], op_size)
+            upd_frame = np.where(tpos.reshape(-1) >= 0, flat[:, np.maximum(tpos.reshape(-1), 0)], -2)
+            op3 = rows_of(operand, op_shape, op_size, out_mask)
+            up3 = rows_of(updates, upd_shape, upd_size, upd_frame.reshape(out_mask.shape[0], *upd_shape))
+        else:
+            op3 = rows_of(operand, op_shape, op_size, None)
+            up3 = rows_of(updates, upd_shape, upd_size, None)
+            if op3[1] is not None and up3[1] is not None:
+                P = max(op3[1].shape[0], up3[1].shape[0])
+                op3 = (op3[0], so.pad_rows(op3[1], P), op3[2])
+                up3 = (up3[0], so.pad_rows(up3[1], P), up3[2])
+        x, J, L = _scatter_rows(mode, op3, up3, tpos, op_size, dev)
+        jac = FwdJacobian(J.reshape(J.shape[0], B, *op_shape), out_mask if sparse else None)
+        if densify_after:
+            jac = jac.as_dense
+        return FwdLaplArray(x.reshape(B, *op_shape), jac, L.reshape(B, *op_shape))
+
+    rule.__name__ = f'scatter_{mode}'
+    return rule
 
 
 def concatenate_rule(args, kwargs, sparsity_threshold):
@@ -964,6 +1201,8 @@ register_function('add_any', _binary_rule('add'))
 register_function('sub', _binary_rule('sub'))
 register_function('mul', _binary_rule('mul'))
 register_function('div', _binary_rule('div'))
+register_function('min', _binary_rule('min'))
+register_function('max', _binary_rule('max'))
 register_function('dot_general', dot_general)
 register_function('layer_norm', layer_norm_rule)
 register_function('reduce_sum', reduce_sum)
@@ -971,7 +1210,12 @@ register_function('reshape', reshape_rule)
 register_function('transpose', transpose_rule)
 register_function('broadcast_in_dim', broadcast_in_dim_rule)
 register_function('slice', getitem_rule)
+register_function('gather', getitem_rule)
 register_function('concatenate', concatenate_rule)
+register_function('scatter', _scatter_rule('set'))          # primitive names of jax.lax.scatter*_p
+register_function('scatter-add', _scatter_rule('add'))
+register_function('scatter_min', _scatter_rule('min'))
+register_function('scatter_max', _scatter_rule('max'))
 register_function('stop_gradient', stop_gradient_rule)
 register_function('sign', sign_rule)
 register_function('reduce_max_values', reduce_max_values)

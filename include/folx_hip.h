@@ -63,7 +63,9 @@ enum folx_hip_binop {
   FOLX_BIN_DIV = 1, /* jax.lax.div, custom Hessian (folx/custom_hessian.py:35-59)   */
   FOLX_BIN_ADD = 2, /* jax.lax.add, LINEAR                                          */
   FOLX_BIN_SUB = 3, /* jax.lax.sub, LINEAR                                          */
-  FOLX_BIN_COUNT = 4
+  FOLX_BIN_MIN = 4, /* jax.lax.min: the smaller operand's triplet, half of each at a tie */
+  FOLX_BIN_MAX = 5, /* jax.lax.max (both LINEAR, folx/wrapped_functions.py:508-513)      */
+  FOLX_BIN_COUNT = 6
 };
 
 /*
@@ -161,6 +163,21 @@ int folx_hip_reduce_max(void* stream, const float* in, float* out, int64_t outer
 int folx_hip_gather_rows(void* stream, const float* data, const int32_t* take, float* out,
                          int32_t k_in, int32_t k_out, int32_t n_slots, int64_t B,
                          int64_t S_outer, int64_t S_inner);
+
+/*
+ * Static gather along the position axis with a sum over slots -- the transposed form of a
+ * scatter with static indices, in which every output position lists the input positions
+ * that land on it:
+ *   out[rb][po][si] = sum_{s < n_slots} ( t = table[po * n_slots + s];
+ *                                         t >= 0 ? data[rb][t][si] : 0 )
+ * data [RB][S_in_outer][S_inner], table int32 [S_out_outer][n_slots] with values in
+ * [-1, S_in_outer), out [RB][S_out_outer][S_inner]; RB = (triplet rows) x (walkers).
+ * The arithmetic of the scatter rules (scatter / scatter-add / scatter_min / scatter_max,
+ * sparse_scatter_jvp, folx/jvp.py:474-673) and of integer-array indexing.
+ */
+int folx_hip_gather_cols(void* stream, const float* data, const int32_t* table, float* out,
+                         int64_t RB, int64_t S_in_outer, int64_t S_out_outer, int32_t n_slots,
+                         int64_t S_inner);
 
 /*
  * Scatter-add form of the same re-indexing (the reference's segment_sum fallback,

@@ -22,6 +22,9 @@ Pinning status (what fixes each function independently of its own formula):
   rules.sparse_slogdet_rule, index_algebra.slogdet_*
                              path choices and table shape the reference's tests expect
                              (test/test_layers.py:341-421) + equality with slogdet_rule
+  rules.scatter_rule, minmax_rule, index_algebra.scatter_out_mask
+                             brute-force fp64 Hessian trace on the cases of
+                             test/test_scatter.py; hand-derived masks
   rules.mhsa_rule            brute-force fp64 Hessian trace of softmax(q k^T) v composed
                              with random linear maps, incl. the padded-sequence masks of
                              test/experimental/pallas/test_attention.py:320-326

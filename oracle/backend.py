@@ -198,6 +198,55 @@ def divide(a, b):
     return multiply(reciprocal(b), a)
 
 
+def _minmax(a, b, is_max):
+    if _is(a) and _is(b):
+        ta, tb = _bcast3(a, b)
+        return OArr(*rules.minmax_rule(*ta, *tb, is_max=is_max))
+    t, c = (a, b) if _is(a) else (b, a)
+    t, c = _with_const(t, c)
+    shp = np.broadcast_shapes(t.x.shape, c.shape)
+    cx = np.broadcast_to(c, shp)
+    tx, tJ, tL = np.broadcast_to(t.x, shp), np.broadcast_to(t.J, (t.P, *shp)), np.broadcast_to(t.lap, shp)
+    return OArr(*rules.minmax_rule(tx, tJ, tL, cx, np.zeros_like(tJ), np.zeros_like(tL), is_max=is_max))
+
+
+def minimum(a, b):
+    return _minmax(a, b, False)
+
+
+def maximum(a, b):
+    return _minmax(a, b, True)
+
+
+def scatter(operand, idx, updates, mode='set'):
+    """``operand.at[idx].set / add / min / max (updates)`` per walker with a static numpy
+    index (in bounds); either argument may be a constant."""
+    like = operand if _is(operand) else updates
+    B, P, dt = like.B, like.P, like.x.dtype
+    op_shape = tuple(operand.shape) if _is(operand) else tuple(np.shape(operand))
+    S_op = int(np.prod(op_shape, dtype=int))
+    tpos = np.arange(S_op).reshape(op_shape)[idx]
+
+    def triple(v, shape):
+        S = int(np.prod(shape, dtype=int))
+        if _is(v):
+            if tuple(v.shape) != tuple(shape):
+                v = broadcast_to(v, shape)
+            return v.x.reshape(B, S), v.J.reshape(v.P, B, S), v.lap.reshape(B, S)
+        c = np.broadcast_to(np.asarray(v, dtype=dt), shape).reshape(1, S)
+        c = np.broadcast_to(c, (B, S))
+        return c, np.zeros((P, B, S), dt), np.zeros((B, S), dt)
+
+    op3 = triple(operand, op_shape)
+    up3 = triple(updates, tpos.shape)
+    if op3[1].shape[0] != up3[1].shape[0]:
+        Pm = max(op3[1].shape[0], up3[1].shape[0])
+        ext = lambda J: np.concatenate([J, np.zeros((Pm - J.shape[0], *J.shape[1:]), J.dtype)], 0)
+        op3, up3 = (op3[0], ext(op3[1]), op3[2]), (up3[0], ext(up3[1]), up3[2])
+    x, J, L = rules.scatter_rule(op3, up3, tpos.reshape(-1), mode)
+    return OArr(x.reshape(B, *op_shape), J.reshape(J.shape[0], B, *op_shape), L.reshape(B, *op_shape))
+
+
 def _unary(name, param=None):
     def fn(a):
         if not _is(a):

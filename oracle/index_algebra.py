@@ -358,3 +358,39 @@ def slogdet_plan(x0_idx, k: int, x_shape, max_n: int):
     if 4 * cost > tangents * n * m * (n + 1) or cost > 2 * tangents * n * m:
         return None
     return tables, transposed
+
+
+# --------------------------------------------------------------------------------------
+# Scatter (folx/jvp.py:474-673)
+# --------------------------------------------------------------------------------------
+
+
+def scatter_out_mask(op_mask, upd_mask, tpos, op_shape, is_set: bool):
+    """Output mask of a scatter with static target positions (folx/jvp.py:536-609): per
+    operand position the ascending union of the operand's dependencies (dropped where a
+    'set' overwrites the position, :549-553) and of the dependencies of every update
+    element landing there; ``-1`` padded at the end, at least one row.
+
+    op_mask (k_op, *op_shape) or None (constant operand), upd_mask (k_upd, *upd_shape) or
+    None, tpos (*upd_shape) flat operand positions (-1 = dropped)."""
+    op_size = int(np.prod(op_shape, dtype=int))
+    tflat = np.asarray(tpos).reshape(-1)
+    deps = [set() for _ in range(op_size)]
+    overwritten = set(int(p) for p in tflat if p >= 0)
+    if op_mask is not None:
+        om = np.broadcast_to(op_mask, (op_mask.shape[0], *op_shape)).reshape(op_mask.shape[0], -1)
+        for p in range(op_size):
+            if is_set and p in overwritten:
+                continue
+            deps[p] |= {int(v) for v in om[:, p] if v >= 0}
+    if upd_mask is not None:
+        um = np.broadcast_to(upd_mask, (upd_mask.shape[0], *np.shape(tpos))).reshape(upd_mask.shape[0], -1)
+        for e, p in enumerate(tflat):
+            if p >= 0:
+                deps[int(p)] |= {int(v) for v in um[:, e] if v >= 0}
+    max_out = max(1, max((len(d) for d in deps), default=0))
+    out = np.full((max_out, op_size), -1, dtype=np.int64)
+    for p, d in enumerate(deps):
+        for r, v in enumerate(sorted(d)):
+            out[r, p] = v
+    return out.reshape(max_out, *op_shape)

@@ -207,6 +207,42 @@ def add_rule(a, Ja, La, b, Jb, Lb, sign=1.0):
     return a + sign * b, Ja + sign * Jb, La + sign * Lb
 
 
+def minmax_rule(a, Ja, La, b, Jb, Lb, is_max=False):
+    """``jax.lax.min`` / ``max`` of two triplets (LINEAR, folx/wrapped_functions.py:508-513):
+    the selected operand's triplet passes through; at a tie each operand contributes half,
+    which is how jax differentiates min / max."""
+    a, b = np.broadcast_arrays(a, b)
+    first = (a > b) if is_max else (a < b)
+    w = np.where(first, 1.0, np.where(a == b, 0.5, 0.0)).astype(a.dtype)
+    y = np.maximum(a, b) if is_max else np.minimum(a, b)
+    return y, w * Ja + (1 - w) * Jb, w * La + (1 - w) * Lb
+
+
+def scatter_rule(op, upd, tpos, mode):
+    """Scatter of an updates triplet into an operand triplet at static positions
+    (``sparse_scatter_jvp``'s arithmetic, folx/jvp.py:474-673, on dense Jacobians).
+
+    op = (x (B, S_op), J (P, B, S_op), lap (B, S_op)), upd likewise with S_upd positions,
+    ``tpos (S_upd,)`` the flat operand position each update element lands on (-1 = dropped).
+    ``mode``: 'set' (a later element overwrites an earlier one), 'add', 'min', 'max'.
+    Updates are applied one element at a time, in order."""
+    x, J, L = (np.array(t, copy=True) for t in op)
+    ux, uJ, uL = upd
+    for e, p in enumerate(np.asarray(tpos).reshape(-1)):
+        if p < 0:
+            continue
+        if mode == 'set':
+            x[..., p], J[..., p], L[..., p] = ux[..., e], uJ[..., e], uL[..., e]
+        elif mode == 'add':
+            x[..., p] += ux[..., e]
+            J[..., p] += uJ[..., e]
+            L[..., p] += uL[..., e]
+        else:
+            x[..., p], J[..., p], L[..., p] = minmax_rule(
+                x[..., p], J[..., p], L[..., p], ux[..., e], uJ[..., e], uL[..., e], is_max=(mode == 'max'))
+    return x, J, L
+
+
 def sum_rule(x, J, lap, axes, keepdims=False):
     """reduce_sum is linear (SUMMATION flag, folx/wrapped_functions.py:388-392): the same
     reduction is applied to x, J rows and lap (folx/jvp.py:104-106)."""

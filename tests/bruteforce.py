@@ -179,6 +179,36 @@ class plain:
         return plain.inv(A) @ b
 
     @staticmethod
+    def minimum(a, b):
+        a, b = plain._b(a, b)
+        return torch.minimum(a, b)
+
+    @staticmethod
+    def maximum(a, b):
+        a, b = plain._b(a, b)
+        return torch.maximum(a, b)
+
+    @staticmethod
+    def scatter(operand, idx, updates, mode='set'):
+        # one scalar at a time, so that every AD mode sees plain arithmetic
+        like = operand if isinstance(operand, torch.Tensor) else updates
+        operand = plain._c(operand, like)
+        shape = tuple(operand.shape)
+        tpos = np.arange(operand.numel()).reshape(shape)[idx]
+        upd = plain._c(updates, like).expand(tpos.shape).reshape(-1)
+        flat = [v for v in operand.reshape(-1)]
+        for e, p in enumerate(tpos.reshape(-1)):
+            if mode == 'set':
+                flat[p] = upd[e]
+            elif mode == 'add':
+                flat[p] = flat[p] + upd[e]
+            elif mode == 'min':
+                flat[p] = torch.minimum(flat[p], upd[e])
+            else:
+                flat[p] = torch.maximum(flat[p], upd[e])
+        return torch.stack(flat).reshape(shape)
+
+    @staticmethod
     def sign(a):
         return torch.sign(a.detach())
 

@@ -42,7 +42,9 @@ def elementwise(name, x, jac, lap, param=0.0, inplace=False):
 
 def binary(op, a, aj, al, b, bj, bl):
     rule = {'mul': rules.mul_rule, 'div': rules.div_rule, 'add': rules.add_rule,
-            'sub': lambda *t: rules.add_rule(*t, sign=-1.0)}[op]
+            'sub': lambda *t: rules.add_rule(*t, sign=-1.0),
+            'min': lambda *t: rules.minmax_rule(*t, is_max=False),
+            'max': lambda *t: rules.minmax_rule(*t, is_max=True)}[op]
     A = [_n(t) for t in (a, aj, al)]
     Bb = [_n(t) for t in (b, bj, bl)]
     shp = np.broadcast_shapes(A[0].shape, Bb[0].shape)
@@ -96,6 +98,18 @@ def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
     return _t(out.reshape(k_out, B, S_outer * S_inner))
 
 
+def gather_cols(data, table, S_inner=1):
+    d = _n(data)
+    t = table.cpu().numpy()
+    RB = d.shape[0]
+    d = d.reshape(RB, -1, S_inner)
+    out = np.zeros((RB, t.shape[0], S_inner))
+    for s in range(t.shape[1]):
+        valid = t[:, s] >= 0
+        out[:, valid] += d[:, t[valid, s]]
+    return _t(out.reshape(RB, -1))
+
+
 def slogdet(A, AJ, AL):
     sign, (ld, jac, lap) = rules.slogdet_rule(_n(A), _n(AJ), _n(AL))
     return _t(sign), _t(ld), _t(jac), _t(lap)
@@ -138,6 +152,6 @@ def install(monkeypatch):
     import folx_amd.kernels as K
 
     for name in ('dense', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
-                 'gather_rows', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa'):
+                 'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))
