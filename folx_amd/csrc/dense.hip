@@ -5,20 +5,30 @@
 // tiles are laid out per segment (x, jac, lap) and never straddle two of them.
 //
 // Tiling: a workgroup owns BM rows x BN columns and walks K in chunks of BK = 16 through
-// double-buffered LDS tiles (global -> registers -> LDS, one barrier per chunk).  For
-// N > 128 the tile is 128 x 256 on 8 wavefronts (each 64 x 64), so a layer of width 256
-// reads its A rows from HBM exactly once and two workgroups share a CU (the stores of one
-// overlap the MFMAs of the other); narrower layers use 128 x {128, 64, 32} tiles on 4
-// wavefronts.  A rows are stored [row][k] with a stride of BK + 4 floats: a lane fetches
-// 4 consecutive k with one 128-bit LDS read and the rows of 8 consecutive lanes fall into
-// distinct bank groups.  The MFMA only needs A and B to agree on which k a lane holds, so
-// the k order inside a group of 8 is permuted to fit that read:
+// double-buffered LDS tiles, one barrier per chunk.  For N > 128 the tile is 128 x 256 on 8
+// wavefronts (each 64 x 64), so a layer of width 256 reads its A rows from HBM exactly once
+// and two workgroups share a CU; narrower layers use 128 x {128, 64, 32} tiles on 4
+// wavefronts.
+//
+// Main path (K a multiple of 16, 16-byte aligned operands): the chunks go from global memory
+// straight into LDS (global_load_lds_dwordx4), no staging registers and no LDS store
+// instructions.  Such a load puts the 16 bytes of lane i at LDS slot (wavefront base + i), so
+// the tile layout is chosen by which global address each lane asks for: an A tile is
+// [row][4 pieces of 4 k], and piece c of a row holds k-chunk c ^ ((row / 2) % 4), which
+// spreads the rows of 8 consecutive lanes over all LDS banks for the 128-bit fragment
+// reads.  The two buffers are separate LDS arrays, so the compiler's memory-counter waits
+// for the buffer being filled do not hold up reads of the buffer being computed on.
+// The MFMA only needs A and B to agree on which k a lane holds, so the k order inside a
+// group of 8 is permuted to fit the 128-bit read:
 //     lane l, register j of group t  <->  k = 8 t + 4 (l / 32) + j.
 // W rows are stored [k][n] and read with consecutive n across lanes.
 //
-// Global loads of the vector path are branch free: out-of-range rows / columns are clamped
-// to a valid address and zeroed by a select, so the loads of the next chunk issue
-// back to back ahead of the MFMAs of the current one.
+// Fallback path (any K, any alignment): global -> registers -> LDS with bounds handled by
+// clamped addresses and selects; A rows use a stride of BK + 4 floats instead of the swizzle.
+//
+// Epilogue: a tile that lies fully inside the matrix is stored without per-element tests,
+// with one 32-bit lane offset for all stores and wave-uniform scalar row arithmetic; the
+// bias is fetched before the K loop.  Edge tiles take a checked path.
 //
 // Workgroup ids are remapped so that the column tiles of one row tile run back to back
 // on the same XCD (ids are dealt round-robin to the 8 XCDs), which keeps the second
@@ -40,6 +50,207 @@ struct Segs {
   int64_t rows[3];
   int64_t tiles[3];
 };
+
+// Register r of a 32x32 accumulator tile holds row 8 (r / 4) + 4 (lane / 32) + r % 4, column
+// lane % 32, so each store instruction writes two 128-byte row segments.
+template <int BM, int BN, int TM, int TN, bool HAS_RES>
+__device__ __forceinline__ void store_tile(const floatx16 (&acc)[TM][TN], const float (&bvals)[TN],
+                                           float* __restrict__ C, const float* __restrict__ Rs, int64_t rows,
+                                           int32_t N, int64_t row0, int32_t col0, int wr, int wc, int l32,
+                                           int lh) {
+  const bool full_tile = (row0 + BM <= rows) && (col0 + BN <= N);
+  if (full_tile) {
+    const uint32_t voff = (uint32_t)((4 * lh * N + l32) * 4);
+    float* cs = C + (row0 + wr) * (int64_t)N + col0 + wc;
+    const float* rsb = HAS_RES ? Rs + (row0 + wr) * (int64_t)N + col0 + wc : nullptr;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          // the residuals of four rows are requested together, then the four rows are stored
+          float rs[4];
+          if constexpr (HAS_RES) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const char* p = (const char*)(rsb + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
+              rs[r] = *(const float*)(p + voff);
+            }
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            char* p = (char*)(cs + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
+            float o = acc[i][j][4 * g + r] + bvals[j];
+            if constexpr (HAS_RES) o += rs[r];
+            *(float*)(p + voff) = o;
+          }
+        }
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int gc = col0 + wc + j * 32 + l32;
+      const bool cok = gc < N;
+      if (cok) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t gr = row0 + wr + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+          if (gr < rows) {
+            float o = acc[i][j][r] + bvals[j];
+            if constexpr (HAS_RES) o += Rs[gr * (int64_t)N + gc];
+            C[gr * (int64_t)N + gc] = o;
+          }
+        }
+      }
+    }
+  }
+}
+
+#define FOLX_GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
+#define FOLX_LPTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// Main path: direct-to-LDS loads.  Requires K % 16 == 0, N % 4 == 0, N >= 4 and 16-byte
+// aligned operands.  Rows / columns past the end are clamped to valid addresses; what they
+// bring in only reaches accumulator rows / columns that are never stored.
+template <int BM, int BN, int WM, int WN, bool HAS_RES>
+__global__ __launch_bounds__(64 * WM * WN, 4) void dense_dma_kernel(Segs sg, const float* __restrict__ W,
+                                                                    const float* __restrict__ bias, int32_t K,
+                                                                    int32_t N, int64_t row_tiles,
+                                                                    int32_t col_tiles) {
+  constexpr int NT = 64 * WM * WN;
+  constexpr int WROWS = BM / WM, WCOLS = BN / WN;
+  constexpr int TM = WROWS / 32, TN = WCOLS / 32;
+  constexpr int TG = BK / 8;
+  constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
+  static_assert(A_V4 % 64 == 0 && W_V4 % 64 == 0, "whole wavefronts per tile chunk");
+  constexpr int A_LD = (A_V4 + NT - 1) / NT, W_LD = (W_V4 + NT - 1) / NT;
+
+  __shared__ __attribute__((aligned(16))) float As0[BM * BK];
+  __shared__ __attribute__((aligned(16))) float As1[BM * BK];
+  __shared__ __attribute__((aligned(16))) float Ws0[BK * BN];
+  __shared__ __attribute__((aligned(16))) float Ws1[BK * BN];
+
+  const int64_t id = blockIdx.x;
+  const int64_t xcd = id % NXCD;
+  const int64_t slot = id / NXCD;
+  const int64_t rt = (slot / col_tiles) * NXCD + xcd;
+  const int32_t ct = (int32_t)(slot % col_tiles);
+  if (rt >= row_tiles) return;
+  int seg = 0;
+  int64_t t = rt;
+  if (t >= sg.tiles[0]) { t -= sg.tiles[0]; seg = 1; if (t >= sg.tiles[1]) { t -= sg.tiles[1]; seg = 2; } }
+  const float* __restrict__ A = sg.in[seg];
+  const int64_t rows = sg.rows[seg];
+  const int64_t row0 = t * BM;
+  const int32_t col0 = ct * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wr = (wave / WN) * WROWS;
+  const int wc = (wave % WN) * WCOLS;
+  const int l32 = lane % 32;
+  const int lh = lane / 32;
+
+  const float* a_p[A_LD];
+  const float* w_p[W_LD];
+#pragma unroll
+  for (int i = 0; i < A_LD; ++i) {
+    const int idx = tid + NT * i;
+    const int r = idx / 4, c = idx % 4;
+    const int kc = c ^ ((r / 2) % 4);
+    int64_t gr = row0 + r;
+    if (gr >= rows) gr = rows - 1;
+    a_p[i] = A + gr * (int64_t)K + kc * 4;
+  }
+#pragma unroll
+  for (int i = 0; i < W_LD; ++i) {
+    const int idx = tid + NT * i;
+    const int k = (idx / (BN / 4)) % BK;
+    int n = col0 + (idx % (BN / 4)) * 4;
+    if (n > N - 4) n = N - 4;
+    w_p[i] = W + (int64_t)k * N + n;
+  }
+  auto issue = [&](int kt, float* as, float* ws) {
+#pragma unroll
+    for (int i = 0; i < A_LD; ++i)
+      if (A_V4 % NT == 0 || wave * 64 + NT * i < A_V4)
+        __builtin_amdgcn_global_load_lds(FOLX_GPTR(a_p[i] + kt * BK), FOLX_LPTR(&as[(wave * 64 + NT * i) * 4]), 16,
+                                         0, 0);
+#pragma unroll
+    for (int i = 0; i < W_LD; ++i)
+      if (W_V4 % NT == 0 || wave * 64 + NT * i < W_V4)
+        __builtin_amdgcn_global_load_lds(FOLX_GPTR(w_p[i] + (int64_t)kt * BK * N),
+                                         FOLX_LPTR(&ws[(wave * 64 + NT * i) * 4]), 16, 0, 0);
+  };
+
+  float bvals[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int gc = col0 + wc + j * 32 + l32;
+    bvals[j] = (seg == 0 && bias != nullptr && gc < N) ? bias[gc] : 0.0f;
+  }
+
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int sw = (l32 / 2) % 4;
+  auto compute = [&](const float* as, const float* ws) {
+#pragma unroll
+    for (int tg = 0; tg < TG; ++tg) {
+      float4 a4[TM];
+      float b[TN][4];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a4[i] = *reinterpret_cast<const float4*>(&as[(wr + i * 32 + l32) * BK + (((tg * 2 + lh) ^ sw) * 4)]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[j][q] = ws[(tg * 8 + lh * 4 + q) * BN + wc + j * 32 + l32];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const float av = q == 0 ? a4[i].x : (q == 1 ? a4[i].y : (q == 2 ? a4[i].z : a4[i].w));
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[j][q], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+  // The loads of a chunk are waited for at the end of the chunk before it; the barrier then
+  // also says that every wavefront is done reading the buffer that is refilled next.
+  const int KT = K / BK;
+  issue(0, As0, Ws0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int kt = 0; kt < KT; kt += 2) {
+    if (kt + 1 < KT) issue(kt + 1, As1, Ws1);
+    compute(As0, Ws0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (kt + 1 < KT) {
+      if (kt + 2 < KT) issue(kt + 2, As0, Ws0);
+      compute(As1, Ws1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+    }
+  }
+  store_tile<BM, BN, TM, TN, HAS_RES>(acc, bvals, sg.out[seg], HAS_RES ? sg.res[seg] : nullptr, rows, N, row0, col0,
+                                      wr, wc, l32, lh);
+}
 
 template <int BM, int BN, int WM, int WN, int MINB, bool VEC, bool HAS_RES>
 __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, const float* __restrict__ W,
@@ -80,11 +291,18 @@ __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, cons
 
   const int tid = threadIdx.x;
   const int lane = tid % 64;
-  const int wave = tid / 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wr = (wave / WN) * WROWS;
   const int wc = (wave % WN) * WCOLS;
   const int l32 = lane % 32;
   const int lh = lane / 32;
+
+  float bvals[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int gc = col0 + wc + j * 32 + l32;
+    bvals[j] = (seg == 0 && bias != nullptr && gc < N) ? bias[gc] : 0.0f;
+  }
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -210,39 +428,8 @@ __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, cons
     __syncthreads();
   }
 
-  // Epilogue: register r of a 32x32 tile holds row 8 (r / 4) + 4 (lane / 32) + r % 4,
-  // column lane % 32, so each store instruction writes two 128-byte row segments.  The
-  // residual of a sub-tile is fetched as a block before that sub-tile is stored.
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int gc = col0 + wc + j * 32 + l32;
-      const bool cok = gc < N;
-      const float bv = (seg == 0 && bias != nullptr && cok) ? bias[gc] : 0.0f;
-      float rs[16];
-      if constexpr (HAS_RES) {
-        const float* __restrict__ Rs = sg.res[seg];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          int64_t gr = row0 + wr + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-          const bool ok = cok && gr < rows;
-          if (gr >= rows) gr = rows - 1;
-          const float v = Rs[gr * (int64_t)N + (cok ? gc : 0)];
-          rs[r] = ok ? v : 0.0f;
-        }
-      }
-      if (cok) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t gr = row0 + wr + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-          float o = acc[i][j][r] + bv;
-          if constexpr (HAS_RES) o += rs[r];
-          if (gr < rows) C[gr * (int64_t)N + gc] = o;
-        }
-      }
-    }
-  }
+  store_tile<BM, BN, TM, TN, HAS_RES>(acc, bvals, C, HAS_RES ? sg.res[seg] : nullptr, rows, N, row0, col0, wr, wc,
+                                      l32, lh);
 }
 
 template <int BM, int BN, int WM, int WN, int MINB>
@@ -255,6 +442,13 @@ int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int3
   const int64_t blocks = groups * NXCD * col_tiles;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   dim3 grid((unsigned)blocks), block(64 * WM * WN);
+  if (vec && K % BK == 0 && N >= 4) {
+    if (has_res)
+      dense_dma_kernel<BM, BN, WM, WN, true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+    else
+      dense_dma_kernel<BM, BN, WM, WN, false><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+    return folx_launch_status();
+  }
   if (vec && has_res)
     dense_kernel<BM, BN, WM, WN, MINB, true, true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
   else if (vec)
