@@ -13,7 +13,8 @@
 //
 // Mapping: wavefront w owns query rows [16 w, 16 w + 16) and every key column, so all
 // row reductions stay inside 16-lane groups of one wavefront.  k, v and the current
-// k'_c, v'_c tiles (double buffered) are shared through LDS; q, q'_c and p live in
+// k'_c, v'_c tiles are shared through LDS (the next pair waits in registers; a single LDS
+// copy keeps the workgroup under 40 KB, so four workgroups share a CU); q, q'_c and p live in
 // registers in MFMA A-operand layout; p'_c goes through a wavefront-private LDS tile to
 // turn the MFMA result layout into the A-operand layout.  As in the GEMM, the k index
 // inside a group of 16 is permuted (lane l, register r <-> k = 4 (l / 16) + r) so that A
@@ -47,7 +48,8 @@ struct MhsaArgs {
   int32_t n, H, d, P;
 };
 
-template <int NW, int DT, bool EDGE>
+// FAST: n = 16 NW, d = 16 DT and no masks -- every bounds / mask test folds away.
+template <int NW, int DT, bool EDGE, bool FAST>
 __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   constexpr int NP = 16 * NW;   // padded sequence length
   constexpr int DP = 16 * DT;   // padded head dim
@@ -60,8 +62,8 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 
   __shared__ __attribute__((aligned(16))) float ks[NP * DS];
   __shared__ __attribute__((aligned(16))) float vs[NP * DS];
-  __shared__ __attribute__((aligned(16))) float kjs[2][NP * DS];
-  __shared__ __attribute__((aligned(16))) float vjs[2][NP * DS];
+  __shared__ __attribute__((aligned(16))) float kjs1[NP * DS];
+  __shared__ __attribute__((aligned(16))) float vjs1[NP * DS];
   __shared__ __attribute__((aligned(16))) float pst[NW][16 * NS];
 
   const int tid = threadIdx.x;
@@ -77,7 +79,10 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   const int64_t base = (b * n) * tok + (int64_t)h * d;  // offset of (b, 0, h, 0)
   const int64_t slice = B * n * tok;                  // stride between Jacobian rows
 
-  auto valid = [&](int i) -> bool { return i < n && (a.mask == nullptr || a.mask[b * n + i] != 0); };
+  auto valid = [&](int i) -> bool {
+    if constexpr (FAST) return true;
+    return i < n && (a.mask == nullptr || a.mask[b * n + i] != 0);
+  };
   // edge-bias entries of this lane in result layout: row 16 w + 4 lg + r, column 16 jt + l16
   const int64_t etok = (int64_t)H * n;
   const int64_t ebase = (b * n) * etok + (int64_t)h * n;
@@ -88,7 +93,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = 16 * w + 4 * lg + r, col = 16 * jt + l16;
-        if (row < n && col < n) acc[jt][r] += src[ebase + (int64_t)row * etok + col];
+        if (FAST || (row < n && col < n)) acc[jt][r] += src[ebase + (int64_t)row * etok + col];
       }
   };
 
@@ -101,7 +106,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       const int j = idx / (DP / 4);
       const int a4 = (idx % (DP / 4)) * 4;
       float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (idx < TILE4 && j < n && a4 < d && (!mask_rows || valid(j)))
+      if (FAST || (idx < TILE4 && j < n && a4 < d && (!mask_rows || valid(j))))
         val = *reinterpret_cast<const float4*>(src + base + (int64_t)j * tok + a4);
       reg[i] = val;
     }
@@ -112,7 +117,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       const int idx = tid + NT * i;
       const int j = idx / (DP / 4);
       const int a4 = (idx % (DP / 4)) * 4;
-      if (idx < TILE4) *reinterpret_cast<float4*>(dst + j * DS + a4) = reg[i];
+      if (FAST || idx < TILE4) *reinterpret_cast<float4*>(dst + j * DS + a4) = reg[i];
     }
   };
   // A-operand registers of this wavefront's 16 rows of an (n x d) array:
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
     for (int t = 0; t < DT; ++t) {
       const int a4 = 4 * lg + 16 * t;
       float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (qrow < n && a4 < d && (!mask_rows || valid(qrow)))
+      if (FAST || (qrow < n && a4 < d && (!mask_rows || valid(qrow))))
         val = *reinterpret_cast<const float4*>(src + base + (int64_t)qrow * tok + a4);
       reg[t] = val;
     }
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   for (int r = 0; r < 4; ++r) rvalid[r] = valid(16 * w + 4 * lg + r);
   bool cvalid[NW], cexist[NW];
 #pragma unroll
-  for (int jt = 0; jt < NW; ++jt) { cexist[jt] = (16 * jt + l16) < n; cvalid[jt] = valid(16 * jt + l16); }
+  for (int jt = 0; jt < NW; ++jt) { cexist[jt] = FAST || (16 * jt + l16) < n; cvalid[jt] = valid(16 * jt + l16); }
 
   // s = q k^T  (A = q registers, B = k from LDS)
   auto qk_product = [&](const float4* areg, const float* btile, floatx4* acc) {
@@ -230,14 +235,26 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) oc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   pv_product(pa, vs, oc);
+  // per-lane offset of (row 16 w + 4 lg, column l16) inside one (n, H, d) slice
+  const int64_t out_off = base + (int64_t)(16 * w + 4 * lg) * tok + l16;
   auto out_store = [&](float* dst, const floatx4* c) {
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    if constexpr (FAST) {
+      float* p = dst + out_off;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int row = 16 * w + 4 * lg + r, col = 16 * dt + l16;
-        if (row < n && col < d) dst[base + (int64_t)row * tok + col] = c[dt][r];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) p[16 * dt] = c[dt][r];
+        p += tok;
       }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = 16 * w + 4 * lg + r, col = 16 * dt + l16;
+          if (row < n && col < d) dst[base + (int64_t)row * tok + col] = c[dt][r];
+        }
+    }
   };
   out_store(a.o, oc);
 
@@ -250,19 +267,21 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
   for (int dt = 0; dt < DT; ++dt) { O2[dt] = floatx4{0.f, 0.f, 0.f, 0.f}; OL[dt] = O2[dt]; }
 
   // pass c < P: Jacobian row c; pass c == P: the Laplacians take the place of the row
-  auto active = [&](int c) -> bool { return c == P || a.imask == nullptr || a.imask[(int64_t)c * B + b] != 0; };
+  auto active = [&](int c) -> bool {
+    if constexpr (FAST) return true;
+    return c == P || a.imask == nullptr || a.imask[(int64_t)c * B + b] != 0;
+  };
   auto src_of = [&](const float* jac, const float* lap, int c) -> const float* {
     return c == P ? lap : jac + (int64_t)c * slice;
   };
 
   float4 qja[DT];
-  int buf = 0;
   if (active(0)) {
     tile_load(src_of(a.kj, a.kl, 0), rk, true);
     tile_load(src_of(a.vj, a.vl, 0), rv, true);
     rows_load(src_of(a.qj, a.ql, 0), qja, true);
-    tile_store(kjs[0], rk);
-    tile_store(vjs[0], rv);
+    tile_store(kjs1, rk);
+    tile_store(vjs1, rv);
   }
   __syncthreads();
 
@@ -282,9 +301,9 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
       for (int jt = 0; jt < NW; ++jt) sj[jt] = floatx4{0.f, 0.f, 0.f, 0.f};
       qk_product(qja, ks, sj);
-      qk_product(qa, kjs[buf], sj);
+      qk_product(qa, kjs1, sj);
       if constexpr (EDGE) edge_add(is_lap ? a.el : a.ej + (int64_t)c * eslice, sj);
-      if (!is_lap) qk_product(qja, kjs[buf], G);
+      if (!is_lap) qk_product(qja, kjs1, G);
       // p'_c = p * (s'_c - rowsum(p s'_c))
       floatx4 pj[NW];
 #pragma unroll
@@ -309,10 +328,10 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       floatx4 ojc[DT];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) ojc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-      pv_product(pa, vjs[buf], ojc);
+      pv_product(pa, vjs1, ojc);
       pv_product(pja, vs, ojc);
       if (!is_lap) {
-        pv_product(pja, vjs[buf], O2);
+        pv_product(pja, vjs1, O2);
         out_store(a.oj + (int64_t)c * slice, ojc);
       } else {
 #pragma unroll
@@ -325,13 +344,13 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       for (int dt = 0; dt < DT; ++dt) z[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
       out_store(a.oj + (int64_t)c * slice, z);
     }
+    __syncthreads();  // every wavefront is done with the current k', v' tiles
     if (nact) {
-      tile_store(kjs[buf ^ 1], rk);
-      tile_store(vjs[buf ^ 1], rv);
+      tile_store(kjs1, rk);
+      tile_store(vjs1, rv);
 #pragma unroll
       for (int t = 0; t < DT; ++t) qja[t] = qjn[t];
     }
-    buf ^= 1;
     __syncthreads();
   }
 
@@ -361,10 +380,15 @@ template <int NW, int DT>
 int launch_mhsa(hipStream_t st, const MhsaArgs& a) {
   const int64_t blocks = a.B * a.H;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-  if (a.e != nullptr)
-    mhsa_kernel<NW, DT, true><<<dim3((unsigned)blocks), dim3(FOLX_WAVE * NW), 0, st>>>(a);
-  else
-    mhsa_kernel<NW, DT, false><<<dim3((unsigned)blocks), dim3(FOLX_WAVE * NW), 0, st>>>(a);
+  const bool fast = a.n == 16 * NW && a.d == 16 * DT && a.mask == nullptr && a.imask == nullptr;
+  const dim3 grid((unsigned)blocks), block(FOLX_WAVE * NW);
+  if (a.e != nullptr) {
+    if (fast) mhsa_kernel<NW, DT, true, true><<<grid, block, 0, st>>>(a);
+    else mhsa_kernel<NW, DT, true, false><<<grid, block, 0, st>>>(a);
+  } else {
+    if (fast) mhsa_kernel<NW, DT, false, true><<<grid, block, 0, st>>>(a);
+    else mhsa_kernel<NW, DT, false, false><<<grid, block, 0, st>>>(a);
+  }
   return folx_launch_status();
 }
 
