@@ -286,10 +286,13 @@ def gather_cols(data, table, S_inner=1):
     return out
 
 
-def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
-    _chk(data, idx)
+def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
+    """out[idx[r, so], b, so, si] += data[r, b, so, si]; ``out`` = an existing (k_out, B, S)
+    row stack to accumulate into (in place), else a zero-filled one is created."""
+    _chk(data, idx, out)
     k_in = data.shape[0]
-    out = torch.zeros((k_out, B, S_outer * S_inner), device=data.device, dtype=torch.float32)
+    if out is None:
+        out = torch.zeros((k_out, B, S_outer * S_inner), device=data.device, dtype=torch.float32)
     check(
         _lib.load().folx_hip_scatter_add_rows(
             _stream(), _p(data), _p(idx), _p(out), k_in, k_out, B, S_outer, S_inner

@@ -128,3 +128,23 @@ def add_jacobians(a: FwdJacobian, b: FwdJacobian) -> FwdJacobian:
     return FwdJacobian(
         torch.cat([a.data, b.data], dim=0), np.concatenate([a.x0_idx, b.x0_idx], axis=0)
     )
+
+
+def add_sparse_rows_(dense: torch.Tensor, data: torch.Tensor, idx: np.ndarray) -> None:
+    """dense[idx[r, pos], b, pos] += data[r, b, pos], in place: adds a sparse Jacobian
+    (``data (k, B, *s)``, mask ``idx (k, *s)``, ``-1`` = no entry) into a dense row stack
+    ``(P, B, *s)`` that the caller owns (e.g. the fresh output of a GEMM), touching only the
+    k stored rows instead of materialising them first."""
+    k, B = data.shape[0], data.shape[1]
+    s = tuple(data.shape[2:])
+    idx = np.broadcast_to(idx, (k, *s))
+    n_inner = ia.split_inner(idx)
+    n_outer_axes = len(s) - n_inner
+    S_outer = int(np.prod(s[:n_outer_axes], dtype=np.int64))
+    S_inner = int(np.prod(s[n_outer_axes:], dtype=np.int64))
+    idx_c = idx[(slice(None), *([slice(None)] * n_outer_axes), *([0] * n_inner))]
+    assert int(idx_c.max(initial=-1)) < dense.shape[0]
+    table = device_table(idx_c.reshape(k, S_outer), data.device)
+    P = dense.shape[0]
+    K.scatter_add_rows(data.contiguous().reshape(k, B, S_outer * S_inner), table, P, B, S_outer, S_inner,
+                       out=dense.reshape(P, B, S_outer * S_inner))

@@ -477,6 +477,17 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
         ):
             res, residual = (residual.x, rj.data, residual.laplacian), None
     y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt, res)
+    if (
+        residual is not None and _is(residual) and new_mask is None and residual.jacobian.weak
+        and tuple(residual.shape) == (*h.shape[:-1], N) and residual.jacobian.max_n < Jy.shape[0]
+    ):
+        # sparse skip connection into a dense result: the GEMM output is fresh and owned
+        # here, so the few stored rows are added into it in place instead of being
+        # materialised to P rows first
+        so.add_sparse_rows_(Jy, residual.jacobian.data, residual.jacobian.x0_idx)
+        y = so.add_rowstacks(y, residual.x)
+        lapy = so.add_rowstacks(lapy, residual.laplacian)
+        residual = None
     out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
     if residual is not None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)

@@ -87,15 +87,19 @@ def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
     return _t(out.reshape(k_out, B, S_outer * S_inner))
 
 
-def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner):
+def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
     d = _n(data).reshape(data.shape[0], B, S_outer, S_inner)
     ix = idx.cpu().numpy()
-    out = np.zeros((k_out, B, S_outer, S_inner))
+    acc = np.zeros((k_out, B, S_outer, S_inner)) if out is None else _n(out).reshape(k_out, B, S_outer, S_inner).copy()
     for r in range(d.shape[0]):
         for so in range(S_outer):
             if ix[r, so] >= 0:
-                out[ix[r, so], :, so] += d[r, :, so]
-    return _t(out.reshape(k_out, B, S_outer * S_inner))
+                acc[ix[r, so], :, so] += d[r, :, so]
+    res = _t(acc.reshape(k_out, B, S_outer * S_inner))
+    if out is not None:
+        out.reshape(k_out, B, S_outer * S_inner).copy_(res)
+        return out
+    return res
 
 
 def gather_cols(data, table, S_inner=1):
