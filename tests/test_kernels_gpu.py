@@ -70,6 +70,12 @@ DENSE_CASES = [
     ((1, 1), 1, 1, 1, False),
     ((2, 64), 6, 512, 512, False),     # large-config width
     ((4, 16), 5, 64, 48, True),        # BN = 64 variant
+    # direct-to-LDS path (K % 16 == 0, N % 4 == 0) at its edges
+    ((1, 3), 2, 16, 4, True),          # one chunk, narrowest output
+    ((3, 50), 7, 48, 100, True),       # odd number of chunks, clamped column loads
+    ((3, 50), 4, 832, 256, False),     # long K, ragged last row tile
+    ((2, 70), 3, 32, 260, True),       # two column tiles, the second nearly empty
+    ((1, 130), 5, 64, 20, False),      # BN = 32 variant, more rows than one tile
 ]
 
 
@@ -293,11 +299,14 @@ def test_layernorm(rows, F, P):
     assert_triplet(got, (ref.x, ref.J, ref.lap), 'layernorm no affine')
 
 
-def test_dense_residual_epilogue():
+@pytest.mark.parametrize('rows,P,Kd,N', [((3, 32), 7, 256, 256),   # full tiles only: the unchecked epilogue
+                                         ((3, 50), 5, 48, 100),    # ragged rows and columns, direct-to-LDS loads
+                                         ((2, 9), 3, 20, 36)])     # register-staged fallback (K % 16 != 0)
+def test_dense_residual_epilogue(rows, P, Kd, N):
     from folx_amd import kernels as K
 
+    print(f'case dense residual rows={rows} P={P} K={Kd} N={N}', flush=True)
     rng = np.random.default_rng(12)
-    rows, P, Kd, N = (3, 32), 7, 256, 256
     x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
     rx, rJ, rL = rand(rng, *rows, N), rand(rng, P, *rows, N), rand(rng, *rows, N)
     W, b = rand(rng, Kd, N) / 16, rand(rng, N)
