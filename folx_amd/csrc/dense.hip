@@ -49,7 +49,14 @@ struct Segs {
   float* out[3];
   int64_t rows[3];
   int64_t tiles[3];
+  // Input rows may come in groups: logical row r sits at physical row
+  // (r / group) * gstride + r % group of its segment (group = 0: contiguous rows).
+  int64_t group, gstride;
 };
+
+__device__ __forceinline__ int64_t phys_row(const Segs& sg, int64_t r) {
+  return sg.group > 0 ? (r / sg.group) * sg.gstride + r % sg.group : r;
+}
 
 // Register r of a 32x32 accumulator tile holds row 8 (r / 4) + 4 (lane / 32) + r % 4, column
 // lane % 32, so each store instruction writes two 128-byte row segments.
@@ -166,7 +173,7 @@ __global__ __launch_bounds__(64 * WM * WN, 4) void dense_dma_kernel(Segs sg, con
     const int kc = c ^ ((r / 2) % 4);
     int64_t gr = row0 + r;
     if (gr >= rows) gr = rows - 1;
-    a_p[i] = A + gr * (int64_t)K + kc * 4;
+    a_p[i] = A + phys_row(sg, gr) * (int64_t)K + kc * 4;
   }
 #pragma unroll
   for (int i = 0; i < W_LD; ++i) {
@@ -327,7 +334,7 @@ __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, cons
     int64_t gr = row0 + a_r[i];
     a_ok[i] = (A_V4 % NT == 0 || idx < A_V4) && gr < rows;
     if (gr >= rows) gr = rows - 1;
-    a_p[i] = A + gr * (int64_t)K;
+    a_p[i] = A + phys_row(sg, gr) * (int64_t)K;
   }
 #pragma unroll
   for (int i = 0; i < W_LD; ++i) {
@@ -462,13 +469,15 @@ int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int3
 
 }  // namespace
 
-extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac,
-                                     const float* lap, const float* W, const float* bias,
-                                     const float* res, const float* res_jac, const float* res_lap,
-                                     float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
-                                     int32_t K, int32_t N) {
-  if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
+extern "C" int folx_hip_dense_rows_fwdlap(void* stream, const float* x, const float* jac,
+                                          const float* lap, const float* W, const float* bias,
+                                          const float* res, const float* res_jac, const float* res_lap,
+                                          float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
+                                          int32_t K, int32_t N, int64_t group, int64_t group_stride) {
+  if (R < 0 || P < 0 || K <= 0 || N <= 0 || group < 0 || (group > 0 && group_stride < group))
+    return FOLX_HIP_EINVAL;
   if (R == 0) return FOLX_HIP_OK;
+  if (group > 0 && R % group != 0) return FOLX_HIP_EINVAL;
   if (!x || !lap || !W || !y || !y_lap || (P > 0 && (!jac || !y_jac))) return FOLX_HIP_EINVAL;
   if ((res != nullptr) != (res_lap != nullptr) || (P > 0 && (res != nullptr) != (res_jac != nullptr)))
     return FOLX_HIP_EINVAL;
@@ -477,6 +486,7 @@ extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* 
   sg.in[0] = x; sg.in[1] = jac; sg.in[2] = lap;
   sg.out[0] = y; sg.out[1] = y_jac; sg.out[2] = y_lap;
   sg.rows[0] = R; sg.rows[1] = (int64_t)P * R; sg.rows[2] = R;
+  sg.group = group; sg.gstride = group_stride;
   if (P == 0) { sg.in[1] = x; sg.out[1] = y; sg.res[1] = res; }  // never dereferenced: 0 tiles
   const bool vec = (K % 4 == 0) && (N % 4 == 0) && folx_aligned16(x) && folx_aligned16(jac) &&
                    folx_aligned16(lap) && folx_aligned16(W);
@@ -486,4 +496,13 @@ extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* 
   if (N > 64) return launch_cfg<128, 128, 2, 2, 3>(st, sg, W, bias, K, N, vec, has_res);
   if (N > 32) return launch_cfg<128, 64, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);
   return launch_cfg<128, 32, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);
+}
+
+extern "C" int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac,
+                                     const float* lap, const float* W, const float* bias,
+                                     const float* res, const float* res_jac, const float* res_lap,
+                                     float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
+                                     int32_t K, int32_t N) {
+  return folx_hip_dense_rows_fwdlap(stream, x, jac, lap, W, bias, res, res_jac, res_lap, y, y_jac, y_lap, R, P, K,
+                                    N, 0, 0);
 }

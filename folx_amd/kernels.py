@@ -92,24 +92,36 @@ def _dims(*vals):
     return (ctypes.c_int64 * len(vals))(*[int(v) for v in vals])
 
 
-def dense(x, jac, lap, W, bias=None, res=None):
+def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
     """x (.., K), jac (P, .., K), lap (.., K), W (K, N) -> triplet with last dim N.
     ``res`` = optional (x, jac, lap) residual triplet of the output shape, added in the
-    GEMM epilogue."""
+    GEMM epilogue.  ``row_slice = (lo, hi)`` restricts the axis in front of the feature axis
+    to [lo, hi): the kernel reads those row groups in place (no copy of the slice)."""
     _chk(x, jac, lap, W, bias)
     rx, rj, rl = res if res is not None else (None, None, None)
     _chk(rx, rj, rl)
     K, N = W.shape
     P = jac.shape[0]
-    R = x.numel() // K
-    y = torch.empty((*x.shape[:-1], N), device=x.device, dtype=torch.float32)
-    yj = torch.empty((P, *x.shape[:-1], N), device=x.device, dtype=torch.float32)
+    lead = tuple(x.shape[:-1])
+    group = gstride = 0
+    xp, jp, lp = _p(x), _p(jac), _p(lap)
+    if row_slice is not None:
+        lo, hi = row_slice
+        n = lead[-1]
+        assert 0 <= lo < hi <= n and len(lead) >= 1
+        lead = (*lead[:-1], hi - lo)
+        group, gstride = hi - lo, n
+        off = lo * K * 4  # bytes from the first row of a group of n to row lo
+        xp, jp, lp = (ctypes.c_void_p(t.data_ptr() + off) for t in (x, jac, lap))
+    R = int(np.prod(lead, dtype=np.int64))
+    y = torch.empty((*lead, N), device=x.device, dtype=torch.float32)
+    yj = torch.empty((P, *lead, N), device=x.device, dtype=torch.float32)
     yl = torch.empty_like(y)
     with _timed('dense_fwdlap', (R, P, K, N, res is not None)):
         check(
-            _lib.load().folx_hip_dense_fwdlap(
-                _stream(), _p(x), _p(jac), _p(lap), _p(W), _p(bias), _p(rx), _p(rj), _p(rl),
-                _p(y), _p(yj), _p(yl), R, P, K, N
+            _lib.load().folx_hip_dense_rows_fwdlap(
+                _stream(), xp, jp, lp, _p(W), _p(bias), _p(rx), _p(rj), _p(rl),
+                _p(y), _p(yj), _p(yl), R, P, K, N, group, gstride
             ),
             'dense_fwdlap',
         )

@@ -80,10 +80,11 @@ def divide(a, b):
 
 
 # linear algebra ----------------------------------------------------------------------------
-def dot(h, W, b=None, residual=None):
+def dot(h, W, b=None, residual=None, row_slice=None):
     """``h @ W (+ b) (+ residual)``: last axis of ``h`` against the first axis of the
-    constant ``W``; ``residual`` is a triplet of the output shape (skip connection)."""
-    return _call('dot_general', (h, W), {'bias': b, 'residual': residual})
+    constant ``W``; ``residual`` is a triplet of the output shape (skip connection).
+    ``row_slice = (lo, hi)`` computes ``h[..., lo:hi, :] @ W`` without copying the slice."""
+    return _call('dot_general', (h, W), {'bias': b, 'residual': residual, 'row_slice': row_slice})
 
 
 def layer_norm(h, gamma=None, beta=None, eps=1e-5):

@@ -184,8 +184,7 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         m = hi - lo
         if m == 0:
             continue
-        hs = xp.getitem(h, (slice(lo, hi),))
-        orb = xp.dot(hs, p.w_orb[s])  # (m, n_det * m)
+        orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))  # (m, n_det * m), spin block read in place
         ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)  # (m, nuc, 1)
         env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
         orb = xp.multiply(orb, env)
@@ -299,8 +298,7 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         m = hi - lo
         if m == 0:
             continue
-        hs = xp.getitem(h, (slice(lo, hi),))
-        orb = xp.dot(hs, p.w_orb[s])
+        orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))
         ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)
         env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
         orb = xp.multiply(orb, env)

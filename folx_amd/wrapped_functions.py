@@ -438,6 +438,16 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     h, W = args
     bias = kwargs.get('bias')
     residual = kwargs.get('residual')
+    row_slice = kwargs.get('row_slice')
+    if row_slice is not None:
+        # the slice is consumed in place by the kernel when the Jacobian needs no re-indexing;
+        # otherwise it is an ordinary ``slice`` in front of the product
+        lo, hi = row_slice
+        plain_rows = _is(h) and not _is(W) and h.ndim >= 2 and (
+            h.jacobian.x0_idx is None or not ia.dot_projection(h.jacobian.x0_idx, -1, sparsity_threshold)[1])
+        if not plain_rows:
+            hs = getitem_rule((h,), {'idx': (Ellipsis, slice(lo, hi), slice(None))}, sparsity_threshold)
+            return dot_general((hs, W), {'bias': bias, 'residual': residual}, sparsity_threshold)
     if not _is(h):
         if _is(W):
             raise NotImplementedError('dot_general: constant @ triplet is not supported; transpose the product')
@@ -458,6 +468,11 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     Kd, N = Wt.shape
     assert h.shape[-1] == Kd, f'dot: contracting {h.shape} with {tuple(Wt.shape)}'
     J, mask = h.jacobian.data, h.jacobian.x0_idx
+    out_lead = tuple(h.shape[:-1])
+    if row_slice is not None:
+        out_lead = (*out_lead[:-1], row_slice[1] - row_slice[0])
+        if mask is not None:
+            mask = np.broadcast_to(mask, (mask.shape[0], *h.shape))[..., row_slice[0]:row_slice[1], :]
     new_mask = None
     if mask is not None:
         proj, aligned = ia.dot_projection(mask, -1, sparsity_threshold)
@@ -467,19 +482,19 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
         else:
             if aligned:
                 J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
-            new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
+            new_mask = np.broadcast_to(proj, (proj.shape[0], *out_lead, N))
     res = None
     if residual is not None and _is(residual):
         rj = residual.jacobian
         if (
             new_mask is None and not rj.weak and rj.data.shape[0] == J.shape[0]
-            and tuple(residual.shape) == (*h.shape[:-1], N)
+            and tuple(residual.shape) == (*out_lead, N)
         ):
             res, residual = (residual.x, rj.data, residual.laplacian), None
-    y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt, res)
+    y, Jy, lapy = K.dense(h.x, J, h.laplacian, Wt, bt, res, row_slice)
     if (
         residual is not None and _is(residual) and new_mask is None and residual.jacobian.weak
-        and tuple(residual.shape) == (*h.shape[:-1], N) and residual.jacobian.max_n < Jy.shape[0]
+        and tuple(residual.shape) == (*out_lead, N) and residual.jacobian.max_n < Jy.shape[0]
     ):
         # sparse skip connection into a dense result: the GEMM output is fresh and owned
         # here, so the few stored rows are added into it in place instead of being

@@ -86,6 +86,22 @@ int folx_hip_dense_fwdlap(void* stream, const float* x, const float* jac, const 
                           float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N);
 
 /*
+ * The same dense layer reading its input rows in groups: logical row r of x (and of every
+ * Jacobian row, and of lap) sits at physical row (r / group) * group_stride + r % group,
+ * counted from the pointer passed in.  That is a slice along the axis in front of the
+ * feature axis (e.g. the spin-up electrons of [B][n][K]: group = n_up, group_stride = n)
+ * consumed in place.  R counts logical rows and is a multiple of group; in jac the row
+ * groups of consecutive Jacobian rows follow each other at the same stride.  group = 0 means
+ * contiguous rows (folx_hip_dense_fwdlap).  Outputs and the residual are contiguous.
+ * Replaces a jax.lax.slice feeding _dot_general_one_constant (folx/wrapped_functions.py:71-171).
+ */
+int folx_hip_dense_rows_fwdlap(void* stream, const float* x, const float* jac, const float* lap,
+                               const float* W, const float* bias, const float* res,
+                               const float* res_jac, const float* res_lap, float* y, float* y_jac,
+                               float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N,
+                               int64_t group, int64_t group_stride);
+
+/*
  * Elementwise activation rule  y = f(x), y_jac[p] = f'(x) * jac[p],
  * y_lap = f'(x) * lap + f''(x) * sum_p jac[p]^2   in one pass over the Jacobian.
  * Replaces dense_elementwise_jvp (folx/jvp.py:687-697), the single-argument branch of

@@ -280,7 +280,10 @@ def integer_pow(a, n):
     return OArr(*rules.elementwise_rule('integer_pow', a.x, a.J, a.lap, n))
 
 
-def dot(h: OArr, W, b=None, residual=None):
+def dot(h: OArr, W, b=None, residual=None, row_slice=None):
+    """``row_slice = (lo, hi)``: the product of ``h[..., lo:hi, :]``."""
+    if row_slice is not None:
+        h = getitem(h, (Ellipsis, slice(*row_slice), slice(None)))
     W = np.asarray(W, dtype=h.x.dtype)
     bb = None if b is None else np.asarray(b, dtype=h.x.dtype)
     out = OArr(*rules.dense_rule(h.x, h.J, h.lap, W, bb))

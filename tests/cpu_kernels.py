@@ -20,8 +20,12 @@ def _t(a):
     return torch.as_tensor(np.ascontiguousarray(a, dtype=np.float32))
 
 
-def dense(x, jac, lap, W, bias=None, res=None):
-    out = rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias))
+def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
+    xs, js, ls = _n(x), _n(jac), _n(lap)
+    if row_slice is not None:
+        lo, hi = row_slice
+        xs, js, ls = xs[..., lo:hi, :], js[..., lo:hi, :], ls[..., lo:hi, :]
+    out = rules.dense_rule(xs, js, ls, _n(W), None if bias is None else _n(bias))
     if res is not None:
         out = tuple(o + _n(r) for o, r in zip(out, res))
     return tuple(_t(a) for a in out)

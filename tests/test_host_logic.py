@@ -345,3 +345,21 @@ def test_ferminet_pair_stream_stays_sparse():
     assert sorted(int(v) for v in seen['g2'].x0_idx[:, i, j, 0]) == [3, 4, 5, 9, 10, 11]
     # a diagonal pair depends on three coordinates only
     assert sorted(set(int(v) for v in seen['g2'].x0_idx[:, 2, 2, 0] if v >= 0)) == [6, 7, 8]
+
+
+@pytest.mark.parametrize('thr', [0, 3, 100])
+def test_dot_row_slice(thr):
+    """``dot(h, W, row_slice=...)`` equals slicing first, for dense Jacobians, for sparse
+    ones that pass through unchanged and for sparse ones that need re-indexing."""
+    rng = np.random.default_rng(9)
+    W1 = rng.normal(size=(3, 8)).astype(np.float32)
+    W2 = rng.normal(size=(8, 5)).astype(np.float32)
+    x = rng.normal(size=(2, 6, 3)).astype(np.float32)
+
+    def fn(xp, t):
+        h = xp.tanh(xp.dot(t, W1))                       # (6, 8), k = 3 per node
+        a = xp.dot(h, W2, row_slice=(1, 4))              # rows pass through
+        b = xp.dot(xp.transpose(h, (1, 0)), W2[:6, :], row_slice=(2, 7))  # contraction over nodes: re-indexed
+        return xp.add(xp.sum(a), xp.sum(b))
+
+    check_against_oracle(fn, x, thr)

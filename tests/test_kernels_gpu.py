@@ -93,6 +93,23 @@ def test_dense(rows, P, Kd, N, bias):
     assert_triplet(got, ref, 'dense')
 
 
+@pytest.mark.parametrize('lead,n,lo,hi,P,Kd,N', [((5,), 32, 0, 16, 9, 256, 256), ((5,), 32, 16, 32, 9, 256, 256),
+                                                 ((2, 3), 7, 2, 5, 4, 48, 20), ((4,), 9, 1, 9, 3, 17, 33),
+                                                 ((300,), 6, 3, 4, 2, 32, 64)])
+def test_dense_row_slice(lead, n, lo, hi, P, Kd, N):
+    """A slice along the axis in front of the feature axis is read in place by the GEMM."""
+    from folx_amd import kernels as K
+
+    print(f'case dense row_slice lead={lead} n={n} [{lo}:{hi}] P={P} K={Kd} N={N}', flush=True)
+    rng = np.random.default_rng(20)
+    x, J, L = rand(rng, *lead, n, Kd), rand(rng, P, *lead, n, Kd), rand(rng, *lead, n, Kd)
+    W, b = rand(rng, Kd, N) / np.sqrt(Kd), rand(rng, N)
+    ref = rules.dense_rule(*f64(x[..., lo:hi, :], J[..., lo:hi, :], L[..., lo:hi, :], W), b.astype(np.float64))
+    got = K.dense(dev(x), dev(J), dev(L), dev(W), dev(b), None, (lo, hi))
+    assert got[0].shape == (*lead, hi - lo, N)
+    assert_triplet(got, ref, 'dense row_slice')
+
+
 def test_dense_linearity_large():
     """Size-independent property at full PsiFormer row counts: the rule is linear, so
     f(a h1 + h2) = a f(h1) + f(h2) row by row, and zero rows map to zero."""
