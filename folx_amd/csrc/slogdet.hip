@@ -4,6 +4,7 @@
 //   1. Gauss-Jordan with partial pivoting on [A | I] in LDS gives A^-1; the pivots give
 //      sign and log|det| (the same pivot sequence as an LU with partial pivoting).
 //   2. tr(A^-1 lap_A) by a lane-strided product.
+//   (The matrices may be strided: a stack [batch][row][member][column] is read in place.)
 //   3. For every Jacobian row p: stage A_jac[p] in LDS (the next row is prefetched into
 //      registers meanwhile), M = A^-1 A_jac[p] with lane (i, column group) holding row i
 //      of A^-1 in registers, ld_jac[p] = tr M, and sum_p tr(M M) through an LDS transpose.
@@ -19,7 +20,8 @@ template <int NP>
 __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
-    float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P) {
+    float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
+    int64_t rstride, int64_t slice) {
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
   constexpr int G = FOLX_WAVE / NP;    // lane groups per row
   constexpr int CPL = NP / G;          // columns of M per lane
@@ -31,12 +33,13 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
 
   const int lane = threadIdx.x;
   const int64_t m = blockIdx.x;
-  const int64_t nn = (int64_t)n * n;
-  const float* a = A + m * nn;
+  // matrix m = (batch m / ND, member m % ND); element (i, j) at base + i * rstride + j
+  const int64_t base = (m / ND) * bstride + (m % ND) * dstride;
+  const float* a = A + base;
 
   float logdet, sgn;
-  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn);
-  float tl = smallmat::trace_inv_times<NP>(aug, AL + m * nn, n, lane);
+  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn, rstride);
+  float tl = smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
 
   // ---- row i of A^-1 in registers -------------------------------------------------------
   const int i = lane % NP;
@@ -49,12 +52,12 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   float mm = 0.0f;
   float pre[EPL];
   auto prefetch = [&](int p) {
-    const float* src = AJ + ((int64_t)p * NM + m) * nn;
+    const float* src = AJ + (int64_t)p * slice + base;
 #pragma unroll
     for (int c = 0; c < EPL; ++c) {
       const int e = lane + c * FOLX_WAVE;  // index into the padded NP x NP tile
       const int r = e / NP, cc = e % NP;
-      pre[c] = (r < n && cc < n) ? src[r * n + cc] : 0.0f;
+      pre[c] = (r < n && cc < n) ? src[r * rstride + cc] : 0.0f;
     }
   };
   if (P > 0) prefetch(0);
@@ -193,23 +196,37 @@ __global__ __launch_bounds__(FOLX_WAVE) void sparse_slogdet_kernel(
 
 }  // namespace
 
-extern "C" int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
-                                       const float* A_lap, float* sign, float* logdet,
-                                       float* ld_jac, float* ld_lap, int64_t NM, int32_t n,
-                                       int32_t P) {
-  if (NM < 0 || n <= 0 || P < 0) return FOLX_HIP_EINVAL;
+extern "C" int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, const float* A_jac,
+                                               const float* A_lap, float* sign, float* logdet,
+                                               float* ld_jac, float* ld_lap, int64_t NB, int64_t ND,
+                                               int32_t n, int32_t P, int64_t batch_stride,
+                                               int64_t member_stride, int64_t row_stride,
+                                               int64_t jac_stride) {
+  if (NB < 0 || ND <= 0 || n <= 0 || P < 0 || row_stride < n) return FOLX_HIP_EINVAL;
+  const int64_t NM = NB * ND;
   if (NM == 0) return FOLX_HIP_OK;
   if (!A || !A_lap || !sign || !logdet || !ld_lap || (P > 0 && (!A_jac || !ld_jac))) return FOLX_HIP_EINVAL;
   if (n > 32 || NM > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)NM), block(FOLX_WAVE);
-  if (n <= 8)
-    slogdet_kernel<8><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P);
-  else if (n <= 16)
-    slogdet_kernel<16><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P);
-  else
-    slogdet_kernel<32><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P);
+#define FOLX_SLD_LAUNCH(NPV)                                                                              \
+  slogdet_kernel<NPV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND, \
+                                              batch_stride, member_stride, row_stride, jac_stride)
+  if (n <= 8) FOLX_SLD_LAUNCH(8);
+  else if (n <= 16) FOLX_SLD_LAUNCH(16);
+  else FOLX_SLD_LAUNCH(32);
+#undef FOLX_SLD_LAUNCH
   return folx_launch_status();
+}
+
+extern "C" int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
+                                       const float* A_lap, float* sign, float* logdet,
+                                       float* ld_jac, float* ld_lap, int64_t NM, int32_t n,
+                                       int32_t P) {
+  if (NM < 0 || n <= 0 || P < 0) return FOLX_HIP_EINVAL;
+  const int64_t nn = (int64_t)n * n;
+  return folx_hip_slogdet_strided_fwdlap(stream, A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, 1, n, P, nn, 0,
+                                         n, NM * nn);
 }
 
 extern "C" int folx_hip_sparse_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,

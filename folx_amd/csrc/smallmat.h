@@ -25,13 +25,14 @@ struct Aug {
 // wavefront of the workgroup.
 template <int NP>
 __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict__ a, int n, int lane,
-                                             float& logdet, float& sgn) {
+                                             float& logdet, float& sgn, int64_t row_stride = 0) {
+  if (row_stride == 0) row_stride = n;  // rows of the matrix follow each other
   constexpr int AUGS = Aug<NP>::stride;
   constexpr int RK = (2 * NP + FOLX_WAVE - 1) / FOLX_WAVE;
   for (int e = lane; e < NP * 2 * NP; e += FOLX_WAVE) {
     const int i = e / (2 * NP), j = e % (2 * NP);
     float v;
-    if (j < NP) v = (i < n && j < n) ? a[i * n + j] : (i == j ? 1.0f : 0.0f);
+    if (j < NP) v = (i < n && j < n) ? a[i * row_stride + j] : (i == j ? 1.0f : 0.0f);
     else v = (j - NP == i) ? 1.0f : 0.0f;
     aug[i * AUGS + j] = v;
   }
@@ -90,12 +91,14 @@ __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict
 
 // tr(A^-1 L) = sum_ij A^-1[j][i] L[i][j], partial sum of this lane.
 template <int NP>
-__device__ __forceinline__ float trace_inv_times(const float* aug, const float* __restrict__ l, int n, int lane) {
+__device__ __forceinline__ float trace_inv_times(const float* aug, const float* __restrict__ l, int n, int lane,
+                                                 int64_t row_stride = 0) {
+  if (row_stride == 0) row_stride = n;
   constexpr int AUGS = Aug<NP>::stride;
   float t = 0.0f;
   for (int e = lane; e < n * n; e += FOLX_WAVE) {
     const int i = e / n, j = e % n;
-    t += aug[j * AUGS + NP + i] * l[e];
+    t += aug[j * AUGS + NP + i] * l[i * row_stride + j];
   }
   return t;
 }

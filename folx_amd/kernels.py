@@ -314,21 +314,30 @@ def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
     return out
 
 
-def slogdet(A, AJ, AL):
-    """A (.., n, n), AJ (P, .., n, n), AL (.., n, n) -> sign, logdet (..), jac (P, ..), lap (..)."""
+def slogdet(A, AJ, AL, row_axis=None):
+    """A (.., n, n), AJ (P, .., n, n), AL (.., n, n) -> sign, logdet (..), jac (P, ..), lap (..).
+    ``row_axis`` (an axis of A, default the one before last) names the axis that holds the
+    matrix rows; the last axis holds the columns and every other axis is a batch axis, in
+    order.  The matrices are read in place, whatever ``row_axis``."""
     _chk(A, AJ, AL)
     n = A.shape[-1]
     P = AJ.shape[0]
-    lead = A.shape[:-2]
-    NM = int(np.prod(lead, dtype=np.int64)) if len(lead) else 1
+    nd = A.dim()
+    ra = nd - 2 if row_axis is None else row_axis % nd
+    assert ra < nd - 1 and A.shape[ra] == n, 'slogdet needs square matrices'
+    outer, mid = tuple(A.shape[:ra]), tuple(A.shape[ra + 1:-1])
+    NB = int(np.prod(outer, dtype=np.int64))
+    ND = int(np.prod(mid, dtype=np.int64))
+    lead = (*outer, *mid)
     sign = torch.empty(lead, device=A.device, dtype=torch.float32)
     ld = torch.empty_like(sign)
     ldj = torch.empty((P, *lead), device=A.device, dtype=torch.float32)
     ldl = torch.empty_like(sign)
-    with _timed('slogdet_fwdlap', (NM, n, P)):
+    with _timed('slogdet_fwdlap', (NB * ND, n, P)):
         check(
-            _lib.load().folx_hip_slogdet_fwdlap(
-                _stream(), _p(A), _p(AJ), _p(AL), _p(sign), _p(ld), _p(ldj), _p(ldl), NM, n, P
+            _lib.load().folx_hip_slogdet_strided_fwdlap(
+                _stream(), _p(A), _p(AJ), _p(AL), _p(sign), _p(ld), _p(ldj), _p(ldl), NB, ND, n, P,
+                n * ND * n, n, ND * n, A.numel()
             ),
             'slogdet_fwdlap',
         )

@@ -107,8 +107,12 @@ def matmul(a, b):
     return np.matmul(a, b)
 
 
-def slogdet(A):
-    return _call('slogdet', (A,))
+def slogdet(A, row_axis=None):
+    """``numpy.linalg.slogdet`` over the last two axes; ``row_axis`` names another axis as the
+    one holding the matrix rows (columns stay on the last axis, all other axes are batch axes
+    in their order), which reads e.g. a dense layer's output (electron, determinant, orbital)
+    in place."""
+    return _call('slogdet', (A,), {'row_axis': row_axis})
 
 
 def det(A):

@@ -188,8 +188,8 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)  # (m, nuc, 1)
         env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
         orb = xp.multiply(orb, env)
-        mats = xp.transpose(xp.reshape(orb, (m, cfg.n_det, m)), (1, 0, 2))  # (n_det, m, m)
-        sg, ld = xp.slogdet(mats)
+        # (electron, determinant, orbital): the matrices are read in place, rows on axis 0
+        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
@@ -302,8 +302,7 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)
         env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
         orb = xp.multiply(orb, env)
-        mats = xp.transpose(xp.reshape(orb, (m, cfg.n_det, m)), (1, 0, 2))
-        sg, ld = xp.slogdet(mats)
+        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])

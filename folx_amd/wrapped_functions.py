@@ -1069,6 +1069,20 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
     (A,) = args
     if not _is(A):
         raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
+    row_axis = kwargs.get('row_axis')
+    if row_axis is not None and row_axis % A.ndim != A.ndim - 2:
+        # matrix rows on another axis than the one before last
+        ra = row_axis % A.ndim
+        assert ra < A.ndim - 1 and A.shape[ra] == A.shape[-1], 'slogdet needs square matrices'
+        if A.jacobian.weak:
+            # the sparse planner works on the canonical layout
+            perm = [a for a in range(A.ndim) if a != ra]
+            perm.insert(A.ndim - 2, ra)
+            return slogdet_wrapper((transpose_rule((A,), {'permutation': perm}, sparsity_threshold),), {},
+                                   sparsity_threshold)
+        sign, ld, ldj, ldl = K.slogdet(A.x.contiguous(), A.jacobian.data.contiguous(), A.laplacian.contiguous(),
+                                       ra + 1)
+        return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
     assert A.shape[-1] == A.shape[-2], 'slogdet needs square matrices'
     fast = _sparse_slogdet(A)
     if fast is not None:

@@ -218,6 +218,22 @@ int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,
                             float* ld_lap, int64_t NM, int32_t n, int32_t P);
 
 /*
+ * The same slogdet rule on matrices read in place from a strided stack: matrix
+ * (b, d), b < NB, d < ND, has element (i, j) at
+ *     b * batch_stride + d * member_stride + i * row_stride + j          (in floats)
+ * of A and A_lap, and at p * jac_stride + the same offset of A_jac.  Outputs are ordered
+ * [b][d] ([P][NB][ND] for ld_jac).  The orbital matrices of a dense layer's output
+ * [B][electron][determinant][orbital] are such a stack (member_stride = n,
+ * row_stride = ND * n, batch_stride = n * ND * n): no transposed copy is needed in front
+ * of folx/slogdet.py:296-344.
+ */
+int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, const float* A_jac,
+                                    const float* A_lap, float* sign, float* logdet, float* ld_jac,
+                                    float* ld_lap, int64_t NB, int64_t ND, int32_t n, int32_t P,
+                                    int64_t batch_stride, int64_t member_stride, int64_t row_stride,
+                                    int64_t jac_stride);
+
+/*
  * slogdet rule for a sparse Jacobian whose coordinates touch few rows, columns or entries
  * of A, from static rank-one factor tables shared by all NM matrices.
  *   A [NM][n][n]   A_jac [k][NM][n][n] (k stored rows)   A_lap [NM][n][n]

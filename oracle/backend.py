@@ -446,7 +446,11 @@ def det(A: OArr):
     return multiply(exp(ld), sg)
 
 
-def slogdet(A: OArr):
+def slogdet(A: OArr, row_axis=None):
+    if row_axis is not None and row_axis % A.ndim != A.ndim - 2:
+        perm = [a for a in range(A.ndim) if a != row_axis % A.ndim]
+        perm.insert(A.ndim - 2, row_axis % A.ndim)
+        A = transpose(A, perm)
     sign, (ld, J, L) = rules.slogdet_rule(A.x, A.J, A.lap)
     return OConst(sign), OArr(ld, J, L)
 

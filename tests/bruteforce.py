@@ -228,7 +228,9 @@ class plain:
         return torch.log(torch.abs(s)) + m.reshape(s.shape), torch.sign(s.detach())
 
     @staticmethod
-    def slogdet(A):
+    def slogdet(A, row_axis=None):
+        if row_axis is not None:
+            A = torch.movedim(A, row_axis, -2)
         sign, ld = torch.linalg.slogdet(A)
         return sign.detach(), ld
 

@@ -118,8 +118,13 @@ def gather_cols(data, table, S_inner=1):
     return _t(out.reshape(RB, -1))
 
 
-def slogdet(A, AJ, AL):
-    sign, (ld, jac, lap) = rules.slogdet_rule(_n(A), _n(AJ), _n(AL))
+def slogdet(A, AJ, AL, row_axis=None):
+    a, aj, al = _n(A), _n(AJ), _n(AL)
+    if row_axis is not None:
+        ra = row_axis % a.ndim
+        a, al = np.moveaxis(a, ra, -2), np.moveaxis(al, ra, -2)
+        aj = np.moveaxis(aj, ra + 1, -2)
+    sign, (ld, jac, lap) = rules.slogdet_rule(a, aj, al)
     return _t(sign), _t(ld), _t(jac), _t(lap)
 
 

@@ -227,6 +227,27 @@ def test_slogdet(n, P, lead):
     np.testing.assert_allclose(gl.cpu().numpy(), lap, rtol=1e-4 * amp, atol=1e-5 * amp * sl)
 
 
+@pytest.mark.parametrize('outer,mid,n,P', [((3,), (4,), 5, 7), ((2, 2), (16,), 16, 9), ((4,), (3, 2), 8, 5),
+                                            ((2,), (1,), 32, 4)])
+def test_slogdet_row_axis(outer, mid, n, P):
+    """Matrices whose rows sit on another axis are read in place: A (*outer, n, *mid, n)."""
+    from folx_amd import kernels as K
+
+    print(f'case slogdet row_axis outer={outer} mid={mid} n={n} P={P}', flush=True)
+    rng = np.random.default_rng(21)
+    shape = (*outer, n, *mid, n)
+    ra = len(outer)
+    A = (rand(rng, *shape) / np.sqrt(n)).astype(np.float32)
+    idx = np.arange(n)
+    np.moveaxis(A, ra, -2)[..., idx, idx] += 2.0   # dominant diagonal: well conditioned
+    J, L = rand(rng, P, *shape), rand(rng, *shape)
+    sign, (ld, jac, lap) = rules.slogdet_rule(*f64(np.moveaxis(A, ra, -2), np.moveaxis(J, ra + 1, -2),
+                                                   np.moveaxis(L, ra, -2)))
+    gs, gld, gj, gl = K.slogdet(dev(A), dev(J), dev(L), ra)
+    np.testing.assert_array_equal(gs.cpu().numpy(), sign)
+    assert_val(gld, ld, 'logdet'), assert_val(gj, jac, 'jac'), assert_lap(gl, lap, 'lap')
+
+
 def test_slogdet_closed_forms_gpu():
     """Well-conditioned closed forms at the strict bar: diagonal matrices and a row swap."""
     from folx_amd import kernels as K
