@@ -162,7 +162,8 @@ def main():
         achieved = flops / (dms / dn * 1e-3) / 1e12
         roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                 'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': f'dense_dma_kernel R={R} P={P} K={Kd} N={N} residual={has_res}', 'launches': dn,
+                'kernel': ('dense_dma_kernel' if Kd % 16 == 0 and N % 4 == 0 else 'dense_kernel')
+                + f' R={R} P={P} K={Kd} N={N} residual={has_res}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
     elif dname == 'mhsa_fwdlap':
         Bc, n, H, d, P = dkey
