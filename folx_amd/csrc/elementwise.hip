@@ -57,6 +57,49 @@ __device__ __forceinline__ void act_eval(float x, float prm, float& y, float& d1
   } else if constexpr (ACT == FOLX_ACT_EXPM1) {
     float e = expf(x);
     y = expm1f(x); d1 = e; d2 = e;
+  } else if constexpr (ACT == FOLX_ACT_SINH) {
+    float sh = sinhf(x), ch = coshf(x);
+    y = sh; d1 = ch; d2 = sh;
+  } else if constexpr (ACT == FOLX_ACT_COSH) {
+    float sh = sinhf(x), ch = coshf(x);
+    y = ch; d1 = sh; d2 = ch;
+  } else if constexpr (ACT == FOLX_ACT_TAN) {
+    float t = tanf(x);
+    y = t; d1 = 1.0f + t * t; d2 = 2.0f * t * d1;
+  } else if constexpr (ACT == FOLX_ACT_ASIN) {
+    float r = 1.0f / sqrtf(1.0f - x * x);
+    y = asinf(x); d1 = r; d2 = x * r * r * r;
+  } else if constexpr (ACT == FOLX_ACT_ACOS) {
+    float r = 1.0f / sqrtf(1.0f - x * x);
+    y = acosf(x); d1 = -r; d2 = -x * r * r * r;
+  } else if constexpr (ACT == FOLX_ACT_ATAN) {
+    float q = 1.0f / (1.0f + x * x);
+    y = atanf(x); d1 = q; d2 = -2.0f * x * q * q;
+  } else if constexpr (ACT == FOLX_ACT_ASINH) {
+    float r = 1.0f / sqrtf(1.0f + x * x);
+    y = asinhf(x); d1 = r; d2 = -x * r * r * r;
+  } else if constexpr (ACT == FOLX_ACT_ACOSH) {
+    float r = 1.0f / sqrtf(x * x - 1.0f);
+    y = acoshf(x); d1 = r; d2 = -x * r * r * r;
+  } else if constexpr (ACT == FOLX_ACT_ATANH) {
+    float q = 1.0f / (1.0f - x * x);
+    y = atanhf(x); d1 = q; d2 = 2.0f * x * q * q;
+  } else if constexpr (ACT == FOLX_ACT_ERF) {
+    float g = 1.1283791670955126f * expf(-x * x);  // 2 / sqrt(pi)
+    y = erff(x); d1 = g; d2 = -2.0f * x * g;
+  } else if constexpr (ACT == FOLX_ACT_ERFC) {
+    float g = 1.1283791670955126f * expf(-x * x);
+    y = erfcf(x); d1 = -g; d2 = 2.0f * x * g;
+  } else if constexpr (ACT == FOLX_ACT_ERF_INV) {
+    float v = erfinvf(x);
+    float g = 0.8862269254527580f * expf(v * v);  // sqrt(pi) / 2
+    y = v; d1 = g; d2 = 2.0f * v * g * g;
+  } else if constexpr (ACT == FOLX_ACT_CBRT) {
+    float c = cbrtf(x);
+    y = c; d1 = c / (3.0f * x); d2 = -2.0f * c / (9.0f * x * x);
+  } else if constexpr (ACT == FOLX_ACT_POW) {
+    float pm2 = powf(x, prm - 2.0f);
+    y = pm2 * x * x; d1 = prm * pm2 * x; d2 = prm * (prm - 1.0f) * pm2;
   } else {  // FOLX_ACT_INTEGER_POW
     int n = (int)prm;
     // x^(n-2) by repeated multiplication on |n-2|, then one or two more factors
@@ -202,6 +245,10 @@ extern "C" int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float para
     FOLX_CASE(FOLX_ACT_LOGISTIC) FOLX_CASE(FOLX_ACT_SOFTPLUS) FOLX_CASE(FOLX_ACT_SIN)
     FOLX_CASE(FOLX_ACT_COS) FOLX_CASE(FOLX_ACT_ABS) FOLX_CASE(FOLX_ACT_LOG1P)
     FOLX_CASE(FOLX_ACT_RECIPROCAL) FOLX_CASE(FOLX_ACT_EXPM1) FOLX_CASE(FOLX_ACT_INTEGER_POW)
+    FOLX_CASE(FOLX_ACT_SINH) FOLX_CASE(FOLX_ACT_COSH) FOLX_CASE(FOLX_ACT_TAN) FOLX_CASE(FOLX_ACT_ASIN)
+    FOLX_CASE(FOLX_ACT_ACOS) FOLX_CASE(FOLX_ACT_ATAN) FOLX_CASE(FOLX_ACT_ASINH) FOLX_CASE(FOLX_ACT_ACOSH)
+    FOLX_CASE(FOLX_ACT_ATANH) FOLX_CASE(FOLX_ACT_ERF) FOLX_CASE(FOLX_ACT_ERFC) FOLX_CASE(FOLX_ACT_ERF_INV)
+    FOLX_CASE(FOLX_ACT_CBRT) FOLX_CASE(FOLX_ACT_POW)
   }
 #undef FOLX_CASE
   return FOLX_HIP_EINVAL;

@@ -15,7 +15,7 @@ import threading
 import numpy as np
 
 from .api import BatchedArray, FwdLaplArray
-from .wrapped_functions import get_laplacian
+from .wrapped_functions import get_laplacian, register_function
 
 _state = threading.local()
 
@@ -56,11 +56,20 @@ def _u(name):
 tanh, exp, log, sqrt, rsqrt, square = _u('tanh'), _u('exp'), _u('log'), _u('sqrt'), _u('rsqrt'), _u('square')
 sin, cos, abs, log1p, expm1 = _u('sin'), _u('cos'), _u('abs'), _u('log1p'), _u('expm1')
 silu, softplus, sigmoid, logistic = _u('silu'), _u('softplus'), _u('sigmoid'), _u('logistic')
+sinh, cosh, tan = _u('sinh'), _u('cosh'), _u('tan')
+arcsin, arccos, arctan = _u('asin'), _u('acos'), _u('atan')
+arcsinh, arccosh, arctanh = _u('asinh'), _u('acosh'), _u('atanh')
+erf, erfc, erf_inv, cbrt = _u('erf'), _u('erfc'), _u('erf_inv'), _u('cbrt')
 reciprocal, negative, sign, stop_gradient = _u('reciprocal'), _u('neg'), _u('sign'), _u('stop_gradient')
 
 
 def integer_pow(a, n: int):
     return _call('integer_pow', (a,), {'y': int(n)})
+
+
+def power(a, c):
+    """``a ** c`` for ``a > 0`` and a constant real exponent (``jax.lax.pow`` with a constant)."""
+    return _call('pow', (a,), {'y': float(c)})
 
 
 def add(a, b):
@@ -256,3 +265,82 @@ def getitem(a, idx):
 
 def concatenate(arrs, axis=-1):
     return _call('concatenate', tuple(arrs), {'dimension': axis})
+
+
+# composed rules ---------------------------------------------------------------------------
+def clip(a, lo=None, hi=None):
+    """``numpy.clip`` with constant bounds (``jax.lax.clamp``): min / max against constants."""
+    out = a
+    if hi is not None:
+        out = minimum(out, hi)
+    if lo is not None:
+        out = maximum(out, lo)
+    return out
+
+
+def where(cond, a, b):
+    """``numpy.where`` with a derivative-free condition (``select_n``): linear in a and b."""
+    c = cond.data.to(dtype=cond.data.dtype).float() if isinstance(cond, BatchedArray) else \
+        np.asarray(cond, dtype=np.float32)
+    ci = BatchedArray(1.0 - c) if isinstance(cond, BatchedArray) else (1.0 - c)
+    cc = BatchedArray(c) if isinstance(cond, BatchedArray) else c
+    return add(multiply(a, cc), multiply(b, ci))
+
+
+def cumsum(a, axis=-1):
+    """Cumulative sum along one axis: a product with a triangular matrix of ones (LINEAR)."""
+    nd = len(_shape(a))
+    ax = axis % nd
+    n = _shape(a)[ax]
+    tri = np.triu(np.ones((n, n), dtype=np.float32))
+    if ax == nd - 1:
+        return dot(a, tri)
+    return swapaxes(dot(swapaxes(a, ax, -1), tri), ax, -1)
+
+
+def _fold(op, a, axis):
+    nd = len(_shape(a))
+    ax = axis % nd
+    n = _shape(a)[ax]
+    if n > 64:
+        raise NotImplementedError('derivative-carrying max / min / prod reductions fold pairwise: axis too long')
+    take = lambda i: getitem(a, tuple(i if d == ax else slice(None) for d in range(nd)))
+    out = take(0)
+    for i in range(1, n):
+        out = op(out, take(i))
+    return out
+
+
+def amax(a, axis=-1):
+    """max along an axis with derivatives (``reduce_max``): pairwise ``maximum`` over the axis."""
+    return _fold(maximum, a, axis)
+
+
+def amin(a, axis=-1):
+    return _fold(minimum, a, axis)
+
+
+def prod(a, axis=-1):
+    """Product along an axis (``reduce_prod``): pairwise ``multiply`` over the axis."""
+    return _fold(multiply, a, axis)
+
+
+def _composed(fn, *kw_names):
+    """Registry rule ``(args, kwargs, sparsity_threshold)`` for a composed function, so that
+    it is reachable under its primitive name like the kernel-backed rules."""
+
+    def rule(args, kwargs, threshold):
+        with sparsity_threshold(threshold):
+            return fn(*args, **{k: kwargs[k] for k in kw_names if k in kwargs})
+
+    rule.__name__ = fn.__name__
+    return rule
+
+
+# primitive names of jax.lax (folx/wrapped_functions.py:376-399, :468-513)
+register_function('clamp', lambda args, kw, thr: _composed(lambda lo, x, hi: clip(x, lo, hi))(args, kw, thr))
+register_function('select_n', lambda args, kw, thr: _composed(lambda c, b, a: where(c, a, b))(args, kw, thr))
+register_function('cumsum', _composed(cumsum, 'axis'))
+register_function('reduce_max', _composed(amax, 'axis'))
+register_function('reduce_min', _composed(amin, 'axis'))
+register_function('reduce_prod', _composed(prod, 'axis'))

@@ -132,6 +132,8 @@ _NP_UNARY = {
     'rsqrt': lambda x: 1 / np.sqrt(x), 'reciprocal': lambda x: 1 / x,
     'logistic': lambda x: 1 / (1 + np.exp(-x)), 'silu': lambda x: x / (1 + np.exp(-x)),
     'softplus': lambda x: np.logaddexp(x, 0), 'neg': np.negative,
+    'sinh': np.sinh, 'cosh': np.cosh, 'tan': np.tan, 'asin': np.arcsin, 'acos': np.arccos, 'atan': np.arctan,
+    'asinh': np.arcsinh, 'acosh': np.arccosh, 'atanh': np.arctanh, 'cbrt': np.cbrt,
 }
 
 
@@ -149,6 +151,12 @@ def _unary_rule(name: str) -> ForwardLaplacian:
         if not _is(a):
             if name == 'integer_pow':
                 return np.asarray(a) ** int(param)
+            if name == 'pow':
+                return np.asarray(a) ** float(param)
+            if name in ('erf', 'erfc', 'erf_inv'):
+                import scipy.special as sp
+
+                return {'erf': sp.erf, 'erfc': sp.erfc, 'erf_inv': sp.erfinv}[name](np.asarray(a))
             return _NP_UNARY[name](np.asarray(a))
         mask = a.jacobian.x0_idx
         x, J, lap = a.x, a.jacobian.data, a.laplacian
@@ -1232,7 +1240,8 @@ def mhsea_forward_laplacian(args, kwargs, sparsity_threshold):
 # --------------------------------------------------------------------------------------
 
 for _n in ['tanh', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'sin', 'cos', 'abs', 'log1p',
-           'expm1', 'integer_pow', 'silu', 'softplus', 'reciprocal']:
+           'expm1', 'integer_pow', 'silu', 'softplus', 'reciprocal', 'sinh', 'cosh', 'tan', 'asin', 'acos', 'atan',
+           'asinh', 'acosh', 'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt', 'pow']:
     register_function(_n, _unary_rule(_n))
 register_function('sigmoid', _unary_rule('logistic'))  # string key, folx/wrapped_functions.py:554
 register_function('neg', neg_rule)

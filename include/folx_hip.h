@@ -36,7 +36,7 @@ int folx_hip_version(void);
 const char* folx_hip_strerror(int code);
 
 /* Elementwise functions of folx_hip_elementwise_fwdlap; the rule needs f, f', f''.
- * Replaces the per-primitive entries of folx/wrapped_functions.py:400-415, :552-556. */
+ * Replaces the per-primitive entries of folx/wrapped_functions.py:400-445, :552-556. */
 enum folx_hip_act {
   FOLX_ACT_TANH = 0,
   FOLX_ACT_SILU = 1,
@@ -54,7 +54,21 @@ enum folx_hip_act {
   FOLX_ACT_RECIPROCAL = 13,
   FOLX_ACT_EXPM1 = 14,
   FOLX_ACT_INTEGER_POW = 15, /* param = exponent (integer value) */
-  FOLX_ACT_COUNT = 16
+  FOLX_ACT_SINH = 16,
+  FOLX_ACT_COSH = 17,
+  FOLX_ACT_TAN = 18,
+  FOLX_ACT_ASIN = 19,
+  FOLX_ACT_ACOS = 20,
+  FOLX_ACT_ATAN = 21,
+  FOLX_ACT_ASINH = 22,
+  FOLX_ACT_ACOSH = 23,
+  FOLX_ACT_ATANH = 24,
+  FOLX_ACT_ERF = 25,
+  FOLX_ACT_ERFC = 26,
+  FOLX_ACT_ERF_INV = 27,
+  FOLX_ACT_CBRT = 28,
+  FOLX_ACT_POW = 29, /* x^param for x > 0, param = constant real exponent (jax.lax.pow_p) */
+  FOLX_ACT_COUNT = 30
 };
 
 /* Binary functions of folx_hip_binary_fwdlap. */

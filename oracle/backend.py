@@ -274,6 +274,15 @@ negative = _unary('neg')
 log1p = _unary('log1p')
 reciprocal = _unary('reciprocal')
 expm1 = _unary('expm1')
+sinh, cosh, tan = _unary('sinh'), _unary('cosh'), _unary('tan')
+arcsin, arccos, arctan = _unary('asin'), _unary('acos'), _unary('atan')
+arcsinh, arccosh, arctanh = _unary('asinh'), _unary('acosh'), _unary('atanh')
+erf, erfc, erf_inv, cbrt = _unary('erf'), _unary('erfc'), _unary('erf_inv'), _unary('cbrt')
+
+
+def power(a, c):
+    """a ** c for a > 0 and a constant real exponent c."""
+    return _unary('pow', float(c))(a)
 
 
 def integer_pow(a, n):
@@ -522,3 +531,62 @@ def multi_head_self_attention(q: OArr, k: OArr, v: OArr, mask=None, input_mask=N
 
 def to_numpy(a):
     return a
+
+
+def clip(a: OArr, lo=None, hi=None):
+    """Constant bounds: inside the bounds the triplet passes, outside it is constant."""
+    lo_ = -np.inf if lo is None else lo
+    hi_ = np.inf if hi is None else hi
+    inside = ((a.x > lo_) & (a.x < hi_)).astype(a.x.dtype)
+    edge = 0.5 * ((a.x == lo_) | (a.x == hi_))  # jax splits a tie between the two arguments
+    w = inside + edge
+    return OArr(np.clip(a.x, lo_, hi_), a.J * w[None], a.lap * w)
+
+
+def where(cond, a, b):
+    c = np.asarray(cond.data if isinstance(cond, OConst) else cond).astype(bool)
+    like = a if _is(a) else b
+    c = np.broadcast_to(c if isinstance(cond, OConst) else c[None], like.x.shape)
+
+    def trip(v):
+        if _is(v):
+            return v.x, v.J, v.lap
+        cv = np.broadcast_to(np.asarray(v, dtype=like.x.dtype), like.x.shape)
+        return cv, np.zeros_like(like.J), np.zeros_like(like.lap)
+
+    (ax, aJ, aL), (bx, bJ, bL) = trip(a), trip(b)
+    P = max(aJ.shape[0], bJ.shape[0])
+    ext = lambda J: np.concatenate([J, np.zeros((P - J.shape[0], *J.shape[1:]), J.dtype)], 0)
+    return OArr(np.where(c, ax, bx), np.where(c[None], ext(aJ), ext(bJ)), np.where(c, aL, bL))
+
+
+def cumsum(a: OArr, axis=-1):
+    ax = axis % a.ndim
+    return OArr(np.cumsum(a.x, ax + 1), np.cumsum(a.J, ax + 2), np.cumsum(a.lap, ax + 1))
+
+
+def _arg_reduce(a: OArr, axis, fn):
+    ax = axis % a.ndim
+    idx = np.expand_dims(fn(a.x, axis=ax + 1), ax + 1)
+    tk = lambda t, off: np.squeeze(np.take_along_axis(t, idx if off == 1 else idx[None].repeat(t.shape[0], 0),
+                                                      ax + off), ax + off)
+    return OArr(tk(a.x, 1), tk(a.J, 2), tk(a.lap, 1))
+
+
+def amax(a: OArr, axis=-1):
+    return _arg_reduce(a, axis, np.argmax)
+
+
+def amin(a: OArr, axis=-1):
+    return _arg_reduce(a, axis, np.argmin)
+
+
+def prod(a: OArr, axis=-1):
+    """f = prod x_i (all x_i != 0): grad_i = f / x_i, H_ij = f / (x_i x_j) for i != j."""
+    ax = axis % a.ndim
+    f = np.prod(a.x, ax + 1)
+    g = np.expand_dims(f, ax + 1) / a.x                       # f / x_i
+    J = (np.expand_dims(g, 0) * a.J).sum(ax + 2)
+    r = a.J / a.x[None]                                        # J_pi / x_i
+    cross = (r.sum(ax + 2) ** 2 - (r * r).sum(ax + 2)).sum(0)  # sum_p sum_{i != j} r_pi r_pj
+    return OArr(f, J, (g * a.lap).sum(ax + 1) + f * cross)

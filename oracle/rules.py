@@ -107,6 +107,76 @@ def _expm1(x):
     return np.expm1(x), e, e
 
 
+def _sinh(x):
+    return np.sinh(x), np.cosh(x), np.sinh(x)
+
+
+def _cosh(x):
+    return np.cosh(x), np.sinh(x), np.cosh(x)
+
+
+def _tan(x):
+    t = np.tan(x)
+    return t, 1 + t * t, 2 * t * (1 + t * t)
+
+
+def _asin(x):
+    r = 1 / np.sqrt(1 - x * x)
+    return np.arcsin(x), r, x * r**3
+
+
+def _acos(x):
+    r = 1 / np.sqrt(1 - x * x)
+    return np.arccos(x), -r, -x * r**3
+
+
+def _atan(x):
+    q = 1 / (1 + x * x)
+    return np.arctan(x), q, -2 * x * q * q
+
+
+def _asinh(x):
+    r = 1 / np.sqrt(1 + x * x)
+    return np.arcsinh(x), r, -x * r**3
+
+
+def _acosh(x):
+    r = 1 / np.sqrt(x * x - 1)
+    return np.arccosh(x), r, -x * r**3
+
+
+def _atanh(x):
+    q = 1 / (1 - x * x)
+    return np.arctanh(x), q, 2 * x * q * q
+
+
+def _erf(x):
+    from scipy.special import erf
+
+    g = 2 / np.sqrt(np.pi) * np.exp(-x * x)
+    return erf(x), g, -2 * x * g
+
+
+def _erfc(x):
+    from scipy.special import erfc
+
+    g = 2 / np.sqrt(np.pi) * np.exp(-x * x)
+    return erfc(x), -g, 2 * x * g
+
+
+def _erf_inv(x):
+    from scipy.special import erfinv
+
+    v = erfinv(x)
+    g = np.sqrt(np.pi) / 2 * np.exp(v * v)
+    return v, g, 2 * v * g * g
+
+
+def _cbrt(x):
+    c = np.cbrt(x)
+    return c, c / (3 * x), -2 * c / (9 * x * x)
+
+
 def _identity(x):
     return x, np.ones_like(x), np.zeros_like(x)
 
@@ -130,6 +200,10 @@ ACTIVATIONS = {
     'reciprocal': _reciprocal,
     'expm1': _expm1,
     'identity': _identity,
+    # the rest of the reference's scalar table (folx/wrapped_functions.py:416-445)
+    'sinh': _sinh, 'cosh': _cosh, 'tan': _tan, 'asin': _asin, 'acos': _acos, 'atan': _atan,
+    'asinh': _asinh, 'acosh': _acosh, 'atanh': _atanh, 'erf': _erf, 'erfc': _erfc, 'erf_inv': _erf_inv,
+    'cbrt': _cbrt,
 }
 
 
@@ -147,6 +221,8 @@ def elementwise_rule(name, x, J, lap, param=None):
     """
     if name == 'integer_pow':
         y, d1, d2 = integer_pow(x, int(param))
+    elif name == 'pow':  # x^param, x > 0, constant real exponent (jax.lax.pow_p)
+        y, d1, d2 = x**param, param * x ** (param - 1), param * (param - 1) * x ** (param - 2)
     elif name == 'scale':  # y = param * x, linear
         y, d1, d2 = param * x, np.full_like(x, param), np.zeros_like(x)
     else:

@@ -57,6 +57,15 @@ class plain:
     log1p = staticmethod(torch.log1p)
     reciprocal = staticmethod(torch.reciprocal)
     expm1 = staticmethod(torch.expm1)
+    sinh, cosh, tan = staticmethod(torch.sinh), staticmethod(torch.cosh), staticmethod(torch.tan)
+    arcsin, arccos, arctan = staticmethod(torch.asin), staticmethod(torch.acos), staticmethod(torch.atan)
+    arcsinh, arccosh, arctanh = staticmethod(torch.asinh), staticmethod(torch.acosh), staticmethod(torch.atanh)
+    erf, erfc, erf_inv = staticmethod(torch.erf), staticmethod(torch.erfc), staticmethod(torch.erfinv)
+    cbrt = staticmethod(lambda t: torch.sign(t) * torch.abs(t) ** (1.0 / 3.0))
+
+    @staticmethod
+    def power(a, c):
+        return a ** float(c)
 
     @staticmethod
     def integer_pow(a, n):
@@ -209,6 +218,32 @@ class plain:
             else:
                 flat[p] = torch.maximum(flat[p], upd[e])
         return torch.stack(flat).reshape(shape)
+
+    @staticmethod
+    def clip(a, lo=None, hi=None):
+        return torch.clamp(a, lo, hi)
+
+    @staticmethod
+    def where(cond, a, b):
+        c = torch.as_tensor(np.asarray(cond)).bool()
+        a, b = plain._b(a, b)
+        return torch.where(c, a, b)
+
+    @staticmethod
+    def cumsum(a, axis=-1):
+        return torch.cumsum(a, dim=axis)
+
+    @staticmethod
+    def amax(a, axis=-1):
+        return a.amax(dim=axis)
+
+    @staticmethod
+    def amin(a, axis=-1):
+        return a.amin(dim=axis)
+
+    @staticmethod
+    def prod(a, axis=-1):
+        return a.prod(dim=axis)
 
     @staticmethod
     def sign(a):

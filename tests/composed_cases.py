@@ -1,0 +1,27 @@
+"""Models exercising the composed rules (clip, where, cumsum, amax / amin, prod) and the
+extended scalar table; shared by the oracle, host-logic and GPU tests.  x has 12 entries."""
+
+import numpy as np
+
+MASK = np.array([True, False, True, True, False, False, True, False, True, True, False, True])
+
+
+def _g(xp, x, sl):
+    return xp.getitem(x, (sl,))
+
+
+CASES = {
+    'clip': lambda xp, x: xp.clip(xp.multiply(xp.sin(x), 2.0), -0.7, 1.1),
+    'where': lambda xp, x: xp.where(MASK, xp.sin(x), xp.multiply(x, x)),
+    'where_const': lambda xp, x: xp.where(MASK, xp.tanh(x), 0.25),
+    'cumsum': lambda xp, x: xp.cumsum(xp.tanh(x)),
+    'cumsum_axis0': lambda xp, x: xp.cumsum(xp.reshape(xp.sin(x), (4, 3)), axis=0),
+    'amax': lambda xp, x: xp.amax(xp.reshape(xp.sin(xp.multiply(x, 1.7)), (3, 4)), axis=-1),
+    'amin_axis0': lambda xp, x: xp.amin(xp.reshape(xp.cos(xp.multiply(x, 1.3)), (3, 4)), axis=0),
+    'prod': lambda xp, x: xp.prod(xp.reshape(xp.add(xp.sin(x), 1.5), (3, 4)), axis=-1),
+    'scalar_table': lambda xp, x: xp.add(
+        xp.add(xp.sinh(_g(xp, x, slice(0, 4))), xp.arctan(_g(xp, x, slice(4, 8)))),
+        xp.multiply(xp.erf(_g(xp, x, slice(8, 12))), xp.power(xp.add(xp.square(_g(xp, x, slice(0, 4))), 0.5), 1.5))),
+    'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
+                                         xp.arccosh(xp.add(xp.square(x), 1.2))),
+}

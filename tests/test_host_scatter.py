@@ -12,6 +12,7 @@ from oracle import backend as ob
 import folx_amd
 from folx_amd import index_algebra as ia
 from folx_amd import numpy as fnp
+import composed_cases
 from scatter_cases import CASES, MIXED, fancy_take, min_max_elementwise
 from test_host_logic import check_against_oracle, run_product
 
@@ -40,6 +41,12 @@ def test_scatter_cases(name, thr):
 @pytest.mark.parametrize('thr', [0, 4, 12])
 def test_scatter_mixed_sparsity(name, thr):
     check_against_oracle(MIXED[name], X, thr)
+
+
+@pytest.mark.parametrize('name', sorted(composed_cases.CASES))
+@pytest.mark.parametrize('thr', [0, 12])
+def test_composed_rules(name, thr):
+    check_against_oracle(composed_cases.CASES[name], X, thr)
 
 
 @pytest.mark.parametrize('thr', [0, 12])

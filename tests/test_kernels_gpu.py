@@ -24,9 +24,11 @@ def rand(rng, *shape):
     return rng.normal(size=shape).astype(np.float32)
 
 
-POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal'}
+POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal', 'cbrt'}
+UNIT = {'asin', 'acos', 'atanh', 'erf_inv'}
 ACTS = ['tanh', 'silu', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'softplus', 'sin', 'cos',
-        'abs', 'log1p', 'reciprocal', 'expm1']
+        'abs', 'log1p', 'reciprocal', 'expm1', 'sinh', 'cosh', 'tan', 'asin', 'acos', 'atan', 'asinh', 'acosh',
+        'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt']
 
 
 @pytest.mark.parametrize('name', ACTS)
@@ -39,6 +41,12 @@ def test_elementwise(name, shape, P):
     x, J, L = rand(rng, *shape), rand(rng, P, *shape), rand(rng, *shape)
     if name in POSITIVE:
         x = np.abs(x) + 0.2
+    if name in UNIT:
+        x = rng.uniform(-0.9, 0.9, size=shape).astype(np.float32)
+    if name == 'acosh':
+        x = np.abs(x) + 1.2
+    if name in ('tan', 'sinh', 'cosh'):
+        x = np.clip(x, -1.3, 1.3)   # stay away from the poles / large magnitudes of fp32
     ref = rules.elementwise_rule(name, *f64(x, J, L))
     got = K.elementwise(name, dev(x), dev(J), dev(L))
     assert_triplet(got, ref, name)
@@ -47,6 +55,17 @@ def test_elementwise(name, shape, P):
     got2 = K.elementwise(name, tx, tJ, tL, inplace=True)
     assert got2[0].data_ptr() == tx.data_ptr()
     assert_triplet(got2, ref, name + ' in-place')
+
+
+@pytest.mark.parametrize('c', [2.5, -0.5, 1.0 / 3.0])
+def test_pow_constant_exponent(c):
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(1)
+    x, J, L = np.abs(rand(rng, 6, 9)) + 0.5, rand(rng, 5, 6, 9), rand(rng, 6, 9)
+    ref = rules.elementwise_rule('pow', *f64(x, J, L), c)
+    got = K.elementwise('pow', dev(x), dev(J), dev(L), param=c)
+    assert_triplet(got, ref, f'pow {c}')
 
 
 @pytest.mark.parametrize('n', [2, 3, -1, -2, 5])

@@ -18,7 +18,10 @@ def _close(a, b, rtol=RTOL, atol=ATOL):
     np.testing.assert_allclose(a, b, rtol=rtol, atol=atol)
 
 
-POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal'}
+POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal', 'cbrt'}
+UNIT = {'asin', 'acos', 'atanh', 'erf_inv'}      # domain (-1, 1)
+PLAIN_NAME = {'neg': 'negative', 'identity': None, 'asin': 'arcsin', 'acos': 'arccos', 'atan': 'arctan',
+              'asinh': 'arcsinh', 'acosh': 'arccosh', 'atanh': 'arctanh'}
 
 
 @pytest.mark.parametrize('name', sorted(rules.ACTIVATIONS))
@@ -27,7 +30,11 @@ def test_activation_closed_forms_vs_autograd(name):
     x = rng.normal(size=64) * 2
     if name in POSITIVE:
         x = np.abs(x) + 0.1
-    tname = {'neg': 'negative', 'identity': None}.get(name, name)
+    if name in UNIT:
+        x = rng.uniform(-0.9, 0.9, size=64)
+    if name == 'acosh':
+        x = np.abs(x) + 1.1
+    tname = PLAIN_NAME.get(name, name)
     f = (lambda t: t) if tname is None else getattr(plain, tname)
     xt = torch.tensor(x, dtype=torch.float64)
     ones = torch.ones_like(xt)
@@ -38,6 +45,18 @@ def test_activation_closed_forms_vs_autograd(name):
     _close(y, f(xt).numpy())
     _close(g1, d1.numpy())
     _close(g2, d2.numpy(), atol=1e-9)
+
+
+@pytest.mark.parametrize('c', [2.5, -0.5, 1.0 / 3.0])
+def test_pow_constant_exponent(c):
+    x = np.random.default_rng(1).uniform(0.2, 3.0, size=32)
+    xt = torch.tensor(x, dtype=torch.float64)
+    ones = torch.ones_like(xt)
+    f = lambda t: t**c
+    df = lambda t: torch.func.jvp(f, (t,), (ones,))[1]
+    y, J, L = rules.elementwise_rule('pow', x, np.ones((1, 32)), np.zeros(32), c)
+    _close(y, f(xt).numpy()), _close(J[0], df(xt).numpy())
+    _close(L, torch.func.jvp(df, (xt,), (ones,))[1].numpy(), atol=1e-9)
 
 
 def test_integer_pow():

@@ -7,6 +7,7 @@ import pytest
 from bruteforce import brute_force, plain
 from oracle import backend as ob
 from oracle import index_algebra as ia
+import composed_cases
 from scatter_cases import CASES, MIXED, fancy_take, min_max_elementwise
 
 
@@ -22,6 +23,11 @@ def _check(fn, x):
 def test_scatter_vs_bruteforce(name):
     fn = CASES.get(name) or MIXED[name]
     _check(fn, np.random.default_rng(50).normal(size=(2, 12)))
+
+
+@pytest.mark.parametrize('name', sorted(composed_cases.CASES))
+def test_composed_rules_vs_bruteforce(name):
+    _check(composed_cases.CASES[name], np.random.default_rng(53).normal(size=(2, 12)))
 
 
 def test_min_max_vs_bruteforce():

@@ -8,6 +8,7 @@ import torch
 
 from oracle import backend as ob
 from oracle import rules
+import composed_cases
 from scatter_cases import CASES, MIXED, fancy_take, min_max_elementwise
 from tolerances import assert_lap, assert_triplet, assert_val
 
@@ -82,6 +83,13 @@ def test_scatter_models(name, thr):
 def test_scatter_mixed_models(name, thr):
     print(f'case scatter mixed model {name} thr={thr}', flush=True)
     _run(MIXED[name], np.random.default_rng(73).normal(size=(5, 12)).astype(np.float32), thr)
+
+
+@pytest.mark.parametrize('name', sorted(composed_cases.CASES))
+@pytest.mark.parametrize('thr', [0, 12])
+def test_composed_rule_models(name, thr):
+    print(f'case composed model {name} thr={thr}', flush=True)
+    _run(composed_cases.CASES[name], np.random.default_rng(77).normal(size=(5, 12)).astype(np.float32), thr)
 
 
 @pytest.mark.parametrize('thr', [0, 12])
