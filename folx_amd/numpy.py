@@ -325,6 +325,66 @@ def prod(a, axis=-1):
     return _fold(multiply, a, axis)
 
 
+def flip(a, axis):
+    nd = len(_shape(a))
+    axes = (axis,) if np.isscalar(axis) else tuple(axis)
+    return _call('rev', (a,), {'dimensions': tuple(ax % nd for ax in axes)})
+
+
+def pad(a, pad_width, constant_values=0.0):
+    """``numpy.pad`` (constant mode): concatenation with constant blocks (``lax.pad``)."""
+    shape = list(_shape(a))
+    pw = [tuple(p) for p in pad_width] if np.ndim(pad_width) == 2 else [tuple(pad_width)] * len(shape)
+    out = a
+    for ax, (lo, hi) in enumerate(pw):
+        parts = []
+        if lo:
+            parts.append(np.full((*shape[:ax], lo, *shape[ax + 1:]), constant_values, dtype=np.float32))
+        parts.append(out)
+        if hi:
+            parts.append(np.full((*shape[:ax], hi, *shape[ax + 1:]), constant_values, dtype=np.float32))
+        if len(parts) > 1:
+            out = concatenate(parts, axis=ax)
+        shape[ax] += lo + hi
+    return out
+
+
+floor, ceil, round = (lambda a: _call('floor', (a,))), (lambda a: _call('ceil', (a,))), (lambda a: _call('round', (a,)))
+greater, greater_equal = (lambda a, b: _call('gt', (a, b))), (lambda a, b: _call('ge', (a, b)))
+less, less_equal = (lambda a, b: _call('lt', (a, b))), (lambda a, b: _call('le', (a, b)))
+equal, not_equal = (lambda a, b: _call('eq', (a, b))), (lambda a, b: _call('ne', (a, b)))
+
+
+def logaddexp(a, b):
+    """log(exp a + exp b) = a + softplus(b - a)."""
+    return add(a, softplus(subtract(b, a)))
+
+
+def _scan(op, a, axis):
+    nd = len(_shape(a))
+    ax = axis % nd
+    n = _shape(a)[ax]
+    if n > 64:
+        raise NotImplementedError('cumulative max / min / prod fold pairwise: axis too long')
+    take = lambda i: getitem(a, tuple(slice(i, i + 1) if d == ax else slice(None) for d in range(nd)))
+    outs = [take(0)]
+    for i in range(1, n):
+        outs.append(op(outs[-1], take(i)))
+    return concatenate(outs, axis=ax)
+
+
+def cumprod(a, axis=-1):
+    return _scan(multiply, a, axis)
+
+
+def cummax(a, axis=-1):
+    return _scan(maximum, a, axis)
+
+
+def cummin(a, axis=-1):
+    return _scan(minimum, a, axis)
+
+
 def _composed(fn, *kw_names):
     """Registry rule ``(args, kwargs, sparsity_threshold)`` for a composed function, so that
     it is reachable under its primitive name like the kernel-backed rules."""
@@ -344,3 +404,8 @@ register_function('cumsum', _composed(cumsum, 'axis'))
 register_function('reduce_max', _composed(amax, 'axis'))
 register_function('reduce_min', _composed(amin, 'axis'))
 register_function('reduce_prod', _composed(prod, 'axis'))
+register_function('cumprod', _composed(cumprod, 'axis'))
+register_function('cummax', _composed(cummax, 'axis'))
+register_function('cummin', _composed(cummin, 'axis'))
+register_function('logaddexp', _composed(logaddexp))
+register_function('pad', _composed(pad, 'constant_values'))

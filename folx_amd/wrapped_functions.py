@@ -703,6 +703,35 @@ def transpose_rule(args, kwargs, sparsity_threshold):
     return _index_rule(fn_t, lambda m: np.transpose(m, (0, *[p + 1 for p in perm])))(a)
 
 
+def rev_rule(args, kwargs, sparsity_threshold):
+    """``lax.rev``: reverse along ``dimensions`` (INDEXING, folx/wrapped_functions.py:505-507)."""
+    (a,) = args
+    dims = tuple(kwargs['dimensions'])
+    fn_t = lambda t, lead: torch.flip(t, [d + lead for d in dims])
+    if not _is(a):
+        return _const_index(a, fn_t)
+    return _index_rule(fn_t, lambda m: np.flip(m, tuple(d + 1 for d in dims)))(a)
+
+
+def _values_only(torch_fn, np_fn):
+    """Piecewise-constant functions (floor, ceil, round, comparisons): the result carries no
+    derivatives (``warp_without_fwd_laplacian``, folx/wrapped_functions.py:446-448, :538-551)."""
+
+    def rule(args, kwargs, sparsity_threshold):
+        vals, like = [], None
+        for a in args:
+            t = a.x if _is(a) else (a.data if isinstance(a, BatchedArray) else None)
+            like = t if t is not None and like is None else like
+            vals.append(t if t is not None else a)
+        if like is None:
+            return np_fn(*[np.asarray(v) for v in vals])
+        tens = [v if isinstance(v, torch.Tensor) else so.device_const(np.asarray(v, dtype=np.float32), like.device)
+                for v in vals]
+        return BatchedArray(torch_fn(*tens).to(torch.float32))
+
+    return rule
+
+
 def broadcast_in_dim_rule(args, kwargs, sparsity_threshold):
     """``broadcast_in_dim(shape, broadcast_dimensions)`` as in lax."""
     (a,) = args
@@ -1257,6 +1286,11 @@ register_function('layer_norm', layer_norm_rule)
 register_function('reduce_sum', reduce_sum)
 register_function('reshape', reshape_rule)
 register_function('transpose', transpose_rule)
+register_function('rev', rev_rule)
+for _n, _tf, _nf in [('floor', torch.floor, np.floor), ('ceil', torch.ceil, np.ceil), ('round', torch.round, np.round),
+                     ('gt', torch.gt, np.greater), ('ge', torch.ge, np.greater_equal), ('lt', torch.lt, np.less),
+                     ('le', torch.le, np.less_equal), ('eq', torch.eq, np.equal), ('ne', torch.ne, np.not_equal)]:
+    register_function(_n, _values_only(_tf, _nf))
 register_function('broadcast_in_dim', broadcast_in_dim_rule)
 register_function('slice', getitem_rule)
 register_function('gather', getitem_rule)

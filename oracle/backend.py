@@ -590,3 +590,66 @@ def prod(a: OArr, axis=-1):
     r = a.J / a.x[None]                                        # J_pi / x_i
     cross = (r.sum(ax + 2) ** 2 - (r * r).sum(ax + 2)).sum(0)  # sum_p sum_{i != j} r_pi r_pj
     return OArr(f, J, (g * a.lap).sum(ax + 1) + f * cross)
+
+
+def flip(a: OArr, axis):
+    axes = (axis,) if np.isscalar(axis) else tuple(axis)
+    ax = tuple(x % a.ndim for x in axes)
+    return OArr(np.flip(a.x, tuple(x + 1 for x in ax)), np.flip(a.J, tuple(x + 2 for x in ax)),
+                np.flip(a.lap, tuple(x + 1 for x in ax)))
+
+
+def pad(a: OArr, pad_width, constant_values=0.0):
+    pw = [tuple(p) for p in pad_width] if np.ndim(pad_width) == 2 else [tuple(pad_width)] * a.ndim
+    return OArr(np.pad(a.x, [(0, 0)] + pw, constant_values=constant_values), np.pad(a.J, [(0, 0), (0, 0)] + pw),
+                np.pad(a.lap, [(0, 0)] + pw))
+
+
+def _cmp(fn):
+    def f(a, b):
+        av = a.x if _is(a) else np.asarray(a)
+        bv = b.x if _is(b) else np.asarray(b)
+        return OConst(fn(av, bv))
+
+    return f
+
+
+greater, greater_equal, less, less_equal = _cmp(np.greater), _cmp(np.greater_equal), _cmp(np.less), _cmp(np.less_equal)
+
+
+def floor(a):
+    return OConst(np.floor(a.x))
+
+
+def logaddexp(a: OArr, b: OArr):
+    """From the Hessian of log(e^a + e^b): weights s = sigmoid(a - b), curvature s (1 - s)."""
+    (ax, aJ, aL), (bx, bJ, bL) = _bcast3(a, b)
+    s = 1.0 / (1.0 + np.exp(bx - ax))
+    d = aJ - bJ
+    return OArr(np.logaddexp(ax, bx), s * aJ + (1 - s) * bJ, s * aL + (1 - s) * bL + s * (1 - s) * (d * d).sum(0))
+
+
+def cumprod(a: OArr, axis=-1):
+    ax = axis % a.ndim
+    n = a.shape[ax]
+    parts = [prod(getitem(a, tuple(slice(0, i + 1) if d == ax else slice(None) for d in range(a.ndim))), axis=ax)
+             for i in range(n)]
+    return OArr(np.stack([p.x for p in parts], ax + 1), np.stack([p.J for p in parts], ax + 2),
+                np.stack([p.lap for p in parts], ax + 1))
+
+
+def _cumarg(a: OArr, axis, red):
+    ax = axis % a.ndim
+    n = a.shape[ax]
+    parts = [red(getitem(a, tuple(slice(0, i + 1) if d == ax else slice(None) for d in range(a.ndim))), axis=ax)
+             for i in range(n)]
+    return OArr(np.stack([p.x for p in parts], ax + 1), np.stack([p.J for p in parts], ax + 2),
+                np.stack([p.lap for p in parts], ax + 1))
+
+
+def cummax(a: OArr, axis=-1):
+    return _cumarg(a, axis, amax)
+
+
+def cummin(a: OArr, axis=-1):
+    return _cumarg(a, axis, amin)

@@ -225,7 +225,7 @@ class plain:
 
     @staticmethod
     def where(cond, a, b):
-        c = torch.as_tensor(np.asarray(cond)).bool()
+        c = cond.bool() if isinstance(cond, torch.Tensor) else torch.as_tensor(np.asarray(cond)).bool()
         a, b = plain._b(a, b)
         return torch.where(c, a, b)
 
@@ -244,6 +244,33 @@ class plain:
     @staticmethod
     def prod(a, axis=-1):
         return a.prod(dim=axis)
+
+    @staticmethod
+    def flip(a, axis):
+        return torch.flip(a, [axis] if np.isscalar(axis) else list(axis))
+
+    @staticmethod
+    def pad(a, pad_width, constant_values=0.0):
+        pw = [tuple(p) for p in pad_width] if np.ndim(pad_width) == 2 else [tuple(pad_width)] * a.ndim
+        flat = [v for p in reversed(pw) for v in p]
+        return torch.nn.functional.pad(a, flat, value=constant_values)
+
+    greater = staticmethod(lambda a, b: (a > plain._c(b, a)).detach())
+    less = staticmethod(lambda a, b: (a < plain._c(b, a)).detach())
+    floor = staticmethod(lambda a: torch.floor(a).detach())
+    logaddexp = staticmethod(torch.logaddexp)
+
+    @staticmethod
+    def cumprod(a, axis=-1):
+        return torch.cumprod(a, dim=axis)
+
+    @staticmethod
+    def cummax(a, axis=-1):
+        return torch.cummax(a, dim=axis).values
+
+    @staticmethod
+    def cummin(a, axis=-1):
+        return torch.cummin(a, dim=axis).values
 
     @staticmethod
     def sign(a):

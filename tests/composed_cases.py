@@ -22,6 +22,12 @@ CASES = {
     'scalar_table': lambda xp, x: xp.add(
         xp.add(xp.sinh(_g(xp, x, slice(0, 4))), xp.arctan(_g(xp, x, slice(4, 8)))),
         xp.multiply(xp.erf(_g(xp, x, slice(8, 12))), xp.power(xp.add(xp.square(_g(xp, x, slice(0, 4))), 0.5), 1.5))),
+    'flip_pad': lambda xp, x: xp.pad(xp.flip(xp.reshape(xp.sin(x), (4, 3)), 0), ((1, 0), (0, 2)), 0.5),
+    'where_data_dependent': lambda xp, x: xp.where(xp.greater(x, 0.1), xp.tanh(x), xp.multiply(xp.cos(x), 0.3)),
+    'logaddexp': lambda xp, x: xp.logaddexp(_g(xp, x, slice(0, 6)), xp.sin(_g(xp, x, slice(6, 12)))),
+    'cumprod': lambda xp, x: xp.cumprod(xp.reshape(xp.add(xp.sin(x), 1.5), (3, 4)), axis=-1),
+    'cummax': lambda xp, x: xp.cummax(xp.reshape(xp.sin(xp.multiply(x, 1.9)), (3, 4)), axis=-1),
+    'cummin_axis0': lambda xp, x: xp.cummin(xp.reshape(xp.cos(xp.multiply(x, 1.4)), (3, 4)), axis=0),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }
