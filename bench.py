@@ -173,6 +173,15 @@ def main():
                 'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
                 'kernel': f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
+    elif dname == 'dense_act_fwdlap':
+        act, R, P, Kd, N = dkey
+        nbytes = 4.0 * ((P + 2) * R * (Kd + N) + Kd * N)
+        achieved = nbytes / (dms / dn * 1e-3) / 1e9
+        roof = {'bound': 'hbm', 'achieved': achieved, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                'frac': achieved / PEAK_HBM_GBS, 'traffic': None,
+                'kernel': f'dense_act_kernel {act} R={R} P={P} K={Kd} N={N}', 'launches': dn,
+                'avg_launch_ms': dms / dn,
+                'mfma_tflops': 2.0 * (P + 2) * R * Kd * N / (dms / dn * 1e-3) / 1e12}
     else:
         roof = {'bound': 'hbm', 'achieved': None, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': None,
                 'traffic': None, 'kernel': f'{dname} {dkey}', 'launches': dn, 'avg_launch_ms': dms / dn}

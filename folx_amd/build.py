@@ -22,6 +22,7 @@ SOURCES = [
     'api.cpp',
     'elementwise.hip',
     'dense.hip',
+    'dense_act.hip',
     'pointwise.hip',
     'reduce.hip',
     'gather.hip',

@@ -128,6 +128,41 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
     return y, yj, yl
 
 
+FUSED_ACTS = ('tanh', 'silu', 'logistic', 'sigmoid', 'softplus', 'exp', 'sin', 'cos', 'square')
+
+
+def dense_act_supported(name, K, N):
+    """Shapes and functions the fused dense + activation kernel is built for."""
+    return name in FUSED_ACTS and 4 <= K <= 128 and K % 4 == 0 and 1 <= N <= 128
+
+
+def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
+    """``f(x @ W + bias)`` as one rule: x (.., K), jac (P, .., K), lap (.., K), W (K, N) ->
+    the activated triplet with last dim N; the pre-activation triplet is never written."""
+    _chk(x, jac, lap, W, bias)
+    K, N = W.shape
+    P = jac.shape[0]
+    lead = tuple(x.shape[:-1])
+    R = int(np.prod(lead, dtype=np.int64))
+    lib = _lib.load()
+    nbytes = int(lib.folx_hip_dense_act_workspace_bytes(R, P, K, N))
+    if nbytes < 0:
+        check(nbytes, 'dense_act_workspace_bytes')
+    ws = torch.empty(nbytes // 4, device=x.device, dtype=torch.float32) if nbytes > 0 else None
+    y = torch.empty((*lead, N), device=x.device, dtype=torch.float32)
+    yj = torch.empty((P, *lead, N), device=x.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    with _timed('dense_act_fwdlap', (name, R, P, K, N)):
+        check(
+            lib.folx_hip_dense_act_fwdlap(
+                _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(W), _p(bias),
+                _p(y), _p(yj), _p(yl), R, P, K, N, _p(ws), nbytes
+            ),
+            f'dense_act_fwdlap[{name}]',
+        )
+    return y, yj, yl
+
+
 def elementwise(name, x, jac, lap, param=0.0, inplace=False):
     _chk(x, jac, lap)
     P = jac.shape[0]

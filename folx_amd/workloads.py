@@ -35,7 +35,7 @@ def mlp_forward(params, x, xp=None):
     if xp is None:
         from . import numpy as xp
     for W, b in params[:-1]:
-        x = xp.silu(xp.dot(x, W, b))
+        x = xp.dot(x, W, b, act='silu')
     W, b = params[-1]
     return xp.sum(xp.dot(x, W, b))
 
@@ -288,10 +288,10 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         d1 = h.shape[-1]
         parts = [h, xp.broadcast_to(hu, (n, d1)), xp.broadcast_to(hd, (n, d1)), gu, gd]
         f = xp.concatenate(parts, axis=-1)
-        hn = xp.tanh(xp.dot(f, L['v'], L['b']))
+        hn = xp.dot(f, L['v'], L['b'], act='tanh')
         h = xp.add(h, hn) if hn.shape == h.shape else hn
         if 'w' in L:
-            gn = xp.tanh(xp.dot(g, L['w'], L['c']))
+            gn = xp.dot(g, L['w'], L['c'], act='tanh')
             g = xp.add(g, gn) if gn.shape == g.shape else gn
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, nu), (nu, n)]):

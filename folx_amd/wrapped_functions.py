@@ -447,6 +447,9 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     bias = kwargs.get('bias')
     residual = kwargs.get('residual')
     row_slice = kwargs.get('row_slice')
+    act = kwargs.get('act')
+    if act is not None:
+        return _dot_then_act(h, W, dict(kwargs), sparsity_threshold)
     if row_slice is not None:
         # the slice is consumed in place by the kernel when the Jacobian needs no re-indexing;
         # otherwise it is an ordinary ``slice`` in front of the product
@@ -514,6 +517,49 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
     if residual is not None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)
+    return out
+
+
+def _dot_then_act(h, W, kwargs, thr: int):
+    """``residual + act(h @ W + bias)``: a Dense + activation layer as ONE rule when the layer
+    is narrow enough for the fused kernel (``kernels.dense_act_supported``) and the result's
+    Jacobian rows are plain (dense, or sparse without an index listed twice at a position,
+    where sum_k J_k^2 is the Hessian term, folx/hessian.py:460-470); otherwise the
+    ``dot_general`` rule followed by the elementwise rule, which is also what defines the
+    result."""
+    act = kwargs.pop('act')
+    param = kwargs.pop('act_param', 0.0)
+    residual = kwargs.pop('residual', None)
+    bias = kwargs.get('bias')
+    fused = (
+        _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
+        and K.dense_act_supported(act, *np.shape(W))
+    )
+    J = new_mask = None
+    if fused:
+        J, mask = h.jacobian.data, h.jacobian.x0_idx
+        N = np.shape(W)[1]
+        if mask is not None:
+            proj, aligned = ia.dot_projection(mask, -1, thr)
+            if proj is None:
+                J = h.jacobian.dense_array
+            elif ia.has_duplicates(proj):
+                fused = False
+            else:
+                if aligned:
+                    J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
+                new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
+    if fused:
+        dev = h.x.device
+        Wt = so.device_const(W, dev)
+        bt = None if bias is None else so.device_const(bias, dev)
+        y, Jy, lapy = K.dense_act(act, h.x, J, h.laplacian, Wt, bt, param)
+        out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
+    else:
+        out = dot_general((h, W), kwargs, thr)
+        out = _LAPLACE_FN_REGISTRY[act]((out,), {'param': param}, thr)
+    if residual is not None:
+        out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)
     return out
 
 

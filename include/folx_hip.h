@@ -128,6 +128,29 @@ int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float param, const fl
                                 float* y_lap, int64_t S, int32_t P);
 
 /*
+ * Narrow dense layer followed by its activation, in one pass:
+ *   y = f(x @ W + bias),  y_jac[p] = f'(z) * (jac[p] @ W),
+ *   y_lap = f'(z) * (lap @ W) + f''(z) * sum_p (jac[p] @ W)^2,      z = x @ W + bias.
+ * The composition of _dot_general_one_constant (folx/wrapped_functions.py:71-171) with the
+ * elementwise rule (folx/jvp.py:687-697, folx/hessian.py:87-112, folx/wrapper.py:120-125)
+ * that follows it in every Dense + activation layer; the pre-activation triplet is never
+ * written.  Layouts as in folx_hip_dense_fwdlap.  Built for 4 <= K <= 128 with K % 4 == 0,
+ * N <= 128, 16-byte aligned inputs and act in {TANH, SILU, LOGISTIC, SOFTPLUS, EXP, SIN, COS,
+ * SQUARE}; anything else returns FOLX_HIP_ENOTSUP and the caller uses the two separate rules.
+ * Outputs must not overlap inputs.
+ * workspace: folx_hip_dense_act_workspace_bytes(R, P, K, N) bytes of device memory (0 for
+ * large R: then it may be NULL), contents irrelevant; it holds partial sums between the two
+ * launches a small batch is split into.  The query returns a negative code for unsupported
+ * shapes.
+ */
+int64_t folx_hip_dense_act_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N);
+int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const float* x,
+                              const float* jac, const float* lap, const float* W,
+                              const float* bias, float* y, float* y_jac, float* y_lap,
+                              int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
+                              int64_t workspace_bytes);
+
+/*
  * Binary elementwise rule for two operands whose Jacobians live on the same row frame
  * (both dense with P rows, or sparse with identical index masks).  The output index
  * space is (n0, n1, n2), row-major; each operand addresses it with element strides

@@ -289,8 +289,12 @@ def integer_pow(a, n):
     return OArr(*rules.elementwise_rule('integer_pow', a.x, a.J, a.lap, n))
 
 
-def dot(h: OArr, W, b=None, residual=None, row_slice=None):
-    """``row_slice = (lo, hi)``: the product of ``h[..., lo:hi, :]``."""
+def dot(h: OArr, W, b=None, residual=None, row_slice=None, act=None):
+    """``row_slice = (lo, hi)``: the product of ``h[..., lo:hi, :]``; ``act``: a scalar function
+    applied to ``h @ W + b`` before the residual is added."""
+    if act is not None:
+        out = _unary({'sigmoid': 'logistic'}.get(act, act))(dot(h, W, b, None, row_slice))
+        return out if residual is None else add(residual, out)
     if row_slice is not None:
         h = getitem(h, (Ellipsis, slice(*row_slice), slice(None)))
     W = np.asarray(W, dtype=h.x.dtype)

@@ -24,11 +24,13 @@ class plain:
         return torch.as_tensor(np.asarray(c), dtype=like.dtype)
 
     @staticmethod
-    def dot(h, W, b=None, residual=None, row_slice=None):
+    def dot(h, W, b=None, residual=None, row_slice=None, act=None):
         if row_slice is not None:
             h = h[..., row_slice[0]:row_slice[1], :]
         y = h @ plain._c(W, h)
         y = y if b is None else y + plain._c(b, h)
+        if act is not None:
+            y = getattr(plain, {'logistic': 'sigmoid'}.get(act, act))(y)
         return y if residual is None else residual + y
 
     @staticmethod

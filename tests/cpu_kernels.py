@@ -31,6 +31,12 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
     return tuple(_t(a) for a in out)
 
 
+def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
+    z = rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias))
+    nm = {'sigmoid': 'logistic'}.get(name, name)
+    return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
+
+
 def layernorm(x, jac, lap, gamma, beta, eps):
     from oracle import backend as ob
 
@@ -164,7 +170,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'dense_act', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

@@ -363,3 +363,25 @@ def test_dot_row_slice(thr):
         return xp.add(xp.sum(a), xp.sum(b))
 
     check_against_oracle(fn, x, thr)
+
+
+@pytest.mark.parametrize('thr', [0, 3, 100])
+def test_dot_act(thr):
+    """``dot(h, W, b, act=...)`` equals the dense rule followed by the elementwise rule: on the
+    fused kernel's shapes (dense and sparse rows), past them (K not a multiple of 4), with a
+    union over the contracted axis and with a residual added after the activation."""
+    rng = np.random.default_rng(10)
+    W0 = rng.normal(size=(3, 8)).astype(np.float32)
+    W1 = rng.normal(size=(8, 8)).astype(np.float32) / 3
+    b1 = rng.normal(size=(8,)).astype(np.float32)
+    W2 = rng.normal(size=(6, 4)).astype(np.float32) / 3
+    W3 = rng.normal(size=(4, 5)).astype(np.float32) / 2
+    x = rng.normal(size=(2, 6, 3)).astype(np.float32)
+
+    def fn(xp, t):
+        h = xp.dot(t, W0, act='tanh')                               # K = 3: two rules
+        h = xp.dot(h, W1, b1, act='silu', residual=h)               # fused, rows pass through
+        g = xp.dot(xp.transpose(h, (1, 0)), W2, act='sigmoid')      # contraction over nodes: union frame
+        return xp.add(xp.sum(xp.dot(g, W3, act='softplus')), xp.sum(h))
+
+    check_against_oracle(fn, x, thr)

@@ -112,6 +112,58 @@ def test_dense(rows, P, Kd, N, bias):
     assert_triplet(got, ref, 'dense')
 
 
+DENSE_ACT_CASES = [
+    # (rows shape, P, K, N, bias, act)
+    ((20, 100), 400, 100, 100, True, 'silu'),   # README MLP hidden layer: Jacobian rows split over workgroups
+    ((20, 100), 400, 4, 100, True, 'silu'),     # its first layer (K = 4)
+    ((7, 100), 4, 100, 100, True, 'silu'),      # sparse storage of the same layer (4 rows)
+    ((3, 256), 6, 32, 32, True, 'tanh'),        # two-electron stream: 4 row strips, one column strip
+    ((1, 130), 5, 64, 64, False, 'tanh'),       # two column strips, ragged last row tile
+    ((2, 33), 9, 128, 128, True, 'softplus'),   # widest layer the kernel takes
+    ((1, 50), 17, 96, 20, True, 'logistic'),    # K / 4 even but not a power of two
+    ((1, 70), 3, 36, 33, True, 'exp'),          # K % 8 == 4, N just past one strip
+    ((1, 1), 0, 8, 1, False, 'sin'),            # no Jacobian rows, one row, one column
+    ((5, 40), 64, 16, 128, True, 'cos'),
+    ((2, 64), 31, 104, 100, False, 'square'),   # odd number of Jacobian rows
+    ((1, 64), 100, 100, 100, True, 'tanh'),     # one row tile, many groups
+]
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,bias,act', DENSE_ACT_CASES)
+def test_dense_act(rows, P, Kd, N, bias, act):
+    """Dense layer + activation as one kernel against the composition of the two oracle rules."""
+    from folx_amd import kernels as K
+
+    print(f'case dense_act rows={rows} P={P} K={Kd} N={N} act={act}', flush=True)
+    rng = np.random.default_rng(21)
+    x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    z = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
+    ref = rules.elementwise_rule(act, *z)
+    assert K.dense_act_supported(act, Kd, N)
+    for rep in range(2):  # the second call finds the counters as the first one left them
+        got = K.dense_act(act, dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
+        assert_triplet(got, ref, f'dense_act call {rep}')
+
+
+def test_dense_act_matches_two_kernels_large():
+    """At a full-size batch the fused kernel and dense + elementwise agree to rounding."""
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(5)
+    R, P, Kd, N = 256 * 100, 4, 100, 100
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.randn(R, Kd, device='cuda', generator=g)
+    W = torch.randn(Kd, N, device='cuda', generator=g) / 10
+    b = torch.randn(N, device='cuda', generator=g)
+    got = K.dense_act('silu', x, J, L, W, b)
+    ref = K.elementwise('silu', *K.dense(x, J, L, W, b))
+    for a, r, nm in zip(got, ref, ('x', 'jac', 'lap')):
+        torch.testing.assert_close(a, r, rtol=2e-5, atol=2e-5, msg=lambda m: f'{nm}: {m}')
+
+
 @pytest.mark.parametrize('lead,n,lo,hi,P,Kd,N', [((5,), 32, 0, 16, 9, 256, 256), ((5,), 32, 16, 32, 9, 256, 256),
                                                  ((2, 3), 7, 2, 5, 4, 48, 20), ((4,), 9, 1, 9, 3, 17, 33),
                                                  ((300,), 6, 3, 4, 2, 32, 64)])
