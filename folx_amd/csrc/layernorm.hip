@@ -7,10 +7,12 @@
 //   y_lap    = g r (lap - mean(lap) - c r^2 mean(c lap))                      (linear part)
 //            + g ( -2 r^3 sum_p b_p (u_p - a_p) + c (3 r^5 sum_p b_p^2 - r^3 sum_p s_p) )
 // which is what the chain mean / sub / square / mean / rsqrt / mul of elementwise and
-// reduction rules evaluates to.  One wavefront owns one row of F features and streams the
-// Jacobian rows once (read once, written once: 8 (P + 2) F bytes per row, HBM bound); the
-// three per-row means are butterfly reductions inside the wavefront, four Jacobian rows
-// in flight at a time.
+// reduction rules evaluates to.  A workgroup of 4 wavefronts owns one row of F features and
+// streams its Jacobian rows once (read once, written once: 8 (P + 2) F bytes per row, HBM
+// bound): wavefront w takes the Jacobian rows p = w, w + 4, ..., four of them in flight at a
+// time, so consecutive workgroups walk consecutive addresses of every Jacobian row.  The
+// three per-row means are butterfly reductions inside the wavefront; the sums over p meet
+// in LDS and wavefront 0 writes y and y_lap.
 #include "common.h"
 
 namespace {
@@ -29,16 +31,18 @@ __device__ __forceinline__ float wave_sum1(float a) {
   return a;
 }
 
-constexpr int ROWS_PER_BLOCK = 4;
+constexpr int PSPLIT = 4;
 
 template <int NV>
-__global__ __launch_bounds__(FOLX_WAVE * ROWS_PER_BLOCK) void layernorm_kernel(
+__global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
     const float* __restrict__ x, const float* __restrict__ jac, const float* __restrict__ lap,
     const float* __restrict__ gamma, const float* __restrict__ beta, float* __restrict__ y,
     float* __restrict__ y_jac, float* __restrict__ y_lap, int64_t R, int32_t F, int32_t P, float eps) {
+  __shared__ float4 redT[PSPLIT][NV * FOLX_WAVE];
+  __shared__ float reds[PSPLIT][2];
   const int lane = threadIdx.x % FOLX_WAVE;
-  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / FOLX_WAVE;
-  if (row >= R) return;
+  const int w = threadIdx.x / FOLX_WAVE;
+  const int64_t row = blockIdx.x;
   const int F4 = F / 4;
   const float invF = 1.0f / (float)F;
   const int64_t S = R * (int64_t)F;  // elements per Jacobian row
@@ -113,13 +117,13 @@ __global__ __launch_bounds__(FOLX_WAVE * ROWS_PER_BLOCK) void layernorm_kernel(
     }
   };
 
-  int p = 0;
-  for (; p + 3 < P; p += 4) {  // four Jacobian rows in flight per wavefront
+  int p = w;
+  for (; p + 3 * PSPLIT < P; p += 4 * PSPLIT) {  // four Jacobian rows in flight per wavefront
     float4 u0[NV], u1[NV], u2[NV], u3[NV];
     load_row(p, u0);
-    load_row(p + 1, u1);
-    load_row(p + 2, u2);
-    load_row(p + 3, u3);
+    load_row(p + PSPLIT, u1);
+    load_row(p + 2 * PSPLIT, u2);
+    load_row(p + 3 * PSPLIT, u3);
     float a1, a2, a3, b1, b2, b3, c1, c2, c3, e1, e2, e3;
     partial(u0, a1, a2, a3);
     partial(u1, b1, b2, b3);
@@ -130,17 +134,35 @@ __global__ __launch_bounds__(FOLX_WAVE * ROWS_PER_BLOCK) void layernorm_kernel(
     wave_sum3(c1, c2, c3);
     wave_sum3(e1, e2, e3);
     finish_row(p, u0, a1, a2, a3);
-    finish_row(p + 1, u1, b1, b2, b3);
-    finish_row(p + 2, u2, c1, c2, c3);
-    finish_row(p + 3, u3, e1, e2, e3);
+    finish_row(p + PSPLIT, u1, b1, b2, b3);
+    finish_row(p + 2 * PSPLIT, u2, c1, c2, c3);
+    finish_row(p + 3 * PSPLIT, u3, e1, e2, e3);
   }
-  for (; p < P; ++p) {
+  for (; p < P; p += PSPLIT) {
     float4 u0[NV];
     load_row(p, u0);
     float a1, a2, a3;
     partial(u0, a1, a2, a3);
     wave_sum3(a1, a2, a3);
     finish_row(p, u0, a1, a2, a3);
+  }
+
+  // the sums over p of the four wavefronts meet in LDS (this barrier also orders every
+  // wavefront's read of x before the write of y, which makes in-place use safe)
+#pragma unroll
+  for (int v = 0; v < NV; ++v) redT[w][v * FOLX_WAVE + lane] = T[v];
+  if (lane == 0) { reds[w][0] = sb2; reds[w][1] = ss; }
+  __syncthreads();
+  if (w != 0) return;
+  sb2 = reds[0][0]; ss = reds[0][1];
+#pragma unroll
+  for (int ww = 1; ww < PSPLIT; ++ww) {
+    sb2 += reds[ww][0]; ss += reds[ww][1];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const float4 t = redT[ww][v * FOLX_WAVE + lane];
+      T[v].x += t.x; T[v].y += t.y; T[v].z += t.z; T[v].w += t.w;
+    }
   }
 
   // value and Laplacian
@@ -190,10 +212,10 @@ extern "C" int folx_hip_layernorm_fwdlap(void* stream, const float* x, const flo
   const void* ptrs[] = {x, jac, lap, gamma, beta, y, y_jac, y_lap};
   for (const void* p : ptrs)
     if (p && !folx_aligned16(p)) return FOLX_HIP_ENOTSUP;
-  const int64_t blocks = (R + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+  const int64_t blocks = R;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)blocks), block(FOLX_WAVE * ROWS_PER_BLOCK);
+  dim3 grid((unsigned)blocks), block(FOLX_WAVE * PSPLIT);
   const int nv = (F / 4 + FOLX_WAVE - 1) / FOLX_WAVE;
   switch (nv) {
     case 1: layernorm_kernel<1><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); break;
