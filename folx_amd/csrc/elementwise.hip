@@ -47,7 +47,7 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void elementwise_kernel(
       for (int u = 0; u < UNROLL; ++u) {
         const float* src = jac + (int64_t)(p + u * PSPLIT) * S + e0;
         if constexpr (VEC == 4) {
-          float4 t = *reinterpret_cast<const float4*>(src);
+          float4 t = folx_ld_stream4(src);
           jv[u][0] = t.x; jv[u][1] = t.y; jv[u][2] = t.z; jv[u][3] = t.w;
         } else {
           jv[u][0] = *src;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void elementwise_kernel(
 #pragma unroll
         for (int v = 0; v < VEC; ++v) { o[v] = d1[v] * jv[u][v]; sq[v] += jv[u][v] * jv[u][v]; }
         if constexpr (VEC == 4) {
-          *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+          folx_st_stream4(dst, make_float4(o[0], o[1], o[2], o[3]));
         } else {
           *dst = o[0];
         }
@@ -70,9 +70,9 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void elementwise_kernel(
       const float* src = jac + (int64_t)p * S + e0;
       float* dst = y_jac + (int64_t)p * S + e0;
       if constexpr (VEC == 4) {
-        float4 t = *reinterpret_cast<const float4*>(src);
+        float4 t = folx_ld_stream4(src);
         sq[0] += t.x * t.x; sq[1] += t.y * t.y; sq[2] += t.z * t.z; sq[3] += t.w * t.w;
-        *reinterpret_cast<float4*>(dst) = make_float4(d1[0] * t.x, d1[1] * t.y, d1[2] * t.z, d1[3] * t.w);
+        folx_st_stream4(dst, make_float4(d1[0] * t.x, d1[1] * t.y, d1[2] * t.z, d1[3] * t.w));
       } else {
         float t = *src;
         sq[0] += t * t;

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
       u[v] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (ok[v]) u[v] = *reinterpret_cast<const float4*>(jac + (int64_t)p * S + off + 4 * (lane + FOLX_WAVE * v));
+      if (ok[v]) u[v] = folx_ld_stream4(jac + (int64_t)p * S + off + 4 * (lane + FOLX_WAVE * v));
     }
   };
   auto partial = [&](const float4* u, float& s1, float& s2, float& s3) {
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
         o.y = g[v].y * r * (dy - c[v].y * cb);
         o.z = g[v].z * r * (dz - c[v].z * cb);
         o.w = g[v].w * r * (dw - c[v].w * cb);
-        *reinterpret_cast<float4*>(y_jac + (int64_t)p * S + off + 4 * (lane + FOLX_WAVE * v)) = o;
+        folx_st_stream4(y_jac + (int64_t)p * S + off + 4 * (lane + FOLX_WAVE * v), o);
       }
     }
   };

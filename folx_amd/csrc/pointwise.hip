@@ -36,9 +36,10 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
     else if constexpr (OP == FOLX_BIN_MIN) { ca = av < bv ? 1.0f : (av == bv ? 0.5f : 0.0f); cb = 1.0f - ca; }
     else { ca = av > bv ? 1.0f : (av == bv ? 0.5f : 0.0f); cb = 1.0f - ca; }
     for (int p = w; p < P; p += PSPLIT) {
-      const float ja = aj[(int64_t)p * a_S + oa];
-      const float jb = bj[(int64_t)p * b_S + ob];
-      yj[(int64_t)p * S + i] = ca * ja + cb * jb;
+      // Jacobian rows are touched once per launch: streaming (non-temporal) accesses
+      const float ja = __builtin_nontemporal_load(&aj[(int64_t)p * a_S + oa]);
+      const float jb = __builtin_nontemporal_load(&bj[(int64_t)p * b_S + ob]);
+      __builtin_nontemporal_store(ca * ja + cb * jb, &yj[(int64_t)p * S + i]);
       if constexpr (OP == FOLX_BIN_MUL || OP == FOLX_BIN_DIV) sab += ja * jb;
       if constexpr (OP == FOLX_BIN_DIV) sbb += jb * jb;
     }
