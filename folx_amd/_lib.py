@@ -39,6 +39,7 @@ SIGNATURES = {
     'folx_hip_inv_fwdlap': (c_int, [_P] * 7 + [c_int64, c_int32, c_int32]),
     'folx_hip_solve_fwdlap': (c_int, [_P] * 10 + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_mhsa_fwdlap': (c_int, [_P] * 15 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
+    'folx_hip_mhsa_sparse_fwdlap': (c_int, [_P] * 14 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
     'folx_hip_mhsea_fwdlap': (c_int, [_P] * 18 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
 }
 

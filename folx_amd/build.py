@@ -28,6 +28,7 @@ SOURCES = [
     'gather.hip',
     'slogdet.hip',
     'mhsa.hip',
+    'mhsa_sparse.hip',
     'layernorm.hip',
     'linsolve.hip',
 ]

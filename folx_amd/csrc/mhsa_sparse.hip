@@ -1,0 +1,358 @@
+// Multi-head self attention with Laplacian for q, k, v whose Jacobians are still sparse by
+// position: sequence position e depends on its own few input coordinates only (the first
+// attention layer of a PsiFormer, where the inputs of electron e are its three coordinates),
+// so the dense Jacobian row c = index[s][e] of q, k and v is zero except in row e.
+// The output is dense (every output position depends on every electron), but with
+//   a = q'_c[e], b = k'_c[e], w = v'_c[e]     alpha[j] = a . k[j]     beta[i] = q[i] . b
+// the rule of the dense kernel (s'_c = q'_c k^T + q k'_c^T, p'_c = p * (s'_c - rowsum(p s'_c)),
+// o'_c = p v'_c + p'_c v, ...) collapses to vector work per Jacobian row:
+//   s'_c[i][j] = [i = e] alpha[j] + beta[i] [j = e]
+//   r_c[i]     = [i = e] rho + p[i][e] beta[i],            rho = sum_j p[e][j] alpha[j]
+//   o'_c[i]    = p[i][e] (w + beta[i] (v[e] - o[i])) + [i = e] (gamma - rho o[e]),
+//                gamma = sum_j p[e][j] alpha[j] v[j]
+// and the second-order part of the Laplacian needs, besides n x n sums of squares of alpha and
+// beta, a single n x n x d product:
+//   lap_o = p lap_v + (pL + M) v + 2 sum_c p'_c[:, e] w_c
+//   M     = p * (T2 - rowsum(p T2) + 2 g (I - diag(p))),   T2 = sum_c (s'_c - r_c)^2,
+//   g[e]  = sum_s a_s . b_s,   pL = p * (sL - rowsum(p sL)),   sL = lap_q k^T + q lap_k^T.
+// That is O(n^2 d) work per (walker, head) instead of O(P n^2 d); the kernel is bound by
+// writing the dense P x n x d output rows.
+//
+// One workgroup of 256 threads per (walker, head); q, k, v, o, p and the n x n accumulators
+// live in LDS (rows of d + 4 floats, so that 16 threads reading 16 bytes each from 16
+// different rows cover all banks); dot products run on 128-bit LDS reads; the three vectors of
+// the next position are fetched while the current one is worked on.
+#include "common.h"
+
+namespace {
+
+struct SAArgs {
+  const float *q, *qs, *ql, *k, *ks, *kl, *v, *vs, *vl;
+  const int32_t* index;  // [K][n] dense Jacobian row of slot s at position e, or -1
+  float *o, *oj, *ol;
+  int64_t B;
+  int32_t n, H, d, K;
+};
+
+constexpr int SA_NT = 256;
+
+// dot product of two 16-byte aligned LDS vectors of 4 * d4 floats
+__device__ __forceinline__ float sa_dot(const float* u, const float* m, int d4) {
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll 4
+  for (int t = 0; t < d4; ++t) {
+    const float4 x = *reinterpret_cast<const float4*>(u + 4 * t);
+    const float4 y = *reinterpret_cast<const float4*>(m + 4 * t);
+    s0 += x.x * y.x; s1 += x.y * y.y; s2 += x.z * y.z; s3 += x.w * y.w;
+  }
+  return (s0 + s1) + (s2 + s3);
+}
+constexpr int SA_MAXPASS = 4;  // n <= 64: rows i = 16 pass + tid / 16
+
+__host__ __device__ inline int64_t sa_lds_floats(int n, int d, int K) {
+  const int dp = d + 4, np1 = n + 1;
+  return 4LL * n * dp + 4LL * n * np1 + 4LL * K * d + 2LL * K * n + 8 + 5LL * n + 8;
+}
+
+__global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const int n = a.n, d = a.d, K = a.K, H = a.H;
+  const int dp = d + 4, np1 = n + 1, d4 = d / 4;
+  float* qS = sm;
+  float* kS = qS + n * dp;
+  float* vS = kS + n * dp;
+  float* oS = vS + n * dp;
+  float* pS = oS + n * dp;
+  float* AA = pS + n * np1;
+  float* BB = AA + n * np1;
+  float* AR = BB + n * np1;
+  float* aS = AR + n * np1;
+  float* bS = aS + K * d;
+  float* wS = bS + K * d;
+  float* gamS = wS + K * d;
+  float* alS = gamS + K * d;
+  float* beS = alS + K * n;
+  float* rhoS = beS + K * n;
+  float* D1 = rhoS + 8;
+  float* D2 = D1 + n;
+  float* R2a = D2 + n;
+  float* gS = R2a + n;
+  float* rsum = gS + n;
+  int* cS = reinterpret_cast<int*>(rsum + n);  // dense rows of the current position's slots
+
+  const int tid = threadIdx.x;
+  const int64_t b = blockIdx.x / H;
+  const int h = (int)(blockIdx.x % H);
+  const int64_t Srow = a.B * n * (int64_t)H * d;  // elements per Jacobian row
+  auto grow = [&](int i) -> int64_t { return ((b * n + i) * (int64_t)H + h) * d; };
+  auto load_tile = [&](const float* src, float* dst) {
+    for (int it = tid; it < n * d4; it += SA_NT) {
+      const int i = it / d4, t4 = it - i * d4;
+      const float4 t = *reinterpret_cast<const float4*>(src + grow(i) + 4 * t4);
+      *reinterpret_cast<float4*>(dst + i * dp + 4 * t4) = t;
+    }
+  };
+
+  load_tile(a.q, qS);
+  load_tile(a.k, kS);
+  load_tile(a.v, vS);
+  for (int it = tid; it < 3 * n * np1; it += SA_NT) AA[it] = 0.0f;  // AA, BB, AR are contiguous
+  __syncthreads();
+
+  // p = softmax(q k^T)
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    pS[i * np1 + j] = sa_dot(qS + i * dp, kS + j * dp, d4);
+  }
+  __syncthreads();
+  if (tid < n) {
+    float* row = pS + tid * np1;
+    float m = row[0];
+    for (int j = 1; j < n; ++j) m = fmaxf(m, row[j]);
+    float z = 0.0f;
+    for (int j = 0; j < n; ++j) { const float ex = expf(row[j] - m); row[j] = ex; z += ex; }
+    const float rz = 1.0f / z;
+    for (int j = 0; j < n; ++j) row[j] *= rz;
+  }
+  __syncthreads();
+  // o = p v
+  for (int it = tid; it < n * d4; it += SA_NT) {
+    const int i = it / d4, t4 = it - i * d4;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
+    for (int j = 0; j < n; ++j) {
+      const float pij = pS[i * np1 + j];
+      const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * t4);
+      acc.x += pij * vv.x; acc.y += pij * vv.y; acc.z += pij * vv.z; acc.w += pij * vv.w;
+    }
+    *reinterpret_cast<float4*>(oS + i * dp + 4 * t4) = acc;
+    *reinterpret_cast<float4*>(a.o + grow(i) + 4 * t4) = acc;
+  }
+
+  // the three vectors (a, b, w) of every slot of one position: one float4 per thread
+  const int nvec = 3 * K * d4;
+  const int pf_which = tid / (K * d4), pf_sl = (tid / d4) % K, pf_t4 = tid % d4;
+  auto fetch = [&](int e) -> float4 {
+    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tid < nvec && a.index[pf_sl * n + e] >= 0) {
+      const float* src = pf_which == 0 ? a.qs : (pf_which == 1 ? a.ks : a.vs);
+      r = *reinterpret_cast<const float4*>(src + pf_sl * Srow + grow(e) + 4 * pf_t4);
+    }
+    return r;
+  };
+  float4 pf = fetch(0);
+
+  float4 t2acc[SA_MAXPASS];
+#pragma unroll
+  for (int ps = 0; ps < SA_MAXPASS; ++ps) t2acc[ps] = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int orow = tid / 16, ot4 = tid % 16;
+
+  for (int e = 0; e < n; ++e) {
+    __syncthreads();  // everyone is done with the previous position's vectors (and with o, p on entry)
+    if (tid < nvec) {
+      float* dst = (pf_which == 0 ? aS : (pf_which == 1 ? bS : wS)) + pf_sl * d + 4 * pf_t4;
+      *reinterpret_cast<float4*>(dst) = pf;
+    }
+    if (tid < K) cS[tid] = a.index[tid * n + e];
+    __syncthreads();
+    if (e + 1 < n) pf = fetch(e + 1);
+
+    // alpha[s][j] = a_s . k[j],  beta[s][i] = q[i] . b_s
+    for (int it = tid; it < 2 * K * n; it += SA_NT) {
+      const int which = it / (K * n), sl = (it / n) % K, x = it % n;
+      const float* u = (which == 0 ? aS : bS) + sl * d;
+      const float* m = (which == 0 ? kS : qS) + x * dp;
+      (which == 0 ? alS : beS)[sl * n + x] = sa_dot(u, m, d4);
+    }
+    __syncthreads();
+    // rho[s] = sum_j p[e][j] alpha[s][j],  gamma[s] = sum_j p[e][j] alpha[s][j] v[j]
+    for (int it = tid; it < K * d4; it += SA_NT) {
+      const int sl = it / d4, t4 = it - sl * d4;
+      float rho = 0.0f;
+      float4 gm = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
+      for (int j = 0; j < n; ++j) {
+        const float pa = pS[e * np1 + j] * alS[sl * n + j];
+        const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * t4);
+        rho += pa;
+        gm.x += pa * vv.x; gm.y += pa * vv.y; gm.z += pa * vv.z; gm.w += pa * vv.w;
+      }
+      *reinterpret_cast<float4*>(gamS + sl * d + 4 * t4) = gm;
+      if (t4 == 0) rhoS[sl] = rho;
+    }
+    __syncthreads();
+
+    // output rows of this position's slots, and their part of 2 sum_c p'_c[:, e] w_c
+    for (int sl = 0; sl < K; ++sl) {
+      const int c = cS[sl];
+      if (c < 0) continue;
+      const float rho = rhoS[sl];
+      const float ale = alS[sl * n + e];
+      if (ot4 < d4) {
+        const float4 w4 = *reinterpret_cast<const float4*>(wS + sl * d + 4 * ot4);
+        const float4 g4 = *reinterpret_cast<const float4*>(gamS + sl * d + 4 * ot4);
+        const float4 v4 = *reinterpret_cast<const float4*>(vS + e * dp + 4 * ot4);
+        const float4 o4 = *reinterpret_cast<const float4*>(oS + e * dp + 4 * ot4);
+        const float wv[4] = {w4.x, w4.y, w4.z, w4.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
+        const float ve[4] = {v4.x, v4.y, v4.z, v4.w}, oe[4] = {o4.x, o4.y, o4.z, o4.w};
+#pragma unroll
+        for (int ps = 0; ps < SA_MAXPASS; ++ps) {
+          const int i = ps * 16 + orow;
+          if (i < n) {
+            const float pie = pS[i * np1 + e];
+            const float bi = beS[sl * n + i];
+            const float4 oi4 = *reinterpret_cast<const float4*>(oS + i * dp + 4 * ot4);
+            const float oi[4] = {oi4.x, oi4.y, oi4.z, oi4.w};
+            float r[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+              r[x] = pie * (wv[x] + bi * (ve[x] - oi[x]));
+              if (i == e) r[x] += gv[x] - rho * oe[x];
+            }
+            folx_st_stream4(a.oj + (int64_t)c * Srow + grow(i) + 4 * ot4, make_float4(r[0], r[1], r[2], r[3]));
+            float cf = pie * bi * (1.0f - pie);
+            if (i == e) cf += pie * (ale - rho);
+            t2acc[ps].x += cf * wv[0]; t2acc[ps].y += cf * wv[1];
+            t2acc[ps].z += cf * wv[2]; t2acc[ps].w += cf * wv[3];
+          }
+        }
+      }
+    }
+    // n x n sums over this position's slots
+    if (tid < n) {
+      const int j = tid;
+      const float pee = pS[e * np1 + e];
+      float aa = 0.0f, ar = 0.0f, bb = 0.0f;
+      for (int sl = 0; sl < K; ++sl) {
+        const float al = alS[sl * n + j], be = beS[sl * n + j];
+        const float rr = rhoS[sl] + pee * beS[sl * n + e];
+        aa += al * al;
+        ar += al * rr;
+        bb += be * be;
+      }
+      AA[e * np1 + j] = aa;
+      AR[e * np1 + j] = ar;
+      BB[j * np1 + e] = bb;
+    }
+    if (tid == SA_NT - 1) {
+      const float pee = pS[e * np1 + e];
+      float d1 = 0.0f, d2 = 0.0f, r2 = 0.0f, g = 0.0f;
+      for (int sl = 0; sl < K; ++sl) {
+        const float ale = alS[sl * n + e], bee = beS[sl * n + e], rho = rhoS[sl];
+        d1 += 2.0f * ale * bee;
+        d2 += bee * rho;
+        r2 += rho * rho + 2.0f * rho * pee * bee;
+        g += sa_dot(aS + sl * d, bS + sl * d, d4);
+      }
+      D1[e] = d1; D2[e] = d2; R2a[e] = r2; gS[e] = g;
+    }
+  }
+  __syncthreads();
+
+  // T2 = S2 - 2 SR + R2, then M (kept in AA)
+  if (tid < n) {
+    const int i = tid;
+    float r2 = R2a[i];
+    for (int e = 0; e < n; ++e) { const float pe = pS[i * np1 + e]; r2 += pe * pe * BB[i * np1 + e]; }
+    R2a[i] = r2;
+  }
+  __syncthreads();
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    const int x = i * np1 + j;
+    float s2 = AA[x] + BB[x], sr = AR[x] + pS[x] * BB[x];
+    if (i == j) { s2 += D1[i]; sr += D2[i]; }
+    AA[x] = s2 - 2.0f * sr + R2a[i];
+  }
+  load_tile(a.ql, oS);  // o is not needed any more
+  __syncthreads();
+  if (tid < n) {
+    const int i = tid;
+    float s = 0.0f;
+    for (int j = 0; j < n; ++j) s += pS[i * np1 + j] * AA[i * np1 + j];
+    rsum[i] = s;
+  }
+  // sL = lap_q k^T (into BB, whose sums of beta^2 are used up)
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    BB[i * np1 + j] = sa_dot(oS + i * dp, kS + j * dp, d4);
+  }
+  __syncthreads();
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    const int x = i * np1 + j;
+    const float pij = pS[x];
+    AA[x] = pij * (AA[x] - rsum[i] + 2.0f * gS[i] * ((i == j ? 1.0f : 0.0f) - pS[i * np1 + i]));
+  }
+  load_tile(a.kl, oS);  // lap_q has been consumed; k itself is not needed any more
+  __syncthreads();
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    BB[i * np1 + j] += sa_dot(qS + i * dp, oS + j * dp, d4);
+  }
+  __syncthreads();
+  if (tid < n) {
+    const int i = tid;
+    float s = 0.0f;
+    for (int j = 0; j < n; ++j) s += pS[i * np1 + j] * BB[i * np1 + j];
+    rsum[i] = s;
+  }
+  load_tile(a.vl, qS);  // q is not needed any more
+  __syncthreads();
+  for (int it = tid; it < n * n; it += SA_NT) {
+    const int i = it / n, j = it - i * n;
+    const int x = i * np1 + j;
+    AA[x] += pS[x] * (BB[x] - rsum[i]);  // pL + M
+  }
+  __syncthreads();
+  // lap_o = p lap_v + (pL + M) v + 2 sum_c p'_c[:, e] w_c
+  if (ot4 < d4) {
+#pragma unroll
+    for (int ps = 0; ps < SA_MAXPASS; ++ps) {
+      const int i = ps * 16 + orow;
+      if (i < n) {
+        float r[4] = {2.0f * t2acc[ps].x, 2.0f * t2acc[ps].y, 2.0f * t2acc[ps].z, 2.0f * t2acc[ps].w};
+#pragma unroll 4
+        for (int j = 0; j < n; ++j) {
+          const float pij = pS[i * np1 + j], mij = AA[i * np1 + j];
+          const float4 vl = *reinterpret_cast<const float4*>(qS + j * dp + 4 * ot4);
+          const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * ot4);
+          r[0] += pij * vl.x + mij * vv.x; r[1] += pij * vl.y + mij * vv.y;
+          r[2] += pij * vl.z + mij * vv.z; r[3] += pij * vl.w + mij * vv.w;
+        }
+        *reinterpret_cast<float4*>(a.ol + grow(i) + 4 * ot4) = make_float4(r[0], r[1], r[2], r[3]);
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int folx_hip_mhsa_sparse_fwdlap(void* stream, const float* q, const float* q_jac, const float* q_lap,
+                                           const float* k, const float* k_jac, const float* k_lap, const float* v,
+                                           const float* v_jac, const float* v_lap, const int32_t* index, float* o,
+                                           float* o_jac, float* o_lap, int64_t B, int32_t n, int32_t H, int32_t d,
+                                           int32_t k_rows) {
+  if (B < 0 || n <= 0 || H <= 0 || d <= 0 || k_rows <= 0) return FOLX_HIP_EINVAL;
+  if (B == 0) return FOLX_HIP_OK;
+  if (!q || !q_jac || !q_lap || !k || !k_jac || !k_lap || !v || !v_jac || !v_lap || !index || !o || !o_jac || !o_lap)
+    return FOLX_HIP_EINVAL;
+  if (n > 16 * SA_MAXPASS || d > 64 || d % 4 != 0 || k_rows > 8 || 3 * k_rows * (d / 4) > SA_NT)
+    return FOLX_HIP_ENOTSUP;
+  const void* ptrs[] = {q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, o, o_jac, o_lap};
+  for (const void* p : ptrs)
+    if (!folx_aligned16(p)) return FOLX_HIP_ENOTSUP;
+  if (B * H > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  const size_t lds = (size_t)sa_lds_floats(n, d, k_rows) * sizeof(float);
+  if (lds > 160 * 1024) return FOLX_HIP_ENOTSUP;
+  if (lds > 64 * 1024) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(mhsa_sparse_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return FOLX_HIP_ENOTSUP;
+  }
+  SAArgs a;
+  a.q = q; a.qs = q_jac; a.ql = q_lap; a.k = k; a.ks = k_jac; a.kl = k_lap; a.v = v; a.vs = v_jac; a.vl = v_lap;
+  a.index = index; a.o = o; a.oj = o_jac; a.ol = o_lap; a.B = B; a.n = n; a.H = H; a.d = d; a.K = k_rows;
+  mhsa_sparse_kernel<<<dim3((unsigned)(B * H)), dim3(SA_NT), lds, (hipStream_t)stream>>>(a);
+  return folx_launch_status();
+}

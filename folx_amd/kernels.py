@@ -467,3 +467,29 @@ def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None)
             'mhsa_fwdlap',
         )
     return o, oj, ol
+
+
+def mhsa_sparse_supported(n, d, k_rows):
+    """Shapes the position-sparse attention kernel is built for."""
+    return n <= 64 and d <= 64 and d % 4 == 0 and 1 <= k_rows <= 8 and 3 * k_rows * (d // 4) <= 256
+
+
+def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
+    """Attention rule for q, k, v (B, n, H, d) whose Jacobians ``*s`` (k_rows, B, n, H, d) are
+    sparse by position; ``index`` int32 (k_rows, n) on the device names the dense row of each
+    slot.  Returns the triplet with a dense ``(P, B, n, H, d)`` Jacobian."""
+    _chk(q, qs, ql, k, ks, kl, v, vs, vl, index)
+    B, n, H, d = q.shape
+    k_rows = qs.shape[0]
+    assert tuple(index.shape) == (k_rows, n) and index.dtype == torch.int32
+    o, ol = torch.empty_like(q), torch.empty_like(q)
+    oj = (torch.empty if all_rows_named else torch.zeros)((P, B, n, H, d), device=q.device, dtype=torch.float32)
+    with _timed('mhsa_sparse_fwdlap', (B, n, H, d, k_rows, P)):
+        check(
+            _lib.load().folx_hip_mhsa_sparse_fwdlap(
+                _stream(), _p(q), _p(qs), _p(ql), _p(k), _p(ks), _p(kl), _p(v), _p(vs), _p(vl),
+                _p(index), _p(o), _p(oj), _p(ol), B, n, H, d, k_rows,
+            ),
+            'mhsa_sparse_fwdlap',
+        )
+    return o, oj, ol

@@ -1262,6 +1262,33 @@ def _mask_tensor(m, shape, device):
     return t.expand(*shape).contiguous()
 
 
+def _position_sparse_index(q, k, v):
+    """``(index (k, n) int32, P, all_rows_named)`` when q, k, v (per-walker shape (n, H, d)) carry
+    the same sparse Jacobian mask, constant over heads and features, in which no input index
+    belongs to two sequence positions -- the structure the position-sparse attention kernel
+    takes; None otherwise (the Jacobians are then materialised as in the reference)."""
+    masks = [t.jacobian.x0_idx for t in (q, k, v)]
+    if any(m is None for m in masks) or q.ndim != 3:
+        return None
+    m0 = np.broadcast_to(masks[0], (masks[0].shape[0], *q.shape))
+    for t, m in zip((k, v), masks[1:]):
+        if m.shape[0] != m0.shape[0] or tuple(t.shape) != tuple(q.shape):
+            return None
+        if not np.array_equal(np.broadcast_to(m, m0.shape), m0):
+            return None
+    index = np.ascontiguousarray(m0[:, :, 0, 0]).astype(np.int32)
+    if not (m0 == index[:, :, None, None]).all():
+        return None
+    n, _, d = q.shape
+    if not K.mhsa_sparse_supported(n, d, index.shape[0]):
+        return None
+    valid = index[index >= 0]
+    if valid.size == 0 or np.unique(valid).size != valid.size:
+        return None
+    P = int(valid.max()) + 1
+    return index, P, bool(valid.size == P)
+
+
 def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
     """Rule of ``multi_head_self_attention`` (``mhsa_forward_laplacian``,
     folx/experimental/pallas/attention/forward_laplacian.py:27-179).
@@ -1278,6 +1305,14 @@ def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
         raise NotImplementedError('multi_head_self_attention needs derivative-carrying q, k, v')
     B, dev = q.B, q.x.device
     n = q.shape[0]
+    if bias is None and mask is None and input_mask is None:
+        sparse = _position_sparse_index(q, k, v)
+        if sparse is not None:
+            index, P, all_named = sparse
+            o, oj, ol = K.mhsa_sparse(
+                q.x, q.jacobian.data, q.laplacian, k.x, k.jacobian.data, k.laplacian, v.x, v.jacobian.data,
+                v.laplacian, so.device_table(index, dev), P, all_named)
+            return FwdLaplArray(o, FwdJacobian(oj, None), ol)
     trip = (q, k, v) if bias is None else (q, k, v, bias)
     Js = [t.jacobian.dense_array for t in trip]
     P = max(J.shape[0] for J in Js)

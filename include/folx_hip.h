@@ -333,6 +333,27 @@ int folx_hip_mhsa_fwdlap(void* stream, const float* q, const float* q_jac, const
                          int32_t d, int32_t P);
 
 /*
+ * The same attention rule (no masks, no edge bias) for q, k, v whose Jacobians are still
+ * sparse by position: sequence position e depends on at most k_rows input coordinates of its
+ * own, index[s][e] (int32 [k_rows][n], shared by all walkers and heads, -1 = empty slot)
+ * naming the dense Jacobian row that slot s of position e stands for; no dense row may be
+ * named twice.  What folx reaches by materialising the three Jacobians first
+ * (folx/experimental/pallas/attention/forward_laplacian.py:166-178 on top of
+ * FwdJacobian.dense_array, folx/api.py:182-190) -- here the zero rows are never built and the
+ * per-row n x n x d products collapse to vector work.
+ *   q, k, v [B][n][H][d]   *_jac [k_rows][B][n][H][d]   *_lap [B][n][H][d]
+ *   o [B][n][H][d]   o_jac [P][B][n][H][d] (dense; only the rows named in index are written,
+ *   the caller zero-fills the others)   o_lap [B][n][H][d]
+ * Built for n <= 64, d <= 64 with d % 4 == 0, k_rows <= 8; FOLX_HIP_ENOTSUP otherwise.
+ */
+int folx_hip_mhsa_sparse_fwdlap(void* stream, const float* q, const float* q_jac,
+                                const float* q_lap, const float* k, const float* k_jac,
+                                const float* k_lap, const float* v, const float* v_jac,
+                                const float* v_lap, const int32_t* index, float* o, float* o_jac,
+                                float* o_lap, int64_t B, int32_t n, int32_t H, int32_t d,
+                                int32_t k_rows);
+
+/*
  * Edge-bias variant: o = softmax(q k^T + e) v with e, e_lap [B][n][H][n], e_jac [P][B][n][H][n]
  * (argument order q, k, e, v as in the reference's rule).  Replaces mhsea_forward_laplacian
  * and its Pallas kernel (folx/experimental/pallas/attention/forward_laplacian.py:495-614,

@@ -166,11 +166,27 @@ def mhsa(q, qj, ql, k, kj, kl, v, vj, vl, mask=None, input_mask=None, edge=None)
     return tuple(_t(a) for a in rules.mhsa_rule(*[_n(t) for t in (q, qj, ql, k, kj, kl, v, vj, vl)], m, im, *ed))
 
 
+def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
+    ix = index.cpu().numpy()
+
+    def dense(xs):
+        xs = _n(xs)
+        J = np.zeros((P, *xs.shape[1:]))
+        for s in range(ix.shape[0]):
+            for e in range(ix.shape[1]):
+                if ix[s, e] >= 0:
+                    J[ix[s, e], :, e] = xs[s, :, e]
+        return J
+
+    return tuple(_t(a) for a in rules.mhsa_rule(_n(q), dense(qs), _n(ql), _n(k), dense(ks), _n(kl),
+                                                _n(v), dense(vs), _n(vl)))
+
+
 def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
     for name in ('dense', 'dense_act', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
-                 'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa'):
+                 'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

@@ -385,3 +385,33 @@ def test_dot_act(thr):
         return xp.add(xp.sum(xp.dot(g, W3, act='softplus')), xp.sum(h))
 
     check_against_oracle(fn, x, thr)
+
+
+def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
+    """q, k, v of the first PsiFormer layer still carry per-electron sparse Jacobians: the rule
+    hands them to the position-sparse kernel and the result equals the densified rule."""
+    import folx_amd
+    from folx_amd import kernels as K
+    from folx_amd import numpy as fnp
+    from folx_amd import wrapped_functions as wf
+    from oracle import backend as ob
+
+    calls = []
+    orig = K.mhsa_sparse
+    monkeypatch.setattr(K, 'mhsa_sparse', lambda *a: (calls.append(a[9].shape), orig(*a))[1])
+    rng = np.random.default_rng(13)
+    n, H, d = 4, 2, 4
+    Wq, Wk, Wv = (rng.normal(size=(3, H * d)).astype(np.float32) for _ in range(3))
+    x = rng.normal(size=(2, n, 3)).astype(np.float32)
+
+    def fn(xp, r):
+        q = xp.reshape(xp.dot(r, Wq), (n, H, d))
+        k = xp.reshape(xp.dot(r, Wk), (n, H, d))
+        v = xp.reshape(xp.dot(r, Wv), (n, H, d))
+        return xp.sum(xp.multi_head_self_attention(q, k, v))
+
+    check_against_oracle(fn, x, 6)
+    assert calls == [(3, n)]
+    calls.clear()
+    check_against_oracle(fn, x, 0)      # dense Jacobians: the ordinary kernel
+    assert calls == []

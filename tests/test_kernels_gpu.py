@@ -389,6 +389,46 @@ def test_mhsa(B, n, H, d, P, valid):
             assert torch.equal(g1, g2)
 
 
+@pytest.mark.parametrize('B,n,H,d,k,missing', [(3, 32, 4, 64, 3, False), (2, 7, 2, 8, 3, True), (1, 64, 1, 64, 3, False),
+                                              (2, 16, 2, 32, 6, False), (2, 5, 3, 12, 1, False), (1, 33, 2, 60, 2, True)])
+def test_mhsa_sparse(B, n, H, d, k, missing):
+    """Attention with position-sparse Jacobians against the dense rule of the oracle on the
+    materialised Jacobians, and against the dense kernel."""
+    from folx_amd import kernels as K
+
+    print(f'case mhsa_sparse B={B} n={n} H={H} d={d} k={k} missing={missing}', flush=True)
+    rng = np.random.default_rng(12)
+    index = rng.permutation(n * k).reshape(k, n).astype(np.int32)   # every dense row named once
+    P = n * k
+    if missing:
+        index[k - 1, n // 2] = -1      # an empty slot: its dense row stays zero
+        index[0, 0] = -1
+    sig = [1 / np.sqrt(d), 1.0, 1.0]
+    vals, sparse, laps, dense = [], [], [], []
+    for s in sig:
+        vals.append(s * rand(rng, B, n, H, d))
+        js = s * rand(rng, k, B, n, H, d)
+        sparse.append(js)
+        laps.append(s * rand(rng, B, n, H, d))
+        J = np.zeros((P, B, n, H, d), dtype=np.float32)
+        for sl in range(k):
+            for e in range(n):
+                if index[sl, e] >= 0:
+                    J[index[sl, e], :, e] = js[sl, :, e]
+        dense.append(J)
+    ref = rules.mhsa_rule(*f64(vals[0], dense[0], laps[0], vals[1], dense[1], laps[1], vals[2], dense[2], laps[2]))
+    assert K.mhsa_sparse_supported(n, d, k)
+    got = K.mhsa_sparse(dev(vals[0]), dev(sparse[0]), dev(laps[0]), dev(vals[1]), dev(sparse[1]), dev(laps[1]),
+                        dev(vals[2]), dev(sparse[2]), dev(laps[2]), dev(index, torch.int32), P, not missing)
+    assert_val(got[0], ref[0], 'o')
+    assert_val(got[1], ref[1], 'o_jac')
+    assert_lap(got[2], ref[2], 'o_lap')
+    full = K.mhsa(dev(vals[0]), dev(dense[0]), dev(laps[0]), dev(vals[1]), dev(dense[1]), dev(laps[1]),
+                  dev(vals[2]), dev(dense[2]), dev(laps[2]), None, None)
+    assert_val(got[1], full[1].double().cpu().numpy(), 'o_jac vs dense kernel')
+    assert_lap(got[2], full[2].double().cpu().numpy(), 'o_lap vs dense kernel')
+
+
 @pytest.mark.parametrize('rows,F,P', [((3, 5), 8, 4), ((2, 32), 256, 9), ((7,), 512, 3), ((4, 3), 100, 5),
                                       ((2, 2), 1024, 2), ((5,), 4, 1)])
 def test_layernorm(rows, F, P):
