@@ -10,7 +10,7 @@ written with).  All arithmetic runs in ``libfolx_hip.so``; there is no CPU path.
 from .api import BatchedArray, FunctionFlags, FwdJacobian, FwdLaplArray
 from .graph import jit
 from .interpreter import forward_laplacian, init_forward_laplacian_state
-from .operators import ForwardLaplacianOperator
+from .operators import ForwardLaplacianOperator, LoopLaplacianOperator, ParallelLaplacianOperator
 from .vmap import batched_vmap, vmap
 from .wrapped_functions import deregister_function, get_laplacian, is_registered, register_function
 
@@ -22,6 +22,8 @@ __all__ = [
     'ForwardLaplacianOperator',
     'batched_vmap',
     'deregister_function',
+    'LoopLaplacianOperator',
+    'ParallelLaplacianOperator',
     'forward_laplacian',
     'get_laplacian',
     'init_forward_laplacian_state',

@@ -15,6 +15,8 @@ nothing but kernel nodes and device-to-device copies.
 
 from __future__ import annotations
 
+import gc
+
 import torch
 
 from .api import BatchedArray, FwdJacobian, FwdLaplArray
@@ -57,8 +59,20 @@ class _Captured:
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            out = fn(self.static_in)
+        # No finalizer may run while the capture is open: a dead reference cycle that still owns
+        # an older graph (or its memory pool) would destroy it through HIP calls that are not
+        # allowed during a capture and end the process.  Such cycles are collected now, and the
+        # collector stays off until the capture is closed (torch.cuda.graph itself no longer
+        # collects before capturing).
+        gc.collect()
+        gc_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                out = fn(self.static_in)
+        finally:
+            if gc_on:
+                gc.enable()
         self.tensors, self.rebuild = _flatten(out)
 
     def __call__(self, x):
@@ -68,26 +82,34 @@ class _Captured:
         return self.rebuild([t.clone() for t in self.tensors])
 
 
-def jit(fn):
-    """Wrap ``fn(x) -> FwdLaplArray | tensors`` (``x`` a device tensor with the walker axis
-    first, e.g. ``vmap(forward_laplacian(f, thr))``) so that repeated calls with the same
-    input shape replay one HIP graph.  The first call per shape runs eagerly."""
-    captured: dict = {}
-    seen: set = set()
+class _Jitted:
+    """Callable returned by ``jit``; an object rather than a function carrying itself as an
+    attribute, so that dropping it frees its graphs at once (no reference cycle)."""
 
-    def wrapped(x):
+    def __init__(self, fn):
+        self.eager = fn
+        self._captured: dict = {}
+        self._seen: set = set()
+
+    def __call__(self, x):
         if not isinstance(x, torch.Tensor):
             x = torch.as_tensor(x, dtype=torch.float32)
         x = x.to(device='cuda', dtype=torch.float32).contiguous()
         key = tuple(x.shape)
-        if key in captured:
-            return captured[key](x)
-        if key not in seen:
-            seen.add(key)
-            return fn(x)
-        captured[key] = _Captured(fn, x)
-        return captured[key](x)
+        if key in self._captured:
+            return self._captured[key](x)
+        if key not in self._seen:
+            self._seen.add(key)
+            return self.eager(x)
+        self._captured[key] = _Captured(self.eager, x)
+        return self._captured[key](x)
 
-    wrapped.batched = wrapped
-    wrapped.eager = fn
-    return wrapped
+    def batched(self, x):
+        return self(x)
+
+
+def jit(fn):
+    """Wrap ``fn(x) -> FwdLaplArray | tensors`` (``x`` a device tensor with the walker axis
+    first, e.g. ``vmap(forward_laplacian(f, thr))``) so that repeated calls with the same
+    input shape replay one HIP graph.  The first call per shape runs eagerly."""
+    return _Jitted(fn)

@@ -415,3 +415,37 @@ def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
     calls.clear()
     check_against_oracle(fn, x, 0)      # dense Jacobians: the ordinary kernel
     assert calls == []
+
+
+@pytest.mark.parametrize('parallel', [False, True])
+def test_loop_and_parallel_operators(parallel):
+    """folx/operators.py:41-79: the Hessian diagonal and the gradient of a scalar function,
+    one pass per coordinate (or all of them stacked along the walker axis); their sum is the
+    forward Laplacian (test/test_operator.py:19-73) and they match AD in float64."""
+    from bruteforce import plain
+
+    rng = np.random.default_rng(14)
+    W1 = rng.normal(size=(3, 5)).astype(np.float32)
+    W2 = rng.normal(size=(5, 4)).astype(np.float32) / 2
+    x = rng.normal(size=(3, 4, 3)).astype(np.float32)
+
+    def f(xp, r):
+        h = xp.tanh(xp.dot(r, W1))
+        m = xp.add(xp.dot(h, W2), np.eye(4, dtype=np.float32) * 2)    # (4, 4), well conditioned
+        return xp.add(xp.slogdet(m)[1], xp.sum(xp.square(h)))
+
+    op = folx_amd.ParallelLaplacianOperator() if parallel else folx_amd.LoopLaplacianOperator()
+    diag, grad = folx_amd.vmap(op(lambda r: f(fnp, r)))(x)
+    assert diag.shape == (3, 12) and grad.shape == (3, 12)
+    lap, jac = folx_amd.vmap(folx_amd.ForwardLaplacianOperator(0)(lambda r: f(fnp, r)))(x)
+    np.testing.assert_allclose(diag.sum(1).numpy(), lap.numpy(), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(grad.numpy(), jac.numpy(), rtol=2e-4, atol=2e-5)
+    for b in range(3):
+        xb = torch.as_tensor(x[b], dtype=torch.float64).reshape(-1)
+        fb = lambda z: f(plain, z.reshape(4, 3))
+        H = torch.func.jacfwd(torch.func.jacrev(fb))(xb)
+        np.testing.assert_allclose(diag[b].numpy(), torch.diagonal(H).numpy(), rtol=2e-4, atol=2e-5)
+        np.testing.assert_allclose(grad[b].numpy(), torch.func.jacrev(fb)(xb).numpy(), rtol=2e-4, atol=2e-5)
+    one_d, one_g = op(lambda r: f(fnp, r))(x[0])
+    np.testing.assert_allclose(one_d.numpy(), diag[0].numpy(), rtol=1e-6)
+    assert one_g.shape == (12,)

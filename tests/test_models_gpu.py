@@ -45,6 +45,28 @@ def test_readme_mlp(thr):
     assert out.jacobian.dense_array.shape == (400, 3)
 
 
+@pytest.mark.parametrize('parallel', [False, True])
+def test_loop_laplacian_operator_on_smallest_config(parallel):
+    """The README MLP at reduced size through LoopLaplacianOperator / ParallelLaplacianOperator
+    (folx/operators.py:41-79; one pass per input coordinate with a single Jacobian row):
+    their Hessian diagonal sums to the forward Laplacian of both storage modes, their
+    gradient is its Jacobian (test/test_operator.py:19-73)."""
+    params = wl.mlp_params(seed=0, in_dim=4, width=32, n_hidden=3)
+    x = np.random.default_rng(5).normal(size=(3, 6, 4)).astype(np.float32)
+    f = lambda t: wl.mlp_forward(params, t, fnp)
+    op = folx_amd.ParallelLaplacianOperator() if parallel else folx_amd.LoopLaplacianOperator()
+    print(f'case loop operator parallel={parallel}', flush=True)
+    diag, grad = folx_amd.vmap(op(f))(x)
+    assert diag.shape == (3, 24) and grad.shape == (3, 24)
+    ref = wl.mlp_forward(params, ob.init_state(x, dtype=np.float64), ob)
+    assert_lap(diag.sum(1), ref.lap, 'loop laplacian')
+    assert_val(grad.T, ref.J, 'loop jacobian')
+    for thr in (0, 4):
+        lap, jac = folx_amd.vmap(folx_amd.ForwardLaplacianOperator(thr)(f))(x)
+        assert_lap(lap, diag.sum(1).double().cpu().numpy(), 'forward vs loop laplacian')
+        assert_val(jac, grad.double().cpu().numpy(), 'forward vs loop jacobian')
+
+
 def test_readme_mlp_sparse_equals_dense():
     params = wl.mlp_params(seed=0)
     x = np.random.default_rng(1).normal(size=(8, 100, 4)).astype(np.float32)
