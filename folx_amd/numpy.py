@@ -68,7 +68,14 @@ def integer_pow(a, n: int):
 
 
 def power(a, c):
-    """``a ** c`` for ``a > 0`` and a constant real exponent (``jax.lax.pow`` with a constant)."""
+    """``a ** c`` for ``a > 0``: a constant real exponent runs the fused scalar rule; an
+    exponent that carries derivatives (or a constant base) goes through ``exp(c log a)``."""
+    from .api import FwdLaplArray as _F
+
+    if isinstance(c, _F) or not np.isscalar(c):
+        if not isinstance(a, _F):
+            return exp(multiply(c, np.log(np.asarray(a, dtype=np.float32))))
+        return exp(multiply(c, log(a)))
     return _call('pow', (a,), {'y': float(c)})
 
 
@@ -357,6 +364,129 @@ less, less_equal = (lambda a, b: _call('lt', (a, b))), (lambda a, b: _call('le',
 equal, not_equal = (lambda a, b: _call('eq', (a, b))), (lambda a, b: _call('ne', (a, b)))
 
 
+trunc, isfinite = (lambda a: _call('trunc', (a,))), (lambda a: _call('is_finite', (a,)))
+logical_and, logical_or = (lambda a, b: _call('and', (a, b))), (lambda a, b: _call('or', (a, b)))
+logical_xor, logical_not = (lambda a, b: _call('xor', (a, b))), (lambda a: _call('not', (a,)))
+
+
+def argmax(a, axis=-1):
+    """Index of the maximum along ``axis`` (no derivatives)."""
+    return _call('argmax', (a,), {'axis': axis % len(_shape(a))})
+
+
+def argmin(a, axis=-1):
+    return _call('argmin', (a,), {'axis': axis % len(_shape(a))})
+
+
+def exp2(a):
+    return exp(multiply(a, np.float32(np.log(2.0))))
+
+
+def remainder(a, b):
+    """C-style remainder ``a - b trunc(a / b)`` (``jax.lax.rem``): the quotient is piecewise
+    constant, so the rule is linear in a and b."""
+    return subtract(a, multiply(b, trunc(divide(a, b))))
+
+
+fmod = remainder
+
+
+def arctan2(y, x):
+    """``atan2(y, x)`` from the two half-plane formulas ``atan(y / x) (+- pi)`` for
+    ``|x| >= |y|`` and ``+-pi/2 - atan(x / y)`` otherwise.  The denominator of the branch
+    that is not taken is replaced by 1 before the division, so no infinity or NaN of a dead
+    branch reaches the result."""
+    big = greater_equal(abs(stop_gradient(x)), abs(stop_gradient(y)))     # |x| >= |y|
+    xs, ys = where(big, x, 1.0), where(big, 1.0, y)
+    ypos = greater_equal(stop_gradient(y), 0.0)
+    xneg = less(stop_gradient(x), 0.0)
+    pi = np.float32(np.pi)
+    sgn = subtract(multiply(ypos, 2.0), 1.0)                                # +1 for y >= 0, else -1
+    off_a = multiply(multiply(xneg, sgn), pi)                               # +-pi on the left half plane
+    branch_a = add(arctan(divide(y, xs)), off_a)
+    branch_b = subtract(multiply(sgn, pi / 2), arctan(divide(x, ys)))
+    return where(big, branch_a, branch_b)
+
+
+def split(a, indices_or_sections, axis=0):
+    """``numpy.split``: equal sections or explicit cut points along ``axis``."""
+    nd = len(_shape(a))
+    ax = axis % nd
+    n = _shape(a)[ax]
+    if np.isscalar(indices_or_sections):
+        k = int(indices_or_sections)
+        assert n % k == 0, 'array split does not result in an equal division'
+        cuts = [i * (n // k) for i in range(k + 1)]
+    else:
+        cuts = [0, *[int(c) for c in indices_or_sections], n]
+    return [getitem(a, tuple(slice(lo, hi) if d == ax else slice(None) for d in range(nd)))
+            for lo, hi in zip(cuts[:-1], cuts[1:])]
+
+
+def stack(arrs, axis=0):
+    arrs = list(arrs)
+    nd = len(_shape(arrs[0])) + 1
+    return concatenate([expand_dims(t, axis % nd) for t in arrs], axis=axis % nd)
+
+
+def unstack(a, axis=0):
+    return [squeeze(t, axis) for t in split(a, _shape(a)[axis % len(_shape(a))], axis)]
+
+
+def tile(a, reps):
+    reps = (reps,) if np.isscalar(reps) else tuple(reps)
+    nd = max(len(reps), len(_shape(a)))
+    reps = (1,) * (nd - len(reps)) + tuple(int(r) for r in reps)
+    out = reshape(a, (1,) * (nd - len(_shape(a))) + tuple(_shape(a)))
+    for ax, r in enumerate(reps):
+        if r > 1:
+            out = concatenate([out] * r, axis=ax)
+    return out
+
+
+def copy(a):
+    return a
+
+
+real = conj = copy      # real arithmetic only: the complex rules of the reference have no use here
+
+
+def imag(a):
+    return multiply(a, 0.0)
+
+
+def astype(a, dtype):
+    """float32 is the only arithmetic type of the path; integer / boolean targets give values
+    without derivatives (``convert_element_type``, folx/wrapped_functions.py:313-352)."""
+    if np.issubdtype(np.dtype(dtype), np.floating):
+        return a
+    return trunc(a) if np.issubdtype(np.dtype(dtype), np.integer) else not_equal(a, 0.0)
+
+
+def dynamic_slice(a, start_indices, slice_sizes):
+    """``jax.lax.dynamic_slice`` for start indices known at trace time (clamped like lax)."""
+    shape = _shape(a)
+    idx = []
+    for s0, sz, n in zip(start_indices, slice_sizes, shape):
+        s0 = int(np.clip(int(s0), 0, n - int(sz)))
+        idx.append(slice(s0, s0 + int(sz)))
+    return getitem(a, tuple(idx))
+
+
+def dynamic_update_slice(a, update, start_indices):
+    """``jax.lax.dynamic_update_slice`` for start indices known at trace time: linear in both
+    operands (a zero-padded update blended in with a 0/1 mask)."""
+    shape, ushape = _shape(a), _shape(update)
+    widths, mask = [], np.zeros(shape, dtype=np.float32)
+    sl = []
+    for s0, un, n in zip(start_indices, ushape, shape):
+        s0 = int(np.clip(int(s0), 0, n - un))
+        widths.append((s0, n - un - s0))
+        sl.append(slice(s0, s0 + un))
+    mask[tuple(sl)] = 1.0
+    return add(multiply(a, 1.0 - mask), pad(update, widths))
+
+
 def logaddexp(a, b):
     """log(exp a + exp b) = a + softplus(b - a)."""
     return add(a, softplus(subtract(b, a)))
@@ -411,3 +541,21 @@ register_function('cummax', _composed(cummax, 'axis'))
 register_function('cummin', _composed(cummin, 'axis'))
 register_function('logaddexp', _composed(logaddexp))
 register_function('pad', _composed(pad, 'constant_values'))
+register_function('atan2', _composed(arctan2))                       # folx/wrapped_functions.py:419
+register_function('rem', _composed(remainder))                       # :438
+register_function('exp2', _composed(exp2))                           # :636
+register_function('split', _composed(split, 'indices_or_sections', 'axis'))   # :628
+register_function('stack', _composed(lambda *arrs, axis=0: stack(arrs, axis), 'axis'))     # :641
+register_function('unstack', _composed(unstack, 'axis'))             # :651
+register_function('tile', _composed(tile, 'reps'))                   # :660
+register_function('copy', _composed(copy))                           # :638
+register_function('squeeze', _composed(lambda a, dimensions: squeeze(a, dimensions[0]) if len(dimensions) == 1
+                                       else reshape(a, [n for i, n in enumerate(_shape(a)) if i not in dimensions]),
+                                       'dimensions'))                # :503
+register_function('real', _composed(real))                           # :358
+register_function('conj', _composed(conj))                           # :356
+register_function('imag', _composed(imag))                           # :357
+register_function('convert_element_type', _composed(lambda a, new_dtype=np.float32: astype(a, new_dtype), 'new_dtype'))
+register_function('dynamic_slice', _composed(lambda a, *start, slice_sizes: dynamic_slice(a, start, slice_sizes),
+                                             'slice_sizes'))          # :468
+register_function('dynamic_update_slice', _composed(lambda a, u, *start: dynamic_update_slice(a, u, start)))  # :488

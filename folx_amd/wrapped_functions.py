@@ -1372,6 +1372,18 @@ for _n, _tf, _nf in [('floor', torch.floor, np.floor), ('ceil', torch.ceil, np.c
                      ('gt', torch.gt, np.greater), ('ge', torch.ge, np.greater_equal), ('lt', torch.lt, np.less),
                      ('le', torch.le, np.less_equal), ('eq', torch.eq, np.equal), ('ne', torch.ne, np.not_equal)]:
     register_function(_n, _values_only(_tf, _nf))
+for _n, _tf, _nf in [('trunc', torch.trunc, np.trunc), ('is_finite', torch.isfinite, np.isfinite),
+                     ('and', lambda a, b: (a != 0) & (b != 0), lambda a, b: np.logical_and(a != 0, b != 0)),
+                     ('or', lambda a, b: (a != 0) | (b != 0), lambda a, b: np.logical_or(a != 0, b != 0)),
+                     ('xor', lambda a, b: (a != 0) ^ (b != 0), lambda a, b: np.logical_xor(a != 0, b != 0)),
+                     ('not', lambda a: a == 0, lambda a: a == 0)]:
+    register_function(_n, _values_only(_tf, _nf))  # folx/wrapped_functions.py:546-550
+register_function('argmax', lambda args, kw, thr: _values_only(
+    lambda a: torch.argmax(a, dim=kw['axis'] + 1 if kw['axis'] >= 0 else kw['axis']),
+    lambda a: np.argmax(a, axis=kw['axis']))(args, kw, thr))          # folx/wrapped_functions.py:448-449
+register_function('argmin', lambda args, kw, thr: _values_only(
+    lambda a: torch.argmin(a, dim=kw['axis'] + 1 if kw['axis'] >= 0 else kw['axis']),
+    lambda a: np.argmin(a, axis=kw['axis']))(args, kw, thr))
 register_function('broadcast_in_dim', broadcast_in_dim_rule)
 register_function('slice', getitem_rule)
 register_function('gather', getitem_rule)

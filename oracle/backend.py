@@ -198,6 +198,79 @@ def divide(a, b):
     return multiply(reciprocal(b), a)
 
 
+def _as_triplet(v, like: OArr) -> OArr:
+    """A constant as a triplet with zero derivatives on ``like``'s row frame."""
+    if _is(v):
+        return v
+    d = v.data if isinstance(v, OConst) else np.asarray(v, dtype=like.x.dtype)[None]
+    x = np.broadcast_to(d, np.broadcast_shapes(d.shape, like.x.shape)).astype(like.x.dtype)
+    return OArr(x, np.zeros((like.J.shape[0], *x.shape), dtype=x.dtype), np.zeros_like(x))
+
+
+def _binary_general(rule, a, b):
+    ref = a if _is(a) else b
+    ta, tb = _bcast3(_as_triplet(a, ref), _as_triplet(b, ref))
+    return OArr(*rule(*ta, *tb))
+
+
+def arctan2(y, x):
+    return _binary_general(rules.atan2_rule, y, x)
+
+
+def remainder(a, b):
+    return _binary_general(rules.rem_rule, a, b)
+
+
+fmod = remainder
+
+
+def exp2(a):
+    return exp(multiply(a, np.log(2.0)))
+
+
+def split(a, indices_or_sections, axis=0):
+    ax = axis % a.ndim
+    n = a.shape[ax]
+    cuts = [i * (n // indices_or_sections) for i in range(indices_or_sections + 1)] if np.isscalar(
+        indices_or_sections) else [0, *indices_or_sections, n]
+    return [getitem(a, tuple(slice(lo, hi) if d == ax else slice(None) for d in range(a.ndim)))
+            for lo, hi in zip(cuts[:-1], cuts[1:])]
+
+
+def stack(arrs, axis=0):
+    nd = arrs[0].ndim + 1
+    return concatenate([expand_dims(t, axis % nd) for t in arrs], axis=axis % nd)
+
+
+def tile(a, reps):
+    reps = (reps,) if np.isscalar(reps) else tuple(reps)
+    nd = max(len(reps), a.ndim)
+    reps = (1,) * (nd - len(reps)) + reps
+    out = reshape(a, (1,) * (nd - a.ndim) + tuple(a.shape))
+    for ax, r in enumerate(reps):
+        if r > 1:
+            out = concatenate([out] * r, axis=ax)
+    return out
+
+
+def dynamic_slice(a, start_indices, slice_sizes):
+    idx = []
+    for s0, sz, n in zip(start_indices, slice_sizes, a.shape):
+        s0 = int(np.clip(int(s0), 0, n - int(sz)))
+        idx.append(slice(s0, s0 + int(sz)))
+    return getitem(a, tuple(idx))
+
+
+def dynamic_update_slice(a, update, start_indices):
+    x, J, L = a.x.copy(), a.J.copy(), a.lap.copy()
+    sl = tuple(slice(int(np.clip(int(s0), 0, n - un)), int(np.clip(int(s0), 0, n - un)) + un)
+               for s0, un, n in zip(start_indices, update.shape, a.shape))
+    x[(slice(None), *sl)] = update.x
+    J[(slice(None), slice(None), *sl)] = update.J
+    L[(slice(None), *sl)] = update.lap
+    return OArr(x, J, L)
+
+
 def _minmax(a, b, is_max):
     if _is(a) and _is(b):
         ta, tb = _bcast3(a, b)
@@ -281,7 +354,9 @@ erf, erfc, erf_inv, cbrt = _unary('erf'), _unary('erfc'), _unary('erf_inv'), _un
 
 
 def power(a, c):
-    """a ** c for a > 0 and a constant real exponent c."""
+    """a ** c for a > 0: constant real exponent, or an exponent / base pair of triplets."""
+    if _is(c) or isinstance(c, OConst) or not np.isscalar(c):
+        return _binary_general(rules.pow_rule, a, c)
     return _unary('pow', float(c))(a)
 
 

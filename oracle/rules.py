@@ -278,6 +278,43 @@ def div_rule(a, Ja, La, b, Jb, Lb):
     return y, Jy, lap
 
 
+def binary_hessian_rule(y, fa, fb, faa, fab, fbb, Ja, La, Jb, Lb):
+    """General two-argument scalar function from its value, gradient (fa, fb) and Hessian
+    (faa, fab, fbb) at every element -- what ``wrap_forward_laplacian`` of a binary jax
+    function evaluates to (folx/jvp.py:676-684 for the Jacobian, folx/hessian.py:115-175 for
+    tr(J^T H J) on the pair of operands):
+        J_y = fa J_a + fb J_b,   lap_y = fa lap_a + fb lap_b + faa |J_a|^2 + 2 fab J_a.J_b + fbb |J_b|^2."""
+    Jy = fa[None] * Ja + fb[None] * Jb
+    lap = fa * La + fb * Lb + faa * (Ja * Ja).sum(0) + 2 * fab * (Ja * Jb).sum(0) + fbb * (Jb * Jb).sum(0)
+    return y, Jy, lap
+
+
+def atan2_rule(a, Ja, La, b, Jb, Lb):
+    """y = atan2(a, b) (``jax.lax.atan2``, folx/wrapped_functions.py:419): with r2 = a^2 + b^2,
+    grad = (b, -a) / r2, Hessian = [[-2ab, a^2 - b^2], [a^2 - b^2, 2ab]] / r2^2."""
+    a, b = np.broadcast_arrays(a, b)
+    r2 = a * a + b * b
+    return binary_hessian_rule(np.arctan2(a, b), b / r2, -a / r2, -2 * a * b / r2 ** 2, (a * a - b * b) / r2 ** 2,
+                               2 * a * b / r2 ** 2, Ja, La, Jb, Lb)
+
+
+def pow_rule(a, Ja, La, b, Jb, Lb):
+    """y = a ** b for a > 0 with both operands variable (``jax.lax.pow``,
+    folx/wrapped_functions.py:384)."""
+    a, b = np.broadcast_arrays(a, b)
+    y, la = a ** b, np.log(a)
+    return binary_hessian_rule(y, b * y / a, y * la, b * (b - 1) * y / a ** 2, y / a * (1 + b * la), y * la * la,
+                               Ja, La, Jb, Lb)
+
+
+def rem_rule(a, Ja, La, b, Jb, Lb):
+    """y = a - b trunc(a / b) (``jax.lax.rem``, folx/wrapped_functions.py:438): the quotient is
+    piecewise constant, so the rule is linear."""
+    a, b = np.broadcast_arrays(a, b)
+    q = np.trunc(a / b)
+    return a - b * q, Ja - q[None] * Jb, La - q * Lb
+
+
 def add_rule(a, Ja, La, b, Jb, Lb, sign=1.0):
     """y = a +- b (LINEAR, folx/wrapped_functions.py:365-370)."""
     return a + sign * b, Ja + sign * Jb, La + sign * Lb

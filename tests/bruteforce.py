@@ -67,6 +67,8 @@ class plain:
 
     @staticmethod
     def power(a, c):
+        if torch.is_tensor(c) or not np.isscalar(c):
+            return (a if torch.is_tensor(a) else plain._c(a, c)) ** (c if torch.is_tensor(c) else plain._c(c, a))
         return a ** float(c)
 
     @staticmethod
@@ -256,6 +258,30 @@ class plain:
         pw = [tuple(p) for p in pad_width] if np.ndim(pad_width) == 2 else [tuple(pad_width)] * a.ndim
         flat = [v for p in reversed(pw) for v in p]
         return torch.nn.functional.pad(a, flat, value=constant_values)
+
+    arctan2 = staticmethod(lambda y, x: torch.atan2(y if torch.is_tensor(y) else plain._c(y, x), plain._c(x, y) if torch.is_tensor(y) else x))
+    remainder = staticmethod(lambda a, b: torch.fmod(a, plain._c(b, a)))
+    fmod = remainder
+    exp2 = staticmethod(torch.exp2)
+    split = staticmethod(lambda a, k, axis=0: list(torch.split(a, a.shape[axis] // k, dim=axis)) if np.isscalar(k)
+                         else list(torch.tensor_split(a, list(k), dim=axis)))
+    stack = staticmethod(lambda arrs, axis=0: torch.stack(list(arrs), dim=axis))
+    tile = staticmethod(lambda a, reps: torch.tile(a, (reps,) if np.isscalar(reps) else tuple(reps)))
+    trunc = staticmethod(lambda a: torch.trunc(a).detach())
+
+    @staticmethod
+    def dynamic_slice(a, start, sizes):
+        idx = tuple(slice(int(np.clip(s0, 0, n - sz)), int(np.clip(s0, 0, n - sz)) + sz)
+                    for s0, sz, n in zip(start, sizes, a.shape))
+        return a[idx]
+
+    @staticmethod
+    def dynamic_update_slice(a, u, start):
+        idx = tuple(slice(int(np.clip(s0, 0, n - un)), int(np.clip(s0, 0, n - un)) + un)
+                    for s0, un, n in zip(start, u.shape, a.shape))
+        out = a.clone()
+        out[idx] = u
+        return out
 
     greater = staticmethod(lambda a, b: (a > plain._c(b, a)).detach())
     less = staticmethod(lambda a, b: (a < plain._c(b, a)).detach())

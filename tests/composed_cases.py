@@ -28,6 +28,19 @@ CASES = {
     'cumprod': lambda xp, x: xp.cumprod(xp.reshape(xp.add(xp.sin(x), 1.5), (3, 4)), axis=-1),
     'cummax': lambda xp, x: xp.cummax(xp.reshape(xp.sin(xp.multiply(x, 1.9)), (3, 4)), axis=-1),
     'cummin_axis0': lambda xp, x: xp.cummin(xp.reshape(xp.cos(xp.multiply(x, 1.4)), (3, 4)), axis=0),
+    # atan2 over all four quadrants and both half-plane branches (x = 12 seeded normals * 0.8)
+    'atan2': lambda xp, x: xp.arctan2(xp.sin(xp.multiply(_g(xp, x, slice(0, 6)), 2.0)),
+                                      xp.add(xp.cos(xp.multiply(_g(xp, x, slice(6, 12)), 3.0)), 0.1)),
+    'atan2_const': lambda xp, x: xp.arctan2(xp.sin(x), -0.4),
+    'pow_variable_exponent': lambda xp, x: xp.power(xp.add(xp.square(_g(xp, x, slice(0, 6))), 0.7),
+                                                    xp.sin(_g(xp, x, slice(6, 12)))),
+    'pow_constant_base': lambda xp, x: xp.power(1.7, xp.tanh(x)),
+    'rem': lambda xp, x: xp.remainder(xp.multiply(x, 3.0), xp.add(xp.cos(x), 1.6)),
+    'exp2': lambda xp, x: xp.exp2(xp.sin(x)),
+    'split_stack_tile': lambda xp, x: xp.tile(xp.stack([xp.multiply(a, b) for a, b in zip(
+        xp.split(xp.sin(x), 2), xp.split(xp.tanh(x), [6]))], axis=1), (2, 1)),
+    'dynamic_slices': lambda xp, x: xp.dynamic_update_slice(
+        xp.reshape(xp.sin(x), (3, 4)), xp.dynamic_slice(xp.reshape(xp.square(x), (3, 4)), (1, 2), (2, 2)), (0, 1)),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }

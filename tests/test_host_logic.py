@@ -449,3 +449,34 @@ def test_loop_and_parallel_operators(parallel):
     one_d, one_g = op(lambda r: f(fnp, r))(x[0])
     np.testing.assert_allclose(one_d.numpy(), diag[0].numpy(), rtol=1e-6)
     assert one_g.shape == (12,)
+
+
+def test_value_only_functions():
+    """argmax / argmin, logical functions, is_finite, trunc and integer conversion give plain
+    values without derivatives (``warp_without_fwd_laplacian``,
+    folx/wrapped_functions.py:445-449, :546-550)."""
+    from folx_amd.api import BatchedArray
+
+    x = np.random.default_rng(15).normal(size=(3, 4, 5)).astype(np.float32)
+    seen = {}
+
+    def f(r):
+        h = fnp.sin(fnp.multiply(r, 2.0))
+        seen['argmax'] = fnp.argmax(h, axis=-1)
+        seen['argmin'] = fnp.argmin(h, axis=0)
+        seen['finite'] = fnp.isfinite(h)
+        seen['and'] = fnp.logical_and(fnp.greater(h, 0.0), fnp.less(h, 0.5))
+        seen['not'] = fnp.logical_not(fnp.greater(h, 0.0))
+        seen['int'] = fnp.astype(fnp.multiply(h, 3.0), np.int32)
+        return fnp.sum(h)
+
+    folx_amd.vmap(folx_amd.forward_laplacian(f, 0))(x)
+    h = np.sin(2.0 * x)
+    for v in seen.values():
+        assert isinstance(v, BatchedArray)
+    np.testing.assert_array_equal(seen['argmax'].data.numpy(), h.argmax(-1))
+    np.testing.assert_array_equal(seen['argmin'].data.numpy(), h.argmin(1))
+    assert seen['finite'].data.numpy().all()
+    np.testing.assert_array_equal(seen['and'].data.numpy() != 0, (h > 0) & (h < 0.5))
+    np.testing.assert_array_equal(seen['not'].data.numpy() != 0, ~(h > 0))
+    np.testing.assert_array_equal(seen['int'].data.numpy(), np.trunc(3.0 * h))
