@@ -15,6 +15,9 @@ Pinning status (what fixes each function independently of its own formula):
   rules.ACTIVATIONS          closed forms checked against torch fp64 jvp-of-jvp
   rules.dense_rule           brute-force fp64 Hessian trace of small MLPs
   rules.binary rules         brute-force fp64 Hessian trace
+  rules.atan2_rule, pow_rule, rem_rule (closed-form gradients and Hessians)
+                             brute-force fp64 Hessian trace of torch.atan2 / pow / fmod over all
+                             four quadrants and both operand orders
   rules.slogdet_rule         numpy.linalg fp64 + brute-force Hessian trace (n <= 6),
                              diagonal / triangular closed forms, row-swap sign
   rules.inv_rule, solve_rule brute-force fp64 Hessian trace through an adjugate/determinant
