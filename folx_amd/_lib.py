@@ -48,7 +48,7 @@ ACT = {
     'logistic': 7, 'sigmoid': 7, 'softplus': 8, 'sin': 9, 'cos': 10, 'abs': 11,
     'log1p': 12, 'reciprocal': 13, 'expm1': 14, 'integer_pow': 15,
     'sinh': 16, 'cosh': 17, 'tan': 18, 'asin': 19, 'acos': 20, 'atan': 21, 'asinh': 22, 'acosh': 23,
-    'atanh': 24, 'erf': 25, 'erfc': 26, 'erf_inv': 27, 'cbrt': 28, 'pow': 29,
+    'atanh': 24, 'erf': 25, 'erfc': 26, 'erf_inv': 27, 'cbrt': 28, 'pow': 29, 'lgamma': 30, 'digamma': 31,
 }
 BINOP = {'mul': 0, 'div': 1, 'add': 2, 'sub': 3, 'min': 4, 'max': 5}
 

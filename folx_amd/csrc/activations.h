@@ -4,6 +4,38 @@
 
 namespace {
 
+// digamma, trigamma and tetragamma (polygamma of order 0, 1, 2) in one pass: the argument is
+// moved to x >= 6 with the recurrences psi_m(x) = psi_m(x + 1) - (-1)^m m! / x^(m+1) and the
+// asymptotic series are summed there; x < 0.5 goes through the reflection formulas
+//   psi(1-x) - psi(x) = pi cot(pi x),  psi1(1-x) + psi1(x) = pi^2 / sin^2(pi x),
+//   psi2(1-x) - psi2(x) = 2 pi^3 cos(pi x) / sin^3(pi x).
+__device__ __forceinline__ void polygamma012(float x, float& p0, float& p1, float& p2) {
+  const bool reflect = x < 0.5f;
+  const float xr = x;
+  if (reflect) x = 1.0f - x;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+  while (x < 6.0f) {
+    const float r = 1.0f / x;
+    s0 -= r;
+    s1 += r * r;
+    s2 -= 2.0f * r * r * r;
+    x += 1.0f;
+  }
+  const float r = 1.0f / x, r2 = r * r;
+  p0 = s0 + logf(x) - 0.5f * r - r2 * (1.0f / 12.0f - r2 * (1.0f / 120.0f - r2 * (1.0f / 252.0f - r2 * (1.0f / 240.0f))));
+  p1 = s1 + r + 0.5f * r2 + r * r2 * (1.0f / 6.0f - r2 * (1.0f / 30.0f - r2 * (1.0f / 42.0f - r2 * (1.0f / 30.0f))));
+  p2 = s2 - r2 - r * r2 - r2 * r2 * (0.5f - r2 * (1.0f / 6.0f - r2 * (1.0f / 6.0f - r2 * (3.0f / 10.0f))));
+  if (reflect) {
+    const float pi = 3.14159265358979f;
+    float sn, cs;
+    sincospif(xr, &sn, &cs);
+    const float ct = cs / sn, cc = 1.0f / (sn * sn);
+    p0 = p0 - pi * ct;
+    p1 = pi * pi * cc - p1;
+    p2 = p2 - 2.0f * pi * pi * pi * cc * ct;
+  }
+}
+
 template <int ACT>
 __device__ __forceinline__ void act_eval(float x, float prm, float& y, float& d1, float& d2) {
   if constexpr (ACT == FOLX_ACT_TANH) {
@@ -89,6 +121,14 @@ __device__ __forceinline__ void act_eval(float x, float prm, float& y, float& d1
   } else if constexpr (ACT == FOLX_ACT_CBRT) {
     float c = cbrtf(x);
     y = c; d1 = c / (3.0f * x); d2 = -2.0f * c / (9.0f * x * x);
+  } else if constexpr (ACT == FOLX_ACT_LGAMMA) {
+    float p0, p1, p2;
+    polygamma012(x, p0, p1, p2);
+    y = lgammaf(x); d1 = p0; d2 = p1;
+  } else if constexpr (ACT == FOLX_ACT_DIGAMMA) {
+    float p0, p1, p2;
+    polygamma012(x, p0, p1, p2);
+    y = p0; d1 = p1; d2 = p2;
   } else if constexpr (ACT == FOLX_ACT_POW) {
     float pm2 = powf(x, prm - 2.0f);
     y = pm2 * x * x; d1 = prm * pm2 * x; d2 = prm * (prm - 1.0f) * pm2;

@@ -147,7 +147,7 @@ extern "C" int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float para
     FOLX_CASE(FOLX_ACT_SINH) FOLX_CASE(FOLX_ACT_COSH) FOLX_CASE(FOLX_ACT_TAN) FOLX_CASE(FOLX_ACT_ASIN)
     FOLX_CASE(FOLX_ACT_ACOS) FOLX_CASE(FOLX_ACT_ATAN) FOLX_CASE(FOLX_ACT_ASINH) FOLX_CASE(FOLX_ACT_ACOSH)
     FOLX_CASE(FOLX_ACT_ATANH) FOLX_CASE(FOLX_ACT_ERF) FOLX_CASE(FOLX_ACT_ERFC) FOLX_CASE(FOLX_ACT_ERF_INV)
-    FOLX_CASE(FOLX_ACT_CBRT) FOLX_CASE(FOLX_ACT_POW)
+    FOLX_CASE(FOLX_ACT_CBRT) FOLX_CASE(FOLX_ACT_POW) FOLX_CASE(FOLX_ACT_LGAMMA) FOLX_CASE(FOLX_ACT_DIGAMMA)
   }
 #undef FOLX_CASE
   return FOLX_HIP_EINVAL;

@@ -60,6 +60,7 @@ sinh, cosh, tan = _u('sinh'), _u('cosh'), _u('tan')
 arcsin, arccos, arctan = _u('asin'), _u('acos'), _u('atan')
 arcsinh, arccosh, arctanh = _u('asinh'), _u('acosh'), _u('atanh')
 erf, erfc, erf_inv, cbrt = _u('erf'), _u('erfc'), _u('erf_inv'), _u('cbrt')
+lgamma, digamma = _u('lgamma'), _u('digamma')
 reciprocal, negative, sign, stop_gradient = _u('reciprocal'), _u('neg'), _u('sign'), _u('stop_gradient')
 
 

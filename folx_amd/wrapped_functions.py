@@ -153,10 +153,11 @@ def _unary_rule(name: str) -> ForwardLaplacian:
                 return np.asarray(a) ** int(param)
             if name == 'pow':
                 return np.asarray(a) ** float(param)
-            if name in ('erf', 'erfc', 'erf_inv'):
+            if name in ('erf', 'erfc', 'erf_inv', 'lgamma', 'digamma'):
                 import scipy.special as sp
 
-                return {'erf': sp.erf, 'erfc': sp.erfc, 'erf_inv': sp.erfinv}[name](np.asarray(a))
+                return {'erf': sp.erf, 'erfc': sp.erfc, 'erf_inv': sp.erfinv, 'lgamma': sp.gammaln,
+                        'digamma': sp.digamma}[name](np.asarray(a))
             return _NP_UNARY[name](np.asarray(a))
         mask = a.jacobian.x0_idx
         x, J, lap = a.x, a.jacobian.data, a.laplacian
@@ -1351,7 +1352,7 @@ def mhsea_forward_laplacian(args, kwargs, sparsity_threshold):
 
 for _n in ['tanh', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'sin', 'cos', 'abs', 'log1p',
            'expm1', 'integer_pow', 'silu', 'softplus', 'reciprocal', 'sinh', 'cosh', 'tan', 'asin', 'acos', 'atan',
-           'asinh', 'acosh', 'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt', 'pow']:
+           'asinh', 'acosh', 'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt', 'pow', 'lgamma', 'digamma']:
     register_function(_n, _unary_rule(_n))
 register_function('sigmoid', _unary_rule('logistic'))  # string key, folx/wrapped_functions.py:554
 register_function('neg', neg_rule)

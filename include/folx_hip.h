@@ -68,7 +68,9 @@ enum folx_hip_act {
   FOLX_ACT_ERF_INV = 27,
   FOLX_ACT_CBRT = 28,
   FOLX_ACT_POW = 29, /* x^param for x > 0, param = constant real exponent (jax.lax.pow_p) */
-  FOLX_ACT_COUNT = 30
+  FOLX_ACT_LGAMMA = 30,  /* log|Gamma(x)|, derivatives digamma and trigamma (jax.lax.lgamma_p) */
+  FOLX_ACT_DIGAMMA = 31, /* derivatives trigamma and tetragamma (jax.lax.digamma_p) */
+  FOLX_ACT_COUNT = 32
 };
 
 /* Binary functions of folx_hip_binary_fwdlap. */

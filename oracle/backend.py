@@ -351,6 +351,7 @@ sinh, cosh, tan = _unary('sinh'), _unary('cosh'), _unary('tan')
 arcsin, arccos, arctan = _unary('asin'), _unary('acos'), _unary('atan')
 arcsinh, arccosh, arctanh = _unary('asinh'), _unary('acosh'), _unary('atanh')
 erf, erfc, erf_inv, cbrt = _unary('erf'), _unary('erfc'), _unary('erf_inv'), _unary('cbrt')
+lgamma, digamma = _unary('lgamma'), _unary('digamma')
 
 
 def power(a, c):

@@ -177,6 +177,26 @@ def _cbrt(x):
     return c, c / (3 * x), -2 * c / (9 * x * x)
 
 
+def _lgamma(x):
+    from scipy.special import digamma, gammaln, polygamma
+
+    return gammaln(x), digamma(x), polygamma(1, x)
+
+
+def _digamma(x):
+    """Values from scipy for x > 0 (its polygamma is defined there); negative arguments by the
+    reflection formulas psi1(1-x) + psi1(x) = pi^2 / sin^2(pi x) and
+    psi2(1-x) - psi2(x) = 2 pi^3 cos(pi x) / sin^3(pi x)."""
+    from scipy.special import digamma, polygamma
+
+    xp = np.where(x > 0, x, 1 - x)
+    p1, p2 = polygamma(1, xp), polygamma(2, xp)
+    s, c = np.sin(np.pi * x), np.cos(np.pi * x)
+    p1 = np.where(x > 0, p1, np.pi ** 2 / s ** 2 - p1)
+    p2 = np.where(x > 0, p2, p2 - 2 * np.pi ** 3 * c / s ** 3)
+    return digamma(x), p1, p2
+
+
 def _identity(x):
     return x, np.ones_like(x), np.zeros_like(x)
 
@@ -203,7 +223,7 @@ ACTIVATIONS = {
     # the rest of the reference's scalar table (folx/wrapped_functions.py:416-445)
     'sinh': _sinh, 'cosh': _cosh, 'tan': _tan, 'asin': _asin, 'acos': _acos, 'atan': _atan,
     'asinh': _asinh, 'acosh': _acosh, 'atanh': _atanh, 'erf': _erf, 'erfc': _erfc, 'erf_inv': _erf_inv,
-    'cbrt': _cbrt,
+    'cbrt': _cbrt, 'lgamma': _lgamma, 'digamma': _digamma,
 }
 
 

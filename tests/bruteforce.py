@@ -64,6 +64,8 @@ class plain:
     arcsinh, arccosh, arctanh = staticmethod(torch.asinh), staticmethod(torch.acosh), staticmethod(torch.atanh)
     erf, erfc, erf_inv = staticmethod(torch.erf), staticmethod(torch.erfc), staticmethod(torch.erfinv)
     cbrt = staticmethod(lambda t: torch.sign(t) * torch.abs(t) ** (1.0 / 3.0))
+    lgamma = staticmethod(torch.lgamma)
+    digamma = staticmethod(torch.digamma)
 
     @staticmethod
     def power(a, c):

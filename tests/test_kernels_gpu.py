@@ -28,7 +28,7 @@ POSITIVE = {'log', 'sqrt', 'rsqrt', 'log1p', 'reciprocal', 'cbrt'}
 UNIT = {'asin', 'acos', 'atanh', 'erf_inv'}
 ACTS = ['tanh', 'silu', 'exp', 'log', 'sqrt', 'rsqrt', 'square', 'logistic', 'softplus', 'sin', 'cos',
         'abs', 'log1p', 'reciprocal', 'expm1', 'sinh', 'cosh', 'tan', 'asin', 'acos', 'atan', 'asinh', 'acosh',
-        'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt']
+        'atanh', 'erf', 'erfc', 'erf_inv', 'cbrt', 'lgamma', 'digamma']
 
 
 @pytest.mark.parametrize('name', ACTS)
@@ -47,6 +47,9 @@ def test_elementwise(name, shape, P):
         x = np.abs(x) + 1.2
     if name in ('tan', 'sinh', 'cosh'):
         x = np.clip(x, -1.3, 1.3)   # stay away from the poles / large magnitudes of fp32
+    if name in ('lgamma', 'digamma'):   # positive arguments, and negative ones away from the poles
+        neg = (rng.integers(-3, 0, size=shape) + rng.uniform(0.25, 0.75, size=shape)).astype(np.float32)
+        x = np.where(rng.uniform(size=shape) < 0.3, neg, rng.uniform(0.3, 9.0, size=shape).astype(np.float32))
     ref = rules.elementwise_rule(name, *f64(x, J, L))
     got = K.elementwise(name, dev(x), dev(J), dev(L))
     assert_triplet(got, ref, name)

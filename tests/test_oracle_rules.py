@@ -34,6 +34,8 @@ def test_activation_closed_forms_vs_autograd(name):
         x = rng.uniform(-0.9, 0.9, size=64)
     if name == 'acosh':
         x = np.abs(x) + 1.1
+    if name in ('lgamma', 'digamma'):   # positive arguments and negative ones away from the poles
+        x = np.concatenate([rng.uniform(0.3, 7.0, size=40), rng.integers(-3, 0, size=24) + rng.uniform(0.25, 0.75, size=24)])
     tname = PLAIN_NAME.get(name, name)
     f = (lambda t: t) if tname is None else getattr(plain, tname)
     xt = torch.tensor(x, dtype=torch.float64)
