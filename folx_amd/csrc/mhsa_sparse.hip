@@ -48,10 +48,11 @@ __device__ __forceinline__ float sa_dot(const float* u, const float* m, int d4) 
   return (s0 + s1) + (s2 + s3);
 }
 constexpr int SA_MAXPASS = 4;  // n <= 64: rows i = 16 pass + tid / 16
+constexpr int SA_E = 4;        // sequence positions worked on together
 
 __host__ __device__ inline int64_t sa_lds_floats(int n, int d, int K) {
   const int dp = d + 4, np1 = n + 1;
-  return 4LL * n * dp + 4LL * n * np1 + 4LL * K * d + 2LL * K * n + 8 + 5LL * n + 8;
+  return 4LL * n * dp + 4LL * n * np1 + SA_E * (4LL * K * d + 2LL * K * n + 2LL * K) + 5LL * n + (int64_t)K * n;
 }
 
 __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
@@ -66,19 +67,20 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
   float* AA = pS + n * np1;
   float* BB = AA + n * np1;
   float* AR = BB + n * np1;
-  float* aS = AR + n * np1;
-  float* bS = aS + K * d;
-  float* wS = bS + K * d;
-  float* gamS = wS + K * d;
-  float* alS = gamS + K * d;
-  float* beS = alS + K * n;
-  float* rhoS = beS + K * n;
-  float* D1 = rhoS + 8;
+  float* aS = AR + n * np1;             // [SA_E][K][d] vectors of the positions in work
+  float* bS = aS + SA_E * K * d;
+  float* wS = bS + SA_E * K * d;
+  float* gamS = wS + SA_E * K * d;
+  float* alS = gamS + SA_E * K * d;     // [SA_E][K][n]
+  float* beS = alS + SA_E * K * n;
+  float* rhoS = beS + SA_E * K * n;     // [SA_E][K]
+  float* gpS = rhoS + SA_E * K;         // [SA_E][K] a_s . b_s
+  float* D1 = gpS + SA_E * K;
   float* D2 = D1 + n;
   float* R2a = D2 + n;
   float* gS = R2a + n;
   float* rsum = gS + n;
-  int* cS = reinterpret_cast<int*>(rsum + n);  // dense rows of the current position's slots
+  int* idxS = reinterpret_cast<int*>(rsum + n);  // [K][n] copy of the index table
 
   const int tid = threadIdx.x;
   const int64_t b = blockIdx.x / H;
@@ -97,6 +99,7 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
   load_tile(a.k, kS);
   load_tile(a.v, vS);
   for (int it = tid; it < 3 * n * np1; it += SA_NT) AA[it] = 0.0f;  // AA, BB, AR are contiguous
+  for (int it = tid; it < K * n; it += SA_NT) idxS[it] = a.index[it];
   __syncthreads();
 
   // p = softmax(q k^T)
@@ -129,103 +132,132 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
     *reinterpret_cast<float4*>(a.o + grow(i) + 4 * t4) = acc;
   }
 
-  // the three vectors (a, b, w) of every slot of one position: one float4 per thread
+  // The vectors (a, b, w) of every slot of SA_E consecutive positions form one group: one
+  // float4 per thread and position, requested one group ahead of its use.
   const int nvec = 3 * K * d4;
   const int pf_which = tid / (K * d4), pf_sl = (tid / d4) % K, pf_t4 = tid % d4;
-  auto fetch = [&](int e) -> float4 {
-    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (tid < nvec && a.index[pf_sl * n + e] >= 0) {
-      const float* src = pf_which == 0 ? a.qs : (pf_which == 1 ? a.ks : a.vs);
-      r = *reinterpret_cast<const float4*>(src + pf_sl * Srow + grow(e) + 4 * pf_t4);
-    }
-    return r;
-  };
-  float4 pf = fetch(0);
-
-  float4 t2acc[SA_MAXPASS];
+  auto fetch = [&](int e0, float4 (&pf)[SA_E]) {
 #pragma unroll
-  for (int ps = 0; ps < SA_MAXPASS; ++ps) t2acc[ps] = make_float4(0.f, 0.f, 0.f, 0.f);
-  const int orow = tid / 16, ot4 = tid % 16;
+    for (int ee = 0; ee < SA_E; ++ee) {
+      pf[ee] = make_float4(0.f, 0.f, 0.f, 0.f);
+      const int e = e0 + ee;
+      if (tid < nvec && e < n && idxS[pf_sl * n + e] >= 0) {
+        const float* src = pf_which == 0 ? a.qs : (pf_which == 1 ? a.ks : a.vs);
+        pf[ee] = *reinterpret_cast<const float4*>(src + pf_sl * Srow + grow(e) + 4 * pf_t4);
+      }
+    }
+  };
+  __syncthreads();  // index table, o and p are in LDS
+  float4 pf[SA_E];
+  fetch(0, pf);
 
-  for (int e = 0; e < n; ++e) {
-    __syncthreads();  // everyone is done with the previous position's vectors (and with o, p on entry)
+  float4 t2acc[SA_MAXPASS], oreg[SA_MAXPASS];
+  const int orow = tid / 16, ot4 = tid % 16;
+#pragma unroll
+  for (int ps = 0; ps < SA_MAXPASS; ++ps) {
+    t2acc[ps] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int i = ps * 16 + orow;
+    oreg[ps] = (i < n && ot4 < d4) ? *reinterpret_cast<const float4*>(oS + i * dp + 4 * ot4)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+
+  for (int e0 = 0; e0 < n; e0 += SA_E) {
+    const int ne = min(SA_E, n - e0);
+    __syncthreads();  // everyone is done with the previous group's vectors
     if (tid < nvec) {
       float* dst = (pf_which == 0 ? aS : (pf_which == 1 ? bS : wS)) + pf_sl * d + 4 * pf_t4;
-      *reinterpret_cast<float4*>(dst) = pf;
+#pragma unroll
+      for (int ee = 0; ee < SA_E; ++ee) *reinterpret_cast<float4*>(dst + ee * K * d) = pf[ee];
     }
-    if (tid < K) cS[tid] = a.index[tid * n + e];
     __syncthreads();
-    if (e + 1 < n) pf = fetch(e + 1);
+    if (e0 + SA_E < n) fetch(e0 + SA_E, pf);
 
-    // alpha[s][j] = a_s . k[j],  beta[s][i] = q[i] . b_s
-    for (int it = tid; it < 2 * K * n; it += SA_NT) {
-      const int which = it / (K * n), sl = (it / n) % K, x = it % n;
-      const float* u = (which == 0 ? aS : bS) + sl * d;
-      const float* m = (which == 0 ? kS : qS) + x * dp;
-      (which == 0 ? alS : beS)[sl * n + x] = sa_dot(u, m, d4);
+    // alpha[e][s][j] = a_es . k[j],  beta[e][s][i] = q[i] . b_es,  gp[e][s] = a_es . b_es
+    const int items = 2 * ne * K * n;
+    for (int it = tid; it < items + ne * K; it += SA_NT) {
+      if (it < items) {
+        const int which = it / (ne * K * n), r = it - which * (ne * K * n);
+        const int es = r / n, x = r - es * n;  // es = ee * K + sl
+        const float* u = (which == 0 ? aS : bS) + es * d;
+        const float* m = (which == 0 ? kS : qS) + x * dp;
+        (which == 0 ? alS : beS)[es * n + x] = sa_dot(u, m, d4);
+      } else {
+        const int es = it - items;
+        gpS[es] = sa_dot(aS + es * d, bS + es * d, d4);
+      }
     }
     __syncthreads();
-    // rho[s] = sum_j p[e][j] alpha[s][j],  gamma[s] = sum_j p[e][j] alpha[s][j] v[j]
-    for (int it = tid; it < K * d4; it += SA_NT) {
-      const int sl = it / d4, t4 = it - sl * d4;
+    // rho[e][s] = sum_j p[e][j] alpha[e][s][j],  gamma[e][s] = sum_j p[e][j] alpha[e][s][j] v[j]
+    for (int it = tid; it < ne * K * d4; it += SA_NT) {
+      const int es = it / d4, t4 = it - es * d4;
+      const int e = e0 + es / K;
       float rho = 0.0f;
       float4 gm = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll 8
       for (int j = 0; j < n; ++j) {
-        const float pa = pS[e * np1 + j] * alS[sl * n + j];
+        const float pa = pS[e * np1 + j] * alS[es * n + j];
         const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * t4);
         rho += pa;
         gm.x += pa * vv.x; gm.y += pa * vv.y; gm.z += pa * vv.z; gm.w += pa * vv.w;
       }
-      *reinterpret_cast<float4*>(gamS + sl * d + 4 * t4) = gm;
-      if (t4 == 0) rhoS[sl] = rho;
+      *reinterpret_cast<float4*>(gamS + es * d + 4 * t4) = gm;
+      if (t4 == 0) rhoS[es] = rho;
     }
     __syncthreads();
 
-    // output rows of this position's slots, and their part of 2 sum_c p'_c[:, e] w_c
-    for (int sl = 0; sl < K; ++sl) {
-      const int c = cS[sl];
-      if (c < 0) continue;
-      const float rho = rhoS[sl];
-      const float ale = alS[sl * n + e];
-      if (ot4 < d4) {
-        const float4 w4 = *reinterpret_cast<const float4*>(wS + sl * d + 4 * ot4);
-        const float4 g4 = *reinterpret_cast<const float4*>(gamS + sl * d + 4 * ot4);
+    // output rows of the group's slots, and their part of 2 sum_c p'_c[:, e] w_c
+    if (ot4 < d4) {
+      for (int ee = 0; ee < ne; ++ee) {
+        const int e = e0 + ee;
         const float4 v4 = *reinterpret_cast<const float4*>(vS + e * dp + 4 * ot4);
         const float4 o4 = *reinterpret_cast<const float4*>(oS + e * dp + 4 * ot4);
-        const float wv[4] = {w4.x, w4.y, w4.z, w4.w}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
-        const float ve[4] = {v4.x, v4.y, v4.z, v4.w}, oe[4] = {o4.x, o4.y, o4.z, o4.w};
+        float pie[SA_MAXPASS];
 #pragma unroll
-        for (int ps = 0; ps < SA_MAXPASS; ++ps) {
-          const int i = ps * 16 + orow;
-          if (i < n) {
-            const float pie = pS[i * np1 + e];
-            const float bi = beS[sl * n + i];
-            const float4 oi4 = *reinterpret_cast<const float4*>(oS + i * dp + 4 * ot4);
-            const float oi[4] = {oi4.x, oi4.y, oi4.z, oi4.w};
-            float r[4];
+        for (int ps = 0; ps < SA_MAXPASS; ++ps) pie[ps] = (ps * 16 + orow < n) ? pS[(ps * 16 + orow) * np1 + e] : 0.0f;
+        for (int sl = 0; sl < K; ++sl) {
+          const int c = idxS[sl * n + e];
+          if (c < 0) continue;
+          const int es = ee * K + sl;
+          const float rho = rhoS[es];
+          const float ale = alS[es * n + e];
+          const float4 w4 = *reinterpret_cast<const float4*>(wS + es * d + 4 * ot4);
+          const float4 g4 = *reinterpret_cast<const float4*>(gamS + es * d + 4 * ot4);
+          float* dst = a.oj + (int64_t)c * Srow + 4 * ot4;
 #pragma unroll
-            for (int x = 0; x < 4; ++x) {
-              r[x] = pie * (wv[x] + bi * (ve[x] - oi[x]));
-              if (i == e) r[x] += gv[x] - rho * oe[x];
+          for (int ps = 0; ps < SA_MAXPASS; ++ps) {
+            const int i = ps * 16 + orow;
+            if (i < n) {
+              const float bi = beS[es * n + i];
+              const float4 oi = oreg[ps];
+              float4 r;
+              r.x = pie[ps] * (w4.x + bi * (v4.x - oi.x));
+              r.y = pie[ps] * (w4.y + bi * (v4.y - oi.y));
+              r.z = pie[ps] * (w4.z + bi * (v4.z - oi.z));
+              r.w = pie[ps] * (w4.w + bi * (v4.w - oi.w));
+              float cf = pie[ps] * bi * (1.0f - pie[ps]);
+              if (i == e) {
+                r.x += g4.x - rho * o4.x; r.y += g4.y - rho * o4.y;
+                r.z += g4.z - rho * o4.z; r.w += g4.w - rho * o4.w;
+                cf += pie[ps] * (ale - rho);
+              }
+              folx_st_stream4(dst + grow(i), r);
+              t2acc[ps].x += cf * w4.x; t2acc[ps].y += cf * w4.y;
+              t2acc[ps].z += cf * w4.z; t2acc[ps].w += cf * w4.w;
             }
-            folx_st_stream4(a.oj + (int64_t)c * Srow + grow(i) + 4 * ot4, make_float4(r[0], r[1], r[2], r[3]));
-            float cf = pie * bi * (1.0f - pie);
-            if (i == e) cf += pie * (ale - rho);
-            t2acc[ps].x += cf * wv[0]; t2acc[ps].y += cf * wv[1];
-            t2acc[ps].z += cf * wv[2]; t2acc[ps].w += cf * wv[3];
           }
         }
       }
     }
-    // n x n sums over this position's slots
-    if (tid < n) {
-      const int j = tid;
+    // n x n sums over the slots of each position of the group
+    for (int it = tid; it < ne * n; it += SA_NT) {
+      const int ee = it / n, j = it - ee * n;
+      const int e = e0 + ee;
       const float pee = pS[e * np1 + e];
       float aa = 0.0f, ar = 0.0f, bb = 0.0f;
       for (int sl = 0; sl < K; ++sl) {
-        const float al = alS[sl * n + j], be = beS[sl * n + j];
-        const float rr = rhoS[sl] + pee * beS[sl * n + e];
+        const int es = ee * K + sl;
+        const float al = alS[es * n + j], be = beS[es * n + j];
+        const float rr = rhoS[es] + pee * beS[es * n + e];
         aa += al * al;
         ar += al * rr;
         bb += be * be;
@@ -234,15 +266,18 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
       AR[e * np1 + j] = ar;
       BB[j * np1 + e] = bb;
     }
-    if (tid == SA_NT - 1) {
+    if (tid >= SA_NT - ne) {
+      const int ee = SA_NT - 1 - tid;
+      const int e = e0 + ee;
       const float pee = pS[e * np1 + e];
       float d1 = 0.0f, d2 = 0.0f, r2 = 0.0f, g = 0.0f;
       for (int sl = 0; sl < K; ++sl) {
-        const float ale = alS[sl * n + e], bee = beS[sl * n + e], rho = rhoS[sl];
+        const int es = ee * K + sl;
+        const float ale = alS[es * n + e], bee = beS[es * n + e], rho = rhoS[es];
         d1 += 2.0f * ale * bee;
         d2 += bee * rho;
         r2 += rho * rho + 2.0f * rho * pee * bee;
-        g += sa_dot(aS + sl * d, bS + sl * d, d4);
+        g += gpS[es];
       }
       D1[e] = d1; D2[e] = d2; R2a[e] = r2; gS[e] = g;
     }
