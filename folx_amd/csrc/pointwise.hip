@@ -75,6 +75,54 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
   }
 }
 
+// Product of a triplet with a dense Jacobian (P rows) and one of the same shape whose Jacobian
+// is sparse (k rows, slot s of element i standing for dense row idx[s][i % S_w]; no row named
+// twice per element):
+//   y = a b,  y_jac[p] = b a_jac[p] + a sum_{s: idx[s] = p} b_jac[s],
+//   y_lap = b a_lap + a b_lap + 2 sum_s a_jac[idx[s]] b_jac[s].
+// Same work split as binary_kernel; each lane keeps its k sparse rows and their indices in
+// registers, so the dense rows of the sparse operand are never built.
+template <int KMAX>
+__global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void mul_sparse_kernel(
+    const float* __restrict__ a, const float* __restrict__ aj, const float* __restrict__ al,
+    const float* __restrict__ b, const float* __restrict__ bj, const float* __restrict__ bl,
+    const int32_t* __restrict__ idx, float* __restrict__ y, float* __restrict__ yj, float* __restrict__ yl,
+    int64_t S, int64_t S_w, int32_t P, int32_t k) {
+  __shared__ float red[PSPLIT][FOLX_WAVE];
+  const int lane = threadIdx.x % FOLX_WAVE;
+  const int w = threadIdx.x / FOLX_WAVE;
+  const int64_t i = (int64_t)blockIdx.x * FOLX_WAVE + lane;
+  const bool active = i < S;
+  float sab = 0.0f, av = 0.0f, bv = 0.0f;
+  if (active) {
+    av = a[i];
+    bv = b[i];
+    const int64_t pos = i % S_w;
+    int32_t ix[KMAX];
+    float bs[KMAX];
+#pragma unroll
+    for (int s = 0; s < KMAX; ++s) {
+      ix[s] = s < k ? idx[(int64_t)s * S_w + pos] : -1;
+      bs[s] = ix[s] >= 0 ? bj[(int64_t)s * S + i] : 0.0f;
+    }
+    for (int p = w; p < P; p += PSPLIT) {
+      const float ja = __builtin_nontemporal_load(&aj[(int64_t)p * S + i]);
+      float o = bv * ja;
+#pragma unroll
+      for (int s = 0; s < KMAX; ++s)
+        if (ix[s] == p) { o += av * bs[s]; sab += ja * bs[s]; }
+      __builtin_nontemporal_store(o, &yj[(int64_t)p * S + i]);
+    }
+  }
+  red[w][lane] = sab;
+  __syncthreads();
+  if (w == 0 && active) {
+    const float s = red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane];
+    y[i] = av * bv;
+    yl[i] = bv * al[i] + av * bl[i] + 2.0f * s;
+  }
+}
+
 __global__ __launch_bounds__(256) void rows_affine_kernel(const float* __restrict__ in,
                                                           float* __restrict__ out, int64_t rows,
                                                           int64_t in_S, int64_t S,
@@ -142,5 +190,29 @@ extern "C" int folx_hip_rows_affine(void* stream, const float* in, float* out, i
   const unsigned gy = (unsigned)(rows < 1024 ? rows : 1024);
   rows_affine_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
       in, out, rows, in_S, S, c, d, alpha, beta, iin, ic, id);
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_mul_sparse_fwdlap(void* stream, const float* a, const float* a_jac, const float* a_lap,
+                                          const float* b, const float* b_jac, const float* b_lap,
+                                          const int32_t* index, float* y, float* y_jac, float* y_lap, int64_t S,
+                                          int64_t S_w, int32_t P, int32_t k_rows) {
+  if (S < 0 || S_w <= 0 || P < 0 || k_rows < 0) return FOLX_HIP_EINVAL;
+  if (S == 0) return FOLX_HIP_OK;
+  if (S % S_w != 0) return FOLX_HIP_EINVAL;
+  if (!a || !a_lap || !b || !b_lap || !y || !y_lap || (P > 0 && (!a_jac || !y_jac)) ||
+      (k_rows > 0 && (!b_jac || !index)))
+    return FOLX_HIP_EINVAL;
+  if (k_rows > 8) return FOLX_HIP_ENOTSUP;
+  const int64_t blocks = (S + FOLX_WAVE - 1) / FOLX_WAVE;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  dim3 grid((unsigned)blocks), block(FOLX_WAVE * PSPLIT);
+  hipStream_t st = (hipStream_t)stream;
+  if (k_rows <= 4)
+    mul_sparse_kernel<4><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
+                                                 k_rows);
+  else
+    mul_sparse_kernel<8><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
+                                                 k_rows);
   return folx_launch_status();
 }

@@ -257,6 +257,28 @@ def binary(op, a, aj, al, b, bj, bl):
     return y, yj, yl
 
 
+def mul_sparse(a, aj, al, b, bj, bl, index):
+    """``a * b`` for triplets of one shape (B, *s): ``aj`` dense (P, B, *s), ``bj`` sparse
+    (k, B, *s) with ``index`` int32 (k, prod(s)) on the device naming the dense row of each
+    slot.  Returns the triplet with P dense rows."""
+    _chk(a, aj, al, b, bj, bl, index)
+    assert tuple(a.shape) == tuple(b.shape)
+    P, k = aj.shape[0], bj.shape[0]
+    S = a.numel()
+    S_w = S // a.shape[0]
+    assert tuple(index.shape) == (k, S_w) and index.dtype == torch.int32
+    y, yj, yl = torch.empty_like(a), torch.empty_like(aj), torch.empty_like(a)
+    with _timed('mul_sparse_fwdlap', (S, P, k)):
+        check(
+            _lib.load().folx_hip_mul_sparse_fwdlap(
+                _stream(), _p(a), _p(aj), _p(al), _p(b), _p(bj), _p(bl), _p(index), _p(y), _p(yj), _p(yl),
+                S, S_w, P, k,
+            ),
+            'mul_sparse_fwdlap',
+        )
+    return y, yj, yl
+
+
 def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta=1.0):
     """out[r] = alpha * in[r] * c + beta * d with broadcasting to ``out_shape``.
     ``inp`` holds ``rows`` rows of shape ``row_shape``; c / d are arrays broadcastable to

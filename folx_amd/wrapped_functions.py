@@ -315,6 +315,17 @@ def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLapl
         y, J, lap = K.binary(op, a.x, Ja, a.laplacian, b.x, Jb, b.laplacian)
         return FwdLaplArray(y, FwdJacobian(J, mask), lap)
 
+    if op == 'mul' and a.jacobian.weak != b.jacobian.weak and tuple(a.shape) == tuple(b.shape):
+        # one dense, one sparse operand of the same shape: the product takes the sparse rows
+        # as they are (same result as densifying them first, which is what follows otherwise)
+        dn, sp = (b, a) if a.jacobian.weak else (a, b)
+        m = np.broadcast_to(sp.jacobian.x0_idx, (sp.jacobian.x0_idx.shape[0], *out_shape))
+        k = m.shape[0]
+        if k <= 8 and sp.jacobian.max_n < dn.jacobian.data.shape[0] and not ia.has_duplicates(m):
+            table = so.device_table(np.ascontiguousarray(m.reshape(k, -1)), a.x.device)
+            y, J, lap = K.mul_sparse(dn.x, dn.jacobian.data, dn.laplacian, sp.x, sp.jacobian.data, sp.laplacian,
+                                     table)
+            return FwdLaplArray(y, FwdJacobian(J, None), lap)
     if not (a.jacobian.weak and b.jacobian.weak):
         # Any dense operand: the reference adds the per-operand results through
         # FwdJacobian.__add__, which densifies (folx/jvp.py:742-796, folx/api.py:233-236).

@@ -168,6 +168,20 @@ int folx_hip_binary_fwdlap(void* stream, int32_t op, const float* a, const float
                            const int64_t* dims, int64_t a_S, int64_t b_S, int32_t P);
 
 /*
+ * Product of two triplets of one shape, a with a dense Jacobian (P rows) and b with a sparse
+ * one (k_rows rows): slot s of element i stands for the dense row index[s][i % S_w]
+ * (int32 [k_rows][S_w], S_w = elements per walker, -1 = empty slot, no row named twice per
+ * element, all < P).  The case of FwdJacobian.__add__ with one dense operand
+ * (folx/api.py:233-236) inside the mul rule (folx/wrapped_functions.py:375-377,
+ * folx/hessian.py:177-188), without first densifying b.
+ *   a, b, *_lap, y, y_lap [S]   a_jac, y_jac [P][S]   b_jac [k_rows][S]      k_rows <= 8
+ */
+int folx_hip_mul_sparse_fwdlap(void* stream, const float* a, const float* a_jac,
+                               const float* a_lap, const float* b, const float* b_jac,
+                               const float* b_lap, const int32_t* index, float* y, float* y_jac,
+                               float* y_lap, int64_t S, int64_t S_w, int32_t P, int32_t k_rows);
+
+/*
  * Fused LayerNorm over the last axis, y = gamma * (x - mean) * rsqrt(var + eps) + beta,
  * for R rows of F features (F % 4 == 0, F <= 1024); gamma / beta [F] or NULL.
  *   x [R][F]   jac [P][R][F]   lap [R][F]   ->   y, y_jac, y_lap of the same shapes.

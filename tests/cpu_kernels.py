@@ -64,6 +64,20 @@ def binary(op, a, aj, al, b, bj, bl):
     return tuple(_t(t) for t in rule(*A, *Bb))
 
 
+def mul_sparse(a, aj, al, b, bj, bl, index):
+    ix = index.cpu().numpy()
+    bjn = _n(bj)
+    P = aj.shape[0]
+    dense = np.zeros((P, *bjn.shape[1:]))
+    flat = dense.reshape(P, bjn.shape[1], -1)
+    src = bjn.reshape(bjn.shape[0], bjn.shape[1], -1)
+    for s in range(ix.shape[0]):
+        for e in range(ix.shape[1]):
+            if ix[s, e] >= 0:
+                flat[ix[s, e], :, e] += src[s, :, e]
+    return tuple(_t(t) for t in rules.mul_rule(_n(a), _n(aj), _n(al), _n(b), dense, _n(bl)))
+
+
 def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta=1.0):
     a = _n(inp).reshape(rows, *row_shape)
     nd = len(out_shape)
@@ -186,7 +200,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'dense_act', 'layernorm', 'elementwise', 'binary', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'dense_act', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

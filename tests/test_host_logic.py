@@ -480,3 +480,24 @@ def test_value_only_functions():
     np.testing.assert_array_equal(seen['and'].data.numpy() != 0, (h > 0) & (h < 0.5))
     np.testing.assert_array_equal(seen['not'].data.numpy() != 0, ~(h > 0))
     np.testing.assert_array_equal(seen['int'].data.numpy(), np.trunc(3.0 * h))
+
+
+def test_dense_times_sparse_keeps_the_sparse_rows(monkeypatch):
+    """``mul`` of a dense-Jacobian triplet with a sparse one of the same shape goes to the
+    kernel that reads the sparse rows in place; the result equals the densified rule."""
+    from folx_amd import kernels as K
+
+    calls = []
+    orig = K.mul_sparse
+    monkeypatch.setattr(K, 'mul_sparse', lambda *a: (calls.append(tuple(a[6].shape)), orig(*a))[1])
+    rng = np.random.default_rng(16)
+    W = rng.normal(size=(3, 4)).astype(np.float32)
+    x = rng.normal(size=(2, 5, 3)).astype(np.float32)
+
+    def fn(xp, r):
+        env = xp.exp(xp.multiply(xp.dot(r, W), -0.3))                   # (5, 4), k = 3 per node
+        mixed = xp.tanh(xp.add(env, xp.mean(env, axis=0, keepdims=True)))   # dense: every node sees all
+        return xp.sum(xp.multiply(mixed, env))
+
+    check_against_oracle(fn, x, 6)
+    assert calls == [(3, 20)]

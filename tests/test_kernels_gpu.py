@@ -432,6 +432,29 @@ def test_mhsa_sparse(B, n, H, d, k, missing):
     assert_lap(got[2], full[2].double().cpu().numpy(), 'o_lap vs dense kernel')
 
 
+@pytest.mark.parametrize('B,shape,P,k', [(3, (5, 7), 12, 3), (2, (16, 256), 96, 3), (1, (4,), 5, 1), (2, (3, 3), 20, 6)])
+def test_mul_sparse(B, shape, P, k):
+    """Product of a dense-Jacobian triplet with a sparse-Jacobian one against the mul rule on
+    the densified operand."""
+    from folx_amd import kernels as K
+
+    print(f'case mul_sparse B={B} shape={shape} P={P} k={k}', flush=True)
+    rng = np.random.default_rng(22)
+    S_w = int(np.prod(shape))
+    table = np.stack([rng.permutation(P)[:k] for _ in range(S_w)], 1).astype(np.int32)   # distinct rows per element
+    table[rng.uniform(size=table.shape) < 0.15] = -1
+    a, aj, al = rand(rng, B, *shape), rand(rng, P, B, *shape), rand(rng, B, *shape)
+    b, bj, bl = rand(rng, B, *shape), rand(rng, k, B, *shape), rand(rng, B, *shape)
+    dense = np.zeros((P, B, S_w))
+    for s_ in range(k):
+        for e in range(S_w):
+            if table[s_, e] >= 0:
+                dense[table[s_, e], :, e] += bj.reshape(k, B, S_w)[s_, :, e]
+    ref = rules.mul_rule(*f64(a, aj, al, b), dense.reshape(P, B, *shape), bl.astype(np.float64))
+    got = K.mul_sparse(dev(a), dev(aj), dev(al), dev(b), dev(bj), dev(bl), dev(table, torch.int32))
+    assert_triplet(got, ref, 'mul_sparse')
+
+
 @pytest.mark.parametrize('rows,F,P', [((3, 5), 8, 4), ((2, 32), 256, 9), ((7,), 512, 3), ((4, 3), 100, 5),
                                       ((2, 2), 1024, 2), ((5,), 4, 1)])
 def test_layernorm(rows, F, P):
