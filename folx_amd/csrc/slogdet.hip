@@ -21,7 +21,7 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
-    int64_t rstride, int64_t slice) {
+    int64_t rstride, int64_t slice, int32_t share) {
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
   constexpr int G = FOLX_WAVE / NP;    // lane groups per row
   constexpr int CPL = NP / G;          // columns of M per lane
@@ -32,7 +32,15 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   __shared__ float mb[NP * MS];
 
   const int lane = threadIdx.x;
-  const int64_t m = blockIdx.x;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  When `share`
+  // neighbouring matrices lie in the same 128-byte lines (rows of n floats side by side), they
+  // are given to the same XCD in consecutive slots, so that every line comes from HBM once.
+  int64_t m = blockIdx.x;
+  if (share > 1) {
+    const int64_t chunk = 8 * (int64_t)share;
+    const int64_t c = m / chunk, r = m % chunk;
+    if ((c + 1) * chunk <= NM) m = c * chunk + (r % 8) * share + r / 8;
+  }
   // matrix m = (batch m / ND, member m % ND); element (i, j) at base + i * rstride + j
   const int64_t base = (m / ND) * bstride + (m % ND) * dstride;
   const float* a = A + base;
@@ -209,9 +217,15 @@ extern "C" int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, con
   if (n > 32 || NM > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)NM), block(FOLX_WAVE);
+  // members stored side by side along the rows with rows shorter than a 128-byte line
+  int32_t share = 1;
+  if (member_stride == n && n * 4 < 128 && ND > 1) {
+    share = 128 / (n * 4);
+    while (share > 1 && ND % share != 0) share /= 2;
+  }
 #define FOLX_SLD_LAUNCH(NPV)                                                                              \
   slogdet_kernel<NPV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND, \
-                                              batch_stride, member_stride, row_stride, jac_stride)
+                                              batch_stride, member_stride, row_stride, jac_stride, share)
   if (n <= 8) FOLX_SLD_LAUNCH(8);
   else if (n <= 16) FOLX_SLD_LAUNCH(16);
   else FOLX_SLD_LAUNCH(32);
