@@ -26,6 +26,7 @@ SIGNATURES = {
     'folx_hip_dense_act_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 8 + [c_int64, c_int32, c_int32, c_int32, _P, c_int64]),
     'folx_hip_layernorm_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_float]),
     'folx_hip_elementwise_fwdlap': (c_int, [_P, c_int32, c_float, _P, _P, _P, _P, _P, _P, c_int64, c_int32]),
+    'folx_hip_exp_envelope_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_binary_fwdlap': (c_int, [_P, c_int32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int64, c_int32]),
     'folx_hip_mul_sparse_fwdlap': (c_int, [_P] * 11 + [c_int64, c_int64, c_int32, c_int32]),
     'folx_hip_rows_affine': (c_int, [_P, _P, _P, c_int64, c_int64, _P, _P, c_float, c_float, _P]),

@@ -152,3 +152,82 @@ extern "C" int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float para
 #undef FOLX_CASE
   return FOLX_HIP_EINVAL;
 }
+
+// Exponential envelope, a fused chain of broadcast, scale, exp, scale and sum:
+//   y[r][o] = sum_I pi[I][o] exp(-sigma[I][o] d[r][I])
+// for a triplet d with few columns I (distances of one electron to the nuclei) and constant
+// sigma, pi.  The function is a sum of scalar functions of the single d[r][I], so with
+// t = pi exp(-sigma d):
+//   y_jac[p] = sum_I (-sigma t) d_jac[p][I],
+//   y_lap    = sum_I (-sigma t) d_lap[I] + sum_I sigma^2 t sum_p d_jac[p][I]^2.
+// A thread owns four consecutive o of one row r; a wavefront therefore reads the same few d
+// values (broadcast loads) and writes 1 KB of every output row.  The kernel reads almost
+// nothing and is bound by writing (P + 2) R O floats.
+namespace {
+
+constexpr int ENV_MAX_I = 8;
+
+__global__ __launch_bounds__(256) void exp_envelope_kernel(const float* __restrict__ d, const float* __restrict__ dj,
+                                                           const float* __restrict__ dl,
+                                                           const float* __restrict__ sigma,
+                                                           const float* __restrict__ pi, float* __restrict__ y,
+                                                           float* __restrict__ yj, float* __restrict__ yl, int64_t R,
+                                                           int32_t nI, int32_t O, int32_t P) {
+  const int O4 = O / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= R * O4) return;
+  const int64_t r = idx / O4;
+  const int o = (int)(idx - r * O4) * 4;
+  float4 g[ENV_MAX_I];  // -sigma t per column I
+  float4 val = make_float4(0.f, 0.f, 0.f, 0.f), lap = val;
+#pragma unroll
+  for (int I = 0; I < ENV_MAX_I; ++I) {
+    g[I] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (I < nI) {
+      const float dv = d[r * nI + I], lv = dl[r * nI + I];
+      float ss = 0.0f;
+      for (int p = 0; p < P; ++p) { const float j = dj[((int64_t)p * R + r) * nI + I]; ss += j * j; }
+      const float4 s4 = *reinterpret_cast<const float4*>(sigma + (int64_t)I * O + o);
+      const float4 p4 = *reinterpret_cast<const float4*>(pi + (int64_t)I * O + o);
+      const float sv[4] = {s4.x, s4.y, s4.z, s4.w}, pv[4] = {p4.x, p4.y, p4.z, p4.w};
+      float t[4], gg[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) { t[x] = pv[x] * expf(-sv[x] * dv); gg[x] = -sv[x] * t[x]; }
+      g[I] = make_float4(gg[0], gg[1], gg[2], gg[3]);
+      val.x += t[0]; val.y += t[1]; val.z += t[2]; val.w += t[3];
+      lap.x += gg[0] * lv + sv[0] * sv[0] * t[0] * ss; lap.y += gg[1] * lv + sv[1] * sv[1] * t[1] * ss;
+      lap.z += gg[2] * lv + sv[2] * sv[2] * t[2] * ss; lap.w += gg[3] * lv + sv[3] * sv[3] * t[3] * ss;
+    }
+  }
+  *reinterpret_cast<float4*>(y + r * O + o) = val;
+  *reinterpret_cast<float4*>(yl + r * O + o) = lap;
+  for (int p = 0; p < P; ++p) {
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int I = 0; I < ENV_MAX_I; ++I)
+      if (I < nI) {
+        const float j = dj[((int64_t)p * R + r) * nI + I];
+        acc.x += g[I].x * j; acc.y += g[I].y * j; acc.z += g[I].z * j; acc.w += g[I].w * j;
+      }
+    folx_st_stream4(yj + ((int64_t)p * R + r) * O + o, acc);
+  }
+}
+
+}  // namespace
+
+extern "C" int folx_hip_exp_envelope_fwdlap(void* stream, const float* d, const float* d_jac, const float* d_lap,
+                                            const float* sigma, const float* pi, float* y, float* y_jac,
+                                            float* y_lap, int64_t R, int32_t n_cols, int32_t O, int32_t P) {
+  if (R < 0 || n_cols <= 0 || O <= 0 || P < 0) return FOLX_HIP_EINVAL;
+  if (R == 0) return FOLX_HIP_OK;
+  if (!d || !d_lap || !sigma || !pi || !y || !y_lap || (P > 0 && (!d_jac || !y_jac))) return FOLX_HIP_EINVAL;
+  if (n_cols > ENV_MAX_I || O % 4 != 0) return FOLX_HIP_ENOTSUP;
+  const void* ptrs[] = {sigma, pi, y, y_jac, y_lap};
+  for (const void* p : ptrs)
+    if (p && !folx_aligned16(p)) return FOLX_HIP_ENOTSUP;
+  const int64_t blocks = (R * (O / 4) + 255) / 256;
+  if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  exp_envelope_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(d, d_jac, d_lap, sigma, pi, y,
+                                                                                      y_jac, y_lap, R, n_cols, O, P);
+  return folx_launch_status();
+}

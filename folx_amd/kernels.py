@@ -181,6 +181,32 @@ def elementwise(name, x, jac, lap, param=0.0, inplace=False):
     return y, yj, yl
 
 
+def exp_envelope_supported(n_cols, O):
+    return 1 <= n_cols <= 8 and O % 4 == 0
+
+
+def exp_envelope(d, dj, dl, sigma, pi):
+    """``sum_I pi[I, o] exp(-sigma[I, o] d[..., I])``: d (.., nI), dj (P, .., nI), sigma / pi
+    (nI, O) -> triplet with last dim O."""
+    _chk(d, dj, dl, sigma, pi)
+    nI, O = sigma.shape
+    assert d.shape[-1] == nI and tuple(pi.shape) == (nI, O)
+    P = dj.shape[0]
+    lead = tuple(d.shape[:-1])
+    R = int(np.prod(lead, dtype=np.int64))
+    y = torch.empty((*lead, O), device=d.device, dtype=torch.float32)
+    yj = torch.empty((P, *lead, O), device=d.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    with _timed('exp_envelope_fwdlap', (R, nI, O, P)):
+        check(
+            _lib.load().folx_hip_exp_envelope_fwdlap(
+                _stream(), _p(d), _p(dj), _p(dl), _p(sigma), _p(pi), _p(y), _p(yj), _p(yl), R, nI, O, P
+            ),
+            'exp_envelope_fwdlap',
+        )
+    return y, yj, yl
+
+
 def layernorm(x, jac, lap, gamma, beta, eps):
     """Fused LayerNorm rule over the last axis."""
     _chk(x, jac, lap, gamma, beta)

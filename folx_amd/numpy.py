@@ -111,6 +111,13 @@ def layer_norm(h, gamma=None, beta=None, eps=1e-5):
     return _call('layer_norm', (h, gamma, beta), {'eps': eps})
 
 
+def exp_envelope(d, sigma, pi):
+    """``sum_I pi[I, o] exp(-sigma[I, o] d[..., I])``: exponential envelopes of orbitals from the
+    electron-nucleus distances ``d (.., n_nuc)`` and constant ``sigma``, ``pi (n_nuc, O)`` (one
+    fused rule; same result as the chain of primitives)."""
+    return _call('exp_envelope', (d, sigma, pi))
+
+
 def matmul(a, b):
     """``numpy.matmul`` for two operands of which at least one carries derivatives."""
     from .api import FwdLaplArray as _F

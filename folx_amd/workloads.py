@@ -185,8 +185,7 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         if m == 0:
             continue
         orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))  # (m, n_det * m), spin block read in place
-        ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)  # (m, nuc, 1)
-        env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
+        env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])  # (m, n_det * m)
         orb = xp.multiply(orb, env)
         # (electron, determinant, orbital): the matrices are read in place, rows on axis 0
         sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
@@ -299,8 +298,7 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         if m == 0:
             continue
         orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))
-        ds = xp.expand_dims(xp.getitem(dist, (slice(lo, hi),)), 2)
-        env = xp.sum(xp.multiply(xp.exp(xp.negative(xp.multiply(ds, p.env_sigma[s]))), p.env_pi[s]), axis=1)
+        env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])
         orb = xp.multiply(orb, env)
         sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
         logdets.append(ld), signs.append(sg)

@@ -633,6 +633,34 @@ def layer_norm_rule(args, kwargs, sparsity_threshold):
     return FwdLaplArray(y, FwdJacobian(Jy, mask), lapy)
 
 
+def exp_envelope_rule(args, kwargs, sparsity_threshold):
+    """Fused rule of ``exp_envelope(d, sigma, pi) = sum_I pi[I, o] exp(-sigma[I, o] d[..., I])``,
+    a custom registered function like ``layer_norm``.  The fused kernel applies when the
+    Jacobian of ``d`` is dense, or sparse with a mask that is constant along the last axis and
+    lists no index twice; other inputs go through the chain of primitive rules
+    (broadcast, mul, neg, exp, mul, reduce_sum), which also defines the result."""
+    d, sigma, pi = args
+    nI, O = (int(v) for v in sigma.shape)
+    fusable = _is(d) and K.exp_envelope_supported(nI, O) and d.shape[-1] == nI
+    mask = d.jacobian.x0_idx if _is(d) else None
+    if fusable and mask is not None:
+        first = np.take(mask, [0], axis=-1)
+        fusable = bool((mask == first).all()) and not ia.has_duplicates(mask)
+    if not fusable:
+        from . import numpy as fnp
+
+        e = fnp.exp(fnp.negative(fnp.multiply(fnp.expand_dims(d, -1), sigma)))
+        return fnp.sum(fnp.multiply(e, pi), axis=-2)
+    dev = d.x.device
+    y, Jy, lapy = K.exp_envelope(d.x, d.jacobian.data, d.laplacian, so.device_const(sigma, dev),
+                                 so.device_const(pi, dev))
+    new_mask = None
+    if mask is not None:
+        first = np.take(np.broadcast_to(mask, (mask.shape[0], *d.shape)), [0], axis=-1)
+        new_mask = np.broadcast_to(first, (mask.shape[0], *d.shape[:-1], O))
+    return FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
+
+
 # --------------------------------------------------------------------------------------
 # reductions
 # --------------------------------------------------------------------------------------
@@ -1376,6 +1404,7 @@ register_function('min', _binary_rule('min'))
 register_function('max', _binary_rule('max'))
 register_function('dot_general', dot_general)
 register_function('layer_norm', layer_norm_rule)
+register_function('exp_envelope', exp_envelope_rule)
 register_function('reduce_sum', reduce_sum)
 register_function('reshape', reshape_rule)
 register_function('transpose', transpose_rule)

@@ -130,6 +130,21 @@ int folx_hip_elementwise_fwdlap(void* stream, int32_t act, float param, const fl
                                 float* y_lap, int64_t S, int32_t P);
 
 /*
+ * Exponential envelope  y[r][o] = sum_I pi[I][o] exp(-sigma[I][o] d[r][I])  of a triplet d with
+ * n_cols <= 8 columns and constant sigma, pi [n_cols][O]: the chain broadcast_in_dim, mul,
+ * neg, exp, mul, reduce_sum that the reference interprets rule by rule (elementwise rules
+ * folx/jvp.py:687-697 / folx/hessian.py:87-112 around LINEAR ones, folx/wrapped_functions.py:361-392)
+ * and XLA fuses afterwards, as one pass that only writes the result.
+ *   d [R][n_cols]  d_jac [P][R][n_cols]  d_lap [R][n_cols]   y [R][O]  y_jac [P][R][O]  y_lap [R][O]
+ * O % 4 == 0.  For a sparse d_jac the rows must not name an index twice per position (the rule
+ * uses sum_p d_jac[p]^2 as in folx/hessian.py:460-470).
+ */
+int folx_hip_exp_envelope_fwdlap(void* stream, const float* d, const float* d_jac,
+                                 const float* d_lap, const float* sigma, const float* pi, float* y,
+                                 float* y_jac, float* y_lap, int64_t R, int32_t n_cols, int32_t O,
+                                 int32_t P);
+
+/*
  * Narrow dense layer followed by its activation, in one pass:
  *   y = f(x @ W + bias),  y_jac[p] = f'(z) * (jac[p] @ W),
  *   y_lap = f'(z) * (lap @ W) + f''(z) * sum_p (jac[p] @ W)^2,      z = x @ W + bias.

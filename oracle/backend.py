@@ -379,6 +379,12 @@ def dot(h: OArr, W, b=None, residual=None, row_slice=None, act=None):
     return out if residual is None else add(residual, out)
 
 
+def exp_envelope(d, sigma, pi):
+    """Exponential envelope as the chain of primitive rules the reference interprets it with."""
+    e = exp(negative(multiply(expand_dims(d, -1), np.asarray(sigma))))
+    return sum(multiply(e, np.asarray(pi)), axis=-2)
+
+
 def layer_norm(h: OArr, gamma=None, beta=None, eps=1e-5):
     """LayerNorm as the chain of primitive rules the reference interprets it with."""
     mu = mean(h, axis=-1, keepdims=True)

@@ -34,6 +34,10 @@ class plain:
         return y if residual is None else residual + y
 
     @staticmethod
+    def exp_envelope(d, sigma, pi):
+        return (torch.exp(-d[..., None] * plain._c(sigma, d)) * plain._c(pi, d)).sum(-2)
+
+    @staticmethod
     def layer_norm(h, gamma=None, beta=None, eps=1e-5):
         mu = h.mean(-1, keepdim=True)
         c = h - mu

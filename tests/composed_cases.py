@@ -41,6 +41,13 @@ CASES = {
         xp.split(xp.sin(x), 2), xp.split(xp.tanh(x), [6]))], axis=1), (2, 1)),
     'dynamic_slices': lambda xp, x: xp.dynamic_update_slice(
         xp.reshape(xp.sin(x), (3, 4)), xp.dynamic_slice(xp.reshape(xp.square(x), (3, 4)), (1, 2), (2, 2)), (0, 1)),
+    # fused exponential envelope: dense input, and (in the host / GPU tests with a threshold) sparse
+    'exp_envelope': lambda xp, x: xp.exp_envelope(
+        xp.add(xp.square(xp.reshape(x, (4, 3))), 0.3),
+        np.linspace(0.4, 1.6, 24, dtype=np.float32).reshape(3, 8), np.cos(np.arange(24, dtype=np.float32)).reshape(3, 8)),
+    'exp_envelope_mixed_rows': lambda xp, x: xp.exp_envelope(
+        xp.reshape(xp.add(xp.square(xp.dot(xp.reshape(x, (4, 3)), np.ones((3, 3), dtype=np.float32))), 0.3), (4, 3)),
+        np.linspace(0.4, 1.6, 12, dtype=np.float32).reshape(3, 4), np.cos(np.arange(12, dtype=np.float32)).reshape(3, 4)),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }

@@ -37,6 +37,13 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
 
 
+def exp_envelope(d, dj, dl, sigma, pi):
+    from oracle import backend as ob
+
+    out = ob.exp_envelope(ob.OArr(_n(d), _n(dj), _n(dl)), _n(sigma), _n(pi))
+    return _t(out.x), _t(out.J), _t(out.lap)
+
+
 def layernorm(x, jac, lap, gamma, beta, eps):
     from oracle import backend as ob
 
@@ -200,7 +207,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'dense_act', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'dense_act', 'exp_envelope', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

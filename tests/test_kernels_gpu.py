@@ -455,6 +455,22 @@ def test_mul_sparse(B, shape, P, k):
     assert_triplet(got, ref, 'mul_sparse')
 
 
+@pytest.mark.parametrize('rows,nI,O,P', [((3, 16), 4, 256, 3), ((2, 5), 3, 8, 7), ((1, 1), 1, 4, 0), ((4, 8), 8, 64, 48)])
+def test_exp_envelope(rows, nI, O, P):
+    """Fused exponential envelope against the chain of primitive rules evaluated by the oracle."""
+    from folx_amd import kernels as K
+    from oracle import backend as ob
+
+    print(f'case exp_envelope rows={rows} nI={nI} O={O} P={P}', flush=True)
+    rng = np.random.default_rng(23)
+    d, J, L = np.abs(rand(rng, *rows, nI)) + 0.2, rand(rng, P, *rows, nI), rand(rng, *rows, nI)
+    sigma, pi = np.abs(rand(rng, nI, O)) + 0.3, rand(rng, nI, O)
+    ref = ob.exp_envelope(ob.OArr(*f64(d, J, L)), sigma.astype(np.float64), pi.astype(np.float64))
+    assert K.exp_envelope_supported(nI, O)
+    got = K.exp_envelope(dev(d), dev(J), dev(L), dev(sigma), dev(pi))
+    assert_triplet(got, (ref.x, ref.J, ref.lap), 'exp_envelope')
+
+
 @pytest.mark.parametrize('rows,F,P', [((3, 5), 8, 4), ((2, 32), 256, 9), ((7,), 512, 3), ((4, 3), 100, 5),
                                       ((2, 2), 1024, 2), ((5,), 4, 1)])
 def test_layernorm(rows, F, P):
