@@ -107,7 +107,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       const int a4 = (idx % (DP / 4)) * 4;
       float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
       if (FAST || (idx < TILE4 && j < n && a4 < d && (!mask_rows || valid(j))))
-        val = *reinterpret_cast<const float4*>(src + base + (int64_t)j * tok + a4);
+        val = folx_ld_stream4(src + base + (int64_t)j * tok + a4);  // every tile is read once
       reg[i] = val;
     }
   };
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
       const int a4 = 4 * lg + 16 * t;
       float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
       if (FAST || (qrow < n && a4 < d && (!mask_rows || valid(qrow))))
-        val = *reinterpret_cast<const float4*>(src + base + (int64_t)qrow * tok + a4);
+        val = folx_ld_stream4(src + base + (int64_t)qrow * tok + a4);
       reg[t] = val;
     }
   };
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(FOLX_WAVE * NW) void mhsa_kernel(MhsaArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) p[16 * dt] = c[dt][r];
+        for (int dt = 0; dt < DT; ++dt) __builtin_nontemporal_store(c[dt][r], &p[16 * dt]);
         p += tok;
       }
     } else {
