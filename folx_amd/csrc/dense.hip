@@ -90,7 +90,7 @@ __device__ __forceinline__ void store_tile(const floatx16 (&acc)[TM][TN], const 
             char* p = (char*)(cs + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
             float o = acc[i][j][4 * g + r] + bvals[j];
             if constexpr (HAS_RES) o += rs[r];
-            *(float*)(p + voff) = o;
+            __builtin_nontemporal_store(o, (float*)(p + voff));  // written once, read by a later launch
           }
         }
       }
