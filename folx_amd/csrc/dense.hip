@@ -82,7 +82,7 @@ __device__ __forceinline__ void store_tile(const floatx16 (&acc)[TM][TN], const 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const char* p = (const char*)(rsb + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
-              rs[r] = *(const float*)(p + voff);
+              rs[r] = __builtin_nontemporal_load((const float*)(p + voff));
             }
           }
 #pragma unroll
