@@ -37,6 +37,7 @@ SIGNATURES = {
     'folx_hip_scatter_add_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int64, c_int64, c_int64]),
     'folx_hip_slogdet_fwdlap': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int32, c_int32]),
     'folx_hip_slogdet_strided_fwdlap': (c_int, [_P] * 8 + [c_int64, c_int64, c_int32, c_int32] + [c_int64] * 4),
+    'folx_hip_slogdet_scaled_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int64, c_int32, c_int32] + [c_int64] * 5 + [c_int32]),
     'folx_hip_sparse_slogdet_fwdlap': (c_int, [_P] * 11 + [c_int64] + [c_int32] * 6),
     'folx_hip_inv_fwdlap': (c_int, [_P] * 7 + [c_int64, c_int32, c_int32]),
     'folx_hip_solve_fwdlap': (c_int, [_P] * 10 + [c_int64, c_int32, c_int32, c_int32]),

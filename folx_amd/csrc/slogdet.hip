@@ -16,12 +16,25 @@ namespace {
 
 using smallmat::wave_sum;
 
-template <int NP>
+// Optional elementwise factor: the matrices are A * F with F a triplet of A's layout whose
+// Jacobian is sparse (kf <= KF rows, slot s of the element at per-walker position q standing for
+// dense row fidx[s][q]).  Product rule on load:
+//   (A F)_jac[p] = F A_jac[p] + A sum_{s: fidx[s] = p} F_jac[s],
+//   (A F)_lap    = F A_lap + A F_lap + 2 sum_s A_jac[fidx[s]] F_jac[s].
+struct Factor {
+  const float *x, *jac, *lap;   // F [..], F_jac [kf][..] (row stride = `slice`), F_lap [..]
+  const int32_t* idx;           // [kf][S_w]
+  int64_t S_w;                  // elements per walker
+  int32_t kf;
+};
+constexpr int KF = 4;
+
+template <int NP, bool HAS_F>
 __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
-    int64_t rstride, int64_t slice, int32_t share) {
+    int64_t rstride, int64_t slice, int32_t share, Factor fc) {
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
   constexpr int G = FOLX_WAVE / NP;    // lane groups per row
   constexpr int CPL = NP / G;          // columns of M per lane
@@ -46,8 +59,8 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   const float* a = A + base;
 
   float logdet, sgn;
-  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn, rstride);
-  float tl = smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
+  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn, rstride, HAS_F ? fc.x + base : nullptr);
+  float tl = HAS_F ? 0.0f : smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
 
   // ---- row i of A^-1 in registers -------------------------------------------------------
   const int i = lane % NP;
@@ -57,6 +70,28 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
 #pragma unroll
   for (int j = 0; j < NP; ++j) ainv[j] = aug[i * AUGS + NP + j];
 
+  // this lane's EPL elements of the padded tile; with a factor also its values at them
+  constexpr int EF = HAS_F ? EPL : 1;
+  float fx[EF], ax[EF], lapx[EF], fj[KF][EF];
+  int32_t fidx[KF][EF];
+  if constexpr (HAS_F) {
+#pragma unroll
+    for (int c = 0; c < EPL; ++c) {
+      const int e = lane + c * FOLX_WAVE;
+      const int r = e / NP, cc = e % NP;
+      const bool ok = r < n && cc < n;
+      const int64_t off = base + r * rstride + cc;
+      fx[c] = ok ? fc.x[off] : 0.0f;
+      ax[c] = ok ? A[off] : 0.0f;
+      lapx[c] = 0.0f;
+#pragma unroll
+      for (int sl = 0; sl < KF; ++sl) {
+        fidx[sl][c] = (ok && sl < fc.kf) ? fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w] : -1;
+        fj[sl][c] = fidx[sl][c] >= 0 ? fc.jac[(int64_t)sl * slice + off] : 0.0f;
+      }
+    }
+  }
+
   float mm = 0.0f;
   float pre[EPL];
   auto prefetch = [&](int p) {
@@ -65,7 +100,15 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     for (int c = 0; c < EPL; ++c) {
       const int e = lane + c * FOLX_WAVE;  // index into the padded NP x NP tile
       const int r = e / NP, cc = e % NP;
-      pre[c] = (r < n && cc < n) ? src[r * rstride + cc] : 0.0f;
+      float v = (r < n && cc < n) ? src[r * rstride + cc] : 0.0f;
+      if constexpr (HAS_F) {
+        float add = 0.0f;
+#pragma unroll
+        for (int sl = 0; sl < KF; ++sl)
+          if (fidx[sl][c] == p) { add += fj[sl][c]; lapx[c] += 2.0f * v * fj[sl][c]; }
+        v = fx[c] * v + ax[c] * add;
+      }
+      pre[c] = v;
     }
   };
   if (P > 0) prefetch(0);
@@ -112,6 +155,18 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     for (int c = 0; c < CPL; ++c) mm += acc[c] * mb[(col0 + c) * MS + i];
     // the next iteration writes the other jb buffer; mb is rewritten only after the
     // barrier that follows that write, when every lane is past this read
+  }
+  if constexpr (HAS_F) {
+#pragma unroll
+    for (int c = 0; c < EPL; ++c) {
+      const int e = lane + c * FOLX_WAVE;
+      const int r = e / NP, cc = e % NP;
+      if (r < n && cc < n) {
+        const int64_t off = base + r * rstride + cc;
+        const float al = fx[c] * AL[off] + ax[c] * fc.lap[off] + lapx[c];
+        tl += aug[cc * AUGS + NP + r] * al;  // tr(A^-1 lap A) = sum A^-1[c][r] lap A[r][c]
+      }
+    }
   }
   mm = wave_sum(mm);
   tl = wave_sum(tl);
@@ -204,6 +259,37 @@ __global__ __launch_bounds__(FOLX_WAVE) void sparse_slogdet_kernel(
 
 }  // namespace
 
+namespace {
+
+int launch_slogdet(hipStream_t st, const float* A, const float* A_jac, const float* A_lap, float* sign, float* logdet,
+                   float* ld_jac, float* ld_lap, int64_t NB, int64_t ND, int32_t n, int32_t P, int64_t batch_stride,
+                   int64_t member_stride, int64_t row_stride, int64_t jac_stride, const Factor* fc) {
+  const int64_t NM = NB * ND;
+  dim3 grid((unsigned)NM), block(FOLX_WAVE);
+  // members stored side by side along the rows with rows shorter than a 128-byte line
+  int32_t share = 1;
+  if (member_stride == n && n * 4 < 128 && ND > 1) {
+    share = 128 / (n * 4);
+    while (share > 1 && ND % share != 0) share /= 2;
+  }
+#define FOLX_SLD_LAUNCH(NPV, HASF)                                                                             \
+  slogdet_kernel<NPV, HASF><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND, \
+                                                    batch_stride, member_stride, row_stride, jac_stride, share,  \
+                                                    fc ? *fc : Factor{})
+  if (fc) {
+    if (n <= 8) FOLX_SLD_LAUNCH(8, true);
+    else FOLX_SLD_LAUNCH(16, true);
+  } else {
+    if (n <= 8) FOLX_SLD_LAUNCH(8, false);
+    else if (n <= 16) FOLX_SLD_LAUNCH(16, false);
+    else FOLX_SLD_LAUNCH(32, false);
+  }
+#undef FOLX_SLD_LAUNCH
+  return folx_launch_status();
+}
+
+}  // namespace
+
 extern "C" int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, const float* A_jac,
                                                const float* A_lap, float* sign, float* logdet,
                                                float* ld_jac, float* ld_lap, int64_t NB, int64_t ND,
@@ -215,22 +301,28 @@ extern "C" int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, con
   if (NM == 0) return FOLX_HIP_OK;
   if (!A || !A_lap || !sign || !logdet || !ld_lap || (P > 0 && (!A_jac || !ld_jac))) return FOLX_HIP_EINVAL;
   if (n > 32 || NM > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-  hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned)NM), block(FOLX_WAVE);
-  // members stored side by side along the rows with rows shorter than a 128-byte line
-  int32_t share = 1;
-  if (member_stride == n && n * 4 < 128 && ND > 1) {
-    share = 128 / (n * 4);
-    while (share > 1 && ND % share != 0) share /= 2;
-  }
-#define FOLX_SLD_LAUNCH(NPV)                                                                              \
-  slogdet_kernel<NPV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND, \
-                                              batch_stride, member_stride, row_stride, jac_stride, share)
-  if (n <= 8) FOLX_SLD_LAUNCH(8);
-  else if (n <= 16) FOLX_SLD_LAUNCH(16);
-  else FOLX_SLD_LAUNCH(32);
-#undef FOLX_SLD_LAUNCH
-  return folx_launch_status();
+  return launch_slogdet((hipStream_t)stream, A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NB, ND, n, P,
+                        batch_stride, member_stride, row_stride, jac_stride, nullptr);
+}
+
+extern "C" int folx_hip_slogdet_scaled_fwdlap(void* stream, const float* A, const float* A_jac, const float* A_lap,
+                                              const float* F, const float* F_jac, const float* F_lap,
+                                              const int32_t* index, float* sign, float* logdet, float* ld_jac,
+                                              float* ld_lap, int64_t NB, int64_t ND, int32_t n, int32_t P,
+                                              int64_t batch_stride, int64_t member_stride, int64_t row_stride,
+                                              int64_t jac_stride, int64_t walker_elems, int32_t k_rows) {
+  if (NB < 0 || ND <= 0 || n <= 0 || P < 0 || row_stride < n || walker_elems <= 0 || k_rows < 0)
+    return FOLX_HIP_EINVAL;
+  const int64_t NM = NB * ND;
+  if (NM == 0) return FOLX_HIP_OK;
+  if (!A || !A_lap || !F || !F_lap || !sign || !logdet || !ld_lap || (P > 0 && (!A_jac || !ld_jac)) ||
+      (k_rows > 0 && (!F_jac || !index)))
+    return FOLX_HIP_EINVAL;
+  if (n > 16 || k_rows > KF || NM > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  Factor fc;
+  fc.x = F; fc.jac = F_jac; fc.lap = F_lap; fc.idx = index; fc.S_w = walker_elems; fc.kf = k_rows;
+  return launch_slogdet((hipStream_t)stream, A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NB, ND, n, P,
+                        batch_stride, member_stride, row_stride, jac_stride, &fc);
 }
 
 extern "C" int folx_hip_slogdet_fwdlap(void* stream, const float* A, const float* A_jac,

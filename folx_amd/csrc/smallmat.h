@@ -25,14 +25,17 @@ struct Aug {
 // wavefront of the workgroup.
 template <int NP>
 __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict__ a, int n, int lane,
-                                             float& logdet, float& sgn, int64_t row_stride = 0) {
+                                             float& logdet, float& sgn, int64_t row_stride = 0,
+                                             const float* __restrict__ factor = nullptr) {
   if (row_stride == 0) row_stride = n;  // rows of the matrix follow each other
   constexpr int AUGS = Aug<NP>::stride;
   constexpr int RK = (2 * NP + FOLX_WAVE - 1) / FOLX_WAVE;
   for (int e = lane; e < NP * 2 * NP; e += FOLX_WAVE) {
     const int i = e / (2 * NP), j = e % (2 * NP);
     float v;
-    if (j < NP) v = (i < n && j < n) ? a[i * row_stride + j] : (i == j ? 1.0f : 0.0f);
+    // with `factor` (same layout as a) the matrix is the elementwise product a * factor
+    if (j < NP) v = (i < n && j < n) ? a[i * row_stride + j] * (factor ? factor[i * row_stride + j] : 1.0f)
+                                     : (i == j ? 1.0f : 0.0f);
     else v = (j - NP == i) ? 1.0f : 0.0f;
     aug[i * AUGS + j] = v;
   }

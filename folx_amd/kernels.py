@@ -397,11 +397,17 @@ def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
     return out
 
 
-def slogdet(A, AJ, AL, row_axis=None):
+def slogdet_scaled_supported(n, k_rows):
+    return n <= 16 and k_rows <= 4
+
+
+def slogdet(A, AJ, AL, row_axis=None, factor=None):
     """A (.., n, n), AJ (P, .., n, n), AL (.., n, n) -> sign, logdet (..), jac (P, ..), lap (..).
     ``row_axis`` (an axis of A, default the one before last) names the axis that holds the
     matrix rows; the last axis holds the columns and every other axis is a batch axis, in
-    order.  The matrices are read in place, whatever ``row_axis``."""
+    order.  The matrices are read in place, whatever ``row_axis``.  ``factor = (F, FJ, FL,
+    index)``: the matrices are ``A * F`` with F of A's shape, FJ (k, ..) sparse rows and
+    ``index`` int32 (k, elements per walker) naming their dense rows."""
     _chk(A, AJ, AL)
     n = A.shape[-1]
     P = AJ.shape[0]
@@ -416,6 +422,21 @@ def slogdet(A, AJ, AL, row_axis=None):
     ld = torch.empty_like(sign)
     ldj = torch.empty((P, *lead), device=A.device, dtype=torch.float32)
     ldl = torch.empty_like(sign)
+    if factor is not None:
+        F, FJ, FL, index = factor
+        _chk(F, FJ, FL, index)
+        assert tuple(F.shape) == tuple(A.shape) and tuple(FJ.shape[1:]) == tuple(A.shape)
+        S_w = A.numel() // A.shape[0]
+        assert tuple(index.shape) == (FJ.shape[0], S_w) and index.dtype == torch.int32
+        with _timed('slogdet_scaled_fwdlap', (NB * ND, n, P, FJ.shape[0])):
+            check(
+                _lib.load().folx_hip_slogdet_scaled_fwdlap(
+                    _stream(), _p(A), _p(AJ), _p(AL), _p(F), _p(FJ), _p(FL), _p(index), _p(sign), _p(ld), _p(ldj),
+                    _p(ldl), NB, ND, n, P, n * ND * n, n, ND * n, A.numel(), S_w, FJ.shape[0]
+                ),
+                'slogdet_scaled_fwdlap',
+            )
+        return sign, ld, ldj, ldl
     with _timed('slogdet_fwdlap', (NB * ND, n, P)):
         check(
             _lib.load().folx_hip_slogdet_strided_fwdlap(

@@ -133,12 +133,14 @@ def matmul(a, b):
     return np.matmul(a, b)
 
 
-def slogdet(A, row_axis=None):
+def slogdet(A, row_axis=None, factor=None):
     """``numpy.linalg.slogdet`` over the last two axes; ``row_axis`` names another axis as the
     one holding the matrix rows (columns stay on the last axis, all other axes are batch axes
     in their order), which reads e.g. a dense layer's output (electron, determinant, orbital)
-    in place."""
-    return _call('slogdet', (A,), {'row_axis': row_axis})
+    in place.  ``factor`` (same shape as ``A``): the matrices are ``A * factor``; orbitals times
+    envelopes are then multiplied while the matrices are loaded.  Same result as
+    ``slogdet(multiply(A, factor))``."""
+    return _call('slogdet', (A,), {'row_axis': row_axis, 'factor': factor})
 
 
 def det(A):

@@ -186,9 +186,10 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
             continue
         orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))  # (m, n_det * m), spin block read in place
         env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])  # (m, n_det * m)
-        orb = xp.multiply(orb, env)
-        # (electron, determinant, orbital): the matrices are read in place, rows on axis 0
-        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
+        # (electron, determinant, orbital): the matrices are read in place, rows on axis 0, and
+        # multiplied by their envelopes while they are loaded
+        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
+                            factor=xp.reshape(env, (m, cfg.n_det, m)))
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
@@ -299,8 +300,8 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
             continue
         orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))
         env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])
-        orb = xp.multiply(orb, env)
-        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0)
+        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
+                            factor=xp.reshape(env, (m, cfg.n_det, m)))
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])

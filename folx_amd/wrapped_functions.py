@@ -1193,6 +1193,26 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
     if not _is(A):
         raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
     row_axis = kwargs.get('row_axis')
+    factor = kwargs.get('factor')
+    if factor is not None:
+        # slogdet(A * factor): with a dense A and a sparse factor of the same shape the product is
+        # formed inside the slogdet kernel; any other combination is the mul rule first
+        fused = None
+        if _is(factor) and not A.jacobian.weak and factor.jacobian.weak and tuple(factor.shape) == tuple(A.shape):
+            m = np.broadcast_to(factor.jacobian.x0_idx, (factor.jacobian.x0_idx.shape[0], *A.shape))
+            k = m.shape[0]
+            if (K.slogdet_scaled_supported(A.shape[-1], k) and factor.jacobian.max_n < A.jacobian.data.shape[0]
+                    and not ia.has_duplicates(m)):
+                fused = (factor.x.contiguous(), factor.jacobian.data.contiguous(), factor.laplacian.contiguous(),
+                         so.device_table(np.ascontiguousarray(m.reshape(k, -1)), A.x.device))
+        if fused is None:
+            A = _LAPLACE_FN_REGISTRY['mul']((A, factor), {}, sparsity_threshold)
+        else:
+            ra = None if row_axis is None else row_axis % A.ndim
+            assert A.shape[ra if ra is not None else -2] == A.shape[-1], 'slogdet needs square matrices'
+            sign, ld, ldj, ldl = K.slogdet(A.x.contiguous(), A.jacobian.data.contiguous(), A.laplacian.contiguous(),
+                                           None if ra is None else ra + 1, fused)
+            return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
     if row_axis is not None and row_axis % A.ndim != A.ndim - 2:
         # matrix rows on another axis than the one before last
         ra = row_axis % A.ndim

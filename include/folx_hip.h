@@ -302,6 +302,23 @@ int folx_hip_slogdet_strided_fwdlap(void* stream, const float* A, const float* A
                                     int64_t jac_stride);
 
 /*
+ * slogdet of the elementwise product A * F, where F is a triplet of A's layout whose Jacobian
+ * is sparse: F_jac [k_rows][..] with row stride jac_stride, slot s of the element at
+ * per-walker position q standing for dense row index[s][q] (int32 [k_rows][walker_elems], -1 =
+ * empty, all < P, no row named twice per element).  The mul rule (folx/wrapped_functions.py:375-377)
+ * applied on the fly in front of slogdet_wrapper (folx/slogdet.py:347-358): orbitals times
+ * envelopes never exist as a tensor.  Other arguments as in folx_hip_slogdet_strided_fwdlap.
+ * Built for n <= 16 and k_rows <= 4; FOLX_HIP_ENOTSUP otherwise.
+ */
+int folx_hip_slogdet_scaled_fwdlap(void* stream, const float* A, const float* A_jac,
+                                   const float* A_lap, const float* F, const float* F_jac,
+                                   const float* F_lap, const int32_t* index, float* sign,
+                                   float* logdet, float* ld_jac, float* ld_lap, int64_t NB,
+                                   int64_t ND, int32_t n, int32_t P, int64_t batch_stride,
+                                   int64_t member_stride, int64_t row_stride, int64_t jac_stride,
+                                   int64_t walker_elems, int32_t k_rows);
+
+/*
  * slogdet rule for a sparse Jacobian whose coordinates touch few rows, columns or entries
  * of A, from static rank-one factor tables shared by all NM matrices.
  *   A [NM][n][n]   A_jac [k][NM][n][n] (k stored rows)   A_lap [NM][n][n]

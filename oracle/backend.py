@@ -541,7 +541,9 @@ def det(A: OArr):
     return multiply(exp(ld), sg)
 
 
-def slogdet(A: OArr, row_axis=None):
+def slogdet(A: OArr, row_axis=None, factor=None):
+    if factor is not None:
+        A = multiply(A, factor)
     if row_axis is not None and row_axis % A.ndim != A.ndim - 2:
         perm = [a for a in range(A.ndim) if a != row_axis % A.ndim]
         perm.insert(A.ndim - 2, row_axis % A.ndim)

@@ -324,7 +324,9 @@ class plain:
         return torch.log(torch.abs(s)) + m.reshape(s.shape), torch.sign(s.detach())
 
     @staticmethod
-    def slogdet(A, row_axis=None):
+    def slogdet(A, row_axis=None, factor=None):
+        if factor is not None:
+            A = A * factor
         if row_axis is not None:
             A = torch.movedim(A, row_axis, -2)
         sign, ld = torch.linalg.slogdet(A)

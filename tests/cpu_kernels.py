@@ -145,8 +145,18 @@ def gather_cols(data, table, S_inner=1):
     return _t(out.reshape(RB, -1))
 
 
-def slogdet(A, AJ, AL, row_axis=None):
+def slogdet(A, AJ, AL, row_axis=None, factor=None):
     a, aj, al = _n(A), _n(AJ), _n(AL)
+    if factor is not None:
+        F, FJ, FL, index = factor
+        ix, fj = index.cpu().numpy(), _n(FJ)
+        dense = np.zeros_like(aj).reshape(aj.shape[0], aj.shape[1], -1)
+        src = fj.reshape(fj.shape[0], fj.shape[1], -1)
+        for s_ in range(ix.shape[0]):
+            for e in range(ix.shape[1]):
+                if ix[s_, e] >= 0:
+                    dense[ix[s_, e], :, e] += src[s_, :, e]
+        a, aj, al = rules.mul_rule(a, aj, al, _n(F), dense.reshape(aj.shape), _n(FL))
     if row_axis is not None:
         ra = row_axis % a.ndim
         a, al = np.moveaxis(a, ra, -2), np.moveaxis(al, ra, -2)

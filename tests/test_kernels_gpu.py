@@ -471,6 +471,40 @@ def test_exp_envelope(rows, nI, O, P):
     assert_triplet(got, (ref.x, ref.J, ref.lap), 'exp_envelope')
 
 
+@pytest.mark.parametrize('B,ND,n,P,k,strided', [(3, 4, 16, 48, 3, True), (2, 3, 8, 24, 3, True), (2, 2, 5, 9, 2, False),
+                                               (1, 16, 16, 96, 3, True), (2, 1, 3, 7, 4, False)])
+def test_slogdet_scaled(B, ND, n, P, k, strided):
+    """slogdet of A * F with the product formed on load (sparse Jacobian of F) against the mul
+    rule followed by the slogdet rule of the oracle."""
+    from folx_amd import kernels as K
+
+    print(f'case slogdet_scaled B={B} ND={ND} n={n} P={P} k={k} strided={strided}', flush=True)
+    rng = np.random.default_rng(24)
+    shape = (n, ND, n) if strided else (ND, n, n)
+    S_w = int(np.prod(shape))
+    diag = 1.5 * np.sqrt(n)    # diagonally dominant enough for fp32 at n = 16
+    A = rand(rng, B, *shape) + (0 if strided else diag * np.eye(n, dtype=np.float32))
+    if strided:
+        A = A + diag * np.eye(n, dtype=np.float32)[:, None, :]
+    AJ, AL = 0.3 * rand(rng, P, B, *shape), 0.3 * rand(rng, B, *shape)
+    F, FJ, FL = 1.0 + 0.2 * rand(rng, B, *shape), 0.3 * rand(rng, k, B, *shape), 0.3 * rand(rng, B, *shape)
+    table = np.stack([rng.permutation(P)[:k] for _ in range(S_w)], 1).astype(np.int32)
+    table[rng.uniform(size=table.shape) < 0.2] = -1
+    dense = np.zeros((P, B, S_w))
+    for s_ in range(k):
+        for e in range(S_w):
+            if table[s_, e] >= 0:
+                dense[table[s_, e], :, e] += FJ.reshape(k, B, S_w)[s_, :, e]
+    prod = rules.mul_rule(*f64(A, AJ, AL, F), dense.reshape(P, B, *shape), FL.astype(np.float64))
+    if strided:
+        prod = (np.moveaxis(prod[0], 1, 2), np.moveaxis(prod[1], 2, 3), np.moveaxis(prod[2], 1, 2))
+    sign, (ld, jac, lap) = rules.slogdet_rule(*prod)
+    got = K.slogdet(dev(A), dev(AJ), dev(AL), 1 if strided else None,
+                    (dev(F), dev(FJ), dev(FL), dev(table, torch.int32)))
+    np.testing.assert_array_equal(got[0].cpu().numpy(), sign)
+    assert_triplet(got[1:], (ld, jac, lap), 'slogdet_scaled')
+
+
 @pytest.mark.parametrize('rows,F,P', [((3, 5), 8, 4), ((2, 32), 256, 9), ((7,), 512, 3), ((4, 3), 100, 5),
                                       ((2, 2), 1024, 2), ((5,), 4, 1)])
 def test_layernorm(rows, F, P):
