@@ -27,9 +27,9 @@ PEAK_HBM_GBS = 8000.0
 # scaled by what the same counter reads for a plain 1 GiB copy: x2.000 and x1.000); the
 # figures and the commands are in profiles/psiformer32_forward_laplacian.txt.
 MEASURED_TRAFFIC_BYTES = {
-    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.701e9,
-    ('dense_fwdlap', (32768, 96, 256, 256, True)): 10.150e9,
-    ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.153e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.594e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, True)): 9.883e9,
+    ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.176e9,
 }
 
 
