@@ -22,6 +22,8 @@
 // live in LDS (rows of d + 4 floats, so that 16 threads reading 16 bytes each from 16
 // different rows cover all banks); dot products run on 128-bit LDS reads; the three vectors of
 // the next position are fetched while the current one is worked on.
+#include <atomic>
+
 #include "common.h"
 
 namespace {
@@ -381,9 +383,15 @@ extern "C" int folx_hip_mhsa_sparse_fwdlap(void* stream, const float* q, const f
   const size_t lds = (size_t)sa_lds_floats(n, d, k_rows) * sizeof(float);
   if (lds > 160 * 1024) return FOLX_HIP_ENOTSUP;
   if (lds > 64 * 1024) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(mhsa_sparse_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return FOLX_HIP_ENOTSUP;
+    // raised once per process to the largest size asked for so far (not a stream operation,
+    // and then never issued again inside a stream capture)
+    static std::atomic<size_t> granted{0};
+    if (lds > granted.load()) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(mhsa_sparse_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
+        return FOLX_HIP_ENOTSUP;
+      granted.store(160 * 1024);
+    }
   }
   SAArgs a;
   a.q = q; a.qs = q_jac; a.ql = q_lap; a.k = k; a.ks = k_jac; a.kl = k_lap; a.v = v; a.vs = v_jac; a.vl = v_lap;
