@@ -48,6 +48,13 @@ def test_argument_checks_return_error_codes(lib):
     assert lib.folx_hip_layernorm_fwdlap(*([null] * 9), 4, 8, 1, 1e-5) == _lib.EINVAL
     assert lib.folx_hip_mhsa_fwdlap(*([null] * 15), 1, 8, 1, 8, 1) == _lib.EINVAL
     assert lib.folx_hip_mhsea_fwdlap(*([null] * 18), 1, 8, 1, 8, 1) == _lib.EINVAL
+    assert lib.folx_hip_dense_act_fwdlap(null, 0, 0.0, *([null] * 8), 4, 1, 8, 8, null, 0) == _lib.EINVAL
+    assert lib.folx_hip_dense_act_workspace_bytes(-1, 1, 8, 8) == _lib.EINVAL
+    assert lib.folx_hip_mhsa_sparse_fwdlap(*([null] * 14), 1, 8, 1, 8, 3) == _lib.EINVAL
+    assert lib.folx_hip_mul_sparse_fwdlap(*([null] * 11), 8, 4, 2, 1) == _lib.EINVAL
+    assert lib.folx_hip_mul_sparse_fwdlap(*([null] * 11), 9, 4, 2, 1) == _lib.EINVAL       # S not a multiple of S_w
+    assert lib.folx_hip_exp_envelope_fwdlap(*([null] * 9), 4, 2, 8, 1) == _lib.EINVAL
+    assert lib.folx_hip_slogdet_scaled_fwdlap(*([null] * 12), 1, 1, 4, 1, 16, 0, 4, 16, 16, 1) == _lib.EINVAL
     # empty problems are fine and launch nothing
     assert lib.folx_hip_dense_fwdlap(*([null] * 12), 0, 1, 8, 8) == _lib.OK
     assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 0, 1) == _lib.OK
@@ -61,6 +68,21 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_mhsa_fwdlap(None, *([one] * 9), None, None, one, one, one, 1, 8, 1, 6, 1) == _lib.ENOTSUP
     assert lib.folx_hip_layernorm_fwdlap(None, one, one, one, None, None, one, one, one, 4, 6, 1, 1e-5) == _lib.ENOTSUP
     assert lib.folx_hip_layernorm_fwdlap(None, one, one, one, None, None, one, one, one, 4, 2048, 1, 1e-5) == _lib.ENOTSUP
+    # fused / structure-aware entry points outside the sizes they are built for: the caller takes
+    # the general rules instead
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 4, 1, 6, 8, None, 0) == _lib.ENOTSUP     # K % 4
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 4, 1, 256, 8, None, 0) == _lib.ENOTSUP   # K > 128
+    assert lib.folx_hip_dense_act_fwdlap(None, 3, 0.0, *([one] * 8), 4, 1, 8, 8, None, 0) == _lib.ENOTSUP     # log: not fused
+    assert lib.folx_hip_dense_act_workspace_bytes(64, 4, 8, 200) == _lib.ENOTSUP
+    assert lib.folx_hip_dense_act_workspace_bytes(1 << 20, 4, 100, 100) == 0                                  # no split
+    assert lib.folx_hip_dense_act_workspace_bytes(2000, 400, 100, 100) > 0                                    # rows split
+    assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 65, 1, 8, 3) == _lib.ENOTSUP
+    assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 8, 1, 6, 3) == _lib.ENOTSUP
+    assert lib.folx_hip_mul_sparse_fwdlap(None, *([one] * 10), 8, 4, 2, 9) == _lib.ENOTSUP
+    assert lib.folx_hip_exp_envelope_fwdlap(None, *([one] * 8), 4, 9, 8, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_exp_envelope_fwdlap(None, *([one] * 8), 4, 2, 6, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_slogdet_scaled_fwdlap(None, *([one] * 11), 1, 1, 32, 1, 1024, 0, 32, 1024, 1024, 1) == _lib.ENOTSUP
+    assert lib.folx_hip_slogdet_scaled_fwdlap(None, *([one] * 11), 1, 1, 8, 1, 64, 0, 8, 64, 64, 5) == _lib.ENOTSUP
 
 
 def test_product_fails_loudly_without_gpu():
