@@ -98,6 +98,11 @@ DENSE_CASES = [
     ((3, 50), 4, 832, 256, False),     # long K, ragged last row tile
     ((2, 70), 3, 32, 260, True),       # two column tiles, the second nearly empty
     ((1, 130), 5, 64, 20, False),      # BN = 32 variant, more rows than one tile
+    # narrow outputs (N <= 4, K % 4 == 0): streaming kernel without MFMA
+    ((5, 33), 7, 64, 3, True),
+    ((2, 70), 3, 256, 4, True),
+    ((20, 100), 40, 100, 1, True),
+    ((1, 1), 0, 4, 2, False),
 ]
 
 
