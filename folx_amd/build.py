@@ -23,6 +23,7 @@ SOURCES = [
     'elementwise.hip',
     'dense.hip',
     'dense_act.hip',
+    'dense_act_wide.hip',
     'pointwise.hip',
     'reduce.hip',
     'gather.hip',

@@ -145,4 +145,27 @@ __device__ __forceinline__ void act_eval(float x, float prm, float& y, float& d1
   }
 }
 
+// The functions the fused dense + activation kernels take, chosen at run time.
+inline bool act_fused(int act) {
+  switch (act) {
+    case FOLX_ACT_TANH: case FOLX_ACT_SILU: case FOLX_ACT_LOGISTIC: case FOLX_ACT_SOFTPLUS:
+    case FOLX_ACT_EXP: case FOLX_ACT_SIN: case FOLX_ACT_COS: case FOLX_ACT_SQUARE:
+      return true;
+  }
+  return false;
+}
+
+__device__ __forceinline__ void act_eval_fused(int act, float x, float prm, float& y, float& d1, float& d2) {
+  switch (act) {
+    case FOLX_ACT_TANH: act_eval<FOLX_ACT_TANH>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_SILU: act_eval<FOLX_ACT_SILU>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_LOGISTIC: act_eval<FOLX_ACT_LOGISTIC>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_SOFTPLUS: act_eval<FOLX_ACT_SOFTPLUS>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_EXP: act_eval<FOLX_ACT_EXP>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_SIN: act_eval<FOLX_ACT_SIN>(x, prm, y, d1, d2); break;
+    case FOLX_ACT_COS: act_eval<FOLX_ACT_COS>(x, prm, y, d1, d2); break;
+    default: act_eval<FOLX_ACT_SQUARE>(x, prm, y, d1, d2); break;
+  }
+}
+
 }  // namespace

@@ -23,6 +23,7 @@
 // workspace; a second, short launch with one workgroup per row tile recomputes f' and f''
 // from the x tile, adds the partials in a fixed order and produces the lap row.
 #include "activations.h"
+#include "dense_act_wide.h"
 
 namespace {
 
@@ -75,15 +76,6 @@ bool plan_dense_act(int64_t R, int32_t P, int32_t K, int32_t N, DAPlan& pl) {
   if (pl.row_tiles * pl.G > 0x7fffffffLL) return false;
   pl.ws_bytes = pl.G > 1 ? pl.row_tiles * pl.G * (int64_t)PART_PER_BLOCK * 4 : 0;
   return true;
-}
-
-bool act_fused(int act) {
-  switch (act) {
-    case FOLX_ACT_TANH: case FOLX_ACT_SILU: case FOLX_ACT_LOGISTIC: case FOLX_ACT_SOFTPLUS:
-    case FOLX_ACT_EXP: case FOLX_ACT_SIN: case FOLX_ACT_COS: case FOLX_ACT_SQUARE:
-      return true;
-  }
-  return false;
 }
 
 template <int KS, int WC>
@@ -325,7 +317,7 @@ void launch_da(hipStream_t st, DAParams prm, const DAPlan& pl) {
 extern "C" int64_t folx_hip_dense_act_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N) {
   DAPlan pl;
   if (R < 0 || P < 0) return FOLX_HIP_EINVAL;
-  if (!plan_dense_act(R, P, K, N, pl)) return FOLX_HIP_ENOTSUP;
+  if (!plan_dense_act(R, P, K, N, pl)) return folx_dense_act_wide_ws_bytes(R, P, K, N);
   return pl.ws_bytes;
 }
 
@@ -336,7 +328,9 @@ extern "C" int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param,
   if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
   if (!act_fused(act)) return FOLX_HIP_ENOTSUP;
   DAPlan pl;
-  if (!plan_dense_act(R, P, K, N, pl)) return FOLX_HIP_ENOTSUP;
+  if (!plan_dense_act(R, P, K, N, pl))
+    return folx_dense_act_wide((hipStream_t)stream, act, param, x, jac, lap, W, bias, y, y_jac, y_lap, R, P, K, N,
+                               workspace, workspace_bytes);
   if (R == 0) return FOLX_HIP_OK;
   if (!x || !lap || !W || !y || !y_lap || (P > 0 && (!jac || !y_jac))) return FOLX_HIP_EINVAL;
   if (!folx_aligned16(x) || !folx_aligned16(lap) || (P > 0 && !folx_aligned16(jac))) return FOLX_HIP_ENOTSUP;

@@ -32,8 +32,9 @@ class LaunchTimer:
 
     active = None
 
-    def __init__(self):
+    def __init__(self, only=None):
         self.records = []
+        self.only = None if only is None else frozenset(only)  # time these entry points only
 
     def __enter__(self):
         LaunchTimer.active = self
@@ -58,13 +59,15 @@ class _timed:
         self.name, self.key = name, key
 
     def __enter__(self):
-        if LaunchTimer.active is not None:
+        lt = LaunchTimer.active
+        self.e0 = None
+        if lt is not None and (lt.only is None or self.name in lt.only):
             self.e0 = torch.cuda.Event(enable_timing=True)
             self.e0.record()
 
     def __exit__(self, *exc):
         lt = LaunchTimer.active
-        if lt is not None:
+        if lt is not None and self.e0 is not None:
             e1 = torch.cuda.Event(enable_timing=True)
             e1.record()
             lt.records.append((self.name, self.key, self.e0, e1))
@@ -131,9 +134,14 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
 FUSED_ACTS = ('tanh', 'silu', 'logistic', 'sigmoid', 'softplus', 'exp', 'sin', 'cos', 'square')
 
 
-def dense_act_supported(name, K, N):
-    """Shapes and functions the fused dense + activation kernel is built for."""
-    return name in FUSED_ACTS and 4 <= K <= 128 and K % 4 == 0 and 1 <= N <= 128
+def dense_act_supported(name, K, N, rows=None):
+    """Shapes and functions the fused dense + activation kernels are built for: narrow layers
+    (K, N <= 128), and wide ones (N > 128, K a multiple of 16) over a multiple of 4 rows."""
+    if name not in FUSED_ACTS:
+        return False
+    if 4 <= K <= 128 and K % 4 == 0 and 1 <= N <= 128:
+        return True
+    return rows is not None and rows > 0 and rows % 4 == 0 and K % 16 == 0 and N > 128 and N % 4 == 0
 
 
 def dense_act(name, x, jac, lap, W, bias=None, param=0.0):

@@ -178,7 +178,7 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         att = xp.multi_head_self_attention(q, k, v)
         h = xp.dot(xp.reshape(att, (n, H * dh)), L['w_o'], None, residual=h)
         hn = layer_norm(xp, h, L['ln2_g'], L['ln2_b'], cfg.ln_eps)
-        h = xp.dot(xp.tanh(xp.dot(hn, L['w_1'], L['b_1'])), L['w_2'], L['b_2'], residual=h)
+        h = xp.dot(xp.dot(hn, L['w_1'], L['b_1'], act='tanh'), L['w_2'], L['b_2'], residual=h)
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, cfg.n_up), (cfg.n_up, n)]):
         m = hi - lo

@@ -545,7 +545,7 @@ def _dot_then_act(h, W, kwargs, thr: int):
     bias = kwargs.get('bias')
     fused = (
         _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
-        and K.dense_act_supported(act, *np.shape(W))
+        and K.dense_act_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1))
     )
     J = new_mask = None
     if fused:

@@ -134,6 +134,13 @@ DENSE_ACT_CASES = [
     ((5, 40), 64, 16, 128, True, 'cos'),
     ((2, 64), 31, 104, 100, False, 'square'),   # odd number of Jacobian rows
     ((1, 64), 100, 100, 100, True, 'tanh'),     # one row tile, many groups
+    # wide layers (N > 128): tiles of 4 positions x 32 Jacobian rows, activation in the GEMM's epilogue
+    ((2, 32), 96, 256, 256, True, 'tanh'),      # transformer MLP: three full groups of 32 Jacobian rows
+    ((3, 16), 48, 832, 256, True, 'tanh'),      # one-electron stream: last group of Jacobian rows half full
+    ((1, 8), 5, 16, 132, False, 'silu'),        # one chunk of K, column tile cut at 132, one partial group
+    ((1, 12), 33, 64, 512, True, 'softplus'),   # two column tiles, 1 row in the second group
+    ((1, 4), 64, 48, 300, True, 'sin'),         # second column tile cut at 44 columns
+    ((5, 4), 1, 32, 256, False, 'square'),      # a single Jacobian row
 ]
 
 
@@ -149,7 +156,7 @@ def test_dense_act(rows, P, Kd, N, bias, act):
     b = rand(rng, N) if bias else None
     z = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
     ref = rules.elementwise_rule(act, *z)
-    assert K.dense_act_supported(act, Kd, N)
+    assert K.dense_act_supported(act, Kd, N, rows=int(np.prod(rows)))
     for rep in range(2):  # the second call finds the counters as the first one left them
         got = K.dense_act(act, dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
         assert_triplet(got, ref, f'dense_act call {rep}')
@@ -170,6 +177,26 @@ def test_dense_act_matches_two_kernels_large():
     ref = K.elementwise('silu', *K.dense(x, J, L, W, b))
     for a, r, nm in zip(got, ref, ('x', 'jac', 'lap')):
         torch.testing.assert_close(a, r, rtol=2e-5, atol=2e-5, msg=lambda m: f'{nm}: {m}')
+
+
+def test_dense_act_wide_matches_two_kernels_large():
+    """A transformer MLP layer at a full chunk: the fused wide path and dense + elementwise
+    agree to rounding (the sums over Jacobian rows are taken in a different order)."""
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(6)
+    R, P, Kd, N = 256 * 32, 96, 256, 256
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.randn(R, Kd, device='cuda', generator=g)
+    W = torch.randn(Kd, N, device='cuda', generator=g) / 16
+    b = torch.randn(N, device='cuda', generator=g)
+    assert K.dense_act_supported('tanh', Kd, N, rows=R)
+    got = K.dense_act('tanh', x, J, L, W, b)
+    ref = K.elementwise('tanh', *K.dense(x, J, L, W, b))
+    for a, r, nm in zip(got, ref, ('x', 'jac', 'lap')):
+        torch.testing.assert_close(a, r, rtol=1e-4 if nm == 'lap' else 2e-5, atol=1e-3 if nm == 'lap' else 2e-5,
+                                   msg=lambda m: f'{nm}: {m}')
 
 
 @pytest.mark.parametrize('lead,n,lo,hi,P,Kd,N', [((5,), 32, 0, 16, 9, 256, 256), ((5,), 32, 16, 32, 9, 256, 256),
