@@ -27,9 +27,13 @@ PEAK_HBM_GBS = 8000.0
 # scaled by what the same counter reads for a plain 1 GiB copy: x2.000 and x1.000); the
 # figures and the commands are in profiles/psiformer32_forward_laplacian.txt.
 MEASURED_TRAFFIC_BYTES = {
-    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.594e9,
-    ('dense_fwdlap', (32768, 96, 256, 256, True)): 9.883e9,
-    ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.176e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, False)): 6.589e9,
+    ('dense_fwdlap', (32768, 96, 256, 256, True)): 9.891e9,
+    ('mhsa_fwdlap', (1024, 32, 4, 64, 96)): 13.177e9,
+    # fused entry points: the sum over their launches (weights fold, per-position rows, x / lap
+    # rows GEMM, Jacobian GEMM, finish)
+    ('norm_dense_fwdlap', (None, 32768, 96, 256, 256)): 7.379e9,
+    ('norm_dense_fwdlap', ('tanh', 32768, 96, 256, 256)): 7.615e9,
 }
 
 
@@ -173,6 +177,18 @@ def main():
                 'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
                 'kernel': f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
+    elif dname == 'norm_dense_fwdlap' or (dname == 'dense_act_fwdlap' and dkey[4] > 128):
+        # the wide fused rules: one GEMM over the Jacobian rows (tiles cut across Jacobian rows)
+        # plus short launches for the x / lap rows; the events bracket the whole entry point
+        act, R, P, Kd, N = dkey
+        flops = 2.0 * (P + 2) * R * Kd * N
+        achieved = flops / (dms / dn * 1e-3) / 1e12
+        norm = dname == 'norm_dense_fwdlap'
+        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
+                'kernel': f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}>'
+                          f' + the short launches of its entry point ({dname}), act={act} R={R} P={P} K={Kd} N={N}',
+                'launches': dn, 'avg_launch_ms': dms / dn}
     elif dname == 'dense_act_fwdlap':
         act, R, P, Kd, N = dkey
         nbytes = 4.0 * ((P + 2) * R * (Kd + N) + Kd * N)

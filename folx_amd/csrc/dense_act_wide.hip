@@ -1,22 +1,39 @@
-// Wide dense layer and its activation without the pass over the pre-activation Jacobian:
-//   z = x @ W + bias          y     = f(z)
-//   zj[p] = jac[p] @ W        yj[p] = f'(z) * zj[p]
-//   zl = lap @ W              yl    = f'(z) * zl + f''(z) * sum_p zj[p]^2
-// for N > 128 and K a multiple of 16 (the narrow layers have their own kernel).  The Jacobian
-// rows are (P * R) x K with R positions; an activation kernel after the GEMM would read and
-// write all of zj once more, here zj never reaches HBM.
+// Wide dense layer (N > 128, K a multiple of 16) with the elementwise work around it folded
+// into the GEMM over the Jacobian rows, so that neither the pre-activation Jacobian nor a
+// normalised copy of the input Jacobian goes through HBM:
 //
-// Three launches on the caller's stream:
-//  1. the plain dense kernel on the x and lap rows only (2 R of the (P + 2) R rows): z goes to
-//     y, zl to y_lap;
-//  2. the Jacobian GEMM below, whose 128-row tiles are cut ACROSS Jacobian rows: a tile holds
+//   (a) dense + activation                    y = f(x @ W + bias)
+//   (b) LayerNorm + dense                     y = LN(x) @ W + bias
+//   (c) LayerNorm + dense + activation        y = f(LN(x) @ W + bias)
+//
+// with LN(x) = gamma * xh + beta, xh = (x - mean) * rs, rs = rsqrt(var + eps) over the K
+// features of a position.  The Jacobian rows are (P * R) x K with R positions.
+//
+// Activation.  With z = ... @ W + bias, zj[p] and zl the pre-activation triplet,
+//   y = f(z),  yj[p] = f'(z) zj[p],  yl = f'(z) zl + f''(z) sum_p zj[p]^2.
+//
+// LayerNorm in front of a matrix product.  For a Jacobian row t (K features of one position)
+// with a = mean(t), b = mean(xh t):   LN'[t] = gamma rs (t - a - b xh), hence
+//   LN'[t] @ W = rs (t @ Wg - a w1 - b w2),   Wg = diag(gamma) W,  w1 = 1^T Wg,  w2 = xh @ Wg,
+// a rank-2 correction of the product of the RAW row with Wg; w2 = z - bias - beta @ W is known
+// from the x row.  The second-order term of LayerNorm, summed over Jacobian rows,
+//   rs^2 gamma (-2 V + xh (3 sum_p b_p^2 - sum_p q_p)),  V = sum_p b_p (t_p - a_p),
+//   q_p = mean(t_p^2) - a_p^2,
+// goes through W as  rs^2 (-2 sum_p b_p (t_p @ Wg - a_p w1) + w2 (3 sum b^2 - sum q)).
+// a_p, b_p and mean(t_p^2) are summed from the A tile while it feeds the MFMAs.
+//
+// Launches on the caller's stream:
+//  1. (LayerNorm only) fold gamma / beta into the weights (Wg, w1, c0 = bias + beta @ W), and
+//     one wavefront per position for xh, rs, LN(x) and the linear part of LN's lap row;
+//  2. the plain dense kernel on the x and lap rows only (2 R of the (P + 2) R rows): z goes to
+//     y, the linear part of zl to y_lap;
+//  3. the Jacobian GEMM below, whose 128-row tiles are cut ACROSS Jacobian rows: a tile holds
 //     4 consecutive positions x 32 consecutive p, ordered position-major, so that each 32 x 32
-//     accumulator block belongs to ONE position.  f'(z) of a block is then one value per lane
-//     (its column), the block is scaled by it on the way out, and the squares of the block sum
-//     to one value per column inside the wavefront (16 registers and the two lane halves).
-//     These sums go to the workspace, one (R, N) slab per group of 32 Jacobian rows;
-//  3. a short elementwise kernel that turns z into f(z) and zl into the lap row, adding the
-//     slabs in a fixed order.
+//     accumulator block belongs to ONE position.  f'(z), w1, w2 and rs of a block are then one
+//     value per lane (its column), and the sums over p inside a block stay inside the
+//     wavefront (16 registers and the two lane halves).  The sums go to the workspace, one
+//     (R, N) slab per group of 32 Jacobian rows;
+//  4. a short elementwise kernel that finishes y and y_lap, adding the slabs in a fixed order.
 //
 // The main loop is the one of the dense kernel: K in chunks of 16 through double-buffered LDS
 // tiles filled by global_load_lds_dwordx4, a 128 x 256 tile on 8 wavefronts of 64 x 64,
@@ -24,6 +41,8 @@
 // (lane l, register j of group t <-> k = 8 t + 4 (l / 32) + j), piece c of an A row stored at
 // slot c ^ ((row / 2) % 4).  Only the address a lane asks for differs: tile row m is
 // Jacobian row p0 + m % 32 of position r0 + m / 32.
+#include <type_traits>
+
 #include "activations.h"
 #include "dense_act_wide.h"
 
@@ -41,8 +60,9 @@ constexpr int WROWS = BM / WM, WCOLS = BN / WN;
 constexpr int TM = WROWS / 32, TN = WCOLS / 32;
 constexpr int TG = BK / 8;
 constexpr int NXCD = 8;
-constexpr int PT = 32;       // Jacobian rows of a tile
-constexpr int RT = BM / PT;  // positions of a tile
+constexpr int PT = 32;         // Jacobian rows of a tile
+constexpr int RT = BM / PT;    // positions of a tile
+constexpr int KMAX_NORM = 512; // xh of a tile's positions sits in LDS
 constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
 constexpr int A_LD = A_V4 / NT, W_LD = W_V4 / NT;
 static_assert(A_V4 % NT == 0 && W_V4 % NT == 0, "every thread loads the same number of pieces");
@@ -50,20 +70,30 @@ static_assert(TM * WM == RT, "one accumulator block row per position");
 
 struct WideParams {
   const float* jac;
-  const float* W;
-  const float* z;  // pre-activation values (R, N), bias included
+  const float* W;    // Wg with LayerNorm
+  const float* z;    // pre-activation values (R, N), bias included
+  const float* xhat; // (R, K)           LayerNorm only
+  const float* rs;   // (R)
+  const float2* wc;  // (N) pairs (w1, c0)
   float* y_jac;
-  float* part;     // (PG, R, N) sums of squares per group of PT Jacobian rows
+  float* ss;         // (PG, R, N) sums of zj^2 per group of PT Jacobian rows     activation only
+  float* s1;         // (PG, R, N) sums of b_p (t_p @ Wg - a_p w1)                LayerNorm only
+  float* sc;         // (PG, R, 2) sums of b_p^2 and of q_p
   int64_t R, row_tiles, pos_tiles;
   int32_t P, K, N, col_tiles, act;
   float prm;
 };
 
-__global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
+template <bool NORM, bool ACT>
+__global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   __shared__ __attribute__((aligned(16))) float As0[BM * BK];
   __shared__ __attribute__((aligned(16))) float As1[BM * BK];
   __shared__ __attribute__((aligned(16))) float Ws0[BK * BN];
   __shared__ __attribute__((aligned(16))) float Ws1[BK * BN];
+  __shared__ __attribute__((aligned(16))) float xhS[NORM ? RT * KMAX_NORM : 4];
+  __shared__ float zS[NORM ? RT * BN : 1];  // pre-activation values of the tile's positions and columns
+  __shared__ float2 wcS[NORM ? BN : 1];     // (w1, c0) of the tile's columns
+  __shared__ float rsS[RT];
 
   // ids are dealt round-robin to the XCDs: the column tiles of a row tile stay on one of them
   const int64_t id = blockIdx.x;
@@ -118,16 +148,33 @@ __global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
                                        FOLX_LPTR(&ws[(wave * 64 + NT * i) * 4]), 16, 0, 0);
   };
 
-  // pre-activation value of this lane's column at the position of each accumulator block
-  float zv[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      int gc = col0 + wc + j * 32 + l32;
+  // The first chunk is on its way while what the epilogue needs per position and column is
+  // staged in LDS: both are waited for together in front of the first barrier.
+  issue(0, As0, Ws0);
+  float zr[TM][TN];  // without LayerNorm there are registers to spare for them
+  if constexpr (NORM) {
+    for (int e = tid; e < RT * BN; e += NT) {
+      int gc = col0 + e % BN;
       if (gc >= N) gc = N - 1;
-      zv[i][j] = a.z[(r0 + wrow * TM + i) * N + gc];
+      zS[e] = a.z[(r0 + e / BN) * N + gc];
     }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        int gc = col0 + wc + j * 32 + l32;
+        if (gc >= N) gc = N - 1;
+        zr[i][j] = a.z[(r0 + wrow * TM + i) * N + gc];
+      }
+  }
+  if constexpr (NORM) {
+    // xh of the tile's RT positions: RT * K consecutive floats
+    const float4* src = reinterpret_cast<const float4*>(a.xhat + r0 * K);
+    for (int e = tid; e < RT * K / 4; e += NT) reinterpret_cast<float4*>(xhS)[e] = src[e];
+    if (tid < BN) wcS[tid] = a.wc[col0 + tid < N ? col0 + tid : N - 1];
+    if (tid < RT) rsS[tid] = a.rs[r0 + tid];
+  }
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -136,9 +183,16 @@ __global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  // LayerNorm's row sums are taken by ONE wavefront per tile row block and SIMD: block i of
+  // tile row group wrow by the wavefront with column index i + 2 * wrow.  That wavefront runs
+  // its own copy of the K loop; the others run the plain one.  Per tile row wr + 32 si + l32,
+  // over the k this lane half reads: sum t, sum xh t, sum t^2.
+  const int si = NORM ? (wave % WN) - 2 * wrow : -1;
+  float sa = 0.0f, sb = 0.0f, s2 = 0.0f;
 
   const int sw = (l32 / 2) % 4;
-  auto compute = [&](const float* as, const float* ws) __attribute__((always_inline)) {
+  auto compute = [&](const float* as, const float* ws, int kt, auto sblk) __attribute__((always_inline)) {
+    constexpr int SI = decltype(sblk)::value;
 #pragma unroll
     for (int tg = 0; tg < TG; ++tg) {
       float4 a4[TM];
@@ -150,6 +204,13 @@ __global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) b[j][q] = ws[(tg * 8 + lh * 4 + q) * BN + wc + j * 32 + l32];
+      if constexpr (SI >= 0) {
+        const float4 xv = *reinterpret_cast<const float4*>(&xhS[(wrow * TM + SI) * K + kt * BK + (tg * 2 + lh) * 4]);
+        const float4 t = a4[SI];
+        sa += (t.x + t.y) + (t.z + t.w);
+        sb = fmaf(t.x, xv.x, fmaf(t.y, xv.y, fmaf(t.z, xv.z, fmaf(t.w, xv.w, sb))));
+        s2 = fmaf(t.x, t.x, fmaf(t.y, t.y, fmaf(t.z, t.z, fmaf(t.w, t.w, s2))));
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
 #pragma unroll
@@ -166,20 +227,56 @@ __global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
   // The loads of a chunk are waited for at the end of the chunk before it; the barrier then
   // also says that every wavefront is done reading the buffer that is refilled next.
   const int KT = K / BK;
-  issue(0, As0, Ws0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  for (int kt = 0; kt < KT; kt += 2) {
-    if (kt + 1 < KT) issue(kt + 1, As1, Ws1);
-    compute(As0, Ws0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (kt + 1 < KT) {
-      if (kt + 2 < KT) issue(kt + 2, As0, Ws0);
-      compute(As1, Ws1);
+  auto kloop = [&](auto sblk) __attribute__((always_inline)) {
+    for (int kt = 0; kt < KT; kt += 2) {
+      if (kt + 1 < KT) issue(kt + 1, As1, Ws1);
+      compute(As0, Ws0, kt, sblk);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
+      if (kt + 1 < KT) {
+        if (kt + 2 < KT) issue(kt + 2, As0, Ws0);
+        compute(As1, Ws1, kt + 1, sblk);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+      }
     }
+  };
+  static_assert(TM == 2, "one loop copy per accumulator block row");
+  if (NORM && si == 0) kloop(std::integral_constant<int, 0>{});
+  else if (NORM && si == 1) kloop(std::integral_constant<int, 1>{});
+  else kloop(std::integral_constant<int, -1>{});
+
+  // The row sums go through LDS (the tiles are no longer read: the loop ended with a barrier)
+  // to the lanes that hold the rows' accumulators.
+  float2* st = reinterpret_cast<float2*>(As0) + wrow * TM * 32;  // [wrow][i][row] (a, b)
+  if constexpr (NORM) {
+    if (si >= 0 && si < TM) {
+      const float invK = 1.0f / (float)K;
+      const bool pv = p0 + l32 < P;
+      const float ta = sa + __shfl_xor(sa, 32, FOLX_WAVE);
+      const float tb = sb + __shfl_xor(sb, 32, FOLX_WAVE);
+      const float t2 = s2 + __shfl_xor(s2, 32, FOLX_WAVE);
+      const float av = pv ? ta * invK : 0.0f;
+      const float bv = pv ? tb * invK : 0.0f;
+      const float qv = pv ? t2 * invK - av * av : 0.0f;
+      if (lh == 0) st[si * 32 + l32] = make_float2(av, bv);
+      if (ct == 0) {  // the two scalar sums of the block
+        float eb = bv * bv, eq = qv;
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) {
+          eb += __shfl_xor(eb, off, FOLX_WAVE);
+          eq += __shfl_xor(eq, off, FOLX_WAVE);
+        }
+        if (lane == 0) {
+          float* o = a.sc + ((int64_t)pg * R + r0 + wrow * TM + si) * 2;
+          o[0] = eb;
+          o[1] = eq;
+        }
+      }
+    }
+    __syncthreads();
   }
 
   // Register r of a block is Jacobian row p0 + 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32.
@@ -188,109 +285,332 @@ __global__ __launch_bounds__(NT, 4) void dense_act_wide_kernel(WideParams a) {
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int64_t pos = r0 + wrow * TM + i;
+    float rsv = 1.0f;
+    if constexpr (NORM) rsv = rsS[wrow * TM + i];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      float f, d1, d2;
-      act_eval_fused(a.act, zv[i][j], a.prm, f, d1, d2);
       const int gc = col0 + wc + j * 32 + l32;
+      float zv;
+      if constexpr (NORM) zv = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
+      else zv = zr[i][j];
+      float d1 = 1.0f;
+      if constexpr (ACT) {
+        float f, d2;
+        act_eval_fused(a.act, zv, a.prm, f, d1, d2);
+      }
+      float w1c = 0.0f, w2c = 0.0f;
+      if constexpr (NORM) {
+        const float2 t = wcS[wc + j * 32 + l32];
+        w1c = t.x;
+        w2c = zv - t.y;
+      }
       float* out = a.y_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc;
-      float ss = 0.0f;
-      if (full_tile) {
+      float ss = 0.0f, s1 = 0.0f;
+      auto rows = [&](auto full) __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float v = acc[i][j][r];
-          ss = fmaf(v, v, ss);
-          __builtin_nontemporal_store(d1 * v, out + (int64_t)(8 * (r / 4) + r % 4) * pstride);
-        }
-      } else {
+        for (int g = 0; g < 4; ++g) {
+          float ap[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+          if constexpr (NORM) {
+            const float4* sp = reinterpret_cast<const float4*>(st + i * 32 + 8 * g + 4 * lh);
+            const float4 u0 = sp[0], u1 = sp[1];
+            ap[0] = u0.x; bp[0] = u0.y; ap[1] = u0.z; bp[1] = u0.w;
+            ap[2] = u1.x; bp[2] = u1.y; ap[3] = u1.z; bp[3] = u1.w;
+          }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int pl = 8 * (r / 4) + r % 4;
-          if (p0 + 4 * lh + pl < P) {
-            const float v = acc[i][j][r];
-            ss = fmaf(v, v, ss);
-            if (gc < N) out[(int64_t)pl * pstride] = d1 * v;
+          for (int rr = 0; rr < 4; ++rr) {
+            const int pl = 8 * g + rr;
+            float v = acc[i][j][4 * g + rr];
+            if constexpr (NORM) {
+              v = fmaf(-ap[rr], w1c, v);
+              s1 = fmaf(bp[rr], v, s1);
+              v = fmaf(-bp[rr], w2c, v) * rsv;
+            }
+            if constexpr (decltype(full)::value) {
+              if constexpr (ACT) ss = fmaf(v, v, ss);
+              __builtin_nontemporal_store(d1 * v, out + (int64_t)pl * pstride);
+            } else if (p0 + 4 * lh + pl < P) {
+              if constexpr (ACT) ss = fmaf(v, v, ss);
+              if (gc < N) out[(int64_t)pl * pstride] = d1 * v;
+            }
           }
         }
+      };
+      if (full_tile) rows(std::true_type{});
+      else rows(std::false_type{});
+      const int64_t so = ((int64_t)pg * R + pos) * N + gc;
+      if constexpr (ACT) {
+        ss += __shfl_xor(ss, 32, FOLX_WAVE);
+        if (lh == 0 && gc < N) a.ss[so] = ss;
       }
-      ss += __shfl_xor(ss, 32, FOLX_WAVE);
-      if (lh == 0 && gc < N) a.part[((int64_t)pg * R + pos) * N + gc] = ss;
+      if constexpr (NORM) {
+        s1 += __shfl_xor(s1, 32, FOLX_WAVE);
+        if (lh == 0 && gc < N) a.s1[so] = s1;
+      }
     }
   }
 }
 
-// y <- f(z), y_lap <- f'(z) zl + f''(z) sum_g part[g]; z and zl are what the first launch left
-// in y and y_lap.  One float4 per thread.
-__global__ __launch_bounds__(256) void dense_act_wide_finish(float* __restrict__ y, float* __restrict__ y_lap,
-                                                             const float* __restrict__ part, int64_t S4,
-                                                             int32_t PG, int32_t act, float prm) {
+// Finishes the x and lap rows.  On entry y holds z and y_lap the part of zl that is linear in
+// the input's lap row (what launch 2 left there).  One float4 per thread.
+template <bool NORM, bool ACT>
+__global__ __launch_bounds__(256) void dense_wide_finish(float* __restrict__ y, float* __restrict__ y_lap,
+                                                         const float* __restrict__ ss, const float* __restrict__ s1,
+                                                         const float* __restrict__ sc, const float* __restrict__ rs,
+                                                         const float2* __restrict__ wc, int64_t S4, int64_t R,
+                                                         int32_t N, int32_t PG, int32_t act, float prm) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= S4) return;
   const float4 z = reinterpret_cast<const float4*>(y)[i];
-  const float4 zl = reinterpret_cast<const float4*>(y_lap)[i];
-  float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-  for (int g = 0; g < PG; ++g) {
-    const float4 t = reinterpret_cast<const float4*>(part)[(int64_t)g * S4 + i];
-    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+  float4 zl = reinterpret_cast<const float4*>(y_lap)[i];
+  if constexpr (NORM) {
+    const int64_t pos = i / (N / 4);
+    const int32_t n = (int32_t)(i % (N / 4)) * 4;
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float eb = 0.0f, eq = 0.0f;
+    for (int g = 0; g < PG; ++g) {
+      const float4 t = reinterpret_cast<const float4*>(s1)[(int64_t)g * S4 + i];
+      v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+      eb += sc[((int64_t)g * R + pos) * 2];
+      eq += sc[((int64_t)g * R + pos) * 2 + 1];
+    }
+    const float r = rs[pos];
+    const float r2 = r * r, e = 3.0f * eb - eq;
+    zl.x += r2 * fmaf(z.x - wc[n].y, e, -2.0f * v.x);
+    zl.y += r2 * fmaf(z.y - wc[n + 1].y, e, -2.0f * v.y);
+    zl.z += r2 * fmaf(z.z - wc[n + 2].y, e, -2.0f * v.z);
+    zl.w += r2 * fmaf(z.w - wc[n + 3].y, e, -2.0f * v.w);
   }
-  float4 f, l;
-  float d1, d2;
-  act_eval_fused(act, z.x, prm, f.x, d1, d2); l.x = fmaf(d1, zl.x, d2 * s.x);
-  act_eval_fused(act, z.y, prm, f.y, d1, d2); l.y = fmaf(d1, zl.y, d2 * s.y);
-  act_eval_fused(act, z.z, prm, f.z, d1, d2); l.z = fmaf(d1, zl.z, d2 * s.z);
-  act_eval_fused(act, z.w, prm, f.w, d1, d2); l.w = fmaf(d1, zl.w, d2 * s.w);
-  reinterpret_cast<float4*>(y)[i] = f;
-  reinterpret_cast<float4*>(y_lap)[i] = l;
+  if constexpr (ACT) {
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int g = 0; g < PG; ++g) {
+      const float4 t = reinterpret_cast<const float4*>(ss)[(int64_t)g * S4 + i];
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    float4 f;
+    float d1, d2;
+    act_eval_fused(act, z.x, prm, f.x, d1, d2); zl.x = fmaf(d1, zl.x, d2 * s.x);
+    act_eval_fused(act, z.y, prm, f.y, d1, d2); zl.y = fmaf(d1, zl.y, d2 * s.y);
+    act_eval_fused(act, z.z, prm, f.z, d1, d2); zl.z = fmaf(d1, zl.z, d2 * s.z);
+    act_eval_fused(act, z.w, prm, f.w, d1, d2); zl.w = fmaf(d1, zl.w, d2 * s.w);
+    reinterpret_cast<float4*>(y)[i] = f;
+  }
+  reinterpret_cast<float4*>(y_lap)[i] = zl;
 }
 
+// Wg = diag(gamma) W and per column the pair (w1, c0) = (1^T Wg, bias + beta @ W).  A block
+// takes 64 columns; its 16 wavefronts split the K rows.
+__global__ __launch_bounds__(1024) void norm_fold_kernel(const float* __restrict__ W, const float* __restrict__ bias,
+                                                         const float* __restrict__ gamma,
+                                                         const float* __restrict__ beta, float* __restrict__ Wg,
+                                                         float2* __restrict__ wc, int32_t K, int32_t N) {
+  __shared__ float ps[16][64], pc[16][64];
+  const int c = threadIdx.x % 64, sl = threadIdx.x / 64;
+  const int n = blockIdx.x * 64 + c;
+  float s = 0.0f, cc = 0.0f;
+  if (n < N) {
+    for (int k = sl; k < K; k += 16) {
+      const float w = W[(int64_t)k * N + n];
+      const float wg = gamma ? gamma[k] * w : w;
+      Wg[(int64_t)k * N + n] = wg;
+      s += wg;
+      if (beta) cc = fmaf(beta[k], w, cc);
+    }
+  }
+  ps[sl][c] = s;
+  pc[sl][c] = cc;
+  __syncthreads();
+  if (sl == 0 && n < N) {
+    float ts = 0.0f, tc = bias ? bias[n] : 0.0f;
+    for (int i = 0; i < 16; ++i) { ts += ps[i][c]; tc += pc[i][c]; }
+    wc[n] = make_float2(ts, tc);
+  }
+}
+
+// One wavefront per position: xh, rs, LN(x) and the part of LN's lap row that is linear in the
+// input's lap row, gamma rs (lap - mean(lap) - xh mean(xh lap)).  K <= 512: two float4 per lane.
+__global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict__ x, const float* __restrict__ lap,
+                                                        const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta, float* __restrict__ xhat,
+                                                        float* __restrict__ rs, float* __restrict__ nx,
+                                                        float* __restrict__ nlap, int64_t R, int32_t K, float eps) {
+  const int lane = threadIdx.x % 64;
+  const int64_t pos = (int64_t)blockIdx.x * 4 + threadIdx.x / 64;
+  if (pos >= R) return;
+  auto wsum = [](float v) __attribute__((always_inline)) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, FOLX_WAVE);
+    return v;
+  };
+  const int nv = K / 4;
+  const float invK = 1.0f / (float)K;
+  float4 xv[2], lv[2];
+  float s = 0.0f, sl = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int e = lane + 64 * c;
+    xv[c] = lv[c] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (e < nv) {
+      xv[c] = reinterpret_cast<const float4*>(x + pos * K)[e];
+      lv[c] = reinterpret_cast<const float4*>(lap + pos * K)[e];
+    }
+    s += (xv[c].x + xv[c].y) + (xv[c].z + xv[c].w);
+    sl += (lv[c].x + lv[c].y) + (lv[c].z + lv[c].w);
+  }
+  const float mean = wsum(s) * invK;
+  const float aL = wsum(sl) * invK;
+  float sv = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    if (lane + 64 * c < nv) {
+      xv[c].x -= mean; xv[c].y -= mean; xv[c].z -= mean; xv[c].w -= mean;
+      sv += xv[c].x * xv[c].x + xv[c].y * xv[c].y + xv[c].z * xv[c].z + xv[c].w * xv[c].w;
+    }
+  }
+  const float r = 1.0f / sqrtf(wsum(sv) * invK + eps);
+  float sbl = 0.0f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    xv[c].x *= r; xv[c].y *= r; xv[c].z *= r; xv[c].w *= r;
+    sbl += xv[c].x * lv[c].x + xv[c].y * lv[c].y + xv[c].z * lv[c].z + xv[c].w * lv[c].w;
+  }
+  const float bL = wsum(sbl) * invK;
+  if (lane == 0) rs[pos] = r;
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    const int e = lane + 64 * c;
+    if (e < nv) {
+      const float4 g = gamma ? reinterpret_cast<const float4*>(gamma)[e] : make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+      const float4 b = beta ? reinterpret_cast<const float4*>(beta)[e] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      reinterpret_cast<float4*>(xhat + pos * K)[e] = xv[c];
+      reinterpret_cast<float4*>(nx + pos * K)[e] =
+          make_float4(fmaf(g.x, xv[c].x, b.x), fmaf(g.y, xv[c].y, b.y), fmaf(g.z, xv[c].z, b.z), fmaf(g.w, xv[c].w, b.w));
+      reinterpret_cast<float4*>(nlap + pos * K)[e] =
+          make_float4(g.x * r * (lv[c].x - aL - bL * xv[c].x), g.y * r * (lv[c].y - aL - bL * xv[c].y),
+                      g.z * r * (lv[c].z - aL - bL * xv[c].z), g.w * r * (lv[c].w - aL - bL * xv[c].w));
+    }
+  }
+}
+
+// Shapes the path takes, launch sizes and the carve-up of the workspace (offsets in floats,
+// every part a multiple of 4 floats).
 struct WidePlan {
   int64_t row_tiles, pos_tiles, blocks, ws_bytes;
+  int64_t o_ss, o_s1, o_sc, o_xhat, o_rs, o_nx, o_nlap, o_wg, o_wc;
   int32_t PG, col_tiles;
 };
 
-bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, WidePlan& pl) {
+bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, WidePlan& pl) {
   if (R <= 0 || R % RT != 0 || P < 1 || K < BK || K % BK != 0 || N <= 128 || N % 4 != 0) return false;
+  if (norm && K > KMAX_NORM) return false;
   pl.PG = (P + PT - 1) / PT;
   pl.pos_tiles = R / RT;
   pl.row_tiles = pl.pos_tiles * pl.PG;
   pl.col_tiles = (N + BN - 1) / BN;
   pl.blocks = (pl.row_tiles + NXCD - 1) / NXCD * NXCD * pl.col_tiles;
   if (pl.blocks > 0x7fffffffLL) return false;
-  if (R * (int64_t)N / 4 + 255 > 0x7fffffffLL * 256) return false;
-  pl.ws_bytes = (int64_t)pl.PG * R * N * 4;
+  if (R * (int64_t)N / 4 / 256 + 1 > 0x7fffffffLL) return false;
+  const int64_t slab = (int64_t)pl.PG * R * N;
+  int64_t o = 0;
+  auto take = [&](int64_t n) { const int64_t at = o; o += (n + 3) / 4 * 4; return at; };
+  pl.o_ss = act ? take(slab) : 0;
+  if (norm) {
+    pl.o_s1 = take(slab);
+    pl.o_sc = take((int64_t)pl.PG * R * 2);
+    pl.o_xhat = take(R * (int64_t)K);
+    pl.o_rs = take(R);
+    pl.o_nx = take(R * (int64_t)K);
+    pl.o_nlap = take(R * (int64_t)K);
+    pl.o_wg = take((int64_t)K * N);
+    pl.o_wc = take(2 * (int64_t)N);
+  }
+  pl.ws_bytes = o * 4;
   return true;
+}
+
+template <bool NORM, bool ACT>
+int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap) {
+  dense_wide_kernel<NORM, ACT><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
+  int rc = folx_launch_status();
+  if (rc != FOLX_HIP_OK) return rc;
+  const int64_t S4 = a.R * (int64_t)a.N / 4;
+  dense_wide_finish<NORM, ACT><<<dim3((unsigned)((S4 + 255) / 256)), dim3(256), 0, st>>>(
+      y, y_lap, a.ss, a.s1, a.sc, a.rs, a.wc, S4, a.R, a.N, pl.PG, a.act, a.prm);
+  return folx_launch_status();
+}
+
+int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x, const float* jac, const float* lap,
+             const float* gamma, const float* beta, float eps, const float* W, const float* bias, float* y,
+             float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
+             int64_t workspace_bytes) {
+  const bool has_act = act >= 0;
+  WidePlan pl;
+  if ((has_act && !act_fused(act)) || !plan_wide(R, P, K, N, norm, has_act, pl)) return FOLX_HIP_ENOTSUP;
+  if (!norm && !has_act) return FOLX_HIP_ENOTSUP;  // that is the plain dense rule
+  if (!x || !jac || !lap || !W || !y || !y_jac || !y_lap) return FOLX_HIP_EINVAL;
+  if (!folx_aligned16(jac) || !folx_aligned16(W) || !folx_aligned16(y) || !folx_aligned16(y_lap))
+    return FOLX_HIP_ENOTSUP;
+  if (norm && (!folx_aligned16(x) || !folx_aligned16(lap) || !folx_aligned16(gamma) || !folx_aligned16(beta)))
+    return FOLX_HIP_ENOTSUP;
+  if (!workspace || workspace_bytes < pl.ws_bytes || !folx_aligned16(workspace)) return FOLX_HIP_EINVAL;
+  float* ws = (float*)workspace;
+  WideParams a;
+  a.jac = jac; a.W = W; a.z = y; a.y_jac = y_jac;
+  a.xhat = nullptr; a.rs = nullptr; a.wc = nullptr;
+  a.ss = ws + pl.o_ss; a.s1 = nullptr; a.sc = nullptr;
+  a.R = R; a.row_tiles = pl.row_tiles; a.pos_tiles = pl.pos_tiles;
+  a.P = P; a.K = K; a.N = N; a.col_tiles = pl.col_tiles; a.act = act; a.prm = param;
+  const float* in_x = x;
+  const float* in_lap = lap;
+  if (norm) {
+    norm_fold_kernel<<<dim3((unsigned)((N + 63) / 64)), dim3(1024), 0, st>>>(W, bias, gamma, beta, ws + pl.o_wg,
+                                                                          (float2*)(ws + pl.o_wc), K, N);
+    int rc = folx_launch_status();
+    if (rc != FOLX_HIP_OK) return rc;
+    norm_rows_kernel<<<dim3((unsigned)((R + 3) / 4)), dim3(256), 0, st>>>(
+        x, lap, gamma, beta, ws + pl.o_xhat, ws + pl.o_rs, ws + pl.o_nx, ws + pl.o_nlap, R, K, eps);
+    rc = folx_launch_status();
+    if (rc != FOLX_HIP_OK) return rc;
+    a.W = ws + pl.o_wg; a.xhat = ws + pl.o_xhat; a.rs = ws + pl.o_rs; a.wc = (const float2*)(ws + pl.o_wc);
+    a.s1 = ws + pl.o_s1; a.sc = ws + pl.o_sc;
+    in_x = ws + pl.o_nx; in_lap = ws + pl.o_nlap;
+  }
+  // z and the linear part of zl through the plain dense kernel: no Jacobian rows, no residual
+  int rc = folx_hip_dense_fwdlap(st, in_x, nullptr, in_lap, W, bias, nullptr, nullptr, nullptr, y, nullptr, y_lap, R,
+                                 0, K, N);
+  if (rc != FOLX_HIP_OK) return rc;
+  if (norm) return has_act ? launch_wide<true, true>(st, a, pl, y, y_lap) : launch_wide<true, false>(st, a, pl, y, y_lap);
+  return launch_wide<false, true>(st, a, pl, y, y_lap);
 }
 
 }  // namespace
 
 int64_t folx_dense_act_wide_ws_bytes(int64_t R, int32_t P, int32_t K, int32_t N) {
   WidePlan pl;
-  if (!plan_wide(R, P, K, N, pl)) return FOLX_HIP_ENOTSUP;
+  if (!plan_wide(R, P, K, N, false, true, pl)) return FOLX_HIP_ENOTSUP;
   return pl.ws_bytes;
 }
 
 int folx_dense_act_wide(hipStream_t st, int32_t act, float param, const float* x, const float* jac, const float* lap,
                         const float* W, const float* bias, float* y, float* y_jac, float* y_lap, int64_t R,
                         int32_t P, int32_t K, int32_t N, void* workspace, int64_t workspace_bytes) {
+  if (act < 0) return FOLX_HIP_ENOTSUP;
+  return run_wide(st, false, act, param, x, jac, lap, nullptr, nullptr, 0.0f, W, bias, y, y_jac, y_lap, R, P, K, N,
+                  workspace, workspace_bytes);
+}
+
+extern "C" int64_t folx_hip_norm_dense_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N, int32_t act) {
+  if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
   WidePlan pl;
-  if (!act_fused(act) || !plan_wide(R, P, K, N, pl)) return FOLX_HIP_ENOTSUP;
-  if (!x || !jac || !lap || !W || !y || !y_jac || !y_lap) return FOLX_HIP_EINVAL;
-  if (!folx_aligned16(jac) || !folx_aligned16(W) || !folx_aligned16(y) || !folx_aligned16(y_lap))
-    return FOLX_HIP_ENOTSUP;
-  if (!workspace || workspace_bytes < pl.ws_bytes || !folx_aligned16(workspace)) return FOLX_HIP_EINVAL;
-  // z and zl through the plain dense kernel: no Jacobian rows, no residual
-  int rc = folx_hip_dense_fwdlap(st, x, nullptr, lap, W, bias, nullptr, nullptr, nullptr, y, nullptr, y_lap, R, 0, K,
-                                 N);
-  if (rc != FOLX_HIP_OK) return rc;
-  WideParams a;
-  a.jac = jac; a.W = W; a.z = y; a.y_jac = y_jac; a.part = (float*)workspace;
-  a.R = R; a.row_tiles = pl.row_tiles; a.pos_tiles = pl.pos_tiles;
-  a.P = P; a.K = K; a.N = N; a.col_tiles = pl.col_tiles; a.act = act; a.prm = param;
-  dense_act_wide_kernel<<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
-  rc = folx_launch_status();
-  if (rc != FOLX_HIP_OK) return rc;
-  const int64_t S4 = R * (int64_t)N / 4;
-  dense_act_wide_finish<<<dim3((unsigned)((S4 + 255) / 256)), dim3(256), 0, st>>>(y, y_lap, (const float*)workspace,
-                                                                                  S4, pl.PG, act, param);
-  return folx_launch_status();
+  if ((act >= 0 && !act_fused(act)) || !plan_wide(R, P, K, N, true, act >= 0, pl)) return FOLX_HIP_ENOTSUP;
+  return pl.ws_bytes;
+}
+
+extern "C" int folx_hip_norm_dense_fwdlap(void* stream, int32_t act, float param, const float* x, const float* jac,
+                                          const float* lap, const float* gamma, const float* beta, float eps,
+                                          const float* W, const float* bias, float* y, float* y_jac, float* y_lap,
+                                          int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
+                                          int64_t workspace_bytes) {
+  if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
+  return run_wide((hipStream_t)stream, true, act, param, x, jac, lap, gamma, beta, eps, W, bias, y, y_jac, y_lap, R, P,
+                  K, N, workspace, workspace_bytes);
 }

@@ -134,14 +134,22 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
 FUSED_ACTS = ('tanh', 'silu', 'logistic', 'sigmoid', 'softplus', 'exp', 'sin', 'cos', 'square')
 
 
-def dense_act_supported(name, K, N, rows=None):
+def _wide_tiles_filled(P):
+    """The wide fused kernels cut their tiles into groups of 32 Jacobian rows; a last group
+    that is mostly empty costs more MFMA work than the fusion saves."""
+    return P is None or 32 * ((P + 31) // 32) <= 1.125 * P
+
+
+def dense_act_supported(name, K, N, rows=None, P=None):
     """Shapes and functions the fused dense + activation kernels are built for: narrow layers
-    (K, N <= 128), and wide ones (N > 128, K a multiple of 16) over a multiple of 4 rows."""
+    (K, N <= 128), and wide ones (N > 128, K a multiple of 16) over a multiple of 4 rows.
+    With ``P`` (Jacobian rows) given, also whether the wide kernel is the faster choice."""
     if name not in FUSED_ACTS:
         return False
     if 4 <= K <= 128 and K % 4 == 0 and 1 <= N <= 128:
         return True
-    return rows is not None and rows > 0 and rows % 4 == 0 and K % 16 == 0 and N > 128 and N % 4 == 0
+    return (rows is not None and rows > 0 and rows % 4 == 0 and K % 16 == 0 and N > 128 and N % 4 == 0
+            and _wide_tiles_filled(P))
 
 
 def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
@@ -167,6 +175,41 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
                 _p(y), _p(yj), _p(yl), R, P, K, N, _p(ws), nbytes
             ),
             f'dense_act_fwdlap[{name}]',
+        )
+    return y, yj, yl
+
+
+def norm_dense_supported(name, K, N, rows, P=None):
+    """Shapes and functions ``norm_dense`` is built for (``name`` None: no activation); with
+    ``P`` (Jacobian rows) given, also whether it is the faster choice."""
+    return ((name is None or name in FUSED_ACTS) and rows > 0 and rows % 4 == 0 and K % 16 == 0 and K <= 512
+            and N > 128 and N % 4 == 0 and _wide_tiles_filled(P))
+
+
+def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):
+    """``f(layer_norm(x) @ W + bias)`` as one rule (``name`` None: no ``f``): x (.., K), jac
+    (P, .., K), lap (.., K), gamma / beta (K) or None, W (K, N) -> triplet with last dim N."""
+    _chk(x, jac, lap, gamma, beta, W, bias)
+    K, N = W.shape
+    P = jac.shape[0]
+    lead = tuple(x.shape[:-1])
+    R = int(np.prod(lead, dtype=np.int64))
+    act = -1 if name is None else ACT[name]
+    lib = _lib.load()
+    nbytes = int(lib.folx_hip_norm_dense_workspace_bytes(R, P, K, N, act))
+    if nbytes < 0:
+        check(nbytes, 'norm_dense_workspace_bytes')
+    ws = torch.empty(nbytes // 4, device=x.device, dtype=torch.float32)
+    y = torch.empty((*lead, N), device=x.device, dtype=torch.float32)
+    yj = torch.empty((P, *lead, N), device=x.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    with _timed('norm_dense_fwdlap', (name, R, P, K, N)):
+        check(
+            lib.folx_hip_norm_dense_fwdlap(
+                _stream(), act, float(param), _p(x), _p(jac), _p(lap), _p(gamma), _p(beta), float(eps), _p(W),
+                _p(bias), _p(y), _p(yj), _p(yl), R, P, K, N, _p(ws), nbytes
+            ),
+            f'norm_dense_fwdlap[{name}]',
         )
     return y, yj, yl
 

@@ -97,13 +97,16 @@ def divide(a, b):
 
 
 # linear algebra ----------------------------------------------------------------------------
-def dot(h, W, b=None, residual=None, row_slice=None, act=None):
+def dot(h, W, b=None, residual=None, row_slice=None, act=None, norm=None):
     """``h @ W (+ b) (+ residual)``: last axis of ``h`` against the first axis of the
     constant ``W``; ``residual`` is a triplet of the output shape (skip connection).
     ``row_slice = (lo, hi)`` computes ``h[..., lo:hi, :] @ W`` without copying the slice.
     ``act`` names a scalar function applied to ``h @ W + b`` (the residual is then added to
-    the activated result): a narrow Dense + activation layer runs as one kernel."""
-    return _call('dot_general', (h, W), {'bias': b, 'residual': residual, 'row_slice': row_slice, 'act': act})
+    the activated result): a Dense + activation layer runs as one rule.
+    ``norm = (gamma, beta, eps)`` applies ``layer_norm`` to ``h`` first, inside the same rule
+    where the kernels allow it."""
+    return _call('dot_general', (h, W),
+                 {'bias': b, 'residual': residual, 'row_slice': row_slice, 'act': act, 'norm': norm})
 
 
 def layer_norm(h, gamma=None, beta=None, eps=1e-5):

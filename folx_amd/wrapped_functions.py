@@ -459,8 +459,7 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     bias = kwargs.get('bias')
     residual = kwargs.get('residual')
     row_slice = kwargs.get('row_slice')
-    act = kwargs.get('act')
-    if act is not None:
+    if kwargs.get('act') is not None or kwargs.get('norm') is not None:
         return _dot_then_act(h, W, dict(kwargs), sparsity_threshold)
     if row_slice is not None:
         # the slice is consumed in place by the kernel when the Jacobian needs no re-indexing;
@@ -533,16 +532,40 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
 
 
 def _dot_then_act(h, W, kwargs, thr: int):
-    """``residual + act(h @ W + bias)``: a Dense + activation layer as ONE rule when the layer
-    is narrow enough for the fused kernel (``kernels.dense_act_supported``) and the result's
-    Jacobian rows are plain (dense, or sparse without an index listed twice at a position,
-    where sum_k J_k^2 is the Hessian term, folx/hessian.py:460-470); otherwise the
-    ``dot_general`` rule followed by the elementwise rule, which is also what defines the
-    result."""
-    act = kwargs.pop('act')
+    """``residual + act(layer_norm(h) @ W + bias)`` with ``act`` and ``layer_norm`` optional.
+    A Dense + activation layer is ONE rule when the fused kernels take its shape
+    (``kernels.dense_act_supported``) and the result's Jacobian rows are plain (dense, or
+    sparse without an index listed twice at a position, where sum_k J_k^2 is the Hessian
+    term, folx/hessian.py:460-470); LayerNorm joins the same rule for dense Jacobians and
+    wide layers (``kernels.norm_dense_supported``).  Otherwise the ``layer_norm`` rule, the
+    ``dot_general`` rule and the elementwise rule one after the other, which is also what
+    defines the result."""
+    act = kwargs.pop('act', None)
     param = kwargs.pop('act_param', 0.0)
     residual = kwargs.pop('residual', None)
+    norm = kwargs.pop('norm', None)
     bias = kwargs.get('bias')
+    if norm is not None:
+        gamma, beta, eps = norm
+        if (
+            _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
+            and h.jacobian.x0_idx is None
+            and K.norm_dense_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1),
+                                       P=h.jacobian.data.shape[0])
+        ):
+            dev = h.x.device
+            g = None if gamma is None else so.device_const(gamma, dev)
+            b = None if beta is None else so.device_const(beta, dev)
+            bt = None if bias is None else so.device_const(bias, dev)
+            y, Jy, lapy = K.norm_dense(act, h.x, h.jacobian.data, h.laplacian, g, b, float(eps),
+                                       so.device_const(W, dev), bt, param)
+            out = FwdLaplArray(y, FwdJacobian(Jy, None), lapy)
+            if residual is not None:
+                out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)
+            return out
+        h = layer_norm_rule((h, gamma, beta), {'eps': eps}, thr)
+    if act is None:
+        return dot_general((h, W), {**kwargs, 'residual': residual}, thr)
     fused = (
         _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
         and K.dense_act_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1))
@@ -561,6 +584,8 @@ def _dot_then_act(h, W, kwargs, thr: int):
                 if aligned:
                     J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
                 new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
+    if fused:  # the number of Jacobian rows decides whether the wide kernel's tiles are well filled
+        fused = K.dense_act_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1), P=J.shape[0])
     if fused:
         dev = h.x.device
         Wt = so.device_const(W, dev)

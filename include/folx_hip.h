@@ -145,19 +145,20 @@ int folx_hip_exp_envelope_fwdlap(void* stream, const float* d, const float* d_ja
                                  int32_t P);
 
 /*
- * Narrow dense layer followed by its activation, in one pass:
+ * Dense layer followed by its activation as one rule:
  *   y = f(x @ W + bias),  y_jac[p] = f'(z) * (jac[p] @ W),
  *   y_lap = f'(z) * (lap @ W) + f''(z) * sum_p (jac[p] @ W)^2,      z = x @ W + bias.
  * The composition of _dot_general_one_constant (folx/wrapped_functions.py:71-171) with the
  * elementwise rule (folx/jvp.py:687-697, folx/hessian.py:87-112, folx/wrapper.py:120-125)
- * that follows it in every Dense + activation layer; the pre-activation triplet is never
- * written.  Layouts as in folx_hip_dense_fwdlap.  Built for 4 <= K <= 128 with K % 4 == 0,
- * N <= 128, 16-byte aligned inputs and act in {TANH, SILU, LOGISTIC, SOFTPLUS, EXP, SIN, COS,
- * SQUARE}; anything else returns FOLX_HIP_ENOTSUP and the caller uses the two separate rules.
- * Outputs must not overlap inputs.
- * workspace: folx_hip_dense_act_workspace_bytes(R, P, K, N) bytes of device memory (0 for
- * large R: then it may be NULL), contents irrelevant; it holds partial sums between the two
- * launches a small batch is split into.  The query returns a negative code for unsupported
+ * that follows it in every Dense + activation layer; the pre-activation Jacobian is never
+ * written.  Layouts as in folx_hip_dense_fwdlap.  Built for narrow layers (4 <= K <= 128 with
+ * K % 4 == 0, N <= 128) and for wide ones (N > 128 with N % 4 == 0, K % 16 == 0, R % 4 == 0,
+ * P >= 1), 16-byte aligned operands and act in {TANH, SILU, LOGISTIC, SOFTPLUS, EXP, SIN,
+ * COS, SQUARE}; anything else returns FOLX_HIP_ENOTSUP and the caller uses the two separate
+ * rules.  Outputs must not overlap inputs.
+ * workspace: folx_hip_dense_act_workspace_bytes(R, P, K, N) bytes of device memory (0 for a
+ * narrow layer with large R: then it may be NULL), contents irrelevant; it holds partial sums
+ * over Jacobian rows between launches.  The query returns a negative code for unsupported
  * shapes.
  */
 int64_t folx_hip_dense_act_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N);
@@ -166,6 +167,30 @@ int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const floa
                               const float* bias, float* y, float* y_jac, float* y_lap,
                               int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
                               int64_t workspace_bytes);
+
+/*
+ * LayerNorm over the K features, then a dense layer, then (act >= 0) an activation, as one
+ * rule:  y = f(LN(x) @ W + bias),  LN(x) = gamma * (x - mean) * rsqrt(var + eps) + beta.
+ * The triplet that results is the one of folx_hip_layernorm_fwdlap followed by
+ * folx_hip_dense_fwdlap and folx_hip_elementwise_fwdlap (the reference interprets the same
+ * chain of primitives, folx/wrapped_functions.py:71-171, :361-415); neither LN's Jacobian
+ * nor the pre-activation Jacobian is written.  The Jacobian rows are multiplied RAW with
+ * diag(gamma) W and LayerNorm's projection is applied to the product as a rank-2 correction
+ * per row, so rows whose mean dwarfs their variation lose digits they would keep in the
+ * three-step form.
+ *   x [R][K]  jac [P][R][K]  lap [R][K]  gamma, beta [K] or NULL  W [K][N]  bias [N] or NULL
+ *   ->  y [R][N]  y_jac [P][R][N]  y_lap [R][N];  act = -1: no activation.
+ * Built for N > 128 with N % 4 == 0, K % 16 == 0, K <= 512, R % 4 == 0, P >= 1, 16-byte aligned
+ * operands and the activations of folx_hip_dense_act_fwdlap; anything else returns
+ * FOLX_HIP_ENOTSUP.  workspace: folx_hip_norm_dense_workspace_bytes(R, P, K, N, act) bytes,
+ * contents irrelevant.  Outputs must not overlap inputs.
+ */
+int64_t folx_hip_norm_dense_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N, int32_t act);
+int folx_hip_norm_dense_fwdlap(void* stream, int32_t act, float param, const float* x,
+                               const float* jac, const float* lap, const float* gamma,
+                               const float* beta, float eps, const float* W, const float* bias,
+                               float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
+                               int32_t K, int32_t N, void* workspace, int64_t workspace_bytes);
 
 /*
  * Binary elementwise rule for two operands whose Jacobians live on the same row frame

@@ -365,9 +365,12 @@ def integer_pow(a, n):
     return OArr(*rules.elementwise_rule('integer_pow', a.x, a.J, a.lap, n))
 
 
-def dot(h: OArr, W, b=None, residual=None, row_slice=None, act=None):
+def dot(h: OArr, W, b=None, residual=None, row_slice=None, act=None, norm=None):
     """``row_slice = (lo, hi)``: the product of ``h[..., lo:hi, :]``; ``act``: a scalar function
-    applied to ``h @ W + b`` before the residual is added."""
+    applied to ``h @ W + b`` before the residual is added; ``norm = (gamma, beta, eps)``:
+    ``layer_norm`` of ``h`` first."""
+    if norm is not None:
+        h = layer_norm(h, *norm)
     if act is not None:
         out = _unary({'sigmoid': 'logistic'}.get(act, act))(dot(h, W, b, None, row_slice))
         return out if residual is None else add(residual, out)

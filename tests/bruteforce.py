@@ -24,7 +24,9 @@ class plain:
         return torch.as_tensor(np.asarray(c), dtype=like.dtype)
 
     @staticmethod
-    def dot(h, W, b=None, residual=None, row_slice=None, act=None):
+    def dot(h, W, b=None, residual=None, row_slice=None, act=None, norm=None):
+        if norm is not None:
+            h = plain.layer_norm(h, *norm)
         if row_slice is not None:
             h = h[..., row_slice[0]:row_slice[1], :]
         y = h @ plain._c(W, h)

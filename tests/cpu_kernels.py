@@ -37,6 +37,13 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
 
 
+def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):
+    n = layernorm(x, jac, lap, gamma, beta, eps)
+    if name is None:
+        return dense(*n, W, bias)
+    return dense_act(name, *n, W, bias, param)
+
+
 def exp_envelope(d, dj, dl, sigma, pi):
     from oracle import backend as ob
 
@@ -217,7 +224,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'dense_act', 'exp_envelope', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'dense_act', 'norm_dense', 'exp_envelope', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

@@ -387,6 +387,40 @@ def test_dot_act(thr):
     check_against_oracle(fn, x, thr)
 
 
+@pytest.mark.parametrize('thr', [0, 6])
+def test_dot_norm(thr, monkeypatch):
+    """``dot(h, W, b, norm=..., act=...)`` equals layer_norm, dense and elementwise rules one
+    after the other: through the fused rule on wide layers over dense Jacobians (with and
+    without an activation, with a residual), and through the three rules on sparse Jacobians
+    and on narrow layers."""
+    from folx_amd import kernels as K
+
+    calls = []
+    orig = K.norm_dense
+    monkeypatch.setattr(K, 'norm_dense', lambda *a: (calls.append(a[0]), orig(*a))[1])
+    rng = np.random.default_rng(12)
+    W0 = rng.normal(size=(3, 16)).astype(np.float32)
+    g0, b0 = (1 + 0.2 * rng.normal(size=16)).astype(np.float32), (0.2 * rng.normal(size=16)).astype(np.float32)
+    W1 = rng.normal(size=(16, 132)).astype(np.float32) / 4
+    c1 = rng.normal(size=(132,)).astype(np.float32)
+    W2 = rng.normal(size=(132, 16)).astype(np.float32) / 11
+    W3 = rng.normal(size=(16, 136)).astype(np.float32) / 4
+    W4 = rng.normal(size=(16, 8)).astype(np.float32) / 4
+    x = rng.normal(size=(2, 10, 3)).astype(np.float32)  # 30 Jacobian rows: one well-filled group of 32
+
+    def fn(xp, t):
+        h = xp.dot(t, W0)                                                    # sparse rows at thr 6
+        a = xp.dot(h, W1, c1, norm=(g0, b0, 1e-5), act='tanh')               # sparse: three rules; dense: fused
+        h = xp.add(xp.dot(a, W2), xp.mean(h, axis=0, keepdims=True))         # mixes electrons: dense from here on
+        u = xp.dot(h, W3, norm=(g0, None, 1e-5))                             # fused, no activation
+        v = xp.dot(h, W3, norm=(None, None, 1e-3), act='silu', residual=u)   # fused, residual added afterwards
+        w = xp.dot(h, W4, norm=(g0, b0, 1e-5), act='sin')                    # narrow: layer_norm, then dense + act
+        return xp.add(xp.sum(v), xp.sum(w))
+
+    check_against_oracle(fn, x, thr)
+    assert calls == (['tanh', None, 'silu'] if thr == 0 else [None, 'silu'])
+
+
 def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
     """q, k, v of the first PsiFormer layer still carry per-electron sparse Jacobians: the rule
     hands them to the position-sparse kernel and the result equals the densified rule."""

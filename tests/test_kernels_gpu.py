@@ -179,6 +179,68 @@ def test_dense_act_matches_two_kernels_large():
         torch.testing.assert_close(a, r, rtol=2e-5, atol=2e-5, msg=lambda m: f'{nm}: {m}')
 
 
+NORM_DENSE_CASES = [
+    # (rows shape, P, K, N, gamma/beta, bias, act)
+    ((2, 32), 96, 256, 256, True, False, None),      # transformer q / k / v projection behind LayerNorm
+    ((2, 32), 96, 256, 256, True, True, 'tanh'),     # transformer MLP behind LayerNorm
+    ((1, 8), 40, 64, 132, False, True, None),        # no gamma / beta, partial group of Jacobian rows, cut column tile
+    ((1, 12), 33, 512, 512, True, True, 'silu'),     # widest K, two column tiles, 1 row in the second group
+    ((3, 4), 1, 16, 300, True, False, 'softplus'),   # one chunk of K, one Jacobian row
+    ((1, 4), 64, 48, 256, True, True, 'sin'),
+]
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,affine,bias,act', NORM_DENSE_CASES)
+def test_norm_dense(rows, P, Kd, N, affine, bias, act):
+    """LayerNorm + dense (+ activation) as one rule against the chain of oracle rules."""
+    from oracle import backend as ob
+
+    from folx_amd import kernels as K
+
+    print(f'case norm_dense rows={rows} P={P} K={Kd} N={N} act={act}', flush=True)
+    rng = np.random.default_rng(23)
+    x, J, L = rand(rng, *rows, Kd) + 0.5, rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    J = J + 0.3 * rand(rng, P, *rows, 1)  # rows with a mean of their own
+    g = (1.0 + 0.3 * rand(rng, Kd)) if affine else None
+    be = 0.2 * rand(rng, Kd) if affine else None
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    h = ob.layer_norm(ob.OArr(*f64(x, J, L)), None if g is None else g.astype(np.float64),
+                      None if be is None else be.astype(np.float64), 1e-5)
+    ref = rules.dense_rule(h.x, h.J, h.lap, W.astype(np.float64), None if b is None else b.astype(np.float64))
+    if act is not None:
+        ref = rules.elementwise_rule(act, *ref)
+    assert K.norm_dense_supported(act, Kd, N, int(np.prod(rows)))
+    opt = lambda t: None if t is None else dev(t)
+    for rep in range(2):  # the workspace of the second call holds what the first one left
+        got = K.norm_dense(act, dev(x), dev(J), dev(L), opt(g), opt(be), 1e-5, dev(W), opt(b))
+        assert_triplet(got, ref, f'norm_dense call {rep}')
+
+
+def test_norm_dense_matches_three_kernels_large():
+    """A transformer layer's LayerNorm + MLP product at a full chunk: the fused rule and
+    layernorm + dense + elementwise agree to rounding."""
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(7)
+    R, P, Kd, N = 256 * 32, 96, 256, 256
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.randn(R, Kd, device='cuda', generator=g)
+    gam = 1 + 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    bet = 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    W = torch.randn(Kd, N, device='cuda', generator=g) / 16
+    b = torch.randn(N, device='cuda', generator=g)
+    for act in (None, 'tanh'):
+        got = K.norm_dense(act, x, J, L, gam, bet, 1e-5, W, b)
+        ref = K.dense(*K.layernorm(x, J, L, gam, bet, 1e-5), W, b)
+        if act is not None:
+            ref = K.elementwise(act, *ref)
+        for a, r, nm in zip(got, ref, ('x', 'jac', 'lap')):
+            torch.testing.assert_close(a, r, rtol=1e-4 if nm == 'lap' else 2e-5, atol=2e-3 if nm == 'lap' else 2e-5,
+                                       msg=lambda m: f'{act} {nm}: {m}')
+
+
 def test_dense_act_wide_matches_two_kernels_large():
     """A transformer MLP layer at a full chunk: the fused wide path and dense + elementwise
     agree to rounding (the sums over Jacobian rows are taken in a different order)."""
