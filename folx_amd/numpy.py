@@ -105,12 +105,25 @@ def dot(h, W, b=None, residual=None, row_slice=None, act=None, norm=None):
     the activated result): a Dense + activation layer runs as one rule.
     ``norm = (gamma, beta, eps)`` applies ``layer_norm`` to ``h`` first, inside the same rule
     where the kernels allow it."""
+    from .wrapped_functions import LazyLayerNorm
+
+    if isinstance(h, LazyLayerNorm):
+        assert norm is None, 'dot: the operand already is a layer_norm'
+        h, norm = h.h, h
     return _call('dot_general', (h, W),
                  {'bias': b, 'residual': residual, 'row_slice': row_slice, 'act': act, 'norm': norm})
 
 
-def layer_norm(h, gamma=None, beta=None, eps=1e-5):
-    """LayerNorm over the last axis (one fused rule; same result as the primitive chain)."""
+def layer_norm(h, gamma=None, beta=None, eps=1e-5, lazy=False):
+    """LayerNorm over the last axis (one fused rule; same result as the primitive chain).
+    ``lazy=True`` returns a handle that only ``dot`` accepts as its first operand: products
+    that can take LayerNorm into their own rule never evaluate it, the others share one
+    evaluation."""
+    from .api import FwdLaplArray as _F
+    from .wrapped_functions import LazyLayerNorm
+
+    if lazy and isinstance(h, _F):
+        return LazyLayerNorm(h, gamma, beta, eps)
     return _call('layer_norm', (h, gamma, beta), {'eps': eps})
 
 

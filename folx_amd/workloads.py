@@ -171,16 +171,16 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
     feats = xp.concatenate([xp.reshape(d, (n, 3 * cfg.n_nuc)), dist, p.spin], axis=-1)
     h = xp.dot(feats, p.w_in)
     for L in p.layers:
-        # LayerNorm is part of the products that consume it: the normalised Jacobian is never
-        # written where the fused rule applies (dense Jacobians)
-        ln1 = (L['ln1_g'], L['ln1_b'], cfg.ln_eps)
-        q = xp.reshape(xp.dot(h, L['w_q'], norm=ln1), (n, H, dh))
-        k = xp.reshape(xp.dot(h, L['w_k'], norm=ln1), (n, H, dh))
-        v = xp.reshape(xp.dot(h, L['w_v'], norm=ln1), (n, H, dh))
+        # the LayerNorms are only consumed by matrix products, which take them into their own
+        # rule where they can (dense Jacobians): the normalised Jacobian is then never written
+        hn = xp.layer_norm(h, L['ln1_g'], L['ln1_b'], cfg.ln_eps, lazy=True)
+        q = xp.reshape(xp.dot(hn, L['w_q']), (n, H, dh))
+        k = xp.reshape(xp.dot(hn, L['w_k']), (n, H, dh))
+        v = xp.reshape(xp.dot(hn, L['w_v']), (n, H, dh))
         att = xp.multi_head_self_attention(q, k, v)
         h = xp.dot(xp.reshape(att, (n, H * dh)), L['w_o'], None, residual=h)
-        ln2 = (L['ln2_g'], L['ln2_b'], cfg.ln_eps)
-        h = xp.dot(xp.dot(h, L['w_1'], L['b_1'], act='tanh', norm=ln2), L['w_2'], L['b_2'], residual=h)
+        hn = xp.layer_norm(h, L['ln2_g'], L['ln2_b'], cfg.ln_eps, lazy=True)
+        h = xp.dot(xp.dot(hn, L['w_1'], L['b_1'], act='tanh'), L['w_2'], L['b_2'], residual=h)
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, cfg.n_up), (cfg.n_up, n)]):
         m = hi - lo

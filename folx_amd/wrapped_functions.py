@@ -546,7 +546,7 @@ def _dot_then_act(h, W, kwargs, thr: int):
     norm = kwargs.pop('norm', None)
     bias = kwargs.get('bias')
     if norm is not None:
-        gamma, beta, eps = norm
+        gamma, beta, eps = (norm.gamma, norm.beta, norm.eps) if isinstance(norm, LazyLayerNorm) else norm
         if (
             _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
             and h.jacobian.x0_idx is None
@@ -563,7 +563,10 @@ def _dot_then_act(h, W, kwargs, thr: int):
             if residual is not None:
                 out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)
             return out
-        h = layer_norm_rule((h, gamma, beta), {'eps': eps}, thr)
+        if isinstance(norm, LazyLayerNorm):
+            h = norm.value(thr)
+        else:
+            h = layer_norm_rule((h, gamma, beta), {'eps': eps}, thr)
     if act is None:
         return dot_general((h, W), {**kwargs, 'residual': residual}, thr)
     fused = (
@@ -624,6 +627,24 @@ def _dot_two_operands(lhs: FwdLaplArray, rhs: FwdLaplArray, thr: int) -> FwdLapl
     if a_vec:
         out = fnp.squeeze(out, -1 if b_vec else -2)
     return out
+
+
+class LazyLayerNorm:
+    """``layer_norm(h, gamma, beta, eps)`` that has not been evaluated yet, for layers whose
+    only consumers are matrix products (``numpy.dot``): a product that can take LayerNorm
+    into its own rule reads ``h`` directly, any other evaluates the ``layer_norm`` rule --
+    once, however many products ask."""
+
+    __slots__ = ('h', 'gamma', 'beta', 'eps', '_value')
+
+    def __init__(self, h, gamma, beta, eps):
+        self.h, self.gamma, self.beta, self.eps = h, gamma, beta, float(eps)
+        self._value = None
+
+    def value(self, sparsity_threshold):
+        if self._value is None:
+            self._value = layer_norm_rule((self.h, self.gamma, self.beta), {'eps': self.eps}, sparsity_threshold)
+        return self._value
 
 
 def layer_norm_rule(args, kwargs, sparsity_threshold):

@@ -388,8 +388,9 @@ def exp_envelope(d, sigma, pi):
     return sum(multiply(e, np.asarray(pi)), axis=-2)
 
 
-def layer_norm(h: OArr, gamma=None, beta=None, eps=1e-5):
-    """LayerNorm as the chain of primitive rules the reference interprets it with."""
+def layer_norm(h: OArr, gamma=None, beta=None, eps=1e-5, lazy=False):
+    """LayerNorm as the chain of primitive rules the reference interprets it with (``lazy`` is
+    a scheduling hint of the device front end; the value is the same)."""
     mu = mean(h, axis=-1, keepdims=True)
     c = subtract(h, mu)
     var = mean(square(c), axis=-1, keepdims=True)

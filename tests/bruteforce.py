@@ -40,7 +40,7 @@ class plain:
         return (torch.exp(-d[..., None] * plain._c(sigma, d)) * plain._c(pi, d)).sum(-2)
 
     @staticmethod
-    def layer_norm(h, gamma=None, beta=None, eps=1e-5):
+    def layer_norm(h, gamma=None, beta=None, eps=1e-5, lazy=False):
         mu = h.mean(-1, keepdim=True)
         c = h - mu
         y = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps)

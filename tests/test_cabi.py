@@ -79,6 +79,18 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_dense_act_workspace_bytes(63, 33, 256, 256) == _lib.ENOTSUP         # wide: rows % 4
     assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 200, 256) == _lib.ENOTSUP         # wide: K % 16
     assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 64, 33, 256, 256, None, 0) == _lib.EINVAL  # no workspace
+    # LayerNorm + dense (+ activation): act = -1 means none
+    assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, -1) > 2 * 64 * 256 * 4
+    assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, 0) > lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, -1)
+    assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 1024, 256, -1) == _lib.ENOTSUP    # K > 512
+    assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 128, -1) == _lib.ENOTSUP     # narrow layer
+    assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, 3) == _lib.ENOTSUP      # log: not fused
+    assert lib.folx_hip_norm_dense_workspace_bytes(-1, 33, 256, 256, -1) == _lib.EINVAL
+    nd = lambda act, R, K, N, ws, nb: lib.folx_hip_norm_dense_fwdlap(None, act, 0.0, one, one, one, one, one, 1e-5, one,
+                                                                    one, one, one, one, R, 33, K, N, ws, nb)
+    assert nd(-1, 64, 256, 256, None, 0) == _lib.EINVAL        # no workspace
+    assert nd(-1, 62, 256, 256, one, 1 << 30) == _lib.ENOTSUP  # rows % 4
+    assert nd(3, 64, 256, 256, one, 1 << 30) == _lib.ENOTSUP   # log: not fused
     assert lib.folx_hip_dense_act_workspace_bytes(2000, 400, 100, 100) > 0                                    # rows split
     assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 65, 1, 8, 3) == _lib.ENOTSUP
     assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 8, 1, 6, 3) == _lib.ENOTSUP

@@ -415,10 +415,21 @@ def test_dot_norm(thr, monkeypatch):
         u = xp.dot(h, W3, norm=(g0, None, 1e-5))                             # fused, no activation
         v = xp.dot(h, W3, norm=(None, None, 1e-3), act='silu', residual=u)   # fused, residual added afterwards
         w = xp.dot(h, W4, norm=(g0, b0, 1e-5), act='sin')                    # narrow: layer_norm, then dense + act
-        return xp.add(xp.sum(v), xp.sum(w))
+        hn = xp.layer_norm(h, g0, b0, 1e-5, lazy=True)                       # a handle that only dot consumes
+        s = xp.add(xp.dot(hn, W3, act='tanh'), xp.dot(hn, W3))               # fused twice, never evaluated
+        t = xp.add(xp.dot(hn, W4), xp.dot(hn, W4, act='cos'))                # narrow: evaluated once for both
+        return xp.add(xp.add(xp.sum(v), xp.sum(w)), xp.add(xp.sum(s), xp.sum(t)))
 
+    from folx_amd import wrapped_functions as wf
+
+    lns = []
+    orig_ln = wf.layer_norm_rule
+    monkeypatch.setattr(wf, 'layer_norm_rule', lambda *a: (lns.append(1), orig_ln(*a))[1])
     check_against_oracle(fn, x, thr)
-    assert calls == (['tanh', None, 'silu'] if thr == 0 else [None, 'silu'])
+    assert calls == (['tanh', None, 'silu', 'tanh', None] if thr == 0 else [None, 'silu', 'tanh', None])
+    # unfused evaluations of layer_norm: the narrow product, the handle's two narrow products
+    # together, and at threshold 6 the product on sparse rows
+    assert len(lns) == (2 if thr == 0 else 3)
 
 
 def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
