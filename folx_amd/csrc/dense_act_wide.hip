@@ -60,13 +60,10 @@ constexpr int WROWS = BM / WM, WCOLS = BN / WN;
 constexpr int TM = WROWS / 32, TN = WCOLS / 32;
 constexpr int TG = BK / 8;
 constexpr int NXCD = 8;
-constexpr int PT = 32;         // Jacobian rows of a tile
-constexpr int RT = BM / PT;    // positions of a tile
 constexpr int KMAX_NORM = 512; // xh of a tile's positions sits in LDS
 constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
 constexpr int A_LD = A_V4 / NT, W_LD = W_V4 / NT;
 static_assert(A_V4 % NT == 0 && W_V4 % NT == 0, "every thread loads the same number of pieces");
-static_assert(TM * WM == RT, "one accumulator block row per position");
 
 struct WideParams {
   const float* jac;
@@ -84,8 +81,14 @@ struct WideParams {
   float prm;
 };
 
-template <bool NORM, bool ACT>
+// PT = Jacobian rows of a tile: 32 (4 positions per tile, one per accumulator block), or 16 for
+// the activation alone (8 positions per tile, two per block: registers 0-7 of a block belong
+// to the first, 8-15 to the second), which wastes less when P is 16 more than a multiple of 32.
+template <bool NORM, bool ACT, int PT>
 __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
+  constexpr int RT = BM / PT;  // positions of a tile
+  constexpr int PB = 32 / PT;  // positions of a 32-row accumulator block
+  static_assert(PT == 32 || (PT == 16 && !NORM), "LayerNorm's row sums assume one position per block");
   __shared__ __attribute__((aligned(16))) float As0[BM * BK];
   __shared__ __attribute__((aligned(16))) float As1[BM * BK];
   __shared__ __attribute__((aligned(16))) float Ws0[BK * BN];
@@ -127,7 +130,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     const int kc = c ^ ((m / 2) % 4);
     int p = p0 + m % PT;
     if (p >= P) p = P - 1;  // reaches accumulator rows that are neither stored nor summed
-    a_p[i] = a.jac + ((int64_t)p * R + r0 + m / PT) * K + kc * 4;
+    a_p[i] = a.jac + ((int64_t)p * R + r0 + m / PT) * K + kc * 4;  // tile row m: position m / PT, row m % PT
   }
 #pragma unroll
   for (int i = 0; i < W_LD; ++i) {
@@ -151,7 +154,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   // The first chunk is on its way while what the epilogue needs per position and column is
   // staged in LDS: both are waited for together in front of the first barrier.
   issue(0, As0, Ws0);
-  float zr[TM][TN];  // without LayerNorm there are registers to spare for them
+  float zr[TM][TN][PB];  // without LayerNorm there are registers to spare for them
   if constexpr (NORM) {
     for (int e = tid; e < RT * BN; e += NT) {
       int gc = col0 + e % BN;
@@ -165,7 +168,8 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
       for (int j = 0; j < TN; ++j) {
         int gc = col0 + wc + j * 32 + l32;
         if (gc >= N) gc = N - 1;
-        zr[i][j] = a.z[(r0 + wrow * TM + i) * N + gc];
+#pragma unroll
+        for (int b = 0; b < PB; ++b) zr[i][j][b] = a.z[(r0 + (wrow * TM + i) * PB + b) * N + gc];
       }
   }
   if constexpr (NORM) {
@@ -279,36 +283,44 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     __syncthreads();
   }
 
-  // Register r of a block is Jacobian row p0 + 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32.
+  // Register r of a block is tile row 8 (r / 4) + 4 (lane / 32) + r % 4 of the block, column
+  // lane % 32: Jacobian row p0 + (that row) % PT of the block's position (that row) / PT.
   const int64_t pstride = R * N;  // floats between consecutive Jacobian rows
   const bool full_tile = (p0 + PT <= P) && (col0 + BN <= N);
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int64_t pos = r0 + wrow * TM + i;
+    const int64_t pos = r0 + (wrow * TM + i) * PB;
     float rsv = 1.0f;
     if constexpr (NORM) rsv = rsS[wrow * TM + i];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int gc = col0 + wc + j * 32 + l32;
-      float zv;
-      if constexpr (NORM) zv = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
-      else zv = zr[i][j];
-      float d1 = 1.0f;
-      if constexpr (ACT) {
-        float f, d2;
-        act_eval_fused(a.act, zv, a.prm, f, d1, d2);
+      float zv[PB], d1[PB];
+#pragma unroll
+      for (int b = 0; b < PB; ++b) {
+        if constexpr (NORM) zv[b] = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
+        else zv[b] = zr[i][j][b];
+        d1[b] = 1.0f;
+        if constexpr (ACT) {
+          float f, d2;
+          act_eval_fused(a.act, zv[b], a.prm, f, d1[b], d2);
+        }
       }
       float w1c = 0.0f, w2c = 0.0f;
       if constexpr (NORM) {
         const float2 t = wcS[wc + j * 32 + l32];
         w1c = t.x;
-        w2c = zv - t.y;
+        w2c = zv[0] - t.y;
       }
       float* out = a.y_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc;
-      float ss = 0.0f, s1 = 0.0f;
+      float ss[PB], s1 = 0.0f;
+#pragma unroll
+      for (int b = 0; b < PB; ++b) ss[b] = 0.0f;
       auto rows = [&](auto full) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+          constexpr int GB = PT / 8;     // register groups per position
+          const int b = g / GB;          // position of this group inside the block
           float ap[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
           if constexpr (NORM) {
             const float4* sp = reinterpret_cast<const float4*>(st + i * 32 + 8 * g + 4 * lh);
@@ -318,19 +330,20 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
           }
 #pragma unroll
           for (int rr = 0; rr < 4; ++rr) {
-            const int pl = 8 * g + rr;
+            const int pl = 8 * (g % GB) + rr;
             float v = acc[i][j][4 * g + rr];
             if constexpr (NORM) {
               v = fmaf(-ap[rr], w1c, v);
               s1 = fmaf(bp[rr], v, s1);
               v = fmaf(-bp[rr], w2c, v) * rsv;
             }
+            float* o = out + (int64_t)pl * pstride + (int64_t)b * N;
             if constexpr (decltype(full)::value) {
-              if constexpr (ACT) ss = fmaf(v, v, ss);
-              __builtin_nontemporal_store(d1 * v, out + (int64_t)pl * pstride);
+              if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
+              __builtin_nontemporal_store(d1[b] * v, o);
             } else if (p0 + 4 * lh + pl < P) {
-              if constexpr (ACT) ss = fmaf(v, v, ss);
-              if (gc < N) out[(int64_t)pl * pstride] = d1 * v;
+              if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
+              if (gc < N) *o = d1[b] * v;
             }
           }
         }
@@ -339,8 +352,11 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
       else rows(std::false_type{});
       const int64_t so = ((int64_t)pg * R + pos) * N + gc;
       if constexpr (ACT) {
-        ss += __shfl_xor(ss, 32, FOLX_WAVE);
-        if (lh == 0 && gc < N) a.ss[so] = ss;
+#pragma unroll
+        for (int b = 0; b < PB; ++b) {
+          const float t = ss[b] + __shfl_xor(ss[b], 32, FOLX_WAVE);
+          if (lh == 0 && gc < N) a.ss[so + (int64_t)b * N] = t;
+        }
       }
       if constexpr (NORM) {
         s1 += __shfl_xor(s1, 32, FOLX_WAVE);
@@ -496,14 +512,16 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict_
 struct WidePlan {
   int64_t row_tiles, pos_tiles, blocks, ws_bytes;
   int64_t o_ss, o_s1, o_sc, o_xhat, o_rs, o_nx, o_nlap, o_wg, o_wc;
-  int32_t PG, col_tiles;
+  int32_t PG, PT, col_tiles;
 };
 
 bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, WidePlan& pl) {
-  if (R <= 0 || R % RT != 0 || P < 1 || K < BK || K % BK != 0 || N <= 128 || N % 4 != 0) return false;
+  if (R <= 0 || R % 4 != 0 || P < 1 || K < BK || K % BK != 0 || N <= 128 || N % 4 != 0) return false;
   if (norm && K > KMAX_NORM) return false;
-  pl.PG = (P + PT - 1) / PT;
-  pl.pos_tiles = R / RT;
+  // groups of 16 Jacobian rows where that leaves fewer empty tile rows
+  pl.PT = (!norm && R % 8 == 0 && (P + 15) / 16 * 16 < (P + 31) / 32 * 32) ? 16 : 32;
+  pl.PG = (P + pl.PT - 1) / pl.PT;
+  pl.pos_tiles = R / (BM / pl.PT);
   pl.row_tiles = pl.pos_tiles * pl.PG;
   pl.col_tiles = (N + BN - 1) / BN;
   pl.blocks = (pl.row_tiles + NXCD - 1) / NXCD * NXCD * pl.col_tiles;
@@ -527,9 +545,9 @@ bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, 
   return true;
 }
 
-template <bool NORM, bool ACT>
+template <bool NORM, bool ACT, int PT>
 int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap) {
-  dense_wide_kernel<NORM, ACT><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
+  dense_wide_kernel<NORM, ACT, PT><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   int rc = folx_launch_status();
   if (rc != FOLX_HIP_OK) return rc;
   const int64_t S4 = a.R * (int64_t)a.N / 4;
@@ -578,8 +596,9 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
   int rc = folx_hip_dense_fwdlap(st, in_x, nullptr, in_lap, W, bias, nullptr, nullptr, nullptr, y, nullptr, y_lap, R,
                                  0, K, N);
   if (rc != FOLX_HIP_OK) return rc;
-  if (norm) return has_act ? launch_wide<true, true>(st, a, pl, y, y_lap) : launch_wide<true, false>(st, a, pl, y, y_lap);
-  return launch_wide<false, true>(st, a, pl, y, y_lap);
+  if (norm)
+    return has_act ? launch_wide<true, true, 32>(st, a, pl, y, y_lap) : launch_wide<true, false, 32>(st, a, pl, y, y_lap);
+  return pl.PT == 16 ? launch_wide<false, true, 16>(st, a, pl, y, y_lap) : launch_wide<false, true, 32>(st, a, pl, y, y_lap);
 }
 
 }  // namespace

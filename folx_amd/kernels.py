@@ -134,10 +134,14 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
 FUSED_ACTS = ('tanh', 'silu', 'logistic', 'sigmoid', 'softplus', 'exp', 'sin', 'cos', 'square')
 
 
-def _wide_tiles_filled(P):
-    """The wide fused kernels cut their tiles into groups of 32 Jacobian rows; a last group
-    that is mostly empty costs more MFMA work than the fusion saves."""
-    return P is None or 32 * ((P + 31) // 32) <= 1.125 * P
+def _wide_tiles_filled(P, rows, norm):
+    """The wide fused kernels cut their tiles into groups of 32 Jacobian rows (16 for the
+    activation alone over a multiple of 8 rows, where that wastes less); a last group that is
+    mostly empty costs more MFMA work than the fusion saves."""
+    if P is None:
+        return True
+    group = 16 if (not norm and rows % 8 == 0 and -(-P // 16) * 16 < -(-P // 32) * 32) else 32
+    return -(-P // group) * group <= 1.125 * P
 
 
 def dense_act_supported(name, K, N, rows=None, P=None):
@@ -149,7 +153,7 @@ def dense_act_supported(name, K, N, rows=None, P=None):
     if 4 <= K <= 128 and K % 4 == 0 and 1 <= N <= 128:
         return True
     return (rows is not None and rows > 0 and rows % 4 == 0 and K % 16 == 0 and N > 128 and N % 4 == 0
-            and _wide_tiles_filled(P))
+            and _wide_tiles_filled(P, rows, False))
 
 
 def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
@@ -183,7 +187,7 @@ def norm_dense_supported(name, K, N, rows, P=None):
     """Shapes and functions ``norm_dense`` is built for (``name`` None: no activation); with
     ``P`` (Jacobian rows) given, also whether it is the faster choice."""
     return ((name is None or name in FUSED_ACTS) and rows > 0 and rows % 4 == 0 and K % 16 == 0 and K <= 512
-            and N > 128 and N % 4 == 0 and _wide_tiles_filled(P))
+            and N > 128 and N % 4 == 0 and _wide_tiles_filled(P, rows, True))
 
 
 def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):

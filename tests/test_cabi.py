@@ -75,7 +75,9 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_dense_act_fwdlap(None, 3, 0.0, *([one] * 8), 4, 1, 8, 8, None, 0) == _lib.ENOTSUP     # log: not fused
     assert lib.folx_hip_dense_act_workspace_bytes(64, 4, 8, 200) == _lib.ENOTSUP
     assert lib.folx_hip_dense_act_workspace_bytes(1 << 20, 4, 100, 100) == 0                                  # no split
-    assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 256, 256) == 2 * 64 * 256 * 4     # wide: 2 groups of 32 rows
+    assert lib.folx_hip_dense_act_workspace_bytes(64, 64, 256, 256) == 2 * 64 * 256 * 4     # wide: 2 groups of 32 rows
+    assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 256, 256) == 3 * 64 * 256 * 4     # wide: 3 groups of 16 rows
+    assert lib.folx_hip_dense_act_workspace_bytes(60, 33, 256, 256) == 2 * 60 * 256 * 4     # rows % 8: groups of 32
     assert lib.folx_hip_dense_act_workspace_bytes(63, 33, 256, 256) == _lib.ENOTSUP         # wide: rows % 4
     assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 200, 256) == _lib.ENOTSUP         # wide: K % 16
     assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 64, 33, 256, 256, None, 0) == _lib.EINVAL  # no workspace

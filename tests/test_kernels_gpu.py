@@ -136,11 +136,13 @@ DENSE_ACT_CASES = [
     ((1, 64), 100, 100, 100, True, 'tanh'),     # one row tile, many groups
     # wide layers (N > 128): tiles of 4 positions x 32 Jacobian rows, activation in the GEMM's epilogue
     ((2, 32), 96, 256, 256, True, 'tanh'),      # transformer MLP: three full groups of 32 Jacobian rows
-    ((3, 16), 48, 832, 256, True, 'tanh'),      # one-electron stream: last group of Jacobian rows half full
-    ((1, 8), 5, 16, 132, False, 'silu'),        # one chunk of K, column tile cut at 132, one partial group
+    ((3, 16), 48, 832, 256, True, 'tanh'),      # one-electron stream: three groups of 16 Jacobian rows
+    ((1, 8), 5, 16, 132, False, 'silu'),        # one chunk of K, column tile cut at 132, one partial group of 16
     ((1, 12), 33, 64, 512, True, 'softplus'),   # two column tiles, 1 row in the second group
     ((1, 4), 64, 48, 300, True, 'sin'),         # second column tile cut at 44 columns
     ((5, 4), 1, 32, 256, False, 'square'),      # a single Jacobian row
+    ((2, 8), 40, 64, 300, True, 'tanh'),        # groups of 16 Jacobian rows, the last one half full, cut column tile
+    ((4, 16), 16, 48, 256, True, 'logistic'),   # exactly one group of 16
 ]
 
 
