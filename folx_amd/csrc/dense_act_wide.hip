@@ -65,6 +65,20 @@ constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
 constexpr int A_LD = A_V4 / NT, W_LD = W_V4 / NT;
 static_assert(A_V4 % NT == 0 && W_V4 % NT == 0, "every thread loads the same number of pieces");
 
+constexpr int MAX_PARTS = 8;
+
+// The Jacobian operand as a concatenation along K of up to MAX_PARTS arrays (widths multiples
+// of 16, so that no chunk of K straddles two).  A broadcast part has one row per `group`
+// consecutive positions (a per-walker feature shown to every electron).
+struct WideParts {
+  const float* jac[MAX_PARTS];
+  int64_t pstride[MAX_PARTS];  // floats between consecutive Jacobian rows of the part
+  int32_t width[MAX_PARTS];
+  int32_t kend[MAX_PARTS];     // first k after the part
+  int32_t bcast[MAX_PARTS];
+  int32_t n, group;
+};
+
 struct WideParams {
   const float* jac;
   const float* W;    // Wg with LayerNorm
@@ -79,13 +93,16 @@ struct WideParams {
   int64_t R, row_tiles, pos_tiles;
   int32_t P, K, N, col_tiles, act;
   float prm;
+  WideParts parts;   // PARTS instances only (jac unused then)
 };
 
 // PT = Jacobian rows of a tile: 32 (4 positions per tile, one per accumulator block), or 16 for
 // the activation alone (8 positions per tile, two per block: registers 0-7 of a block belong
 // to the first, 8-15 to the second), which wastes less when P is 16 more than a multiple of 32.
-template <bool NORM, bool ACT, int PT>
+template <bool NORM, bool ACT, int PT, bool PARTS>
 __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
+  static_assert(!PARTS || !NORM, "LayerNorm reads one array");
+  static_assert(!PARTS || A_LD == 1, "one A piece per thread");
   constexpr int RT = BM / PT;  // positions of a tile
   constexpr int PB = 32 / PT;  // positions of a 32-row accumulator block
   static_assert(PT == 32 || (PT == 16 && !NORM), "LayerNorm's row sums assume one position per block");
@@ -123,6 +140,8 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
 
   const float* a_p[A_LD];
   const float* w_p[W_LD];
+  int64_t a_pos = 0, a_posg = 0;  // PARTS: this thread's position, and its row in a broadcast part
+  int32_t a_row = 0, a_kc = 0;    //        its Jacobian row and 16-byte piece
 #pragma unroll
   for (int i = 0; i < A_LD; ++i) {
     const int idx = tid + NT * i;
@@ -130,7 +149,15 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     const int kc = c ^ ((m / 2) % 4);
     int p = p0 + m % PT;
     if (p >= P) p = P - 1;  // reaches accumulator rows that are neither stored nor summed
-    a_p[i] = a.jac + ((int64_t)p * R + r0 + m / PT) * K + kc * 4;  // tile row m: position m / PT, row m % PT
+    if constexpr (PARTS) {
+      a_pos = r0 + m / PT;
+      a_posg = a_pos / a.parts.group;
+      a_row = p;
+      a_kc = kc * 4;
+      a_p[i] = nullptr;
+    } else {
+      a_p[i] = a.jac + ((int64_t)p * R + r0 + m / PT) * K + kc * 4;  // tile row m: position m / PT, row m % PT
+    }
   }
 #pragma unroll
   for (int i = 0; i < W_LD; ++i) {
@@ -141,10 +168,21 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     w_p[i] = a.W + (int64_t)k * N + n;
   }
   auto issue = [&](int kt, float* as, float* ws) __attribute__((always_inline)) {
+    if constexpr (PARTS) {
+      // the part this chunk of K lies in: the same for the whole workgroup
+      const int k0 = kt * BK;
+      int sp = 0;
+      while (sp + 1 < a.parts.n && k0 >= a.parts.kend[sp]) ++sp;
+      const int32_t wd = a.parts.width[sp];
+      const float* src = a.parts.jac[sp] + (int64_t)a_row * a.parts.pstride[sp] +
+                         (a.parts.bcast[sp] ? a_posg : a_pos) * wd + (k0 - (a.parts.kend[sp] - wd)) + a_kc;
+      __builtin_amdgcn_global_load_lds(FOLX_GPTR(src), FOLX_LPTR(&as[(wave * 64) * 4]), 16, 0, 0);
+    } else {
 #pragma unroll
-    for (int i = 0; i < A_LD; ++i)
-      __builtin_amdgcn_global_load_lds(FOLX_GPTR(a_p[i] + kt * BK), FOLX_LPTR(&as[(wave * 64 + NT * i) * 4]), 16, 0,
-                                       0);
+      for (int i = 0; i < A_LD; ++i)
+        __builtin_amdgcn_global_load_lds(FOLX_GPTR(a_p[i] + kt * BK), FOLX_LPTR(&as[(wave * 64 + NT * i) * 4]), 16,
+                                         0, 0);
+    }
 #pragma unroll
     for (int i = 0; i < W_LD; ++i)
       __builtin_amdgcn_global_load_lds(FOLX_GPTR(w_p[i] + (int64_t)kt * BK * N),
@@ -545,9 +583,9 @@ bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, 
   return true;
 }
 
-template <bool NORM, bool ACT, int PT>
+template <bool NORM, bool ACT, int PT, bool PARTS = false>
 int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap) {
-  dense_wide_kernel<NORM, ACT, PT><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
+  dense_wide_kernel<NORM, ACT, PT, PARTS><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   int rc = folx_launch_status();
   if (rc != FOLX_HIP_OK) return rc;
   const int64_t S4 = a.R * (int64_t)a.N / 4;
@@ -559,12 +597,13 @@ int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* 
 int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x, const float* jac, const float* lap,
              const float* gamma, const float* beta, float eps, const float* W, const float* bias, float* y,
              float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
-             int64_t workspace_bytes) {
+             int64_t workspace_bytes, const WideParts* parts = nullptr) {
   const bool has_act = act >= 0;
   WidePlan pl;
   if ((has_act && !act_fused(act)) || !plan_wide(R, P, K, N, norm, has_act, pl)) return FOLX_HIP_ENOTSUP;
   if (!norm && !has_act) return FOLX_HIP_ENOTSUP;  // that is the plain dense rule
-  if (!x || !jac || !lap || !W || !y || !y_jac || !y_lap) return FOLX_HIP_EINVAL;
+  if (parts && norm) return FOLX_HIP_ENOTSUP;
+  if (!x || (!jac && !parts) || !lap || !W || !y || !y_jac || !y_lap) return FOLX_HIP_EINVAL;
   if (!folx_aligned16(jac) || !folx_aligned16(W) || !folx_aligned16(y) || !folx_aligned16(y_lap))
     return FOLX_HIP_ENOTSUP;
   if (norm && (!folx_aligned16(x) || !folx_aligned16(lap) || !folx_aligned16(gamma) || !folx_aligned16(beta)))
@@ -598,6 +637,11 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
   if (rc != FOLX_HIP_OK) return rc;
   if (norm)
     return has_act ? launch_wide<true, true, 32>(st, a, pl, y, y_lap) : launch_wide<true, false, 32>(st, a, pl, y, y_lap);
+  if (parts) {
+    a.parts = *parts;
+    return pl.PT == 16 ? launch_wide<false, true, 16, true>(st, a, pl, y, y_lap)
+                       : launch_wide<false, true, 32, true>(st, a, pl, y, y_lap);
+  }
   return pl.PT == 16 ? launch_wide<false, true, 16>(st, a, pl, y, y_lap) : launch_wide<false, true, 32>(st, a, pl, y, y_lap);
 }
 
@@ -632,4 +676,35 @@ extern "C" int folx_hip_norm_dense_fwdlap(void* stream, int32_t act, float param
   if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
   return run_wide((hipStream_t)stream, true, act, param, x, jac, lap, gamma, beta, eps, W, bias, y, y_jac, y_lap, R, P,
                   K, N, workspace, workspace_bytes);
+}
+
+extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float param, const float* x,
+                                               const float* lap, int32_t n_parts, const float* const* jac_parts,
+                                               const int32_t* widths, const int32_t* broadcast, int32_t group,
+                                               const float* W, const float* bias, float* y, float* y_jac,
+                                               float* y_lap, int64_t R, int32_t P, int32_t N, void* workspace,
+                                               int64_t workspace_bytes) {
+  if (R < 0 || P < 0 || N <= 0 || n_parts < 1 || group < 1 || !jac_parts || !widths || !broadcast)
+    return FOLX_HIP_EINVAL;
+  if (n_parts > MAX_PARTS || act < 0 || R % group != 0) return FOLX_HIP_ENOTSUP;
+  WideParts parts;
+  parts.n = n_parts;
+  parts.group = group;
+  int32_t K = 0;
+  for (int i = 0; i < n_parts; ++i) {
+    if (widths[i] <= 0 || widths[i] % BK != 0) return FOLX_HIP_ENOTSUP;
+    if (!jac_parts[i]) return FOLX_HIP_EINVAL;
+    if (!folx_aligned16(jac_parts[i])) return FOLX_HIP_ENOTSUP;
+    parts.jac[i] = jac_parts[i];
+    parts.width[i] = widths[i];
+    parts.bcast[i] = broadcast[i] ? 1 : 0;
+    parts.pstride[i] = (broadcast[i] ? R / group : R) * (int64_t)widths[i];
+    K += widths[i];
+    parts.kend[i] = K;
+  }
+  for (int i = n_parts; i < MAX_PARTS; ++i) {
+    parts.jac[i] = nullptr; parts.width[i] = 0; parts.bcast[i] = 0; parts.pstride[i] = 0; parts.kend[i] = K;
+  }
+  return run_wide((hipStream_t)stream, false, act, param, x, nullptr, lap, nullptr, nullptr, 0.0f, W, bias, y, y_jac,
+                  y_lap, R, P, K, N, workspace, workspace_bytes, &parts);
 }

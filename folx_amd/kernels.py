@@ -183,6 +183,43 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return y, yj, yl
 
 
+def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0):
+    """``dense_act`` of a wide layer whose Jacobian operand is the concatenation along the
+    feature axis of ``jac_parts`` (never formed): part i is (P, rows_i, widths[i]) with rows_i
+    the layer's rows, or one row per ``group`` of them where ``broadcast[i]``; x and lap are
+    the concatenated arrays (.., K)."""
+    _chk(x, lap, W, bias, *jac_parts)
+    K, N = W.shape
+    assert sum(widths) == K and x.shape[-1] == K
+    P = jac_parts[0].shape[0]
+    lead = tuple(x.shape[:-1])
+    R = int(np.prod(lead, dtype=np.int64))
+    n = len(jac_parts)
+    for J, w, bc in zip(jac_parts, widths, broadcast):
+        assert J.is_contiguous() and J.shape[0] == P and J.numel() == P * (R // group if bc else R) * w
+    x, lap = x.contiguous(), lap.contiguous()
+    lib = _lib.load()
+    nbytes = int(lib.folx_hip_dense_act_workspace_bytes(R, P, K, N))
+    if nbytes < 0:
+        check(nbytes, 'dense_act_workspace_bytes')
+    ws = torch.empty(max(nbytes // 4, 1), device=x.device, dtype=torch.float32)
+    y = torch.empty((*lead, N), device=x.device, dtype=torch.float32)
+    yj = torch.empty((P, *lead, N), device=x.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    ptrs = (ctypes.c_void_p * n)(*[J.data_ptr() for J in jac_parts])
+    wd = (ctypes.c_int32 * n)(*[int(w) for w in widths])
+    bc = (ctypes.c_int32 * n)(*[int(bool(b)) for b in broadcast])
+    with _timed('dense_act_fwdlap', (name, R, P, K, N)):
+        check(
+            lib.folx_hip_dense_act_parts_fwdlap(
+                _stream(), ACT[name], float(param), _p(x), _p(lap), n, ptrs, wd, bc, int(group), _p(W), _p(bias),
+                _p(y), _p(yj), _p(yl), R, P, N, _p(ws), nbytes
+            ),
+            f'dense_act_parts_fwdlap[{name}]',
+        )
+    return y, yj, yl
+
+
 def norm_dense_supported(name, K, N, rows, P=None):
     """Shapes and functions ``norm_dense`` is built for (``name`` None: no activation); with
     ``P`` (Jacobian rows) given, also whether it is the faster choice."""

@@ -287,8 +287,13 @@ def squeeze(a, axis):
     return reshape(a, shape)
 
 
-def broadcast_to(a, shape):
+def broadcast_to(a, shape, lazy=False):
+    """``lazy=True`` returns a handle that only a lazy ``concatenate`` accepts."""
     shape = tuple(shape)
+    if lazy and isinstance(a, FwdLaplArray):
+        from .wrapped_functions import LazyBroadcast
+
+        return LazyBroadcast(a, shape)
     src = _shape(a)
     off = len(shape) - len(src)
     return _call('broadcast_in_dim', (a,), {'shape': shape, 'broadcast_dimensions': tuple(range(off, len(shape)))})
@@ -298,8 +303,17 @@ def getitem(a, idx):
     return _call('slice', (a,), {'idx': idx})
 
 
-def concatenate(arrs, axis=-1):
-    return _call('concatenate', tuple(arrs), {'dimension': axis})
+def concatenate(arrs, axis=-1, lazy=False):
+    """``lazy=True`` (last axis only) returns a handle that only ``dot`` accepts as its first
+    operand: a product that can read its operand in parts never forms the concatenation."""
+    from .wrapped_functions import LazyBroadcast, LazyConcat
+
+    arrs = tuple(arrs)
+    if lazy and axis == -1 and all(isinstance(t, (FwdLaplArray, LazyBroadcast)) for t in arrs):
+        return LazyConcat(arrs)
+    thr = current_threshold()
+    arrs = tuple(t.value(thr) if isinstance(t, LazyBroadcast) else t for t in arrs)
+    return _call('concatenate', arrs, {'dimension': axis})
 
 
 # composed rules ---------------------------------------------------------------------------

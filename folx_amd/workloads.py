@@ -288,8 +288,10 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         gu = xp.mean(xp.getitem(g, (slice(None), slice(0, nu))), axis=1)
         gd = xp.mean(xp.getitem(g, (slice(None), slice(nu, n))), axis=1)
         d1 = h.shape[-1]
-        parts = [h, xp.broadcast_to(hu, (n, d1)), xp.broadcast_to(hd, (n, d1)), gu, gd]
-        f = xp.concatenate(parts, axis=-1)
+        # the feature vector is only consumed by the product below, which reads it part by
+        # part where it can: neither the broadcasts nor the concatenation are then formed
+        parts = [h, xp.broadcast_to(hu, (n, d1), lazy=True), xp.broadcast_to(hd, (n, d1), lazy=True), gu, gd]
+        f = xp.concatenate(parts, axis=-1, lazy=True)
         hn = xp.dot(f, L['v'], L['b'], act='tanh')
         h = xp.add(h, hn) if hn.shape == h.shape else hn
         if 'w' in L:

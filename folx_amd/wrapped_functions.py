@@ -456,6 +456,8 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     is what the reference's general path produces for this case (folx/jvp.py:224-230).
     """
     h, W = args
+    if isinstance(h, LazyConcat):
+        return _dot_parts(h, W, kwargs, sparsity_threshold)
     bias = kwargs.get('bias')
     residual = kwargs.get('residual')
     row_slice = kwargs.get('row_slice')
@@ -645,6 +647,98 @@ class LazyLayerNorm:
         if self._value is None:
             self._value = layer_norm_rule((self.h, self.gamma, self.beta), {'eps': self.eps}, sparsity_threshold)
         return self._value
+
+
+class LazyBroadcast:
+    """``broadcast_to(a, shape)`` that has not been evaluated; a lazy ``concatenate`` is the
+    only consumer that can take it as it is."""
+
+    __slots__ = ('a', 'shape', '_value')
+
+    def __init__(self, a, shape):
+        self.a, self.shape, self._value = a, tuple(shape), None
+
+    def value(self, sparsity_threshold):
+        if self._value is None:
+            off = len(self.shape) - self.a.ndim
+            self._value = _LAPLACE_FN_REGISTRY['broadcast_in_dim'](
+                (self.a,), {'shape': self.shape, 'broadcast_dimensions': tuple(range(off, len(self.shape)))},
+                sparsity_threshold)
+        return self._value
+
+
+class LazyConcat:
+    """``concatenate(parts, axis=-1)`` that has not been evaluated, for feature vectors whose only
+    consumer is a matrix product (``numpy.dot``): a product that can read its operand in parts
+    never forms the concatenation (nor the broadcasts among the parts), any other evaluates
+    it once."""
+
+    __slots__ = ('parts', '_value')
+
+    def __init__(self, parts):
+        self.parts, self._value = tuple(parts), None
+
+    def value(self, sparsity_threshold):
+        if self._value is None:
+            parts = tuple(t.value(sparsity_threshold) if isinstance(t, LazyBroadcast) else t for t in self.parts)
+            self._value = concatenate_rule(parts, {'dimension': -1}, sparsity_threshold)
+        return self._value
+
+
+def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
+    """``act(concatenate(parts) @ W + bias)`` with the Jacobian read part by part
+    (``kernels.dense_act_parts``) when every part is a triplet of the output's leading shape,
+    or a per-walker vector broadcast to it, with a width that is a multiple of 16, and the
+    layer is one the wide fused kernel takes; otherwise the concatenation is evaluated and
+    the product goes the usual way."""
+    act, param, residual = kwargs.get('act'), kwargs.get('act_param', 0.0), kwargs.get('residual')
+    ok = (act is not None and kwargs.get('norm') is None and kwargs.get('row_slice') is None and not _is(W)
+          and np.ndim(W) == 2 and 1 <= len(lc.parts) <= 8)
+    lead = None
+    if ok:
+        for t in lc.parts:
+            src = t.a if isinstance(t, LazyBroadcast) else t
+            if not _is(src) or src.ndim < 1 or src.shape[-1] % 16 != 0:
+                ok = False
+                break
+            if isinstance(t, LazyBroadcast):
+                ok = ok and src.ndim == 1 and t.shape[-1] == src.shape[-1]
+                tl = tuple(t.shape[:-1])
+            else:
+                tl = tuple(src.shape[:-1])
+            if lead is None:
+                lead = tl
+            ok = ok and tl == lead
+    if ok:
+        first = lc.parts[0].a if isinstance(lc.parts[0], LazyBroadcast) else lc.parts[0]
+        B, dev = first.B, first.x.device
+        group = int(np.prod(lead, dtype=np.int64))
+        Ktot = sum((t.a if isinstance(t, LazyBroadcast) else t).shape[-1] for t in lc.parts)
+        srcs = [t.a if isinstance(t, LazyBroadcast) else t for t in lc.parts]
+        P = max(u.jacobian.max_n + 1 if u.jacobian.weak else u.jacobian.data.shape[0] for u in srcs)
+        ok = (np.shape(W)[0] == Ktot and np.shape(W)[1] > 128 and group >= 1
+              and K.dense_act_supported(act, Ktot, np.shape(W)[1], rows=B * group, P=P))
+    if not ok:
+        kw = dict(kwargs)
+        return dot_general((lc.value(thr), W), kw, thr)
+    xs, ls, Js, widths, flags = [], [], [], [], []
+    for t, u in zip(lc.parts, srcs):
+        J = so.pad_rows(u.jacobian.dense_array, P).contiguous()
+        if isinstance(t, LazyBroadcast):
+            shp = (B, *([1] * len(lead)), u.shape[-1])
+            xs.append(u.x.reshape(shp).expand(B, *lead, u.shape[-1]))
+            ls.append(u.laplacian.reshape(shp).expand(B, *lead, u.shape[-1]))
+        else:
+            xs.append(u.x), ls.append(u.laplacian)
+        Js.append(J), widths.append(u.shape[-1]), flags.append(isinstance(t, LazyBroadcast))
+    bias = kwargs.get('bias')
+    y, Jy, lapy = K.dense_act_parts(act, torch.cat(xs, dim=-1), torch.cat(ls, dim=-1), Js, widths, flags, group,
+                                    so.device_const(W, dev), None if bias is None else so.device_const(bias, dev),
+                                    param)
+    out = FwdLaplArray(y, FwdJacobian(Jy, None), lapy)
+    if residual is not None:
+        out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)
+    return out
 
 
 def layer_norm_rule(args, kwargs, sparsity_threshold):

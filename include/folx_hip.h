@@ -169,6 +169,27 @@ int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const floa
                               int64_t workspace_bytes);
 
 /*
+ * folx_hip_dense_act_fwdlap for a wide layer whose input is a concatenation along the feature
+ * axis that is never formed: part i contributes widths[i] consecutive features (multiples of
+ * 16, at most 8 parts, K = their sum), jac_parts[i] is its Jacobian [P][rows_i][widths[i]]
+ * with rows_i = R, or R / group when broadcast[i] is set: then the part has one row per
+ * `group` consecutive rows of the layer (a per-walker feature shown to every electron,
+ * jax.lax.broadcast_in_dim before jax.lax.concatenate in the reference's trace; rules
+ * folx/wrapped_functions.py:361-376 on the way into _dot_general_one_constant, :71-171).
+ * x and lap are the concatenated [R][K] arrays (1 / (P + 2) of the data; only the Jacobian
+ * is read in parts).  jac_parts, widths and broadcast are HOST arrays.  Same shapes,
+ * activations and workspace as the wide path of folx_hip_dense_act_fwdlap
+ * (folx_hip_dense_act_workspace_bytes(R, P, K, N)); FOLX_HIP_ENOTSUP otherwise.
+ */
+int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float param, const float* x,
+                                    const float* lap, int32_t n_parts,
+                                    const float* const* jac_parts, const int32_t* widths,
+                                    const int32_t* broadcast, int32_t group, const float* W,
+                                    const float* bias, float* y, float* y_jac, float* y_lap,
+                                    int64_t R, int32_t P, int32_t N, void* workspace,
+                                    int64_t workspace_bytes);
+
+/*
  * LayerNorm over the K features, then a dense layer, then (act >= 0) an activation, as one
  * rule:  y = f(LN(x) @ W + bias),  LN(x) = gamma * (x - mean) * rsqrt(var + eps) + beta.
  * The triplet that results is the one of folx_hip_layernorm_fwdlap followed by

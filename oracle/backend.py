@@ -440,8 +440,8 @@ def expand_dims(a: OArr, axis):
     )
 
 
-def broadcast_to(a: OArr, shape):
-    shape = tuple(shape)
+def broadcast_to(a: OArr, shape, lazy=False):
+    shape = tuple(shape)  # ``lazy`` is a scheduling hint of the device front end; the value is the same
     ex = len(shape) - a.ndim
     x = a.x.reshape(a.B, *([1] * ex), *a.shape)
     J = a.J.reshape(a.P, a.B, *([1] * ex), *a.shape)
@@ -461,7 +461,7 @@ def getitem(a: OArr, idx):
     )
 
 
-def concatenate(arrs, axis=-1):
+def concatenate(arrs, axis=-1, lazy=False):
     first = [t for t in arrs if _is(t)][0]
     nd = first.ndim
     axis = axis % nd

@@ -140,7 +140,7 @@ class plain:
         return a.unsqueeze(axis)
 
     @staticmethod
-    def broadcast_to(a, shape):
+    def broadcast_to(a, shape, lazy=False):
         return a.expand(tuple(shape))
 
     @staticmethod
@@ -148,7 +148,7 @@ class plain:
         return a[idx]
 
     @staticmethod
-    def concatenate(arrs, axis=-1):
+    def concatenate(arrs, axis=-1, lazy=False):
         like = [t for t in arrs if isinstance(t, torch.Tensor)][0]
         return torch.cat([plain._c(t, like) for t in arrs], dim=axis)
 

@@ -37,6 +37,18 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
 
 
+def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0):
+    P = jac_parts[0].shape[0]
+    lead = tuple(x.shape[:-1])
+    R = int(np.prod(lead))
+    Js = []
+    for J, w, bc in zip(jac_parts, widths, broadcast):
+        Jn = _n(J).reshape(P, R // group if bc else R, w)
+        Js.append(np.repeat(Jn, group, axis=1) if bc else Jn)
+    J = _t(np.concatenate(Js, axis=-1).reshape(P, *lead, sum(widths)))
+    return dense_act(name, x, J, lap, W, bias, param)
+
+
 def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):
     n = layernorm(x, jac, lap, gamma, beta, eps)
     if name is None:
@@ -224,7 +236,7 @@ def install(monkeypatch):
     import folx_amd.interpreter as interp
     import folx_amd.kernels as K
 
-    for name in ('dense', 'dense_act', 'norm_dense', 'exp_envelope', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
+    for name in ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'exp_envelope', 'layernorm', 'elementwise', 'binary', 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max',
                  'gather_rows', 'gather_cols', 'scatter_add_rows', 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse'):
         monkeypatch.setattr(K, name, globals()[name])
     monkeypatch.setattr(interp, '_device', lambda: torch.device('cpu'))

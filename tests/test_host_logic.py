@@ -432,6 +432,44 @@ def test_dot_norm(thr, monkeypatch):
     assert len(lns) == (2 if thr == 0 else 3)
 
 
+@pytest.mark.parametrize('thr', [0, 6])
+def test_dot_of_lazy_concatenate(thr, monkeypatch):
+    """``dot(concatenate(parts, lazy=True), W, b, act=...)`` equals the evaluated chain: read
+    part by part where the fused kernel applies (widths that are multiples of 16, a wide
+    layer; per-walker vectors broadcast among the parts, a sparse part densified), evaluated
+    once otherwise (a narrow layer, a width of 8)."""
+    from folx_amd import kernels as K
+
+    calls = []
+    orig = K.dense_act_parts
+    monkeypatch.setattr(K, 'dense_act_parts', lambda *a: (calls.append((tuple(a[4]), tuple(a[5]), a[6])), orig(*a))[1])
+    rng = np.random.default_rng(14)
+    n = 10
+    W0 = rng.normal(size=(3, 16)).astype(np.float32)
+    Wm = rng.normal(size=(16, 32)).astype(np.float32) / 4
+    W1 = rng.normal(size=(16 + 32 + 16 + 16, 132)).astype(np.float32) / 9
+    b1 = rng.normal(size=(132,)).astype(np.float32)
+    W2 = rng.normal(size=(16 + 16, 24)).astype(np.float32) / 6
+    W3 = rng.normal(size=(16 + 8, 136)).astype(np.float32) / 5
+    x = rng.normal(size=(2, n, 3)).astype(np.float32)
+
+    def fn(xp, t):
+        e = xp.dot(t, W0)                                   # (n, 16), sparse rows at thr 6
+        m = xp.mean(xp.tanh(e), axis=0)                     # (16,) per walker, dense
+        h = xp.tanh(xp.dot(xp.add(e, m), Wm))               # (n, 32) dense
+        parts = [e, h, xp.broadcast_to(m, (n, 16), lazy=True), xp.broadcast_to(xp.square(m), (n, 16), lazy=True)]
+        f = xp.concatenate(parts, axis=-1, lazy=True)
+        a = xp.dot(f, W1, b1, act='tanh')                   # fused: four parts, two of them broadcast
+        f2 = xp.concatenate([e, xp.broadcast_to(m, (n, 16), lazy=True)], axis=-1, lazy=True)
+        b = xp.dot(f2, W2, act='silu')                      # narrow layer: concatenation evaluated
+        f3 = xp.concatenate([e, xp.getitem(h, (slice(None), slice(0, 8)))], axis=-1, lazy=True)
+        c = xp.dot(f3, W3, act='sin', residual=None)        # a width of 8: concatenation evaluated
+        return xp.add(xp.add(xp.sum(a), xp.sum(b)), xp.sum(c))
+
+    check_against_oracle(fn, x, thr)
+    assert calls == [((16, 32, 16, 16), (False, False, True, True), n)]
+
+
 def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
     """q, k, v of the first PsiFormer layer still carry per-electron sparse Jacobians: the rule
     hands them to the position-sparse kernel and the result equals the densified rule."""

@@ -243,6 +243,37 @@ def test_norm_dense_matches_three_kernels_large():
                                        msg=lambda m: f'{act} {nm}: {m}')
 
 
+@pytest.mark.parametrize('B,n,P,widths,bcast,N,act', [
+    (4, 16, 48, (256, 256, 256, 32, 32), (0, 1, 1, 0, 0), 256, 'tanh'),   # FermiNet-style one-electron layer
+    (2, 6, 30, (16, 32), (1, 0), 132, 'silu'),                            # groups of 32 rows (12 positions), broadcast part first
+    (1, 8, 5, (48,), (0,), 300, 'sin'),                                   # a single part
+    (3, 8, 17, (16, 16, 16, 16, 16, 16, 16, 16), (0, 1, 0, 1, 0, 1, 0, 1), 256, 'softplus'),  # eight parts
+])
+def test_dense_act_parts(B, n, P, widths, bcast, N, act):
+    """The wide dense + activation rule reading its Jacobian operand part by part equals the
+    oracle's rules on the concatenated operand."""
+    from folx_amd import kernels as K
+
+    print(f'case dense_act_parts B={B} n={n} P={P} widths={widths} bcast={bcast} N={N}', flush=True)
+    rng = np.random.default_rng(29)
+    Kd = sum(widths)
+    xs, ls, Js, Jd = [], [], [], []
+    for w, bc in zip(widths, bcast):
+        lead = (B,) if bc else (B, n)
+        xp_, lp_, Jp = rand(rng, *lead, w), rand(rng, *lead, w), rand(rng, P, *lead, w)
+        Js.append(Jp)
+        if bc:
+            xp_, lp_, Jp = (np.broadcast_to(np.expand_dims(t, -2), (*t.shape[:-1], n, w)) for t in (xp_, lp_, Jp))
+        xs.append(xp_), ls.append(lp_), Jd.append(Jp)
+    x, L, J = np.concatenate(xs, -1), np.concatenate(ls, -1), np.concatenate(Jd, -1)
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N)
+    ref = rules.elementwise_rule(act, *rules.dense_rule(*f64(x, J, L, W), b.astype(np.float64)))
+    for rep in range(2):
+        got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b))
+        assert_triplet(got, ref, f'dense_act_parts call {rep}')
+
+
 def test_dense_act_wide_matches_two_kernels_large():
     """A transformer MLP layer at a full chunk: the fused wide path and dense + elementwise
     agree to rounding (the sums over Jacobian rows are taken in a different order)."""
