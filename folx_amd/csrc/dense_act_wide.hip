@@ -87,6 +87,7 @@ struct WideParams {
   const float* rs;   // (R)
   const float2* wc;  // (N) pairs (w1, c0)
   float* y_jac;
+  const float* res_jac;  // optional (P, R, N) added to the activated Jacobian rows     PARTS instances only
   float* ss;         // (PG, R, N) sums of zj^2 per group of PT Jacobian rows     activation only
   float* s1;         // (PG, R, N) sums of b_p (t_p @ Wg - a_p w1)                LayerNorm only
   float* sc;         // (PG, R, 2) sums of b_p^2 and of q_p
@@ -354,7 +355,9 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
       float ss[PB], s1 = 0.0f;
 #pragma unroll
       for (int b = 0; b < PB; ++b) ss[b] = 0.0f;
-      auto rows = [&](auto full) __attribute__((always_inline)) {
+      const float* resp = nullptr;
+      if constexpr (PARTS) resp = a.res_jac ? a.res_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc : nullptr;
+      auto rows = [&](auto full, auto has_res) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           constexpr int GB = PT / 8;     // register groups per position
@@ -375,19 +378,27 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
               s1 = fmaf(bp[rr], v, s1);
               v = fmaf(-bp[rr], w2c, v) * rsv;
             }
-            float* o = out + (int64_t)pl * pstride + (int64_t)b * N;
+            const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
+            float* o = out + off;
             if constexpr (decltype(full)::value) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
-              __builtin_nontemporal_store(d1[b] * v, o);
+              float w = d1[b] * v;
+              if constexpr (decltype(has_res)::value) w += __builtin_nontemporal_load(resp + off);
+              __builtin_nontemporal_store(w, o);
             } else if (p0 + 4 * lh + pl < P) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
-              if (gc < N) *o = d1[b] * v;
+              if (gc < N) *o = d1[b] * v + (decltype(has_res)::value ? resp[off] : 0.0f);
             }
           }
         }
       };
-      if (full_tile) rows(std::true_type{});
-      else rows(std::false_type{});
+      if (PARTS && resp != nullptr) {
+        if (full_tile) rows(std::true_type{}, std::true_type{});
+        else rows(std::false_type{}, std::true_type{});
+      } else {
+        if (full_tile) rows(std::true_type{}, std::false_type{});
+        else rows(std::false_type{}, std::false_type{});
+      }
       const int64_t so = ((int64_t)pg * R + pos) * N + gc;
       if constexpr (ACT) {
 #pragma unroll
@@ -411,7 +422,9 @@ __global__ __launch_bounds__(256) void dense_wide_finish(float* __restrict__ y, 
                                                          const float* __restrict__ ss, const float* __restrict__ s1,
                                                          const float* __restrict__ sc, const float* __restrict__ rs,
                                                          const float2* __restrict__ wc, int64_t S4, int64_t R,
-                                                         int32_t N, int32_t PG, int32_t act, float prm) {
+                                                         int32_t N, int32_t PG, int32_t act, float prm,
+                                                         const float* __restrict__ res,
+                                                         const float* __restrict__ res_lap) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= S4) return;
   const float4 z = reinterpret_cast<const float4*>(y)[i];
@@ -446,7 +459,15 @@ __global__ __launch_bounds__(256) void dense_wide_finish(float* __restrict__ y, 
     act_eval_fused(act, z.y, prm, f.y, d1, d2); zl.y = fmaf(d1, zl.y, d2 * s.y);
     act_eval_fused(act, z.z, prm, f.z, d1, d2); zl.z = fmaf(d1, zl.z, d2 * s.z);
     act_eval_fused(act, z.w, prm, f.w, d1, d2); zl.w = fmaf(d1, zl.w, d2 * s.w);
+    if (res) {
+      const float4 r = reinterpret_cast<const float4*>(res)[i];
+      f.x += r.x; f.y += r.y; f.z += r.z; f.w += r.w;
+    }
     reinterpret_cast<float4*>(y)[i] = f;
+  }
+  if (res_lap) {
+    const float4 r = reinterpret_cast<const float4*>(res_lap)[i];
+    zl.x += r.x; zl.y += r.y; zl.z += r.z; zl.w += r.w;
   }
   reinterpret_cast<float4*>(y_lap)[i] = zl;
 }
@@ -584,20 +605,22 @@ bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, 
 }
 
 template <bool NORM, bool ACT, int PT, bool PARTS = false>
-int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap) {
+int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap,
+                const float* res = nullptr, const float* res_lap = nullptr) {
   dense_wide_kernel<NORM, ACT, PT, PARTS><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   int rc = folx_launch_status();
   if (rc != FOLX_HIP_OK) return rc;
   const int64_t S4 = a.R * (int64_t)a.N / 4;
   dense_wide_finish<NORM, ACT><<<dim3((unsigned)((S4 + 255) / 256)), dim3(256), 0, st>>>(
-      y, y_lap, a.ss, a.s1, a.sc, a.rs, a.wc, S4, a.R, a.N, pl.PG, a.act, a.prm);
+      y, y_lap, a.ss, a.s1, a.sc, a.rs, a.wc, S4, a.R, a.N, pl.PG, a.act, a.prm, res, res_lap);
   return folx_launch_status();
 }
 
 int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x, const float* jac, const float* lap,
              const float* gamma, const float* beta, float eps, const float* W, const float* bias, float* y,
              float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
-             int64_t workspace_bytes, const WideParts* parts = nullptr) {
+             int64_t workspace_bytes, const WideParts* parts = nullptr, const float* res = nullptr,
+             const float* res_jac = nullptr, const float* res_lap = nullptr) {
   const bool has_act = act >= 0;
   WidePlan pl;
   if ((has_act && !act_fused(act)) || !plan_wide(R, P, K, N, norm, has_act, pl)) return FOLX_HIP_ENOTSUP;
@@ -611,7 +634,7 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
   if (!workspace || workspace_bytes < pl.ws_bytes || !folx_aligned16(workspace)) return FOLX_HIP_EINVAL;
   float* ws = (float*)workspace;
   WideParams a;
-  a.jac = jac; a.W = W; a.z = y; a.y_jac = y_jac;
+  a.jac = jac; a.W = W; a.z = y; a.y_jac = y_jac; a.res_jac = res_jac;
   a.xhat = nullptr; a.rs = nullptr; a.wc = nullptr;
   a.ss = ws + pl.o_ss; a.s1 = nullptr; a.sc = nullptr;
   a.R = R; a.row_tiles = pl.row_tiles; a.pos_tiles = pl.pos_tiles;
@@ -639,8 +662,8 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
     return has_act ? launch_wide<true, true, 32>(st, a, pl, y, y_lap) : launch_wide<true, false, 32>(st, a, pl, y, y_lap);
   if (parts) {
     a.parts = *parts;
-    return pl.PT == 16 ? launch_wide<false, true, 16, true>(st, a, pl, y, y_lap)
-                       : launch_wide<false, true, 32, true>(st, a, pl, y, y_lap);
+    return pl.PT == 16 ? launch_wide<false, true, 16, true>(st, a, pl, y, y_lap, res, res_lap)
+                       : launch_wide<false, true, 32, true>(st, a, pl, y, y_lap, res, res_lap);
   }
   return pl.PT == 16 ? launch_wide<false, true, 16>(st, a, pl, y, y_lap) : launch_wide<false, true, 32>(st, a, pl, y, y_lap);
 }
@@ -681,11 +704,14 @@ extern "C" int folx_hip_norm_dense_fwdlap(void* stream, int32_t act, float param
 extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float param, const float* x,
                                                const float* lap, int32_t n_parts, const float* const* jac_parts,
                                                const int32_t* widths, const int32_t* broadcast, int32_t group,
-                                               const float* W, const float* bias, float* y, float* y_jac,
-                                               float* y_lap, int64_t R, int32_t P, int32_t N, void* workspace,
-                                               int64_t workspace_bytes) {
+                                               const float* W, const float* bias, const float* res,
+                                               const float* res_jac, const float* res_lap, float* y,
+                                               float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t N,
+                                               void* workspace, int64_t workspace_bytes) {
   if (R < 0 || P < 0 || N <= 0 || n_parts < 1 || group < 1 || !jac_parts || !widths || !broadcast)
     return FOLX_HIP_EINVAL;
+  if ((res != nullptr) != (res_jac != nullptr) || (res != nullptr) != (res_lap != nullptr)) return FOLX_HIP_EINVAL;
+  if (!folx_aligned16(res) || !folx_aligned16(res_lap)) return FOLX_HIP_ENOTSUP;
   if (n_parts > MAX_PARTS || act < 0 || R % group != 0) return FOLX_HIP_ENOTSUP;
   WideParts parts;
   parts.n = n_parts;
@@ -706,5 +732,5 @@ extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float 
     parts.jac[i] = nullptr; parts.width[i] = 0; parts.bcast[i] = 0; parts.pstride[i] = 0; parts.kend[i] = K;
   }
   return run_wide((hipStream_t)stream, false, act, param, x, nullptr, lap, nullptr, nullptr, 0.0f, W, bias, y, y_jac,
-                  y_lap, R, P, K, N, workspace, workspace_bytes, &parts);
+                  y_lap, R, P, K, N, workspace, workspace_bytes, &parts, res, res_jac, res_lap);
 }

@@ -292,8 +292,10 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
         # part where it can: neither the broadcasts nor the concatenation are then formed
         parts = [h, xp.broadcast_to(hu, (n, d1), lazy=True), xp.broadcast_to(hd, (n, d1), lazy=True), gu, gd]
         f = xp.concatenate(parts, axis=-1, lazy=True)
-        hn = xp.dot(f, L['v'], L['b'], act='tanh')
-        h = xp.add(h, hn) if hn.shape == h.shape else hn
+        if L['v'].shape[1] == d1:  # residual layer: the skip connection is added in the product's epilogue
+            h = xp.dot(f, L['v'], L['b'], act='tanh', residual=h)
+        else:
+            h = xp.dot(f, L['v'], L['b'], act='tanh')
         if 'w' in L:
             gn = xp.dot(g, L['w'], L['c'], act='tanh')
             g = xp.add(g, gn) if gn.shape == g.shape else gn

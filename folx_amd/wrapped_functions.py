@@ -732,11 +732,15 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
             xs.append(u.x), ls.append(u.laplacian)
         Js.append(J), widths.append(u.shape[-1]), flags.append(isinstance(t, LazyBroadcast))
     bias = kwargs.get('bias')
+    res = None  # a skip connection with the same dense rows goes into the kernel's epilogue
+    if (_is(residual) and residual.jacobian.x0_idx is None and residual.jacobian.data.shape[0] == P
+            and tuple(residual.shape) == (*lead, np.shape(W)[1])):
+        res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
     y, Jy, lapy = K.dense_act_parts(act, torch.cat(xs, dim=-1), torch.cat(ls, dim=-1), Js, widths, flags, group,
                                     so.device_const(W, dev), None if bias is None else so.device_const(bias, dev),
-                                    param)
+                                    param, res)
     out = FwdLaplArray(y, FwdJacobian(Jy, None), lapy)
-    if residual is not None:
+    if residual is not None and res is None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)
     return out
 

@@ -180,12 +180,15 @@ int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const floa
  * is read in parts).  jac_parts, widths and broadcast are HOST arrays.  Same shapes,
  * activations and workspace as the wide path of folx_hip_dense_act_fwdlap
  * (folx_hip_dense_act_workspace_bytes(R, P, K, N)); FOLX_HIP_ENOTSUP otherwise.
+ * res / res_jac / res_lap (all or none; shapes of y / y_jac / y_lap) are added to the
+ * activated result: the skip connection of a residual layer (add_p after the activation).
  */
 int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float param, const float* x,
                                     const float* lap, int32_t n_parts,
                                     const float* const* jac_parts, const int32_t* widths,
                                     const int32_t* broadcast, int32_t group, const float* W,
-                                    const float* bias, float* y, float* y_jac, float* y_lap,
+                                    const float* bias, const float* res, const float* res_jac,
+                                    const float* res_lap, float* y, float* y_jac, float* y_lap,
                                     int64_t R, int32_t P, int32_t N, void* workspace,
                                     int64_t workspace_bytes);
 

@@ -37,7 +37,7 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
 
 
-def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0):
+def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None):
     P = jac_parts[0].shape[0]
     lead = tuple(x.shape[:-1])
     R = int(np.prod(lead))
@@ -46,7 +46,8 @@ def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=N
         Jn = _n(J).reshape(P, R // group if bc else R, w)
         Js.append(np.repeat(Jn, group, axis=1) if bc else Jn)
     J = _t(np.concatenate(Js, axis=-1).reshape(P, *lead, sum(widths)))
-    return dense_act(name, x, J, lap, W, bias, param)
+    out = dense_act(name, x, J, lap, W, bias, param)
+    return out if res is None else tuple(o + r for o, r in zip(out, res))
 
 
 def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):

@@ -460,6 +460,7 @@ def test_dot_of_lazy_concatenate(thr, monkeypatch):
         parts = [e, h, xp.broadcast_to(m, (n, 16), lazy=True), xp.broadcast_to(xp.square(m), (n, 16), lazy=True)]
         f = xp.concatenate(parts, axis=-1, lazy=True)
         a = xp.dot(f, W1, b1, act='tanh')                   # fused: four parts, two of them broadcast
+        a = xp.dot(f, W1, b1, act='tanh', residual=a)       # again, with a dense skip connection in the epilogue
         f2 = xp.concatenate([e, xp.broadcast_to(m, (n, 16), lazy=True)], axis=-1, lazy=True)
         b = xp.dot(f2, W2, act='silu')                      # narrow layer: concatenation evaluated
         f3 = xp.concatenate([e, xp.getitem(h, (slice(None), slice(0, 8)))], axis=-1, lazy=True)
@@ -467,7 +468,7 @@ def test_dot_of_lazy_concatenate(thr, monkeypatch):
         return xp.add(xp.add(xp.sum(a), xp.sum(b)), xp.sum(c))
 
     check_against_oracle(fn, x, thr)
-    assert calls == [((16, 32, 16, 16), (False, False, True, True), n)]
+    assert calls == [((16, 32, 16, 16), (False, False, True, True), n)] * 2
 
 
 def test_first_attention_layer_takes_position_sparse_path(monkeypatch):

@@ -272,6 +272,11 @@ def test_dense_act_parts(B, n, P, widths, bcast, N, act):
     for rep in range(2):
         got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b))
         assert_triplet(got, ref, f'dense_act_parts call {rep}')
+    # with a skip connection added in the epilogue
+    res = (rand(rng, B, n, N), rand(rng, P, B, n, N), rand(rng, B, n, N))
+    got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b), 0.0,
+                            tuple(dev(t) for t in res))
+    assert_triplet(got, tuple(a + r.astype(np.float64) for a, r in zip(ref, res)), 'dense_act_parts + residual')
 
 
 def test_dense_act_wide_matches_two_kernels_large():
