@@ -35,5 +35,5 @@ Pinning status (what fixes each function independently of its own formula):
   index_algebra (rest)       brute-force set enumeration on small masks
   parity unpinned            bit-level fp32 rounding of XLA's dots/reductions (the
                              reference pins nothing below rtol 2e-5 either), and the
-                             flax ``lecun_normal`` draws of BASELINE configs 1-2 (need jax)
+                             flax ``lecun_normal`` draws of the README MLP configurations (need jax)
 """

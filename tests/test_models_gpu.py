@@ -37,7 +37,7 @@ def check(fn, x, thr, what):
 
 @pytest.mark.parametrize('thr', [0, 4])
 def test_readme_mlp(thr):
-    """BASELINE configs 1 and 2 (README.md:41-70) at full model size, 3 walkers."""
+    """The reference README MLP (README.md:41-70), dense and sparse, at full model size, 3 walkers."""
     params = wl.mlp_params(seed=0)
     x = np.random.default_rng(0).normal(size=(3, 100, 4)).astype(np.float32)
     fn = lambda xp, t: wl.mlp_forward(params, t, xp)
@@ -96,7 +96,7 @@ SMALL_FERMI = wl.FermiNetConfig(n_elec=6, n_nuc=2, n_layers=3, w1=16, w2=8, n_de
 
 @pytest.mark.parametrize('thr', [0, 6])
 def test_ferminet_small_vs_oracle_and_loop_laplacian(thr):
-    """BASELINE config 3 in miniature: sparse pair stream (k = 6), dense one-electron stream."""
+    """The FermiNet-style configuration in miniature: sparse pair stream (k = 6), dense one-electron stream."""
     p = wl.ferminet_params(SMALL_FERMI)
     x = wl.sample_electrons(4, SMALL_FERMI.n_elec, 1.0, seed=3)
     fn = lambda xp, t: wl.ferminet_forward(p, t, xp)
