@@ -15,6 +15,48 @@ import numpy as np
 
 INT = np.int64
 
+# The maps below depend on the masks' contents only, and a model asks for the same ones at
+# every evaluation: results are kept by content (the reference gets the same effect from
+# tracing once under jit).  Cached arrays are shared between callers and read-only.
+_MEMO: dict = {}
+_MEMO_MAX = 4096
+
+
+def _freeze(v):
+    if isinstance(v, np.ndarray):
+        v.flags.writeable = False
+    elif isinstance(v, tuple):
+        for t in v:
+            _freeze(t)
+    return v
+
+
+def _key_of(v):
+    if isinstance(v, np.ndarray):
+        return ('a', v.shape, v.dtype.str, hash(np.ascontiguousarray(v).tobytes()))
+    if isinstance(v, (list, tuple)):
+        return tuple(_key_of(t) for t in v)
+    if isinstance(v, np.generic):
+        return v.item()
+    return v
+
+
+def _memo(fn):
+    """Keeps results of a pure function of integer arrays and plain values by content."""
+    import functools
+
+    @functools.wraps(fn)
+    def wrapped(*args):
+        key = (fn.__name__, _key_of(args))
+        hit = _MEMO.get(key)
+        if hit is None:
+            if len(_MEMO) >= _MEMO_MAX:
+                _MEMO.clear()
+            hit = _MEMO[key] = _freeze(fn(*args))
+        return hit
+
+    return wrapped
+
 
 # --------------------------------------------------------------------------------------
 # small helpers
@@ -27,6 +69,7 @@ def init_mask(shape) -> np.ndarray:
     return np.arange(n, dtype=np.int32).reshape(1, *shape)
 
 
+@_memo
 def has_duplicates(mask: np.ndarray | None) -> bool:
     """True iff a position lists a valid index twice (folx/hessian.py:71-84)."""
     if mask is None or mask.shape[0] <= 1:
@@ -147,6 +190,7 @@ def reduction_frame(masks: Sequence[np.ndarray], axes) -> np.ndarray:
     return np.moveaxis(out, -1, 0)
 
 
+@_memo
 def sum_out_mask(mask: np.ndarray, axes):
     """Index part of ``sparse_sum_jvp`` (folx/jvp.py:108-146).
 
@@ -179,6 +223,15 @@ def sum_out_mask(mask: np.ndarray, axes):
     return np.moveaxis(idx_out, -1, 0), slot
 
 
+@_memo
+def rows_distinct(mask: np.ndarray) -> bool:
+    """No two rows of the mask are the same over all positions."""
+    k = mask.shape[0]
+    flat = np.ascontiguousarray(mask).reshape(k, -1)
+    return all(not np.array_equal(flat[i], flat[j]) for i in range(k) for j in range(i))
+
+
+@_memo
 def merge_rows(masks: Sequence[np.ndarray]):
     """Row merge of a multi-operand elementwise op (folx/jvp.py:294-317): broadcast and
     concatenate the masks along the row axis, merge identical rows with

@@ -337,7 +337,7 @@ def _binary_both(op: str, a: FwdLaplArray, b: FwdLaplArray, thr: int) -> FwdLapl
     mb = np.broadcast_to(b.jacobian.x0_idx, (b.jacobian.x0_idx.shape[0], *out_shape))
     ka, kb = ma.shape[0], mb.shape[0]
     if ka == kb and np.array_equal(ma, mb) and not ia.has_duplicates(ma) and (
-        ka == 1 or np.unique(ma.reshape(ka, -1), axis=0).shape[0] == ka
+        ka == 1 or ia.rows_distinct(ma)
     ):
         # identical masks: merged rows = the rows themselves, and the intersection /
         # union frame is the mask itself, so one fused launch on k rows is the rule
