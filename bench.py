@@ -186,8 +186,10 @@ def main():
         norm = dname == 'norm_dense_fwdlap'
         roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                 'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}>'
-                          f' + the short launches of its entry point ({dname}), act={act} R={R} P={P} K={Kd} N={N}',
+                'kernel': f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}, '
+                          f'{"32, false" if norm else "16 | 32, parts"}> + the short launches of its entry point '
+                          f'({dname}: x / lap rows GEMM, finish; with LayerNorm also weight fold and per-position rows), '
+                          f'act={act} R={R} P={P} K={Kd} N={N}',
                 'launches': dn, 'avg_launch_ms': dms / dn}
     elif dname == 'dense_act_fwdlap':
         act, R, P, Kd, N = dkey
