@@ -36,6 +36,7 @@ SIGNATURES = {
     'folx_hip_mul_sparse_fwdlap': (c_int, [_P] * 11 + [c_int64, c_int64, c_int32, c_int32]),
     'folx_hip_rows_affine': (c_int, [_P, _P, _P, c_int64, c_int64, _P, _P, c_float, c_float, _P]),
     'folx_hip_reduce_sum': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_float]),
+    'folx_hip_reduce_sum_window': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_float]),
     'folx_hip_reduce_max': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64]),
     'folx_hip_gather_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64]),
     'folx_hip_gather_cols': (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int32, c_int64]),

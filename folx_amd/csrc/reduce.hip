@@ -1,5 +1,7 @@
 // Reductions over a middle axis: in [rows][outer][red][inner] -> out [rows][outer][inner].
-// The sum rule is linear, so the same kernel serves x, the Jacobian rows and lap.
+// The sum rule is linear, so the same kernel serves x, the Jacobian rows and lap.  The
+// reduced axis may be a window [lo, hi) of a longer axis (a slice that is summed right away is
+// read where it lies): `span` is the full length of that axis in memory.
 #include "common.h"
 
 namespace {
@@ -9,12 +11,13 @@ namespace {
 template <bool MAX>
 __global__ __launch_bounds__(256) void reduce_mid_kernel(const float* __restrict__ in,
                                                          float* __restrict__ out, int64_t total,
-                                                         int64_t red, int64_t inner, float alpha) {
+                                                         int64_t red, int64_t inner, int64_t span, int64_t lo,
+                                                         float alpha) {
   const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (o >= total) return;
   const int64_t ii = o % inner;
   const int64_t ro = o / inner;  // (row, outer) flattened
-  const float* src = in + ro * red * inner + ii;
+  const float* src = in + (ro * span + lo) * inner + ii;
   float acc = MAX ? -INFINITY : 0.0f;
   for (int64_t r = 0; r < red; ++r) {
     const float v = src[r * inner];
@@ -27,11 +30,11 @@ __global__ __launch_bounds__(256) void reduce_mid_kernel(const float* __restrict
 template <bool MAX>
 __global__ __launch_bounds__(256) void reduce_last_kernel(const float* __restrict__ in,
                                                           float* __restrict__ out, int64_t total,
-                                                          int64_t red, float alpha) {
+                                                          int64_t red, int64_t span, int64_t lo, float alpha) {
   const int lane = threadIdx.x % FOLX_WAVE;
   const int64_t o = (int64_t)blockIdx.x * (256 / FOLX_WAVE) + threadIdx.x / FOLX_WAVE;
   if (o >= total) return;
-  const float* src = in + o * red;
+  const float* src = in + o * span + lo;
   float acc = MAX ? -INFINITY : 0.0f;
   for (int64_t r = lane; r < red; r += FOLX_WAVE) {
     const float v = src[r];
@@ -47,19 +50,19 @@ __global__ __launch_bounds__(256) void reduce_last_kernel(const float* __restric
 
 template <bool MAX>
 int launch_reduce(hipStream_t st, const float* in, float* out, int64_t rows, int64_t outer,
-                  int64_t red, int64_t inner, float alpha) {
-  if (rows < 0 || outer < 0 || red < 0 || inner < 0) return FOLX_HIP_EINVAL;
+                  int64_t red, int64_t inner, float alpha, int64_t span, int64_t lo) {
+  if (rows < 0 || outer < 0 || red < 0 || inner < 0 || lo < 0 || lo + red > span) return FOLX_HIP_EINVAL;
   const int64_t total = rows * outer * inner;
   if (total == 0) return FOLX_HIP_OK;
   if (!in || !out) return FOLX_HIP_EINVAL;
   if (inner == 1 && red >= 16) {
     const int64_t blocks = (total + 3) / 4;
     if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-    reduce_last_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, alpha);
+    reduce_last_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, span, lo, alpha);
   } else {
     const int64_t blocks = (total + 255) / 256;
     if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-    reduce_mid_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, inner, alpha);
+    reduce_mid_kernel<MAX><<<dim3((unsigned)blocks), dim3(256), 0, st>>>(in, out, total, red, inner, span, lo, alpha);
   }
   return folx_launch_status();
 }
@@ -68,10 +71,17 @@ int launch_reduce(hipStream_t st, const float* in, float* out, int64_t rows, int
 
 extern "C" int folx_hip_reduce_sum(void* stream, const float* in, float* out, int64_t rows,
                                    int64_t outer, int64_t red, int64_t inner, float alpha) {
-  return launch_reduce<false>((hipStream_t)stream, in, out, rows, outer, red, inner, alpha);
+  return launch_reduce<false>((hipStream_t)stream, in, out, rows, outer, red, inner, alpha, red, 0);
+}
+
+extern "C" int folx_hip_reduce_sum_window(void* stream, const float* in, float* out, int64_t rows,
+                                          int64_t outer, int64_t span, int64_t lo, int64_t hi, int64_t inner,
+                                          float alpha) {
+  if (hi < lo) return FOLX_HIP_EINVAL;
+  return launch_reduce<false>((hipStream_t)stream, in, out, rows, outer, hi - lo, inner, alpha, span, lo);
 }
 
 extern "C" int folx_hip_reduce_max(void* stream, const float* in, float* out, int64_t outer,
                                    int64_t red, int64_t inner) {
-  return launch_reduce<true>((hipStream_t)stream, in, out, 1, outer, red, inner, 1.0f);
+  return launch_reduce<true>((hipStream_t)stream, in, out, 1, outer, red, inner, 1.0f, red, 0);
 }

@@ -427,14 +427,19 @@ def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta
     return out
 
 
-def reduce_sum(inp, rows, outer, red, inner, alpha=1.0):
+def reduce_sum(inp, rows, outer, red, inner, alpha=1.0, window=None):
+    """inp (rows, outer, red, inner) -> (rows, outer, inner); ``window = (lo, hi)`` sums that
+    part of the reduced axis only."""
     _chk(inp)
     out = torch.empty((rows, outer, inner), device=inp.device, dtype=torch.float32)
     with _timed('reduce_sum', (rows, outer, red, inner)):
-        check(
-            _lib.load().folx_hip_reduce_sum(_stream(), _p(inp), _p(out), rows, outer, red, inner, float(alpha)),
-            'reduce_sum',
-        )
+        if window is None:
+            rc = _lib.load().folx_hip_reduce_sum(_stream(), _p(inp), _p(out), rows, outer, red, inner, float(alpha))
+        else:
+            lo, hi = window
+            rc = _lib.load().folx_hip_reduce_sum_window(_stream(), _p(inp), _p(out), rows, outer, red, int(lo), int(hi),
+                                                        inner, float(alpha))
+        check(rc, 'reduce_sum')
     return out
 
 

@@ -210,20 +210,25 @@ def _axes(axis, nd):
     return tuple(a % nd for a in axis)
 
 
-def sum(a, axis=None, keepdims=False):
+def sum(a, axis=None, keepdims=False, window=None):
+    """``window = (lo, hi)`` with a single ``axis``: the sum of ``a[..., lo:hi, ...]`` along that
+    axis, without forming the slice."""
     shape = _shape(a)
     axes = _axes(axis, len(shape))
-    out = _call('reduce_sum', (a,), {'axes': axes})
+    if window is not None and not isinstance(a, FwdLaplArray):
+        a = getitem(a, tuple(slice(*window) if i == axes[0] else slice(None) for i in range(axes[0] + 1)))
+        window = None
+    out = _call('reduce_sum', (a,), {'axes': axes} if window is None else {'axes': axes, 'window': tuple(window)})
     if keepdims:
         out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
     return out
 
 
-def mean(a, axis=None, keepdims=False):
+def mean(a, axis=None, keepdims=False, window=None):
     shape = _shape(a)
     axes = _axes(axis, len(shape))
-    n = int(np.prod([shape[i] for i in axes], dtype=int))
-    return multiply(sum(a, axis, keepdims), 1.0 / n)
+    n = int(np.prod([shape[i] for i in axes], dtype=int)) if window is None else int(window[1] - window[0])
+    return multiply(sum(a, axis, keepdims, window), 1.0 / n)
 
 
 def amax_const(a, axis, keepdims=False):

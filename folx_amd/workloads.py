@@ -278,15 +278,16 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
     g = xp.concatenate([rij, xp.expand_dims(rn, 2)], axis=-1)  # (n, n, 4)
 
     def spin_means(t, axis_len):
-        up = xp.mean(xp.getitem(t, (slice(0, nu),)), axis=0) if nu > 0 else None
-        dn = xp.mean(xp.getitem(t, (slice(nu, n),)), axis=0) if n - nu > 0 else None
+        # means over the electrons of one spin: the slices are summed where they lie
+        up = xp.mean(t, axis=0, window=(0, nu)) if nu > 0 else None
+        dn = xp.mean(t, axis=0, window=(nu, n)) if n - nu > 0 else None
         return up, dn
 
     for li, L in enumerate(p.layers):
         hu, hd = spin_means(h, n)  # (d1,) each
         # means over the second electron of every pair: (n, d2)
-        gu = xp.mean(xp.getitem(g, (slice(None), slice(0, nu))), axis=1)
-        gd = xp.mean(xp.getitem(g, (slice(None), slice(nu, n))), axis=1)
+        gu = xp.mean(g, axis=1, window=(0, nu))
+        gd = xp.mean(g, axis=1, window=(nu, n))
         d1 = h.shape[-1]
         # the feature vector is only consumed by the product below, which reads it part by
         # part where it can: neither the broadcasts nor the concatenation are then formed

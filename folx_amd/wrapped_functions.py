@@ -818,15 +818,17 @@ def _norm_axes(axes, nd):
     return tuple(sorted(set(a % nd for a in axes)))
 
 
-def _reduce_tensor(t: torch.Tensor, lead: int, axes, alpha=1.0) -> torch.Tensor:
-    """Sum ``t`` over logical ``axes``; ``lead`` = number of leading non-logical axes."""
+def _reduce_tensor(t: torch.Tensor, lead: int, axes, alpha=1.0, window=None) -> torch.Tensor:
+    """Sum ``t`` over logical ``axes``; ``lead`` = number of leading non-logical axes.
+    ``window = (lo, hi)`` (one axis only) sums that part of the axis."""
     shape = list(t.shape)
+    assert window is None or len(axes) == 1
     for ax in sorted(axes, reverse=True):
         full_ax = ax + lead
         outer = int(np.prod(shape[:full_ax], dtype=np.int64))
         red = shape[full_ax]
         inner = int(np.prod(shape[full_ax + 1 :], dtype=np.int64))
-        t = K.reduce_sum(t.contiguous().reshape(-1), 1, outer, red, inner, alpha)
+        t = K.reduce_sum(t.contiguous().reshape(-1), 1, outer, red, inner, alpha, window)
         alpha = 1.0
         del shape[full_ax]
         t = t.reshape(shape)
@@ -847,6 +849,20 @@ def reduce_sum(args, kwargs, sparsity_threshold):
     axes = _norm_axes(kwargs.get('axes'), a.ndim)
     if len(axes) == 0:
         return a
+    window = kwargs.get('window')
+    if window is not None:
+        # the sum of a slice along the reduced axis: read in place for dense Jacobians,
+        # otherwise the slice rule followed by the plain sum
+        assert len(axes) == 1
+        lo, hi = (int(v) for v in window)
+        assert 0 <= lo <= hi <= a.shape[axes[0]]
+        if a.jacobian.x0_idx is not None:
+            idx = tuple(slice(lo, hi) if i == axes[0] else slice(None) for i in range(axes[0] + 1))
+            part = getitem_rule((a,), {'idx': idx}, sparsity_threshold)
+            return reduce_sum((part,), {'axes': kwargs.get('axes')}, sparsity_threshold)
+        return FwdLaplArray(_reduce_tensor(a.x, 1, axes, 1.0, (lo, hi)),
+                            FwdJacobian(_reduce_tensor(a.jacobian.data, 2, axes, 1.0, (lo, hi)), None),
+                            _reduce_tensor(a.laplacian, 1, axes, 1.0, (lo, hi)))
     x = _reduce_tensor(a.x, 1, axes)
     lap = _reduce_tensor(a.laplacian, 1, axes)
     J, mask = a.jacobian.data, a.jacobian.x0_idx

@@ -279,6 +279,16 @@ int folx_hip_rows_affine(void* stream, const float* in, float* out, int64_t rows
 int folx_hip_reduce_sum(void* stream, const float* in, float* out, int64_t rows,
                         int64_t outer, int64_t red, int64_t inner, float alpha);
 
+/*
+ * The same sum over a window [lo, hi) of the middle axis, read where it lies:
+ * in [rows][outer][span][inner] -> out [rows][outer][inner] = alpha * sum_{lo <= r < hi}.
+ * A slice (slice_p, folx/wrapped_functions.py:446-466) whose only consumer is reduce_sum_p:
+ * spin-wise means over the electron axis.
+ */
+int folx_hip_reduce_sum_window(void* stream, const float* in, float* out, int64_t rows,
+                               int64_t outer, int64_t span, int64_t lo, int64_t hi,
+                               int64_t inner, float alpha);
+
 /* max over the middle axis of a value array (no derivatives): [outer][red][inner] ->
  * [outer][inner].  Used for the stop-gradient shift of logsumexp. */
 int folx_hip_reduce_max(void* stream, const float* in, float* out, int64_t outer,

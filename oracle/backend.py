@@ -400,17 +400,21 @@ def layer_norm(h: OArr, gamma=None, beta=None, eps=1e-5, lazy=False):
     return y if beta is None else add(y, beta)
 
 
-def sum(a: OArr, axis=None, keepdims=False):
+def sum(a: OArr, axis=None, keepdims=False, window=None):
+    """``window = (lo, hi)``: the sum of the slice ``lo:hi`` along the (single) axis."""
     if axis is None:
         axis = tuple(range(a.ndim))
+    if window is not None:
+        ax = int(np.atleast_1d(axis)[0]) % a.ndim
+        a = getitem(a, tuple(slice(*window) if i == ax else slice(None) for i in range(ax + 1)))
     return OArr(*rules.sum_rule(a.x, a.J, a.lap, axis, keepdims))
 
 
-def mean(a: OArr, axis=None, keepdims=False):
+def mean(a: OArr, axis=None, keepdims=False, window=None):
     if axis is None:
         axis = tuple(range(a.ndim))
-    n = int(np.prod([a.shape[i] for i in np.atleast_1d(axis)]))
-    return multiply(sum(a, axis, keepdims), 1.0 / n)
+    n = int(np.prod([a.shape[i] for i in np.atleast_1d(axis)])) if window is None else int(window[1] - window[0])
+    return multiply(sum(a, axis, keepdims, window), 1.0 / n)
 
 
 def reshape(a: OArr, shape):

@@ -112,15 +112,19 @@ class plain:
         return a / b
 
     @staticmethod
-    def sum(a, axis=None, keepdims=False):
+    def sum(a, axis=None, keepdims=False, window=None):
         if axis is None:
             return a.sum()
+        if window is not None:
+            a = a.narrow(axis, window[0], window[1] - window[0])
         return a.sum(dim=axis, keepdim=keepdims)
 
     @staticmethod
-    def mean(a, axis=None, keepdims=False):
+    def mean(a, axis=None, keepdims=False, window=None):
         if axis is None:
             return a.mean()
+        if window is not None:
+            a = a.narrow(axis, window[0], window[1] - window[0])
         return a.mean(dim=axis, keepdim=keepdims)
 
     @staticmethod

@@ -117,8 +117,11 @@ def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta
     return _t(np.broadcast_to(out, (rows, *out_shape)))
 
 
-def reduce_sum(inp, rows, outer, red, inner, alpha=1.0):
-    return _t(alpha * _n(inp).reshape(rows, outer, red, inner).sum(2))
+def reduce_sum(inp, rows, outer, red, inner, alpha=1.0, window=None):
+    v = _n(inp).reshape(rows, outer, red, inner)
+    if window is not None:
+        v = v[:, :, window[0]:window[1]]
+    return _t(alpha * v.sum(2))
 
 
 def reduce_max(inp, outer, red, inner):

@@ -81,6 +81,8 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_dense_act_workspace_bytes(63, 33, 256, 256) == _lib.ENOTSUP         # wide: rows % 4
     assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 200, 256) == _lib.ENOTSUP         # wide: K % 16
     assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 64, 33, 256, 256, None, 0) == _lib.EINVAL  # no workspace
+    assert lib.folx_hip_reduce_sum_window(None, one, one, 2, 3, 8, 5, 9, 4, 1.0) == _lib.EINVAL   # window past the axis
+    assert lib.folx_hip_reduce_sum_window(None, one, one, 2, 3, 8, 5, 4, 4, 1.0) == _lib.EINVAL   # hi < lo
     # Jacobian operand in parts: host arrays of pointers, widths and broadcast flags
     ptrs, wd, bc = (ctypes.c_void_p * 2)(16, 32), (ctypes.c_int32 * 2)(16, 32), (ctypes.c_int32 * 2)(0, 1)
     parts = lambda wd_, R, group, ws, nb: lib.folx_hip_dense_act_parts_fwdlap(

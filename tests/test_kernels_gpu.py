@@ -387,6 +387,10 @@ def test_reduce(outer, red, inner):
     assert_val(got, 0.25 * inp.astype(np.float64).sum(2))
     got = K.reduce_max(dev(inp[0]), outer, red, inner)
     assert_val(got, inp[0].max(1))
+    # a window of the reduced axis, read in place (empty, inner, trailing, whole)
+    for lo, hi in ((0, 0), (1, max(1, red - 1)), (red // 2, red), (0, red)):
+        got = K.reduce_sum(dev(inp), rows, outer, red, inner, alpha=2.0, window=(lo, hi))
+        assert_val(got, 2.0 * inp.astype(np.float64)[:, :, lo:hi].sum(2))
 
 
 def test_gather_and_scatter_rows():
