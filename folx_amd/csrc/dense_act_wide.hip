@@ -190,17 +190,13 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
                                        FOLX_LPTR(&ws[(wave * 64 + NT * i) * 4]), 16, 0, 0);
   };
 
-  // The first chunk is on its way while what the epilogue needs per position and column is
-  // staged in LDS: both are waited for together in front of the first barrier.
-  issue(0, As0, Ws0);
-  float zr[TM][TN][PB];  // without LayerNorm there are registers to spare for them
-  if constexpr (NORM) {
-    for (int e = tid; e < RT * BN; e += NT) {
-      int gc = col0 + e % BN;
-      if (gc >= N) gc = N - 1;
-      zS[e] = a.z[(r0 + e / BN) * N + gc];
-    }
-  } else {
+  // Without LayerNorm the epilogue only needs f'(z) of this lane's columns at its blocks'
+  // positions, and there are registers to spare for it: z is asked for first, then the first
+  // chunk, and f' is evaluated while the chunk is on its way.  With LayerNorm what the
+  // epilogue needs per position and column is staged in LDS behind the first chunk, and both
+  // are waited for together in front of the first barrier.
+  float dr[TM][TN][PB];
+  if constexpr (!NORM) {
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -208,8 +204,27 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
         int gc = col0 + wc + j * 32 + l32;
         if (gc >= N) gc = N - 1;
 #pragma unroll
-        for (int b = 0; b < PB; ++b) zr[i][j][b] = a.z[(r0 + (wrow * TM + i) * PB + b) * N + gc];
+        for (int b = 0; b < PB; ++b) dr[i][j][b] = a.z[(r0 + (wrow * TM + i) * PB + b) * N + gc];
       }
+  }
+  issue(0, As0, Ws0);
+  if constexpr (NORM) {
+    for (int e = tid; e < RT * BN; e += NT) {
+      int gc = col0 + e % BN;
+      if (gc >= N) gc = N - 1;
+      zS[e] = a.z[(r0 + e / BN) * N + gc];
+    }
+  } else if constexpr (ACT) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int b = 0; b < PB; ++b) {
+          float f, d1, d2;
+          act_eval_fused(a.act, dr[i][j][b], a.prm, f, d1, d2);
+          dr[i][j][b] = d1;
+        }
   }
   if constexpr (NORM) {
     // xh of the tile's RT positions: RT * K consecutive floats
@@ -337,12 +352,16 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
       float zv[PB], d1[PB];
 #pragma unroll
       for (int b = 0; b < PB; ++b) {
-        if constexpr (NORM) zv[b] = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
-        else zv[b] = zr[i][j][b];
+        zv[b] = 0.0f;
         d1[b] = 1.0f;
-        if constexpr (ACT) {
-          float f, d2;
-          act_eval_fused(a.act, zv[b], a.prm, f, d1[b], d2);
+        if constexpr (NORM) {
+          zv[b] = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
+          if constexpr (ACT) {
+            float f, d2;
+            act_eval_fused(a.act, zv[b], a.prm, f, d1[b], d2);
+          }
+        } else if constexpr (ACT) {
+          d1[b] = dr[i][j][b];
         }
       }
       float w1c = 0.0f, w2c = 0.0f;
