@@ -121,7 +121,21 @@ def test_psiformer_full_architecture_two_walkers(name):
     x = wl.sample_electrons(2, cfg.n_elec, sigma, seed=2)
     fn = lambda xp, t: forward(p, t, xp)
     print(f'case {name} full architecture', flush=True)
-    out = run(fn, x, thr)
+    from folx_amd import kernels as K
+
+    with K.LaunchTimer() as lt:
+        out = run(fn, x, thr)
+    used = {}
+    for (entry, key), (calls, _) in lt.summary().items():
+        used[entry] = used.get(entry, 0) + calls
+    if name.startswith('psiformer'):
+        # the fused rules are the ones that run: LayerNorm inside 3 products of layers 2-4 and the
+        # 4 MLP products; the only stand-alone LayerNorm is the first layer's (sparse rows), once
+        assert used.get('norm_dense_fwdlap', 0) == 3 * 3 + 4, used
+        assert used.get('layernorm_fwdlap', 0) == 1, used
+    else:
+        # one-electron layers 2-4 read their concatenated input in parts, activation in the epilogue
+        assert used.get('dense_act_fwdlap', 0) >= 3, used
     r64 = fn(ob, ob.init_state(x, dtype=np.float64))
     r32 = fn(ob, ob.init_state(x, dtype=np.float32))
     J = out.jacobian.dense_array.cpu().numpy().astype(np.float64)
