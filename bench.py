@@ -40,8 +40,8 @@ MEASURED_TRAFFIC_BYTES = {
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=5)
-    ap.add_argument('--warmup', type=int, default=2)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='psiformer32')
     ap.add_argument('--walkers', type=int, default=0, help='override the batch (0 = the configuration default)')
     ap.add_argument('--chunk', type=int, default=1024, help='walkers per batched_vmap chunk')
