@@ -19,7 +19,7 @@ INT = np.int64
 # every evaluation: results are kept by content (the reference gets the same effect from
 # tracing once under jit).  Cached arrays are shared between callers and read-only.
 _MEMO: dict = {}
-_MEMO_MAX = 4096
+_MEMO_MAX = 1024
 
 
 def _freeze(v):
@@ -33,7 +33,7 @@ def _freeze(v):
 
 def _key_of(v):
     if isinstance(v, np.ndarray):
-        return ('a', v.shape, v.dtype.str, hash(np.ascontiguousarray(v).tobytes()))
+        return ('a', v.shape, v.dtype.str, np.ascontiguousarray(v).tobytes())  # exact: the contents are the key
     if isinstance(v, (list, tuple)):
         return tuple(_key_of(t) for t in v)
     if isinstance(v, np.generic):
