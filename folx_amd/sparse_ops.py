@@ -51,8 +51,11 @@ def device_const(arr, device) -> torch.Tensor:
 
 
 def clear_caches():
+    from . import index_algebra
+
     _TABLE_CACHE.clear()
     _CONST_CACHE.clear()
+    index_algebra._MEMO.clear()
 
 
 def zeros(shape, device) -> torch.Tensor:
