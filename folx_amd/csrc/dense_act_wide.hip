@@ -35,6 +35,11 @@
 //     (R, N) slab per group of 32 Jacobian rows;
 //  4. a short elementwise kernel that finishes y and y_lap, adding the slabs in a fixed order.
 //
+// Variant (a) also reads a CONCATENATED operand part by part (a chunk of 16 features lies in
+// exactly one part; a part may hold one row per walker that all of the walker's positions
+// share) and adds a skip connection in its epilogue, so that a layer fed by
+// [own features, per-walker means, ...] forms neither the broadcasts nor the concatenation.
+//
 // The main loop is the one of the dense kernel: K in chunks of 16 through double-buffered LDS
 // tiles filled by global_load_lds_dwordx4, a 128 x 256 tile on 8 wavefronts of 64 x 64,
 // v_mfma_f32_32x32x2_f32 with the k order inside a group of 8 permuted to fit 128-bit reads
