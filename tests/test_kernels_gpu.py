@@ -279,6 +279,72 @@ def test_dense_act_parts(B, n, P, widths, bcast, N, act):
     assert_triplet(got, tuple(a + r.astype(np.float64) for a, r in zip(ref, res)), 'dense_act_parts + residual')
 
 
+def test_norm_dense_full_chunk_properties():
+    """At the benchmark's chunk size (32768 positions, 96 Jacobian rows): the fused rule is
+    linear in the Jacobian rows up to its quadratic lap term, so doubling them doubles y_jac bit
+    for bit (a power of two) and leaves y alone; and every position is computed from its own
+    data in a fixed order, so reversing the positions reverses the results bit for bit."""
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(11)
+    R, P, Kd, N = 1024 * 32, 96, 256, 256
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.randn(R, Kd, device='cuda', generator=g)
+    gam = 1 + 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    bet = 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    W = torch.randn(Kd, N, device='cuda', generator=g) / 16
+    b = torch.randn(N, device='cuda', generator=g)
+    print('case norm_dense full chunk', flush=True)
+    y, yj, yl = K.norm_dense('tanh', x, J, L, gam, bet, 1e-5, W, b)
+    assert torch.isfinite(yj).all() and torch.isfinite(yl).all()
+    J.mul_(2.0)
+    y2, yj2, yl2 = K.norm_dense('tanh', x, J, L, gam, bet, 1e-5, W, b)
+    assert torch.equal(y2, y)
+    yj.mul_(2.0)
+    assert torch.equal(yj2, yj)
+    del yj
+    # positions reversed (J is the doubled one)
+    xr, Lr = x.flip(0).contiguous(), L.flip(0).contiguous()
+    J = J.flip(1).contiguous()
+    y3, yj3, yl3 = K.norm_dense('tanh', xr, J, Lr, gam, bet, 1e-5, W, b)
+    assert torch.equal(y3, y2.flip(0)) and torch.equal(yl3, yl2.flip(0))
+    assert torch.equal(yj3, yj2.flip(1))
+
+
+def test_dense_act_parts_full_chunk_equals_concatenated():
+    """At the FermiNet-style chunk size (1024 walkers x 16 electrons, 48 Jacobian rows, 832
+    features in five parts, two of them per-walker): reading the operand in parts does the
+    same arithmetic in the same order as reading the concatenated array, so the results are
+    equal bit for bit."""
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(12)
+    B, n, P, N = 1024, 16, 48, 256
+    widths, bcast = (256, 256, 256, 32, 32), (0, 1, 1, 0, 0)
+    xs, ls, Js, Jd = [], [], [], []
+    for w, bc in zip(widths, bcast):
+        lead = (B,) if bc else (B, n)
+        xp_ = torch.randn(*lead, w, device='cuda', generator=g)
+        lp_ = torch.randn(*lead, w, device='cuda', generator=g)
+        Jp = torch.randn(P, *lead, w, device='cuda', generator=g)
+        Js.append(Jp)
+        ex = (lambda t: t.unsqueeze(-2).expand(*t.shape[:-1], n, w)) if bc else (lambda t: t)
+        xs.append(ex(xp_)), ls.append(ex(lp_)), Jd.append(ex(Jp))
+    x, L, J = torch.cat(xs, -1), torch.cat(ls, -1), torch.cat(Jd, -1)
+    W = torch.randn(sum(widths), N, device='cuda', generator=g) / 29
+    b = torch.randn(N, device='cuda', generator=g)
+    print('case dense_act_parts full chunk', flush=True)
+    ref = K.dense_act('tanh', x, J, L, W, b)
+    got = K.dense_act_parts('tanh', x, L, Js, widths, bcast, n, W, b)
+    for a, r in zip(got, ref):
+        assert torch.equal(a, r)
+    res = tuple(torch.randn_like(t) for t in ref)
+    got = K.dense_act_parts('tanh', x, L, Js, widths, bcast, n, W, b, 0.0, res)
+    for a, r, s_ in zip(got, ref, res):
+        torch.testing.assert_close(a, r + s_, rtol=2e-6, atol=2e-6)  # the epilogue adds with one rounding (fma)
+
+
 def test_dense_act_wide_matches_two_kernels_large():
     """A transformer MLP layer at a full chunk: the fused wide path and dense + elementwise
     agree to rounding (the sums over Jacobian rows are taken in a different order)."""
