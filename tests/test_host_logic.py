@@ -471,6 +471,31 @@ def test_dot_of_lazy_concatenate(thr, monkeypatch):
     assert calls == [((16, 32, 16, 16), (False, False, True, True), n)] * 2
 
 
+@pytest.mark.parametrize('thr', [0, 6])
+def test_readme_fused_layer_forms(thr):
+    """The layer forms the README shows (activation and skip connection in the product, lazy
+    layer_norm, lazy concatenation with a windowed mean broadcast among its parts)."""
+    rng = np.random.default_rng(15)
+    n, n_up, d = 8, 3, 16
+    W0 = rng.normal(size=(3, d)).astype(np.float32)
+    W, b = rng.normal(size=(d, d)).astype(np.float32) / 4, rng.normal(size=(d,)).astype(np.float32)
+    gamma, beta = (1 + 0.1 * rng.normal(size=d)).astype(np.float32), (0.1 * rng.normal(size=d)).astype(np.float32)
+    Wq, Wk = (rng.normal(size=(d, d)).astype(np.float32) / 4 for _ in range(2))
+    V, c = rng.normal(size=(2 * d, d)).astype(np.float32) / 5, rng.normal(size=(d,)).astype(np.float32)
+    x0 = rng.normal(size=(2, n, 3)).astype(np.float32)
+
+    def fn(xp, t):
+        x = xp.dot(t, W0)
+        h = xp.dot(x, W, b, act='tanh', residual=x)
+        hn = xp.layer_norm(h, gamma, beta, 1e-5, lazy=True)
+        q, k = xp.dot(hn, Wq), xp.dot(hn, Wk)
+        f = xp.concatenate([h, xp.broadcast_to(xp.mean(h, axis=0, window=(0, n_up)), h.shape, lazy=True)], lazy=True)
+        h = xp.dot(f, V, c, act='tanh', residual=h)
+        return xp.add(xp.sum(xp.multiply(q, k)), xp.sum(h))
+
+    check_against_oracle(fn, x0, thr)
+
+
 def test_first_attention_layer_takes_position_sparse_path(monkeypatch):
     """q, k, v of the first PsiFormer layer still carry per-electron sparse Jacobians: the rule
     hands them to the position-sparse kernel and the result equals the densified rule."""
