@@ -5,11 +5,13 @@
 //      sign and log|det| (the same pivot sequence as an LU with partial pivoting).
 //   2. tr(A^-1 lap_A) by a lane-strided product.
 //   (The matrices may be strided: a stack [batch][row][member][column] is read in place.)
-//   3. For every Jacobian row p: stage A_jac[p] in LDS (the next row is prefetched into
-//      registers meanwhile), M = A^-1 A_jac[p] with lane (i, column group) holding row i
-//      of A^-1 in registers, ld_jac[p] = tr M, and sum_p tr(M M) through an LDS transpose.
-// The Jacobian is read exactly once, so the kernel is bound by HBM bandwidth as long as
-// the 2 n^3 flops per row stay hidden (they do for n <= 32 on the vector ALUs).
+//   3. For every Jacobian row p: A_jac[p] goes from global memory straight into MFMA
+//      operand registers (the next row is prefetched meanwhile), M = A^-1 A_jac[p] and its
+//      transpose are two MFMA products of the same registers (operands swapped),
+//      sum_p tr(M M) is the elementwise product of the two accumulators, ld_jac[p] = tr M
+//      the lane-wise product of the operands, reduced over the wavefront 16 rows at a time
+//      through LDS.
+// The Jacobian is read exactly once; 4 n^3 flops per row on the matrix cores.
 #include "smallmat.h"
 
 namespace {
@@ -29,6 +31,38 @@ struct Factor {
 };
 constexpr int KF = 4;
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// One MFMA tile covers the matrix: 16 x 16 (v_mfma_f32_16x16x4_f32) for n <= 16, 32 x 32
+// (v_mfma_f32_32x32x2_f32) above.  Lane l holds, for step t, the element (k = KS t + l / MP,
+// lr = l % MP) of an operand: as A operand that is row lr, column k; as B operand row k,
+// column lr.  With a[t] = Ainv[lr][k] and j[t] = J[k][lr]:
+//   mfma(a, j) accumulates M   = Ainv J      (A = Ainv,  B = J)
+//   mfma(j, a) accumulates M^T = J^T Ainv^T  (A = J^T,   B = Ainv^T) -- the SAME registers,
+// so the transpose that tr(M M) = sum_ab M[a][b] M^T[a][b] needs costs a second product and
+// no data movement, and tr M = sum over lanes and steps of a[t] j[t].
+template <int MP>
+struct Tile;
+template <>
+struct Tile<16> {
+  static constexpr int KS = 4, STEPS = 4, CR = 4;
+  typedef floatx4 acc_t;
+  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Tile<32> {
+  static constexpr int KS = 2, STEPS = 16, CR = 16;
+  typedef floatx16 acc_t;
+  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
+
 template <int NP, bool HAS_F>
 __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
@@ -36,13 +70,11 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
     int64_t rstride, int64_t slice, int32_t share, Factor fc) {
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
-  constexpr int G = FOLX_WAVE / NP;    // lane groups per row
-  constexpr int CPL = NP / G;          // columns of M per lane
-  constexpr int MS = NP + 1;           // row stride of the M staging tile
-  constexpr int EPL = NP * NP / FOLX_WAVE;  // Jacobian elements prefetched per lane
+  constexpr int MP = NP <= 16 ? 16 : 32;
+  typedef Tile<MP> T;
+  constexpr int STEPS = T::STEPS;  // = elements of the padded MP x MP tile per lane
   __shared__ float aug[NP * AUGS];
-  __shared__ __attribute__((aligned(16))) float jb[2][NP * NP];
-  __shared__ float mb[NP * MS];
+  __shared__ float trs[TRB][FOLX_WAVE + 1];
 
   const int lane = threadIdx.x;
   // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  When `share`
@@ -62,109 +94,106 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn, rstride, HAS_F ? fc.x + base : nullptr);
   float tl = HAS_F ? 0.0f : smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
 
-  // ---- row i of A^-1 in registers -------------------------------------------------------
-  const int i = lane % NP;
-  const int g = lane / NP;
-  const int col0 = g * CPL;
-  float ainv[NP];
+  // this lane's elements (k, lr) of the padded tile: A^-1 transposed-in-place as the MFMA
+  // operand, and with a factor also F, A and the factor's sparse Jacobian rows at them
+  const int lr = lane % MP;
+  const int lq = lane / MP;
+  float ainv[STEPS];
+  bool ok[STEPS];
+  int64_t eoff[STEPS];
 #pragma unroll
-  for (int j = 0; j < NP; ++j) ainv[j] = aug[i * AUGS + NP + j];
-
-  // this lane's EPL elements of the padded tile; with a factor also its values at them
-  constexpr int EF = HAS_F ? EPL : 1;
+  for (int t = 0; t < STEPS; ++t) {
+    const int k = T::KS * t + lq;
+    ok[t] = k < n && lr < n;
+    eoff[t] = (int64_t)k * rstride + lr;
+    ainv[t] = ok[t] ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
+  }
+  constexpr int EF = HAS_F ? STEPS : 1;
   float fx[EF], ax[EF], lapx[EF], fj[KF][EF];
   int32_t fidx[KF][EF];
   if constexpr (HAS_F) {
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) {
-      const int e = lane + c * FOLX_WAVE;
-      const int r = e / NP, cc = e % NP;
-      const bool ok = r < n && cc < n;
-      const int64_t off = base + r * rstride + cc;
-      fx[c] = ok ? fc.x[off] : 0.0f;
-      ax[c] = ok ? A[off] : 0.0f;
-      lapx[c] = 0.0f;
+    for (int t = 0; t < STEPS; ++t) {
+      const int64_t off = base + eoff[t];
+      fx[t] = ok[t] ? fc.x[off] : 0.0f;
+      ax[t] = ok[t] ? A[off] : 0.0f;
+      lapx[t] = 0.0f;
 #pragma unroll
       for (int sl = 0; sl < KF; ++sl) {
-        fidx[sl][c] = (ok && sl < fc.kf) ? fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w] : -1;
-        fj[sl][c] = fidx[sl][c] >= 0 ? fc.jac[(int64_t)sl * slice + off] : 0.0f;
+        fidx[sl][t] = (ok[t] && sl < fc.kf) ? fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w] : -1;
+        fj[sl][t] = fidx[sl][t] >= 0 ? fc.jac[(int64_t)sl * slice + off] : 0.0f;
       }
     }
   }
 
+  // Jacobian rows are requested D rows ahead: with one row in flight per wavefront the kernel
+  // would be bound by the latency of its own loads, not by HBM bandwidth.
+  constexpr int D = MP == 16 ? 4 : 1;
   float mm = 0.0f;
-  float pre[EPL];
-  auto prefetch = [&](int p) {
+  float raw[D][STEPS];
+  auto request = [&](float (&dst)[STEPS], int p) __attribute__((always_inline)) {
     const float* src = AJ + (int64_t)p * slice + base;
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) {
-      const int e = lane + c * FOLX_WAVE;  // index into the padded NP x NP tile
-      const int r = e / NP, cc = e % NP;
-      float v = (r < n && cc < n) ? src[r * rstride + cc] : 0.0f;
-      if constexpr (HAS_F) {
-        float add = 0.0f;
-#pragma unroll
-        for (int sl = 0; sl < KF; ++sl)
-          if (fidx[sl][c] == p) { add += fj[sl][c]; lapx[c] += 2.0f * v * fj[sl][c]; }
-        v = fx[c] * v + ax[c] * add;
-      }
-      pre[c] = v;
-    }
+    for (int t = 0; t < STEPS; ++t) dst[t] = ok[t] ? src[eoff[t]] : 0.0f;  // A_jac[p][k][lr]
   };
-  if (P > 0) prefetch(0);
-  for (int p = 0; p < P; ++p) {
-    float* J = jb[p & 1];
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) J[lane + c * FOLX_WAVE] = pre[c];
-    __syncthreads();
-    if (p + 1 < P) prefetch(p + 1);
-
-    // trace of M without forming it: sum_{j,i} Ainv[i][j] J[j][i]
-    float tr = 0.0f;
+  for (int d = 0; d < D; ++d)
+    if (d < P) request(raw[d], d);
+  for (int p0 = 0; p0 < P; p0 += D) {
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) {
-      const int e = lane + c * FOLX_WAVE;
-      const int j = e / NP, ii = e % NP;
-      tr += aug[ii * AUGS + NP + j] * J[e];
-    }
-    tr = wave_sum(tr);
-    if (lane == 0) jac_out[(int64_t)p * NM + m] = tr;
-
-    // M[i][col0 .. col0 + CPL)
-    float acc[CPL];
+    for (int d = 0; d < D; ++d) {
+      const int p = p0 + d;
+      if (p < P) {
+        float jv[STEPS];
 #pragma unroll
-    for (int c = 0; c < CPL; ++c) acc[c] = 0.0f;
+        for (int t = 0; t < STEPS; ++t) {
+          float v = raw[d][t];
+          if constexpr (HAS_F) {
+            float add = 0.0f;
 #pragma unroll
-    for (int j = 0; j < NP; ++j) {
-      if constexpr (CPL % 4 == 0) {
-#pragma unroll
-        for (int c = 0; c < CPL; c += 4) {
-          const float4 v = *reinterpret_cast<const float4*>(&J[j * NP + col0 + c]);
-          acc[c + 0] += ainv[j] * v.x; acc[c + 1] += ainv[j] * v.y;
-          acc[c + 2] += ainv[j] * v.z; acc[c + 3] += ainv[j] * v.w;
+            for (int sl = 0; sl < KF; ++sl)
+              if (fidx[sl][t] == p) { add += fj[sl][t]; lapx[t] += 2.0f * v * fj[sl][t]; }
+            v = fx[t] * v + ax[t] * add;
+          }
+          jv[t] = v;
         }
-      } else {
+        if (p + D < P) request(raw[d], p + D);
+        typename T::acc_t c, ct;
 #pragma unroll
-        for (int c = 0; c < CPL; ++c) acc[c] += ainv[j] * J[j * NP + col0 + c];
+        for (int r = 0; r < T::CR; ++r) { c[r] = 0.0f; ct[r] = 0.0f; }
+        float tr = 0.0f;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+          c = T::mfma(ainv[t], jv[t], c);    // M   = Ainv J
+          ct = T::mfma(jv[t], ainv[t], ct);  // M^T
+          tr = fmaf(ainv[t], jv[t], tr);     // this lane's part of tr M
+        }
+#pragma unroll
+        for (int r = 0; r < T::CR; ++r) mm = fmaf(c[r], ct[r], mm);
+        trs[p % TRB][lane] = tr;
+        if ((p + 1) % TRB == 0 || p + 1 == P) {
+          // ld_jac of the last rows: four lanes per row add up 16 of its 64 parts each
+          const int pb = p / TRB * TRB, pe = p + 1 - pb;
+          __syncthreads();
+          const int row = lane % TRB, part = lane / TRB;
+          float sm = 0.0f;
+#pragma unroll
+          for (int l = 0; l < FOLX_WAVE / 4; ++l) sm += trs[row][part * (FOLX_WAVE / 4) + l];
+          sm += __shfl_xor(sm, 16, FOLX_WAVE);
+          sm += __shfl_xor(sm, 32, FOLX_WAVE);
+          if (part == 0 && row < pe) jac_out[(int64_t)(pb + row) * NM + m] = sm;
+          __syncthreads();
+        }
       }
     }
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) mb[i * MS + col0 + c] = acc[c];
-    __syncthreads();
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) mm += acc[c] * mb[(col0 + c) * MS + i];
-    // the next iteration writes the other jb buffer; mb is rewritten only after the
-    // barrier that follows that write, when every lane is past this read
   }
   if constexpr (HAS_F) {
 #pragma unroll
-    for (int c = 0; c < EPL; ++c) {
-      const int e = lane + c * FOLX_WAVE;
-      const int r = e / NP, cc = e % NP;
-      if (r < n && cc < n) {
-        const int64_t off = base + r * rstride + cc;
-        const float al = fx[c] * AL[off] + ax[c] * fc.lap[off] + lapx[c];
-        tl += aug[cc * AUGS + NP + r] * al;  // tr(A^-1 lap A) = sum A^-1[c][r] lap A[r][c]
+    for (int t = 0; t < STEPS; ++t) {
+      if (ok[t]) {
+        const int64_t off = base + eoff[t];
+        const float al = fx[t] * AL[off] + ax[t] * fc.lap[off] + lapx[t];
+        tl += ainv[t] * al;  // tr(A^-1 lap A) = sum A^-1[lr][k] lap A[k][lr]
       }
     }
   }
