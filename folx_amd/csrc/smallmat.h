@@ -19,77 +19,75 @@ struct Aug {
 };
 
 // Gauss-Jordan with partial pivoting on [A | I]; afterwards aug[i * stride + NP + j] is
-// A^-1[i][j].  The pivots give sign and log|det| (the pivot sequence is the one of an LU
-// with partial pivoting, first maximum wins as in idamax).  Padding rows/columns carry a
-// unit diagonal, so the elimination leaves them alone.  Called by all 64 lanes of the one
-// wavefront of the workgroup.
+// A^-1[i][j] (the left half of aug is not written).  The pivots give sign and log|det| (the
+// pivot sequence is the one of an LU with partial pivoting, first maximum wins as in idamax).
+// Padding rows/columns carry a unit diagonal, so the elimination leaves them alone.  Called
+// by all 64 lanes of the one wavefront of the workgroup.
+//
+// The elimination runs in registers: lane j < 2 NP holds column j of [A | I], one register per
+// row.  A pivot step reads column k into wave-uniform values (v_readlane, the lane index is a
+// compile-time constant because the loop over k is unrolled), picks the pivot among them,
+// swaps the two rows in every lane's registers and updates each column with NP multiply-adds:
+// no LDS round trip and no barrier inside the chain of NP dependent steps.
 template <int NP>
 __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict__ a, int n, int lane,
                                              float& logdet, float& sgn, int64_t row_stride = 0,
                                              const float* __restrict__ factor = nullptr) {
+  static_assert(2 * NP <= FOLX_WAVE, "one lane per column of [A | I]");
   if (row_stride == 0) row_stride = n;  // rows of the matrix follow each other
   constexpr int AUGS = Aug<NP>::stride;
-  constexpr int RK = (2 * NP + FOLX_WAVE - 1) / FOLX_WAVE;
-  for (int e = lane; e < NP * 2 * NP; e += FOLX_WAVE) {
-    const int i = e / (2 * NP), j = e % (2 * NP);
+  float col[NP];
+#pragma unroll
+  for (int r = 0; r < NP; ++r) {
     float v;
     // with `factor` (same layout as a) the matrix is the elementwise product a * factor
-    if (j < NP) v = (i < n && j < n) ? a[i * row_stride + j] * (factor ? factor[i * row_stride + j] : 1.0f)
-                                     : (i == j ? 1.0f : 0.0f);
-    else v = (j - NP == i) ? 1.0f : 0.0f;
-    aug[i * AUGS + j] = v;
+    if (lane < NP) v = (r < n && lane < n) ? a[r * row_stride + lane] * (factor ? factor[r * row_stride + lane] : 1.0f)
+                                           : (r == lane ? 1.0f : 0.0f);
+    else v = (lane - NP == r) ? 1.0f : 0.0f;
+    col[r] = v;
   }
-  __syncthreads();
-
   logdet = 0.0f;
   sgn = 1.0f;
-  for (int k = 0; k < n; ++k) {
-    float best = -1.0f;
-    int bi = k;
-    if (lane >= k && lane < n) { best = fabsf(aug[lane * AUGS + k]); bi = lane; }
 #pragma unroll
-    for (int off = FOLX_WAVE / 2; off > 0; off >>= 1) {
-      const float ob = __shfl_xor(best, off, FOLX_WAVE);
-      const int oi = __shfl_xor(bi, off, FOLX_WAVE);
-      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
-    }
-    if (bi != k) {
-      for (int j = lane; j < 2 * NP; j += FOLX_WAVE) {
-        const float t = aug[k * AUGS + j];
-        aug[k * AUGS + j] = aug[bi * AUGS + j];
-        aug[bi * AUGS + j] = t;
-      }
-      sgn = -sgn;
-      __syncthreads();
-    }
-    const float pv = aug[k * AUGS + k];
-    logdet += logf(fabsf(pv));
-    if (pv < 0.0f) sgn = -sgn;
-    if (pv == 0.0f) sgn = 0.0f;
-    const float rp = 1.0f / pv;
-    __syncthreads();
-    float rowk[RK];
+  for (int k = 0; k < NP; ++k) {
+    if (k < n) {
+      float ck[NP];  // column k, the same in every lane
 #pragma unroll
-    for (int c = 0; c < RK; ++c) {
-      const int j = lane + c * FOLX_WAVE;
-      if (j < 2 * NP) {
-        rowk[c] = aug[k * AUGS + j] * rp;
-        aug[k * AUGS + j] = rowk[c];
-      }
-    }
-    __syncthreads();
-    for (int i = 0; i < n; ++i) {
-      if (i == k) continue;
-      const float f = aug[i * AUGS + k];
-      __syncthreads();  // everyone has read f before column k of row i is overwritten
+      for (int r = 0; r < NP; ++r) ck[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(col[r]), k));
+      int piv = k;
+      float best = fabsf(ck[k]);
 #pragma unroll
-      for (int c = 0; c < RK; ++c) {
-        const int j = lane + c * FOLX_WAVE;
-        if (j < 2 * NP) aug[i * AUGS + j] -= f * rowk[c];
+      for (int r = k + 1; r < NP; ++r)
+        if (r < n && fabsf(ck[r]) > best) { best = fabsf(ck[r]); piv = r; }
+      if (piv != k) {
+        // rows k and piv change places, in column k's copy and in this lane's column
+        float ckp = ck[k], mine = col[k];
+#pragma unroll
+        for (int r = k + 1; r < NP; ++r)
+          if (r == piv) {
+            const float t = ck[r]; ck[r] = ckp; ckp = t;
+            const float u = col[r]; col[r] = mine; mine = u;
+          }
+        ck[k] = ckp;
+        col[k] = mine;
+        sgn = -sgn;
       }
+      const float pv = ck[k];
+      logdet += logf(fabsf(pv));
+      if (pv < 0.0f) sgn = -sgn;
+      if (pv == 0.0f) sgn = 0.0f;
+      const float pr = col[k] * (1.0f / pv);
+#pragma unroll
+      for (int r = 0; r < NP; ++r)
+        if (r != k) col[r] = fmaf(-ck[r], pr, col[r]);
+      col[k] = pr;
     }
-    __syncthreads();
   }
+  if (lane >= NP && lane < 2 * NP) {
+#pragma unroll
+    for (int r = 0; r < NP; ++r) aug[r * AUGS + lane] = col[r];
+  }
+  __syncthreads();
 }
 
 // tr(A^-1 L) = sum_ij A^-1[j][i] L[i][j], partial sum of this lane.
