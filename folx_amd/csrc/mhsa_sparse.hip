@@ -18,7 +18,7 @@
 // That is O(n^2 d) work per (walker, head) instead of O(P n^2 d); the kernel is bound by
 // writing the dense P x n x d output rows.
 //
-// One workgroup of 256 threads per (walker, head); q, k, v, o, p and the n x n accumulators
+// One workgroup of 512 threads per (walker, head); q, k, v, o, p and the n x n accumulators
 // live in LDS (rows of d + 4 floats, so that 16 threads reading 16 bytes each from 16
 // different rows cover all banks); dot products run on 128-bit LDS reads; the three vectors of
 // the next position are fetched while the current one is worked on.
@@ -36,7 +36,8 @@ struct SAArgs {
   int32_t n, H, d, K;
 };
 
-constexpr int SA_NT = 256;
+constexpr int SA_NT = 512;  // two workgroups per CU (LDS and 128 registers): four wavefronts per SIMD
+constexpr int SA_RP = SA_NT / 16;  // output rows per pass: 16 threads of 16 bytes cover a row of d <= 64
 
 // dot product of two 16-byte aligned LDS vectors of 4 * d4 floats
 __device__ __forceinline__ float sa_dot(const float* u, const float* m, int d4) {
@@ -49,7 +50,7 @@ __device__ __forceinline__ float sa_dot(const float* u, const float* m, int d4) 
   }
   return (s0 + s1) + (s2 + s3);
 }
-constexpr int SA_MAXPASS = 4;  // n <= 64: rows i = 16 pass + tid / 16
+constexpr int SA_MAXPASS = 64 / SA_RP;  // n <= 64: rows i = SA_RP pass + tid / 16
 constexpr int SA_E = 4;        // sequence positions worked on together
 
 __host__ __device__ inline int64_t sa_lds_floats(int n, int d, int K) {
@@ -57,7 +58,7 @@ __host__ __device__ inline int64_t sa_lds_floats(int n, int d, int K) {
   return 4LL * n * dp + 4LL * n * np1 + SA_E * (4LL * K * d + 2LL * K * n + 2LL * K) + 5LL * n + (int64_t)K * n;
 }
 
-__global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
+__global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   const int n = a.n, d = a.d, K = a.K, H = a.H;
   const int dp = d + 4, np1 = n + 1, d4 = d / 4;
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
 #pragma unroll
   for (int ps = 0; ps < SA_MAXPASS; ++ps) {
     t2acc[ps] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int i = ps * 16 + orow;
+    const int i = ps * SA_RP + orow;
     oreg[ps] = (i < n && ot4 < d4) ? *reinterpret_cast<const float4*>(oS + i * dp + 4 * ot4)
                                    : make_float4(0.f, 0.f, 0.f, 0.f);
   }
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
         const float4 o4 = *reinterpret_cast<const float4*>(oS + e * dp + 4 * ot4);
         float pie[SA_MAXPASS];
 #pragma unroll
-        for (int ps = 0; ps < SA_MAXPASS; ++ps) pie[ps] = (ps * 16 + orow < n) ? pS[(ps * 16 + orow) * np1 + e] : 0.0f;
+        for (int ps = 0; ps < SA_MAXPASS; ++ps) pie[ps] = (ps * SA_RP + orow < n) ? pS[(ps * SA_RP + orow) * np1 + e] : 0.0f;
         for (int sl = 0; sl < K; ++sl) {
           const int c = idxS[sl * n + e];
           if (c < 0) continue;
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
           float* dst = a.oj + (int64_t)c * Srow + 4 * ot4;
 #pragma unroll
           for (int ps = 0; ps < SA_MAXPASS; ++ps) {
-            const int i = ps * 16 + orow;
+            const int i = ps * SA_RP + orow;
             if (i < n) {
               const float bi = beS[es * n + i];
               const float4 oi = oreg[ps];
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(SA_NT) void mhsa_sparse_kernel(SAArgs a) {
   if (ot4 < d4) {
 #pragma unroll
     for (int ps = 0; ps < SA_MAXPASS; ++ps) {
-      const int i = ps * 16 + orow;
+      const int i = ps * SA_RP + orow;
       if (i < n) {
         float r[4] = {2.0f * t2acc[ps].x, 2.0f * t2acc[ps].y, 2.0f * t2acc[ps].z, 2.0f * t2acc[ps].w};
 #pragma unroll 4
@@ -374,7 +375,7 @@ extern "C" int folx_hip_mhsa_sparse_fwdlap(void* stream, const float* q, const f
   if (B == 0) return FOLX_HIP_OK;
   if (!q || !q_jac || !q_lap || !k || !k_jac || !k_lap || !v || !v_jac || !v_lap || !index || !o || !o_jac || !o_lap)
     return FOLX_HIP_EINVAL;
-  if (n > 16 * SA_MAXPASS || d > 64 || d % 4 != 0 || k_rows > 8 || 3 * k_rows * (d / 4) > SA_NT)
+  if (n > SA_RP * SA_MAXPASS || d > 64 || d % 4 != 0 || k_rows > 8 || 3 * k_rows * (d / 4) > SA_NT)
     return FOLX_HIP_ENOTSUP;
   const void* ptrs[] = {q, q_jac, q_lap, k, k_jac, k_lap, v, v_jac, v_lap, o, o_jac, o_lap};
   for (const void* p : ptrs)

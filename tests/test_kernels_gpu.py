@@ -595,7 +595,8 @@ def test_mhsa(B, n, H, d, P, valid):
 
 
 @pytest.mark.parametrize('B,n,H,d,k,missing', [(3, 32, 4, 64, 3, False), (2, 7, 2, 8, 3, True), (1, 64, 1, 64, 3, False),
-                                              (2, 16, 2, 32, 6, False), (2, 5, 3, 12, 1, False), (1, 33, 2, 60, 2, True)])
+                                              (2, 16, 2, 32, 6, False), (2, 5, 3, 12, 1, False), (1, 33, 2, 60, 2, True),
+                                              (1, 12, 1, 64, 8, False)])
 def test_mhsa_sparse(B, n, H, d, k, missing):
     """Attention with position-sparse Jacobians against the dense rule of the oracle on the
     materialised Jacobians, and against the dense kernel."""
