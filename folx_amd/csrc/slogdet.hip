@@ -64,7 +64,7 @@ struct Tile<32> {
 constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
 
 template <int NP, bool HAS_F>
-__global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
+__global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
@@ -105,7 +105,9 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   for (int t = 0; t < STEPS; ++t) {
     const int k = T::KS * t + lq;
     ok[t] = k < n && lr < n;
-    eoff[t] = (int64_t)k * rstride + lr;
+    // elements of the padding ask for element (0, 0): loads are never branched around, so
+    // that all of them are in flight before the first wait
+    eoff[t] = ok[t] ? (int64_t)k * rstride + lr : 0;
     ainv[t] = ok[t] ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
   }
   constexpr int EF = HAS_F ? STEPS : 1;
@@ -115,13 +117,27 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
       const int64_t off = base + eoff[t];
-      fx[t] = ok[t] ? fc.x[off] : 0.0f;
-      ax[t] = ok[t] ? A[off] : 0.0f;
+      fx[t] = fc.x[off];
+      ax[t] = A[off];
       lapx[t] = 0.0f;
 #pragma unroll
       for (int sl = 0; sl < KF; ++sl) {
-        fidx[sl][t] = (ok[t] && sl < fc.kf) ? fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w] : -1;
-        fj[sl][t] = fidx[sl][t] >= 0 ? fc.jac[(int64_t)sl * slice + off] : 0.0f;
+        fidx[sl][t] = -1;
+        fj[sl][t] = 0.0f;
+        if (sl < fc.kf) {  // the same for all lanes
+          fidx[sl][t] = fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w];
+          fj[sl][t] = fc.jac[(int64_t)sl * slice + off];
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      fx[t] = ok[t] ? fx[t] : 0.0f;
+      ax[t] = ok[t] ? ax[t] : 0.0f;
+#pragma unroll
+      for (int sl = 0; sl < KF; ++sl) {
+        fidx[sl][t] = ok[t] ? fidx[sl][t] : -1;
+        fj[sl][t] = fidx[sl][t] >= 0 ? fj[sl][t] : 0.0f;
       }
     }
   }
@@ -134,7 +150,7 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   auto request = [&](float (&dst)[STEPS], int p) __attribute__((always_inline)) {
     const float* src = AJ + (int64_t)p * slice + base;
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) dst[t] = ok[t] ? src[eoff[t]] : 0.0f;  // A_jac[p][k][lr]
+    for (int t = 0; t < STEPS; ++t) dst[t] = src[eoff[t]];  // A_jac[p][k][lr], padding masked when used
   };
 #pragma unroll
   for (int d = 0; d < D; ++d)
@@ -147,7 +163,7 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
         float jv[STEPS];
 #pragma unroll
         for (int t = 0; t < STEPS; ++t) {
-          float v = raw[d][t];
+          float v = ok[t] ? raw[d][t] : 0.0f;
           if constexpr (HAS_F) {
             float add = 0.0f;
 #pragma unroll
@@ -173,8 +189,11 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
         trs[p % TRB][lane] = tr;
         if ((p + 1) % TRB == 0 || p + 1 == P) {
           // ld_jac of the last rows: four lanes per row add up 16 of its 64 parts each
+          // The workgroup is one wavefront and LDS serves a wavefront's accesses in issue
+          // order, so the other lanes' writes above are seen without a barrier; a barrier's
+          // fence would also wait for the Jacobian rows requested ahead.
           const int pb = p / TRB * TRB, pe = p + 1 - pb;
-          __syncthreads();
+          asm volatile("" ::: "memory");
           const int row = lane % TRB, part = lane / TRB;
           float sm = 0.0f;
 #pragma unroll
@@ -182,7 +201,7 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
           sm += __shfl_xor(sm, 16, FOLX_WAVE);
           sm += __shfl_xor(sm, 32, FOLX_WAVE);
           if (part == 0 && row < pe) jac_out[(int64_t)(pb + row) * NM + m] = sm;
-          __syncthreads();
+          asm volatile("" ::: "memory");
         }
       }
     }
@@ -190,11 +209,10 @@ __global__ __launch_bounds__(FOLX_WAVE) void slogdet_kernel(
   if constexpr (HAS_F) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
-      if (ok[t]) {
-        const int64_t off = base + eoff[t];
-        const float al = fx[t] * AL[off] + ax[t] * fc.lap[off] + lapx[t];
-        tl += ainv[t] * al;  // tr(A^-1 lap A) = sum A^-1[lr][k] lap A[k][lr]
-      }
+      // fx, ax, lapx and ainv are zero at the padding
+      const int64_t off = base + eoff[t];
+      const float al = fx[t] * AL[off] + ax[t] * fc.lap[off] + lapx[t];
+      tl += ainv[t] * al;  // tr(A^-1 lap A) = sum A^-1[lr][k] lap A[k][lr]
     }
   }
   mm = wave_sum(mm);

@@ -36,15 +36,28 @@ __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict
   static_assert(2 * NP <= FOLX_WAVE, "one lane per column of [A | I]");
   if (row_stride == 0) row_stride = n;  // rows of the matrix follow each other
   constexpr int AUGS = Aug<NP>::stride;
+  // All loads are issued before the first one is waited for: lanes and rows outside the
+  // matrix ask for element (0, 0) instead of branching around the load.
   float col[NP];
+  const bool in_cols = lane < n;
+  if (factor) {  // the matrix is the elementwise product a * factor (same layout)
+    float fv[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) {
+      const int64_t off = (in_cols && r < n) ? r * row_stride + lane : 0;
+      col[r] = a[off];
+      fv[r] = factor[off];
+    }
+#pragma unroll
+    for (int r = 0; r < NP; ++r) col[r] *= fv[r];
+  } else {
+#pragma unroll
+    for (int r = 0; r < NP; ++r) col[r] = a[(in_cols && r < n) ? r * row_stride + lane : 0];
+  }
 #pragma unroll
   for (int r = 0; r < NP; ++r) {
-    float v;
-    // with `factor` (same layout as a) the matrix is the elementwise product a * factor
-    if (lane < NP) v = (r < n && lane < n) ? a[r * row_stride + lane] * (factor ? factor[r * row_stride + lane] : 1.0f)
-                                           : (r == lane ? 1.0f : 0.0f);
-    else v = (lane - NP == r) ? 1.0f : 0.0f;
-    col[r] = v;
+    const float unit = (lane < NP ? lane : lane - NP) == r ? 1.0f : 0.0f;  // padding and the right half
+    col[r] = (in_cols && r < n) ? col[r] : unit;
   }
   logdet = 0.0f;
   sgn = 1.0f;
