@@ -167,8 +167,8 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
           if constexpr (HAS_F) {
             float add = 0.0f;
 #pragma unroll
-            for (int sl = 0; sl < KF; ++sl)
-              if (fidx[sl][t] == p) { add += fj[sl][t]; lapx[t] += 2.0f * v * fj[sl][t]; }
+            for (int sl = 0; sl < KF; ++sl) add += fidx[sl][t] == p ? fj[sl][t] : 0.0f;
+            lapx[t] = fmaf(2.0f * v, add, lapx[t]);  // cross term 2 dA . dF of the product's Laplacian
             v = fx[t] * v + ax[t] * add;
           }
           jv[t] = v;
