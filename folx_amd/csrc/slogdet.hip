@@ -63,7 +63,8 @@ struct Tile<32> {
 
 constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
 
-template <int NP, bool HAS_F>
+// KFT = slots of the factor's sparse Jacobian the kernel keeps in registers (>= fc.kf).
+template <int NP, bool HAS_F, int KFT = KF>
 __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
@@ -111,8 +112,8 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
     ainv[t] = ok[t] ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
   }
   constexpr int EF = HAS_F ? STEPS : 1;
-  float fx[EF], ax[EF], lapx[EF], fj[KF][EF];
-  int32_t fidx[KF][EF];
+  float fx[EF], ax[EF], lapx[EF], fj[KFT][EF];
+  int32_t fidx[KFT][EF];
   if constexpr (HAS_F) {
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
       ax[t] = A[off];
       lapx[t] = 0.0f;
 #pragma unroll
-      for (int sl = 0; sl < KF; ++sl) {
+      for (int sl = 0; sl < KFT; ++sl) {
         fidx[sl][t] = -1;
         fj[sl][t] = 0.0f;
         if (sl < fc.kf) {  // the same for all lanes
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
       fx[t] = ok[t] ? fx[t] : 0.0f;
       ax[t] = ok[t] ? ax[t] : 0.0f;
 #pragma unroll
-      for (int sl = 0; sl < KF; ++sl) {
+      for (int sl = 0; sl < KFT; ++sl) {
         fidx[sl][t] = ok[t] ? fidx[sl][t] : -1;
         fj[sl][t] = fidx[sl][t] >= 0 ? fj[sl][t] : 0.0f;
       }
@@ -144,7 +145,7 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
 
   // Jacobian rows are requested D rows ahead: with one row in flight per wavefront the kernel
   // would be bound by the latency of its own loads, not by HBM bandwidth.
-  constexpr int D = MP == 16 ? 4 : 1;
+  constexpr int D = MP == 16 ? ((HAS_F && KFT < KF) ? 6 : 4) : 1;
   float mm = 0.0f;
   float raw[D][STEPS];
   auto request = [&](float (&dst)[STEPS], int p) __attribute__((always_inline)) {
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
           if constexpr (HAS_F) {
             float add = 0.0f;
 #pragma unroll
-            for (int sl = 0; sl < KF; ++sl) add += fidx[sl][t] == p ? fj[sl][t] : 0.0f;
+            for (int sl = 0; sl < KFT; ++sl) add += fidx[sl][t] == p ? fj[sl][t] : 0.0f;
             lapx[t] = fmaf(2.0f * v, add, lapx[t]);  // cross term 2 dA . dF of the product's Laplacian
             v = fx[t] * v + ax[t] * add;
           }
@@ -319,17 +320,19 @@ int launch_slogdet(hipStream_t st, const float* A, const float* A_jac, const flo
     share = 128 / (n * 4);
     while (share > 1 && ND % share != 0) share /= 2;
   }
-#define FOLX_SLD_LAUNCH(NPV, HASF)                                                                             \
-  slogdet_kernel<NPV, HASF><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND, \
-                                                    batch_stride, member_stride, row_stride, jac_stride, share,  \
-                                                    fc ? *fc : Factor{})
+#define FOLX_SLD_LAUNCH(NPV, HASF, KFV)                                                                   \
+  slogdet_kernel<NPV, HASF, KFV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, \
+                                                         ND, batch_stride, member_stride, row_stride, jac_stride, \
+                                                         share, fc ? *fc : Factor{})
   if (fc) {
-    if (n <= 8) FOLX_SLD_LAUNCH(8, true);
-    else FOLX_SLD_LAUNCH(16, true);
+    // three slots (the coordinates of one electron) leave registers for two more rows in flight
+    const bool three = fc->kf <= 3;
+    if (n <= 8) { if (three) FOLX_SLD_LAUNCH(8, true, 3); else FOLX_SLD_LAUNCH(8, true, KF); }
+    else { if (three) FOLX_SLD_LAUNCH(16, true, 3); else FOLX_SLD_LAUNCH(16, true, KF); }
   } else {
-    if (n <= 8) FOLX_SLD_LAUNCH(8, false);
-    else if (n <= 16) FOLX_SLD_LAUNCH(16, false);
-    else FOLX_SLD_LAUNCH(32, false);
+    if (n <= 8) FOLX_SLD_LAUNCH(8, false, KF);
+    else if (n <= 16) FOLX_SLD_LAUNCH(16, false, KF);
+    else FOLX_SLD_LAUNCH(32, false, KF);
   }
 #undef FOLX_SLD_LAUNCH
   return folx_launch_status();

@@ -675,7 +675,8 @@ def test_exp_envelope(rows, nI, O, P):
 
 
 @pytest.mark.parametrize('B,ND,n,P,k,strided', [(3, 4, 16, 48, 3, True), (2, 3, 8, 24, 3, True), (2, 2, 5, 9, 2, False),
-                                               (1, 16, 16, 96, 3, True), (2, 1, 3, 7, 4, False)])
+                                               (1, 16, 16, 96, 3, True), (2, 1, 3, 7, 4, False),
+                                               (2, 2, 12, 20, 4, False), (1, 3, 16, 50, 3, False), (2, 2, 7, 11, 1, False)])
 def test_slogdet_scaled(B, ND, n, P, k, strided):
     """slogdet of A * F with the product formed on load (sparse Jacobian of F) against the mul
     rule followed by the slogdet rule of the oracle."""
