@@ -13,7 +13,8 @@ from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBPATH = os.path.join(_HERE, 'lib', 'libfolx_hip.so')
 
-OK, EINVAL, ENOTSUP, ELAUNCH = 0, -1, -2, -3
+OK, EINVAL, ENOTSUP, ELAUNCH, ESCRATCH = 0, -1, -2, -3, -4
+STATIC_SCRATCH_BYTES = 64 << 20
 
 # name -> (restype, argtypes); mirrors include/folx_hip.h one to one
 _P = c_void_p
@@ -29,6 +30,8 @@ SIGNATURES = {
     'folx_hip_norm_dense_workspace_bytes': (c_int64, [c_int64, c_int32, c_int32, c_int32, c_int32]),
     'folx_hip_norm_dense_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 5 + [c_float] + [_P] * 5
                                    + [c_int64, c_int32, c_int32, c_int32, _P, c_int64]),
+    'folx_hip_norm_dense_static_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 5 + [c_float] + [_P] * 5
+                                          + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_layernorm_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_float]),
     'folx_hip_elementwise_fwdlap': (c_int, [_P, c_int32, c_float, _P, _P, _P, _P, _P, _P, c_int64, c_int32]),
     'folx_hip_exp_envelope_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_int32]),

@@ -9,6 +9,7 @@ extern "C" const char* folx_hip_strerror(int code) {
     case FOLX_HIP_EINVAL: return "invalid argument (null pointer, negative size or inconsistent shape)";
     case FOLX_HIP_ENOTSUP: return "size not supported by the gfx950 kernels";
     case FOLX_HIP_ELAUNCH: return "kernel launch failed (hipGetLastError)";
+    case FOLX_HIP_ESCRATCH: return "shape needs more scratch memory than the library's static 64 MiB array";
     default: return "unknown folx_hip error code";
   }
 }

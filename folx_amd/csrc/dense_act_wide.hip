@@ -46,6 +46,7 @@
 // (lane l, register j of group t <-> k = 8 t + 4 (l / 32) + j), piece c of an A row stored at
 // slot c ^ ((row / 2) % 4).  Only the address a lane asks for differs: tile row m is
 // Jacobian row p0 + m % 32 of position r0 + m / 32.
+#include <mutex>
 #include <type_traits>
 
 #include "activations.h"
@@ -757,4 +758,62 @@ extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float 
   }
   return run_wide((hipStream_t)stream, false, act, param, x, nullptr, lap, nullptr, nullptr, 0.0f, W, bias, y, y_jac,
                   y_lap, R, P, K, N, workspace, workspace_bytes, &parts, res, res_jac, res_lap);
+}
+
+// ---- folx_hip_norm_dense_fwdlap on the library's own scratch memory -------------------------
+//
+// For callers that cannot bring a workspace because they cannot allocate one (code under HIP
+// graph capture, tight serving loops).  The workspace of run_wide() is a file-scope device
+// array; every GPU the library runs on holds its own copy of it, at its own address, until the
+// process ends.  In host code the array's name is only a handle of the symbol, so the device
+// address is asked for once per device (hipGetSymbolAddress, with that device current) and
+// kept; everything below uses the pointer, never the name.
+namespace {
+
+constexpr int64_t SCRATCH_BYTES = FOLX_HIP_STATIC_SCRATCH_BYTES;
+constexpr int MAX_DEVICES = 64;
+
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+namespace {
+
+void* g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each device, once known
+std::mutex g_scratch_mutex;
+
+// Address of this device's copy of `scratch`; nullptr when the runtime refuses.
+void* scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int folx_hip_norm_dense_static_fwdlap(void* stream, int32_t act, float param, const float* x,
+                                                 const float* jac, const float* lap, const float* gamma,
+                                                 const float* beta, float eps, const float* W, const float* bias,
+                                                 float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
+                                                 int32_t K, int32_t N) {
+  if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
+  WidePlan pl;
+  if ((act >= 0 && !act_fused(act)) || !plan_wide(R, P, K, N, true, act >= 0, pl)) return FOLX_HIP_ENOTSUP;
+  if (pl.ws_bytes > SCRATCH_BYTES) return FOLX_HIP_ESCRATCH;
+  void* ptr = scratch_of_current_device();
+  if (!ptr) return FOLX_HIP_ELAUNCH;
+  // Nothing in the workspace has to start at zero: every launch of run_wide() writes the part
+  // it owns (folded weights, per-position rows, one slab of sums per group of Jacobian rows)
+  // in full before a later launch on the same stream reads it.
+  return run_wide((hipStream_t)stream, true, act, param, x, jac, lap, gamma, beta, eps, W, bias, y, y_jac, y_lap, R, P,
+                  K, N, ptr, SCRATCH_BYTES);
 }

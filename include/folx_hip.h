@@ -29,6 +29,11 @@ extern "C" {
 #define FOLX_HIP_EINVAL (-1)   /* null pointer, negative size, inconsistent shape      */
 #define FOLX_HIP_ENOTSUP (-2)  /* size outside what the kernels are built for          */
 #define FOLX_HIP_ELAUNCH (-3)  /* hipGetLastError() != hipSuccess after the launch     */
+#define FOLX_HIP_ESCRATCH (-4) /* needs more than FOLX_HIP_STATIC_SCRATCH_BYTES of scratch */
+
+/* Size of the library's own scratch array (folx_hip_norm_dense_static_fwdlap): 64 MiB of
+ * device memory on every GPU the library has been used on, held until the process ends. */
+#define FOLX_HIP_STATIC_SCRATCH_BYTES (64ll << 20)
 
 /* Library version (major * 10000 + minor * 100 + patch). */
 int folx_hip_version(void);
@@ -215,6 +220,27 @@ int folx_hip_norm_dense_fwdlap(void* stream, int32_t act, float param, const flo
                                const float* beta, float eps, const float* W, const float* bias,
                                float* y, float* y_jac, float* y_lap, int64_t R, int32_t P,
                                int32_t K, int32_t N, void* workspace, int64_t workspace_bytes);
+
+/*
+ * folx_hip_norm_dense_fwdlap without a workspace argument, for callers that cannot allocate
+ * device memory: code under HIP graph capture, serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference (jax owns all memory there).  Same arguments, shape
+ * limits, kernels and bit-for-bit the same results as folx_hip_norm_dense_fwdlap; the
+ * partial sums and per-position rows live in a device array of FOLX_HIP_STATIC_SCRATCH_BYTES
+ * that is part of the library's code object (one copy per GPU).  The call allocates and frees
+ * nothing.  Shapes whose folx_hip_norm_dense_workspace_bytes() exceeds that size return
+ * FOLX_HIP_ESCRATCH and launch nothing (R = 4096 rows at P = 96, K = N = 256 with an
+ * activation need 36 MiB; the size grows linearly in R).  All calls on one GPU share the
+ * array: calls that may overlap in time on one GPU (different streams, or threads) race and
+ * must be serialised by the caller; calls on one stream are ordered and safe.  The first call
+ * on a device looks the array's address up (hipGetSymbolAddress), so make that call outside a
+ * graph capture.
+ */
+int folx_hip_norm_dense_static_fwdlap(void* stream, int32_t act, float param, const float* x,
+                                      const float* jac, const float* lap, const float* gamma,
+                                      const float* beta, float eps, const float* W,
+                                      const float* bias, float* y, float* y_jac, float* y_lap,
+                                      int64_t R, int32_t P, int32_t K, int32_t N);
 
 /*
  * Binary elementwise rule for two operands whose Jacobians live on the same row frame

@@ -105,6 +105,15 @@ def test_unsupported_sizes(lib):
     assert nd(-1, 64, 256, 256, None, 0) == _lib.EINVAL        # no workspace
     assert nd(-1, 62, 256, 256, one, 1 << 30) == _lib.ENOTSUP  # rows % 4
     assert nd(3, 64, 256, 256, one, 1 << 30) == _lib.ENOTSUP   # log: not fused
+    # the same rule on the library's own scratch array: size checks come before any GPU call
+    nds = lambda act, R, K, N: lib.folx_hip_norm_dense_static_fwdlap(None, act, 0.0, one, one, one, one, one, 1e-5, one,
+                                                                     one, one, one, one, R, 33, K, N)
+    assert nds(-1, 62, 256, 256) == _lib.ENOTSUP      # rows % 4
+    assert nds(3, 64, 256, 256) == _lib.ENOTSUP       # log: not fused
+    assert nds(-1, -4, 256, 256) == _lib.EINVAL
+    assert lib.folx_hip_norm_dense_workspace_bytes(1 << 17, 33, 256, 256, 0) > _lib.STATIC_SCRATCH_BYTES
+    assert nds(0, 1 << 17, 256, 256) == _lib.ESCRATCH  # beyond the 64 MiB array: refused, nothing launched
+    assert b'scratch' in lib.folx_hip_strerror(_lib.ESCRATCH)
     assert lib.folx_hip_dense_act_workspace_bytes(2000, 400, 100, 100) > 0                                    # rows split
     assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 65, 1, 8, 3) == _lib.ENOTSUP
     assert lib.folx_hip_mhsa_sparse_fwdlap(None, *([one] * 13), 1, 8, 1, 6, 3) == _lib.ENOTSUP
