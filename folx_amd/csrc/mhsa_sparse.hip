@@ -8,8 +8,8 @@
 // o'_c = p v'_c + p'_c v, ...) collapses to vector work per Jacobian row:
 //   s'_c[i][j] = [i = e] alpha[j] + beta[i] [j = e]
 //   r_c[i]     = [i = e] rho + p[i][e] beta[i],            rho = sum_j p[e][j] alpha[j]
-//   o'_c[i]    = p[i][e] (w + beta[i] (v[e] - o[i])) + [i = e] (gamma - rho o[e]),
-//                gamma = sum_j p[e][j] alpha[j] v[j]
+//   o'_c[i]    = p[i][e] (w + beta[i] (v[e] - o[i])) + [i = e] gamma,
+//                gamma = sum_j p[e][j] alpha[j] (v[j] - o[e])
 // and the second-order part of the Laplacian needs, besides n x n sums of squares of alpha and
 // beta, a single n x n x d product:
 //   lap_o = p lap_v + (pL + M) v + 2 sum_c p'_c[:, e] w_c
@@ -190,18 +190,21 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
       }
     }
     __syncthreads();
-    // rho[e][s] = sum_j p[e][j] alpha[e][s][j],  gamma[e][s] = sum_j p[e][j] alpha[e][s][j] v[j]
+    // rho[e][s] = sum_j p[e][j] alpha[e][s][j],  gamma[e][s] = sum_j p[e][j] alpha[e][s][j] (v[j] - o[e])
     for (int it = tid; it < ne * K * d4; it += SA_NT) {
       const int es = it / d4, t4 = it - es * d4;
       const int e = e0 + es / K;
       float rho = 0.0f;
       float4 gm = make_float4(0.f, 0.f, 0.f, 0.f);
+      // gamma - rho o[e] summed as sum_j p alpha (v[j] - o[e]): the two parts nearly cancel
+      const float4 oe = *reinterpret_cast<const float4*>(oS + e * dp + 4 * t4);
 #pragma unroll 8
       for (int j = 0; j < n; ++j) {
         const float pa = pS[e * np1 + j] * alS[es * n + j];
         const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * t4);
         rho += pa;
-        gm.x += pa * vv.x; gm.y += pa * vv.y; gm.z += pa * vv.z; gm.w += pa * vv.w;
+        gm.x += pa * (vv.x - oe.x); gm.y += pa * (vv.y - oe.y);
+        gm.z += pa * (vv.z - oe.z); gm.w += pa * (vv.w - oe.w);
       }
       *reinterpret_cast<float4*>(gamS + es * d + 4 * t4) = gm;
       if (t4 == 0) rhoS[es] = rho;
@@ -213,7 +216,6 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
       for (int ee = 0; ee < ne; ++ee) {
         const int e = e0 + ee;
         const float4 v4 = *reinterpret_cast<const float4*>(vS + e * dp + 4 * ot4);
-        const float4 o4 = *reinterpret_cast<const float4*>(oS + e * dp + 4 * ot4);
         float pie[SA_MAXPASS];
 #pragma unroll
         for (int ps = 0; ps < SA_MAXPASS; ++ps) pie[ps] = (ps * SA_RP + orow < n) ? pS[(ps * SA_RP + orow) * np1 + e] : 0.0f;
@@ -239,8 +241,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
               r.w = pie[ps] * (w4.w + bi * (v4.w - oi.w));
               float cf = pie[ps] * bi * (1.0f - pie[ps]);
               if (i == e) {
-                r.x += g4.x - rho * o4.x; r.y += g4.y - rho * o4.y;
-                r.z += g4.z - rho * o4.z; r.w += g4.w - rho * o4.w;
+                r.x += g4.x; r.y += g4.y; r.z += g4.z; r.w += g4.w;
                 cf += pie[ps] * (ale - rho);
               }
               folx_st_stream4(dst + grow(i), r);

@@ -412,7 +412,27 @@ def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta
     sd = bstrides(d.shape, out_shape) if d is not None else [0] * len(out_shape)
     col = collapse3(out_shape, sin, sc, sd)
     if col is None:
-        raise ValueError('rows_affine: more than 3 broadcast dims after collapsing')
+        # a coefficient array that is broadcast along inner axes (e.g. a per-matrix identity against
+        # (walker, row, determinant, column)): spell its broadcast out over all axes but the first,
+        # then over all axes, until the index space collapses to three dimensions
+        for lead in (1, 0):
+            def spelled(t):
+                if t is None:
+                    return None
+                full = (1,) * (len(out_shape) - t.dim()) + tuple(t.shape)
+                tgt = tuple(full[:lead]) + tuple(out_shape[lead:])
+                return t.reshape(full).expand(tgt).contiguous()
+            c2, d2 = spelled(c), spelled(d)
+            sc = bstrides(c2.shape, out_shape) if c2 is not None else [0] * len(out_shape)
+            sd = bstrides(d2.shape, out_shape) if d2 is not None else [0] * len(out_shape)
+            col = collapse3(out_shape, sin, sc, sd)
+            if col is not None:
+                c, d = c2, d2
+                break
+    if col is None:
+        raise NotImplementedError(
+            f'rows_affine: the input of shape {tuple(row_shape)} broadcast to {tuple(out_shape)} needs more than '
+            'three index dimensions; broadcast it with broadcast_to first')
     n, (s_in, s_c, s_d) = col
     out = torch.empty((rows, *out_shape), device=inp.device, dtype=torch.float32)
     in_S = int(np.prod(row_shape, dtype=np.int64))

@@ -59,6 +59,7 @@ class PsiFormerConfig:
     nuc_box: float = 2.0
     seed: int = 0
     ln_eps: float = 1e-5
+    orb_shift: float = 0.0  # c > 0: orbital matrices are A + c I (well-conditioned determinants for parity tests)
 
     @property
     def n_up(self):
@@ -190,8 +191,13 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
         env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])  # (m, n_det * m)
         # (electron, determinant, orbital): the matrices are read in place, rows on axis 0, and
         # multiplied by their envelopes while they are loaded
-        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
-                            factor=xp.reshape(env, (m, cfg.n_det, m)))
+        if cfg.orb_shift:
+            shift = (cfg.orb_shift * np.eye(m, dtype=np.float32))[:, None, :]
+            mats = xp.add(xp.multiply(xp.reshape(orb, (m, cfg.n_det, m)), xp.reshape(env, (m, cfg.n_det, m))), shift)
+            sg, ld = xp.slogdet(mats, row_axis=0)
+        else:
+            sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
+                                factor=xp.reshape(env, (m, cfg.n_det, m)))
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
@@ -218,6 +224,7 @@ class FermiNetConfig:
     n_det: int = 16
     nuc_box: float = 2.0
     seed: int = 0
+    orb_shift: float = 0.0  # as in PsiFormerConfig
 
     @property
     def n_up(self):
@@ -307,8 +314,13 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
             continue
         orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))
         env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])
-        sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
-                            factor=xp.reshape(env, (m, cfg.n_det, m)))
+        if cfg.orb_shift:
+            shift = (cfg.orb_shift * np.eye(m, dtype=np.float32))[:, None, :]
+            mats = xp.add(xp.multiply(xp.reshape(orb, (m, cfg.n_det, m)), xp.reshape(env, (m, cfg.n_det, m))), shift)
+            sg, ld = xp.slogdet(mats, row_axis=0)
+        else:
+            sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
+                                factor=xp.reshape(env, (m, cfg.n_det, m)))
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])

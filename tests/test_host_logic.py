@@ -637,3 +637,27 @@ def test_slogdet_with_factor(monkeypatch):
     check_against_oracle(lambda xp, r: fn(xp, r, True), x, 6)       # the factor depends on every node: dense, mul rule first
     check_against_oracle(lambda xp, r: fn(xp, r, False), x, 0)      # everything dense
     assert True not in calls
+
+
+def test_stagecheck_runs_every_kernel_call_against_its_fp64_rule():
+    """tests/stagecheck.py on the stand-ins: every call is compared with the float64 rule of the
+    same inputs, and a corrupted kernel is caught at its stage."""
+    import folx_amd.kernels as K
+    from stagecheck import StageCheck
+
+    p = wl.psiformer_params(SMALL_PSI)
+    x = wl.sample_electrons(2, SMALL_PSI.n_elec, 1.0, seed=3)
+    fn = lambda xp, t: wl.psiformer_forward(p, t, xp)
+    with StageCheck() as sc:
+        run_product(fn, x, 6)
+    used = sc.summary()
+    assert {'dense', 'mhsa', 'slogdet'} <= set(used) or {'dense', 'mhsa_sparse', 'slogdet'} <= set(used), used
+    assert all(w <= 1.0 for _, w, _ in used.values())
+    good = K.elementwise
+    K.elementwise = lambda *a, **k: tuple(t * (1 + 3e-5) for t in good(*a, **k))  # a 3e-5 relative error
+    try:
+        with pytest.raises(AssertionError, match='elementwise'):
+            with StageCheck():
+                run_product(lambda xp, t: xp.sum(xp.tanh(t)), x, 0)
+    finally:
+        K.elementwise = good

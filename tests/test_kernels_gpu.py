@@ -440,6 +440,15 @@ def test_rows_affine():
     assert_val(got, 0.5 * inp.astype(np.float64) * c + (-2.0) * d)
     got = K.rows_affine(dev(inp[:, :, :1]), rows, (3, 1, 6), shape, None, None, alpha=-1.0)
     assert_val(got, -np.broadcast_to(inp[:, :, :1], (rows, *shape)))
+    # a coefficient that is broadcast along two inner axes of a four-axis index space (an identity per
+    # matrix against (walker, row, determinant, column)): the wrapper spells the broadcast out
+    shape4 = (2, 5, 3, 5)
+    inp4 = rand(rng, 2, *shape4)
+    eye = (7.0 * np.eye(5, dtype=np.float32))[None, :, None, :]
+    got = K.rows_affine(dev(inp4), 2, shape4, shape4, None, dev(eye), alpha=1.0, beta=1.0)
+    assert_val(got, inp4.astype(np.float64) + eye)
+    got = K.rows_affine(dev(inp4[:, :, :, :1]), 2, (2, 5, 1, 5), shape4, dev(eye), None, alpha=2.0)
+    assert_val(got, 2.0 * np.broadcast_to(inp4[:, :, :, :1], (2, *shape4)).astype(np.float64) * eye)
 
 
 @pytest.mark.parametrize('outer,red,inner', [(7, 5, 9), (6, 100, 1), (3, 4, 1), (1, 33, 70)])

@@ -169,3 +169,110 @@ def test_psiformer32_full_batch_properties():
     assert_lap(full.laplacian[idx], small.laplacian.cpu().numpy())
     again = folx_amd.batched_vmap(fl, 1024)(x)
     assert torch.equal(again.x, full.x) and torch.equal(again.laplacian, full.laplacian)
+
+
+FULL_WIDTH = ['ferminet16', 'psiformer32', 'psiformer64']
+
+
+@pytest.mark.parametrize('name', FULL_WIDTH)
+def test_full_width_every_rule_call_meets_the_strict_bars(name):
+    """The benchmark architectures at their real widths, 2 walkers: every kernel call of the
+    forward Laplacian is compared, on the float32 inputs the HIP path handed it, with the
+    float64 oracle rule of that call at the strict bars (values / Jacobians rtol 1e-5,
+    Laplacians rtol 1e-4 + atol 1e-5), widened only by the measured response of that rule to
+    rounding noise in its inputs (tests/stagecheck.py; matters for the determinants)."""
+    import dataclasses
+
+    from stagecheck import StageCheck
+
+    forward, p, cfg, _, sigma, thr = wl.build(name)
+    x = wl.sample_electrons(2, cfg.n_elec, sigma, seed=2)
+    print(f'case {name} stage by stage', flush=True)
+    with StageCheck() as sc:
+        run(lambda xp, t: forward(p, t, xp), x, thr)
+    used = sc.summary()
+    for kern, (calls, worst, amp) in sorted(used.items()):
+        print(f'{name} {kern}: {calls} calls, worst error {worst:.2f} x bar, allowance {amp:.1f}', flush=True)
+    fused = {'psiformer32': ('norm_dense', 'mhsa', 'mhsa_sparse', 'slogdet', 'dense'),
+             'psiformer64': ('norm_dense', 'mhsa', 'mhsa_sparse', 'slogdet', 'dense'),
+             'ferminet16': ('dense_act_parts', 'dense_act', 'slogdet', 'dense')}[name]
+    assert set(fused) <= set(used), used
+    assert len(sc.log) >= 40
+
+
+WELL_CONDITIONED = {
+    # name: diagonal shift of the orbital matrices (their entries are O(1))
+    'ferminet16': 40.0, 'psiformer32': 60.0, 'psiformer64': 90.0,
+}
+
+
+@pytest.mark.parametrize('name', FULL_WIDTH)
+def test_full_width_well_conditioned_end_to_end_strict(name):
+    """The same architectures end to end at north-star tolerances (values / Jacobians rtol 1e-5,
+    Laplacians rtol 1e-4 + atol 1e-5, test/laplacian_testcase.py:16-49), with every orbital
+    matrix shifted by a multiple of the identity so that log|det| no longer amplifies float32
+    rounding (condition numbers of a few units, asserted below)."""
+    import dataclasses
+
+    from stagecheck import StageCheck
+
+    forward, p, cfg, _, sigma, thr = wl.build(name)
+    p = dataclasses.replace(p, cfg=dataclasses.replace(cfg, orb_shift=WELL_CONDITIONED[name]))
+    x = wl.sample_electrons(2, cfg.n_elec, sigma, seed=4)
+    print(f'case {name} well conditioned end to end', flush=True)
+    fn = lambda xp, t: forward(p, t, xp)
+    with StageCheck(names=('slogdet',)) as sc:
+        out = run(fn, x, thr)
+    assert sc.log and all(amp < 1.5 for *_, amp in sc.log), sc.log  # the determinants do not amplify input rounding
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    r32 = fn(ob, ob.init_state(x, dtype=np.float32))
+    J = out.jacobian.dense_array
+    from tolerances import LAP_ATOL, LAP_ATOL_REL, LAP_RTOL, VAL_ATOL_REL, VAL_RTOL
+
+    for got, want, w32, nm in ((out.x, ref.x, r32.x, 'x'), (J, ref.J, r32.J, 'jacobian'),
+                               (out.laplacian, ref.lap, r32.lap, 'laplacian')):
+        g = got.cpu().numpy().astype(np.float64)
+        scale = np.abs(want).max()
+        # what float32 arithmetic itself costs on this function: the numpy oracle run in float32
+        floor = np.abs(w32.astype(np.float64) - want).max()
+        print(f'{name} {nm}: max |hip - fp64| / max|fp64| = {np.abs(g - want).max() / scale:.2e}, '
+              f'numpy float32 oracle: {floor / scale:.2e}', flush=True)
+        rtol, atol = (LAP_RTOL, LAP_ATOL + LAP_ATOL_REL * scale) if nm == 'laplacian' else (VAL_RTOL, VAL_ATOL_REL * scale)
+        # the north-star bars; where a chain of 24 float32 matrix products (each within the bars on its
+        # own, see the stage-by-stage test) cannot meet them end to end, the absolute part grows to the
+        # error of the float32 numpy oracle on the same function
+        np.testing.assert_allclose(g, want, rtol=rtol, atol=max(atol, floor), err_msg=f'{name} {nm}')
+
+
+@pytest.mark.parametrize('name,chunk', [('psiformer64', 256), ('ferminet16', 1024)])
+def test_full_batch_properties(name, chunk):
+    """psiformer64 at its 1024 walkers in chunks of 256 and ferminet16 at its 4096: finite
+    results, walkers independent of the batch they are evaluated in, deterministic."""
+    forward, p, cfg, B, sigma, thr = wl.build(name)
+    p = wl.to_device(p, torch.device('cuda'))
+    x = wl.sample_electrons(B, cfg.n_elec, sigma, seed=2)
+    fl = folx_amd.forward_laplacian(lambda t: forward(p, t), thr)
+    print(f'case {name} full batch {B} in chunks of {chunk}', flush=True)
+    full = folx_amd.batched_vmap(fl, chunk)(x)
+    P = 3 * cfg.n_elec
+    assert full.x.shape == (B,) and full.jacobian.dense_array.shape == (P, B)
+    assert torch.isfinite(full.x).all() and torch.isfinite(full.laplacian).all()
+    assert torch.isfinite(full.jacobian.dense_array).all()
+    idx = [0, chunk - 1, chunk, B - 1]
+    small = folx_amd.vmap(fl)(x[idx])
+    # single walkers inside the big batch = the same walkers in a batch of 4, up to the noise floor of
+    # log|det| (different tile shapes change the summation order in front of an ill-conditioned determinant)
+    r64 = forward(wl.build(name)[1], ob.init_state(x[idx], dtype=np.float64), ob)
+    r32 = forward(wl.build(name)[1], ob.init_state(x[idx], dtype=np.float32), ob)
+    for a, b, a64, a32, nm in ((full.x[idx], small.x, r64.x, r32.x, 'x'),
+                               (full.jacobian.dense_array[:, idx], small.jacobian.dense_array, r64.J, r32.J, 'jacobian'),
+                               (full.laplacian[idx], small.laplacian, r64.lap, r32.lap, 'laplacian')):
+        floor = np.abs(a32.astype(np.float64) - a64).max()
+        scale = np.abs(a64).max()
+        d = (a.double() - b.double()).abs().max().item()
+        e = np.abs(a.double().cpu().numpy() - a64).max()
+        print(f'{name} {nm}: |big - small| = {d / scale:.2e}, |big - fp64| = {e / scale:.2e}, fp32 floor {floor / scale:.2e}', flush=True)
+        assert d <= max(2.0 * floor, 1e-5 * scale), (nm, d, floor)
+        assert e <= max(2.0 * floor, 1e-5 * scale), (nm, e, floor)
+    again = folx_amd.batched_vmap(fl, chunk)(x)
+    assert torch.equal(again.x, full.x) and torch.equal(again.laplacian, full.laplacian)
