@@ -32,6 +32,7 @@ SIGNATURES = {
                                    + [c_int64, c_int32, c_int32, c_int32, _P, c_int64]),
     'folx_hip_norm_dense_static_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 5 + [c_float] + [_P] * 5
                                           + [c_int64, c_int32, c_int32, c_int32]),
+    'folx_hip_dot_two_fwdlap': (c_int, [_P] * 10 + [c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, _P]),
     'folx_hip_layernorm_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_float]),
     'folx_hip_elementwise_fwdlap': (c_int, [_P, c_int32, c_float, _P, _P, _P, _P, _P, _P, c_int64, c_int32]),
     'folx_hip_exp_envelope_fwdlap': (c_int, [_P] * 9 + [c_int64, c_int32, c_int32, c_int32]),

@@ -24,6 +24,7 @@ SOURCES = [
     'dense.hip',
     'dense_act.hip',
     'dense_act_wide.hip',
+    'dot_two.hip',
     'pointwise.hip',
     'reduce.hip',
     'gather.hip',

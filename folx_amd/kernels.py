@@ -260,6 +260,45 @@ def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):
     return y, yj, yl
 
 
+DOT_TWO_KMAX = 128
+
+
+def dot_two(a, aj, al, b, bj, bl):
+    """Batched product of two triplets: a (NB0, NB1, I, Kc), b (NB0, NB1, Kc, J), Jacobians with a
+    leading row axis (P, ...), all float32 on the GPU.  The operands may be VIEWS (transposed,
+    sliced, head-interleaved): the kernel addresses them through their strides; only the
+    Jacobians must share the strides of their values.  Returns contiguous y (NB0, NB1, I, J),
+    y_jac (P, NB0, NB1, I, J), y_lap."""
+    for t in (a, aj, al, b, bj, bl):
+        assert t.is_cuda and t.dtype == torch.float32
+    NB0, NB1, I, Kc = a.shape
+    J = b.shape[-1]
+    P = aj.shape[0]
+    assert tuple(b.shape) == (NB0, NB1, Kc, J) and tuple(aj.shape) == (P, *a.shape) and tuple(bj.shape) == (P, *b.shape)
+    assert al.shape == a.shape and bl.shape == b.shape and Kc <= DOT_TWO_KMAX
+
+    def same_layout(t, u_strides):  # u is addressed with t's strides
+        return all(st == su for st, su, n in zip(t.stride(), u_strides, t.shape) if n > 1)
+
+    assert (same_layout(a, al.stride()) and same_layout(b, bl.stride())
+            and (P == 0 or (same_layout(a, aj.stride()[1:]) and same_layout(b, bj.stride()[1:])))), \
+        'dot_two: value, Laplacian and Jacobian rows of an operand must share one layout'
+    y = torch.empty((NB0, NB1, I, J), device=a.device, dtype=torch.float32)
+    yj = torch.empty((P, NB0, NB1, I, J), device=a.device, dtype=torch.float32)
+    yl = torch.empty_like(y)
+    strides = (ctypes.c_int64 * 10)(*a.stride(), aj.stride(0) if P else 0, b.stride(0), b.stride(1), b.stride(2),
+                                    b.stride(3), bj.stride(0) if P else 0)
+    with _timed('dot_two_fwdlap', (NB0 * NB1, I, J, Kc, P)):
+        check(
+            _lib.load().folx_hip_dot_two_fwdlap(
+                _stream(), _p(a), _p(aj), _p(al), _p(b), _p(bj), _p(bl), _p(y), _p(yj), _p(yl),
+                NB0, NB1, I, J, Kc, P, strides,
+            ),
+            'dot_two_fwdlap',
+        )
+    return y, yj, yl
+
+
 def elementwise(name, x, jac, lap, param=0.0, inplace=False):
     _chk(x, jac, lap)
     P = jac.shape[0]
@@ -360,6 +399,14 @@ def binary(op, a, aj, al, b, bj, bl):
     P = aj.shape[0]
     assert bj.shape[0] == P
     out_shape = torch.broadcast_shapes(a.shape, b.shape)
+    # the kernel addresses an operand's Jacobian rows with the strides of its values: rows that were
+    # re-indexed at the full output shape take their (smaller) value and Laplacian arrays along
+    if tuple(aj.shape[1:]) != tuple(a.shape):
+        assert tuple(aj.shape[1:]) == tuple(out_shape), (aj.shape, a.shape, out_shape)
+        a, al = a.expand(out_shape).contiguous(), al.expand(out_shape).contiguous()
+    if tuple(bj.shape[1:]) != tuple(b.shape):
+        assert tuple(bj.shape[1:]) == tuple(out_shape), (bj.shape, b.shape, out_shape)
+        b, bl = b.expand(out_shape).contiguous(), bl.expand(out_shape).contiguous()
     col = collapse3(out_shape, bstrides(a.shape, out_shape), bstrides(b.shape, out_shape))
     if col is None:
         a, aj, al = (t.expand(*t.shape[: t.dim() - a.dim()], *out_shape).contiguous() for t in (a, aj, al))

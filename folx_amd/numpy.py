@@ -149,6 +149,46 @@ def matmul(a, b):
     return np.matmul(a, b)
 
 
+def einsum(subscripts: str, a, b):
+    """Two-operand ``numpy.einsum`` (explicit ``->`` form, no repeated index inside an operand, no
+    ellipsis) lowered to transposes and one ``matmul``: indices shared by both operands and the
+    output are batch axes, shared ones missing from the output are contracted, the others are
+    the free axes of their operand -- the dimension numbers ``jnp.einsum`` hands to
+    ``dot_general`` (folx/wrapped_functions.py:174-309)."""
+    ins, out = subscripts.replace(' ', '').split('->')
+    sa, sb = ins.split(',')
+    assert len(set(sa)) == len(sa) and len(set(sb)) == len(sb) and '.' not in subscripts, subscripts
+    for idx, t in ((sa, a), (sb, b)):  # indices of one operand only that the output drops are summed first
+        drop = [i for i, c in enumerate(idx) if c not in out and c not in (sb if idx is sa else sa)]
+        if drop:
+            red = sum(t, axis=tuple(drop))
+            kept = ''.join(c for i, c in enumerate(idx) if i not in drop)
+            if idx is sa:
+                a, sa = red, kept
+            else:
+                b, sb = red, kept
+    batch = [c for c in sa if c in sb and c in out]
+    contract = [c for c in sa if c in sb and c not in out]
+    fa = [c for c in sa if c not in sb]
+    fb = [c for c in sb if c not in sa]
+    dim = {c: n for idx, t in ((sa, a), (sb, b)) for c, n in zip(idx, _shape(t))}
+    size = lambda cs: int(np.prod([dim[c] for c in cs], dtype=np.int64))
+    at = transpose(a, [sa.index(c) for c in batch + fa + contract])
+    bt = transpose(b, [sb.index(c) for c in batch + contract + fb])
+    bshape = [dim[c] for c in batch]
+    y = matmul(reshape(at, (*bshape, size(fa), size(contract))), reshape(bt, (*bshape, size(contract), size(fb))))
+    y = reshape(y, (*bshape, *[dim[c] for c in fa], *[dim[c] for c in fb]))
+    cur = batch + fa + fb
+    return y if cur == list(out) else transpose(y, [cur.index(c) for c in out])
+
+
+def softmax(a, axis=-1):
+    """``jax.nn.softmax``: the shift by the maximum is a constant (stop_gradient), then exp, sum
+    and div through their rules."""
+    e = exp(subtract(a, amax_const(a, axis, keepdims=True)))
+    return divide(e, sum(e, axis, keepdims=True))
+
+
 def slogdet(A, row_axis=None, factor=None):
     """``numpy.linalg.slogdet`` over the last two axes; ``row_axis`` names another axis as the
     one holding the matrix rows (columns stay on the last axis, all other axes are batch axes

@@ -607,16 +607,51 @@ def _dot_then_act(h, W, kwargs, thr: int):
 
 def _dot_two_operands(lhs: FwdLaplArray, rhs: FwdLaplArray, thr: int) -> FwdLaplArray:
     """Matrix product of two derivative-carrying operands with ``numpy.matmul`` shapes,
-    ``lhs (..., i, k) @ rhs (..., k, j)`` (1-D operands as in matmul).  Both operands are
-    rearranged so that the contracted axis is last and broadcast against each other, then
-    multiplied and summed -- the decomposition the reference takes for this case
-    (``rearrange`` + ``mul_sum``, folx/wrapped_functions.py:47-68, :253-286); the rules of
-    ``mul`` (JVP both ways + 2 tr(J_l J_r^T), folx/hessian.py:177-188) and ``reduce_sum``
-    then give the triplet."""
+    ``lhs (..., i, k) @ rhs (..., k, j)`` (1-D operands as in matmul).
+
+    Dense Jacobians (or sparse ones for which the reference takes its general path): ONE rule,
+    ``kernels.dot_two`` -- JVP both ways plus the DOT_PRODUCT Hessian term 2 tr(J_l J_r^T)
+    (folx/wrapped_functions.py:294-309, folx/hessian.py:177-188) as batched matrix products;
+    the (..., i, j, k) intermediate is never formed.
+
+    Both operands sparse and the product's sparse Jacobian cheaper than the dense ones (the cost
+    gate of folx/wrapped_functions.py:253-262): the reference's ``rearrange`` + ``mul_sum``
+    decomposition (:47-68, :263-286) through the ``mul`` and ``reduce_sum`` rules, which keeps
+    the result sparse."""
+    a_vec, b_vec = lhs.ndim == 1, rhs.ndim == 1
+    la = (1, lhs.shape[0]) if a_vec else tuple(lhs.shape)
+    rb = (rhs.shape[0], 1) if b_vec else tuple(rhs.shape)
+    assert la[-1] == rb[-2], f'matmul: contracting {tuple(lhs.shape)} with {tuple(rhs.shape)}'
+    same_batch = la[:-2] == rb[:-2]
+    use_mul_sum = not same_batch or la[-1] > K.DOT_TWO_KMAX
+    if same_batch and lhs.jacobian.weak and rhs.jacobian.weak:
+        inter = int(np.prod((*la, rb[-1]), dtype=np.int64))
+        in_size = max(int(np.prod(la, dtype=np.int64)), int(np.prod(rb, dtype=np.int64)))
+        k_mul = lhs.jacobian.data.shape[0] + rhs.jacobian.data.shape[0]
+        n_dense = max(lhs.jacobian.max_n, rhs.jacobian.max_n) + 1
+        use_mul_sum = use_mul_sum or inter == in_size or k_mul * inter < n_dense * in_size
+    if use_mul_sum:
+        return _dot_mul_sum(lhs, rhs, a_vec, b_vec)
+    Ja, Jb = lhs.jacobian.dense_array, rhs.jacobian.dense_array
+    P = max(Ja.shape[0], Jb.shape[0])
+    Ja, Jb = so.pad_rows(Ja, P), so.pad_rows(Jb, P)
+    B = lhs.B
+    NB0 = B * int(np.prod(la[:-2], dtype=np.int64))
+    va = lambda t, lead: t.reshape(*lead, NB0, 1, la[-2], la[-1])
+    vb = lambda t, lead: t.reshape(*lead, NB0, 1, rb[-2], rb[-1])
+    y, Jy, lapy = K.dot_two(va(lhs.x.contiguous(), ()), va(Ja.contiguous(), (P,)), va(lhs.laplacian.contiguous(), ()),
+                            vb(rhs.x.contiguous(), ()), vb(Jb.contiguous(), (P,)), vb(rhs.laplacian.contiguous(), ()))
+    out_shape = (*la[:-2], *(() if a_vec else (la[-2],)), *(() if b_vec else (rb[-1],)))
+    return FwdLaplArray(y.reshape(B, *out_shape), FwdJacobian(Jy.reshape(P, B, *out_shape), None),
+                        lapy.reshape(B, *out_shape))
+
+
+def _dot_mul_sum(lhs: FwdLaplArray, rhs: FwdLaplArray, a_vec: bool, b_vec: bool) -> FwdLaplArray:
+    """Both operands are rearranged so that the contracted axis is last and broadcast against
+    each other, then multiplied and summed (folx/wrapped_functions.py:47-68, :263-286)."""
     from . import numpy as fnp
 
     a, b = lhs, rhs
-    a_vec, b_vec = a.ndim == 1, b.ndim == 1
     if a_vec:
         a = fnp.expand_dims(a, 0)
     if b_vec:

@@ -243,6 +243,29 @@ int folx_hip_norm_dense_static_fwdlap(void* stream, int32_t act, float param, co
                                       int64_t R, int32_t P, int32_t K, int32_t N);
 
 /*
+ * Matrix product of two operands that both carry derivatives, for a batch of NB0 * NB1 matrix
+ * pairs a (I x Kc), b (Kc x J) with dense Jacobians on the same P rows:
+ *   y = a b,   y_jac[p] = a_jac[p] b + a b_jac[p],
+ *   y_lap = a_lap b + a b_lap + 2 sum_p a_jac[p] b_jac[p].
+ * Replaces the two-operand paths of dot_general (folx/wrapped_functions.py:205-309: rearrange
+ * :47-68 + the dot_last einsum :294-309 under dense_split_jvp, folx/jvp.py:676-684) with the
+ * DOT_PRODUCT Hessian term 2 tr(J_l J_r^T) (dot_product_jac_hessian_jac, folx/hessian.py:177-188);
+ * the (batch, i, j, k) broadcast intermediate of that path is never formed.
+ * Operands are addressed through element strides (HOST array of 10 non-negative values):
+ *   strides = {a_sb0, a_sb1, a_si, a_sk, a_sp,  b_sb0, b_sb1, b_sk, b_sj, b_sp}
+ *   a(b0, b1, i, k) at a[b0 a_sb0 + b1 a_sb1 + i a_si + k a_sk], likewise a_lap; Jacobian row p
+ *   adds p * a_sp.  b(b0, b1, k, j) at b[b0 b_sb0 + b1 b_sb1 + k b_sk + j b_sj], rows p * b_sp.
+ * so that transposed operands (q k^T) and head-interleaved layouts ([walker][electron][head][d]
+ * read as batch (walker, head)) need no copy.  Outputs are contiguous:
+ *   y, y_lap [NB0][NB1][I][J]   y_jac [P][NB0][NB1][I][J].
+ * Built for Kc <= 128 (FOLX_HIP_ENOTSUP beyond; the caller then multiplies and sums).
+ */
+int folx_hip_dot_two_fwdlap(void* stream, const float* a, const float* a_jac, const float* a_lap,
+                            const float* b, const float* b_jac, const float* b_lap, float* y,
+                            float* y_jac, float* y_lap, int64_t NB0, int32_t NB1, int32_t I,
+                            int32_t J, int32_t Kc, int32_t P, const int64_t* strides);
+
+/*
  * Binary elementwise rule for two operands whose Jacobians live on the same row frame
  * (both dense with P rows, or sparse with identical index masks).  The output index
  * space is (n0, n1, n2), row-major; each operand addresses it with element strides

@@ -521,8 +521,8 @@ def logsumexp(a: OArr, axis=-1, b=None):
 
 
 def matmul(a, b):
-    """numpy.matmul semantics; two triplets go through multiply + sum like the reference's
-    mul_sum decomposition (folx/wrapped_functions.py:253-286)."""
+    """numpy.matmul semantics; two triplets go through ``rules.dot_two_rule`` (the dot_last
+    path of the reference, folx/wrapped_functions.py:294-309)."""
     if _is(a) and not _is(b):
         return dot(a, b)
     if _is(a) and _is(b):
@@ -531,8 +531,10 @@ def matmul(a, b):
             a = expand_dims(a, 0)
         if bv:
             b = expand_dims(b, 1)
-        bt = swapaxes(b, -1, -2)
-        out = sum(multiply(expand_dims(a, -2), expand_dims(bt, -3)), axis=-1)
+        Ja, Jb = _padJ(a, b)
+        lead = np.broadcast_shapes(a.x.shape[:-2], b.x.shape[:-2])
+        bc = lambda t, off: np.broadcast_to(t, (*t.shape[:off], *lead, *t.shape[-2:]))
+        out = OArr(*rules.dot_two_rule(bc(a.x, 0), bc(Ja, 1), bc(a.lap, 0), bc(b.x, 0), bc(Jb, 1), bc(b.lap, 0)))
         if bv:
             out = squeeze(out, -1)
         if av:
@@ -541,6 +543,29 @@ def matmul(a, b):
     bt = swapaxes(b, -1, -2) if b.ndim > 1 else b
     out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
     return swapaxes(out, -1, -2) if out.ndim > 1 else out
+
+
+def einsum(subscripts, a, b):
+    """Two-operand einsum of triplets, evaluated directly: linear in each operand, Hessian term
+    2 sum_p einsum(Ja_p, Jb_p) (folx/hessian.py:177-188)."""
+    ins, out = subscripts.replace(' ', '').split('->')
+    sa, sb = ins.split(',')
+    if not _is(a) or not _is(b):
+        t, c, tfirst = (a, np.asarray(b), True) if _is(a) else (b, np.asarray(a), False)
+        st, sc = (sa, sb) if tfirst else (sb, sa)
+        f = lambda v, lead: np.einsum(f'{lead}{st},{sc}->{lead}{out}', v, c)
+        return OArr(f(t.x, 'Z'), f(t.J, 'YZ'), f(t.lap, 'Z'))
+    Ja, Jb = _padJ(a, b)
+    e = lambda u, lu, v, lv, lo: np.einsum(f'{lu}{sa},{lv}{sb}->{lo}{out}', u, v)
+    x = e(a.x, 'Z', b.x, 'Z', 'Z')
+    J = e(Ja, 'YZ', b.x, 'Z', 'YZ') + e(a.x, 'Z', Jb, 'YZ', 'YZ')
+    lap = e(a.lap, 'Z', b.x, 'Z', 'Z') + e(a.x, 'Z', b.lap, 'Z', 'Z') + 2.0 * e(Ja, 'YZ', Jb, 'YZ', 'Z')
+    return OArr(x, J, lap)
+
+
+def softmax(a: OArr, axis=-1):
+    e = exp(subtract(a, amax_const(a, axis, keepdims=True)))
+    return divide(e, sum(e, axis, keepdims=True))
 
 
 def det(A: OArr):

@@ -268,6 +268,20 @@ def dense_rule(x, J, lap, W, b=None):
     return y, J @ W, lap @ W
 
 
+def dot_two_rule(a, Ja, La, b, Jb, Lb):
+    """y = a @ b over the last two axes with BOTH operands carrying derivatives (dense Jacobians
+    on the same rows): the product is linear in each operand (JVP both ways,
+    folx/jvp.py:676-684) and its Hessian couples the two operands through the identity, so
+    tr(J^T H J) = 2 sum_p Ja_p @ Jb_p (dot_product_jac_hessian_jac, folx/hessian.py:177-188,
+    for the dot_last einsum of folx/wrapped_functions.py:294-309).
+    Pinned by AD Hessian traces in tests/test_oracle_rules.py and by equality with the
+    multiply-and-sum decomposition (mul_rule + sum_rule)."""
+    y = a @ b
+    Jy = Ja @ b[None] + a[None] @ Jb
+    lap = La @ b + a @ Lb + 2.0 * np.einsum('p...ik,p...kj->...ij', Ja, Jb)
+    return y, Jy, lap
+
+
 # --------------------------------------------------------------------------------------
 # Binary elementwise rules with both operands carrying derivatives (dense Jacobians).
 # --------------------------------------------------------------------------------------

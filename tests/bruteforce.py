@@ -170,6 +170,15 @@ class plain:
         return a @ b
 
     @staticmethod
+    def einsum(subscripts, a, b):
+        a, b = plain._b(a, b)
+        return torch.einsum(subscripts, a, b)
+
+    @staticmethod
+    def softmax(a, axis=-1):
+        return torch.softmax(a, dim=axis)
+
+    @staticmethod
     def det(A):
         n = A.shape[-1]
         if n == 1:

@@ -63,6 +63,10 @@ def norm_dense(name, x, jac, lap, gamma, beta, eps, W, bias=None, param=0.0):
     return dense_act(name, *n, W, bias, param)
 
 
+def dot_two(a, aj, al, b, bj, bl):
+    return tuple(_t(t) for t in rules.dot_two_rule(_n(a), _n(aj), _n(al), _n(b), _n(bj), _n(bl)))
+
+
 def exp_envelope(d, dj, dl, sigma, pi):
     from oracle import backend as ob
 
@@ -242,7 +246,7 @@ def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
                                                 _n(v), dense(vs), _n(vl)))
 
 
-KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
+KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
                 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_cols', 'scatter_add_rows',
                 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
 

@@ -26,7 +26,7 @@ from tolerances import LAP_ATOL, LAP_ATOL_REL, LAP_RTOL, VAL_ATOL_REL, VAL_RTOL
 
 NOISE = 2.0 ** -22  # relative size of the input perturbation that measures a rule's own sensitivity
 
-_TRIPLETS = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
+_TRIPLETS = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
              'mul_sparse', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
 _SINGLE = ('rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_cols', 'scatter_add_rows')
 _DETS = ('slogdet', 'sparse_slogdet')

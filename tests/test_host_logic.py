@@ -276,7 +276,21 @@ MATMUL_FNS = {
     'attn_like': lambda xp, x: xp.matmul(xp.exp(xp.multiply(xp.matmul(x, xp.swapaxes(x, -1, -2)), 0.1)), x),
     'vec_mat': lambda xp, x: xp.matmul(xp.getitem(x, (0,)), xp.swapaxes(xp.cos(x), -1, -2)),  # (3,)@(3,4)
     'const_left': lambda xp, x: xp.matmul(np.arange(8.0).reshape(2, 4) / 8, xp.tanh(x)),      # (2,4)@(4,3)
+    # test/test_layers.py:141-171: attention and a rectangular product of two functions of x
+    'attn': lambda xp, x: xp.matmul(xp.exp(xp.matmul(xp.multiply(x, 0.3), xp.swapaxes(x, -2, -1))), x),
+    'rect': lambda xp, x: xp.matmul(xp.sin(x), xp.cos(xp.swapaxes(x, -2, -1))),
+    # test/test_layers.py:173-206: einsums with degenerate broadcast dimensions
+    'ein_n1': lambda xp, x: xp.einsum('nk,mk->nm', x, xp.sin(xp.getitem(x, (slice(0, 1),)))),
+    'ein_1n': lambda xp, x: xp.einsum('nk,mk->nm', xp.getitem(x, (slice(0, 1),)), xp.sin(x)),
+    'ein_vec': lambda xp, x: xp.einsum('k,mk->m', xp.getitem(x, (0,)), xp.sin(xp.getitem(x, (slice(0, 3),)))),
+    'ein_mpnn': lambda xp, x: xp.einsum('ijh,jh->ih', xp.sin(xp.multiply(xp.expand_dims(x, 1), xp.expand_dims(x, 0))),
+                                        xp.cos(x)),
+    # test/test_composite.py:45-83: softmax attention from three projections, summed
+    'softmax_attn': lambda xp, x: xp.sum(xp.matmul(
+        xp.softmax(xp.matmul(xp.dot(x, _ATT_W[0]), xp.swapaxes(xp.dot(x, _ATT_W[1]), -1, -2)), axis=-1),
+        xp.dot(x, _ATT_W[2]))),
 }
+_ATT_W = [np.random.default_rng(40 + i).normal(size=(3, 8)).astype(np.float32) / 2 for i in range(3)]
 
 
 @pytest.mark.parametrize('name', sorted(MATMUL_FNS))

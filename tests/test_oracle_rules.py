@@ -308,3 +308,40 @@ def test_mhsea_vs_bruteforce(n, H, d, valid):
     _close(out.x[:, m], by[:, m], atol=1e-9)
     _close(out.J[:, :, m], bJ[:, :, m], atol=1e-9)
     _close(out.lap[:, m], bL[:, m], rtol=1e-5, atol=1e-8)
+
+
+def test_dot_two_rule_vs_autograd_and_mul_sum():
+    """rules.dot_two_rule: (i) equals the multiply-and-sum decomposition built from mul_rule and
+    sum_rule (both pinned by AD above), (ii) the Hessian trace of u(x) @ v(x) by torch AD."""
+    import torch
+
+    rng = np.random.default_rng(3)
+    P, B, I, Kc, J = 5, 2, 3, 4, 6
+    a, La, b, Lb = (rng.normal(size=s) for s in ((B, I, Kc), (B, I, Kc), (B, Kc, J), (B, Kc, J)))
+    Ja, Jb = rng.normal(size=(P, B, I, Kc)), rng.normal(size=(P, B, Kc, J))
+    y, Jy, ly = rules.dot_two_rule(a, Ja, La, b, Jb, Lb)
+    bt = np.swapaxes
+    m = rules.mul_rule(a[:, :, None, :], Ja[:, :, :, None, :], La[:, :, None, :],
+                       bt(b, -1, -2)[:, None], bt(Jb, -1, -2)[:, :, None], bt(Lb, -1, -2)[:, None])
+    sy, sJ, sl = rules.sum_rule(*m, axes=(2,))
+    np.testing.assert_allclose(y, sy, rtol=1e-12)
+    np.testing.assert_allclose(Jy, sJ, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(ly, sl, rtol=1e-12, atol=1e-12)
+    # AD: f(x) = tanh(x A) @ sin(x C) for x in R^5, with the operands' triplets from the chain rule
+    n = 5
+    A, C = rng.normal(size=(n, I * Kc)), rng.normal(size=(n, Kc * J))
+    x = torch.tensor(rng.normal(size=n), dtype=torch.float64)
+    At, Ct = torch.tensor(A), torch.tensor(C)
+    u = lambda t: torch.tanh(t @ At).reshape(I, Kc)
+    v = lambda t: torch.sin(t @ Ct).reshape(Kc, J)
+    f = lambda t: (u(t) @ v(t)).reshape(-1)
+    jac = lambda g: torch.autograd.functional.jacobian(g, x)
+    hess_tr = lambda g, m_: torch.stack([torch.autograd.functional.hessian(lambda t: g(t).reshape(-1)[i], x).trace()
+                                         for i in range(m_)])
+    tri = lambda g, shp: (g(x).numpy()[None], np.moveaxis(jac(lambda t: g(t).reshape(-1)).numpy(), -1, 0).reshape(n, 1, *shp),
+                          hess_tr(g, int(np.prod(shp))).numpy().reshape(1, *shp))
+    ua, vb = tri(u, (I, Kc)), tri(v, (Kc, J))
+    got = rules.dot_two_rule(*ua, *vb)
+    want = tri(lambda t: u(t) @ v(t), (I, J))
+    for g_, w_ in zip(got, want):
+        np.testing.assert_allclose(g_, w_, rtol=1e-9, atol=1e-10)
