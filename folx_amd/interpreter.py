@@ -45,6 +45,19 @@ def init_forward_laplacian_state(x: torch.Tensor, sparsity: bool, weights=None) 
     return FwdLaplArray(x, FwdJacobian(data, None), lap)
 
 
+def _force_tree(out):
+    """Evaluate whatever the function returned unevaluated (``wrapped_functions.Deferred``)."""
+    from .wrapped_functions import Deferred
+
+    if isinstance(out, Deferred):
+        return out.value()
+    if isinstance(out, (tuple, list)):
+        return type(out)(_force_tree(t) for t in out)
+    if isinstance(out, dict):
+        return {k: _force_tree(v) for k, v in out.items()}
+    return out
+
+
 class ForwardLaplacianFn:
     """Callable returned by ``forward_laplacian``.  ``f(x)`` treats ``x`` as ONE sample of
     shape ``shape`` (the reference's un-vmapped call); ``f.batched(x)`` takes
@@ -82,7 +95,7 @@ class ForwardLaplacianFn:
             else:
                 lapl_args.append(a)
         with fnp.sparsity_threshold(thr):
-            return self.fn(*lapl_args, **kwargs)
+            return _force_tree(self.fn(*lapl_args, **kwargs))
 
     def __call__(self, *args, weights=None, **kwargs):
         lifted = []

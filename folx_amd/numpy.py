@@ -35,11 +35,27 @@ def sparsity_threshold(value: int):
 
 
 def _call(name, args, kwargs=None):
+    """Look the rule up and call it.  Deferred values among the arguments are evaluated first
+    (also one level inside tuples and among the keyword values): only the functions below that
+    know how to absorb one hand it on, through ``_call_keep``."""
+    from .wrapped_functions import force
+
+    kwargs = {k: force(v) for k, v in (kwargs or {}).items()}
+    return get_laplacian(name, wrap_if_missing=True)(tuple(force(a) for a in args), kwargs, current_threshold())
+
+
+def _call_keep(name, args, kwargs=None):
     return get_laplacian(name, wrap_if_missing=True)(tuple(args), kwargs or {}, current_threshold())
 
 
+def _is_triplet(a):
+    from .wrapped_functions import Deferred
+
+    return isinstance(a, (FwdLaplArray, Deferred))
+
+
 def _shape(a):
-    if isinstance(a, (FwdLaplArray, BatchedArray)):
+    if isinstance(a, BatchedArray) or _is_triplet(a):
         return tuple(a.shape)
     return tuple(np.shape(a))
 
@@ -47,6 +63,11 @@ def _shape(a):
 # elementwise -------------------------------------------------------------------------------
 def _u(name):
     def fn(a):
+        from .kernels import FUSED_ACTS
+        from .wrapped_functions import LazyDot
+
+        if isinstance(a, LazyDot) and name in FUSED_ACTS and a.kwargs.get('act') is None:
+            return a.with_(act=name)  # Dense + activation: one rule where the kernels take the shape
         return _call(name, (a,))
 
     fn.__name__ = name
@@ -81,6 +102,19 @@ def power(a, c):
 
 
 def add(a, b):
+    from .wrapped_functions import LazyDot, force
+
+    for d, o in ((b, a), (a, b)):
+        if not isinstance(d, LazyDot) or d._value is not None:  # an evaluated product is an ordinary triplet
+            continue
+        if not _is_triplet(o) and not isinstance(o, BatchedArray):
+            # a constant vector along the feature axis in front of the activation: the bias
+            if (d.kwargs.get('act') is None and d.kwargs.get('bias') is None and np.ndim(o) == 1
+                    and _shape(o) == (d.shape[-1],)):
+                return d.with_(bias=o)
+        elif _is_triplet(o) and tuple(o.shape) == tuple(d.shape):
+            return d.value_with_residual(force(o))  # skip connection: added in the product's epilogue
+        break
     return _call('add', (a, b))
 
 
@@ -89,6 +123,10 @@ def subtract(a, b):
 
 
 def multiply(a, b):
+    from .wrapped_functions import LazyMul, force
+
+    if _is_triplet(a) and _is_triplet(b) and tuple(a.shape) == tuple(b.shape) and len(a.shape) >= 2:
+        return LazyMul(force(a), force(b), current_threshold())  # slogdet can take the factor on load
     return _call('mul', (a, b))
 
 
@@ -98,32 +136,46 @@ def divide(a, b):
 
 # linear algebra ----------------------------------------------------------------------------
 def dot(h, W, b=None, residual=None, row_slice=None, act=None, norm=None):
-    """``h @ W (+ b) (+ residual)``: last axis of ``h`` against the first axis of the
-    constant ``W``; ``residual`` is a triplet of the output shape (skip connection).
-    ``row_slice = (lo, hi)`` computes ``h[..., lo:hi, :] @ W`` without copying the slice.
-    ``act`` names a scalar function applied to ``h @ W + b`` (the residual is then added to
-    the activated result): a Dense + activation layer runs as one rule.
-    ``norm = (gamma, beta, eps)`` applies ``layer_norm`` to ``h`` first, inside the same rule
-    where the kernels allow it."""
-    from .wrapped_functions import LazyLayerNorm
+    """``h @ W``: last axis of ``h`` against the first axis of the constant ``W``.
+
+    Written plainly, ``tanh(dot(layer_norm(h, g, be), W) + bias) + skip`` runs as ONE rule where
+    the kernels take the shape: ``dot`` absorbs a ``layer_norm``, a ``concatenate`` along the
+    feature axis or a slice of rows in front of it, and returns a deferred value that absorbs the
+    bias, the activation and the skip connection that follow (``wrapped_functions.Deferred``).
+
+    The keyword form states the same fusion explicitly and evaluates at once: ``b`` bias,
+    ``residual`` a triplet of the output shape, ``row_slice = (lo, hi)`` for
+    ``h[..., lo:hi, :] @ W``, ``act`` a scalar function applied to ``h @ W + b`` (the residual is
+    added to the activated result), ``norm = (gamma, beta, eps)`` a LayerNorm of ``h``."""
+    from .wrapped_functions import LazyConcat, LazyDot, LazyLayerNorm, LazySlice, force
 
     if isinstance(h, LazyLayerNorm):
         assert norm is None, 'dot: the operand already is a layer_norm'
         h, norm = h.h, h
-    return _call('dot_general', (h, W),
-                 {'bias': b, 'residual': residual, 'row_slice': row_slice, 'act': act, 'norm': norm})
+    elif isinstance(h, LazySlice) and row_slice is None and h.ndim >= 2 and h.axis == h.ndim - 2:
+        h, row_slice = h.a, (h.lo, h.hi)
+    elif not isinstance(h, LazyConcat):
+        h = force(h)
+    kwargs = {'bias': b, 'row_slice': row_slice, 'act': act, 'norm': norm}
+    explicit = residual is not None or act is not None
+    if explicit or not _is_triplet(h) or _is_triplet(W) or np.ndim(W) != 2:
+        return _call_keep('dot_general', (h, force(W)), {**kwargs, 'residual': force(residual)})
+    lead = tuple(h.shape[:-1])
+    if row_slice is not None:
+        lead = (*lead[:-1], row_slice[1] - row_slice[0])
+    return LazyDot(h, W, kwargs, (*lead, int(np.shape(W)[1])), current_threshold())
 
 
-def layer_norm(h, gamma=None, beta=None, eps=1e-5, lazy=False):
-    """LayerNorm over the last axis (one fused rule; same result as the primitive chain).
-    ``lazy=True`` returns a handle that only ``dot`` accepts as its first operand: products
-    that can take LayerNorm into their own rule never evaluate it, the others share one
-    evaluation."""
-    from .api import FwdLaplArray as _F
-    from .wrapped_functions import LazyLayerNorm
+def layer_norm(h, gamma=None, beta=None, eps=1e-5, lazy=True):
+    """LayerNorm over the last axis (one fused rule; same result as the primitive chain).  The
+    result is deferred: products that can take LayerNorm into their own rule never evaluate it,
+    all other consumers share one evaluation."""
+    from .wrapped_functions import LazyLayerNorm, force
 
-    if lazy and isinstance(h, _F):
-        return LazyLayerNorm(h, gamma, beta, eps)
+    del lazy
+    h = force(h)
+    if isinstance(h, FwdLaplArray):
+        return LazyLayerNorm(h, gamma, beta, eps, current_threshold())
     return _call('layer_norm', (h, gamma, beta), {'eps': eps})
 
 
@@ -136,13 +188,11 @@ def exp_envelope(d, sigma, pi):
 
 def matmul(a, b):
     """``numpy.matmul`` for two operands of which at least one carries derivatives."""
-    from .api import FwdLaplArray as _F
-
-    if isinstance(a, _F) and not isinstance(b, _F) and len(_shape(b)) == 2:
+    if _is_triplet(a) and not _is_triplet(b) and len(_shape(b)) == 2:
         return dot(a, b)
-    if isinstance(a, _F) and isinstance(b, _F):
+    if _is_triplet(a) and _is_triplet(b):
         return _call('dot_general', (a, b), {})
-    if isinstance(b, _F):  # constant @ triplet = (triplet^T @ constant^T)^T
+    if _is_triplet(b):  # constant @ triplet = (triplet^T @ constant^T)^T
         bt = swapaxes(b, -1, -2) if len(_shape(b)) > 1 else b
         out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
         return swapaxes(out, -1, -2) if len(_shape(out)) > 1 else out
@@ -196,6 +246,12 @@ def slogdet(A, row_axis=None, factor=None):
     in place.  ``factor`` (same shape as ``A``): the matrices are ``A * factor``; orbitals times
     envelopes are then multiplied while the matrices are loaded.  Same result as
     ``slogdet(multiply(A, factor))``."""
+    from .wrapped_functions import LazyMul, LazyTranspose
+
+    if isinstance(A, LazyTranspose) and row_axis is None and factor is None:
+        A, row_axis = A.a, A.row_axis       # matrix rows on another axis: read in place
+    if isinstance(A, LazyMul) and factor is None:
+        A, factor = A.a, A.b                # slogdet(A * F): the product is formed while the matrices are loaded
     return _call('slogdet', (A,), {'row_axis': row_axis, 'factor': factor})
 
 
@@ -253,9 +309,19 @@ def _axes(axis, nd):
 def sum(a, axis=None, keepdims=False, window=None):
     """``window = (lo, hi)`` with a single ``axis``: the sum of ``a[..., lo:hi, ...]`` along that
     axis, without forming the slice."""
+    from .wrapped_functions import LazySlice
+
+    if isinstance(a, LazySlice) and window is None and _axes(axis, a.ndim) == (a.axis,):
+        a, window = a.a, (a.lo, a.hi)       # the sum of a slice along the reduced axis: read in place
+        shape = _shape(a)
+        axes = _axes(axis, len(shape))
+        out = _call('reduce_sum', (a,), {'axes': axes, 'window': tuple(window)})
+        if keepdims:
+            out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
+        return out
     shape = _shape(a)
     axes = _axes(axis, len(shape))
-    if window is not None and not isinstance(a, FwdLaplArray):
+    if window is not None and not _is_triplet(a):
         a = getitem(a, tuple(slice(*window) if i == axes[0] else slice(None) for i in range(axes[0] + 1)))
         window = None
     out = _call('reduce_sum', (a,), {'axes': axes} if window is None else {'axes': axes, 'window': tuple(window)})
@@ -305,8 +371,13 @@ def reshape(a, shape):
 
 
 def transpose(a, axes=None):
+    from .wrapped_functions import LazyMul, LazyTranspose
+
     nd = len(_shape(a))
     axes = tuple(range(nd))[::-1] if axes is None else tuple(ax % nd for ax in axes)
+    if nd >= 3 and isinstance(a, (FwdLaplArray, LazyMul)) and axes[-1] == nd - 1 and axes[-2] != nd - 2 \
+            and list(axes[:-2]) == [i for i in range(nd - 1) if i != axes[-2]]:
+        return LazyTranspose(a, axes, current_threshold())  # one axis moved in front of the last: slogdet reads it in place
     return _call('transpose', (a,), {'permutation': axes})
 
 
@@ -332,32 +403,48 @@ def squeeze(a, axis):
     return reshape(a, shape)
 
 
-def broadcast_to(a, shape, lazy=False):
-    """``lazy=True`` returns a handle that only a lazy ``concatenate`` accepts."""
-    shape = tuple(shape)
-    if lazy and isinstance(a, FwdLaplArray):
-        from .wrapped_functions import LazyBroadcast
+def broadcast_to(a, shape, lazy=True):
+    """A vector broadcast along new leading axes is deferred: a concatenation that a product
+    reads in parts takes it as it is, everything else evaluates it."""
+    from .wrapped_functions import LazyBroadcast, force
 
-        return LazyBroadcast(a, shape)
+    del lazy
+    shape = tuple(int(n) for n in shape)
+    a = force(a)
+    if isinstance(a, FwdLaplArray) and a.ndim == 1 and len(shape) >= 2 and shape[-1] == a.shape[-1]:
+        return LazyBroadcast(a, shape, current_threshold())  # a per-walker vector shown to every row
     src = _shape(a)
     off = len(shape) - len(src)
     return _call('broadcast_in_dim', (a,), {'shape': shape, 'broadcast_dimensions': tuple(range(off, len(shape)))})
 
 
 def getitem(a, idx):
+    from .wrapped_functions import LazySlice, force
+
+    a = force(a)
+    if isinstance(a, FwdLaplArray):
+        # a contiguous window along ONE axis, everything else taken whole: deferred, so that the product
+        # or the sum that reads it can take the window in place
+        items = idx if isinstance(idx, tuple) else (idx,)
+        if all(isinstance(i, slice) for i in items) and len(items) <= a.ndim:
+            cut = [(ax, *i.indices(a.shape[ax])) for ax, i in enumerate(items)
+                   if i.indices(a.shape[ax]) != (0, a.shape[ax], 1)]
+            if len(cut) == 1 and cut[0][3] == 1 and cut[0][1] < cut[0][2]:
+                return LazySlice(a, cut[0][0], cut[0][1], cut[0][2], current_threshold())
     return _call('slice', (a,), {'idx': idx})
 
 
-def concatenate(arrs, axis=-1, lazy=False):
-    """``lazy=True`` (last axis only) returns a handle that only ``dot`` accepts as its first
-    operand: a product that can read its operand in parts never forms the concatenation."""
-    from .wrapped_functions import LazyBroadcast, LazyConcat
+def concatenate(arrs, axis=-1, lazy=True):
+    """Along the last axis of triplets the result is deferred: a product that can read its operand
+    in parts never forms the concatenation (nor the broadcasts among the parts)."""
+    from .wrapped_functions import LazyBroadcast, LazyConcat, force
 
-    arrs = tuple(arrs)
-    if lazy and axis == -1 and all(isinstance(t, (FwdLaplArray, LazyBroadcast)) for t in arrs):
-        return LazyConcat(arrs)
-    thr = current_threshold()
-    arrs = tuple(t.value(thr) if isinstance(t, LazyBroadcast) else t for t in arrs)
+    del lazy
+    arrs = tuple(t if isinstance(t, LazyBroadcast) else force(t) for t in arrs)
+    nd = len(_shape(arrs[0]))
+    if axis % nd == nd - 1 and nd >= 2 and len(arrs) > 1 and all(isinstance(t, (FwdLaplArray, LazyBroadcast)) for t in arrs) \
+            and all(tuple(t.shape[:-1]) == tuple(arrs[0].shape[:-1]) for t in arrs):
+        return LazyConcat(arrs, current_threshold())
     return _call('concatenate', arrs, {'dimension': axis})
 
 

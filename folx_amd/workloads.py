@@ -35,9 +35,9 @@ def mlp_forward(params, x, xp=None):
     if xp is None:
         from . import numpy as xp
     for W, b in params[:-1]:
-        x = xp.dot(x, W, b, act='silu')
+        x = xp.silu(xp.add(xp.dot(x, W), b))
     W, b = params[-1]
-    return xp.sum(xp.dot(x, W, b))
+    return xp.sum(xp.add(xp.dot(x, W), b))
 
 
 # --------------------------------------------------------------------------------------
@@ -172,32 +172,34 @@ def psiformer_forward(p: PsiFormerParams, r, xp=None):
     feats = xp.concatenate([xp.reshape(d, (n, 3 * cfg.n_nuc)), dist, p.spin], axis=-1)
     h = xp.dot(feats, p.w_in)
     for L in p.layers:
-        # the LayerNorms are only consumed by matrix products, which take them into their own
-        # rule where they can (dense Jacobians): the normalised Jacobian is then never written
-        hn = xp.layer_norm(h, L['ln1_g'], L['ln1_b'], cfg.ln_eps, lazy=True)
+        hn = xp.layer_norm(h, L['ln1_g'], L['ln1_b'], cfg.ln_eps)
         q = xp.reshape(xp.dot(hn, L['w_q']), (n, H, dh))
         k = xp.reshape(xp.dot(hn, L['w_k']), (n, H, dh))
         v = xp.reshape(xp.dot(hn, L['w_v']), (n, H, dh))
         att = xp.multi_head_self_attention(q, k, v)
-        h = xp.dot(xp.reshape(att, (n, H * dh)), L['w_o'], None, residual=h)
-        hn = xp.layer_norm(h, L['ln2_g'], L['ln2_b'], cfg.ln_eps, lazy=True)
-        h = xp.dot(xp.dot(hn, L['w_1'], L['b_1'], act='tanh'), L['w_2'], L['b_2'], residual=h)
+        h = xp.add(h, xp.dot(xp.reshape(att, (n, H * dh)), L['w_o']))
+        hn = xp.layer_norm(h, L['ln2_g'], L['ln2_b'], cfg.ln_eps)
+        mlp = xp.tanh(xp.add(xp.dot(hn, L['w_1']), L['b_1']))
+        h = xp.add(h, xp.add(xp.dot(mlp, L['w_2']), L['b_2']))
+    return log_psi_from_orbitals(xp, cfg, p, h, dist)
+
+
+def log_psi_from_orbitals(xp, cfg, p, h, dist):
+    """log|sum_k det(orbitals_k^up) det(orbitals_k^down)| from the one-electron stream ``h (n, width)``
+    and the electron-nucleus distances ``dist (n, n_nuc)``: orbitals = (h @ w_orb) * envelopes."""
+    n = cfg.n_elec
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, cfg.n_up), (cfg.n_up, n)]):
         m = hi - lo
         if m == 0:
             continue
-        orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))  # (m, n_det * m), spin block read in place
+        orb = xp.dot(xp.getitem(h, (slice(lo, hi),)), p.w_orb[s])                                # (m, n_det * m)
         env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])  # (m, n_det * m)
-        # (electron, determinant, orbital): the matrices are read in place, rows on axis 0, and
-        # multiplied by their envelopes while they are loaded
+        # (electron, determinant, orbital) -> one (m x m) matrix per determinant
+        mats = xp.multiply(xp.reshape(orb, (m, cfg.n_det, m)), xp.reshape(env, (m, cfg.n_det, m)))
         if cfg.orb_shift:
-            shift = (cfg.orb_shift * np.eye(m, dtype=np.float32))[:, None, :]
-            mats = xp.add(xp.multiply(xp.reshape(orb, (m, cfg.n_det, m)), xp.reshape(env, (m, cfg.n_det, m))), shift)
-            sg, ld = xp.slogdet(mats, row_axis=0)
-        else:
-            sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
-                                factor=xp.reshape(env, (m, cfg.n_det, m)))
+            mats = xp.add(mats, (cfg.orb_shift * np.eye(m, dtype=np.float32))[:, None, :])
+        sg, ld = xp.slogdet(xp.transpose(mats, (1, 0, 2)))
         logdets.append(ld), signs.append(sg)
     total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
     sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
@@ -284,48 +286,19 @@ def ferminet_forward(p: FermiNetParams, r, xp=None):
     rn = xp.multiply(xp.sqrt(r2), 1.0 - p.eye)
     g = xp.concatenate([rij, xp.expand_dims(rn, 2)], axis=-1)  # (n, n, 4)
 
-    def spin_means(t, axis_len):
-        # means over the electrons of one spin: the slices are summed where they lie
-        up = xp.mean(t, axis=0, window=(0, nu)) if nu > 0 else None
-        dn = xp.mean(t, axis=0, window=(nu, n)) if n - nu > 0 else None
-        return up, dn
-
+    up, dn = slice(0, nu), slice(nu, n)
     for li, L in enumerate(p.layers):
-        hu, hd = spin_means(h, n)  # (d1,) each
-        # means over the second electron of every pair: (n, d2)
-        gu = xp.mean(g, axis=1, window=(0, nu))
-        gd = xp.mean(g, axis=1, window=(nu, n))
+        # means over the electrons of one spin, (d1,) each, and over the second electron of every pair, (n, d2)
+        hu, hd = xp.mean(xp.getitem(h, (up,)), axis=0), xp.mean(xp.getitem(h, (dn,)), axis=0)
+        gu, gd = xp.mean(xp.getitem(g, (slice(None), up)), axis=1), xp.mean(xp.getitem(g, (slice(None), dn)), axis=1)
         d1 = h.shape[-1]
-        # the feature vector is only consumed by the product below, which reads it part by
-        # part where it can: neither the broadcasts nor the concatenation are then formed
-        parts = [h, xp.broadcast_to(hu, (n, d1), lazy=True), xp.broadcast_to(hd, (n, d1), lazy=True), gu, gd]
-        f = xp.concatenate(parts, axis=-1, lazy=True)
-        if L['v'].shape[1] == d1:  # residual layer: the skip connection is added in the product's epilogue
-            h = xp.dot(f, L['v'], L['b'], act='tanh', residual=h)
-        else:
-            h = xp.dot(f, L['v'], L['b'], act='tanh')
+        f = xp.concatenate([h, xp.broadcast_to(hu, (n, d1)), xp.broadcast_to(hd, (n, d1)), gu, gd], axis=-1)
+        hn = xp.tanh(xp.add(xp.dot(f, L['v']), L['b']))
+        h = xp.add(h, hn) if L['v'].shape[1] == d1 else hn  # residual layer where the widths match
         if 'w' in L:
-            gn = xp.dot(g, L['w'], L['c'], act='tanh')
+            gn = xp.tanh(xp.add(xp.dot(g, L['w']), L['c']))
             g = xp.add(g, gn) if gn.shape == g.shape else gn
-    logdets, signs = [], []
-    for s, (lo, hi) in enumerate([(0, nu), (nu, n)]):
-        m = hi - lo
-        if m == 0:
-            continue
-        orb = xp.dot(h, p.w_orb[s], row_slice=(lo, hi))
-        env = xp.exp_envelope(xp.getitem(dist, (slice(lo, hi),)), p.env_sigma[s], p.env_pi[s])
-        if cfg.orb_shift:
-            shift = (cfg.orb_shift * np.eye(m, dtype=np.float32))[:, None, :]
-            mats = xp.add(xp.multiply(xp.reshape(orb, (m, cfg.n_det, m)), xp.reshape(env, (m, cfg.n_det, m))), shift)
-            sg, ld = xp.slogdet(mats, row_axis=0)
-        else:
-            sg, ld = xp.slogdet(xp.reshape(orb, (m, cfg.n_det, m)), row_axis=0,
-                                factor=xp.reshape(env, (m, cfg.n_det, m)))
-        logdets.append(ld), signs.append(sg)
-    total = logdets[0] if len(logdets) == 1 else xp.add(logdets[0], logdets[1])
-    sign = signs[0] if len(signs) == 1 else xp.multiply(signs[0], signs[1])
-    logpsi, _ = xp.logsumexp(total, axis=0, b=sign)
-    return logpsi
+    return log_psi_from_orbitals(xp, cfg, p, h, dist)
 
 
 def sample_electrons(n_walkers, n_elec, sigma, seed):

@@ -666,58 +666,205 @@ def _dot_mul_sum(lhs: FwdLaplArray, rhs: FwdLaplArray, a_vec: bool, b_vec: bool)
     return out
 
 
-class LazyLayerNorm:
-    """``layer_norm(h, gamma, beta, eps)`` that has not been evaluated yet, for layers whose
-    only consumers are matrix products (``numpy.dot``): a product that can take LayerNorm
-    into its own rule reads ``h`` directly, any other evaluates the ``layer_norm`` rule --
-    once, however many products ask."""
+class Deferred:
+    """The result of a rule that has not been evaluated yet.
 
-    __slots__ = ('h', 'gamma', 'beta', 'eps', '_value')
+    The reference sees a whole jaxpr before anything runs and XLA fuses the emitted operations
+    afterwards; a define-by-run front end sees one call at a time.  The functions of
+    ``folx_amd.numpy`` therefore return a handle of this kind where a later call may be able to
+    take the operation into its own rule (LayerNorm into the product that consumes it, an
+    activation and a skip connection into the product in front of them, a slice into the
+    product or the sum that reads it, a concatenation into the product, an elementwise factor
+    and a transposition into ``slogdet``).  A consumer that knows the handle absorbs it; every
+    other use -- any rule, an attribute such as ``.x`` or ``.jacobian``, the end of
+    ``forward_laplacian`` -- evaluates it through the ordinary rule, once (``value``).  Either
+    way the triplet is the one the ordinary rules define."""
 
-    def __init__(self, h, gamma, beta, eps):
+    __slots__ = ('_value', 'thr')
+
+    def __init__(self, thr: int):
+        self._value, self.thr = None, int(thr)
+
+    def _evaluate(self) -> FwdLaplArray:
+        raise NotImplementedError
+
+    def value(self, sparsity_threshold=None) -> FwdLaplArray:
+        if self._value is None:
+            from . import numpy as fnp
+
+            with fnp.sparsity_threshold(self.thr if sparsity_threshold is None else sparsity_threshold):
+                self._value = self._evaluate()
+        return self._value
+
+    # the surface of a FwdLaplArray -----------------------------------------------------------------
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape, dtype=int))
+
+    x = property(lambda self: self.value().x)
+    jacobian = property(lambda self: self.value().jacobian)
+    laplacian = property(lambda self: self.value().laplacian)
+    B = property(lambda self: self.value().B)
+    dtype = property(lambda self: torch.float32)
+    dense_jacobian = property(lambda self: self.value().jacobian.dense_array)
+
+    def __iter__(self):
+        return iter(self.value())
+
+    def __repr__(self):
+        return f'{type(self).__name__}(shape={self.shape}, evaluated={self._value is not None})'
+
+
+for _name in ('__add__', '__radd__', '__sub__', '__rsub__', '__mul__', '__rmul__', '__truediv__', '__rtruediv__',
+              '__neg__', '__matmul__', '__getitem__', 'reshape', 'sum'):
+    setattr(Deferred, _name, getattr(FwdLaplArray, _name))  # the same sugar: everything goes through folx_amd.numpy
+
+
+def force(v):
+    """``v`` with every deferred value (also inside a tuple or list) replaced by its triplet."""
+    if isinstance(v, Deferred):
+        return v.value()
+    if isinstance(v, (tuple, list)) and any(isinstance(t, Deferred) for t in v):
+        return type(v)(force(t) for t in v)
+    return v
+
+
+class LazyLayerNorm(Deferred):
+    """``layer_norm(h, gamma, beta, eps)``: a product that can take LayerNorm into its own rule
+    reads ``h`` directly, any other consumer evaluates the ``layer_norm`` rule -- once, however
+    many ask."""
+
+    __slots__ = ('h', 'gamma', 'beta', 'eps')
+
+    def __init__(self, h, gamma, beta, eps, thr=0):
+        super().__init__(thr)
         self.h, self.gamma, self.beta, self.eps = h, gamma, beta, float(eps)
-        self._value = None
 
-    def value(self, sparsity_threshold):
-        if self._value is None:
-            self._value = layer_norm_rule((self.h, self.gamma, self.beta), {'eps': self.eps}, sparsity_threshold)
-        return self._value
+    shape = property(lambda self: tuple(self.h.shape))
 
-
-class LazyBroadcast:
-    """``broadcast_to(a, shape)`` that has not been evaluated; a lazy ``concatenate`` is the
-    only consumer that can take it as it is."""
-
-    __slots__ = ('a', 'shape', '_value')
-
-    def __init__(self, a, shape):
-        self.a, self.shape, self._value = a, tuple(shape), None
-
-    def value(self, sparsity_threshold):
-        if self._value is None:
-            off = len(self.shape) - self.a.ndim
-            self._value = _LAPLACE_FN_REGISTRY['broadcast_in_dim'](
-                (self.a,), {'shape': self.shape, 'broadcast_dimensions': tuple(range(off, len(self.shape)))},
-                sparsity_threshold)
-        return self._value
+    def _evaluate(self):
+        return layer_norm_rule((self.h, self.gamma, self.beta), {'eps': self.eps}, self.thr)
 
 
-class LazyConcat:
-    """``concatenate(parts, axis=-1)`` that has not been evaluated, for feature vectors whose only
-    consumer is a matrix product (``numpy.dot``): a product that can read its operand in parts
-    never forms the concatenation (nor the broadcasts among the parts), any other evaluates
-    it once."""
+class LazyBroadcast(Deferred):
+    """``broadcast_to(a, shape)``; a concatenation that a product reads in parts takes it as it is."""
 
-    __slots__ = ('parts', '_value')
+    __slots__ = ('a', 'shape')
 
-    def __init__(self, parts):
-        self.parts, self._value = tuple(parts), None
+    def __init__(self, a, shape, thr=0):
+        super().__init__(thr)
+        self.a, self.shape = a, tuple(shape)
 
-    def value(self, sparsity_threshold):
-        if self._value is None:
-            parts = tuple(t.value(sparsity_threshold) if isinstance(t, LazyBroadcast) else t for t in self.parts)
-            self._value = concatenate_rule(parts, {'dimension': -1}, sparsity_threshold)
-        return self._value
+    def _evaluate(self):
+        off = len(self.shape) - self.a.ndim
+        return _LAPLACE_FN_REGISTRY['broadcast_in_dim'](
+            (self.a,), {'shape': self.shape, 'broadcast_dimensions': tuple(range(off, len(self.shape)))}, self.thr)
+
+
+class LazyConcat(Deferred):
+    """``concatenate(parts, axis=-1)``: a product that can read its operand in parts never forms
+    the concatenation (nor the broadcasts among the parts)."""
+
+    __slots__ = ('parts',)
+
+    def __init__(self, parts, thr=0):
+        super().__init__(thr)
+        self.parts = tuple(parts)
+
+    @property
+    def shape(self):
+        lead = tuple(self.parts[0].shape[:-1])
+        return (*lead, int(np.sum([t.shape[-1] for t in self.parts])))
+
+    def _evaluate(self):
+        return concatenate_rule(tuple(force(t) for t in self.parts), {'dimension': -1}, self.thr)
+
+
+class LazySlice(Deferred):
+    """``a[..., lo:hi, ...]`` along ONE axis: a product reads the rows in place (axis in front of
+    the feature axis), a sum over that axis reads its window in place."""
+
+    __slots__ = ('a', 'axis', 'lo', 'hi')
+
+    def __init__(self, a, axis, lo, hi, thr=0):
+        super().__init__(thr)
+        self.a, self.axis, self.lo, self.hi = a, int(axis), int(lo), int(hi)
+
+    @property
+    def shape(self):
+        s = list(self.a.shape)
+        s[self.axis] = self.hi - self.lo
+        return tuple(s)
+
+    def _evaluate(self):
+        idx = tuple(slice(self.lo, self.hi) if i == self.axis else slice(None) for i in range(self.axis + 1))
+        return getitem_rule((self.a,), {'idx': idx}, self.thr)
+
+
+class LazyDot(Deferred):
+    """``h @ W`` with a constant ``W`` whose epilogue is still open: a constant vector added to it
+    becomes the bias, a scalar function applied to it the activation of the same rule, a triplet
+    of its shape added to it the skip connection.  ``kwargs`` are those of the ``dot_general``
+    rule (bias, act, norm, row_slice); evaluation is that rule."""
+
+    __slots__ = ('h', 'W', 'kwargs', 'shape')
+
+    def __init__(self, h, W, kwargs, shape, thr=0):
+        super().__init__(thr)
+        self.h, self.W, self.kwargs, self.shape = h, W, dict(kwargs), tuple(shape)
+
+    def with_(self, **kw):
+        return LazyDot(self.h, self.W, {**self.kwargs, **kw}, self.shape, self.thr)
+
+    def _evaluate(self, residual=None):
+        return dot_general((self.h, self.W), {**self.kwargs, 'residual': residual}, self.thr)
+
+    def value_with_residual(self, residual):
+        """``residual + (this product)`` as one rule; the handle itself stays unevaluated."""
+        from . import numpy as fnp
+
+        with fnp.sparsity_threshold(self.thr):
+            return self._evaluate(residual)
+
+
+class LazyMul(Deferred):
+    """``a * b`` of two triplets of one shape; ``slogdet`` multiplies a factor while it loads its
+    matrices."""
+
+    __slots__ = ('a', 'b')
+
+    def __init__(self, a, b, thr=0):
+        super().__init__(thr)
+        self.a, self.b = a, b
+
+    shape = property(lambda self: tuple(self.a.shape))
+
+    def _evaluate(self):
+        return _LAPLACE_FN_REGISTRY['mul']((self.a, self.b), {}, self.thr)
+
+
+class LazyTranspose(Deferred):
+    """``transpose(a, perm)`` that moves one axis in front of the last one and keeps the order of
+    the others: the layout ``slogdet`` reads in place (matrix rows on another axis)."""
+
+    __slots__ = ('a', 'perm')
+
+    def __init__(self, a, perm, thr=0):
+        super().__init__(thr)
+        self.a, self.perm = a, tuple(perm)
+
+    shape = property(lambda self: tuple(self.a.shape[i] for i in self.perm))
+
+    @property
+    def row_axis(self):
+        return self.perm[-2]
+
+    def _evaluate(self):
+        return transpose_rule((force(self.a),), {'permutation': self.perm}, self.thr)
 
 
 def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
