@@ -54,8 +54,10 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(workload, budget_s):
-    """The numpy oracle (fp32, dense Jacobians) on a bounded sample of the same workload."""
+def cpu_baseline(workload, budget_s, gpu_out=None):
+    """The numpy oracle (fp32, dense Jacobians) on a bounded sample of the same workload: the first
+    n walkers of the batch the GPU was timed on, whose GPU results (``gpu_out``) are compared with
+    the oracle's in the same run."""
     from oracle import backend as ob
 
     from folx_amd import workloads as wl
@@ -69,23 +71,40 @@ def cpu_baseline(workload, budget_s):
         threads = 1
 
     def run(n):
-        x = wl.sample_inputs(workload, n, seed=2)
+        x = wl.sample_inputs(workload, n, seed=2)  # the first n walkers of the GPU's batch (same seed, row-major draws)
         t0 = time.perf_counter()
         out = forward(p, ob.init_state(x, dtype=np.float32), ob)
         dt = time.perf_counter() - t0
         assert np.isfinite(out.lap).all()
-        return dt
+        return dt, out
 
-    t1 = run(1)
+    t1, out = run(1)
     n = int(max(1, min(64, budget_s / max(t1, 1e-3))))
-    dt = run(n) if n > 1 else t1
-    return {
+    if n > 1:
+        dt, out = run(n)
+    else:
+        dt = t1
+    res = {
         'value': n / dt,
         'unit': 'walkers/s',
         'cores': threads,
         'kind': 'port',
         'sample': f'{n} walkers of {workload}, numpy fp32 oracle with dense Jacobians, {dt:.1f} s',
     }
+    if gpu_out is not None:
+        # same walkers, GPU path against the CPU oracle: largest difference over the largest reference entry.
+        # Both sides are float32; log|det| of the randomly initialised orbital matrices amplifies their
+        # rounding (the oracle's own float32 / float64 difference is 3e-4 on psiformer32), which is what
+        # these figures show -- the parity bars are enforced stage by stage in tests/.
+        gx, gJ, gl = gpu_out
+        rel = lambda g, r: float(np.abs(g[..., :n].astype(np.float64) - r).max() / max(np.abs(r).max(), 1e-30))
+        res['gpu_vs_oracle_max_rel'] = {
+            'value': rel(gx[None], np.asarray(out.x, dtype=np.float64)[None]),
+            'jacobian': rel(gJ, np.asarray(out.J, dtype=np.float64).reshape(out.J.shape[0], -1)[:, :n]),
+            'laplacian': rel(gl[None], np.asarray(out.lap, dtype=np.float64)[None]),
+            'walkers': n,
+        }
+    return res
 
 
 def describe(cfg):
@@ -226,8 +245,20 @@ def main():
         'roofline': roof,
         'kernel_ms_per_step': {k: v / args.steps for k, v in sorted(per_kernel.items(), key=lambda kv: -kv[1])},
     }
+    if roof is not None and roof.get('traffic') is not None:
+        roof['traffic_source'] = ('profiles/psiformer32_forward_laplacian.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this '
+                                  'command in earlier runs (counters cannot be read inside the timed run)')
     if not args.no_cpu:
-        line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds)
+        gpu_out = None
+        if tuple(out.x.shape) == (B,):
+            gpu_out = (out.x.cpu().numpy(), out.jacobian.dense_array.reshape(-1, B).cpu().numpy(), out.laplacian.cpu().numpy())
+        line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds, gpu_out)
+    # the reference itself (JAX on the host cores) can only be timed where jax is installed
+    import importlib.util
+
+    if importlib.util.find_spec('jax') is None:
+        line['reference_jax_cpu'] = 'unavailable on this host (jax is not installed)'
+        print('reference JAX-CPU: unavailable on this host', file=sys.stderr)
     print(json.dumps(line))
 
 

@@ -94,6 +94,8 @@ struct WideParams {
   const float2* wc;  // (N) pairs (w1, c0)
   float* y_jac;
   const float* res_jac;  // optional (P, R, N) added to the activated Jacobian rows     PARTS instances only
+  const float* pre_jac;  // optional (P, R / pre_group, N) added to the PRE-activation Jacobian rows: position r takes
+  int64_t pre_group;     // row r / pre_group (a per-walker term shared by the walker's positions)   PARTS instances only
   float* ss;         // (PG, R, N) sums of zj^2 per group of PT Jacobian rows     activation only
   float* s1;         // (PG, R, N) sums of b_p (t_p @ Wg - a_p w1)                LayerNorm only
   float* sc;         // (PG, R, 2) sums of b_p^2 and of q_p
@@ -381,8 +383,21 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
 #pragma unroll
       for (int b = 0; b < PB; ++b) ss[b] = 0.0f;
       const float* resp = nullptr;
-      if constexpr (PARTS) resp = a.res_jac ? a.res_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc : nullptr;
-      auto rows = [&](auto full, auto has_res) __attribute__((always_inline)) {
+      const float* prep[PB];
+      int64_t pre_pstride = 0;
+#pragma unroll
+      for (int b = 0; b < PB; ++b) prep[b] = nullptr;
+      if constexpr (PARTS) {
+        resp = a.res_jac ? a.res_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc : nullptr;
+        if (a.pre_jac) {
+          pre_pstride = (R / a.pre_group) * N;
+          const int gcc = gc < N ? gc : N - 1;
+#pragma unroll
+          for (int b = 0; b < PB; ++b)
+            prep[b] = a.pre_jac + ((pos + b) / a.pre_group) * N + gcc;
+        }
+      }
+      auto rows = [&](auto full, auto has_res, auto has_pre) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           constexpr int GB = PT / 8;     // register groups per position
@@ -405,6 +420,11 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
             }
             const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
             float* o = out + off;
+            if constexpr (decltype(has_pre)::value) {
+              int prow = p0 + 4 * lh + pl;  // rows past P of a ragged tile are neither stored nor summed
+              if constexpr (!decltype(full)::value) prow = prow < P ? prow : P - 1;
+              v += prep[b][(int64_t)prow * pre_pstride];
+            }
             if constexpr (decltype(full)::value) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
               float w = d1[b] * v;
@@ -417,12 +437,20 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
           }
         }
       };
-      if (PARTS && resp != nullptr) {
-        if (full_tile) rows(std::true_type{}, std::true_type{});
-        else rows(std::false_type{}, std::true_type{});
+      if (PARTS && prep[0] != nullptr) {
+        if (resp != nullptr) {
+          if (full_tile) rows(std::true_type{}, std::true_type{}, std::true_type{});
+          else rows(std::false_type{}, std::true_type{}, std::true_type{});
+        } else {
+          if (full_tile) rows(std::true_type{}, std::false_type{}, std::true_type{});
+          else rows(std::false_type{}, std::false_type{}, std::true_type{});
+        }
+      } else if (PARTS && resp != nullptr) {
+        if (full_tile) rows(std::true_type{}, std::true_type{}, std::false_type{});
+        else rows(std::false_type{}, std::true_type{}, std::false_type{});
       } else {
-        if (full_tile) rows(std::true_type{}, std::false_type{});
-        else rows(std::false_type{}, std::false_type{});
+        if (full_tile) rows(std::true_type{}, std::false_type{}, std::false_type{});
+        else rows(std::false_type{}, std::false_type{}, std::false_type{});
       }
       const int64_t so = ((int64_t)pg * R + pos) * N + gc;
       if constexpr (ACT) {
@@ -591,6 +619,23 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float* __restrict_
   }
 }
 
+// y[r][c] += pre[r / group][c], y_lap likewise: the per-walker pre-activation term on the x and lap
+// rows (one float4 per thread).
+__global__ __launch_bounds__(256) void wide_add_pre_kernel(float* __restrict__ y, float* __restrict__ y_lap,
+                                                           const float* __restrict__ pre,
+                                                           const float* __restrict__ pre_lap, int64_t S4, int32_t N4,
+                                                           int64_t group) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= S4) return;
+  const int64_t src = (i / N4 / group) * N4 + i % N4;
+  float4 a = reinterpret_cast<float4*>(y)[i], b = reinterpret_cast<float4*>(y_lap)[i];
+  const float4 p = reinterpret_cast<const float4*>(pre)[src], q = reinterpret_cast<const float4*>(pre_lap)[src];
+  a.x += p.x; a.y += p.y; a.z += p.z; a.w += p.w;
+  b.x += q.x; b.y += q.y; b.z += q.z; b.w += q.w;
+  reinterpret_cast<float4*>(y)[i] = a;
+  reinterpret_cast<float4*>(y_lap)[i] = b;
+}
+
 // Shapes the path takes, launch sizes and the carve-up of the workspace (offsets in floats,
 // every part a multiple of 4 floats).
 struct WidePlan {
@@ -645,7 +690,8 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
              const float* gamma, const float* beta, float eps, const float* W, const float* bias, float* y,
              float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
              int64_t workspace_bytes, const WideParts* parts = nullptr, const float* res = nullptr,
-             const float* res_jac = nullptr, const float* res_lap = nullptr) {
+             const float* res_jac = nullptr, const float* res_lap = nullptr, const float* pre = nullptr,
+             const float* pre_jac = nullptr, const float* pre_lap = nullptr, int64_t pre_group = 1) {
   const bool has_act = act >= 0;
   WidePlan pl;
   if ((has_act && !act_fused(act)) || !plan_wide(R, P, K, N, norm, has_act, pl)) return FOLX_HIP_ENOTSUP;
@@ -660,6 +706,7 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
   float* ws = (float*)workspace;
   WideParams a;
   a.jac = jac; a.W = W; a.z = y; a.y_jac = y_jac; a.res_jac = res_jac;
+  a.pre_jac = pre_jac; a.pre_group = pre_group;
   a.xhat = nullptr; a.rs = nullptr; a.wc = nullptr;
   a.ss = ws + pl.o_ss; a.s1 = nullptr; a.sc = nullptr;
   a.R = R; a.row_tiles = pl.row_tiles; a.pos_tiles = pl.pos_tiles;
@@ -683,6 +730,13 @@ int run_wide(hipStream_t st, bool norm, int32_t act, float param, const float* x
   int rc = folx_hip_dense_fwdlap(st, in_x, nullptr, in_lap, W, bias, nullptr, nullptr, nullptr, y, nullptr, y_lap, R,
                                  0, K, N);
   if (rc != FOLX_HIP_OK) return rc;
+  if (pre) {
+    const int64_t S4 = R * (int64_t)N / 4;
+    wide_add_pre_kernel<<<dim3((unsigned)((S4 + 255) / 256)), dim3(256), 0, st>>>(y, y_lap, pre, pre_lap, S4, N / 4,
+                                                                              pre_group);
+    rc = folx_launch_status();
+    if (rc != FOLX_HIP_OK) return rc;
+  }
   if (norm)
     return has_act ? launch_wide<true, true, 32>(st, a, pl, y, y_lap) : launch_wide<true, false, 32>(st, a, pl, y, y_lap);
   if (parts) {
@@ -730,13 +784,16 @@ extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float 
                                                const float* lap, int32_t n_parts, const float* const* jac_parts,
                                                const int32_t* widths, const int32_t* broadcast, int32_t group,
                                                const float* W, const float* bias, const float* res,
-                                               const float* res_jac, const float* res_lap, float* y,
+                                               const float* res_jac, const float* res_lap, const float* pre,
+                                               const float* pre_jac, const float* pre_lap, float* y,
                                                float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t N,
                                                void* workspace, int64_t workspace_bytes) {
   if (R < 0 || P < 0 || N <= 0 || n_parts < 1 || group < 1 || !jac_parts || !widths || !broadcast)
     return FOLX_HIP_EINVAL;
   if ((res != nullptr) != (res_jac != nullptr) || (res != nullptr) != (res_lap != nullptr)) return FOLX_HIP_EINVAL;
-  if (!folx_aligned16(res) || !folx_aligned16(res_lap)) return FOLX_HIP_ENOTSUP;
+  if ((pre != nullptr) != (pre_jac != nullptr) || (pre != nullptr) != (pre_lap != nullptr)) return FOLX_HIP_EINVAL;
+  if (!folx_aligned16(res) || !folx_aligned16(res_lap) || !folx_aligned16(pre) || !folx_aligned16(pre_lap))
+    return FOLX_HIP_ENOTSUP;
   if (n_parts > MAX_PARTS || act < 0 || R % group != 0) return FOLX_HIP_ENOTSUP;
   WideParts parts;
   parts.n = n_parts;
@@ -757,7 +814,8 @@ extern "C" int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float 
     parts.jac[i] = nullptr; parts.width[i] = 0; parts.bcast[i] = 0; parts.pstride[i] = 0; parts.kend[i] = K;
   }
   return run_wide((hipStream_t)stream, false, act, param, x, nullptr, lap, nullptr, nullptr, 0.0f, W, bias, y, y_jac,
-                  y_lap, R, P, K, N, workspace, workspace_bytes, &parts, res, res_jac, res_lap);
+                  y_lap, R, P, K, N, workspace, workspace_bytes, &parts, res, res_jac, res_lap, pre, pre_jac, pre_lap,
+                  group);
 }
 
 // ---- folx_hip_norm_dense_fwdlap on the library's own scratch memory -------------------------

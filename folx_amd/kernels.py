@@ -183,13 +183,14 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return y, yj, yl
 
 
-def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None):
+def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None, pre=None):
     """``dense_act`` of a wide layer whose Jacobian operand is the concatenation along the
     feature axis of ``jac_parts`` (never formed): part i is (P, rows_i, widths[i]) with rows_i
     the layer's rows, or one row per ``group`` of them where ``broadcast[i]``; x and lap are
     the concatenated arrays (.., K); ``res`` = (x, jac, lap) of the output's shape is added to
-    the activated result."""
-    _chk(x, lap, W, bias, *jac_parts, *(res or ()))
+    the activated result; ``pre`` = (x (rows / group, N), jac (P, rows / group, N), lap) is added
+    to the pre-activation triplet, one row per ``group`` of the layer's rows."""
+    _chk(x, lap, W, bias, *jac_parts, *(res or ()), *(pre or ()))
     K, N = W.shape
     assert sum(widths) == K and x.shape[-1] == K
     P = jac_parts[0].shape[0]
@@ -211,6 +212,10 @@ def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=N
     if res is not None:
         assert rx.is_contiguous() and rj.is_contiguous() and rl.is_contiguous()
         assert tuple(rx.shape) == tuple(y.shape) and tuple(rj.shape) == tuple(yj.shape)
+    px, pj, pl = (None, None, None) if pre is None else pre
+    if pre is not None:
+        assert px.is_contiguous() and pj.is_contiguous() and pl.is_contiguous() and R % group == 0
+        assert px.numel() == (R // group) * N and pj.numel() == P * (R // group) * N and pl.numel() == px.numel()
     ptrs = (ctypes.c_void_p * n)(*[J.data_ptr() for J in jac_parts])
     wd = (ctypes.c_int32 * n)(*[int(w) for w in widths])
     bc = (ctypes.c_int32 * n)(*[int(bool(b)) for b in broadcast])
@@ -218,7 +223,7 @@ def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=N
         check(
             lib.folx_hip_dense_act_parts_fwdlap(
                 _stream(), ACT[name], float(param), _p(x), _p(lap), n, ptrs, wd, bc, int(group), _p(W), _p(bias),
-                _p(rx), _p(rj), _p(rl), _p(y), _p(yj), _p(yl), R, P, N, _p(ws), nbytes
+                _p(rx), _p(rj), _p(rl), _p(px), _p(pj), _p(pl), _p(y), _p(yj), _p(yl), R, P, N, _p(ws), nbytes
             ),
             f'dense_act_parts_fwdlap[{name}]',
         )

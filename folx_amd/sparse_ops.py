@@ -55,6 +55,7 @@ def clear_caches():
 
     _TABLE_CACHE.clear()
     _CONST_CACHE.clear()
+    _ROWS_CACHE.clear()
     index_algebra._MEMO.clear()
 
 
@@ -157,3 +158,27 @@ def add_sparse_rows_(dense: torch.Tensor, data: torch.Tensor, idx: np.ndarray) -
     P = dense.shape[0]
     K.scatter_add_rows(data.contiguous().reshape(k, B, S_outer * S_inner), table, P, B, S_outer, S_inner,
                        out=dense.reshape(P, B, S_outer * S_inner))
+
+
+_ROWS_CACHE: dict = {}
+
+
+def weight_rows(W: torch.Tensor, ranges: tuple) -> torch.Tensor:
+    """Rows ``[lo, hi)`` of a weight matrix for each range, concatenated (a contiguous copy unless one
+    range covers it).  Kept per (tensor object, version, ranges): torch bumps ``_version`` on every
+    in-place update of ``W``, so a changed weight is never served from the cache, and an entry only
+    counts while the tensor it was made from is alive; at most 64 entries are held."""
+    import weakref
+
+    if len(ranges) == 1:
+        lo, hi = ranges[0]
+        return W[lo:hi]  # consecutive rows of a row-major matrix are contiguous
+    key = (id(W), W._version, ranges)
+    hit = _ROWS_CACHE.get(key)
+    if hit is not None and hit[0]() is W:
+        return hit[1]
+    if len(_ROWS_CACHE) >= 64:
+        _ROWS_CACHE.pop(next(iter(_ROWS_CACHE)))
+    rows = torch.cat([W[lo:hi] for lo, hi in ranges], dim=0).contiguous()
+    _ROWS_CACHE[key] = (weakref.ref(W), rows)
+    return rows

@@ -903,8 +903,34 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
     if not ok:
         kw = dict(kwargs)
         return dot_general((lc.value(thr), W), kw, thr)
+    bias = kwargs.get('bias')
+    res = None  # a skip connection with the same dense rows goes into the kernel's epilogue
+    if (_is(residual) and residual.jacobian.x0_idx is None and residual.jacobian.data.shape[0] == P
+            and tuple(residual.shape) == (*lead, np.shape(W)[1])):
+        res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
+    Wt = so.device_const(W, dev)
+    bt = None if bias is None else so.device_const(bias, dev)
+    is_b = [isinstance(t, LazyBroadcast) for t in lc.parts]
+    wds = [u.shape[-1] for u in srcs]
+    ends = np.cumsum(wds)
+    ranges = [(int(e - w), int(e)) for e, w in zip(ends, wds)]
+    pre = None
+    if any(is_b) and not all(is_b) and group > 1:
+        # The per-walker (broadcast) parts meet their rows of W ONCE per walker: a dense layer on B
+        # rows whose result enters the main product in front of the activation.  The main product
+        # then only contracts the per-position parts -- for a FermiNet layer 320 of 832 features.
+        ub = [u for u, b_ in zip(srcs, is_b) if b_]
+        Wb = so.weight_rows(Wt, tuple(r for r, b_ in zip(ranges, is_b) if b_))
+        cat = lambda ts: ts[0] if len(ts) == 1 else torch.cat(ts, dim=-1)
+        pre = K.dense(cat([u.x for u in ub]), cat([so.pad_rows(u.jacobian.dense_array, P) for u in ub]),
+                      cat([u.laplacian for u in ub]), Wb, None)
+        keep = [i for i, b_ in enumerate(is_b) if not b_]
+        Wt = so.weight_rows(Wt, tuple(ranges[i] for i in keep))
+        parts_, srcs_ = [lc.parts[i] for i in keep], [srcs[i] for i in keep]
+    else:
+        parts_, srcs_ = list(lc.parts), srcs
     xs, ls, Js, widths, flags = [], [], [], [], []
-    for t, u in zip(lc.parts, srcs):
+    for t, u in zip(parts_, srcs_):
         J = so.pad_rows(u.jacobian.dense_array, P).contiguous()
         if isinstance(t, LazyBroadcast):
             shp = (B, *([1] * len(lead)), u.shape[-1])
@@ -913,14 +939,8 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
         else:
             xs.append(u.x), ls.append(u.laplacian)
         Js.append(J), widths.append(u.shape[-1]), flags.append(isinstance(t, LazyBroadcast))
-    bias = kwargs.get('bias')
-    res = None  # a skip connection with the same dense rows goes into the kernel's epilogue
-    if (_is(residual) and residual.jacobian.x0_idx is None and residual.jacobian.data.shape[0] == P
-            and tuple(residual.shape) == (*lead, np.shape(W)[1])):
-        res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
-    y, Jy, lapy = K.dense_act_parts(act, torch.cat(xs, dim=-1), torch.cat(ls, dim=-1), Js, widths, flags, group,
-                                    so.device_const(W, dev), None if bias is None else so.device_const(bias, dev),
-                                    param, res)
+    cat = lambda ts: ts[0] if len(ts) == 1 else torch.cat(ts, dim=-1)
+    y, Jy, lapy = K.dense_act_parts(act, cat(xs), cat(ls), Js, widths, flags, group, Wt, bt, param, res, pre)
     out = FwdLaplArray(y, FwdJacobian(Jy, None), lapy)
     if residual is not None and res is None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, thr)

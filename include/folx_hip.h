@@ -187,13 +187,19 @@ int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const floa
  * (folx_hip_dense_act_workspace_bytes(R, P, K, N)); FOLX_HIP_ENOTSUP otherwise.
  * res / res_jac / res_lap (all or none; shapes of y / y_jac / y_lap) are added to the
  * activated result: the skip connection of a residual layer (add_p after the activation).
+ * pre [R / group][N], pre_jac [P][R / group][N], pre_lap [R / group][N] (all or none) are added
+ * to the PRE-activation triplet, row r taking row r / group: the product of the per-walker
+ * (broadcast) features with their rows of the weight matrix, computed once per walker by the
+ * caller (folx_hip_dense_fwdlap on R / group rows) instead of once per position -- the parts
+ * passed here are then only the per-position ones, with their rows of W.
  */
 int folx_hip_dense_act_parts_fwdlap(void* stream, int32_t act, float param, const float* x,
                                     const float* lap, int32_t n_parts,
                                     const float* const* jac_parts, const int32_t* widths,
                                     const int32_t* broadcast, int32_t group, const float* W,
                                     const float* bias, const float* res, const float* res_jac,
-                                    const float* res_lap, float* y, float* y_jac, float* y_lap,
+                                    const float* res_lap, const float* pre, const float* pre_jac,
+                                    const float* pre_lap, float* y, float* y_jac, float* y_lap,
                                     int64_t R, int32_t P, int32_t N, void* workspace,
                                     int64_t workspace_bytes);
 

@@ -40,7 +40,7 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
 
 
-def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None):
+def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None, pre=None):
     P = jac_parts[0].shape[0]
     lead = tuple(x.shape[:-1])
     R = int(np.prod(lead))
@@ -50,6 +50,10 @@ def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=N
         Js.append(np.repeat(Jn, group, axis=1) if bc else Jn)
     J = np.concatenate(Js, axis=-1).reshape(P, *lead, sum(widths))
     z = rules.dense_rule(_n(x), J, _n(lap), _n(W), None if bias is None else _n(bias))
+    if pre is not None:  # one row per group of consecutive rows, added in front of the activation
+        N = z[0].shape[-1]
+        rep = lambda t, lead_: np.repeat(_n(t).reshape(*lead_, R // group, N), group, axis=len(lead_)).reshape(*lead_, *lead, N)
+        z = (z[0] + rep(pre[0], ()), z[1] + rep(pre[1], (P,)), z[2] + rep(pre[2], ()))
     out = rules.elementwise_rule({'sigmoid': 'logistic'}.get(name, name), *z, param)
     if res is not None:
         out = tuple(o + _n(r) for o, r in zip(out, res))

@@ -86,13 +86,16 @@ def test_unsupported_sizes(lib):
     # Jacobian operand in parts: host arrays of pointers, widths and broadcast flags
     ptrs, wd, bc = (ctypes.c_void_p * 2)(16, 32), (ctypes.c_int32 * 2)(16, 32), (ctypes.c_int32 * 2)(0, 1)
     parts = lambda wd_, R, group, ws, nb: lib.folx_hip_dense_act_parts_fwdlap(
-        None, 0, 0.0, one, one, 2, ptrs, wd_, bc, group, one, one, None, None, None, one, one, one, R, 33, 256, ws, nb)
+        None, 0, 0.0, one, one, 2, ptrs, wd_, bc, group, one, one, None, None, None, None, None, None, one, one, one, R, 33,
+        256, ws, nb)
     assert parts(wd, 64, 4, None, 0) == _lib.EINVAL                                  # no workspace
     assert parts((ctypes.c_int32 * 2)(16, 24), 64, 4, one, 1 << 30) == _lib.ENOTSUP  # width % 16
     assert parts(wd, 64, 5, one, 1 << 30) == _lib.ENOTSUP                            # rows % group
     assert parts(wd, 64, 0, one, 1 << 30) == _lib.EINVAL
     assert lib.folx_hip_dense_act_parts_fwdlap(None, 0, 0.0, one, one, 2, ptrs, wd, bc, 4, one, one, one, None, None,
-                                               one, one, one, 64, 33, 256, one, 1 << 30) == _lib.EINVAL  # part of a residual
+                                               None, None, None, one, one, one, 64, 33, 256, one, 1 << 30) == _lib.EINVAL  # part of a residual
+    assert lib.folx_hip_dense_act_parts_fwdlap(None, 0, 0.0, one, one, 2, ptrs, wd, bc, 4, one, one, None, None, None,
+                                               one, one, None, one, one, one, 64, 33, 256, one, 1 << 30) == _lib.EINVAL  # part of a pre-activation term
     # LayerNorm + dense (+ activation): act = -1 means none
     assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, -1) > 2 * 64 * 256 * 4
     assert lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, 0) > lib.folx_hip_norm_dense_workspace_bytes(64, 33, 256, 256, -1)

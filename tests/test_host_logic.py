@@ -450,13 +450,13 @@ def test_dot_norm(thr, monkeypatch):
 def test_dot_of_lazy_concatenate(thr, monkeypatch):
     """``dot(concatenate(parts, lazy=True), W, b, act=...)`` equals the evaluated chain: read
     part by part where the fused kernel applies (widths that are multiples of 16, a wide
-    layer; per-walker vectors broadcast among the parts, a sparse part densified), evaluated
+    layer; per-walker vectors among the parts multiplied once per walker, a sparse part densified), evaluated
     once otherwise (a narrow layer, a width of 8)."""
     from folx_amd import kernels as K
 
     calls = []
     orig = K.dense_act_parts
-    monkeypatch.setattr(K, 'dense_act_parts', lambda *a: (calls.append((tuple(a[4]), tuple(a[5]), a[6])), orig(*a))[1])
+    monkeypatch.setattr(K, 'dense_act_parts', lambda *a: (calls.append((tuple(a[4]), tuple(a[5]), a[6], None if a[11] is None else tuple(a[11][1].shape))), orig(*a))[1])
     rng = np.random.default_rng(14)
     n = 10
     W0 = rng.normal(size=(3, 16)).astype(np.float32)
@@ -482,7 +482,9 @@ def test_dot_of_lazy_concatenate(thr, monkeypatch):
         return xp.add(xp.add(xp.sum(a), xp.sum(b)), xp.sum(c))
 
     check_against_oracle(fn, x, thr)
-    assert calls == [((16, 32, 16, 16), (False, False, True, True), n)] * 2
+    # the two per-walker parts meet their rows of W once per walker (pre-activation term (P, walkers, 132));
+    # the product itself reads the two per-position parts
+    assert calls == [((16, 32), (False, False), n, (3 * n, 2, 132))] * 2
 
 
 @pytest.mark.parametrize('thr', [0, 6])

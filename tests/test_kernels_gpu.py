@@ -277,6 +277,17 @@ def test_dense_act_parts(B, n, P, widths, bcast, N, act):
     got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b), 0.0,
                             tuple(dev(t) for t in res))
     assert_triplet(got, tuple(a + r.astype(np.float64) for a, r in zip(ref, res)), 'dense_act_parts + residual')
+    # with a per-walker term added in front of the activation (and the skip connection behind it)
+    pre = (rand(rng, B, N), rand(rng, P, B, N), rand(rng, B, N))
+    z = rules.dense_rule(*f64(x, J, L, W), b.astype(np.float64))
+    z = tuple(t + np.expand_dims(q.astype(np.float64), -2) for t, q in zip(z, pre))
+    ref = rules.elementwise_rule(act, *z)
+    got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b), 0.0, None,
+                            tuple(dev(t) for t in pre))
+    assert_triplet(got, ref, 'dense_act_parts + pre-activation term')
+    got = K.dense_act_parts(act, dev(x), dev(L), [dev(t) for t in Js], widths, bcast, n, dev(W), dev(b), 0.0,
+                            tuple(dev(t) for t in res), tuple(dev(t) for t in pre))
+    assert_triplet(got, tuple(a + r.astype(np.float64) for a, r in zip(ref, res)), 'dense_act_parts + pre + residual')
 
 
 def test_norm_dense_full_chunk_properties():
