@@ -43,6 +43,8 @@ SIGNATURES = {
     'folx_hip_reduce_sum_window': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_float]),
     'folx_hip_reduce_max': (c_int, [_P, _P, _P, c_int64, c_int64, c_int64]),
     'folx_hip_gather_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64]),
+    'folx_hip_gather_reduce_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int32, c_int64, c_int64, c_int32, c_int64,
+                                            c_int64, c_float]),
     'folx_hip_gather_cols': (c_int, [_P, _P, _P, _P, c_int64, c_int64, c_int64, c_int32, c_int64]),
     'folx_hip_scatter_add_rows': (c_int, [_P, _P, _P, _P, c_int32, c_int32, c_int64, c_int64, c_int64]),
     'folx_hip_slogdet_fwdlap': (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int64, c_int32, c_int32]),

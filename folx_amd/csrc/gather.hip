@@ -48,6 +48,52 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float* __restric
   }
 }
 
+// The same re-indexing with a SUM OVER AN AXIS of the data folded in: the sources of a target
+// row are (row r, entry j of the reduced axis) pairs, encoded r * RED + j, and the data keeps its
+// own layout [k][B][O][RED][IV][IC] (the reduced axis in the middle, the table constant along
+// IC), so neither a slice of the reduced axis nor a permuted copy is formed:
+//   out[t][b][o][iv][ic] = alpha * sum_s data[e / RED][b][o][e % RED][iv][ic],  e = take[t][s][o * IV + iv]
+template <int VEC>
+__global__ __launch_bounds__(256) void gather_reduce_rows_kernel(const float* __restrict__ data,
+                                                                 const int32_t* __restrict__ take,
+                                                                 float* __restrict__ out, int32_t n_slots,
+                                                                 int64_t B, int64_t O, int32_t RED, int64_t IV,
+                                                                 int64_t IC, float alpha) {
+  const int64_t S_out = O * IV * IC;          // elements of one output row and walker
+  const int64_t S_in = S_out * RED;           // elements of one input row and walker
+  const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (e >= S_out) return;
+  const int64_t q = e / IC, ic = e % IC;      // q = o * IV + iv
+  const int64_t o = q / IV, iv = q % IV;
+  const int32_t t = blockIdx.z;
+  int32_t src[8];
+  const int32_t ns = n_slots < 8 ? n_slots : 8;
+  for (int s = 0; s < ns; ++s) src[s] = take[((int64_t)t * n_slots + s) * (O * IV) + q];
+  const int64_t b0 = (int64_t)blockIdx.y * GATHER_WPT;
+  const int64_t b1 = b0 + GATHER_WPT < B ? b0 + GATHER_WPT : B;
+  for (int64_t b = b0; b < b1; ++b) {
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+    for (int s = 0; s < n_slots; ++s) {
+      const int32_t en = s < 8 ? src[s] : take[((int64_t)t * n_slots + s) * (O * IV) + q];
+      if (en >= 0) {
+        const int32_t r = en / RED, j = en % RED;
+        const float* p = data + ((int64_t)r * B + b) * S_in + ((o * RED + j) * IV + iv) * IC + ic;
+        if constexpr (VEC == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(p);
+          acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+        } else {
+          acc[0] += *p;
+        }
+      }
+    }
+    float* dst = out + ((int64_t)t * B + b) * S_out + e;
+    if constexpr (VEC == 4) *reinterpret_cast<float4*>(dst) = make_float4(alpha * acc[0], alpha * acc[1], alpha * acc[2], alpha * acc[3]);
+    else *dst = alpha * acc[0];
+  }
+}
+
 __global__ __launch_bounds__(256) void scatter_add_rows_kernel(const float* __restrict__ data,
                                                                const int32_t* __restrict__ idx,
                                                                float* __restrict__ out, int64_t B,
@@ -141,5 +187,24 @@ extern "C" int folx_hip_gather_cols(void* stream, const float* data, const int32
   const unsigned gy = (unsigned)(RB < 4096 ? RB : 4096);
   gather_cols_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
       data, table, out, RB, S_in_outer * S_inner, S_out_outer, n_slots, S_inner);
+  return folx_launch_status();
+}
+
+extern "C" int folx_hip_gather_reduce_rows(void* stream, const float* data, const int32_t* take, float* out,
+                                           int32_t k_in, int32_t k_out, int32_t n_slots, int64_t B, int64_t O,
+                                           int32_t RED, int64_t IV, int64_t IC, float alpha) {
+  if (k_in < 0 || k_out < 0 || n_slots < 0 || B < 0 || O < 0 || RED < 0 || IV < 0 || IC < 0) return FOLX_HIP_EINVAL;
+  const int64_t S_out = O * IV * IC;
+  if (k_out == 0 || B == 0 || S_out == 0) return FOLX_HIP_OK;
+  if (!take || !out || (k_in > 0 && RED > 0 && !data)) return FOLX_HIP_EINVAL;
+  if ((int64_t)k_in * RED > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  const bool vec4 = IC % 4 == 0 && folx_aligned16(data) && folx_aligned16(out);
+  const int64_t threads = vec4 ? S_out / 4 : S_out;
+  const int64_t gx = (threads + 255) / 256, gy = (B + GATHER_WPT - 1) / GATHER_WPT;
+  if (gx > 0x7fffffffLL || gy > 65535 || k_out > 65535) return FOLX_HIP_ENOTSUP;
+  dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)k_out);
+  hipStream_t st = (hipStream_t)stream;
+  if (vec4) gather_reduce_rows_kernel<4><<<grid, dim3(256), 0, st>>>(data, take, out, n_slots, B, O, RED, IV, IC, alpha);
+  else gather_reduce_rows_kernel<1><<<grid, dim3(256), 0, st>>>(data, take, out, n_slots, B, O, RED, IV, IC, alpha);
   return folx_launch_status();
 }

@@ -537,6 +537,23 @@ def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
     return out
 
 
+def gather_reduce_rows(data, take, k_out, n_slots, B, O, RED, IV, IC, alpha=1.0):
+    """data (k_in, B, O, RED, IV, IC) in its own layout, take int32 (k_out, n_slots, O * IV) with
+    entries r * RED + j (or -1) -> out (k_out, B, O * IV * IC) = alpha * sum over the named
+    (row, reduced-axis entry) pairs."""
+    _chk(data, take)
+    k_in = data.shape[0]
+    assert data.numel() == k_in * B * O * RED * IV * IC and take.numel() == k_out * n_slots * O * IV
+    out = torch.empty((k_out, B, O * IV * IC), device=data.device, dtype=torch.float32)
+    with _timed('gather_reduce_rows', (k_in, k_out, n_slots, B, O, RED, IV, IC)):
+        check(
+            _lib.load().folx_hip_gather_reduce_rows(_stream(), _p(data), _p(take), _p(out), k_in, k_out, n_slots, B, O,
+                                                    RED, IV, IC, float(alpha)),
+            'gather_reduce_rows',
+        )
+    return out
+
+
 def gather_cols(data, table, S_inner=1):
     """out[rb, po, si] = sum_s data[rb, table[po, s], si]: ``data`` (RB, S_in_outer * S_inner),
     ``table`` int32 (S_out_outer, n_slots) on the device -> (RB, S_out_outer * S_inner)."""

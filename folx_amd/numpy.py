@@ -306,25 +306,25 @@ def _axes(axis, nd):
     return tuple(a % nd for a in axis)
 
 
-def sum(a, axis=None, keepdims=False, window=None):
+def sum(a, axis=None, keepdims=False, window=None, scale=None):
     """``window = (lo, hi)`` with a single ``axis``: the sum of ``a[..., lo:hi, ...]`` along that
-    axis, without forming the slice."""
+    axis, without forming the slice (what ``sum(a[..., lo:hi, ...], axis)`` becomes by itself).
+    ``scale``: a constant factor applied in the same rule (the ``1 / n`` of ``mean``)."""
     from .wrapped_functions import LazySlice
 
     if isinstance(a, LazySlice) and window is None and _axes(axis, a.ndim) == (a.axis,):
         a, window = a.a, (a.lo, a.hi)       # the sum of a slice along the reduced axis: read in place
-        shape = _shape(a)
-        axes = _axes(axis, len(shape))
-        out = _call('reduce_sum', (a,), {'axes': axes, 'window': tuple(window)})
-        if keepdims:
-            out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
-        return out
     shape = _shape(a)
     axes = _axes(axis, len(shape))
     if window is not None and not _is_triplet(a):
         a = getitem(a, tuple(slice(*window) if i == axes[0] else slice(None) for i in range(axes[0] + 1)))
         window = None
-    out = _call('reduce_sum', (a,), {'axes': axes} if window is None else {'axes': axes, 'window': tuple(window)})
+    kw = {'axes': axes}
+    if window is not None:
+        kw['window'] = tuple(window)
+    if scale is not None:
+        kw['scale'] = float(scale)
+    out = _call('reduce_sum', (a,), kw)
     if keepdims:
         out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
     return out
@@ -334,7 +334,7 @@ def mean(a, axis=None, keepdims=False, window=None):
     shape = _shape(a)
     axes = _axes(axis, len(shape))
     n = int(np.prod([shape[i] for i in axes], dtype=int)) if window is None else int(window[1] - window[0])
-    return multiply(sum(a, axis, keepdims, window), 1.0 / n)
+    return sum(a, axis, keepdims, window, scale=1.0 / n)
 
 
 def amax_const(a, axis, keepdims=False):

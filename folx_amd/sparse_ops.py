@@ -108,6 +108,41 @@ def materialize(data: torch.Tensor, idx: np.ndarray, n_out: int) -> torch.Tensor
     return out.reshape(n_out, B, *s)
 
 
+def materialize_reduced(data: torch.Tensor, slot: np.ndarray, n_out: int, axis: int, shape, window=None,
+                        alpha: float = 1.0) -> torch.Tensor:
+    """``alpha * sum`` over logical axis ``axis`` (its window ``[lo, hi)``) of sparse rows into their
+    output slots: out[t, b, kept] = alpha * sum of data[r, b, .., j, ..] over (r, j) with
+    slot[r, .., j, ..] == t (folx/jvp.py:144-171).  data (k, B, *shape) is read where it lies
+    (``folx_hip_gather_reduce_rows``); ``slot`` (k, *shape) with the window already cut out of the
+    reduced axis when ``window`` is given."""
+    k, B = data.shape[0], data.shape[1]
+    shape = tuple(shape)
+    RED = shape[axis]
+    lo, hi = (0, RED) if window is None else window
+    before, after = shape[:axis], shape[axis + 1:]
+    if n_out == 0 or k == 0 or hi == lo:
+        return zeros((n_out, B, *before, *after), data.device)
+    # (k * RED, *kept) slot map with the row id r * RED + j; entries outside the window name no slot
+    full = np.full((k, *before, RED, *after), -1, dtype=np.int32)
+    full[(slice(None), *([slice(None)] * axis), slice(lo, hi))] = slot
+    sp = np.moveaxis(full, axis + 1, 1).reshape(k * RED, *before, *after)
+    n_const = min(ia.split_inner(sp), len(after))  # trailing kept axes along which the map is constant
+    n_var = len(after) - n_const
+    O = int(np.prod(before, dtype=np.int64))
+    IV = int(np.prod(after[:n_var], dtype=np.int64))
+    IC = int(np.prod(after[n_var:], dtype=np.int64))
+    idx_c = sp[(slice(None), *([slice(None)] * (len(before) + n_var)), *([0] * n_const))]
+    key = _key(np.ascontiguousarray(idx_c), 'take_reduced', n_out)
+    cached = _TABLE_CACHE.get((key, str(data.device)))
+    if cached is None:
+        take = ia.gather_table(idx_c, n_out)
+        cached = (device_table(take.reshape(n_out, take.shape[1], O * IV), data.device), take.shape[1])
+        _TABLE_CACHE[(key, str(data.device))] = cached
+    table, n_slots = cached
+    out = K.gather_reduce_rows(data.contiguous(), table, n_out, n_slots, B, O, RED, IV, IC, alpha)
+    return out.reshape(n_out, B, *before, *after)
+
+
 def pad_rows(data: torch.Tensor, P: int) -> torch.Tensor:
     """Zero-extend a dense Jacobian to P rows (folx/utils.py:432-450)."""
     if data.shape[0] == P:

@@ -1041,57 +1041,65 @@ def reduce_sum(args, kwargs, sparsity_threshold):
     """``reduce_sum`` (SUMMATION, folx/wrapped_functions.py:388-392).  Dense: the same sum
     on x, rows and lap.  Sparse (``sparse_sum_jvp``, folx/jvp.py:89-176): static output
     mask, rows gathered into their output slots; past the threshold the rows are summed
-    straight into the dense Jacobian (:128-140)."""
+    straight into the dense Jacobian (:128-140).
+
+    ``kwargs['window'] = (lo, hi)`` (one axis): the sum of that slice of the axis, read in place
+    (a ``slice`` whose only consumer is the sum).  ``kwargs['scale']``: a constant factor applied
+    in the same launches (the ``1 / n`` of a mean; LINEAR, folx/wrapped_functions.py:361-376)."""
     (a,) = args
+    scale = float(kwargs.get('scale', 1.0))
     if not _is(a):
         if isinstance(a, BatchedArray):
             axes = _norm_axes(kwargs.get('axes'), a.ndim)
-            return BatchedArray(_reduce_tensor(a.data, 1, axes))
-        return np.sum(np.asarray(a), axis=kwargs.get('axes'))
+            return BatchedArray(_reduce_tensor(a.data, 1, axes, scale))
+        return scale * np.sum(np.asarray(a), axis=kwargs.get('axes'))
     axes = _norm_axes(kwargs.get('axes'), a.ndim)
     if len(axes) == 0:
-        return a
+        return a if scale == 1.0 else _affine_const(a, scale, mul=True, alpha=1.0, beta=0.0)
     window = kwargs.get('window')
     if window is not None:
-        # the sum of a slice along the reduced axis: read in place for dense Jacobians,
-        # otherwise the slice rule followed by the plain sum
         assert len(axes) == 1
-        lo, hi = (int(v) for v in window)
-        assert 0 <= lo <= hi <= a.shape[axes[0]]
-        if a.jacobian.x0_idx is not None:
-            idx = tuple(slice(lo, hi) if i == axes[0] else slice(None) for i in range(axes[0] + 1))
-            part = getitem_rule((a,), {'idx': idx}, sparsity_threshold)
-            return reduce_sum((part,), {'axes': kwargs.get('axes')}, sparsity_threshold)
-        return FwdLaplArray(_reduce_tensor(a.x, 1, axes, 1.0, (lo, hi)),
-                            FwdJacobian(_reduce_tensor(a.jacobian.data, 2, axes, 1.0, (lo, hi)), None),
-                            _reduce_tensor(a.laplacian, 1, axes, 1.0, (lo, hi)))
-    x = _reduce_tensor(a.x, 1, axes)
-    lap = _reduce_tensor(a.laplacian, 1, axes)
+        window = (int(window[0]), int(window[1]))
+        assert 0 <= window[0] <= window[1] <= a.shape[axes[0]]
+    x = _reduce_tensor(a.x, 1, axes, scale, window)
+    lap = _reduce_tensor(a.laplacian, 1, axes, scale, window)
     J, mask = a.jacobian.data, a.jacobian.x0_idx
     if mask is None:
-        return FwdLaplArray(x, FwdJacobian(_reduce_tensor(J, 2, axes), None), lap)
+        return FwdLaplArray(x, FwdJacobian(_reduce_tensor(J, 2, axes, scale, window), None), lap)
 
-    idx_out, slot = ia.sum_out_mask(mask, axes)
+    k = mask.shape[0]
+    mask = np.broadcast_to(mask, (k, *a.shape))
+    if window is not None:
+        # the index frame of the sum is the one of the slice (folx/jvp.py:108-146 on the sliced mask)
+        cut = tuple(slice(*window) if i == axes[0] + 1 else slice(None) for i in range(mask.ndim))
+        mask_w = mask[cut]
+    else:
+        mask_w = mask
+    idx_out, slot = ia.sum_out_mask(mask_w, axes)
     if idx_out.shape[0] > sparsity_threshold:
         logging.info(
             f'reduce_sum: output ({idx_out.shape[0]}) reaches sparsity threshold '
             f'({sparsity_threshold}); switching to dense'
         )
         n_out = int(mask.max()) + 1
-        slot, out_mask = mask, None
+        slot, out_mask = mask_w, None
     else:
         n_out, out_mask = idx_out.shape[0], idx_out
-    k = mask.shape[0]
     red_ax = [ax + 1 for ax in axes]
     first = slot
     for ax in red_ax:
         first = np.take(first, [0], axis=ax)
+    kept_shape = [n for i, n in enumerate(a.shape) if i not in axes]
     if (slot == first).all():
         # every row keeps one slot along the reduced axes: reduce rows, then re-slot
-        Jr = _reduce_tensor(J, 2, axes)
-        slot_c = first.reshape(k, *[n for i, n in enumerate(a.shape) if i not in axes])
+        Jr = _reduce_tensor(J, 2, axes, scale, window)
+        slot_c = first.reshape(k, *kept_shape)
         ident = n_out == k and (slot_c == np.arange(k).reshape(k, *([1] * (slot_c.ndim - 1)))).all()
         Jo = Jr if ident else so.materialize(Jr, slot_c, n_out)
+    elif len(axes) == 1:
+        # slots vary along the reduced axis: gather (row, entry of the axis) pairs into their slots, the
+        # data read where it lies (no slice of the window, no permuted copy)
+        Jo = so.materialize_reduced(J, slot, n_out, axes[0], a.shape, window, scale)
     else:
         # fold the reduced axes into the row axis, then gather (rows, reduced) -> slots
         nd = a.ndim
@@ -1102,6 +1110,8 @@ def reduce_sum(args, kwargs, sparsity_threshold):
         sp = np.transpose(slot, [0] + [ax + 1 for ax in axes] + [i + 1 for i in kept])
         sp = sp.reshape(k * R, *[a.shape[i] for i in kept])
         Jo = so.materialize(Jp, sp, n_out)
+        if scale != 1.0:
+            Jo = _scale_rows(Jo, Jo.shape[0], scale)
     return FwdLaplArray(x, FwdJacobian(Jo, out_mask), lap)
 
 

@@ -363,6 +363,22 @@ int folx_hip_gather_rows(void* stream, const float* data, const int32_t* take, f
                          int64_t S_outer, int64_t S_inner);
 
 /*
+ * The same re-indexing with a sum over one axis of the data folded in (sparse_sum_jvp,
+ * folx/jvp.py:89-176, for slots that vary along the reduced axis; what _factorized_dense_row_sum,
+ * folx/jvp.py:37-86, reaches with a gather after regrouping).  The data keeps its own layout
+ * [k_in][B][O][RED][IV][IC] -- the reduced axis in the middle -- and a source is a (row r, entry j
+ * of the reduced axis) pair encoded r * RED + j:
+ *   out[t][b][o][iv][ic] = alpha * sum_{s < n_slots} ( e = take[(t * n_slots + s) * O * IV + o * IV + iv];
+ *                                                      e >= 0 ? data[e / RED][b][o][e % RED][iv][ic] : 0 )
+ * take int32 [k_out][n_slots][O][IV] with values in [-1, k_in * RED); out [k_out][B][O][IV][IC].
+ * A window of the reduced axis (a slice_p in front of the sum) is a table that names no entry
+ * outside it; alpha is the 1 / n of a mean.
+ */
+int folx_hip_gather_reduce_rows(void* stream, const float* data, const int32_t* take, float* out,
+                                int32_t k_in, int32_t k_out, int32_t n_slots, int64_t B, int64_t O,
+                                int32_t RED, int64_t IV, int64_t IC, float alpha);
+
+/*
  * Static gather along the position axis with a sum over slots -- the transposed form of a
  * scatter with static indices, in which every output position lists the input positions
  * that land on it:

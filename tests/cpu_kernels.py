@@ -155,6 +155,20 @@ def gather_rows(data, take, k_out, n_slots, B, S_outer, S_inner):
     return _t(out.reshape(k_out, B, S_outer * S_inner))
 
 
+def gather_reduce_rows(data, take, k_out, n_slots, B, O, RED, IV, IC, alpha=1.0):
+    d = _n(data).reshape(data.shape[0], B, O, RED, IV, IC)
+    tk = take.cpu().numpy().reshape(k_out, n_slots, O, IV)
+    out = np.zeros((k_out, B, O, IV, IC))
+    for t in range(k_out):
+        for s_ in range(n_slots):
+            for o in range(O):
+                for iv in range(IV):
+                    e = tk[t, s_, o, iv]
+                    if e >= 0:
+                        out[t, :, o, iv] += d[e // RED, :, o, e % RED, iv]
+    return _t(alpha * out.reshape(k_out, B, O * IV * IC))
+
+
 def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
     d = _n(data).reshape(data.shape[0], B, S_outer, S_inner)
     ix = idx.cpu().numpy()
@@ -251,7 +265,7 @@ def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
 
 
 KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
-                'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_cols', 'scatter_add_rows',
+                'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_reduce_rows', 'gather_cols', 'scatter_add_rows',
                 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
 
 

@@ -28,7 +28,7 @@ NOISE = 2.0 ** -22  # relative size of the input perturbation that measures a ru
 
 _TRIPLETS = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
              'mul_sparse', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
-_SINGLE = ('rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_cols', 'scatter_add_rows')
+_SINGLE = ('rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_reduce_rows', 'gather_cols', 'scatter_add_rows')
 _DETS = ('slogdet', 'sparse_slogdet')
 
 

@@ -788,3 +788,31 @@ def test_mhsea(B, n, H, d, P, valid):
     assert_val(got[0][:, m], ref[0][:, m], 'o')
     assert_val(got[1][:, :, m], ref[1][:, :, m], 'o_jac')
     assert_lap(got[2][:, m], ref[2][:, m], 'o_lap')
+
+
+@pytest.mark.parametrize('k_in,k_out,n_slots,B,O,RED,IV,IC', [
+    (6, 48, 8, 5, 16, 16, 1, 32),     # pair stream of a FermiNet-style layer: sum over the second electron
+    (3, 7, 2, 9, 4, 5, 3, 1),         # table varies along an axis behind the reduced one, scalar tail
+    (2, 2, 1, 3, 1, 7, 1, 6),         # tail not a multiple of four
+    (4, 5, 11, 2, 3, 4, 2, 8),        # more slots than the kernel keeps in registers
+])
+def test_gather_reduce_rows(k_in, k_out, n_slots, B, O, RED, IV, IC):
+    """Re-indexing with the sum over an axis folded in, data read in its own layout."""
+    from folx_amd import kernels as K
+
+    print(f'case gather_reduce_rows {(k_in, k_out, n_slots, B, O, RED, IV, IC)}', flush=True)
+    rng = np.random.default_rng(31)
+    data = rand(rng, k_in, B, O, RED, IV, IC)
+    take = rng.integers(-1, k_in * RED, size=(k_out, n_slots, O, IV)).astype(np.int32)
+    ref = np.zeros((k_out, B, O, IV, IC))
+    d64 = data.astype(np.float64)
+    for t in range(k_out):
+        for s in range(n_slots):
+            for o in range(O):
+                for iv in range(IV):
+                    e = take[t, s, o, iv]
+                    if e >= 0:
+                        ref[t, :, o, iv] += d64[e // RED, :, o, e % RED, iv]
+    got = K.gather_reduce_rows(dev(data), dev(take.reshape(k_out, n_slots, O * IV), torch.int32), k_out, n_slots, B, O, RED,
+                               IV, IC, 0.125)
+    assert_val(got.reshape(ref.shape), 0.125 * ref)
