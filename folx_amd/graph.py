@@ -74,6 +74,11 @@ class _Captured:
             if gc_on:
                 gc.enable()
         self.tensors, self.rebuild = _flatten(out)
+        # the graph reads the cached index tables and constants by address: they stay alive with it,
+        # whatever the caches drop later
+        from . import sparse_ops
+
+        self._keepalive = sparse_ops.cached_tensors()
 
     def __call__(self, x):
         self.static_in.copy_(x)
@@ -107,9 +112,24 @@ class _Jitted:
     def batched(self, x):
         return self(x)
 
+    def invalidate(self):
+        """Drop the captured graphs: the next calls run eagerly and capture again.  Needed after
+        anything the function closes over has been REPLACED -- a weight rebound to a new tensor, a
+        numpy weight or constant changed (those are baked in by content at capture), another
+        sparsity threshold.  Device tensors updated IN PLACE need nothing: the graph reads them by
+        address."""
+        self._captured.clear()
+        self._seen.clear()
+
 
 def jit(fn):
     """Wrap ``fn(x) -> FwdLaplArray | tensors`` (``x`` a device tensor with the walker axis
     first, e.g. ``vmap(forward_laplacian(f, thr))``) so that repeated calls with the same
-    input shape replay one HIP graph.  The first call per shape runs eagerly."""
+    input shape replay one HIP graph.  The first call per shape runs eagerly.
+
+    Unlike ``jax.jit``, which takes parameters as traced arguments, the graph bakes in whatever
+    ``fn`` closes over: device tensors by address (update them in place, e.g. ``w.copy_(new)``,
+    and replays see the new values), numpy arrays by their content at capture time.  After
+    rebinding a weight to another tensor or changing a numpy weight call ``.invalidate()`` on the
+    returned object."""
     return _Jitted(fn)

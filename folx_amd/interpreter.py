@@ -26,22 +26,29 @@ def _device():
     return torch.device('cuda', torch.cuda.current_device())
 
 
-def init_forward_laplacian_state(x: torch.Tensor, sparsity: bool, weights=None) -> FwdLaplArray:
+def init_forward_laplacian_state(x: torch.Tensor, sparsity: bool, weights=None, offset: int = 0,
+                                 total: int | None = None) -> FwdLaplArray:
     """Initial triplet for an input ``x (B, *shape)`` (folx/interpreter.py:267-298):
     sparse -> one row holding the weights with ``x0_idx = arange(n).reshape(shape)``
-    (:286-293); dense -> ``diag(weights)`` reshaped to ``(n, *shape)`` (:295); lap = 0."""
+    (:286-293); dense -> ``diag(weights)`` reshaped to ``(n, *shape)`` (:295); lap = 0.
+
+    With several differentiated arguments the inputs share one index space, numbered in
+    argument order (the reference flattens the argument tree, :331-340): this argument's
+    coordinates are ``offset .. offset + n`` of ``total``."""
     B = x.shape[0]
     shape = tuple(x.shape[1:])
     n = int(np.prod(shape, dtype=int))
+    total = n if total is None else int(total)
     dev = x.device
     w = np.ones(shape, dtype=np.float32) if weights is None else np.broadcast_to(
         np.asarray(weights, dtype=np.float32), shape)
     lap = so.zeros(x.shape, dev)
     if sparsity:
         data = so.device_const(np.ascontiguousarray(w), dev).reshape(1, 1, *shape).expand(1, B, *shape).contiguous()
-        return FwdLaplArray(x, FwdJacobian(data, ia.init_mask(shape)), lap)
-    eye = (np.eye(n, dtype=np.float32) * w.reshape(-1)).reshape(n, 1, *shape)
-    data = so.device_const(eye, dev).expand(n, B, *shape).contiguous()
+        return FwdLaplArray(x, FwdJacobian(data, ia.init_mask(shape) + np.int32(offset)), lap)
+    eye = np.zeros((total, n), dtype=np.float32)
+    eye[offset:offset + n] = np.eye(n, dtype=np.float32) * w.reshape(-1)
+    data = so.device_const(eye.reshape(total, 1, *shape), dev).expand(total, B, *shape).contiguous()
     return FwdLaplArray(x, FwdJacobian(data, None), lap)
 
 
@@ -83,15 +90,19 @@ class ForwardLaplacianFn:
             elif isinstance(a, (torch.Tensor, np.ndarray)):
                 size += int(np.prod(a.shape[1:], dtype=int))
         thr = self._threshold(size)
-        n_arr = len([a for a in args if isinstance(a, (torch.Tensor, np.ndarray))])
-        if n_arr > 1 and not all(isinstance(a, FwdLaplArray) for a in args):
-            raise NotImplementedError('forward_laplacian differentiates one array argument (or pre-built triplets)')
-        for a in args:
+        # several array arguments are differentiated together: one index space, numbered in argument order
+        sizes = [int(np.prod(a.shape[1:], dtype=int)) if isinstance(a, (torch.Tensor, np.ndarray)) else 0 for a in args]
+        total, offset = int(np.sum(sizes)), 0
+        if isinstance(weights, (tuple, list)):
+            assert len(weights) == len(args), 'weights: one entry per argument'
+        for i, a in enumerate(args):
             if isinstance(a, (FwdLaplArray, BatchedArray)):
                 lapl_args.append(a)
             elif isinstance(a, (torch.Tensor, np.ndarray)):
                 x = torch.as_tensor(a, dtype=torch.float32).to(dev).contiguous()
-                lapl_args.append(init_forward_laplacian_state(x, thr > 0, weights))
+                w = weights[i] if isinstance(weights, (tuple, list)) else weights
+                lapl_args.append(init_forward_laplacian_state(x, thr > 0, w, offset, total))
+                offset += sizes[i]
             else:
                 lapl_args.append(a)
         with fnp.sparsity_threshold(thr):

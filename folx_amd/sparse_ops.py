@@ -15,8 +15,55 @@ from . import index_algebra as ia
 from . import kernels as K
 from .api import FwdJacobian
 
-_TABLE_CACHE: dict = {}
-_CONST_CACHE: dict = {}
+class _ByteLRU:
+    """Least-recently-used cache of device tensors (or tuples holding some) bounded by bytes: a loop
+    that keeps handing over fresh numpy constants or masks cannot grow it without limit.  An entry
+    that is dropped stays alive for as long as something else refers to it (a captured HIP graph
+    keeps the tensors it reads, ``graph._Captured``)."""
+
+    def __init__(self, max_bytes: int):
+        from collections import OrderedDict
+
+        self.max_bytes, self.bytes, self.d = int(max_bytes), 0, OrderedDict()
+
+    @staticmethod
+    def _size(v) -> int:
+        if isinstance(v, torch.Tensor):
+            return v.numel() * v.element_size()
+        if isinstance(v, (tuple, list)):
+            return sum(_ByteLRU._size(t) for t in v)
+        return 0
+
+    def get(self, key, default=None):
+        hit = self.d.get(key)
+        if hit is None:
+            return default
+        self.d.move_to_end(key)
+        return hit
+
+    def __setitem__(self, key, value):
+        if key in self.d:
+            self.bytes -= self._size(self.d[key])
+        self.d[key] = value
+        self.d.move_to_end(key)
+        self.bytes += self._size(value)
+        while self.bytes > self.max_bytes and len(self.d) > 1:
+            _, old = self.d.popitem(last=False)
+            self.bytes -= self._size(old)
+
+    def __len__(self):
+        return len(self.d)
+
+    def values(self):
+        return list(self.d.values())
+
+    def clear(self):
+        self.d.clear()
+        self.bytes = 0
+
+
+_TABLE_CACHE = _ByteLRU(1 << 30)   # int32 gather / scatter tables, keyed by the content of the host mask
+_CONST_CACHE = _ByteLRU(1 << 30)   # float32 constants and numpy weights, keyed by content
 _MAX_TABLE_ENTRIES = 1 << 27  # beyond this the scatter-add kernel is used instead
 
 
@@ -48,6 +95,14 @@ def device_const(arr, device) -> torch.Tensor:
         t = torch.as_tensor(a).to(device)
         _CONST_CACHE[key] = t
     return t
+
+
+def cached_tensors() -> list:
+    """Every device tensor the caches hold right now (what a captured graph must keep alive)."""
+    out = []
+    for v in _TABLE_CACHE.values() + _CONST_CACHE.values() + [r[1] for r in _ROWS_CACHE.values()]:
+        out.extend(t for t in (v if isinstance(v, (tuple, list)) else (v,)) if isinstance(t, torch.Tensor))
+    return out
 
 
 def clear_caches():
@@ -94,7 +149,9 @@ def materialize(data: torch.Tensor, idx: np.ndarray, n_out: int) -> torch.Tensor
         # row-strided stores at 4.8 (k = 3 of 96 rows at 1024 x 32 x 256: 0.58 vs 0.69 ms).
         filled = float((take >= 0).any(axis=1).mean()) if take.size else 1.0
         # (only where no two rows land on the same entry: the scatter adds atomically, and
-        # the order of colliding additions would differ from run to run)
+        # the order of colliding additions would differ from run to run.  A table past
+        # _MAX_TABLE_ENTRIES -- 512 MiB of int32 -- takes the scatter form even with collisions:
+        # its result is then exact up to the order of the atomic additions, i.e. to rounding.)
         if take.size > _MAX_TABLE_ENTRIES or (filled <= 0.25 and n_slots == 1):
             cached = ('scatter', device_table(idx_c.reshape(k, S_outer), data.device), 0)
         else:

@@ -41,15 +41,21 @@ def batched_vmap(fn, max_batch_size: int):
     batched = vmap(fn)
 
     def result(x, *args, **kwargs):
+        import numpy as np
+
         B = x.shape[0]
         if B <= max_batch_size:
             return batched(x, *args, **kwargs)
+        # every further array argument with the same leading walker axis is chunked along with x
+        # (in_axes = 0 of the reference); anything else is passed to every chunk as it is
+        walker = [isinstance(a, (torch.Tensor, np.ndarray)) and a.ndim >= 1 and a.shape[0] == B for a in args]
+        cut = lambda lo, hi: [a[lo:hi] if w else a for a, w in zip(args, walker)]
         rem = B % max_batch_size
         parts = []
         if rem > 0:
-            parts.append(batched(x[:rem], *args, **kwargs))
+            parts.append(batched(x[:rem], *cut(0, rem), **kwargs))
         for s in range(rem, B, max_batch_size):
-            parts.append(batched(x[s : s + max_batch_size], *args, **kwargs))
+            parts.append(batched(x[s : s + max_batch_size], *cut(s, s + max_batch_size), **kwargs))
         return _cat(parts)
 
     return result

@@ -1566,6 +1566,7 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
         raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
     row_axis = kwargs.get('row_axis')
     factor = kwargs.get('factor')
+    _check_matrix_size('slogdet', A.shape[-1])
     if factor is not None:
         # slogdet(A * factor): with a dense A and a sparse factor of the same shape the product is
         # formed inside the slogdet kernel; any other combination is the mul rule first
@@ -1607,12 +1608,21 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
     return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
 
 
+def _check_matrix_size(what: str, n: int, m: int = 1):
+    """The determinant / inverse / solve kernels keep one matrix per wavefront: n, m <= 32."""
+    if n > 32 or m > 32:
+        raise NotImplementedError(
+            f'{what}: the gfx950 kernels are built for matrices of at most 32 x 32 (and at most 32 right-hand sides); '
+            f'got n = {n}' + (f', m = {m}' if m > 1 else ''))
+
+
 def inv_wrapper(args, kwargs, sparsity_threshold):
     """Matrix inverse (``inv_wrapper``, folx/linear_solve.py:114-145); dense output."""
     (A,) = args
     if not _is(A):
         raise NotImplementedError('inverse of a constant: call numpy.linalg.inv')
     assert A.shape[-1] == A.shape[-2], 'inv needs square matrices'
+    _check_matrix_size('inv', A.shape[-1])
     C, CJ, CL = K.inv(A.x.contiguous(), A.jacobian.dense_array.contiguous(), A.laplacian.contiguous())
     return FwdLaplArray(C, FwdJacobian(CJ, None), CL)
 
@@ -1664,6 +1674,7 @@ def solve_wrapper(args, kwargs, sparsity_threshold):
     P = (AJ if AJ is not None else bJ).shape[0]
     full_A, full_b = (B, *batch, n, n), (B, *batch, n, m)
     ex = lambda t, shape: None if t is None else t.expand(*shape).contiguous()
+    _check_matrix_size('solve', n, m)
     y, yJ, yL = K.solve(ex(Ax, full_A), ex(AJ, (P, *full_A)), ex(AL, full_A),
                         ex(bx, full_b), ex(bJ, (P, *full_b)), ex(bL, full_b), P)
     if vector:
@@ -1730,13 +1741,28 @@ def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
     ``input_mask`` (P, B) or (P,) marks active input coordinates; either may be None.
     Jacobians are densified as in the reference (:166-178).
     """
-    del sparsity_threshold
     q, k, v, mask, input_mask = (tuple(args) + (None, None))[:5]
     bias = kwargs.get('bias')
     if not (_is(q) and _is(k) and _is(v)):
         raise NotImplementedError('multi_head_self_attention needs derivative-carrying q, k, v')
     B, dev = q.B, q.x.device
     n = q.shape[0]
+    d = q.shape[-1]
+    if n > 64 or d > 64 or d % 4 != 0:
+        # beyond what the attention kernels are built for: the same function from its primitives
+        # (two products of derivative-carrying operands around a softmax), as the reference
+        # evaluates attention that is written with einsum (folx/wrapped_functions.py:205-309)
+        if mask is not None or input_mask is not None:
+            raise NotImplementedError(
+                f'multi_head_self_attention with masks is built for n <= 64 and d <= 64 with d % 4 == 0 (got n = {n}, '
+                f'd = {d}); without masks larger shapes run through the matmul and softmax rules')
+        from . import numpy as fnp
+
+        with fnp.sparsity_threshold(sparsity_threshold):
+            sc = fnp.einsum('nhd,mhd->hnm', q, k)
+            if bias is not None:
+                sc = fnp.add(sc, fnp.transpose(bias, (1, 0, 2)))
+            return force(fnp.einsum('hnm,mhd->nhd', fnp.softmax(sc, axis=-1), v))
     if bias is None and mask is None and input_mask is None:
         sparse = _position_sparse_index(q, k, v)
         if sparse is not None:

@@ -36,3 +36,30 @@ def test_graph_replay_equals_eager(name):
         # unrelated eager work between replays
         junk = eager(torch.as_tensor(wl.sample_electrons(8, cfg.n_elec, 1.0, seed=99)).cuda())
         assert torch.isfinite(junk.x).all()
+
+
+def test_jit_weights_in_place_and_invalidate():
+    """The graph reads device weights by address: an in-place update is seen by the next replay;
+    a weight rebound to another tensor needs ``invalidate()``, after which the function is captured
+    again."""
+    from folx_amd import numpy as fnp
+
+    g = torch.Generator(device='cuda').manual_seed(2)
+    box = {'W': torch.randn(6, 8, device='cuda', generator=g) / 2}
+    fn = lambda r: fnp.sum(fnp.tanh(fnp.dot(r, box['W'])))
+    eager = folx_amd.vmap(folx_amd.forward_laplacian(fn, 0))
+    jitted = folx_amd.jit(eager)
+    x = torch.randn(5, 3, 6, device='cuda', generator=g)
+    for _ in range(3):
+        out = jitted(x)
+    assert torch.equal(out.laplacian, eager(x).laplacian)
+    box['W'].mul_(1.5)                      # in place: same address
+    assert torch.equal(jitted(x).laplacian, eager(x).laplacian)
+    box['W'] = box['W'] * 0.5               # rebound: another tensor
+    stale = jitted(x)
+    assert not torch.equal(stale.laplacian, eager(x).laplacian)
+    jitted.invalidate()
+    for _ in range(3):
+        out = jitted(x)
+    assert torch.equal(out.laplacian, eager(x).laplacian)
+    assert torch.equal(out.jacobian.dense_array, eager(x).jacobian.dense_array)

@@ -677,3 +677,61 @@ def test_stagecheck_runs_every_kernel_call_against_its_fp64_rule():
                 run_product(lambda xp, t: xp.sum(xp.tanh(t)), x, 0)
     finally:
         K.elementwise = good
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_forward_laplacian_of_several_arguments(thr):
+    """Two differentiated array arguments share one index space, numbered in argument order
+    (folx/interpreter.py:319-340): the result equals the one-argument function of their
+    concatenation; batched_vmap chunks both along the walker axis."""
+    rng = np.random.default_rng(21)
+    A, C = rng.normal(size=(3, 5)).astype(np.float32), rng.normal(size=(2, 5)).astype(np.float32)
+    x, y = rng.normal(size=(5, 4, 3)).astype(np.float32), rng.normal(size=(5, 4, 2)).astype(np.float32)
+
+    def two(xp, u, v):
+        return xp.sum(xp.multiply(xp.tanh(xp.dot(u, A)), xp.sin(xp.dot(v, C))))
+
+    def one(xp, z):  # z (4, 5) = [u | v] along the last axis, flattened argument by argument
+        u = xp.reshape(xp.getitem(z, (slice(0, 12),)), (4, 3))
+        v = xp.reshape(xp.getitem(z, (slice(12, 20),)), (4, 2))
+        return two(xp, u, v)
+
+    fl = folx_amd.forward_laplacian(lambda u, v: two(fnp, u, v), thr)
+    got = folx_amd.vmap(fl)(x, y)
+    z = np.concatenate([x.reshape(5, -1), y.reshape(5, -1)], axis=1)
+    ref = one(ob, ob.init_state(z, dtype=np.float64))
+    J = got.jacobian.dense_array.numpy()
+    assert J.shape == (20, 5)
+    np.testing.assert_allclose(got.x.numpy(), ref.x, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(J, ref.J, rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(got.laplacian.numpy(), ref.lap, rtol=1e-4, atol=1e-5)
+    chunked = folx_amd.batched_vmap(fl, 2)(x, y)
+    np.testing.assert_allclose(chunked.laplacian.numpy(), got.laplacian.numpy(), rtol=1e-6)
+    np.testing.assert_allclose(chunked.jacobian.dense_array.numpy(), J, rtol=1e-6, atol=1e-7)
+
+
+def test_attention_beyond_the_kernel_sizes_runs_through_matmul_and_softmax():
+    """n > 64 or d > 64 (or d % 4 != 0): the attention rule evaluates the same function from the
+    two-operand product and softmax rules; with masks it says what the kernel is built for."""
+    rng = np.random.default_rng(22)
+    n, H, d = 5, 2, 6   # d % 4 != 0
+    Wq, Wk, Wv = (rng.normal(size=(3, H * d)).astype(np.float32) / 2 for _ in range(3))
+    x = rng.normal(size=(2, n, 3)).astype(np.float32)
+
+    def fn(xp, t):
+        q, k, v = (xp.reshape(xp.dot(t, w), (n, H, d)) for w in (Wq, Wk, Wv))
+        return xp.sum(xp.tanh(xp.multi_head_self_attention(q, k, v)))
+
+    check_against_oracle(fn, x, 0)
+    check_against_oracle(fn, x, 6)
+    with pytest.raises(NotImplementedError, match='n <= 64'):
+        run_product(lambda xp, t: xp.sum(xp.multi_head_self_attention(
+            *(xp.reshape(xp.dot(t, w), (n, H, d)) for w in (Wq, Wk, Wv)), mask=np.ones(n, bool))), x, 0)
+
+
+def test_matrix_rules_name_their_size_limit():
+    x = np.random.default_rng(23).normal(size=(1, 33 * 33)).astype(np.float32)
+    with pytest.raises(NotImplementedError, match='32 x 32'):
+        run_product(lambda xp, t: xp.slogdet(xp.reshape(t, (33, 33)))[1], x, 0)
+    with pytest.raises(NotImplementedError, match='32 x 32'):
+        run_product(lambda xp, t: xp.sum(xp.inv(xp.reshape(t, (33, 33)))), x, 0)
