@@ -144,15 +144,12 @@ def materialize(data: torch.Tensor, idx: np.ndarray, n_out: int) -> torch.Tensor
     if cached is None:
         take = ia.gather_table(idx_c, n_out)
         n_slots = take.shape[1]
-        # A mostly empty result (few sparse rows spread over many dense ones) is a fill plus a
-        # scatter of the rows that exist: the fill writes at 6.8 TB/s, the gather kernel's
-        # row-strided stores at 4.8 (k = 3 of 96 rows at 1024 x 32 x 256: 0.58 vs 0.69 ms).
-        filled = float((take >= 0).any(axis=1).mean()) if take.size else 1.0
-        # (only where no two rows land on the same entry: the scatter adds atomically, and
-        # the order of colliding additions would differ from run to run.  A table past
-        # _MAX_TABLE_ENTRIES -- 512 MiB of int32 -- takes the scatter form even with collisions:
-        # its result is then exact up to the order of the atomic additions, i.e. to rounding.)
-        if take.size > _MAX_TABLE_ENTRIES or (filled <= 0.25 and n_slots == 1):
+        # The gather kernel writes every output entry exactly once, in memory order (5.9 TB/s also for a
+        # mostly empty result: k = 3 of 96 rows at 1024 x 32 x 256 in 0.56 ms; a fill followed by an atomic
+        # scatter of the rows that exist takes 0.58 ms and depends on the order of colliding additions).
+        # Only a table past _MAX_TABLE_ENTRIES -- 512 MiB of int32 -- takes the scatter form: its result is
+        # then exact up to the order of the atomic additions, i.e. to rounding.
+        if take.size > _MAX_TABLE_ENTRIES:
             cached = ('scatter', device_table(idx_c.reshape(k, S_outer), data.device), 0)
         else:
             cached = ('gather', device_table(take.reshape(n_out, n_slots, S_outer), data.device), n_slots)
