@@ -919,11 +919,10 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
         # The per-walker (broadcast) parts meet their rows of W ONCE per walker: a dense layer on B
         # rows whose result enters the main product in front of the activation.  The main product
         # then only contracts the per-position parts -- for a FermiNet layer 320 of 832 features.
-        ub = [u for u, b_ in zip(srcs, is_b) if b_]
-        Wb = so.weight_rows(Wt, tuple(r for r, b_ in zip(ranges, is_b) if b_))
-        cat = lambda ts: ts[0] if len(ts) == 1 else torch.cat(ts, dim=-1)
-        pre = K.dense(cat([u.x for u in ub]), cat([so.pad_rows(u.jacobian.dense_array, P) for u in ub]),
-                      cat([u.laplacian for u in ub]), Wb, None)
+        for u, (lo, hi) in [(u, r) for u, r, b_ in zip(srcs, ranges, is_b) if b_]:
+            # one product per broadcast part, each adding the sum so far in its epilogue (no concatenation)
+            pre = K.dense(u.x, so.pad_rows(u.jacobian.dense_array, P), u.laplacian, so.weight_rows(Wt, ((lo, hi),)), None,
+                          pre)
         keep = [i for i, b_ in enumerate(is_b) if not b_]
         Wt = so.weight_rows(Wt, tuple(ranges[i] for i in keep))
         parts_, srcs_ = [lc.parts[i] for i in keep], [srcs[i] for i in keep]
