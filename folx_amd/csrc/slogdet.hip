@@ -1,8 +1,9 @@
 // slogdet rule for many small matrices with dense Jacobians.
 //
 // One wavefront owns one n x n matrix (n <= 32, padded to NP in {8, 16, 32}):
-//   1. Gauss-Jordan with partial pivoting on [A | I] in LDS gives A^-1; the pivots give
-//      sign and log|det| (the same pivot sequence as an LU with partial pivoting).
+//   1. Gauss-Jordan with partial pivoting on [A | I] in registers (lane j holds column j,
+//      smallmat.h) gives A^-1; the pivots give sign and log|det| (the same pivot sequence
+//      as an LU with partial pivoting).
 //   2. tr(A^-1 lap_A) by a lane-strided product.
 //   (The matrices may be strided: a stack [batch][row][member][column] is read in place.)
 //   3. For every Jacobian row p: A_jac[p] goes from global memory straight into MFMA

@@ -1,6 +1,8 @@
 """Synthetic workloads of the benchmark configurations, written against an operator
 namespace ``xp`` (``folx_amd.numpy`` by default) so that the identical model definition
-can be evaluated by other back ends that expose the same functions.
+can be evaluated by other back ends that expose the same functions.  The models use plain
+calls only (``dot``, ``add``, ``tanh``, ``getitem``, ``mean``, ``concatenate``, ``multiply``,
+``transpose``, ``slogdet`` ...): which of them run as one fused rule is the front end's business.
 
 Weights are seeded ``numpy.random.default_rng`` draws with variance ``1 / fan_in``
 (lecun-normal-like) and zero biases; positions are per-walker arrays without the walker
