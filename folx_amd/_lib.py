@@ -24,7 +24,7 @@ SIGNATURES = {
     'folx_hip_dense_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_dense_rows_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64]),
     'folx_hip_dense_act_workspace_bytes': (c_int64, [c_int64, c_int32, c_int32, c_int32]),
-    'folx_hip_dense_act_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 8 + [c_int64, c_int32, c_int32, c_int32, _P, c_int64]),
+    'folx_hip_dense_act_fwdlap': (c_int, [_P, c_int32, c_float] + [_P] * 11 + [c_int64, c_int32, c_int32, c_int32, _P, c_int64]),
     'folx_hip_dense_act_parts_fwdlap': (c_int, [_P, c_int32, c_float, _P, _P, c_int32, _P, _P, _P, c_int32] + [_P] * 11
                                         + [c_int64, c_int32, c_int32, _P, c_int64]),
     'folx_hip_norm_dense_workspace_bytes': (c_int64, [c_int64, c_int32, c_int32, c_int32, c_int32]),

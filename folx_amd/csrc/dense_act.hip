@@ -22,6 +22,8 @@
 // per row tile in a first launch, each of which leaves its partial sums of squares in the
 // workspace; a second, short launch with one workgroup per row tile recomputes f' and f''
 // from the x tile, adds the partials in a fixed order and produces the lap row.
+#include <type_traits>
+
 #include "activations.h"
 #include "dense_act_wide.h"
 
@@ -42,6 +44,7 @@ constexpr int PART_PER_BLOCK = TM * 16 * NTHR;
 
 struct DAParams {
   const float *x, *jac, *lap, *W, *bias;
+  const float *res, *res_jac, *res_lap;  // optional triplet of the output's shape added to the activated result
   float *y, *y_jac, *y_lap;
   float* part;
   int64_t R;
@@ -193,17 +196,27 @@ __global__ __launch_bounds__(NTHR, 2) void dense_act_kernel(DAParams a) {
   const bool full = r0 + BR <= R;
   const uint32_t voff = (uint32_t)((4 * lh * N + l32) * 4);
   const int64_t step1 = (int64_t)N * 4, step5 = (int64_t)N * 20;
-  auto store = [&](float* out_rows /* row r0 of the output */, auto&& value) __attribute__((always_inline)) {
+  auto store_impl = [&](float* out_rows /* row r0 of the output */, const float* res_rows, auto&& value, auto has_res)
+      __attribute__((always_inline)) {
     if (!col_ok) return;
     gchar* rowp = (gchar*)(out_rows + (int64_t)wrow * N + wcol);
+    const gchar* resp = nullptr;
+    if constexpr (decltype(has_res)::value) resp = (const gchar*)(res_rows + (int64_t)wrow * N + wcol);
     if (full) {
 #pragma unroll
       for (int t = 0; t < TM; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          *(gfloat*)(rowp + voff) = value(t, r);
-          rowp += (r % 4 == 3) ? step5 : step1;
+          float v = value(t, r);
+          if constexpr (decltype(has_res)::value) v += *(const gfloat*)(resp + voff);
+          *(gfloat*)(rowp + voff) = v;
+          const int64_t st = (r % 4 == 3) ? step5 : step1;
+          rowp += st;
           asm volatile("" : "+s"(rowp));
+          if constexpr (decltype(has_res)::value) {
+            resp += st;
+            asm volatile("" : "+s"(resp));
+          }
         }
     } else {
 #pragma unroll
@@ -211,11 +224,25 @@ __global__ __launch_bounds__(NTHR, 2) void dense_act_kernel(DAParams a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = t * 32 + 8 * (r / 4) + r % 4;
-          if (r0 + wrow + row + 4 * lh < R) *(gfloat*)(rowp + voff) = value(t, r);
-          rowp += (r % 4 == 3) ? step5 : step1;
+          if (r0 + wrow + row + 4 * lh < R) {
+            float v = value(t, r);
+            if constexpr (decltype(has_res)::value) v += *(const gfloat*)(resp + voff);
+            *(gfloat*)(rowp + voff) = v;
+          }
+          const int64_t st = (r % 4 == 3) ? step5 : step1;
+          rowp += st;
           asm volatile("" : "+s"(rowp));
+          if constexpr (decltype(has_res)::value) {
+            resp += st;
+            asm volatile("" : "+s"(resp));
+          }
         }
     }
+  };
+  // res_rows = row r0 of the matching residual array, or nullptr (the same for the whole workgroup)
+  auto store = [&](float* out_rows, const float* res_rows, auto&& value) __attribute__((always_inline)) {
+    if (res_rows != nullptr) store_impl(out_rows, res_rows, value, std::true_type{});
+    else store_impl(out_rows, res_rows, value, std::false_type{});
   };
 
   float d1[TM][16], d2[TM][16], ssq[TM][16];
@@ -240,12 +267,14 @@ __global__ __launch_bounds__(NTHR, 2) void dense_act_kernel(DAParams a) {
     for (int t = 0; t < TM; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) ssq[t][r] += acc[t][r] * acc[t][r];
-    store(a.y_jac + ((int64_t)(p0 + it - 1) * R + r0) * N, [&](int t, int r) { return d1[t][r] * acc[t][r]; });
+    const int64_t joff = ((int64_t)(p0 + it - 1) * R + r0) * N;
+    store(a.y_jac + joff, a.res_jac ? a.res_jac + joff : nullptr, [&](int t, int r) { return d1[t][r] * acc[t][r]; });
   };
   auto lap_step = [&](const float* cur) __attribute__((always_inline)) {
     floatx16 acc[TM];
     compute(cur, acc);
-    store(a.y_lap + r0 * N, [&](int t, int r) { return d1[t][r] * acc[t][r] + d2[t][r] * ssq[t][r]; });
+    store(a.y_lap + r0 * N, a.res_lap ? a.res_lap + r0 * N : nullptr,
+          [&](int t, int r) { return d1[t][r] * acc[t][r] + d2[t][r] * ssq[t][r]; });
   };
 
   issue(tile_src(0), As0);
@@ -270,7 +299,8 @@ __global__ __launch_bounds__(NTHR, 2) void dense_act_kernel(DAParams a) {
         break;
     }
 #undef FOLX_DA_CASE
-    if (mode == 0 || (mode == 1 && g == 0)) store(a.y + r0 * N, [&](int t, int r) { return o[t][r]; });
+    if (mode == 0 || (mode == 1 && g == 0))
+      store(a.y + r0 * N, a.res ? a.res + r0 * N : nullptr, [&](int t, int r) { return o[t][r]; });
   }
   // Jacobian rows: odd steps read As1, even steps As0
   int it = 1;
@@ -322,15 +352,20 @@ extern "C" int64_t folx_hip_dense_act_workspace_bytes(int64_t R, int32_t P, int3
 }
 
 extern "C" int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const float* x, const float* jac,
-                                         const float* lap, const float* W, const float* bias, float* y,
+                                         const float* lap, const float* W, const float* bias, const float* res,
+                                         const float* res_jac, const float* res_lap, float* y,
                                          float* y_jac, float* y_lap, int64_t R, int32_t P, int32_t K, int32_t N,
                                          void* workspace, int64_t workspace_bytes) {
   if (R < 0 || P < 0 || K <= 0 || N <= 0) return FOLX_HIP_EINVAL;
+  if ((res != nullptr) != (res_lap != nullptr) || (P > 0 && (res != nullptr) != (res_jac != nullptr)))
+    return FOLX_HIP_EINVAL;
   if (!act_fused(act)) return FOLX_HIP_ENOTSUP;
   DAPlan pl;
-  if (!plan_dense_act(R, P, K, N, pl))
+  if (!plan_dense_act(R, P, K, N, pl)) {
+    if (res) return FOLX_HIP_ENOTSUP;  // the wide path adds a skip connection only when it reads its operand in parts
     return folx_dense_act_wide((hipStream_t)stream, act, param, x, jac, lap, W, bias, y, y_jac, y_lap, R, P, K, N,
                                workspace, workspace_bytes);
+  }
   if (R == 0) return FOLX_HIP_OK;
   if (!x || !lap || !W || !y || !y_lap || (P > 0 && (!jac || !y_jac))) return FOLX_HIP_EINVAL;
   if (!folx_aligned16(x) || !folx_aligned16(lap) || (P > 0 && !folx_aligned16(jac))) return FOLX_HIP_ENOTSUP;
@@ -338,6 +373,7 @@ extern "C" int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param,
     return FOLX_HIP_EINVAL;
   DAParams prm;
   prm.x = x; prm.jac = jac; prm.lap = lap; prm.W = W; prm.bias = bias;
+  prm.res = res; prm.res_jac = res_jac; prm.res_lap = res_lap;
   prm.y = y; prm.y_jac = y_jac; prm.y_lap = y_lap;
   prm.part = (float*)workspace;
   prm.R = R; prm.P = P; prm.K = K; prm.N = N; prm.G = pl.G; prm.PG = pl.PG; prm.act = act; prm.prm = param; prm.mode = 0;

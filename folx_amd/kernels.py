@@ -156,10 +156,17 @@ def dense_act_supported(name, K, N, rows=None, P=None):
             and _wide_tiles_filled(P, rows, False))
 
 
-def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
+def dense_act_residual_supported(K, N):
+    """Layers whose fused kernel adds a skip connection in its epilogue (the narrow ones)."""
+    return 4 <= K <= 128 and K % 4 == 0 and N <= 128
+
+
+def dense_act(name, x, jac, lap, W, bias=None, param=0.0, res=None):
     """``f(x @ W + bias)`` as one rule: x (.., K), jac (P, .., K), lap (.., K), W (K, N) ->
-    the activated triplet with last dim N; the pre-activation triplet is never written."""
-    _chk(x, jac, lap, W, bias)
+    the activated triplet with last dim N; the pre-activation triplet is never written.
+    ``res`` = (x, jac, lap) of the output's shape is added to the activated result (narrow
+    layers only)."""
+    _chk(x, jac, lap, W, bias, *(res or ()))
     K, N = W.shape
     P = jac.shape[0]
     lead = tuple(x.shape[:-1])
@@ -172,11 +179,14 @@ def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
     y = torch.empty((*lead, N), device=x.device, dtype=torch.float32)
     yj = torch.empty((P, *lead, N), device=x.device, dtype=torch.float32)
     yl = torch.empty_like(y)
+    rx, rj, rl = (None, None, None) if res is None else res
+    if res is not None:
+        assert tuple(rx.shape) == tuple(y.shape) and tuple(rj.shape) == tuple(yj.shape) and tuple(rl.shape) == tuple(y.shape)
     with _timed('dense_act_fwdlap', (name, R, P, K, N)):
         check(
             lib.folx_hip_dense_act_fwdlap(
                 _stream(), ACT[name], float(param), _p(x), _p(jac), _p(lap), _p(W), _p(bias),
-                _p(y), _p(yj), _p(yl), R, P, K, N, _p(ws), nbytes
+                _p(rx), _p(rj), _p(rl), _p(y), _p(yj), _p(yl), R, P, K, N, _p(ws), nbytes
             ),
             f'dense_act_fwdlap[{name}]',
         )

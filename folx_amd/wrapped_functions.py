@@ -595,7 +595,21 @@ def _dot_then_act(h, W, kwargs, thr: int):
         dev = h.x.device
         Wt = so.device_const(W, dev)
         bt = None if bias is None else so.device_const(bias, dev)
-        y, Jy, lapy = K.dense_act(act, h.x, J, h.laplacian, Wt, bt, param)
+        res = None
+        if (_is(residual) and K.dense_act_residual_supported(*np.shape(W))
+                and tuple(residual.shape) == (*h.shape[:-1], np.shape(W)[1])
+                and residual.jacobian.data.shape[0] == J.shape[0]):
+            # a skip connection on the same row frame (both dense, or the same sparse mask) is added in
+            # the kernel's epilogue (the add rule would take the identical-masks branch, _binary_both)
+            rm = residual.jacobian.x0_idx
+            same = (rm is None and new_mask is None) or (
+                rm is not None and new_mask is not None
+                and np.array_equal(np.broadcast_to(rm, (rm.shape[0], *residual.shape)), new_mask)
+                and not ia.has_duplicates(new_mask) and (new_mask.shape[0] == 1 or ia.rows_distinct(new_mask)))
+            if same:
+                res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
+                residual = None
+        y, Jy, lapy = K.dense_act(act, h.x, J, h.laplacian, Wt, bt, param, res)
         out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
     else:
         out = dot_general((h, W), kwargs, thr)

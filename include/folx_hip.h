@@ -161,6 +161,9 @@ int folx_hip_exp_envelope_fwdlap(void* stream, const float* d, const float* d_ja
  * P >= 1), 16-byte aligned operands and act in {TANH, SILU, LOGISTIC, SOFTPLUS, EXP, SIN,
  * COS, SQUARE}; anything else returns FOLX_HIP_ENOTSUP and the caller uses the two separate
  * rules.  Outputs must not overlap inputs.
+ * res / res_jac / res_lap (all or none; shapes of y / y_jac / y_lap) are added to the activated
+ * result -- the skip connection of a residual layer (add_p, LINEAR, folx/wrapped_functions.py:365-367);
+ * narrow layers only (FOLX_HIP_ENOTSUP for a wide one: folx_hip_dense_act_parts_fwdlap takes it).
  * workspace: folx_hip_dense_act_workspace_bytes(R, P, K, N) bytes of device memory (0 for a
  * narrow layer with large R: then it may be NULL), contents irrelevant; it holds partial sums
  * over Jacobian rows between launches.  The query returns a negative code for unsupported
@@ -169,7 +172,8 @@ int folx_hip_exp_envelope_fwdlap(void* stream, const float* d, const float* d_ja
 int64_t folx_hip_dense_act_workspace_bytes(int64_t R, int32_t P, int32_t K, int32_t N);
 int folx_hip_dense_act_fwdlap(void* stream, int32_t act, float param, const float* x,
                               const float* jac, const float* lap, const float* W,
-                              const float* bias, float* y, float* y_jac, float* y_lap,
+                              const float* bias, const float* res, const float* res_jac,
+                              const float* res_lap, float* y, float* y_jac, float* y_lap,
                               int64_t R, int32_t P, int32_t K, int32_t N, void* workspace,
                               int64_t workspace_bytes);
 

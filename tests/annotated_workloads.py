@@ -97,8 +97,10 @@ def ferminet_forward(p, r, xp=None):
         else:
             h = xp.dot(f, L['v'], L['b'], act='tanh')
         if 'w' in L:
-            gn = xp.dot(g, L['w'], L['c'], act='tanh')
-            g = xp.add(g, gn) if gn.shape == g.shape else gn
+            if L['w'].shape[0] == L['w'].shape[1]:  # residual layer of the pair stream: skip connection in the epilogue
+                g = xp.dot(g, L['w'], L['c'], act='tanh', residual=g)
+            else:
+                g = xp.dot(g, L['w'], L['c'], act='tanh')
     logdets, signs = [], []
     for s, (lo, hi) in enumerate([(0, nu), (nu, n)]):
         m = hi - lo

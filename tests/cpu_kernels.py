@@ -34,10 +34,13 @@ def dense(x, jac, lap, W, bias=None, res=None, row_slice=None):
     return tuple(_t(a) for a in out)
 
 
-def dense_act(name, x, jac, lap, W, bias=None, param=0.0):
+def dense_act(name, x, jac, lap, W, bias=None, param=0.0, res=None):
     z = rules.dense_rule(_n(x), _n(jac), _n(lap), _n(W), None if bias is None else _n(bias))
     nm = {'sigmoid': 'logistic'}.get(name, name)
-    return tuple(_t(a) for a in rules.elementwise_rule(nm, *z, param))
+    out = rules.elementwise_rule(nm, *z, param)
+    if res is not None:
+        out = tuple(o + _n(r) for o, r in zip(out, res))
+    return tuple(_t(a) for a in out)
 
 
 def dense_act_parts(name, x, lap, jac_parts, widths, broadcast, group, W, bias=None, param=0.0, res=None, pre=None):

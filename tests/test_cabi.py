@@ -48,7 +48,7 @@ def test_argument_checks_return_error_codes(lib):
     assert lib.folx_hip_layernorm_fwdlap(*([null] * 9), 4, 8, 1, 1e-5) == _lib.EINVAL
     assert lib.folx_hip_mhsa_fwdlap(*([null] * 15), 1, 8, 1, 8, 1) == _lib.EINVAL
     assert lib.folx_hip_mhsea_fwdlap(*([null] * 18), 1, 8, 1, 8, 1) == _lib.EINVAL
-    assert lib.folx_hip_dense_act_fwdlap(null, 0, 0.0, *([null] * 8), 4, 1, 8, 8, null, 0) == _lib.EINVAL
+    assert lib.folx_hip_dense_act_fwdlap(null, 0, 0.0, *([null] * 11), 4, 1, 8, 8, null, 0) == _lib.EINVAL
     assert lib.folx_hip_dense_act_workspace_bytes(-1, 1, 8, 8) == _lib.EINVAL
     assert lib.folx_hip_mhsa_sparse_fwdlap(*([null] * 14), 1, 8, 1, 8, 3) == _lib.EINVAL
     assert lib.folx_hip_mul_sparse_fwdlap(*([null] * 11), 8, 4, 2, 1) == _lib.EINVAL
@@ -70,9 +70,9 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_layernorm_fwdlap(None, one, one, one, None, None, one, one, one, 4, 2048, 1, 1e-5) == _lib.ENOTSUP
     # fused / structure-aware entry points outside the sizes they are built for: the caller takes
     # the general rules instead
-    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 4, 1, 6, 8, None, 0) == _lib.ENOTSUP     # K % 4
-    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 4, 1, 256, 8, None, 0) == _lib.ENOTSUP   # K > 128
-    assert lib.folx_hip_dense_act_fwdlap(None, 3, 0.0, *([one] * 8), 4, 1, 8, 8, None, 0) == _lib.ENOTSUP     # log: not fused
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 5), None, None, None, *([one] * 3), 4, 1, 6, 8, None, 0) == _lib.ENOTSUP     # K % 4
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 5), None, None, None, *([one] * 3), 4, 1, 256, 8, None, 0) == _lib.ENOTSUP   # K > 128
+    assert lib.folx_hip_dense_act_fwdlap(None, 3, 0.0, *([one] * 5), None, None, None, *([one] * 3), 4, 1, 8, 8, None, 0) == _lib.ENOTSUP     # log: not fused
     assert lib.folx_hip_dense_act_workspace_bytes(64, 4, 8, 200) == _lib.ENOTSUP
     assert lib.folx_hip_dense_act_workspace_bytes(1 << 20, 4, 100, 100) == 0                                  # no split
     assert lib.folx_hip_dense_act_workspace_bytes(64, 64, 256, 256) == 2 * 64 * 256 * 4     # wide: 2 groups of 32 rows
@@ -80,7 +80,9 @@ def test_unsupported_sizes(lib):
     assert lib.folx_hip_dense_act_workspace_bytes(60, 33, 256, 256) == 2 * 60 * 256 * 4     # rows % 8: groups of 32
     assert lib.folx_hip_dense_act_workspace_bytes(63, 33, 256, 256) == _lib.ENOTSUP         # wide: rows % 4
     assert lib.folx_hip_dense_act_workspace_bytes(64, 33, 200, 256) == _lib.ENOTSUP         # wide: K % 16
-    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 8), 64, 33, 256, 256, None, 0) == _lib.EINVAL  # no workspace
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 5), None, None, None, *([one] * 3), 64, 33, 256, 256, None, 0) == _lib.EINVAL  # no workspace
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 11), 64, 33, 256, 256, one, 1 << 30) == _lib.ENOTSUP  # skip connection on a wide layer
+    assert lib.folx_hip_dense_act_fwdlap(None, 0, 0.0, *([one] * 5), one, None, None, *([one] * 3), 4, 1, 8, 8, None, 0) == _lib.EINVAL    # part of a residual
     assert lib.folx_hip_reduce_sum_window(None, one, one, 2, 3, 8, 5, 9, 4, 1.0) == _lib.EINVAL   # window past the axis
     assert lib.folx_hip_reduce_sum_window(None, one, one, 2, 3, 8, 5, 4, 4, 1.0) == _lib.EINVAL   # hi < lo
     # Jacobian operand in parts: host arrays of pointers, widths and broadcast flags

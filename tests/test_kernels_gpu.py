@@ -162,6 +162,11 @@ def test_dense_act(rows, P, Kd, N, bias, act):
     for rep in range(2):  # the second call finds the counters as the first one left them
         got = K.dense_act(act, dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
         assert_triplet(got, ref, f'dense_act call {rep}')
+    if K.dense_act_residual_supported(Kd, N):  # narrow layers add a skip connection in their epilogue
+        res = (rand(rng, *rows, N), rand(rng, P, *rows, N), rand(rng, *rows, N))
+        got = K.dense_act(act, dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b), 0.0,
+                          tuple(dev(t) for t in res))
+        assert_triplet(got, tuple(a + r.astype(np.float64) for a, r in zip(ref, res)), 'dense_act + residual')
 
 
 def test_dense_act_matches_two_kernels_large():
