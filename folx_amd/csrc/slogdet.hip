@@ -1,18 +1,16 @@
-// slogdet rule for many small matrices with dense Jacobians.
+// slogdet rule for many small matrices with dense Jacobians (n <= 32).
 //
-// One wavefront owns one n x n matrix (n <= 32, padded to NP in {8, 16, 32}):
+// A wavefront owns one n x n matrix (two for n <= 8):
 //   1. Gauss-Jordan with partial pivoting on [A | I] in registers (lane j holds column j,
 //      smallmat.h) gives A^-1; the pivots give sign and log|det| (the same pivot sequence
 //      as an LU with partial pivoting).
-//   2. tr(A^-1 lap_A) by a lane-strided product.
-//   (The matrices may be strided: a stack [batch][row][member][column] is read in place.)
-//   3. For every Jacobian row p: A_jac[p] goes from global memory straight into MFMA
-//      operand registers (the next row is prefetched meanwhile), M = A^-1 A_jac[p] and its
-//      transpose are two MFMA products of the same registers (operands swapped),
-//      sum_p tr(M M) is the elementwise product of the two accumulators, ld_jac[p] = tr M
-//      the lane-wise product of the operands, reduced over the wavefront 16 rows at a time
-//      through LDS.
-// The Jacobian is read exactly once; 4 n^3 flops per row on the matrix cores.
+//   2. For every Jacobian row p: A_jac[p] goes from global memory straight into MFMA
+//      operand registers (rows are requested several rows ahead), M = A^-1 A_jac[p] on the
+//      matrix cores, ld_jac[p] = tr M from the lane-wise product of the operands, and
+//      sum_p tr(M M) from M and its transpose.
+//   3. tr(A^-1 lap_A) from the same operand registers.
+// The matrices may be strided: a stack [batch][row][member][column] is read in place.
+// The Jacobian is read exactly once.
 #include "smallmat.h"
 
 namespace {
@@ -35,186 +33,91 @@ constexpr int KF = 4;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// One MFMA tile covers the matrix: 16 x 16 (v_mfma_f32_16x16x4_f32) for n <= 16, 32 x 32
-// (v_mfma_f32_32x32x2_f32) above.  Lane l holds, for step t, the element (k = KS t + l / MP,
-// lr = l % MP) of an operand: as A operand that is row lr, column k; as B operand row k,
-// column lr.  With a[t] = Ainv[lr][k] and j[t] = J[k][lr]:
+constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
+
+// 16 < n <= 32: one 32 x 32 tile (v_mfma_f32_32x32x2_f32) per wavefront.  Lane l holds, for step
+// t, the element (k = 2 t + l / 32, lr = l % 32) of an operand: as A operand that is row lr,
+// column k; as B operand row k, column lr.  With a[t] = Ainv[lr][k] and j[t] = J[k][lr]:
 //   mfma(a, j) accumulates M   = Ainv J      (A = Ainv,  B = J)
 //   mfma(j, a) accumulates M^T = J^T Ainv^T  (A = J^T,   B = Ainv^T) -- the SAME registers,
 // so the transpose that tr(M M) = sum_ab M[a][b] M^T[a][b] needs costs a second product and
 // no data movement, and tr M = sum over lanes and steps of a[t] j[t].
-template <int MP>
-struct Tile;
-template <>
-struct Tile<16> {
-  static constexpr int KS = 4, STEPS = 4, CR = 4;
-  typedef floatx4 acc_t;
-  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Tile<32> {
-  static constexpr int KS = 2, STEPS = 16, CR = 16;
-  typedef floatx16 acc_t;
-  static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
-  }
-};
-
-constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
-
-// KFT = slots of the factor's sparse Jacobian the kernel keeps in registers (>= fc.kf).
-template <int NP, bool HAS_F, int KFT = KF>
-__global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
+__global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet32_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
     float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
-    int64_t rstride, int64_t slice, int32_t share, Factor fc) {
+    int64_t rstride, int64_t slice) {
+  constexpr int NP = 32, STEPS = 16;
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
-  constexpr int MP = NP <= 16 ? 16 : 32;
-  typedef Tile<MP> T;
-  constexpr int STEPS = T::STEPS;  // = elements of the padded MP x MP tile per lane
   __shared__ float aug[NP * AUGS];
   __shared__ float trs[TRB][FOLX_WAVE + 1];
 
   const int lane = threadIdx.x;
-  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  When `share`
-  // neighbouring matrices lie in the same 128-byte lines (rows of n floats side by side), they
-  // are given to the same XCD in consecutive slots, so that every line comes from HBM once.
-  int64_t m = blockIdx.x;
-  if (share > 1) {
-    const int64_t chunk = 8 * (int64_t)share;
-    const int64_t c = m / chunk, r = m % chunk;
-    if ((c + 1) * chunk <= NM) m = c * chunk + (r % 8) * share + r / 8;
-  }
+  const int64_t m = blockIdx.x;
   // matrix m = (batch m / ND, member m % ND); element (i, j) at base + i * rstride + j
   const int64_t base = (m / ND) * bstride + (m % ND) * dstride;
-  const float* a = A + base;
 
   float logdet, sgn;
-  smallmat::gauss_jordan<NP>(aug, a, n, lane, logdet, sgn, rstride, HAS_F ? fc.x + base : nullptr);
-  float tl = HAS_F ? 0.0f : smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
+  smallmat::gauss_jordan<NP>(aug, A + base, n, lane, logdet, sgn, rstride);
+  float tl = smallmat::trace_inv_times<NP>(aug, AL + base, n, lane, rstride);
 
-  // this lane's elements (k, lr) of the padded tile: A^-1 transposed-in-place as the MFMA
-  // operand, and with a factor also F, A and the factor's sparse Jacobian rows at them
-  const int lr = lane % MP;
-  const int lq = lane / MP;
+  // this lane's elements (k, lr) of the padded tile
+  const int lr = lane % 32;
+  const int lq = lane / 32;
   float ainv[STEPS];
   bool ok[STEPS];
   int64_t eoff[STEPS];
 #pragma unroll
   for (int t = 0; t < STEPS; ++t) {
-    const int k = T::KS * t + lq;
+    const int k = 2 * t + lq;
     ok[t] = k < n && lr < n;
     // elements of the padding ask for element (0, 0): loads are never branched around, so
     // that all of them are in flight before the first wait
     eoff[t] = ok[t] ? (int64_t)k * rstride + lr : 0;
     ainv[t] = ok[t] ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
   }
-  constexpr int EF = HAS_F ? STEPS : 1;
-  float fx[EF], ax[EF], lapx[EF], fj[KFT][EF];
-  int32_t fidx[KFT][EF];
-  if constexpr (HAS_F) {
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-      const int64_t off = base + eoff[t];
-      fx[t] = fc.x[off];
-      ax[t] = A[off];
-      lapx[t] = 0.0f;
-#pragma unroll
-      for (int sl = 0; sl < KFT; ++sl) {
-        fidx[sl][t] = -1;
-        fj[sl][t] = 0.0f;
-        if (sl < fc.kf) {  // the same for all lanes
-          fidx[sl][t] = fc.idx[(int64_t)sl * fc.S_w + off % fc.S_w];
-          fj[sl][t] = fc.jac[(int64_t)sl * slice + off];
-        }
-      }
-    }
-#pragma unroll
-    for (int t = 0; t < STEPS; ++t) {
-      fx[t] = ok[t] ? fx[t] : 0.0f;
-      ax[t] = ok[t] ? ax[t] : 0.0f;
-#pragma unroll
-      for (int sl = 0; sl < KFT; ++sl) {
-        fidx[sl][t] = ok[t] ? fidx[sl][t] : -1;
-        fj[sl][t] = fidx[sl][t] >= 0 ? fj[sl][t] : 0.0f;
-      }
-    }
-  }
 
-  // Jacobian rows are requested D rows ahead: with one row in flight per wavefront the kernel
-  // would be bound by the latency of its own loads, not by HBM bandwidth.
-  constexpr int D = MP == 16 ? ((HAS_F && KFT < KF) ? 6 : 4) : 1;
   float mm = 0.0f;
-  float raw[D][STEPS];
-  auto request = [&](float (&dst)[STEPS], int p) __attribute__((always_inline)) {
+  float raw[STEPS];
+  auto request = [&](int p) __attribute__((always_inline)) {
     const float* src = AJ + (int64_t)p * slice + base;
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) dst[t] = src[eoff[t]];  // A_jac[p][k][lr], padding masked when used
+    for (int t = 0; t < STEPS; ++t) raw[t] = src[eoff[t]];  // A_jac[p][k][lr], padding masked when used
   };
+  if (P > 0) request(0);
+  for (int p = 0; p < P; ++p) {
+    float jv[STEPS];
 #pragma unroll
-  for (int d = 0; d < D; ++d)
-    if (d < P) request(raw[d], d);
-  for (int p0 = 0; p0 < P; p0 += D) {
+    for (int t = 0; t < STEPS; ++t) jv[t] = ok[t] ? raw[t] : 0.0f;
+    if (p + 1 < P) request(p + 1);  // the next row is on its way during the products
+    floatx16 c, ct;
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int p = p0 + d;
-      if (p < P) {
-        float jv[STEPS];
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) {
-          float v = ok[t] ? raw[d][t] : 0.0f;
-          if constexpr (HAS_F) {
-            float add = 0.0f;
-#pragma unroll
-            for (int sl = 0; sl < KFT; ++sl) add += fidx[sl][t] == p ? fj[sl][t] : 0.0f;
-            lapx[t] = fmaf(2.0f * v, add, lapx[t]);  // cross term 2 dA . dF of the product's Laplacian
-            v = fx[t] * v + ax[t] * add;
-          }
-          jv[t] = v;
-        }
-        if (p + D < P) request(raw[d], p + D);
-        typename T::acc_t c, ct;
-#pragma unroll
-        for (int r = 0; r < T::CR; ++r) { c[r] = 0.0f; ct[r] = 0.0f; }
-        float tr = 0.0f;
-#pragma unroll
-        for (int t = 0; t < STEPS; ++t) {
-          c = T::mfma(ainv[t], jv[t], c);    // M   = Ainv J
-          ct = T::mfma(jv[t], ainv[t], ct);  // M^T
-          tr = fmaf(ainv[t], jv[t], tr);     // this lane's part of tr M
-        }
-#pragma unroll
-        for (int r = 0; r < T::CR; ++r) mm = fmaf(c[r], ct[r], mm);
-        trs[p % TRB][lane] = tr;
-        if ((p + 1) % TRB == 0 || p + 1 == P) {
-          // ld_jac of the last rows: four lanes per row add up 16 of its 64 parts each
-          // The workgroup is one wavefront and LDS serves a wavefront's accesses in issue
-          // order, so the other lanes' writes above are seen without a barrier; a barrier's
-          // fence would also wait for the Jacobian rows requested ahead.
-          const int pb = p / TRB * TRB, pe = p + 1 - pb;
-          asm volatile("" ::: "memory");
-          const int row = lane % TRB, part = lane / TRB;
-          float sm = 0.0f;
-#pragma unroll
-          for (int l = 0; l < FOLX_WAVE / 4; ++l) sm += trs[row][part * (FOLX_WAVE / 4) + l];
-          sm += __shfl_xor(sm, 16, FOLX_WAVE);
-          sm += __shfl_xor(sm, 32, FOLX_WAVE);
-          if (part == 0 && row < pe) jac_out[(int64_t)(pb + row) * NM + m] = sm;
-          asm volatile("" ::: "memory");
-        }
-      }
-    }
-  }
-  if constexpr (HAS_F) {
+    for (int r = 0; r < 16; ++r) { c[r] = 0.0f; ct[r] = 0.0f; }
+    float tr = 0.0f;
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
-      // fx, ax, lapx and ainv are zero at the padding
-      const int64_t off = base + eoff[t];
-      const float al = fx[t] * AL[off] + ax[t] * fc.lap[off] + lapx[t];
-      tl += ainv[t] * al;  // tr(A^-1 lap A) = sum A^-1[lr][k] lap A[k][lr]
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(ainv[t], jv[t], c, 0, 0, 0);    // M   = Ainv J
+      ct = __builtin_amdgcn_mfma_f32_32x32x2f32(jv[t], ainv[t], ct, 0, 0, 0);  // M^T
+      tr = fmaf(ainv[t], jv[t], tr);                                          // this lane's part of tr M
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mm = fmaf(c[r], ct[r], mm);
+    trs[p % TRB][lane] = tr;
+    if ((p + 1) % TRB == 0 || p + 1 == P) {
+      // ld_jac of the last rows: four lanes per row add up 16 of its 64 parts each.
+      // The workgroup is one wavefront and LDS serves a wavefront's accesses in issue
+      // order, so the other lanes' writes above are seen without a barrier; a barrier's
+      // fence would also wait for the Jacobian row requested ahead.
+      const int pb = p / TRB * TRB, pe = p + 1 - pb;
+      asm volatile("" ::: "memory");
+      const int row = lane % TRB, part = lane / TRB;
+      float sm = 0.0f;
+#pragma unroll
+      for (int l = 0; l < FOLX_WAVE / 4; ++l) sm += trs[row][part * (FOLX_WAVE / 4) + l];
+      sm += __shfl_xor(sm, 16, FOLX_WAVE);
+      sm += __shfl_xor(sm, 32, FOLX_WAVE);
+      if (part == 0 && row < pe) jac_out[(int64_t)(pb + row) * NM + m] = sm;
+      asm volatile("" ::: "memory");
     }
   }
   mm = wave_sum(mm);
@@ -223,6 +126,279 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet_kernel(
     sign_out[m] = sgn;
     logdet_out[m] = logdet;
     lap_out[m] = tl - mm;
+  }
+}
+
+// n <= 16: one 16 x 16 MFMA tile per wavefront, holding one matrix (NP = 16) or two 8 x 8 matrices
+// on its diagonal blocks (NP = 8: the operands are [Ainv_0; Ainv_1] and [J_0 | J_1], K = 8, and
+// only the diagonal blocks of the product are used).  Lane l holds, for step t, the element
+// (k = 4 t + l / 16, column l % NP) of matrix (l % 16) / NP.  Per Jacobian row:
+//   M = Ainv J      NP / 4 MFMA steps (the matrix pipe and the vector ALU do not overlap on a
+//                   SIMD, so the second product M^T of the 32 x 32 kernel above is not formed),
+//   tr M            lane-wise products of the operands, summed 16 rows at a time through LDS,
+//   tr(M M)         M goes to LDS transposed (one 128-bit write per lane) and comes back as M^T in
+//                   the accumulator layout; the product with the previous row's M is taken
+//                   while this row's MFMAs run.
+// Rows are requested D rows ahead with scalar base + 32-bit lane offset addressing.
+constexpr int SLD_WPB = 4;  // wavefronts per workgroup
+
+template <int NP, bool HAS_F, int KFT = KF>
+__global__ __launch_bounds__(FOLX_WAVE * SLD_WPB, 4) void slogdet16_kernel(
+    const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
+    float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
+    float* __restrict__ lap_out, int64_t NM, int32_t n, int32_t P, int64_t ND, int64_t bstride, int64_t dstride,
+    int64_t rstride, int64_t slice, int32_t share, Factor fc) {
+  constexpr int G = 16 / NP;      // matrices per wavefront
+  constexpr int STEPS = NP / 4;   // MFMA steps = elements per lane
+  constexpr int AUGS = smallmat::Aug<NP>::stride;
+  constexpr int TS = 20;          // row stride of the transposed product in LDS (floats)
+  constexpr int TRN = 8;          // Jacobian rows whose traces are reduced together
+  // per wavefront: [A | I] during the elimination; afterwards the transposed product and the
+  // staged trace parts take its place
+  constexpr int WS = 16 * TS + TRN * (FOLX_WAVE + 1);
+  static_assert(G * smallmat::Aug<NP>::size <= WS && WS % 4 == 0, "LDS overlay");
+  __shared__ __attribute__((aligned(16))) float ws_all[SLD_WPB][WS];
+  __shared__ float fst_all[HAS_F ? SLD_WPB : 1][HAS_F ? 2 * KFT : 1][STEPS][FOLX_WAVE];
+
+  // The wavefronts of a workgroup work on neighbouring matrices and do not share data; they are
+  // one workgroup so that they start together and (with a barrier every D rows) stay together:
+  // where members lie side by side along the matrix rows, the pieces of a row that the SLD_WPB
+  // wavefronts ask for at about the same time are then one contiguous stretch of memory.
+  const int lane = threadIdx.x % FOLX_WAVE, wv = threadIdx.x / FOLX_WAVE;
+  float* aug = ws_all[wv];
+  float* mt = ws_all[wv];
+  float (*trs)[FOLX_WAVE + 1] = reinterpret_cast<float (*)[FOLX_WAVE + 1]>(ws_all[wv] + 16 * TS);
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  When `share`
+  // neighbouring workgroups read the same 128-byte lines (rows of n floats side by side), they
+  // are given to the same XCD in consecutive slots, so that every line comes from HBM once.
+  const int64_t NW = (NM + G - 1) / G;
+  int64_t wg = blockIdx.x;
+  if (share > 1) {
+    const int64_t chunk = 8 * (int64_t)share;
+    const int64_t c = wg / chunk, r = wg % chunk;
+    if ((c + 1) * chunk <= gridDim.x) wg = c * chunk + (r % 8) * share + r / 8;
+  }
+  const int64_t w = wg * SLD_WPB + wv;
+  // a wavefront past the end goes through the motions on matrix 0 (it has to meet the others at
+  // the barriers) and stores nothing
+  const bool wvalid = w < NW;
+  const int64_t m0 = wvalid ? w * G : 0;  // first matrix of this wavefront
+  auto matrix_base = [&](int64_t m) -> int64_t { return (m / ND) * bstride + (m % ND) * dstride; };
+  const int64_t base0 = matrix_base(m0);  // the same for all lanes
+
+  // tile mapping
+  const int lr = lane % 16, lq = lane / 16;
+  const int g = lr / NP, cl = lr % NP;
+  const int64_t mm_ = m0 + g;  // this lane's matrix
+  const bool mvalid = wvalid && mm_ < NM;
+  const int64_t base = mvalid ? matrix_base(mm_) : base0;
+  const uint32_t delta = (uint32_t)(base - base0);  // the launcher checks sign and range
+  bool ok[STEPS];
+  uint32_t eoff[STEPS], boff[STEPS];  // element offset inside the matrix, byte offset from base0
+#pragma unroll
+  for (int t = 0; t < STEPS; ++t) {
+    const int k = 4 * t + lq;
+    ok[t] = mvalid && k < n && cl < n;
+    // elements of the padding ask for element (0, 0) of the first matrix: loads are never
+    // branched around.  What they bring in meets a zero of A^-1 in every product below.
+    eoff[t] = ok[t] ? (uint32_t)(k * rstride + cl) : 0u;
+    boff[t] = ok[t] ? 4u * (delta + eoff[t]) : 0u;
+  }
+  // Jacobian rows are requested D rows ahead: with one row in flight per wavefront the kernel
+  // would be bound by the latency of its own loads, not by HBM bandwidth.  The first D rows are
+  // asked for before the elimination, which touches no memory after its own loads.
+  constexpr int D = 8;
+  float raw[D][STEPS];
+  auto request = [&](float (&dst)[STEPS], int p) __attribute__((always_inline)) {
+    const char* src = reinterpret_cast<const char*>(AJ + (int64_t)p * slice + base0);  // the same for all lanes
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      // the 32-bit offset is made opaque here so that it is widened next to the load, which then
+      // takes the scalar base + lane offset form (no 64-bit address arithmetic per load)
+      uint32_t o = boff[t];
+      asm volatile("" : "+v"(o));
+      dst[t] = *reinterpret_cast<const float*>(src + o);  // A_jac[p][k][cl] of this lane's matrix
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+    if (d < P) request(raw[d], d);
+
+
+  // elimination: lane mapping of smallmat (NP = 8: lanes 16 g .. 16 g + 15 work on matrix g)
+  float logdet, sgn;
+  if constexpr (G == 1) {
+    smallmat::gauss_jordan<NP>(aug, A + base0, n, lane, logdet, sgn, rstride, HAS_F ? fc.x + base0 : nullptr);
+  } else {
+    const int64_t mg = m0 + lane / 16;
+    const bool valid = wvalid && lane / 16 < G && mg < NM;
+    const int64_t bg = valid ? matrix_base(mg) : base0;
+    smallmat::gauss_jordan_groups<NP, G>(aug, A + bg, valid, n, lane, logdet, sgn, rstride,
+                                         HAS_F ? fc.x + bg : nullptr);
+    if (valid && lane % 16 == 0) {
+      sign_out[mg] = sgn;
+      logdet_out[mg] = logdet;
+    }
+  }
+
+  float ainv[STEPS];
+#pragma unroll
+  for (int t = 0; t < STEPS; ++t)  // Ainv[cl][k]
+    ainv[t] = ok[t] ? aug[g * smallmat::Aug<NP>::size + cl * AUGS + NP + 4 * t + lq] : 0.0f;
+  // With a factor: F and A at this lane's elements stay in registers; the factor's sparse Jacobian
+  // rows and their dense row numbers, needed for a few rows only, wait in LDS (fst[2 s][t][lane] row
+  // number, fst[2 s + 1][t][lane] value).
+  constexpr int EF = HAS_F ? STEPS : 1;
+  float fx[EF], ax[EF], lapx[EF];
+  int flo[EF], fhi[EF];
+  if constexpr (HAS_F) {
+    float (*fst)[STEPS][FOLX_WAVE] = fst_all[wv];
+    const int64_t wpos = base % fc.S_w;  // position of the matrix inside its walker's elements
+    float fj[KFT][STEPS];
+    int32_t fidx[KFT][STEPS];
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      const int64_t off = base + eoff[t];
+      int64_t q = wpos + eoff[t];  // eoff < S_w (checked by the launcher)
+      q = q >= fc.S_w ? q - fc.S_w : q;
+      fx[t] = fc.x[off];
+      ax[t] = A[off];
+      lapx[t] = 0.0f;
+#pragma unroll
+      for (int sl = 0; sl < KFT; ++sl) {
+        fidx[sl][t] = -1;
+        fj[sl][t] = 0.0f;
+        if (sl < fc.kf) {  // the same for all lanes
+          fidx[sl][t] = fc.idx[(int64_t)sl * fc.S_w + q];
+          fj[sl][t] = fc.jac[(int64_t)sl * slice + off];
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < STEPS; ++t) {
+      fx[t] = ok[t] ? fx[t] : 0.0f;
+      ax[t] = ok[t] ? ax[t] : 0.0f;
+      int mn = 0x7fffffff, mx = -1;
+#pragma unroll
+      for (int sl = 0; sl < KFT; ++sl) {
+        const int32_t id = ok[t] ? fidx[sl][t] : -1;
+        fst[2 * sl][t][lane] = __int_as_float(id);
+        fst[2 * sl + 1][t][lane] = id >= 0 ? fj[sl][t] : 0.0f;
+        mn = id >= 0 ? min(mn, id) : mn;
+        mx = max(mx, id);
+      }
+      // Rows of the dense Jacobian that the factor's slots of step t stand for, over the whole
+      // wavefront: the range test in the loop is scalar, so a row outside [flo, fhi] costs one
+      // multiplication per element and no compares.
+#pragma unroll
+      for (int off = FOLX_WAVE / 2; off > 0; off >>= 1) {
+        mn = min(mn, __shfl_xor(mn, off, FOLX_WAVE));
+        mx = max(mx, __shfl_xor(mx, off, FOLX_WAVE));
+      }
+      flo[t] = __builtin_amdgcn_readfirstlane(mn);
+      fhi[t] = __builtin_amdgcn_readfirstlane(mx);
+    }
+  }
+
+  float mm = 0.0f;
+  floatx4 cp;  // M of the previous row
+#pragma unroll
+  for (int r = 0; r < 4; ++r) cp[r] = 0.0f;
+  const int mt_w = lr * TS + 4 * lq;   // M[4 lq + r][lr] -> transposed tile, row lr, columns 4 lq + r
+  const int mt_r = 4 * lq * TS + lr;   // M^T[4 lq + r][lr] = transposed tile row 4 lq + r, column lr
+  // sum_ab M[a][b] M^T[a][b] of the row whose M is in cp (LDS serves the one wavefront's accesses
+  // in issue order: no barrier between the write and the reads)
+  auto square_trace = [&]() __attribute__((always_inline)) {
+    *reinterpret_cast<floatx4*>(&mt[mt_w]) = cp;
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int r = 0; r < 4; ++r) mm = fmaf(cp[r], mt[mt_r + r * TS], mm);
+    asm volatile("" ::: "memory");
+  };
+  for (int p0 = 0; p0 < P; p0 += D) {
+    __builtin_amdgcn_s_barrier();  // no fence: nothing is shared, and the rows requested ahead stay in flight
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      int p = p0 + d;
+      asm volatile("" : "+s"(p));  // a scalar of its own: compared with directly, not through p0 - index
+      if (p < P) {
+        float jv[STEPS];
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+          float v = raw[d][t];
+          if constexpr (HAS_F) {
+            const float rv = v;
+            v = fx[t] * rv;
+            if (p >= flo[t] && p <= fhi[t]) {  // the same for all lanes
+              float add = 0.0f;
+#pragma unroll
+              for (int sl = 0; sl < KFT; ++sl)
+                add += __float_as_int(fst_all[wv][2 * sl][t][lane]) == p ? fst_all[wv][2 * sl + 1][t][lane] : 0.0f;
+              lapx[t] = fmaf(2.0f * rv, add, lapx[t]);  // cross term 2 dA . dF of the product's Laplacian
+              v = fmaf(ax[t], add, v);
+            }
+          }
+          jv[t] = v;
+        }
+        if (p + D < P) request(raw[d], p + D);
+        floatx4 c;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) c[r] = 0.0f;
+        float tr = 0.0f;
+#pragma unroll
+        for (int t = 0; t < STEPS; ++t) {
+          c = __builtin_amdgcn_mfma_f32_16x16x4f32(ainv[t], jv[t], c, 0, 0, 0);  // M = Ainv J
+          tr = fmaf(ainv[t], jv[t], tr);                                       // this lane's part of tr M
+        }
+        // tr(M M) of the previous row, while this row's products are in the matrix pipe
+        square_trace();
+        cp = c;
+        trs[p % TRN][lane] = tr;
+        if ((p + 1) % TRN == 0 || p + 1 == P) {
+          // ld_jac of the last rows: eight lanes per row add up 8 of its 64 parts each; the eight
+          // lanes of a part belong to one matrix (NP = 8: part % 2).  LDS serves a wavefront's
+          // accesses in issue order, so the other lanes' writes above are seen without a
+          // barrier; a barrier's fence would also wait for the rows requested ahead.
+          const int pb = p / TRN * TRN, pe = p + 1 - pb;
+          asm volatile("" ::: "memory");
+          const int row = lane % TRN, part = lane / TRN;
+          float sm = 0.0f;
+#pragma unroll
+          for (int l = 0; l < 8; ++l) sm += trs[row][part * 8 + l];
+          if constexpr (G == 1) sm += __shfl_xor(sm, 8, FOLX_WAVE);
+          sm += __shfl_xor(sm, 16, FOLX_WAVE);
+          sm += __shfl_xor(sm, 32, FOLX_WAVE);
+          if (wvalid && part < G && row < pe && m0 + part < NM) jac_out[(int64_t)(pb + row) * NM + m0 + part] = sm;
+          asm volatile("" ::: "memory");
+        }
+      }
+    }
+  }
+  square_trace();  // the last row
+  if constexpr (G == 2) mm = (lq / 2 == g) ? mm : 0.0f;  // only the diagonal blocks belong to a matrix
+
+  // tr(A^-1 lap A), with a factor lap (A F) = F lap A + A lap F + the cross term collected above
+  float tl = 0.0f;
+#pragma unroll
+  for (int t = 0; t < STEPS; ++t) {
+    const int64_t off = base + eoff[t];
+    float al = AL[off];
+    if constexpr (HAS_F) al = fx[t] * al + ax[t] * fc.lap[off] + lapx[t];
+    tl += ainv[t] * al;  // sum A^-1[cl][k] lap A[k][cl]; ainv is zero at the padding
+  }
+  float res = tl - mm;
+  // sum over the lanes of one matrix: all of them (NP = 16) or those with the same lr / 8
+#pragma unroll
+  for (int off = 1; off < FOLX_WAVE; off <<= 1)
+    if (G == 1 || off != 8) res += __shfl_xor(res, off, FOLX_WAVE);
+  if constexpr (G == 1) {
+    if (wvalid && lane == 0) {
+      sign_out[m0] = sgn;
+      logdet_out[m0] = logdet;
+      lap_out[m0] = res;
+    }
+  } else {
+    if (lq == 0 && cl == 0 && mvalid) lap_out[mm_] = res;
   }
 }
 
@@ -314,26 +490,43 @@ int launch_slogdet(hipStream_t st, const float* A, const float* A_jac, const flo
                    float* ld_jac, float* ld_lap, int64_t NB, int64_t ND, int32_t n, int32_t P, int64_t batch_stride,
                    int64_t member_stride, int64_t row_stride, int64_t jac_stride, const Factor* fc) {
   const int64_t NM = NB * ND;
-  dim3 grid((unsigned)NM), block(FOLX_WAVE);
-  // members stored side by side along the rows with rows shorter than a 128-byte line
+  dim3 block(FOLX_WAVE);
+  if (n > 16) {
+    if (fc) return FOLX_HIP_ENOTSUP;
+    slogdet32_kernel<<<dim3((unsigned)NM), block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND,
+                                                           batch_stride, member_stride, row_stride, jac_stride);
+    return folx_launch_status();
+  }
+  // n <= 16: lane offsets inside a wavefront's matrices are 32-bit, counted from its first matrix
+  const int G = n <= 8 ? 2 : 1;
+  if (row_stride < 0 || (int64_t)n * row_stride >= (1LL << 29)) return FOLX_HIP_ENOTSUP;
+  if (G == 2 && (batch_stride < 0 || member_stride < 0 || batch_stride < (ND - 1) * member_stride ||
+                 batch_stride + member_stride >= (1LL << 29)))
+    return FOLX_HIP_ENOTSUP;
+  const int64_t NW = (NM + G - 1) / G;
+  dim3 grid((unsigned)((NW + SLD_WPB - 1) / SLD_WPB));
+  block = dim3(FOLX_WAVE * SLD_WPB);
+  // members stored side by side along the rows with rows shorter than a 128-byte line: the
+  // wavefronts that read the same lines run on the same XCD
   int32_t share = 1;
   if (member_stride == n && n * 4 < 128 && ND > 1) {
     share = 128 / (n * 4);
     while (share > 1 && ND % share != 0) share /= 2;
+    share /= G * SLD_WPB;
+    if (share < 1) share = 1;
   }
-#define FOLX_SLD_LAUNCH(NPV, HASF, KFV)                                                                   \
-  slogdet_kernel<NPV, HASF, KFV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, \
-                                                         ND, batch_stride, member_stride, row_stride, jac_stride, \
-                                                         share, fc ? *fc : Factor{})
+#define FOLX_SLD_LAUNCH(NPV, HASF, KFV)                                                                     \
+  slogdet16_kernel<NPV, HASF, KFV><<<grid, block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, \
+                                                           ND, batch_stride, member_stride, row_stride, jac_stride, \
+                                                           share, fc ? *fc : Factor{})
   if (fc) {
-    // three slots (the coordinates of one electron) leave registers for two more rows in flight
+    // three slots (the coordinates of one electron) need a quarter less LDS than four
     const bool three = fc->kf <= 3;
     if (n <= 8) { if (three) FOLX_SLD_LAUNCH(8, true, 3); else FOLX_SLD_LAUNCH(8, true, KF); }
     else { if (three) FOLX_SLD_LAUNCH(16, true, 3); else FOLX_SLD_LAUNCH(16, true, KF); }
   } else {
     if (n <= 8) FOLX_SLD_LAUNCH(8, false, KF);
-    else if (n <= 16) FOLX_SLD_LAUNCH(16, false, KF);
-    else FOLX_SLD_LAUNCH(32, false, KF);
+    else FOLX_SLD_LAUNCH(16, false, KF);
   }
 #undef FOLX_SLD_LAUNCH
   return folx_launch_status();
@@ -370,6 +563,7 @@ extern "C" int folx_hip_slogdet_scaled_fwdlap(void* stream, const float* A, cons
       (k_rows > 0 && (!F_jac || !index)))
     return FOLX_HIP_EINVAL;
   if (n > 16 || k_rows > KF || NM > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
+  if ((int64_t)(n - 1) * row_stride + n > walker_elems) return FOLX_HIP_ENOTSUP;  // a matrix lies inside one walker
   Factor fc;
   fc.x = F; fc.jac = F_jac; fc.lap = F_lap; fc.idx = index; fc.S_w = walker_elems; fc.kf = k_rows;
   return launch_slogdet((hipStream_t)stream, A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NB, ND, n, P,

@@ -103,6 +103,88 @@ __device__ __forceinline__ void gauss_jordan(float* aug, const float* __restrict
   __syncthreads();
 }
 
+// The same elimination for G <= 4 matrices with n <= 8 at once: lanes 16 g .. 16 g + 15 hold the
+// 16 columns of [A_g | I], one register per row.  The pivot column is fetched from lane 16 g + k
+// of the own group (ds_bpermute) and the row exchange is a pair of selects per row, because the
+// pivot row differs from group to group.  `a` is this lane's matrix (element (i, j) at
+// a[i * row_stride + j]); a lane with `valid` false eliminates a unit matrix and stores nothing.
+// A^-1 of group g ends up at aug[g * Aug<NP>::size + i * stride + NP + j]; logdet and sgn are
+// those of the lane's own group.
+template <int NP, int G>
+__device__ __forceinline__ void gauss_jordan_groups(float* aug, const float* __restrict__ a, bool valid, int n,
+                                                    int lane, float& logdet, float& sgn, int64_t row_stride,
+                                                    const float* __restrict__ factor = nullptr) {
+  static_assert(2 * NP == 16, "sixteen lanes per matrix");
+  constexpr int AUGS = Aug<NP>::stride;
+  const int j = lane % 16, grp = lane / 16;
+  const bool in_cols = valid && j < n;
+  float col[NP];
+  if (factor) {
+    float fv[NP];
+#pragma unroll
+    for (int r = 0; r < NP; ++r) {
+      const int64_t off = (in_cols && r < n) ? r * row_stride + j : 0;
+      col[r] = a[off];
+      fv[r] = factor[off];
+    }
+#pragma unroll
+    for (int r = 0; r < NP; ++r) col[r] *= fv[r];
+  } else {
+#pragma unroll
+    for (int r = 0; r < NP; ++r) col[r] = a[(in_cols && r < n) ? r * row_stride + j : 0];
+  }
+#pragma unroll
+  for (int r = 0; r < NP; ++r) {
+    const float unit = (j < NP ? j : j - NP) == r ? 1.0f : 0.0f;
+    col[r] = (in_cols && r < n) ? col[r] : unit;
+  }
+  logdet = 0.0f;
+  sgn = 1.0f;
+#pragma unroll
+  for (int k = 0; k < NP; ++k) {
+    if (k < n) {
+      float ck[NP];  // column k of the own group's matrix
+#pragma unroll
+      for (int r = 0; r < NP; ++r) ck[r] = __shfl(col[r], 16 * grp + k, FOLX_WAVE);
+      int piv = k;
+      float best = fabsf(ck[k]);
+#pragma unroll
+      for (int r = k + 1; r < NP; ++r) {
+        const bool take = r < n && fabsf(ck[r]) > best;
+        best = take ? fabsf(ck[r]) : best;
+        piv = take ? r : piv;
+      }
+      float ckp = ck[k], mine = col[k];
+#pragma unroll
+      for (int r = k + 1; r < NP; ++r) {
+        const bool sw = r == piv;
+        const float t = ck[r], u = col[r];
+        ck[r] = sw ? ckp : t;
+        ckp = sw ? t : ckp;
+        col[r] = sw ? mine : u;
+        mine = sw ? u : mine;
+      }
+      ck[k] = ckp;
+      col[k] = mine;
+      sgn = piv != k ? -sgn : sgn;
+      const float pv = ck[k];
+      logdet += logf(fabsf(pv));
+      sgn = pv < 0.0f ? -sgn : sgn;
+      sgn = pv == 0.0f ? 0.0f : sgn;
+      const float pr = col[k] * (1.0f / pv);
+#pragma unroll
+      for (int r = 0; r < NP; ++r)
+        if (r != k) col[r] = fmaf(-ck[r], pr, col[r]);
+      col[k] = pr;
+    }
+  }
+  if (j >= NP && grp < G) {
+#pragma unroll
+    for (int r = 0; r < NP; ++r) aug[grp * Aug<NP>::size + r * AUGS + j] = col[r];
+  }
+  __syncthreads();
+}
+
 // tr(A^-1 L) = sum_ij A^-1[j][i] L[i][j], partial sum of this lane.
 template <int NP>
 __device__ __forceinline__ float trace_inv_times(const float* aug, const float* __restrict__ l, int n, int lane,

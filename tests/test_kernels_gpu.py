@@ -506,7 +506,11 @@ def test_gather_and_scatter_rows():
 
 
 @pytest.mark.parametrize('n,P,lead', [(1, 3, (4,)), (2, 5, (3, 2)), (5, 7, (6,)), (8, 24, (4, 3)),
-                                      (16, 96, (5, 4)), (32, 20, (3, 2)), (11, 4, (7,))])
+                                      (16, 96, (5, 4)), (32, 20, (3, 2)), (11, 4, (7,)),
+                                      # two matrices per wavefront with an odd count; one matrix; a
+                                      # workgroup whose last wavefronts have no matrix; rows past a
+                                      # multiple of the staging depth
+                                      (5, 7, (7,)), (8, 13, (1,)), (16, 19, (9,)), (3, 1, (2, 5))])
 def test_slogdet(n, P, lead):
     from folx_amd import kernels as K
 
@@ -529,7 +533,9 @@ def test_slogdet(n, P, lead):
 
 
 @pytest.mark.parametrize('outer,mid,n,P', [((3,), (4,), 5, 7), ((2, 2), (16,), 16, 9), ((4,), (3, 2), 8, 5),
-                                            ((2,), (1,), 32, 4)])
+                                            ((2,), (1,), 32, 4),
+                                            # pairs of 4 x 4 matrices that straddle two batch entries
+                                            ((3,), (3,), 4, 6), ((5,), (16,), 8, 48)])
 def test_slogdet_row_axis(outer, mid, n, P):
     """Matrices whose rows sit on another axis are read in place: A (*outer, n, *mid, n)."""
     from folx_amd import kernels as K
