@@ -44,6 +44,14 @@ def _call(name, args, kwargs=None):
     return get_laplacian(name, wrap_if_missing=True)(tuple(force(a) for a in args), kwargs, current_threshold())
 
 
+def call(name_or_fn, *args, **kwargs):
+    """Apply the rule registered under ``name_or_fn`` to ``args`` -- what the reference's interpreter
+    does when it meets a primitive or a jitted function of that name (folx/interpreter.py:186-216).
+    A callable that has no rule of its own (a torch function of per-walker tensors) goes through
+    the generic rule (``folx_amd.wrapper.wrap_forward_laplacian``)."""
+    return _call(name_or_fn, args, kwargs)
+
+
 def _call_keep(name, args, kwargs=None):
     return get_laplacian(name, wrap_if_missing=True)(tuple(args), kwargs or {}, current_threshold())
 

@@ -3,8 +3,21 @@
 from __future__ import annotations
 
 from dataclasses import dataclass
+from typing import Any, Callable, Protocol
 
 from .interpreter import forward_laplacian
+
+
+class Laplacian(Protocol):
+    """folx/operators.py:19-20: ``x -> (laplacian, jacobian)``."""
+
+    def __call__(self, x: Any) -> tuple: ...
+
+
+class LaplacianOperator(Protocol):
+    """folx/operators.py:23-24: ``f -> Laplacian``."""
+
+    def __call__(self, f: Callable) -> Laplacian: ...
 
 
 class _Laplacian:

@@ -29,28 +29,35 @@ from .api import BatchedArray, FwdJacobian, FwdLaplArray
 
 ForwardLaplacian = Callable[[tuple, dict, int], Any]
 
-_LAPLACE_FN_REGISTRY: dict[str, ForwardLaplacian] = {}
+_LAPLACE_FN_REGISTRY: dict[Any, ForwardLaplacian] = {}
 
 
-def register_function(primitive_or_name: str, laplacian: ForwardLaplacian):
+def register_function(primitive_or_name, laplacian: ForwardLaplacian):
     """Register a rule under a primitive / function name (folx/wrapped_functions.py:564)."""
     _LAPLACE_FN_REGISTRY[primitive_or_name] = laplacian
 
 
-def deregister_function(primitive_or_name: str):
+def deregister_function(primitive_or_name):
     del _LAPLACE_FN_REGISTRY[primitive_or_name]
 
 
-def is_registered(primitive_or_name: str) -> bool:
+def is_registered(primitive_or_name) -> bool:
     return primitive_or_name in _LAPLACE_FN_REGISTRY
 
 
-def get_laplacian(primitive_or_name: str, wrap_if_missing: bool = False) -> ForwardLaplacian | None:
-    """folx/wrapped_functions.py:597-618.  ``wrap_if_missing`` cannot be honoured (there
-    is no autodiff to derive a rule from) and raises instead."""
+def get_laplacian(primitive_or_name, wrap_if_missing: bool = False) -> ForwardLaplacian | None:
+    """folx/wrapped_functions.py:597-618.  Keys are the reference's primitive / function names, or
+    a callable.  ``wrap_if_missing``: a callable without a rule of its own (a torch function of
+    per-walker tensors) gets the generic rule of ``folx_amd.wrapper.wrap_forward_laplacian``,
+    as the reference wraps an unknown primitive; a bare name has nothing to differentiate and
+    raises."""
     if primitive_or_name in _LAPLACE_FN_REGISTRY:
         return _LAPLACE_FN_REGISTRY[primitive_or_name]
     if wrap_if_missing:
+        if callable(primitive_or_name):
+            from .wrapper import wrap_forward_laplacian
+
+            return wrap_forward_laplacian(primitive_or_name)
         raise KeyError(
             f'{primitive_or_name!r} has no forward-Laplacian rule; register one with '
             'folx_amd.register_function'

@@ -1,0 +1,192 @@
+"""Rules built from a function instead of written by hand (folx/wrapper.py:73-176).
+
+``wrap_forward_laplacian(fn)`` turns a function of per-walker arrays into a forward-Laplacian
+rule::
+
+    y = fn(x),   J_y[p] = J_f(x) J_x[p],   lap_y = J_f(x) lap_x + sum_p J_x[p]^T H_f(x) J_x[p]
+
+(folx/wrapper.py:118-125).  The reference takes ``J_f`` and ``H_f`` from jax's autodiff; here
+``fn`` is written with torch and its derivatives come from ``torch.func`` in forward mode:
+``jvp`` for ``J_f t`` and ``jvp`` of ``jvp`` for ``t^T H_f t`` (no Hessian is ever formed), mapped
+over the Jacobian rows and the walkers with ``torch.func.vmap``.
+
+This is the ONE rule whose arithmetic does not run in ``libfolx_hip.so``: what it computes is
+defined by the caller's function alone, so it runs wherever PyTorch runs that function (on the
+GPU, through PyTorch's kernels).  Nothing that ``folx_amd`` registers by itself goes through it;
+it serves functions and primitives that have no hand-written rule (``register_function(name,
+wrap_forward_laplacian(fn))``, ``get_laplacian(fn, wrap_if_missing=True)``).  The Jacobians
+are taken dense, as the reference's full-Hessian path does past the sparsity threshold.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Callable
+
+import numpy as np
+import torch
+
+from .api import BatchedArray, FunctionFlags, FwdJacobian, FwdLaplArray
+
+__all__ = ['wrap_forward_laplacian', 'warp_without_fwd_laplacian', 'wrap_elementwise']
+
+
+def _is(a):
+    return isinstance(a, FwdLaplArray)
+
+
+def _force(a):
+    from .wrapped_functions import Deferred, force
+
+    return force(a) if isinstance(a, Deferred) else a
+
+
+def _device_of(args):
+    for a in args:
+        if _is(a):
+            return a.x.device
+        if isinstance(a, BatchedArray):
+            return a.data.device
+    return None
+
+
+def _dense_rows(t: FwdLaplArray, P: int) -> torch.Tensor:
+    """Dense Jacobian (P, B, *shape): a sparse one is materialised, missing trailing rows are zero."""
+    J = t.jacobian.dense_array
+    if J.shape[0] < P:
+        pad = J.new_zeros((P - J.shape[0], *J.shape[1:]))
+        J = torch.cat([J, pad], dim=0)
+    return J
+
+
+def _tree_map(f, tree, *rest):
+    if isinstance(tree, (tuple, list)):
+        return type(tree)(_tree_map(f, t, *[r[i] for r in rest]) for i, t in enumerate(tree))
+    return f(tree, *rest)
+
+
+def wrap_forward_laplacian(
+    fn: Callable,
+    in_axes=None,
+    flags: FunctionFlags = FunctionFlags.GENERAL,
+    name: str | None = None,
+    index_static_args=None,
+    custom_jac_hessian_jac=None,
+):
+    """folx/wrapper.py:73-138.  ``fn(*arrays, **kwargs)`` sees ONE walker: torch tensors without
+    the walker axis where the rule is given ``FwdLaplArray`` / ``BatchedArray`` arguments, and the
+    other arguments (numpy arrays, scalars, anything else) as they are.  It returns a tensor or a
+    tuple / list of tensors.
+
+    ``flags``: ``LINEAR`` skips the second-order term, as in the reference; the other flags
+    choose cheaper forms of the same term there and change nothing here.  ``in_axes`` and
+    ``index_static_args`` (which axes / arguments the reference may leave out of the Hessian) do
+    not change the result and are accepted for compatibility.  ``custom_jac_hessian_jac`` is the
+    reference's hook for a hand-written second-order term; a hand-written rule registered with
+    ``register_function`` takes its place here, so anything but ``None`` raises."""
+    if custom_jac_hessian_jac is not None:
+        raise NotImplementedError(
+            'custom_jac_hessian_jac: write the whole rule by hand and register it with register_function'
+        )
+    linear = (flags & FunctionFlags.LINEAR) == FunctionFlags.LINEAR
+    label = name or getattr(fn, '__name__', 'wrapped')
+
+    def new_fn(args: tuple, kwargs: dict[str, Any], sparsity_threshold: int):
+        from torch.func import jvp, vmap
+
+        args = tuple(_force(a) for a in args)
+        dev = _device_of(args)
+        lapl_pos = [i for i, a in enumerate(args) if _is(a)]
+        bat_pos = [i for i, a in enumerate(args) if isinstance(a, BatchedArray)]
+
+        def const(a):
+            if isinstance(a, np.ndarray) and dev is not None and a.dtype.kind == 'f':
+                return torch.as_tensor(np.ascontiguousarray(a, dtype=np.float32), device=dev)
+            return a
+
+        consts = [None if (i in lapl_pos or i in bat_pos) else const(a) for i, a in enumerate(args)]
+
+        def call(xs, bs):
+            full = list(consts)
+            for i, x in zip(lapl_pos, xs):
+                full[i] = x
+            for i, b in zip(bat_pos, bs):
+                full[i] = b
+            return fn(*full, **kwargs)
+
+        bvals = tuple(args[i].data for i in bat_pos)
+        if not lapl_pos:  # nothing carries derivatives: a plain forward pass (folx/wrapper.py:112-114)
+            if not bat_pos:
+                return call((), ())
+            out = vmap(lambda bs: call((), bs))(bvals)
+            return _tree_map(lambda t: BatchedArray(t.to(torch.float32)) if t.is_floating_point() else BatchedArray(t),
+                             out)
+
+        ts = [args[i] for i in lapl_pos]
+        P = max(t.jacobian.max_n + (1 if t.jacobian.weak else 0) for t in ts)
+        xs = tuple(t.x for t in ts)                                   # (B, *shape)
+        Js = tuple(_dense_rows(t, P).transpose(0, 1) for t in ts)     # (B, P, *shape)
+        laps = tuple(t.laplacian for t in ts)
+
+        def per_walker(xw, Jw, lw, bw):
+            g = lambda *z: call(z, bw)  # noqa: E731
+            first = lambda tv: jvp(g, xw, tv)[1]  # noqa: E731   J_f t
+            y = g(*xw)
+            Jy = vmap(first)(Jw)
+            lap = first(lw)
+            if not linear:
+                second = lambda tv: jvp(lambda *z: jvp(g, z, tv)[1], xw, tv)[1]  # noqa: E731   t^T H_f t
+                quad = vmap(second)(Jw)
+                lap = _tree_map(lambda l, q: l + q.sum(0), lap, quad)
+            return y, Jy, lap
+
+        y, Jy, lap = vmap(per_walker)(xs, Js, laps, bvals)
+
+        def pack(yv, jv, lv):
+            return FwdLaplArray(yv.contiguous(), FwdJacobian(jv.transpose(0, 1).contiguous(), None), lv.contiguous())
+
+        return _tree_map(pack, y, Jy, lap)
+
+    new_fn.__name__ = f'fwd_laplacian_{label}'
+    return new_fn
+
+
+def warp_without_fwd_laplacian(fn: Callable):
+    """folx/wrapper.py:141-154 (the reference's spelling): a rule that drops the derivatives of its
+    arguments and calls ``fn`` on the values, one walker at a time.  For functions whose result
+    carries no derivative (comparisons, rounding, index computations)."""
+
+    def wrapped(args, kwargs, sparsity_threshold: int):
+        from torch.func import vmap
+
+        args = tuple(_force(a) for a in args)
+        pos = [i for i, a in enumerate(args) if _is(a) or isinstance(a, BatchedArray)]
+        if not pos:
+            return fn(*args, **kwargs)
+        vals = tuple(args[i].x if _is(args[i]) else args[i].data for i in pos)
+
+        def call(vs):
+            full = list(args)
+            for i, v in zip(pos, vs):
+                full[i] = v
+            return fn(*full, **kwargs)
+
+        return _tree_map(BatchedArray, vmap(call)(vals))
+
+    return wrapped
+
+
+def wrap_elementwise(fn: Callable):
+    """folx/wrapper.py:157-176: ``fn`` is applied to the value, to the Jacobian rows and to the
+    Laplacian as they are (a linear map that acts on every element alone, e.g. a change of
+    sign or of units); the sparsity pattern is kept."""
+
+    def wrapped(args, kwargs, sparsity_threshold: int):
+        assert len(args) == 1
+        (x,) = (_force(args[0]),)
+        if _is(x):
+            return FwdLaplArray(fn(x.x), FwdJacobian(fn(x.jacobian.data), x.jacobian.x0_idx), fn(x.laplacian))
+        if isinstance(x, BatchedArray):
+            return BatchedArray(fn(x.data))
+        return fn(x)
+
+    return wrapped

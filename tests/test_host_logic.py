@@ -735,3 +735,74 @@ def test_matrix_rules_name_their_size_limit():
         run_product(lambda xp, t: xp.slogdet(xp.reshape(t, (33, 33)))[1], x, 0)
     with pytest.raises(NotImplementedError, match='32 x 32'):
         run_product(lambda xp, t: xp.sum(xp.inv(xp.reshape(t, (33, 33)))), x, 0)
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_generic_rule_built_from_a_torch_function(thr):
+    """folx/wrapper.py:73-138, folx/wrapped_functions.py:597-618: a function without a rule of
+    its own gets J_f J and J_f lap + sum_p J_p^T H_f J_p from autodiff (two arguments with
+    Jacobians, a constant, a tuple of results); checked against the Hessian trace of the whole
+    composition."""
+    rng = np.random.default_rng(44)
+    x = rng.normal(size=(3, 4, 3)).astype(np.float32)
+    w = rng.normal(size=(3, 2)).astype(np.float32)
+
+    def op(a, b, wc):  # per walker: a (4, 3), b (4,), wc (3, 2)
+        z = torch.sin(a @ wc) * b[:, None]
+        return z, torch.exp(-b) * a.sum()
+
+    rule = folx_amd.wrap_forward_laplacian(op)
+    folx_amd.register_function('my_op', rule)
+    try:
+        def model(r):
+            h = fnp.tanh(r)
+            s = fnp.sum(fnp.square(r), axis=-1)
+            z, e = fnp.call('my_op', h, s, w)
+            return fnp.add(fnp.sum(fnp.square(z)), fnp.sum(e))
+
+        out = folx_amd.vmap(folx_amd.forward_laplacian(model, thr))(x)
+    finally:
+        folx_amd.deregister_function('my_op')
+
+    def whole(t):
+        z, e = op(torch.tanh(t), (t * t).sum(-1), torch.as_tensor(w, dtype=t.dtype))
+        return (z * z).sum() + e.sum()
+
+    by, bJ, bL = brute_force(whole, x.astype(np.float64))
+    got = triplet_np(out)
+    np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[1], bJ.reshape(got[1].shape), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
+
+    # a callable without a registered rule is wrapped on the fly; a linear one skips the Hessian term
+    lin = folx_amd.wrap_forward_laplacian(lambda a: 2.0 * a.flip(0), flags=folx_amd.FunctionFlags.LINEAR)
+    out2 = folx_amd.vmap(folx_amd.forward_laplacian(
+        lambda r: fnp.sum(fnp.multiply(fnp.call(torch.cos, fnp.sin(r)), lin((fnp.sin(r),), {}, thr))), thr))(x)
+    by, bJ, bL = brute_force(lambda t: (torch.cos(torch.sin(t)) * 2.0 * torch.sin(t).flip(0)).sum(), x.astype(np.float64))
+    got = triplet_np(out2)
+    np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[1], bJ.reshape(got[1].shape), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
+
+
+def test_rules_that_carry_no_derivatives_or_act_elementwise():
+    """folx/wrapper.py:141-176."""
+    from folx_amd.api import BatchedArray
+
+    x = np.random.default_rng(45).normal(size=(2, 5)).astype(np.float32)
+    seen = {}
+
+    def f(r):
+        h = fnp.sin(r)
+        seen['count'] = folx_amd.warp_without_fwd_laplacian(lambda t, thr_: (t > thr_).sum())((h, 0.25), {}, 0)
+        y = folx_amd.wrap_elementwise(lambda t: -3.0 * t)((h,), {}, 0)
+        return fnp.sum(fnp.square(y))
+
+    out = folx_amd.vmap(folx_amd.forward_laplacian(f, 0))(x)
+    assert isinstance(seen['count'], BatchedArray)
+    np.testing.assert_array_equal(seen['count'].data.numpy(), (np.sin(x) > 0.25).sum(-1))
+    by, bJ, bL = brute_force(lambda t: (9.0 * torch.sin(t) ** 2).sum(), x.astype(np.float64))
+    got = triplet_np(out)
+    np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[1], bJ.reshape(got[1].shape), rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
