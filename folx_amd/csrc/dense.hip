@@ -70,26 +70,34 @@ __device__ __forceinline__ void store_tile(const floatx16 (&acc)[TM][TN], const 
     const uint32_t voff = (uint32_t)((4 * lh * N + l32) * 4);
     float* cs = C + (row0 + wr) * (int64_t)N + col0 + wc;
     const float* rsb = HAS_RES ? Rs + (row0 + wr) * (int64_t)N + col0 + wc : nullptr;
+    // The residuals of four rows are requested together, one group of four rows ahead of their
+    // use (across accumulator blocks): the stores cannot be told apart from the residual array,
+    // so a load written after a group's stores would wait for them to be issued, and every
+    // group would pay a memory round trip of its own.
+    float rs[2][4];
+    auto fetch = [&](int step, float (&dst)[4]) __attribute__((always_inline)) {
+      const int g = step % 4, j = (step / 4) % TN, i = step / (4 * TN);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const char* p = (const char*)(rsb + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
+        dst[r] = __builtin_nontemporal_load((const float*)(p + voff));
+      }
+    };
+    if constexpr (HAS_RES) fetch(0, rs[0]);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          // the residuals of four rows are requested together, then the four rows are stored
-          float rs[4];
-          if constexpr (HAS_RES) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const char* p = (const char*)(rsb + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
-              rs[r] = __builtin_nontemporal_load((const float*)(p + voff));
-            }
-          }
+          const int step = (i * TN + j) * 4 + g;
+          if constexpr (HAS_RES)
+            if (step + 1 < TM * TN * 4) fetch(step + 1, rs[(step + 1) & 1]);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             char* p = (char*)(cs + (int64_t)(i * 32 + 8 * g + r) * N + j * 32);
             float o = acc[i][j][4 * g + r] + bvals[j];
-            if constexpr (HAS_RES) o += rs[r];
+            if constexpr (HAS_RES) o += rs[step & 1][r];
             __builtin_nontemporal_store(o, (float*)(p + voff));  // written once, read by a later launch
           }
         }

@@ -398,10 +398,39 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
         }
       }
       auto rows = [&](auto full, auto has_res, auto has_pre) __attribute__((always_inline)) {
+        constexpr int GB = PT / 8;     // register groups per position
+        constexpr bool FULL = decltype(full)::value, RES = decltype(has_res)::value, PRE = decltype(has_pre)::value;
+        // What the epilogue reads from memory (skip connection, per-walker pre-activation term) is
+        // asked for one register group ahead of its use: the stores of a group cannot be told
+        // apart from these arrays, so a load written after them would wait for them to be issued,
+        // and every group would pay a round trip of its own.
+        float rbuf[2][4], pbuf[2][4];
+        auto fetch = [&](int g, float (&rb)[4], float (&pb)[4]) __attribute__((always_inline)) {
+          const int b = g / GB;
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const int pl = 8 * (g % GB) + rr;
+            const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
+            const bool live = FULL || (p0 + 4 * lh + pl < P && gc < N);
+            rb[rr] = 0.0f;
+            pb[rr] = 0.0f;
+            if constexpr (PRE) {
+              int prow = p0 + 4 * lh + pl;  // rows past P of a ragged tile are neither stored nor summed
+              if constexpr (!FULL) prow = prow < P ? prow : P - 1;
+              pb[rr] = prep[b][(int64_t)prow * pre_pstride];
+            }
+            if constexpr (RES) {
+              if constexpr (FULL) rb[rr] = __builtin_nontemporal_load(resp + off);
+              else if (live) rb[rr] = resp[off];
+            }
+          }
+        };
+        if constexpr (RES || PRE) fetch(0, rbuf[0], pbuf[0]);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          constexpr int GB = PT / 8;     // register groups per position
           const int b = g / GB;          // position of this group inside the block
+          if constexpr (RES || PRE)
+            if (g + 1 < 4) fetch(g + 1, rbuf[(g + 1) & 1], pbuf[(g + 1) & 1]);
           float ap[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
           if constexpr (NORM) {
             const float4* sp = reinterpret_cast<const float4*>(st + i * 32 + 8 * g + 4 * lh);
@@ -420,19 +449,15 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
             }
             const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
             float* o = out + off;
-            if constexpr (decltype(has_pre)::value) {
-              int prow = p0 + 4 * lh + pl;  // rows past P of a ragged tile are neither stored nor summed
-              if constexpr (!decltype(full)::value) prow = prow < P ? prow : P - 1;
-              v += prep[b][(int64_t)prow * pre_pstride];
-            }
-            if constexpr (decltype(full)::value) {
+            if constexpr (PRE) v += pbuf[g & 1][rr];
+            if constexpr (FULL) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
               float w = d1[b] * v;
-              if constexpr (decltype(has_res)::value) w += __builtin_nontemporal_load(resp + off);
+              if constexpr (RES) w += rbuf[g & 1][rr];
               __builtin_nontemporal_store(w, o);
             } else if (p0 + 4 * lh + pl < P) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
-              if (gc < N) *o = d1[b] * v + (decltype(has_res)::value ? resp[off] : 0.0f);
+              if (gc < N) *o = d1[b] * v + (RES ? rbuf[g & 1][rr] : 0.0f);
             }
           }
         }
