@@ -72,18 +72,33 @@ __global__ __launch_bounds__(256) void gather_reduce_rows_kernel(const float* __
   float acc[VEC];
 #pragma unroll
   for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
-  for (int s = 0; s < n_slots; ++s) {
-    const int32_t en = take[((int64_t)t * n_slots + s) * (O * IV) + q];
-    if (en >= 0) {
-      const int32_t r = en / RED, j = en % RED;
-      const float* p = data + ((int64_t)r * B + b) * S_in + ((o * RED + j) * IV + iv) * IC + ic;
-      if constexpr (VEC == 4) {
-        const float4 v = folx_ld_stream4(p);
-        acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
-      } else {
-        acc[0] += *p;
+  // Eight slots at a time: first their table entries, then all their loads, then the sums in slot
+  // order -- a slot-by-slot loop would wait for a table entry and then for its load, eight times over.
+  for (int s0 = 0; s0 < n_slots; s0 += 8) {
+    int32_t en[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      en[u] = s0 + u < n_slots ? take[((int64_t)t * n_slots + s0 + u) * (O * IV) + q] : -1;
+    float val[8][VEC];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) val[u][v] = 0.0f;
+      if (en[u] >= 0) {
+        const int32_t r = en[u] / RED, j = en[u] % RED;
+        const float* p = data + ((int64_t)r * B + b) * S_in + ((o * RED + j) * IV + iv) * IC + ic;
+        if constexpr (VEC == 4) {
+          const float4 v = folx_ld_stream4(p);
+          val[u][0] = v.x; val[u][1] = v.y; val[u][2] = v.z; val[u][3] = v.w;
+        } else {
+          val[u][0] = *p;
+        }
       }
     }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) acc[v] += val[u][v];
   }
   float* dst = out + ((int64_t)t * B + b) * S_out + e;
   if constexpr (VEC == 4) folx_st_stream4(dst, make_float4(alpha * acc[0], alpha * acc[1], alpha * acc[2], alpha * acc[3]));

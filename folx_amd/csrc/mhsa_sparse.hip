@@ -20,8 +20,9 @@
 //
 // One workgroup of 512 threads per (walker, head); q, k, v, o, p and the n x n accumulators
 // live in LDS (rows of d + 4 floats, so that 16 threads reading 16 bytes each from 16
-// different rows cover all banks); dot products run on 128-bit LDS reads; the three vectors of
-// the next position are fetched while the current one is worked on.
+// different rows cover all banks); the n x n x d products (scores, alpha, beta, the Laplacian's
+// score term) run on the matrix cores from those rows, the sums over j on 128-bit LDS reads; the
+// vectors of the next group of positions are fetched while the current one is worked on.
 #include <atomic>
 
 #include "common.h"
@@ -53,9 +54,82 @@ __device__ __forceinline__ float sa_dot(const float* u, const float* m, int d4) 
 constexpr int SA_MAXPASS = 64 / SA_RP;  // n <= 64: rows i = SA_RP pass + tid / 16
 constexpr int SA_E = 4;        // sequence positions worked on together
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// Workgroup barrier for data exchanged through LDS only.  __syncthreads() also waits for every
+// global load and store of the wavefront to complete (its fence covers global memory), which
+// here would expose the latency of the vectors requested one group ahead and of the output
+// rows just stored, once per group.
+__device__ __forceinline__ void sa_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// One 16 x 16 tile of X Y^T on the matrix cores (v_mfma_f32_16x16x4_f32): X and Y are row-major in
+// LDS, C[r][c] = sum_k X[r][k] Y[c][k] over k < 4 * d4.  Lane l feeds X[l % 16][4 s + l / 16] and
+// Y[l % 16][4 s + l / 16] in step s and receives C[4 (l / 16) + i][l % 16] in register i.  With row
+// strides of 4 (mod 32) floats the 64 reads of a step fall on all banks twice, the minimum.  Rows
+// past the end of X or Y (still inside the workgroup's LDS: every operand is followed by other
+// arrays) only reach tile rows / columns that the caller does not keep.
+__device__ __forceinline__ floatx4 sa_tile_nt(const float* X, int ldx, const float* Y, int ldy, int d4, int lane) {
+  const float* xp = X + (lane % 16) * ldx + lane / 16;
+  const float* yp = Y + (lane % 16) * ldy + lane / 16;
+  // two accumulators, even and odd steps: independent chains for the matrix pipe, and half as many
+  // roundings in a row for every element
+  floatx4 c0 = {0.0f, 0.0f, 0.0f, 0.0f}, c1 = {0.0f, 0.0f, 0.0f, 0.0f};
+  int s = 0;
+  for (; s + 8 <= d4; s += 8) {  // the operands of eight steps are read before the first product
+    float xv[8], yv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { xv[u] = xp[4 * (s + u)]; yv[u] = yp[4 * (s + u)]; }
+#pragma unroll
+    for (int u = 0; u < 8; u += 2) {
+      c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u], yv[u], c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u + 1], yv[u + 1], c1, 0, 0, 0);
+    }
+  }
+  for (; s < d4; ++s) c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(xp[4 * s], yp[4 * s], c0, 0, 0, 0);
+  return c0 + c1;
+}
+
+// Two products at once, C0 = X0 Y0^T (rows < nr0 of X0, rows < nc0 of Y0) and C1 = X1 Y1^T, their
+// 16 x 16 tiles dealt to the workgroup's wavefronts as one list; `put(which, r, c, value)`
+// receives every element.  (One product: nr1 = 0.)
+template <class Put>
+__device__ __forceinline__ void sa_products_nt(const float* X0, int ldx0, int nr0, const float* Y0, int ldy0, int nc0,
+                                               const float* X1, int ldx1, int nr1, const float* Y1, int ldy1, int nc1,
+                                               int d4, int tid, Put put) {
+  const int lane = tid % 64, wave = tid / 64;
+  const int tc0 = (nc0 + 15) / 16, t0 = ((nr0 + 15) / 16) * tc0;
+  const int tc1 = (nc1 + 15) / 16, t1 = ((nr1 + 15) / 16) * tc1;
+  for (int t = wave; t < t0 + t1; t += SA_NT / 64) {
+    const bool second = t >= t0;
+    const int tt = second ? t - t0 : t, tc = second ? tc1 : tc0;
+    const int r0 = (tt / tc) * 16, c0 = (tt % tc) * 16;
+    const float* X = second ? X1 : X0;
+    const float* Y = second ? Y1 : Y0;
+    const int ldx = second ? ldx1 : ldx0, ldy = second ? ldy1 : ldy0;
+    const floatx4 c = sa_tile_nt(X + r0 * ldx, ldx, Y + c0 * ldy, ldy, d4, lane);
+    const int col = c0 + lane % 16;
+    const int nr = second ? nr1 : nr0, nc = second ? nc1 : nc0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = r0 + 4 * (lane / 16) + i;
+      if (row < nr && col < nc) put(second, row, col, c[i]);
+    }
+  }
+}
+
+template <class Put>
+__device__ __forceinline__ void sa_product_nt(const float* X, int ldx, int nr, const float* Y, int ldy, int nc,
+                                              int d4, int tid, Put put) {
+  sa_products_nt(X, ldx, nr, Y, ldy, nc, X, ldx, 0, Y, ldy, 0, d4, tid,
+                 [&](bool, int r, int c, float v) { put(r, c, v); });
+}
+
 __host__ __device__ inline int64_t sa_lds_floats(int n, int d, int K) {
   const int dp = d + 4, np1 = n + 1;
-  return 4LL * n * dp + 4LL * n * np1 + SA_E * (4LL * K * d + 2LL * K * n + 2LL * K) + 5LL * n + (int64_t)K * n;
+  return 4LL * n * dp + 4LL * n * np1 + SA_E * (2LL * K * dp + 2LL * K * d + 2LL * K * n + 2LL * K) + 5LL * n +
+         (int64_t)K * n;
 }
 
 __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
@@ -70,9 +144,9 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
   float* AA = pS + n * np1;
   float* BB = AA + n * np1;
   float* AR = BB + n * np1;
-  float* aS = AR + n * np1;             // [SA_E][K][d] vectors of the positions in work
-  float* bS = aS + SA_E * K * d;
-  float* wS = bS + SA_E * K * d;
+  float* aS = AR + n * np1;             // [SA_E][K][dp] vectors a, b of the positions in work (MFMA operands)
+  float* bS = aS + SA_E * K * dp;
+  float* wS = bS + SA_E * K * dp;       // [SA_E][K][d]
   float* gamS = wS + SA_E * K * d;
   float* alS = gamS + SA_E * K * d;     // [SA_E][K][n]
   float* beS = alS + SA_E * K * n;
@@ -103,14 +177,11 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
   load_tile(a.v, vS);
   for (int it = tid; it < 3 * n * np1; it += SA_NT) AA[it] = 0.0f;  // AA, BB, AR are contiguous
   for (int it = tid; it < K * n; it += SA_NT) idxS[it] = a.index[it];
-  __syncthreads();
+  sa_barrier();
 
   // p = softmax(q k^T)
-  for (int it = tid; it < n * n; it += SA_NT) {
-    const int i = it / n, j = it - i * n;
-    pS[i * np1 + j] = sa_dot(qS + i * dp, kS + j * dp, d4);
-  }
-  __syncthreads();
+  sa_product_nt(qS, dp, n, kS, dp, n, d4, tid, [&](int i, int j, float v) { pS[i * np1 + j] = v; });
+  sa_barrier();
   if (tid < n) {
     float* row = pS + tid * np1;
     float m = row[0];
@@ -120,7 +191,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     const float rz = 1.0f / z;
     for (int j = 0; j < n; ++j) row[j] *= rz;
   }
-  __syncthreads();
+  sa_barrier();
   // o = p v
   for (int it = tid; it < n * d4; it += SA_NT) {
     const int i = it / d4, t4 = it - i * d4;
@@ -139,18 +210,23 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
   // float4 per thread and position, requested one group ahead of its use.
   const int nvec = 3 * K * d4;
   const int pf_which = tid / (K * d4), pf_sl = (tid / d4) % K, pf_t4 = tid % d4;
+  // this thread's source array and offset inside a position's vectors, in registers (selected once:
+  // an array chosen per lane inside the loop would be read from the argument block with a
+  // vector load, a memory round trip in front of every request)
+  const float* pf_src = a.qs;
+  if (pf_which == 1) pf_src = a.ks;
+  if (pf_which == 2) pf_src = a.vs;
+  pf_src += pf_sl * Srow + 4 * pf_t4;
   auto fetch = [&](int e0, float4 (&pf)[SA_E]) {
 #pragma unroll
     for (int ee = 0; ee < SA_E; ++ee) {
       pf[ee] = make_float4(0.f, 0.f, 0.f, 0.f);
       const int e = e0 + ee;
-      if (tid < nvec && e < n && idxS[pf_sl * n + e] >= 0) {
-        const float* src = pf_which == 0 ? a.qs : (pf_which == 1 ? a.ks : a.vs);
-        pf[ee] = *reinterpret_cast<const float4*>(src + pf_sl * Srow + grow(e) + 4 * pf_t4);
-      }
+      if (tid < nvec && e < n && idxS[pf_sl * n + e] >= 0)
+        pf[ee] = *reinterpret_cast<const float4*>(pf_src + grow(e));
     }
   };
-  __syncthreads();  // index table, o and p are in LDS
+  sa_barrier();  // index table, o and p are in LDS
   float4 pf[SA_E];
   fetch(0, pf);
 
@@ -166,30 +242,24 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
 
   for (int e0 = 0; e0 < n; e0 += SA_E) {
     const int ne = min(SA_E, n - e0);
-    __syncthreads();  // everyone is done with the previous group's vectors
+    sa_barrier();  // everyone is done with the previous group's vectors
     if (tid < nvec) {
-      float* dst = (pf_which == 0 ? aS : (pf_which == 1 ? bS : wS)) + pf_sl * d + 4 * pf_t4;
+      const int ld = pf_which == 2 ? d : dp;
+      float* dst = (pf_which == 0 ? aS : (pf_which == 1 ? bS : wS)) + pf_sl * ld + 4 * pf_t4;
 #pragma unroll
-      for (int ee = 0; ee < SA_E; ++ee) *reinterpret_cast<float4*>(dst + ee * K * d) = pf[ee];
+      for (int ee = 0; ee < SA_E; ++ee) *reinterpret_cast<float4*>(dst + ee * K * ld) = pf[ee];
     }
-    __syncthreads();
+    sa_barrier();
     if (e0 + SA_E < n) fetch(e0 + SA_E, pf);
 
     // alpha[e][s][j] = a_es . k[j],  beta[e][s][i] = q[i] . b_es,  gp[e][s] = a_es . b_es
-    const int items = 2 * ne * K * n;
-    for (int it = tid; it < items + ne * K; it += SA_NT) {
-      if (it < items) {
-        const int which = it / (ne * K * n), r = it - which * (ne * K * n);
-        const int es = r / n, x = r - es * n;  // es = ee * K + sl
-        const float* u = (which == 0 ? aS : bS) + es * d;
-        const float* m = (which == 0 ? kS : qS) + x * dp;
-        (which == 0 ? alS : beS)[es * n + x] = sa_dot(u, m, d4);
-      } else {
-        const int es = it - items;
-        gpS[es] = sa_dot(aS + es * d, bS + es * d, d4);
-      }
+    sa_products_nt(aS, dp, ne * K, kS, dp, n, bS, dp, ne * K, qS, dp, n, d4, tid,
+                   [&](bool beta, int es, int x, float v) { (beta ? beS : alS)[es * n + x] = v; });
+    if (tid >= SA_NT - ne * K) {  // the last wavefront has no tile when n <= 48
+      const int es = SA_NT - 1 - tid;
+      gpS[es] = sa_dot(aS + es * dp, bS + es * dp, d4);
     }
-    __syncthreads();
+    sa_barrier();
     // rho[e][s] = sum_j p[e][j] alpha[e][s][j],  gamma[e][s] = sum_j p[e][j] alpha[e][s][j] (v[j] - o[e])
     for (int it = tid; it < ne * K * d4; it += SA_NT) {
       const int es = it / d4, t4 = it - es * d4;
@@ -209,7 +279,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
       *reinterpret_cast<float4*>(gamS + es * d + 4 * t4) = gm;
       if (t4 == 0) rhoS[es] = rho;
     }
-    __syncthreads();
+    sa_barrier();
 
     // output rows of the group's slots, and their part of 2 sum_c p'_c[:, e] w_c
     if (ot4 < d4) {
@@ -286,7 +356,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
       D1[e] = d1; D2[e] = d2; R2a[e] = r2; gS[e] = g;
     }
   }
-  __syncthreads();
+  sa_barrier();
 
   // T2 = S2 - 2 SR + R2, then M (kept in AA)
   if (tid < n) {
@@ -295,7 +365,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     for (int e = 0; e < n; ++e) { const float pe = pS[i * np1 + e]; r2 += pe * pe * BB[i * np1 + e]; }
     R2a[i] = r2;
   }
-  __syncthreads();
+  sa_barrier();
   for (int it = tid; it < n * n; it += SA_NT) {
     const int i = it / n, j = it - i * n;
     const int x = i * np1 + j;
@@ -304,7 +374,7 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     AA[x] = s2 - 2.0f * sr + R2a[i];
   }
   load_tile(a.ql, oS);  // o is not needed any more
-  __syncthreads();
+  sa_barrier();
   if (tid < n) {
     const int i = tid;
     float s = 0.0f;
@@ -312,11 +382,8 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     rsum[i] = s;
   }
   // sL = lap_q k^T (into BB, whose sums of beta^2 are used up)
-  for (int it = tid; it < n * n; it += SA_NT) {
-    const int i = it / n, j = it - i * n;
-    BB[i * np1 + j] = sa_dot(oS + i * dp, kS + j * dp, d4);
-  }
-  __syncthreads();
+  sa_product_nt(oS, dp, n, kS, dp, n, d4, tid, [&](int i, int j, float v) { BB[i * np1 + j] = v; });
+  sa_barrier();
   for (int it = tid; it < n * n; it += SA_NT) {
     const int i = it / n, j = it - i * n;
     const int x = i * np1 + j;
@@ -324,12 +391,9 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     AA[x] = pij * (AA[x] - rsum[i] + 2.0f * gS[i] * ((i == j ? 1.0f : 0.0f) - pS[i * np1 + i]));
   }
   load_tile(a.kl, oS);  // lap_q has been consumed; k itself is not needed any more
-  __syncthreads();
-  for (int it = tid; it < n * n; it += SA_NT) {
-    const int i = it / n, j = it - i * n;
-    BB[i * np1 + j] += sa_dot(qS + i * dp, oS + j * dp, d4);
-  }
-  __syncthreads();
+  sa_barrier();
+  sa_product_nt(qS, dp, n, oS, dp, n, d4, tid, [&](int i, int j, float v) { BB[i * np1 + j] += v; });
+  sa_barrier();
   if (tid < n) {
     const int i = tid;
     float s = 0.0f;
@@ -337,13 +401,13 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
     rsum[i] = s;
   }
   load_tile(a.vl, qS);  // q is not needed any more
-  __syncthreads();
+  sa_barrier();
   for (int it = tid; it < n * n; it += SA_NT) {
     const int i = it / n, j = it - i * n;
     const int x = i * np1 + j;
     AA[x] += pS[x] * (BB[x] - rsum[i]);  // pL + M
   }
-  __syncthreads();
+  sa_barrier();
   // lap_o = p lap_v + (pL + M) v + 2 sum_c p'_c[:, e] w_c
   if (ot4 < d4) {
 #pragma unroll

@@ -744,7 +744,8 @@ def mhsa_sparse_supported(n, d, k_rows):
     if not (n <= 64 and d <= 64 and d % 4 == 0 and 1 <= k_rows <= 8 and 3 * k_rows * (d // 4) <= 512):
         return False
     # the kernel's LDS footprint (floats), at most 160 KB per workgroup
-    lds = 4 * n * (d + 4) + 4 * n * (n + 1) + 4 * (4 * k_rows * d + 2 * k_rows * n + 2 * k_rows) + 5 * n + k_rows * n
+    lds = (4 * n * (d + 4) + 4 * n * (n + 1) + 4 * (2 * k_rows * (d + 4) + 2 * k_rows * d + 2 * k_rows * n + 2 * k_rows)
+           + 5 * n + k_rows * n)
     return 4 * lds <= 160 * 1024
 
 
