@@ -198,45 +198,46 @@ __global__ __launch_bounds__(NTHR, 2) void dense_act_kernel(DAParams a) {
   const int64_t step1 = (int64_t)N * 4, step5 = (int64_t)N * 20;
   auto store_impl = [&](float* out_rows /* row r0 of the output */, const float* res_rows, auto&& value, auto has_res)
       __attribute__((always_inline)) {
-    constexpr bool RES = decltype(has_res)::value;
     if (!col_ok) return;
     gchar* rowp = (gchar*)(out_rows + (int64_t)wrow * N + wcol);
     const gchar* resp = nullptr;
-    if constexpr (RES) resp = (const gchar*)(res_rows + (int64_t)wrow * N + wcol);
-    auto row_ok = [&](int t, int r) { return full || r0 + wrow + t * 32 + 8 * (r / 4) + r % 4 + 4 * lh < R; };
-    // The skip connection's rows are asked for four rows ahead of their use, through a running
-    // pointer of their own: the stores cannot be told apart from that array, so a load written
-    // after a row's store would wait for it to be issued, and every row would pay a round trip.
-    float rbuf[2][4];
-    auto fetch = [&](int t, int g, float (&dst)[4]) __attribute__((always_inline)) {
+    if constexpr (decltype(has_res)::value) resp = (const gchar*)(res_rows + (int64_t)wrow * N + wcol);
+    if (full) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        dst[q] = 0.0f;
-        if (row_ok(t, 4 * g + q)) dst[q] = *(const gfloat*)(resp + voff);
-        resp += q == 3 ? step5 : step1;
-        asm volatile("" : "+s"(resp));
-      }
-    };
-    if constexpr (RES) fetch(0, 0, rbuf[0]);
+      for (int t = 0; t < TM; ++t)
 #pragma unroll
-    for (int t = 0; t < TM; ++t)
+        for (int r = 0; r < 16; ++r) {
+          float v = value(t, r);
+          if constexpr (decltype(has_res)::value) v += *(const gfloat*)(resp + voff);
+          *(gfloat*)(rowp + voff) = v;
+          const int64_t st = (r % 4 == 3) ? step5 : step1;
+          rowp += st;
+          asm volatile("" : "+s"(rowp));
+          if constexpr (decltype(has_res)::value) {
+            resp += st;
+            asm volatile("" : "+s"(resp));
+          }
+        }
+    } else {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int step = t * 4 + g;
-        if constexpr (RES)
-          if (step + 1 < TM * 4) fetch((step + 1) / 4, (step + 1) % 4, rbuf[(step + 1) & 1]);
+      for (int t = 0; t < TM; ++t)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int r = 4 * g + q;
-          if (row_ok(t, r)) {
+        for (int r = 0; r < 16; ++r) {
+          const int row = t * 32 + 8 * (r / 4) + r % 4;
+          if (r0 + wrow + row + 4 * lh < R) {
             float v = value(t, r);
-            if constexpr (RES) v += rbuf[step & 1][q];
+            if constexpr (decltype(has_res)::value) v += *(const gfloat*)(resp + voff);
             *(gfloat*)(rowp + voff) = v;
           }
-          rowp += q == 3 ? step5 : step1;
+          const int64_t st = (r % 4 == 3) ? step5 : step1;
+          rowp += st;
           asm volatile("" : "+s"(rowp));
+          if constexpr (decltype(has_res)::value) {
+            resp += st;
+            asm volatile("" : "+s"(resp));
+          }
         }
-      }
+    }
   };
   // res_rows = row r0 of the matching residual array, or nullptr (the same for the whole workgroup)
   auto store = [&](float* out_rows, const float* res_rows, auto&& value) __attribute__((always_inline)) {
