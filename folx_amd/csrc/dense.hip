@@ -33,6 +33,8 @@
 // Workgroup ids are remapped so that the column tiles of one row tile run back to back
 // on the same XCD (ids are dealt round-robin to the 8 XCDs), which keeps the second
 // read of an A tile in that XCD's L2 when N needs more than one column tile.
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -447,6 +449,73 @@ __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, cons
                                       l32, lh);
 }
 
+// N = 1 (a layer with one output per position, e.g. the last layer of a node-wise network): the
+// rule is a matrix-vector product, bound by reading the rows once.  A group of 32 lanes owns a
+// row at a time: 128-bit loads of up to 128 features per pass, the weights in registers, the
+// sum over the group by lane exchanges.  Rows are in the three segments of the stacked operand.
+__global__ __launch_bounds__(256) void dense_n1_kernel(Segs sg, const float* __restrict__ W, const float* __restrict__ bias,
+                                                       int32_t K, int64_t total_rows) {
+  const int lane32 = threadIdx.x % 32;
+  const int64_t g0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) / 32;
+  const int64_t ngroups = (int64_t)gridDim.x * 8;
+  const int passes = (K + 127) / 128;
+  const float b0 = bias != nullptr ? bias[0] : 0.0f;
+  auto locate = [&](int64_t r, int& seg, int64_t& t) {
+    seg = 0;
+    t = r;
+    if (t >= sg.rows[0]) { t -= sg.rows[0]; seg = 1; if (t >= sg.rows[1]) { t -= sg.rows[1]; seg = 2; } }
+  };
+  auto finish = [&](float acc, int seg, int64_t t) {
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 32);
+    if (lane32 == 0) {
+      float o = acc + (seg == 0 ? b0 : 0.0f);
+      if (sg.res[seg] != nullptr) o += sg.res[seg][t];
+      sg.out[seg][t] = o;
+    }
+  };
+  if (passes == 1) {
+    // Four rows in flight per group of lanes: their loads are all issued before the first sum.
+    constexpr int U = 4;
+    const int k = 4 * lane32;
+    const bool on = k < K;
+    const float4 w = on ? *reinterpret_cast<const float4*>(W + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int64_t r = g0; r < total_rows; r += U * ngroups) {
+      int seg[U];
+      int64_t t[U];
+      float4 a[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t ru = r + u * ngroups;
+        locate(ru < total_rows ? ru : r, seg[u], t[u]);
+        a[u] = on ? folx_ld_stream4(sg.in[seg[u]] + phys_row(sg, t[u]) * (int64_t)K + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (r + u * ngroups < total_rows)
+          finish(fmaf(a[u].x, w.x, fmaf(a[u].y, w.y, fmaf(a[u].z, w.z, a[u].w * w.w))), seg[u], t[u]);
+      }
+    }
+    return;
+  }
+  for (int64_t r = g0; r < total_rows; r += ngroups) {
+    int seg;
+    int64_t t;
+    locate(r, seg, t);
+    const float* row = sg.in[seg] + phys_row(sg, t) * (int64_t)K;
+    float acc = 0.0f;
+    for (int ps = 0; ps < passes; ++ps) {
+      const int k = ps * 128 + 4 * lane32;
+      if (k < K) {
+        const float4 a = folx_ld_stream4(row + k);
+        const float4 w = *reinterpret_cast<const float4*>(W + k);
+        acc = fmaf(a.x, w.x, fmaf(a.y, w.y, fmaf(a.z, w.z, fmaf(a.w, w.w, acc))));
+      }
+    }
+    finish(acc, seg, t);
+  }
+}
+
 template <int BM, int BN, int WM, int WN, int MINB>
 int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int32_t K, int32_t N,
                bool vec, bool has_res) {
@@ -500,6 +569,12 @@ extern "C" int folx_hip_dense_rows_fwdlap(void* stream, const float* x, const fl
                    folx_aligned16(lap) && folx_aligned16(W);
   const bool has_res = res != nullptr;
   hipStream_t st = (hipStream_t)stream;
+  if (N == 1 && K % 4 == 0 && folx_aligned16(x) && folx_aligned16(jac) && folx_aligned16(lap) && folx_aligned16(W)) {
+    const int64_t total = (int64_t)(P + 2) * R;
+    const int64_t blocks = std::min<int64_t>((total + 31) / 32, 256 * 32);
+    dense_n1_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(sg, W, bias, K, total);
+    return folx_launch_status();
+  }
   if (N > 128) return launch_cfg<128, 256, 2, 4, 2>(st, sg, W, bias, K, N, vec, has_res);
   if (N > 64) return launch_cfg<128, 128, 2, 2, 3>(st, sg, W, bias, K, N, vec, has_res);
   if (N > 32) return launch_cfg<128, 64, 4, 1, 3>(st, sg, W, bias, K, N, vec, has_res);

@@ -98,11 +98,14 @@ DENSE_CASES = [
     ((3, 50), 4, 832, 256, False),     # long K, ragged last row tile
     ((2, 70), 3, 32, 260, True),       # two column tiles, the second nearly empty
     ((1, 130), 5, 64, 20, False),      # BN = 32 variant, more rows than one tile
-    # narrow outputs (N <= 4, K % 4 == 0): streaming kernel without MFMA
+    # narrow outputs; N = 1 with K % 4 == 0 is a matrix-vector kernel without MFMA
     ((5, 33), 7, 64, 3, True),
     ((2, 70), 3, 256, 4, True),
-    ((20, 100), 40, 100, 1, True),
+    ((20, 100), 40, 100, 1, True),     # last layer of the README MLP
     ((1, 1), 0, 4, 2, False),
+    ((1, 1), 0, 4, 1, False),          # one row, one 128-bit load
+    ((3, 37), 5, 300, 1, True),        # three passes over K, the last one partial
+    ((2, 9), 3, 18, 1, True),          # K % 4 != 0: N = 1 through the GEMM
 ]
 
 
@@ -383,7 +386,7 @@ def test_dense_act_wide_matches_two_kernels_large():
 
 @pytest.mark.parametrize('lead,n,lo,hi,P,Kd,N', [((5,), 32, 0, 16, 9, 256, 256), ((5,), 32, 16, 32, 9, 256, 256),
                                                  ((2, 3), 7, 2, 5, 4, 48, 20), ((4,), 9, 1, 9, 3, 17, 33),
-                                                 ((300,), 6, 3, 4, 2, 32, 64)])
+                                                 ((300,), 6, 3, 4, 2, 32, 64), ((7,), 6, 1, 5, 3, 40, 1)])
 def test_dense_row_slice(lead, n, lo, hi, P, Kd, N):
     """A slice along the axis in front of the feature axis is read in place by the GEMM."""
     from folx_amd import kernels as K
@@ -761,7 +764,8 @@ def test_layernorm(rows, F, P):
 
 @pytest.mark.parametrize('rows,P,Kd,N', [((3, 32), 7, 256, 256),   # full tiles only: the unchecked epilogue
                                          ((3, 50), 5, 48, 100),    # ragged rows and columns, direct-to-LDS loads
-                                         ((2, 9), 3, 20, 36)])     # register-staged fallback (K % 16 != 0)
+                                         ((2, 9), 3, 20, 36),      # register-staged fallback (K % 16 != 0)
+                                         ((4, 11), 6, 100, 1)])    # matrix-vector kernel (N = 1)
 def test_dense_residual_epilogue(rows, P, Kd, N):
     from folx_amd import kernels as K
 
