@@ -21,6 +21,8 @@ _P = c_void_p
 SIGNATURES = {
     'folx_hip_version': (c_int, []),
     'folx_hip_strerror': (c_char_p, [c_int]),
+    'folx_hip_set_gemm_mode': (c_int, [c_int]),
+    'folx_hip_get_gemm_mode': (c_int, []),
     'folx_hip_dense_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_dense_rows_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int32, c_int32, c_int32, c_int64, c_int64]),
     'folx_hip_dense_act_workspace_bytes': (c_int64, [c_int64, c_int32, c_int32, c_int32]),
@@ -65,6 +67,7 @@ ACT = {
     'sinh': 16, 'cosh': 17, 'tan': 18, 'asin': 19, 'acos': 20, 'atan': 21, 'asinh': 22, 'acosh': 23,
     'atanh': 24, 'erf': 25, 'erfc': 26, 'erf_inv': 27, 'cbrt': 28, 'pow': 29, 'lgamma': 30, 'digamma': 31,
 }
+GEMM_MODE = {'f32': 0, 'bf16x3': 1}
 BINOP = {'mul': 0, 'div': 1, 'add': 2, 'sub': 3, 'min': 4, 'max': 5}
 
 _lib = None
@@ -89,6 +92,11 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
+    mode = os.environ.get('FOLX_AMD_GEMM')
+    if mode is not None:
+        if mode not in GEMM_MODE:
+            raise FolxHipError(f'FOLX_AMD_GEMM={mode!r}: expected one of {sorted(GEMM_MODE)}')
+        lib.folx_hip_set_gemm_mode(GEMM_MODE[mode])
     _lib = lib
     return lib
 

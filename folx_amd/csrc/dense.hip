@@ -36,6 +36,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "split_bf16.h"
 
 namespace {
 
@@ -449,6 +450,164 @@ __global__ __launch_bounds__(64 * WM * WN, MINB) void dense_kernel(Segs sg, cons
                                       l32, lh);
 }
 
+// The 128 x 256 tile of dense_dma_kernel with the products taken on the bf16 matrix pipe from
+// operands split into three bf16 pieces each.  A (streamed once) and W (K x N, from L2) both
+// come through registers, one chunk of 16 k ahead, and every element is split once per
+// workgroup on its way into LDS:
+//   A stage: [piece][g][row][8 bf16]      k = 8 g + e, one 16-byte fragment per (g, row)
+//   W stage: [piece][g][kp][col] dwords   k = 8 g + 2 kp and + 1, read as four 32-bit values
+// (lane l of a 32 x 32 x 16 product holds row or column l % 32 and the 8 k of g = l / 32).
+// Thread t stages row t / 4, k quarter t % 4 of the A chunk; wavefront w stages rows 2 w and
+// 2 w + 1 of the W chunk, lane l their columns 4 l .. 4 l + 3, so that a pair of k lands in one
+// 32-bit word.  The barrier between chunks only waits for LDS, not for the requests of the
+// next chunk.  Same epilogue as the fp32 kernel.  Requires K % 16 == 0, N % 4 == 0, N >= 4
+// and 16-byte aligned operands.
+template <bool HAS_RES>
+__global__ __launch_bounds__(512, 4) void dense_split_kernel(Segs sg, const float* __restrict__ W,
+                                                             const float* __restrict__ bias, int32_t K, int32_t N,
+                                                             int64_t row_tiles, int32_t col_tiles) {
+  using namespace folx_split;
+  constexpr int BM = 128, BN = 256, WN = 4, TM = 2, TN = 2;
+  constexpr int A_PLANE = 2 * BM * 16;     // bytes of one piece of an A chunk
+  constexpr int W_PLANE = 2 * 4 * BN * 4;  // and of a W chunk
+  __shared__ __attribute__((aligned(16))) char As0[3 * A_PLANE];
+  __shared__ __attribute__((aligned(16))) char As1[3 * A_PLANE];
+  __shared__ __attribute__((aligned(16))) char Ws0[3 * W_PLANE];
+  __shared__ __attribute__((aligned(16))) char Ws1[3 * W_PLANE];
+
+  const int64_t id = blockIdx.x;
+  const int64_t xcd = id % NXCD;
+  const int64_t slot = id / NXCD;
+  const int64_t rt = (slot / col_tiles) * NXCD + xcd;
+  const int32_t ct = (int32_t)(slot % col_tiles);
+  if (rt >= row_tiles) return;
+  int seg = 0;
+  int64_t t = rt;
+  if (t >= sg.tiles[0]) { t -= sg.tiles[0]; seg = 1; if (t >= sg.tiles[1]) { t -= sg.tiles[1]; seg = 2; } }
+  const float* __restrict__ A = sg.in[seg];
+  const int64_t rows = sg.rows[seg];
+  const int64_t row0 = t * BM;
+  const int32_t col0 = ct * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wr = (wave / WN) * 64;
+  const int wc = (wave % WN) * 64;
+  const int l32 = lane % 32;
+  const int lh = lane / 32;
+
+  const int a_row = tid / 4, a_q = tid % 4;
+  int64_t gr = row0 + a_row;
+  if (gr >= rows) gr = rows - 1;  // rows past the end: copies of the last one, never stored
+  const float* a_src = A + phys_row(sg, gr) * (int64_t)K + a_q * 4;
+  const int a_dst = ((a_q / 2) * BM + a_row) * 16 + (a_q % 2) * 8;
+  int wn = col0 + lane * 4;
+  if (wn > N - 4) wn = N - 4;  // columns past the end likewise
+  const float* w_src = W + (int64_t)(2 * wave) * N + wn;
+  const int w_dst = (wave * BN + lane * 4) * 4;  // (g, kp) = (wave / 4, wave % 4)
+
+  auto put_a = [&](const float4& v, char* as) __attribute__((always_inline)) {
+    unsigned p1a, p2a, p3a, p1b, p2b, p3b;
+    split_pair(v.x, v.y, p1a, p2a, p3a);
+    split_pair(v.z, v.w, p1b, p2b, p3b);
+    uint2v q;
+    q[0] = p1a; q[1] = p1b; *reinterpret_cast<uint2v*>(as + a_dst) = q;
+    q[0] = p2a; q[1] = p2b; *reinterpret_cast<uint2v*>(as + A_PLANE + a_dst) = q;
+    q[0] = p3a; q[1] = p3b; *reinterpret_cast<uint2v*>(as + 2 * A_PLANE + a_dst) = q;
+  };
+  auto put_w = [&](const float4& r0, const float4& r1, char* ws) __attribute__((always_inline)) {
+    unsigned a1[4], a2[4], a3[4];
+    split_pair(r0.x, r1.x, a1[0], a2[0], a3[0]);
+    split_pair(r0.y, r1.y, a1[1], a2[1], a3[1]);
+    split_pair(r0.z, r1.z, a1[2], a2[2], a3[2]);
+    split_pair(r0.w, r1.w, a1[3], a2[3], a3[3]);
+    uint4v q1, q2, q3;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) { q1[c] = a1[c]; q2[c] = a2[c]; q3[c] = a3[c]; }
+    *reinterpret_cast<uint4v*>(ws + w_dst) = q1;
+    *reinterpret_cast<uint4v*>(ws + W_PLANE + w_dst) = q2;
+    *reinterpret_cast<uint4v*>(ws + 2 * W_PLANE + w_dst) = q3;
+  };
+
+  float bvals[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int gc = col0 + wc + j * 32 + l32;
+    bvals[j] = (seg == 0 && bias != nullptr && gc < N) ? bias[gc] : 0.0f;
+  }
+  floatx16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto compute = [&](const char* as, const char* ws) __attribute__((always_inline)) {
+    bf16x8 fb[TN][3];
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        uint4v v;
+#pragma unroll
+        for (int kp = 0; kp < 4; ++kp)
+          v[kp] = *reinterpret_cast<const unsigned*>(ws + p * W_PLANE + ((lh * 4 + kp) * BN + wc + j * 32 + l32) * 4);
+        fb[j][p] = __builtin_bit_cast(bf16x8, v);
+      }
+    bf16x8 fa[TM];
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+      if (q == 0 || kPieceA[q] != kPieceA[q - 1]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa[i] = *reinterpret_cast<const bf16x8*>(as + kPieceA[q] * A_PLANE + (lh * BM + wr + i * 32 + l32) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j][kPieceB[q]], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int KT = K / 16;
+  float4 ra, rw0, rw1;
+  auto fetch = [&](int kt) __attribute__((always_inline)) {
+    ra = folx_ld_stream4(a_src + kt * 16);
+    rw0 = *reinterpret_cast<const float4*>(w_src + (int64_t)kt * 16 * N);
+    rw1 = *reinterpret_cast<const float4*>(w_src + (int64_t)kt * 16 * N + N);
+  };
+  // chunk kt + 1 is split into the other stage and chunk kt + 2 requested before the products
+  // of chunk kt; the barrier waits for LDS only
+  fetch(0);
+  put_a(ra, As0);
+  put_w(rw0, rw1, Ws0);
+  if (KT > 1) fetch(1);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  for (int kt = 0; kt < KT; kt += 2) {
+    if (kt + 1 < KT) {
+      put_a(ra, As1);
+      put_w(rw0, rw1, Ws1);
+      if (kt + 2 < KT) fetch(kt + 2);
+    }
+    compute(As0, Ws0);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (kt + 1 < KT) {
+      if (kt + 2 < KT) {
+        put_a(ra, As0);
+        put_w(rw0, rw1, Ws0);
+        if (kt + 3 < KT) fetch(kt + 3);
+      }
+      compute(As1, Ws1);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+  }
+  store_tile<BM, BN, TM, TN, HAS_RES>(acc, bvals, sg.out[seg], HAS_RES ? sg.res[seg] : nullptr, rows, N, row0, col0,
+                                      wr, wc, l32, lh);
+}
+
 // N = 1 (a layer with one output per position, e.g. the last layer of a node-wise network): the
 // rule is a matrix-vector product, bound by reading the rows once.  A group of 32 lanes owns a
 // row at a time: 128-bit loads of up to 128 features per pass, the weights in registers, the
@@ -526,6 +685,15 @@ int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int3
   const int64_t blocks = groups * NXCD * col_tiles;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   dim3 grid((unsigned)blocks), block(64 * WM * WN);
+  if constexpr (BM == 128 && BN == 256) {
+    if (vec && K % BK == 0 && N >= 4 && folx_gemm_mode() == FOLX_HIP_GEMM_BF16X3) {
+      if (has_res)
+        dense_split_kernel<true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+      else
+        dense_split_kernel<false><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);
+      return folx_launch_status();
+    }
+  }
   if (vec && K % BK == 0 && N >= 4) {
     if (has_res)
       dense_dma_kernel<BM, BN, WM, WN, true><<<grid, block, 0, st>>>(sg, W, bias, K, N, row_tiles, col_tiles);

@@ -81,6 +81,21 @@ class _timed:
             lt.records.append((self.name, self.key, self.e0, e1))
 
 
+def set_gemm_mode(mode: str):
+    """How the wide dense rules form their fp32 products: ``'f32'`` (FP32 matrix instructions, the
+    default) or ``'bf16x3'`` (operands split exactly into three bf16 pieces, six exact piece
+    products per product accumulated in fp32: same accuracy, the faster matrix pipe).  Process
+    wide; the environment variable ``FOLX_AMD_GEMM`` sets it when the library is loaded."""
+    if mode not in _lib.GEMM_MODE:
+        raise ValueError(f'gemm mode {mode!r}: expected one of {sorted(_lib.GEMM_MODE)}')
+    _lib.check(_lib.load().folx_hip_set_gemm_mode(_lib.GEMM_MODE[mode]), 'set_gemm_mode')
+
+
+def get_gemm_mode() -> str:
+    code = _lib.load().folx_hip_get_gemm_mode()
+    return next(k for k, v in _lib.GEMM_MODE.items() if v == code)
+
+
 def _p(t):
     if t is None:
         return None

@@ -40,6 +40,24 @@ int folx_hip_version(void);
 /* Static description of a return code. */
 const char* folx_hip_strerror(int code);
 
+/* How the wide dense rules (K % 16 == 0, N > 128, 16-byte aligned operands) form their fp32
+ * products.  No counterpart in the reference, which leaves the choice to XLA
+ * (jax.default_matmul_precision).
+ *   FOLX_HIP_GEMM_F32    v_mfma_f32_32x32x2_f32 on the fp32 operands (the default).
+ *   FOLX_HIP_GEMM_BF16X3 every operand element is split exactly into three bf16 pieces and a
+ *                        product is the sum of the six piece products of weight >= 2^-16, each
+ *                        exact, accumulated in fp32 on v_mfma_f32_32x32x16_bf16.  The dropped
+ *                        terms weigh <= 2^-24 of a product, the rounding of one fp32
+ *                        multiply-add, so results agree with the fp32 form to fp32 rounding;
+ *                        inputs, outputs and accumulators stay fp32.  Kernels without a split
+ *                        form run as under FOLX_HIP_GEMM_F32.
+ * The mode is process wide and read at every launch; set it before launching, not while other
+ * threads launch.  folx_hip_set_gemm_mode returns FOLX_HIP_EINVAL for any other value. */
+#define FOLX_HIP_GEMM_F32 0
+#define FOLX_HIP_GEMM_BF16X3 1
+int folx_hip_set_gemm_mode(int mode);
+int folx_hip_get_gemm_mode(void);
+
 /* Elementwise functions of folx_hip_elementwise_fwdlap; the rule needs f, f', f''.
  * Replaces the per-primitive entries of folx/wrapped_functions.py:400-445, :552-556. */
 enum folx_hip_act {

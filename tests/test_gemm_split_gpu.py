@@ -1,0 +1,101 @@
+"""The wide dense rules with their products on the bf16 matrix pipe (operands split into three
+bf16 pieces, ``set_gemm_mode('bf16x3')``): same parity bars against the fp64 oracle as the
+fp32 form, on the shapes that reach the split kernels and around their edges."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import rules
+from tolerances import assert_triplet
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.as_tensor(np.ascontiguousarray(a, dtype=np.float32), device='cuda')
+
+
+def f64(*arrs):
+    return tuple(np.asarray(a, dtype=np.float64) for a in arrs)
+
+
+def rand(rng, *shape):
+    return rng.standard_normal(shape).astype(np.float32)
+
+
+@pytest.fixture
+def split_mode():
+    from folx_amd import kernels as K
+
+    K.set_gemm_mode('bf16x3')
+    assert K.get_gemm_mode() == 'bf16x3'
+    yield K
+    K.set_gemm_mode('f32')
+
+
+DENSE_CASES = [
+    # (rows shape, P, K, N, bias, residual)
+    ((3, 32), 7, 256, 256, True, False),    # the PsiFormer layer shape, full tiles
+    ((3, 32), 7, 256, 256, True, True),     # with the skip connection in the epilogue
+    ((3, 50), 4, 832, 256, False, False),   # long K, ragged last row tile
+    ((1, 3), 2, 16, 132, True, False),      # one chunk, one row tile mostly empty, columns clamped
+    ((2, 70), 3, 48, 260, True, True),      # odd number of chunks, second column tile nearly empty
+    ((1, 130), 5, 32, 512, False, False),   # two full column tiles
+    ((5, 33), 0, 64, 200, True, False),     # no Jacobian rows
+]
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,bias,res', DENSE_CASES)
+def test_dense_split(split_mode, rows, P, Kd, N, bias, res):
+    K = split_mode
+    print(f'case dense bf16x3 rows={rows} P={P} K={Kd} N={N} res={res}', flush=True)
+    rng = np.random.default_rng(31)
+    x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    ref = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
+    r = None
+    if res:
+        rx, rJ, rL = rand(rng, *rows, N), rand(rng, P, *rows, N), rand(rng, *rows, N)
+        ref = tuple(a + c for a, c in zip(ref, f64(rx, rJ, rL)))
+        r = (dev(rx), dev(rJ), dev(rL))
+    got = K.dense(dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b), r)
+    assert_triplet(got, ref, 'dense bf16x3')
+
+
+def test_dense_split_row_slice(split_mode):
+    K = split_mode
+    rng = np.random.default_rng(32)
+    lead, n, lo, hi, P, Kd, N = (5,), 32, 16, 32, 9, 256, 256
+    x, J, L = rand(rng, *lead, n, Kd), rand(rng, P, *lead, n, Kd), rand(rng, *lead, n, Kd)
+    W, b = rand(rng, Kd, N) / np.sqrt(Kd), rand(rng, N)
+    ref = rules.dense_rule(*f64(x[..., lo:hi, :], J[..., lo:hi, :], L[..., lo:hi, :], W), b.astype(np.float64))
+    got = K.dense(dev(x), dev(J), dev(L), dev(W), dev(b), None, (lo, hi))
+    assert_triplet(got, ref, 'dense bf16x3 row_slice')
+
+
+def test_dense_split_error_is_that_of_fp32():
+    """Entries spread over twelve decades, so that every piece of the split carries weight: the
+    error against fp64 is within that of the fp32 matrix instructions (x 1.5 for noise) and far
+    below what a product of two bf16 pieces alone would leave (2^-16)."""
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(33)
+    rows, P, Kd, N = (4, 64), 6, 256, 256
+    mag = lambda *s: (rand(rng, *s) * np.exp(rng.uniform(-14, 14, size=s))).astype(np.float32)  # noqa: E731
+    x, J, L, W = mag(*rows, Kd), mag(P, *rows, Kd), mag(*rows, Kd), mag(Kd, N)
+    ref = rules.dense_rule(*f64(x, J, L, W), None)
+    # per output entry: error relative to sum_k |a_k w_k|, the scale that bounds any summation order
+    bound = np.abs(f64(J)[0]) @ np.abs(f64(W)[0])
+    errs = {}
+    try:
+        for mode in ('f32', 'bf16x3'):
+            K.set_gemm_mode(mode)
+            got = K.dense(dev(x), dev(J), dev(L), dev(W), None)
+            errs[mode] = float((np.abs(got[1].cpu().numpy().astype(np.float64) - ref[1]) / bound).max())
+    finally:
+        K.set_gemm_mode('f32')
+    print('relative to sum |a w|:', errs, flush=True)
+    assert errs['bf16x3'] <= 1.5 * errs['f32'] + 1e-9
+    assert errs['bf16x3'] < 2.0 ** -20
