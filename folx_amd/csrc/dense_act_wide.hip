@@ -51,6 +51,7 @@
 
 #include "activations.h"
 #include "dense_act_wide.h"
+#include "split_bf16.h"
 
 namespace {
 
@@ -67,6 +68,7 @@ constexpr int TM = WROWS / 32, TN = WCOLS / 32;
 constexpr int TG = BK / 8;
 constexpr int NXCD = 8;
 constexpr int KMAX_NORM = 512; // xh of a tile's positions sits in LDS
+constexpr int KMAX_NORM_SPLIT = 256;  // bf16x3 form: its larger tiles leave room for 256 features
 constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
 constexpr int A_LD = A_V4 / NT, W_LD = W_V4 / NT;
 static_assert(A_V4 % NT == 0 && W_V4 % NT == 0, "every thread loads the same number of pieces");
@@ -108,20 +110,31 @@ struct WideParams {
 // PT = Jacobian rows of a tile: 32 (4 positions per tile, one per accumulator block), or 16 for
 // the activation alone (8 positions per tile, two per block: registers 0-7 of a block belong
 // to the first, 8-15 to the second), which wastes less when P is 16 more than a multiple of 32.
-template <bool NORM, bool ACT, int PT, bool PARTS>
+// SPLIT: the products on the bf16 matrix pipe from operands split into three bf16 pieces, with
+// the loop of dense_split_kernel: A and W chunks come through registers and every element is
+// split once per workgroup on its way into LDS (A stage [piece][g][row][8 bf16], W stage
+// [piece][g][kp][col] dwords).  The thread that stages four k of a tile row also has their fp32
+// values, so LayerNorm's row sums are taken there (and added over the four threads of a row
+// after the loop) instead of from the fragments of chosen wavefronts; the per-column values the
+// epilogue needs (z, w1, c0) are fetched from memory after the loop, which leaves LDS for two
+// workgroups per CU.
+template <bool NORM, bool ACT, int PT, bool PARTS, bool SPLIT>
 __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   static_assert(!PARTS || !NORM, "LayerNorm reads one array");
   static_assert(!PARTS || A_LD == 1, "one A piece per thread");
+  static_assert(!SPLIT || (!PARTS && PT == 32), "the split form reads one array in groups of 32 rows");
+  constexpr int A_PLANE = 2 * BM * 16;     // SPLIT: bytes of one piece of an A chunk
+  constexpr int W_PLANE = 2 * 4 * BN * 4;  //        and of a W chunk
   constexpr int RT = BM / PT;  // positions of a tile
   constexpr int PB = 32 / PT;  // positions of a 32-row accumulator block
   static_assert(PT == 32 || (PT == 16 && !NORM), "LayerNorm's row sums assume one position per block");
-  __shared__ __attribute__((aligned(16))) float As0[BM * BK];
-  __shared__ __attribute__((aligned(16))) float As1[BM * BK];
-  __shared__ __attribute__((aligned(16))) float Ws0[BK * BN];
-  __shared__ __attribute__((aligned(16))) float Ws1[BK * BN];
-  __shared__ __attribute__((aligned(16))) float xhS[NORM ? RT * KMAX_NORM : 4];
-  __shared__ float zS[NORM ? RT * BN : 1];  // pre-activation values of the tile's positions and columns
-  __shared__ float2 wcS[NORM ? BN : 1];     // (w1, c0) of the tile's columns
+  __shared__ __attribute__((aligned(16))) float As0[SPLIT ? 3 * A_PLANE / 4 : BM * BK];
+  __shared__ __attribute__((aligned(16))) float As1[SPLIT ? 3 * A_PLANE / 4 : BM * BK];
+  __shared__ __attribute__((aligned(16))) float Ws0[SPLIT ? 3 * W_PLANE / 4 : BK * BN];
+  __shared__ __attribute__((aligned(16))) float Ws1[SPLIT ? 3 * W_PLANE / 4 : BK * BN];
+  __shared__ __attribute__((aligned(16))) float xhS[NORM ? RT * (SPLIT ? KMAX_NORM_SPLIT : KMAX_NORM) : 4];
+  __shared__ float zS[NORM && !SPLIT ? RT * BN : 1];  // pre-activation values of the tile's positions and columns
+  __shared__ float2 wcS[NORM && !SPLIT ? BN : 1];     // (w1, c0) of the tile's columns
   __shared__ float rsS[RT];
 
   // ids are dealt round-robin to the XCDs: the column tiles of a row tile stay on one of them
@@ -215,8 +228,31 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
         for (int b = 0; b < PB; ++b) dr[i][j][b] = a.z[(r0 + (wrow * TM + i) * PB + b) * N + gc];
       }
   }
-  issue(0, As0, Ws0);
-  if constexpr (NORM) {
+  // SPLIT staging: thread t has k quarter t % 4 of tile row t / 4; wavefront w has rows 2 w and
+  // 2 w + 1 of the W chunk, lane l their columns 4 l .. 4 l + 3
+  const float* sa_src = nullptr;
+  const float* sw_src = nullptr;
+  int sa_dst = 0, sw_dst = 0;
+  float4 ra = make_float4(0.f, 0.f, 0.f, 0.f), rw0 = ra, rw1 = ra;
+  if constexpr (SPLIT) {
+    const int m = tid / 4, q = tid % 4;
+    int p = p0 + m % PT;
+    if (p >= P) p = P - 1;
+    sa_src = a.jac + ((int64_t)p * R + r0 + m / PT) * K + q * 4;
+    sa_dst = ((q / 2) * BM + m) * 16 + (q % 2) * 8;
+    int wn = col0 + lane * 4;
+    if (wn > N - 4) wn = N - 4;
+    sw_src = a.W + (int64_t)(2 * wave) * N + wn;
+    sw_dst = (wave * BN + lane * 4) * 4;
+  }
+  auto fetch = [&](int kt) __attribute__((always_inline)) {
+    ra = folx_ld_stream4(sa_src + kt * BK);
+    rw0 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N);
+    rw1 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N + N);
+  };
+  if constexpr (SPLIT) fetch(0);
+  else issue(0, As0, Ws0);
+  if constexpr (NORM && !SPLIT) {
     for (int e = tid; e < RT * BN; e += NT) {
       int gc = col0 + e % BN;
       if (gc >= N) gc = N - 1;
@@ -238,7 +274,8 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     // xh of the tile's RT positions: RT * K consecutive floats
     const float4* src = reinterpret_cast<const float4*>(a.xhat + r0 * K);
     for (int e = tid; e < RT * K / 4; e += NT) reinterpret_cast<float4*>(xhS)[e] = src[e];
-    if (tid < BN) wcS[tid] = a.wc[col0 + tid < N ? col0 + tid : N - 1];
+    if constexpr (!SPLIT)
+      if (tid < BN) wcS[tid] = a.wc[col0 + tid < N ? col0 + tid : N - 1];
     if (tid < RT) rsS[tid] = a.rs[r0 + tid];
   }
 
@@ -290,11 +327,94 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     }
   };
 
+  const int KT = K / BK;
+  if constexpr (SPLIT) {
+    using namespace folx_split;
+    // chunk kt of this thread's registers into a stage; LayerNorm's sums from the fp32 values
+    auto put = [&](int kt, float* asf, float* wsf) __attribute__((always_inline)) {
+      char* as = reinterpret_cast<char*>(asf);
+      char* ws = reinterpret_cast<char*>(wsf);
+      if constexpr (NORM) {
+        const float4 xv = *reinterpret_cast<const float4*>(&xhS[(tid / (4 * PT)) * K + kt * BK + (tid % 4) * 4]);
+        sa += (ra.x + ra.y) + (ra.z + ra.w);
+        sb = fmaf(ra.x, xv.x, fmaf(ra.y, xv.y, fmaf(ra.z, xv.z, fmaf(ra.w, xv.w, sb))));
+        s2 = fmaf(ra.x, ra.x, fmaf(ra.y, ra.y, fmaf(ra.z, ra.z, fmaf(ra.w, ra.w, s2))));
+      }
+      unsigned p1a, p2a, p3a, p1b, p2b, p3b;
+      split_pair(ra.x, ra.y, p1a, p2a, p3a);
+      split_pair(ra.z, ra.w, p1b, p2b, p3b);
+      uint2v q;
+      q[0] = p1a; q[1] = p1b; *reinterpret_cast<uint2v*>(as + sa_dst) = q;
+      q[0] = p2a; q[1] = p2b; *reinterpret_cast<uint2v*>(as + A_PLANE + sa_dst) = q;
+      q[0] = p3a; q[1] = p3b; *reinterpret_cast<uint2v*>(as + 2 * A_PLANE + sa_dst) = q;
+      unsigned a1[4], a2[4], a3[4];
+      split_pair(rw0.x, rw1.x, a1[0], a2[0], a3[0]);
+      split_pair(rw0.y, rw1.y, a1[1], a2[1], a3[1]);
+      split_pair(rw0.z, rw1.z, a1[2], a2[2], a3[2]);
+      split_pair(rw0.w, rw1.w, a1[3], a2[3], a3[3]);
+      uint4v q1, q2, q3;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) { q1[c] = a1[c]; q2[c] = a2[c]; q3[c] = a3[c]; }
+      *reinterpret_cast<uint4v*>(ws + sw_dst) = q1;
+      *reinterpret_cast<uint4v*>(ws + W_PLANE + sw_dst) = q2;
+      *reinterpret_cast<uint4v*>(ws + 2 * W_PLANE + sw_dst) = q3;
+    };
+    auto products = [&](const float* asf, const float* wsf) __attribute__((always_inline)) {
+      const char* as = reinterpret_cast<const char*>(asf);
+      const char* ws = reinterpret_cast<const char*>(wsf);
+      bf16x8 fb[TN][3];
+#pragma unroll
+      for (int p = 0; p < 3; ++p)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          uint4v v;
+#pragma unroll
+          for (int kp = 0; kp < 4; ++kp)
+            v[kp] = *reinterpret_cast<const unsigned*>(ws + p * W_PLANE + ((lh * 4 + kp) * BN + wc + j * 32 + l32) * 4);
+          fb[j][p] = __builtin_bit_cast(bf16x8, v);
+        }
+      bf16x8 fa[TM];
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        if (q == 0 || kPieceA[q] != kPieceA[q - 1]) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            fa[i] = *reinterpret_cast<const bf16x8*>(as + kPieceA[q] * A_PLANE + (lh * BM + wr + i * 32 + l32) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j][kPieceB[q]], acc[i][j], 0, 0, 0);
+      }
+    };
+    __syncthreads();  // xh of the tile's positions is in LDS (the first chunk has landed as well)
+    put(0, As0, Ws0);
+    if (KT > 1) fetch(1);
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int kt = 0; kt < KT; kt += 2) {
+      if (kt + 1 < KT) {
+        put(kt + 1, As1, Ws1);
+        if (kt + 2 < KT) fetch(kt + 2);
+      }
+      products(As0, Ws0);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (kt + 1 < KT) {
+        if (kt + 2 < KT) {
+          put(kt + 2, As0, Ws0);
+          if (kt + 3 < KT) fetch(kt + 3);
+        }
+        products(As1, Ws1);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      }
+    }
+  }
   // The loads of a chunk are waited for at the end of the chunk before it; the barrier then
   // also says that every wavefront is done reading the buffer that is refilled next.
-  const int KT = K / BK;
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
+  if constexpr (!SPLIT) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
   auto kloop = [&](auto sblk) __attribute__((always_inline)) {
     for (int kt = 0; kt < KT; kt += 2) {
       if (kt + 1 < KT) issue(kt + 1, As1, Ws1);
@@ -310,14 +430,62 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     }
   };
   static_assert(TM == 2, "one loop copy per accumulator block row");
-  if (NORM && si == 0) kloop(std::integral_constant<int, 0>{});
-  else if (NORM && si == 1) kloop(std::integral_constant<int, 1>{});
-  else kloop(std::integral_constant<int, -1>{});
+  if constexpr (!SPLIT) {
+    if (NORM && si == 0) kloop(std::integral_constant<int, 0>{});
+    else if (NORM && si == 1) kloop(std::integral_constant<int, 1>{});
+    else kloop(std::integral_constant<int, -1>{});
+  }
+  // SPLIT: what the epilogue needs per column, asked for while the row sums are put together
+  float zpre[TM][TN];
+  float2 wcpre[TN];
+  if constexpr (NORM && SPLIT) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int gc = col0 + wc + j * 32 + l32;
+      if (gc >= N) gc = N - 1;
+      wcpre[j] = a.wc[gc];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) zpre[i][j] = a.z[(r0 + wrow * TM + i) * N + gc];
+    }
+  }
 
   // The row sums go through LDS (the tiles are no longer read: the loop ended with a barrier)
   // to the lanes that hold the rows' accumulators.
   float2* st = reinterpret_cast<float2*>(As0) + wrow * TM * 32;  // [wrow][i][row] (a, b)
-  if constexpr (NORM) {
+  if constexpr (NORM && SPLIT) {
+    // the four threads of a tile row add their quarters; thread 4 m keeps row m
+    float ta = sa + __shfl_xor(sa, 1, FOLX_WAVE), tb = sb + __shfl_xor(sb, 1, FOLX_WAVE);
+    float t2 = s2 + __shfl_xor(s2, 1, FOLX_WAVE);
+    ta += __shfl_xor(ta, 2, FOLX_WAVE);
+    tb += __shfl_xor(tb, 2, FOLX_WAVE);
+    t2 += __shfl_xor(t2, 2, FOLX_WAVE);
+    const int m = tid / 4;
+    const float invK = 1.0f / (float)K;
+    const bool keep = tid % 4 == 0 && p0 + m % PT < P;
+    const float av = keep ? ta * invK : 0.0f;
+    const float bv = keep ? tb * invK : 0.0f;
+    const float qv = keep ? t2 * invK - av * av : 0.0f;
+    float2* rowsums = reinterpret_cast<float2*>(As0);   // [tile row]
+    float2* wavesums = rowsums + BM;                     // [wavefront]: 16 rows of one position each
+    if (tid % 4 == 0) rowsums[m] = make_float2(av, bv);
+    if (ct == 0) {  // the two scalar sums of a position: two wavefronts each
+      float eb = bv * bv, eq = qv;
+#pragma unroll
+      for (int off = 32; off >= 4; off >>= 1) {
+        eb += __shfl_xor(eb, off, FOLX_WAVE);
+        eq += __shfl_xor(eq, off, FOLX_WAVE);
+      }
+      if (lane == 0) wavesums[wave] = make_float2(eb, eq);
+    }
+    __syncthreads();
+    if (ct == 0 && tid < RT) {
+      const float2 u = wavesums[2 * tid], v = wavesums[2 * tid + 1];
+      float* o = a.sc + ((int64_t)pg * R + r0 + tid) * 2;
+      o[0] = u.x + v.x;
+      o[1] = u.y + v.y;
+    }
+  }
+  if constexpr (NORM && !SPLIT) {
     if (si >= 0 && si < TM) {
       const float invK = 1.0f / (float)K;
       const bool pv = p0 + l32 < P;
@@ -363,7 +531,8 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
         zv[b] = 0.0f;
         d1[b] = 1.0f;
         if constexpr (NORM) {
-          zv[b] = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
+          if constexpr (SPLIT) zv[b] = zpre[i][j];
+          else zv[b] = zS[(wrow * TM + i) * BN + wc + j * 32 + l32];
           if constexpr (ACT) {
             float f, d2;
             act_eval_fused(a.act, zv[b], a.prm, f, d1[b], d2);
@@ -374,7 +543,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
       }
       float w1c = 0.0f, w2c = 0.0f;
       if constexpr (NORM) {
-        const float2 t = wcS[wc + j * 32 + l32];
+        const float2 t = SPLIT ? wcpre[j] : wcS[wc + j * 32 + l32];
         w1c = t.x;
         w2c = zv[0] - t.y;
       }
@@ -702,7 +871,13 @@ bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, 
 template <bool NORM, bool ACT, int PT, bool PARTS = false>
 int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap,
                 const float* res = nullptr, const float* res_lap = nullptr) {
-  dense_wide_kernel<NORM, ACT, PT, PARTS><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
+  bool split = false;
+  if constexpr (!PARTS && PT == 32)
+    split = folx_gemm_mode() == FOLX_HIP_GEMM_BF16X3 && (!NORM || a.K <= KMAX_NORM_SPLIT);
+  if constexpr (!PARTS && PT == 32) {
+    if (split) dense_wide_kernel<NORM, ACT, PT, PARTS, true><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
+  }
+  if (!split) dense_wide_kernel<NORM, ACT, PT, PARTS, false><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   int rc = folx_launch_status();
   if (rc != FOLX_HIP_OK) return rc;
   const int64_t S4 = a.R * (int64_t)a.N / 4;

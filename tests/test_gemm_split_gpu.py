@@ -99,3 +99,88 @@ def test_dense_split_error_is_that_of_fp32():
     print('relative to sum |a w|:', errs, flush=True)
     assert errs['bf16x3'] <= 1.5 * errs['f32'] + 1e-9
     assert errs['bf16x3'] < 2.0 ** -20
+
+
+NORM_DENSE_CASES = [
+    # (rows shape, P, K, N, gamma/beta, bias, act)
+    ((2, 32), 96, 256, 256, True, False, None),      # transformer q / k / v projection behind LayerNorm
+    ((2, 32), 96, 256, 256, True, True, 'tanh'),     # transformer MLP behind LayerNorm
+    ((1, 8), 40, 64, 132, False, True, None),        # no gamma / beta, partial group of Jacobian rows, cut column tile
+    ((3, 4), 1, 16, 300, True, False, 'softplus'),   # one chunk of K, one Jacobian row
+    ((1, 4), 64, 48, 256, True, True, 'sin'),        # odd number of chunks
+    ((1, 12), 33, 512, 512, True, True, 'silu'),     # K past the split form's 256: runs on the fp32 instructions
+]
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,affine,bias,act', NORM_DENSE_CASES)
+def test_norm_dense_split(split_mode, rows, P, Kd, N, affine, bias, act):
+    """LayerNorm + dense (+ activation) with the Jacobian product on the bf16 pipe."""
+    from oracle import backend as ob
+
+    K = split_mode
+    print(f'case norm_dense bf16x3 rows={rows} P={P} K={Kd} N={N} act={act}', flush=True)
+    rng = np.random.default_rng(23)
+    x, J, L = rand(rng, *rows, Kd) + 0.5, rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    J = J + 0.3 * rand(rng, P, *rows, 1)  # rows with a mean of their own
+    g = (1.0 + 0.3 * rand(rng, Kd)) if affine else None
+    be = 0.2 * rand(rng, Kd) if affine else None
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    h = ob.layer_norm(ob.OArr(*f64(x, J, L)), None if g is None else g.astype(np.float64),
+                      None if be is None else be.astype(np.float64), 1e-5)
+    ref = rules.dense_rule(h.x, h.J, h.lap, W.astype(np.float64), None if b is None else b.astype(np.float64))
+    if act is not None:
+        ref = rules.elementwise_rule(act, *ref)
+    opt = lambda t: None if t is None else dev(t)  # noqa: E731
+    for rep in range(2):  # the workspace of the second call holds what the first one left
+        got = K.norm_dense(act, dev(x), dev(J), dev(L), opt(g), opt(be), 1e-5, dev(W), opt(b))
+        assert_triplet(got, ref, f'norm_dense bf16x3 call {rep}')
+
+
+@pytest.mark.parametrize('rows,P,Kd,N,bias,act', [
+    ((2, 32), 96, 256, 256, True, 'tanh'),    # transformer MLP layer
+    ((1, 8), 40, 64, 132, True, 'silu'),      # partial group of Jacobian rows, cut column tile
+    ((3, 4), 1, 16, 300, False, 'softplus'),  # one chunk of K, one Jacobian row
+])
+def test_dense_act_wide_split(split_mode, rows, P, Kd, N, bias, act):
+    K = split_mode
+    print(f'case dense_act wide bf16x3 rows={rows} P={P} K={Kd} N={N} act={act}', flush=True)
+    rng = np.random.default_rng(35)
+    x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
+    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    b = rand(rng, N) if bias else None
+    ref = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
+    ref = rules.elementwise_rule(act, *ref)
+    assert K.dense_act_supported(act, Kd, N, rows=int(np.prod(rows)))
+    got = K.dense_act(act, dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
+    assert_triplet(got, ref, 'dense_act wide bf16x3')
+
+
+def test_norm_dense_split_full_chunk_properties(split_mode):
+    """At the benchmark's chunk size: doubling the Jacobian rows doubles y_jac bit for bit (the
+    pieces of 2 t are twice the pieces of t) and leaves y alone."""
+    K = split_mode
+    g = torch.Generator(device='cuda').manual_seed(11)
+    R, P, Kd, N = 1024 * 32, 96, 256, 256
+    x = torch.randn(R, Kd, device='cuda', generator=g)
+    J = torch.randn(P, R, Kd, device='cuda', generator=g)
+    L = torch.randn(R, Kd, device='cuda', generator=g)
+    gam = 1 + 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    bet = 0.2 * torch.randn(Kd, device='cuda', generator=g)
+    W = torch.randn(Kd, N, device='cuda', generator=g) / 16
+    b = torch.randn(N, device='cuda', generator=g)
+    print('case norm_dense bf16x3 full chunk', flush=True)
+    y, yj, yl = K.norm_dense('tanh', x, J, L, gam, bet, 1e-5, W, b)
+    assert torch.isfinite(yj).all() and torch.isfinite(yl).all()
+    K.set_gemm_mode('f32')
+    y0, yj0, yl0 = K.norm_dense('tanh', x, J, L, gam, bet, 1e-5, W, b)
+    K.set_gemm_mode('bf16x3')
+    torch.testing.assert_close(y, y0, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(yj, yj0, rtol=2e-5, atol=2e-5)
+    torch.testing.assert_close(yl, yl0, rtol=1e-4, atol=2e-3)
+    del yj0, yl0
+    J.mul_(2.0)
+    y2, yj2, yl2 = K.norm_dense('tanh', x, J, L, gam, bet, 1e-5, W, b)
+    assert torch.equal(y2, y)
+    yj.mul_(2.0)
+    assert torch.equal(yj2, yj)
