@@ -73,22 +73,24 @@ __device__ __forceinline__ void sa_barrier() {
 __device__ __forceinline__ floatx4 sa_tile_nt(const float* X, int ldx, const float* Y, int ldy, int d4, int lane) {
   const float* xp = X + (lane % 16) * ldx + lane / 16;
   const float* yp = Y + (lane % 16) * ldy + lane / 16;
-  // two accumulators, even and odd steps: independent chains for the matrix pipe, and half as many
-  // roundings in a row for every element
-  floatx4 c0 = {0.0f, 0.0f, 0.0f, 0.0f}, c1 = {0.0f, 0.0f, 0.0f, 0.0f};
+  // four accumulators, steps dealt round: independent chains for the matrix pipe, and a quarter
+  // as many roundings in a row for every element (the partial sums are added pairwise)
+  floatx4 c0 = {0.0f, 0.0f, 0.0f, 0.0f}, c1 = c0, c2 = c0, c3 = c0;
   int s = 0;
   for (; s + 8 <= d4; s += 8) {  // the operands of eight steps are read before the first product
     float xv[8], yv[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) { xv[u] = xp[4 * (s + u)]; yv[u] = yp[4 * (s + u)]; }
 #pragma unroll
-    for (int u = 0; u < 8; u += 2) {
+    for (int u = 0; u < 8; u += 4) {
       c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u], yv[u], c0, 0, 0, 0);
       c1 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u + 1], yv[u + 1], c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u + 2], yv[u + 2], c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[u + 3], yv[u + 3], c3, 0, 0, 0);
     }
   }
   for (; s < d4; ++s) c0 = __builtin_amdgcn_mfma_f32_16x16x4f32(xp[4 * s], yp[4 * s], c0, 0, 0, 0);
-  return c0 + c1;
+  return (c0 + c1) + (c2 + c3);
 }
 
 // Two products at once, C0 = X0 Y0^T (rows < nr0 of X0, rows < nc0 of Y0) and C1 = X1 Y1^T, their
@@ -195,13 +197,31 @@ __global__ __launch_bounds__(SA_NT, 4) void mhsa_sparse_kernel(SAArgs a) {
   // o = p v
   for (int it = tid; it < n * d4; it += SA_NT) {
     const int i = it / d4, t4 = it - i * d4;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 8
-    for (int j = 0; j < n; ++j) {
+    // four partial sums (keys j % 4), added pairwise: a quarter as many roundings in a row, which
+    // the Jacobian rows feel through v - o
+    float4 part[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) part[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    int j = 0;
+    for (; j + 4 <= n; j += 4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float pij = pS[i * np1 + j + u];
+        const float4 vv = *reinterpret_cast<const float4*>(vS + (j + u) * dp + 4 * t4);
+        part[u].x = fmaf(pij, vv.x, part[u].x); part[u].y = fmaf(pij, vv.y, part[u].y);
+        part[u].z = fmaf(pij, vv.z, part[u].z); part[u].w = fmaf(pij, vv.w, part[u].w);
+      }
+    }
+    for (; j < n; ++j) {
       const float pij = pS[i * np1 + j];
       const float4 vv = *reinterpret_cast<const float4*>(vS + j * dp + 4 * t4);
-      acc.x += pij * vv.x; acc.y += pij * vv.y; acc.z += pij * vv.z; acc.w += pij * vv.w;
+      part[0].x = fmaf(pij, vv.x, part[0].x); part[0].y = fmaf(pij, vv.y, part[0].y);
+      part[0].z = fmaf(pij, vv.z, part[0].z); part[0].w = fmaf(pij, vv.w, part[0].w);
     }
+    const float4 acc = make_float4((part[0].x + part[1].x) + (part[2].x + part[3].x),
+                                   (part[0].y + part[1].y) + (part[2].y + part[3].y),
+                                   (part[0].z + part[1].z) + (part[2].z + part[3].z),
+                                   (part[0].w + part[1].w) + (part[2].w + part[3].w));
     *reinterpret_cast<float4*>(oS + i * dp + 4 * t4) = acc;
     *reinterpret_cast<float4*>(a.o + grow(i) + 4 * t4) = acc;
   }

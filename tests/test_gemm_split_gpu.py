@@ -184,3 +184,13 @@ def test_norm_dense_split_full_chunk_properties(split_mode):
     assert torch.equal(y2, y)
     yj.mul_(2.0)
     assert torch.equal(yj2, yj)
+
+
+@pytest.mark.parametrize('name', ['psiformer32', 'psiformer64'])
+def test_full_width_models_split(split_mode, name):
+    """The transformer benchmarks at their real widths with the bf16x3 products: every rule call
+    within the strict bars of its fp64 oracle rule, and the well-conditioned end-to-end check."""
+    import test_models_gpu as tm
+
+    tm.test_full_width_every_rule_call_meets_the_strict_bars(name)
+    tm.test_full_width_well_conditioned_end_to_end_strict(name)
