@@ -20,6 +20,7 @@ import time
 
 import numpy as np
 
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense FP32 matrix peak
 PEAK_HBM_GBS = 8000.0
 
@@ -47,6 +48,11 @@ def parse():
     ap.add_argument('--chunk', type=int, default=1024, help='walkers per batched_vmap chunk')
     ap.add_argument('--cpu-seconds', type=float, default=20.0, help='budget of the CPU baseline sample')
     ap.add_argument('--no-cpu', action='store_true')
+    ap.add_argument('--gemm', choices=('f32', 'bf16x3'), default='f32',
+                    help='products of the wide dense rules: FP32 matrix instructions (default) or the exact '
+                         'three-piece bf16 split on the bf16 matrix pipe')
+    ap.add_argument('--no-split-leg', action='store_true',
+                    help='skip the short second measurement with --gemm bf16x3 that a default run appends')
     ap.add_argument('--graph', action='store_true',
                     help='replay each chunk as a captured HIP graph (no per-kernel timing, no roofline)')
     ap.add_argument('--calibrate-copy', action='store_true',
@@ -54,7 +60,7 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(workload, budget_s, gpu_out=None):
+def cpu_baseline(workload, budget_s, gpu_out=None, gpu_out_split=None):
     """The numpy oracle (fp32, dense Jacobians) on a bounded sample of the same workload: the first
     n walkers of the batch the GPU was timed on, whose GPU results (``gpu_out``) are compared with
     the oracle's in the same run."""
@@ -96,14 +102,20 @@ def cpu_baseline(workload, budget_s, gpu_out=None):
         # Both sides are float32; log|det| of the randomly initialised orbital matrices amplifies their
         # rounding (the oracle's own float32 / float64 difference is 3e-4 on psiformer32), which is what
         # these figures show -- the parity bars are enforced stage by stage in tests/.
-        gx, gJ, gl = gpu_out
         rel = lambda g, r: float(np.abs(g[..., :n].astype(np.float64) - r).max() / max(np.abs(r).max(), 1e-30))
-        res['gpu_vs_oracle_max_rel'] = {
-            'value': rel(gx[None], np.asarray(out.x, dtype=np.float64)[None]),
-            'jacobian': rel(gJ, np.asarray(out.J, dtype=np.float64).reshape(out.J.shape[0], -1)[:, :n]),
-            'laplacian': rel(gl[None], np.asarray(out.lap, dtype=np.float64)[None]),
-            'walkers': n,
-        }
+
+        def against_oracle(triplet):
+            gx, gJ, gl = triplet
+            return {
+                'value': rel(gx[None], np.asarray(out.x, dtype=np.float64)[None]),
+                'jacobian': rel(gJ, np.asarray(out.J, dtype=np.float64).reshape(out.J.shape[0], -1)[:, :n]),
+                'laplacian': rel(gl[None], np.asarray(out.lap, dtype=np.float64)[None]),
+                'walkers': n,
+            }
+
+        res['gpu_vs_oracle_max_rel'] = against_oracle(gpu_out)
+        if gpu_out_split is not None:  # the run with the bf16x3 products, same walkers
+            res['bf16x3_vs_oracle_max_rel'] = against_oracle(gpu_out_split)
     return res
 
 
@@ -131,6 +143,7 @@ def main():
     from folx_amd import kernels as K
     from folx_amd import workloads as wl
 
+    K.set_gemm_mode(args.gemm)
     forward, params_np, cfg, B, sigma, thr = wl.build(args.workload)
     if args.walkers:
         B = args.walkers
@@ -193,7 +206,8 @@ def main():
         achieved = flops / (dms / dn * 1e-3) / 1e12
         roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
                 'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': ('dense_dma_kernel' if Kd % 16 == 0 and N % 4 == 0 else 'dense_kernel')
+                'kernel': (('dense_split_kernel' if args.gemm == 'bf16x3' and N > 128 else 'dense_dma_kernel')
+                           if Kd % 16 == 0 and N % 4 == 0 else 'dense_kernel')
                 + f' R={R} P={P} K={Kd} N={N} residual={has_res}', 'launches': dn,
                 'avg_launch_ms': dms / dn}
     elif dname == 'mhsa_fwdlap':
@@ -249,6 +263,7 @@ def main():
             'walkers': B,
             'chunk': args.chunk,
             'jacobian_rows': int(out.jacobian.dense_array.shape[0]),
+            'gemm': args.gemm,
         },
         'roofline': roof,
         # from the one untimed step in which every entry point carried events
@@ -257,11 +272,40 @@ def main():
     if roof is not None and roof.get('traffic') is not None:
         roof['traffic_source'] = ('profiles/psiformer32_forward_laplacian.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this '
                                   'command in earlier runs (counters cannot be read inside the timed run)')
+    if args.gemm == 'bf16x3' and roof is not None and roof['bound'] == 'mfma' and 'mhsa' not in roof['kernel']:
+        # six bf16 piece products per fp32 product: the matrix pipe's bf16 peak over six
+        roof['peak'] = PEAK_BF16_MFMA_TFLOPS / 6.0
+        roof['frac'] = roof['achieved'] / roof['peak']
+        roof['peak_note'] = 'bf16 dense peak 2500 TFLOP/s / 6 piece products per fp32 product'
+    if args.gemm == 'f32' and not args.no_split_leg and not args.graph:
+        # the same step with the products of the wide dense rules on the bf16 pipe (three exact bf16
+        # pieces per operand): reported beside the headline, never as `value`
+        K.set_gemm_mode('bf16x3')
+        try:
+            out2 = step(x)
+            torch.cuda.synchronize()
+            n2 = max(1, min(args.steps, 5))
+            t0 = time.perf_counter()
+            for _ in range(n2):
+                out2 = step(x)
+            torch.cuda.synchronize()
+            dt2 = time.perf_counter() - t0
+        finally:
+            K.set_gemm_mode('f32')
+        line['bf16x3_products'] = {
+            'value': B * n2 / dt2, 'unit': 'walkers/s', 'steps': n2, 'ms_per_step': 1e3 * dt2 / n2,
+            'how': 'FOLX_AMD_GEMM=bf16x3 / folx_hip_set_gemm_mode(1); fp32 inputs, outputs and accumulators'}
+    else:
+        out2 = None
     if not args.no_cpu:
-        gpu_out = None
-        if tuple(out.x.shape) == (B,):
-            gpu_out = (out.x.cpu().numpy(), out.jacobian.dense_array.reshape(-1, B).cpu().numpy(), out.laplacian.cpu().numpy())
-        line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds, gpu_out)
+        host = lambda o: (o.x.cpu().numpy(), o.jacobian.dense_array.reshape(-1, B).cpu().numpy(),  # noqa: E731
+                          o.laplacian.cpu().numpy())
+        gpu_out = host(out) if tuple(out.x.shape) == (B,) else None
+        gpu_out2 = host(out2) if out2 is not None and gpu_out is not None else None
+        line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds, gpu_out, gpu_out2)
+        if 'bf16x3_vs_oracle_max_rel' in line['cpu_baseline']:  # same walkers, same oracle run as the headline's figures
+            line['bf16x3_products']['gpu_vs_oracle_max_rel'] = line['cpu_baseline'].pop('bf16x3_vs_oracle_max_rel')
+    del out2
     # the reference itself (JAX on the host cores) can only be timed where jax is installed
     import importlib.util
 
