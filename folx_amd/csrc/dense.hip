@@ -575,7 +575,9 @@ __global__ __launch_bounds__(512, 4) void dense_split_kernel(Segs sg, const floa
   const int KT = K / 16;
   float4 ra, rw0, rw1;
   auto fetch = [&](int kt) __attribute__((always_inline)) {
-    ra = folx_ld_stream4(a_src + kt * 16);
+    // (a plain load: the other half of each 128-byte line is asked for one chunk later and
+    // should still be in L2 then, which a non-temporal request does not promise)
+    ra = *reinterpret_cast<const float4*>(a_src + kt * 16);
     rw0 = *reinterpret_cast<const float4*>(w_src + (int64_t)kt * 16 * N);
     rw1 = *reinterpret_cast<const float4*>(w_src + (int64_t)kt * 16 * N + N);
   };

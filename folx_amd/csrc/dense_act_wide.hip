@@ -68,7 +68,7 @@ constexpr int TM = WROWS / 32, TN = WCOLS / 32;
 constexpr int TG = BK / 8;
 constexpr int NXCD = 8;
 constexpr int KMAX_NORM = 512; // xh of a tile's positions sits in LDS
-constexpr int KMAX_NORM_SPLIT = 256;  // bf16x3 form: its larger tiles leave room for 256 features
+constexpr int KMAX_NORM_SPLIT = 512;  // bf16x3 form: with xh of 4 x 512 features its LDS is exactly half a CU's
 constexpr int A_V4 = BM * BK / 4, W_V4 = BK * BN / 4;
 constexpr int A_LD = A_V4 / NT, W_LD = W_V4 / NT;
 static_assert(A_V4 % NT == 0 && W_V4 % NT == 0, "every thread loads the same number of pieces");
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   __shared__ __attribute__((aligned(16))) float xhS[NORM ? RT * (SPLIT ? KMAX_NORM_SPLIT : KMAX_NORM) : 4];
   __shared__ float zS[NORM && !SPLIT ? RT * BN : 1];  // pre-activation values of the tile's positions and columns
   __shared__ float2 wcS[NORM && !SPLIT ? BN : 1];     // (w1, c0) of the tile's columns
-  __shared__ float rsS[RT];
+  __shared__ float rsS[SPLIT ? 1 : RT];  // SPLIT: rs is read from memory in the epilogue
 
   // ids are dealt round-robin to the XCDs: the column tiles of a row tile stay on one of them
   const int64_t id = blockIdx.x;
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     sw_dst = (wave * BN + lane * 4) * 4;
   }
   auto fetch = [&](int kt) __attribute__((always_inline)) {
-    ra = folx_ld_stream4(sa_src + kt * BK);
+    ra = *reinterpret_cast<const float4*>(sa_src + kt * BK);  // plain: the line's other half follows one chunk later
     rw0 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N);
     rw1 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N + N);
   };
@@ -276,7 +276,8 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     for (int e = tid; e < RT * K / 4; e += NT) reinterpret_cast<float4*>(xhS)[e] = src[e];
     if constexpr (!SPLIT)
       if (tid < BN) wcS[tid] = a.wc[col0 + tid < N ? col0 + tid : N - 1];
-    if (tid < RT) rsS[tid] = a.rs[r0 + tid];
+    if constexpr (!SPLIT)
+      if (tid < RT) rsS[tid] = a.rs[r0 + tid];
   }
 
   floatx16 acc[TM][TN];
@@ -521,7 +522,7 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   for (int i = 0; i < TM; ++i) {
     const int64_t pos = r0 + (wrow * TM + i) * PB;
     float rsv = 1.0f;
-    if constexpr (NORM) rsv = rsS[wrow * TM + i];
+    if constexpr (NORM) rsv = SPLIT ? a.rs[r0 + wrow * TM + i] : rsS[wrow * TM + i];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int gc = col0 + wc + j * 32 + l32;

@@ -108,7 +108,7 @@ NORM_DENSE_CASES = [
     ((1, 8), 40, 64, 132, False, True, None),        # no gamma / beta, partial group of Jacobian rows, cut column tile
     ((3, 4), 1, 16, 300, True, False, 'softplus'),   # one chunk of K, one Jacobian row
     ((1, 4), 64, 48, 256, True, True, 'sin'),        # odd number of chunks
-    ((1, 12), 33, 512, 512, True, True, 'silu'),     # K past the split form's 256: runs on the fp32 instructions
+    ((1, 12), 33, 512, 512, True, True, 'silu'),     # widest K of the LayerNorm form, two column tiles
 ]
 
 
