@@ -677,6 +677,62 @@ __global__ __launch_bounds__(256) void dense_n1_kernel(Segs sg, const float* __r
   }
 }
 
+// The same for contiguous rows (no row groups) and K <= 256: the rows of a block are read as ONE
+// flat run of 128-bit pieces, consecutive lanes consecutive pieces (every lane busy, whole lines
+// per request, a handful of instructions per piece instead of a reduction tree per row).  Piece
+// f of the block lies in row f / (K / 4) at k = 4 (f % (K / 4)); its product with the four
+// weights goes to LDS, and after a barrier thread r adds the K / 4 partial sums of row r
+// (stride K / 4 floats between threads: no bank conflict when K / 4 is odd, e.g. K = 100).
+constexpr int N1_ROWS = 64;    // rows per block
+constexpr int N1_MAXK4 = 64;   // K <= 256
+__global__ __launch_bounds__(256) void dense_n1_flat_kernel(Segs sg, const float* __restrict__ W,
+                                                            const float* __restrict__ bias, int32_t K) {
+  __shared__ __attribute__((aligned(16))) float wS[4 * N1_MAXK4];
+  __shared__ float part[N1_ROWS * N1_MAXK4];
+  int seg = 0;
+  int64_t t = blockIdx.x;
+  if (t >= sg.tiles[0]) { t -= sg.tiles[0]; seg = 1; if (t >= sg.tiles[1]) { t -= sg.tiles[1]; seg = 2; } }
+  const int K4 = K / 4;
+  const int64_t row0 = t * N1_ROWS;
+  const int nrows = (int)(sg.rows[seg] - row0 < N1_ROWS ? sg.rows[seg] - row0 : N1_ROWS);
+  const int nf = nrows * K4;
+  const float* base = sg.in[seg] + row0 * (int64_t)K;
+  const int tid = threadIdx.x;
+  if (tid < K4) reinterpret_cast<float4*>(wS)[tid] = *reinterpret_cast<const float4*>(W + 4 * tid);
+  // up to 16 pieces per thread, eight requests in flight
+  constexpr int U = 8;
+  const int step = 256 % K4;
+  int k4 = tid % K4;
+  __syncthreads();
+  for (int f0 = tid; f0 < nf; f0 += U * 256) {
+    float4 a[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int f = f0 + u * 256;
+      a[u] = folx_ld_stream4(base + 4 * (int64_t)(f < nf ? f : f0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int f = f0 + u * 256;
+      const float4 w = reinterpret_cast<const float4*>(wS)[k4];
+      if (f < nf) part[f] = fmaf(a[u].x, w.x, fmaf(a[u].y, w.y, fmaf(a[u].z, w.z, a[u].w * w.w)));
+      k4 += step;
+      if (k4 >= K4) k4 -= K4;
+    }
+  }
+  __syncthreads();
+  if (tid < nrows) {
+    const float* pr = part + tid * K4;
+    float s0 = 0.0f, s1 = 0.0f;
+    int c = 0;
+    for (; c + 2 <= K4; c += 2) { s0 += pr[c]; s1 += pr[c + 1]; }
+    if (c < K4) s0 += pr[c];
+    float o = s0 + s1 + (seg == 0 && bias != nullptr ? bias[0] : 0.0f);
+    if (sg.res[seg] != nullptr) o += sg.res[seg][row0 + tid];
+    sg.out[seg][row0 + tid] = o;
+  }
+}
+
 template <int BM, int BN, int WM, int WN, int MINB>
 int launch_cfg(hipStream_t st, Segs& sg, const float* W, const float* bias, int32_t K, int32_t N,
                bool vec, bool has_res) {
@@ -740,6 +796,14 @@ extern "C" int folx_hip_dense_rows_fwdlap(void* stream, const float* x, const fl
   const bool has_res = res != nullptr;
   hipStream_t st = (hipStream_t)stream;
   if (N == 1 && K % 4 == 0 && folx_aligned16(x) && folx_aligned16(jac) && folx_aligned16(lap) && folx_aligned16(W)) {
+    if (group == 0 && K <= 4 * N1_MAXK4) {
+      int64_t tiles = 0;
+      for (int s = 0; s < 3; ++s) { sg.tiles[s] = (sg.rows[s] + N1_ROWS - 1) / N1_ROWS; tiles += sg.tiles[s]; }
+      if (tiles <= 0x7fffffffLL) {
+        dense_n1_flat_kernel<<<dim3((unsigned)tiles), dim3(256), 0, st>>>(sg, W, bias, K);
+        return folx_launch_status();
+      }
+    }
     const int64_t total = (int64_t)(P + 2) * R;
     const int64_t blocks = std::min<int64_t>((total + 31) / 32, 256 * 32);
     dense_n1_kernel<<<dim3((unsigned)blocks), dim3(256), 0, st>>>(sg, W, bias, K, total);

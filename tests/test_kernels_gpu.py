@@ -104,7 +104,8 @@ DENSE_CASES = [
     ((20, 100), 40, 100, 1, True),     # last layer of the README MLP
     ((1, 1), 0, 4, 2, False),
     ((1, 1), 0, 4, 1, False),          # one row, one 128-bit load
-    ((3, 37), 5, 300, 1, True),        # three passes over K, the last one partial
+    ((3, 37), 5, 300, 1, True),        # K > 256: one row per 32 lanes, three passes over K
+    ((3, 50), 2, 256, 1, False),       # widest K of the flat-run kernel, ragged last block of rows
     ((2, 9), 3, 18, 1, True),          # K % 4 != 0: N = 1 through the GEMM
 ]
 
