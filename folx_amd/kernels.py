@@ -85,7 +85,8 @@ def set_gemm_mode(mode: str):
     """How the wide dense rules form their fp32 products: ``'f32'`` (FP32 matrix instructions, the
     default) or ``'bf16x3'`` (operands split exactly into three bf16 pieces, six exact piece
     products per product accumulated in fp32: same accuracy, the faster matrix pipe).  Process
-    wide; the environment variable ``FOLX_AMD_GEMM`` sets it when the library is loaded."""
+    wide; the environment variable ``FOLX_AMD_GEMM`` sets it when the library is loaded.  A HIP
+    graph captured by ``folx_amd.jit`` keeps the kernels of the mode it was captured under."""
     if mode not in _lib.GEMM_MODE:
         raise ValueError(f'gemm mode {mode!r}: expected one of {sorted(_lib.GEMM_MODE)}')
     _lib.check(_lib.load().folx_hip_set_gemm_mode(_lib.GEMM_MODE[mode]), 'set_gemm_mode')
