@@ -8,6 +8,9 @@
 // fp32 multiply-add.  Six bf16 products of depth 16 take 6 x 8 passes on the matrix pipe for
 // the work of 8 v_mfma_f32_32x32x2_f32 (8 x 16 passes): 2.7 times the FP32 rate.
 //
+// An infinite element (or one that rounds to a bf16 infinity) turns into NaN: x - bf16(x) is
+// inf - inf.  Finite inputs, the case the rules are used for, are represented exactly.
+//
 // The mode is process wide (folx_hip_set_gemm_mode); kernels that have no split form ignore it.
 #pragma once
 #include "common.h"

@@ -50,7 +50,10 @@ const char* folx_hip_strerror(int code);
  *                        terms weigh <= 2^-24 of a product, the rounding of one fp32
  *                        multiply-add, so results agree with the fp32 form to fp32 rounding;
  *                        inputs, outputs and accumulators stay fp32.  Kernels without a split
- *                        form run as under FOLX_HIP_GEMM_F32.
+ *                        form run as under FOLX_HIP_GEMM_F32.  Where the two forms differ: an
+ *                        infinite operand element (or one within 2^-9 of FLT_MAX, which rounds
+ *                        to a bf16 infinity) gives NaN instead of an infinity, because its
+ *                        remainder x - bf16(x) is inf - inf.
  * The mode is process wide and read at every launch; set it before launching, not while other
  * threads launch.  folx_hip_set_gemm_mode returns FOLX_HIP_EINVAL for any other value. */
 #define FOLX_HIP_GEMM_F32 0
