@@ -29,13 +29,16 @@ def test_exports_every_declared_symbol(lib):
 
 def test_gemm_mode_switch(lib):
     """The mode is a host-side flag: setting and reading it needs no GPU."""
-    assert lib.folx_hip_get_gemm_mode() == _lib.GEMM_MODE['f32']  # the default
+    if 'FOLX_AMD_GEMM' not in os.environ:
+        assert lib.folx_hip_get_gemm_mode() == _lib.GEMM_MODE['f32']  # the default
+    before = lib.folx_hip_get_gemm_mode()
     assert lib.folx_hip_set_gemm_mode(_lib.GEMM_MODE['bf16x3']) == _lib.OK
     assert lib.folx_hip_get_gemm_mode() == _lib.GEMM_MODE['bf16x3']
     assert lib.folx_hip_set_gemm_mode(7) == _lib.EINVAL
     assert lib.folx_hip_get_gemm_mode() == _lib.GEMM_MODE['bf16x3']  # unchanged by the refused call
     assert lib.folx_hip_set_gemm_mode(_lib.GEMM_MODE['f32']) == _lib.OK
     assert lib.folx_hip_get_gemm_mode() == _lib.GEMM_MODE['f32']
+    assert lib.folx_hip_set_gemm_mode(before) == _lib.OK
 
 
 def test_version_and_strerror(lib):

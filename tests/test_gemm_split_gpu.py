@@ -28,10 +28,11 @@ def rand(rng, *shape):
 def split_mode():
     from folx_amd import kernels as K
 
+    before = K.get_gemm_mode()  # 'f32' unless FOLX_AMD_GEMM says otherwise
     K.set_gemm_mode('bf16x3')
     assert K.get_gemm_mode() == 'bf16x3'
     yield K
-    K.set_gemm_mode('f32')
+    K.set_gemm_mode(before)
 
 
 DENSE_CASES = [
@@ -89,13 +90,14 @@ def test_dense_split_error_is_that_of_fp32():
     # per output entry: error relative to sum_k |a_k w_k|, the scale that bounds any summation order
     bound = np.abs(f64(J)[0]) @ np.abs(f64(W)[0])
     errs = {}
+    before = K.get_gemm_mode()
     try:
         for mode in ('f32', 'bf16x3'):
             K.set_gemm_mode(mode)
             got = K.dense(dev(x), dev(J), dev(L), dev(W), None)
             errs[mode] = float((np.abs(got[1].cpu().numpy().astype(np.float64) - ref[1]) / bound).max())
     finally:
-        K.set_gemm_mode('f32')
+        K.set_gemm_mode(before)
     print('relative to sum |a w|:', errs, flush=True)
     assert errs['bf16x3'] <= 1.5 * errs['f32'] + 1e-9
     assert errs['bf16x3'] < 2.0 ** -20
