@@ -281,6 +281,7 @@ def main():
         # the same step with the products of the wide dense rules on the bf16 pipe (three exact bf16
         # pieces per operand): reported beside the headline, never as `value`
         K.set_gemm_mode('bf16x3')
+        out2 = None
         try:
             out2 = step(x)
             torch.cuda.synchronize()
@@ -290,11 +291,14 @@ def main():
                 out2 = step(x)
             torch.cuda.synchronize()
             dt2 = time.perf_counter() - t0
+            line['bf16x3_products'] = {
+                'value': B * n2 / dt2, 'unit': 'walkers/s', 'steps': n2, 'ms_per_step': 1e3 * dt2 / n2,
+                'how': 'FOLX_AMD_GEMM=bf16x3 / folx_hip_set_gemm_mode(1); fp32 inputs, outputs and accumulators'}
+        except Exception as e:  # the side measurement must not take the headline line down with it
+            out2 = None
+            line['bf16x3_products'] = {'error': f'{type(e).__name__}: {e}'}
         finally:
             K.set_gemm_mode('f32')
-        line['bf16x3_products'] = {
-            'value': B * n2 / dt2, 'unit': 'walkers/s', 'steps': n2, 'ms_per_step': 1e3 * dt2 / n2,
-            'how': 'FOLX_AMD_GEMM=bf16x3 / folx_hip_set_gemm_mode(1); fp32 inputs, outputs and accumulators'}
     else:
         out2 = None
     if not args.no_cpu:
@@ -304,7 +308,7 @@ def main():
         gpu_out2 = host(out2) if out2 is not None and gpu_out is not None else None
         line['cpu_baseline'] = cpu_baseline(args.workload, args.cpu_seconds, gpu_out, gpu_out2)
         if 'bf16x3_vs_oracle_max_rel' in line['cpu_baseline']:  # same walkers, same oracle run as the headline's figures
-            line['bf16x3_products']['gpu_vs_oracle_max_rel'] = line['cpu_baseline'].pop('bf16x3_vs_oracle_max_rel')
+            line.setdefault('bf16x3_products', {})['gpu_vs_oracle_max_rel'] = line['cpu_baseline'].pop('bf16x3_vs_oracle_max_rel')
     del out2
     # the reference itself (JAX on the host cores) can only be timed where jax is installed
     import importlib.util
