@@ -30,6 +30,10 @@
 // with one 32-bit lane offset for all stores and wave-uniform scalar row arithmetic; the
 // bias is fetched before the K loop.  Edge tiles take a checked path.
 //
+// Two more forms of the rule live here: N = 1 (a matrix-vector product, dense_n1_flat_kernel /
+// dense_n1_kernel) and, when folx_hip_set_gemm_mode asks for it, the 128 x 256 tile with every
+// fp32 product taken as six exact products of bf16 pieces (dense_split_kernel, split_bf16.h).
+//
 // Workgroup ids are remapped so that the column tiles of one row tile run back to back
 // on the same XCD (ids are dealt round-robin to the 8 XCDs), which keeps the second
 // read of an A tile in that XCD's L2 when N needs more than one column tile.
