@@ -117,12 +117,13 @@ struct WideParams {
 // values, so LayerNorm's row sums are taken there (and added over the four threads of a row
 // after the loop) instead of from the fragments of chosen wavefronts; the per-column values the
 // epilogue needs (z, w1, c0) are fetched from memory after the loop, which leaves LDS for two
-// workgroups per CU.
+// workgroups per CU.  A concatenated operand (PARTS) is staged the same way, the part of a chunk
+// and the address inside it found per chunk as in the direct-to-LDS form.
 template <bool NORM, bool ACT, int PT, bool PARTS, bool SPLIT>
 __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
   static_assert(!PARTS || !NORM, "LayerNorm reads one array");
   static_assert(!PARTS || A_LD == 1, "one A piece per thread");
-  static_assert(!SPLIT || (!PARTS && PT == 32), "the split form reads one array in groups of 32 rows");
+  static_assert(!SPLIT || !NORM || PT == 32, "LayerNorm's row sums assume groups of 32 rows");
   constexpr int A_PLANE = 2 * BM * 16;     // SPLIT: bytes of one piece of an A chunk
   constexpr int W_PLANE = 2 * 4 * BN * 4;  //        and of a W chunk
   constexpr int RT = BM / PT;  // positions of a tile
@@ -238,7 +239,14 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     const int m = tid / 4, q = tid % 4;
     int p = p0 + m % PT;
     if (p >= P) p = P - 1;
-    sa_src = a.jac + ((int64_t)p * R + r0 + m / PT) * K + q * 4;
+    if constexpr (PARTS) {  // the part and the address inside it are found per chunk
+      a_pos = r0 + m / PT;
+      a_posg = a_pos / a.parts.group;
+      a_row = p;
+      a_kc = q * 4;
+    } else {
+      sa_src = a.jac + ((int64_t)p * R + r0 + m / PT) * K + q * 4;
+    }
     sa_dst = ((q / 2) * BM + m) * 16 + (q % 2) * 8;
     int wn = col0 + lane * 4;
     if (wn > N - 4) wn = N - 4;
@@ -246,7 +254,16 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     sw_dst = (wave * BN + lane * 4) * 4;
   }
   auto fetch = [&](int kt) __attribute__((always_inline)) {
-    ra = *reinterpret_cast<const float4*>(sa_src + kt * BK);  // plain: the line's other half follows one chunk later
+    if constexpr (PARTS) {
+      const int k0 = kt * BK;
+      int sp = 0;
+      while (sp + 1 < a.parts.n && k0 >= a.parts.kend[sp]) ++sp;
+      const int32_t wd = a.parts.width[sp];
+      ra = *reinterpret_cast<const float4*>(a.parts.jac[sp] + (int64_t)a_row * a.parts.pstride[sp] +
+                                            (a.parts.bcast[sp] ? a_posg : a_pos) * wd + (k0 - (a.parts.kend[sp] - wd)) + a_kc);
+    } else {
+      ra = *reinterpret_cast<const float4*>(sa_src + kt * BK);  // plain: the line's other half follows one chunk later
+    }
     rw0 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N);
     rw1 = *reinterpret_cast<const float4*>(sw_src + (int64_t)kt * BK * N + N);
   };
@@ -872,12 +889,8 @@ bool plan_wide(int64_t R, int32_t P, int32_t K, int32_t N, bool norm, bool act, 
 template <bool NORM, bool ACT, int PT, bool PARTS = false>
 int launch_wide(hipStream_t st, const WideParams& a, const WidePlan& pl, float* y, float* y_lap,
                 const float* res = nullptr, const float* res_lap = nullptr) {
-  bool split = false;
-  if constexpr (!PARTS && PT == 32)
-    split = folx_gemm_mode() == FOLX_HIP_GEMM_BF16X3 && (!NORM || a.K <= KMAX_NORM_SPLIT);
-  if constexpr (!PARTS && PT == 32) {
-    if (split) dense_wide_kernel<NORM, ACT, PT, PARTS, true><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
-  }
+  const bool split = folx_gemm_mode() == FOLX_HIP_GEMM_BF16X3 && (!NORM || a.K <= KMAX_NORM_SPLIT);
+  if (split) dense_wide_kernel<NORM, ACT, PT, PARTS, true><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   if (!split) dense_wide_kernel<NORM, ACT, PT, PARTS, false><<<dim3((unsigned)pl.blocks), dim3(NT), 0, st>>>(a);
   int rc = folx_launch_status();
   if (rc != FOLX_HIP_OK) return rc;

@@ -196,3 +196,16 @@ def test_full_width_models_split(split_mode, name):
 
     tm.test_full_width_every_rule_call_meets_the_strict_bars(name)
     tm.test_full_width_well_conditioned_end_to_end_strict(name)
+
+
+@pytest.mark.parametrize('B,n,P,widths,bcast,N,act', [
+    (2, 6, 30, (16, 32), (1, 0), 132, 'silu'),                            # groups of 32 rows, broadcast part first
+    (1, 8, 5, (48,), (0,), 300, 'sin'),                                   # a single part
+    (3, 8, 17, (16, 16, 16, 16, 16, 16, 16, 16), (0, 1, 0, 1, 0, 1, 0, 1), 256, 'softplus'),  # eight parts
+    (4, 16, 16, (64, 32), (0, 1), 256, 'tanh'),                           # P = 16: groups of 16 rows, 8 positions per tile
+])
+def test_dense_act_parts_split(split_mode, B, n, P, widths, bcast, N, act):
+    """The concatenated-operand layer (skip connection, per-walker pre-activation term) under the bf16x3 products."""
+    import test_kernels_gpu as tk
+
+    tk.test_dense_act_parts(B, n, P, widths, bcast, N, act)
