@@ -44,7 +44,9 @@ struct DotTwoArgs {
 };
 
 // MAXLD = values per thread of one tile: 32 * Kp / 256 with Kp = Kc rounded up to 16
-template <int MAXLD>
+// CONSTB: b carries no derivatives (a constant with batch axes, e.g. per-head weights): the rule is
+// linear in a, y_jac[p] = a_jac[p] b and y_lap = a_lap b, one product chain per row and no b rows.
+template <int MAXLD, bool CONSTB>
 __global__ __launch_bounds__(DT_NT) void dot_two_kernel(DotTwoArgs g) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   const int Kc = g.Kc;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(DT_NT) void dot_two_kernel(DotTwoArgs g) {
   put_b(Bs, rb);
   // first row in flight: Jacobian row 0, or the Laplacian operands when there are no rows
   fetch_a(g.P > 0 ? g.aj : g.al, ra);
-  fetch_b(g.P > 0 ? g.bj : g.bl, rb);
+  if constexpr (!CONSTB) fetch_b(g.P > 0 ? g.bj : g.bl, rb);
   __syncthreads();
 
   // A operand of step (t, r): tile[16 wi + l16][16 t + 4 lg + r]; B operand: tile[16 t + 4 lg + r][16 wj + l16]
@@ -156,12 +158,12 @@ __global__ __launch_bounds__(DT_NT) void dot_two_kernel(DotTwoArgs g) {
   floatx4 lap2 = {0.f, 0.f, 0.f, 0.f};  // sum_p a_jac[p] b_jac[p]
   for (int p = 0; p <= g.P; ++p) {
     put_a(AJs, ra);
-    put_b(BJs, rb);
+    if constexpr (!CONSTB) put_b(BJs, rb);
     __syncthreads();
     if (p < g.P) {  // next row: Jacobian row p + 1, or the Laplacian operands after the last one
       const bool last = p + 1 == g.P;
       fetch_a(last ? g.al : g.aj + (int64_t)(p + 1) * g.a_sp, ra);
-      fetch_b(last ? g.bl : g.bj + (int64_t)(p + 1) * g.b_sp, rb);
+      if constexpr (!CONSTB) fetch_b(last ? g.bl : g.bj + (int64_t)(p + 1) * g.b_sp, rb);
     }
     floatx4 acc = {0.f, 0.f, 0.f, 0.f}, cross = {0.f, 0.f, 0.f, 0.f};
     for (int t = 0; t < kt; ++t) {
@@ -169,12 +171,15 @@ __global__ __launch_bounds__(DT_NT) void dot_two_kernel(DotTwoArgs g) {
       const float4 ajv = *reinterpret_cast<const float4*>(aj_row + 16 * t);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float bv = b_col[(16 * t + r) * DT_BS], bjv = bj_col[(16 * t + r) * DT_BS];
-        const float ar = r == 0 ? av.x : (r == 1 ? av.y : (r == 2 ? av.z : av.w));
+        const float bv = b_col[(16 * t + r) * DT_BS];
         const float ajr = r == 0 ? ajv.x : (r == 1 ? ajv.y : (r == 2 ? ajv.z : ajv.w));
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ajr, bv, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ar, bjv, acc, 0, 0, 0);
-        cross = __builtin_amdgcn_mfma_f32_16x16x4f32(ajr, bjv, cross, 0, 0, 0);
+        if constexpr (!CONSTB) {
+          const float bjv = bj_col[(16 * t + r) * DT_BS];
+          const float ar = r == 0 ? av.x : (r == 1 ? av.y : (r == 2 ? av.z : av.w));
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ar, bjv, acc, 0, 0, 0);
+          cross = __builtin_amdgcn_mfma_f32_16x16x4f32(ajr, bjv, cross, 0, 0, 0);
+        }
       }
     }
     if (p < g.P) {
@@ -197,7 +202,9 @@ extern "C" int folx_hip_dot_two_fwdlap(void* stream, const float* a, const float
   if (Kc > DT_KMAX) return FOLX_HIP_ENOTSUP;
   const int64_t NB = NB0 * NB1;
   if (NB == 0 || I == 0 || J == 0) return FOLX_HIP_OK;
-  if (!a || !a_lap || !b || !b_lap || !y || !y_lap || (P > 0 && (!a_jac || !b_jac || !y_jac))) return FOLX_HIP_EINVAL;
+  const bool constb = !b_jac && !b_lap;  // b without derivatives
+  if (!a || !a_lap || !b || !y || !y_lap || (P > 0 && (!a_jac || !y_jac))) return FOLX_HIP_EINVAL;
+  if (!constb && (!b_lap || (P > 0 && !b_jac))) return FOLX_HIP_EINVAL;
   DotTwoArgs g;
   g.a = a; g.aj = a_jac; g.al = a_lap; g.b = b; g.bj = b_jac; g.bl = b_lap;
   g.y = y; g.yj = y_jac; g.yl = y_lap;
@@ -216,20 +223,28 @@ extern "C" int folx_hip_dot_two_fwdlap(void* stream, const float* a, const float
   const size_t lds = sizeof(float) * (2 * DT_TILE * (Kp + 4) + 2 * Kp * DT_BS);
   hipStream_t st = (hipStream_t)stream;
   const int nld = DT_TILE * Kp / DT_NT;  // 2, 4, ..., 16
-  if (nld <= 4) dot_two_kernel<4><<<dim3((unsigned)blocks), dim3(DT_NT), lds, st>>>(g);
-  else if (nld <= 8) dot_two_kernel<8><<<dim3((unsigned)blocks), dim3(DT_NT), lds, st>>>(g);
-  else {
+  const dim3 grid((unsigned)blocks), block(DT_NT);
+  if (nld <= 4) {
+    if (constb) dot_two_kernel<4, true><<<grid, block, lds, st>>>(g);
+    else dot_two_kernel<4, false><<<grid, block, lds, st>>>(g);
+  } else if (nld <= 8) {
+    if (constb) dot_two_kernel<8, true><<<grid, block, lds, st>>>(g);
+    else dot_two_kernel<8, false><<<grid, block, lds, st>>>(g);
+  } else {
     if (lds > 64 * 1024) {
       // raised once per process (not a stream operation, so never issued inside a stream capture twice)
       static std::atomic<bool> granted{false};
       if (!granted.load()) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(dot_two_kernel<16>),
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(dot_two_kernel<16, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(dot_two_kernel<16, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess)
           return FOLX_HIP_ENOTSUP;
         granted.store(true);
       }
     }
-    dot_two_kernel<16><<<dim3((unsigned)blocks), dim3(DT_NT), lds, st>>>(g);
+    if (constb) dot_two_kernel<16, true><<<grid, block, lds, st>>>(g);
+    else dot_two_kernel<16, false><<<grid, block, lds, st>>>(g);
   }
   return folx_launch_status();
 }

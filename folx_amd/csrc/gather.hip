@@ -138,19 +138,66 @@ __global__ __launch_bounds__(256) void gather_rows_flat_kernel(const float* __re
   else *q = acc[0];
 }
 
+// out[idx[r][so]][b][so][si] += data[r][b][so][si]   (idx < 0: the entry is skipped)
+// A thread owns VEC consecutive floats of one walker and walks the stored rows r in order, so
+// every output entry is updated by one thread in a fixed order: no atomics, the same bits on
+// every run, also where several stored rows of a position name the same target row.  Eight rows
+// at a time: their table entries, then their data and the target values they land on, all in
+// flight together; rows of a group that share a target are folded into the first of them.
+template <int VEC>
 __global__ __launch_bounds__(256) void scatter_add_rows_kernel(const float* __restrict__ data,
                                                                const int32_t* __restrict__ idx,
-                                                               float* __restrict__ out, int64_t B,
-                                                               int64_t S_outer, int64_t S_inner) {
+                                                               float* out, int32_t k_in, int32_t k_out,
+                                                               int64_t B, int64_t S_outer, int64_t S_inner) {
   const int64_t S = S_outer * S_inner;
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= S) return;
+  const int64_t f = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+  if (f >= B * S) return;
+  const int64_t b = f / S, e = f - b * S;
   const int64_t so = e / S_inner;
-  const int32_t r = blockIdx.z;
-  const int32_t t = idx[(int64_t)r * S_outer + so];
-  if (t < 0) return;
-  for (int64_t b = blockIdx.y; b < B; b += gridDim.y)
-    atomicAdd(&out[((int64_t)t * B + b) * S + e], data[((int64_t)r * B + b) * S + e]);
+  for (int r0 = 0; r0 < k_in; r0 += 8) {
+    int32_t t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      t[u] = r0 + u < k_in ? idx[(int64_t)(r0 + u) * S_outer + so] : -1;
+      if (t[u] >= k_out) t[u] = -1;  // a target outside the output is never written
+    }
+    float val[8][VEC], cur[8][VEC];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) val[u][v] = cur[u][v] = 0.0f;
+      if (t[u] >= 0) {
+        const float* p = data + ((int64_t)(r0 + u) * B + b) * S + e;
+        const float* q = out + ((int64_t)t[u] * B + b) * S + e;
+        if constexpr (VEC == 4) {
+          const float4 a = folx_ld_stream4(p);
+          val[u][0] = a.x; val[u][1] = a.y; val[u][2] = a.z; val[u][3] = a.w;
+          const float4 c = *reinterpret_cast<const float4*>(q);
+          cur[u][0] = c.x; cur[u][1] = c.y; cur[u][2] = c.z; cur[u][3] = c.w;
+        } else {
+          val[u][0] = *p;
+          cur[u][0] = *q;
+        }
+      }
+    }
+    // the first row of a group that names a target collects the later ones, in row order
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (t[u] < 0) continue;
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) cur[u][v] += val[u][v];
+#pragma unroll
+      for (int w = u + 1; w < 8; ++w)
+        if (t[w] == t[u]) {
+#pragma unroll
+          for (int v = 0; v < VEC; ++v) cur[u][v] += val[w][v];
+          t[w] = -1;
+        }
+      float* q = out + ((int64_t)t[u] * B + b) * S + e;
+      if constexpr (VEC == 4) *reinterpret_cast<float4*>(q) = make_float4(cur[u][0], cur[u][1], cur[u][2], cur[u][3]);
+      else *q = cur[u][0];
+    }
+  }
 }
 
 // Static gather along the position axis with a sum over slots (the transposed form of a
@@ -218,12 +265,16 @@ extern "C" int folx_hip_scatter_add_rows(void* stream, const float* data, const 
   const int64_t S = S_outer * S_inner;
   if (k_in == 0 || B == 0 || S == 0) return FOLX_HIP_OK;
   if (!data || !idx || !out) return FOLX_HIP_EINVAL;
-  if (k_in > 65535) return FOLX_HIP_ENOTSUP;
-  const int64_t blocks = (S + 255) / 256;
+  const bool vec4 = S_inner % 4 == 0 && folx_aligned16(data) && folx_aligned16(out);
+  const int64_t threads = vec4 ? B * S / 4 : B * S;
+  const int64_t blocks = (threads + 255) / 256;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
-  const unsigned gy = (unsigned)(B < 4096 ? B : 4096);
-  scatter_add_rows_kernel<<<dim3((unsigned)blocks, gy, (unsigned)k_in), dim3(256), 0, (hipStream_t)stream>>>(
-      data, idx, out, B, S_outer, S_inner);
+  if (vec4)
+    scatter_add_rows_kernel<4><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        data, idx, out, k_in, k_out, B, S_outer, S_inner);
+  else
+    scatter_add_rows_kernel<1><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        data, idx, out, k_in, k_out, B, S_outer, S_inner);
   return folx_launch_status();
 }
 

@@ -338,6 +338,49 @@ def dot_two(a, aj, al, b, bj, bl):
     return y, yj, yl
 
 
+def dot_const(a, aj, al, W):
+    """Batched product of a triplet with a constant that has a batch axis: a (B, Bt, I, Kc), aj (P, B, Bt, I, Kc),
+    al like a, W (Bt, Kc, J) float32 on the GPU -> contiguous y (B, Bt, I, J), y_jac (P, B, Bt, I, J), y_lap.  The
+    operands may be views; W is read once per batch element (walker stride 0).  Contracted lengths beyond the
+    kernel's tile depth are cut into slices of the contracted axis (views) whose products are added."""
+    for t in (a, aj, al, W):
+        assert t.is_cuda and t.dtype == torch.float32
+    B, Bt, I, Kc = a.shape
+    J = W.shape[-1]
+    P = aj.shape[0]
+    assert tuple(W.shape) == (Bt, Kc, J) and tuple(aj.shape) == (P, *a.shape) and al.shape == a.shape
+
+    def same_layout(t, u_strides):
+        return all(st == su for st, su, n in zip(t.stride(), u_strides, t.shape) if n > 1)
+
+    if not (same_layout(a, al.stride()) and (P == 0 or same_layout(a, aj.stride()[1:]))):
+        a, aj, al = a.contiguous(), aj.contiguous(), al.contiguous()
+    out = None
+    for k0 in range(0, max(Kc, 1), DOT_TWO_KMAX):
+        k1 = min(Kc, k0 + DOT_TWO_KMAX)
+        ac, ajc, alc, Wc = a[..., k0:k1], aj[..., k0:k1], al[..., k0:k1], W[:, k0:k1, :]
+        y = torch.empty((B, Bt, I, J), device=a.device, dtype=torch.float32)
+        yj = torch.empty((P, B, Bt, I, J), device=a.device, dtype=torch.float32)
+        yl = torch.empty_like(y)
+        strides = (ctypes.c_int64 * 10)(*ac.stride(), ajc.stride(0) if P else 0, 0, Wc.stride(0), Wc.stride(1),
+                                        Wc.stride(2), 0)
+        with _timed('dot_const_fwdlap', (B * Bt, I, J, k1 - k0, P)):
+            check(
+                _lib.load().folx_hip_dot_two_fwdlap(
+                    _stream(), _p(ac), _p(ajc), _p(alc), _p(Wc), None, None, _p(y), _p(yj), _p(yl),
+                    B, Bt, I, J, k1 - k0, P, strides,
+                ),
+                'dot_two_fwdlap (constant operand)',
+            )
+        if out is None:
+            out = (y, yj, yl)
+        else:
+            add = lambda o, n: o if o.numel() == 0 else rows_affine(o, 1, (o.numel(),), (o.numel(),), None,
+                                                                    n.reshape(-1), 1.0, 1.0).reshape(o.shape)
+            out = tuple(add(o, n) for o, n in zip(out, (y, yj, yl)))
+    return out
+
+
 def elementwise(name, x, jac, lap, param=0.0, inplace=False):
     _chk(x, jac, lap)
     P = jac.shape[0]

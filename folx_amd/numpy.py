@@ -194,32 +194,138 @@ def exp_envelope(d, sigma, pi):
     return _call('exp_envelope', (d, sigma, pi))
 
 
+def _tr(a, perm):
+    """transpose that leaves an identity permutation (and a constant's laziness) alone"""
+    perm = [int(i) for i in perm]
+    if perm == list(range(len(perm))):
+        return a
+    return transpose(a, perm) if _is_triplet(a) else np.transpose(np.asarray(a), perm)
+
+
+def _rs(a, shape):
+    shape = tuple(int(n) for n in shape)
+    if _shape(a) == shape:
+        return a
+    return reshape(a, shape) if _is_triplet(a) else np.reshape(np.asarray(a), shape)
+
+
+def dot_general(lhs, rhs, dimension_numbers):
+    """``jax.lax.dot_general``: ``dimension_numbers = ((lhs_contract, rhs_contract), (lhs_batch,
+    rhs_batch))``, output axes ordered batch, lhs free, rhs free.  Either operand (or both) may
+    carry derivatives, any axes may be contracted and a constant operand may have batch axes
+    (per-head weights), as in ``_dot_general_one_constant`` and ``dot_general`` of the reference
+    (folx/wrapped_functions.py:71-171, :174-309).
+
+    Lowering.  One constant operand without batch axes: the operand with derivatives is brought
+    to ``(free..., contract)`` and meets the constant as one matrix through ``dot`` (so the bias /
+    activation / LayerNorm fusions still apply).  One constant operand with batch axes: one
+    batched product ``(batch, i, k) x (batch, k, j)`` whose constant side is read once per batch
+    element.  Two operands with derivatives: the batched two-operand rule through ``matmul``."""
+    (lc, rc), (lb, rb) = dimension_numbers
+    sl, sr = _shape(lhs), _shape(rhs)
+    lc, lb = [int(i) % len(sl) for i in lc], [int(i) % len(sl) for i in lb]
+    rc, rb = [int(i) % len(sr) for i in rc], [int(i) % len(sr) for i in rb]
+    assert len(lc) == len(rc) and len(lb) == len(rb), dimension_numbers
+    assert [sl[i] for i in lc] == [sr[i] for i in rc] and [sl[i] for i in lb] == [sr[i] for i in rb], \
+        f'dot_general: {sl} and {sr} do not match under {dimension_numbers}'
+    lf = [i for i in range(len(sl)) if i not in lc and i not in lb]
+    rf = [i for i in range(len(sr)) if i not in rc and i not in rb]
+    size = lambda shp, idx: int(np.prod([shp[i] for i in idx], dtype=np.int64))
+    bshape = [sl[i] for i in lb]
+    lshape, rshape = [sl[i] for i in lf], [sr[i] for i in rf]
+    Bt, I, J, Kc = size(sl, lb), size(sl, lf), size(sr, rf), size(sl, lc)
+    tl, trr = _is_triplet(lhs), _is_triplet(rhs)
+    if isinstance(lhs, BatchedArray) or isinstance(rhs, BatchedArray):
+        raise NotImplementedError('dot_general on walker-varying constants')
+    if not tl and not trr:
+        y = np.matmul(np.transpose(np.asarray(lhs), lb + lf + lc).reshape(*bshape, I, Kc),
+                      np.transpose(np.asarray(rhs), rb + rc + rf).reshape(*bshape, Kc, J))
+        return y.reshape(*bshape, *lshape, *rshape)
+    if tl and trr:
+        y = matmul(_rs(_tr(lhs, lb + lf + lc), (*bshape, I, Kc)), _rs(_tr(rhs, rb + rc + rf), (*bshape, Kc, J)))
+        return _rs(y, (*bshape, *lshape, *rshape))
+    # exactly one operand carries derivatives: h; the other one is the constant W
+    h, hb, hf, hc, hshape = (lhs, lb, lf, lc, lshape) if tl else (rhs, rb, rf, rc, rshape)
+    W, Wb, Wf, Wc, Wshape = (rhs, rb, rf, rc, rshape) if tl else (lhs, lb, lf, lc, lshape)
+    Ih, Jw = (I, J) if tl else (J, I)
+    W = np.asarray(W)
+    if not hb:
+        Wm = np.transpose(W, Wc + Wf).reshape(Kc, Jw)
+        y = dot(_rs(_tr(h, hf + hc), (*hshape, Kc)), Wm)
+        y = _rs(y, (*hshape, *Wshape))
+        nh, nw = len(hshape), len(Wshape)
+        return y if tl else _tr(y, [*range(nh, nh + nw), *range(nh)])
+    Wm = np.transpose(W, Wb + Wc + Wf).reshape(Bt, Kc, Jw)
+    y = _call('dot_general', (_rs(_tr(h, hb + hf + hc), (Bt, Ih, Kc)), Wm), {'batched_const': True})
+    y = _rs(y, (*bshape, *hshape, *Wshape))
+    nb, nh, nw = len(bshape), len(hshape), len(Wshape)
+    return y if tl else _tr(y, [*range(nb), *range(nb + nh, nb + nh + nw), *range(nb, nb + nh)])
+
+
 def matmul(a, b):
-    """``numpy.matmul`` for two operands of which at least one carries derivatives."""
-    if _is_triplet(a) and not _is_triplet(b) and len(_shape(b)) == 2:
-        return dot(a, b)
-    if _is_triplet(a) and _is_triplet(b):
+    """``numpy.matmul``: 1-D operands are vectors, leading axes broadcast against each other.
+    Either operand may be a constant of any rank (a matrix, a vector, per-head matrices)."""
+    ta, tb = _is_triplet(a), _is_triplet(b)
+    if not ta and not tb:
+        return np.matmul(a, b)
+    if ta and not tb and np.ndim(b) == 2:
+        return dot(a, b)                          # the plain layer: keeps every fusion of ``dot``
+    if ta and tb:
         return _call('dot_general', (a, b), {})
-    if _is_triplet(b):  # constant @ triplet = (triplet^T @ constant^T)^T
-        bt = swapaxes(b, -1, -2) if len(_shape(b)) > 1 else b
-        out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
-        return swapaxes(out, -1, -2) if len(_shape(out)) > 1 else out
-    return np.matmul(a, b)
+    sa, sb = _shape(a), _shape(b)
+    a_vec, b_vec = len(sa) == 1, len(sb) == 1
+    la, lb_ = list(sa[:-2]) if not a_vec else [], list(sb[:-2]) if not b_vec else []
+    L = max(len(la), len(lb_))
+    # leading axes, right-aligned: both present and equal -> batch; one absent or of size 1 -> free axis of the other
+    a_lead, b_lead, kinds = [], [], []
+    for pos in range(L):
+        ia_, ib_ = pos - (L - len(la)), pos - (L - len(lb_))
+        na = la[ia_] if ia_ >= 0 else None
+        nb = lb_[ib_] if ib_ >= 0 else None
+        if na is not None and nb is not None and na == nb:
+            kinds.append('batch'); a_lead.append(na); b_lead.append(nb)
+        elif nb is None or (nb == 1 and na is not None):
+            kinds.append('a'); a_lead.append(na)
+        elif na is None or na == 1:
+            kinds.append('b'); b_lead.append(nb)
+        else:
+            raise ValueError(f'matmul: shapes {sa} and {sb} do not broadcast')
+    a2 = _rs(a, (*a_lead, *sa[(-1 if a_vec else -2):]))   # size-1 axes that only broadcast are dropped
+    b2 = _rs(b, (*b_lead, *sb[(-1 if b_vec else -2):]))
+    na_, nb_ = len(a_lead), len(b_lead)
+    a_pos = iter(range(na_))
+    b_pos = iter(range(nb_))
+    axes_a, axes_b = {}, {}
+    for pos, kind in enumerate(kinds):
+        if kind in ('batch', 'a'):
+            axes_a[pos] = next(a_pos)
+        if kind in ('batch', 'b'):
+            axes_b[pos] = next(b_pos)
+    batch = [pos for pos, kind in enumerate(kinds) if kind == 'batch']
+    dn = (([len(_shape(a2)) - 1], [nb_ if not b_vec else nb_]),
+          ([axes_a[pos] for pos in batch], [axes_b[pos] for pos in batch]))
+    y = dot_general(a2, b2, dn)
+    # dot_general's order: batch, a's free axes (leads, i), b's free axes (leads, j)
+    order = [('lead', pos) for pos in batch]
+    order += [('lead', pos) for pos, kind in enumerate(kinds) if kind == 'a'] + ([] if a_vec else [('i', 0)])
+    order += [('lead', pos) for pos, kind in enumerate(kinds) if kind == 'b'] + ([] if b_vec else [('j', 0)])
+    want = [('lead', pos) for pos in range(L)] + ([] if a_vec else [('i', 0)]) + ([] if b_vec else [('j', 0)])
+    return _tr(y, [order.index(t) for t in want])
 
 
 def einsum(subscripts: str, a, b):
     """Two-operand ``numpy.einsum`` (explicit ``->`` form, no repeated index inside an operand, no
-    ellipsis) lowered to transposes and one ``matmul``: indices shared by both operands and the
-    output are batch axes, shared ones missing from the output are contracted, the others are
-    the free axes of their operand -- the dimension numbers ``jnp.einsum`` hands to
-    ``dot_general`` (folx/wrapped_functions.py:174-309)."""
+    ellipsis) as one ``dot_general``: indices shared by both operands and the output are batch
+    axes, shared ones missing from the output are contracted, the others are the free axes of
+    their operand -- the dimension numbers ``jnp.einsum`` hands to ``dot_general``
+    (folx/wrapped_functions.py:174-309)."""
     ins, out = subscripts.replace(' ', '').split('->')
     sa, sb = ins.split(',')
     assert len(set(sa)) == len(sa) and len(set(sb)) == len(sb) and '.' not in subscripts, subscripts
     for idx, t in ((sa, a), (sb, b)):  # indices of one operand only that the output drops are summed first
         drop = [i for i, c in enumerate(idx) if c not in out and c not in (sb if idx is sa else sa)]
         if drop:
-            red = sum(t, axis=tuple(drop))
+            red = sum(t, axis=tuple(drop)) if _is_triplet(t) else np.sum(np.asarray(t), axis=tuple(drop))
             kept = ''.join(c for i, c in enumerate(idx) if i not in drop)
             if idx is sa:
                 a, sa = red, kept
@@ -229,15 +335,11 @@ def einsum(subscripts: str, a, b):
     contract = [c for c in sa if c in sb and c not in out]
     fa = [c for c in sa if c not in sb]
     fb = [c for c in sb if c not in sa]
-    dim = {c: n for idx, t in ((sa, a), (sb, b)) for c, n in zip(idx, _shape(t))}
-    size = lambda cs: int(np.prod([dim[c] for c in cs], dtype=np.int64))
-    at = transpose(a, [sa.index(c) for c in batch + fa + contract])
-    bt = transpose(b, [sb.index(c) for c in batch + contract + fb])
-    bshape = [dim[c] for c in batch]
-    y = matmul(reshape(at, (*bshape, size(fa), size(contract))), reshape(bt, (*bshape, size(contract), size(fb))))
-    y = reshape(y, (*bshape, *[dim[c] for c in fa], *[dim[c] for c in fb]))
+    dn = (([sa.index(c) for c in contract], [sb.index(c) for c in contract]),
+          ([sa.index(c) for c in batch], [sb.index(c) for c in batch]))
+    y = dot_general(a, b, dn)
     cur = batch + fa + fb
-    return y if cur == list(out) else transpose(y, [cur.index(c) for c in out])
+    return _tr(y, [cur.index(c) for c in out])
 
 
 def softmax(a, axis=-1):

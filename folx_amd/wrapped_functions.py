@@ -463,6 +463,8 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     is what the reference's general path produces for this case (folx/jvp.py:224-230).
     """
     h, W = args
+    if kwargs.get('batched_const'):
+        return _dot_batched_const(h, W, sparsity_threshold)
     if isinstance(h, LazyConcat):
         return _dot_parts(h, W, kwargs, sparsity_threshold)
     bias = kwargs.get('bias')
@@ -538,6 +540,36 @@ def dot_general(args, kwargs, sparsity_threshold: int = 0):
     if residual is not None:
         out = _LAPLACE_FN_REGISTRY['add']((residual, out), {}, sparsity_threshold)
     return out
+
+
+def _dot_batched_const(h: FwdLaplArray, W, thr: int) -> FwdLaplArray:
+    """``h (Bt, I, Kc) x W (Bt, Kc, J) -> (Bt, I, J)`` per walker, ``W`` a constant with a batch axis
+    (per-head weights): the case of ``_dot_general_one_constant`` in which the constant operand has
+    batch dimensions (folx/wrapped_functions.py:71-171; the front end has brought any dimension
+    numbers to this form).  Linear in ``h``: the product is applied to x, to every Jacobian row
+    and to the Laplacian (:167-169) by one launch of the batched product kernel, which reads the
+    constant once per batch element.  Sparse rows pass through when their mask is constant along
+    the contracted axis, are aligned to the per-position union over it otherwise, and a union
+    wider than the threshold densifies (:113-157)."""
+    dev = h.x.device
+    Wt = so.device_const(W, dev)
+    Bt, I, Kc = h.shape
+    assert tuple(Wt.shape[:2]) == (Bt, Kc), f'dot_general: contracting {tuple(h.shape)} with {tuple(Wt.shape)}'
+    N = Wt.shape[2]
+    J, mask = h.jacobian.data, h.jacobian.x0_idx
+    new_mask = None
+    if mask is not None:
+        mask = np.broadcast_to(mask, (mask.shape[0], Bt, I, Kc))
+        proj, aligned = ia.dot_projection(mask, -1, thr)
+        if proj is None:
+            logging.info('dot_general: union over the contracted axis exceeds the sparsity threshold; densifying')
+            J = h.jacobian.dense_array
+        else:
+            if aligned:
+                J = so.materialize(J, ia.get_index_mask(mask, proj), proj.shape[0])
+            new_mask = np.broadcast_to(proj, (proj.shape[0], Bt, I, N))
+    y, Jy, lapy = K.dot_const(h.x, J, h.laplacian, Wt)
+    return FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
 
 
 def _dot_then_act(h, W, kwargs, thr: int):

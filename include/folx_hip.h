@@ -290,6 +290,10 @@ int folx_hip_norm_dense_static_fwdlap(void* stream, int32_t act, float param, co
  * read as batch (walker, head)) need no copy.  Outputs are contiguous:
  *   y, y_lap [NB0][NB1][I][J]   y_jac [P][NB0][NB1][I][J].
  * Built for Kc <= 128 (FOLX_HIP_ENOTSUP beyond; the caller then multiplies and sums).
+ * b_jac == NULL and b_lap == NULL: b is a constant with batch axes (per-head weight matrices,
+ * a stride of 0 on the axes it does not vary along), the case of _dot_general_one_constant in
+ * which the constant operand has batch dimensions (folx/wrapped_functions.py:71-171, the three
+ * products at :167-169): y = a b, y_jac[p] = a_jac[p] b, y_lap = a_lap b.
  */
 int folx_hip_dot_two_fwdlap(void* stream, const float* a, const float* a_jac, const float* a_lap,
                             const float* b, const float* b_jac, const float* b_lap, float* y,
@@ -420,9 +424,12 @@ int folx_hip_gather_cols(void* stream, const float* data, const int32_t* table, 
 
 /*
  * Scatter-add form of the same re-indexing (the reference's segment_sum fallback,
- * folx/api.py:110-114, folx/jvp.py:170-171): out must be zero-filled by the caller;
- *   out[idx[r][so]][b][so][si] += data[r][b][so][si]   for idx >= 0.
- * idx int32 [k_in][S_outer] with values in [-1, k_out).
+ * folx/api.py:110-114, folx/jvp.py:170-171), accumulating into what out already holds (zeros
+ * for a plain re-indexing, a dense row stack for a sparse Jacobian added to it in place,
+ * folx/api.py:230-236):
+ *   out[idx[r][so]][b][so][si] += data[r][b][so][si]   for 0 <= idx < k_out.
+ * idx int32 [k_in][S_outer].  Every output entry is updated by one thread in row order: no
+ * atomics, identical bits on every run, also when rows of a position share a target.
  */
 int folx_hip_scatter_add_rows(void* stream, const float* data, const int32_t* idx,
                               float* out, int32_t k_in, int32_t k_out, int64_t B,

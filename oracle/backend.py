@@ -520,29 +520,52 @@ def logsumexp(a: OArr, axis=-1, b=None):
     return val, sign(s)
 
 
+def _letters(n, used=''):
+    pool = [c for c in 'abcdefghijklmnopqrstuvwx' if c not in used]
+    return ''.join(pool[:n])
+
+
+def dot_general(lhs, rhs, dimension_numbers):
+    """``jax.lax.dot_general`` on triplets and constants (output axes: batch, lhs free, rhs free),
+    evaluated as one einsum (folx/wrapped_functions.py:71-171 for one constant operand,
+    :174-309 for two operands with derivatives)."""
+    (lc, rc), (lb, rb) = dimension_numbers
+    nl, nr = len(np.shape(lhs) if not _is(lhs) else lhs.shape), len(np.shape(rhs) if not _is(rhs) else rhs.shape)
+    lc, lb = [i % nl for i in lc], [i % nl for i in lb]
+    rc, rb = [i % nr for i in rc], [i % nr for i in rb]
+    sl = list(_letters(nl))
+    sr = list(_letters(nr, used=''.join(sl)))
+    for i, j in zip(lc, rc):
+        sr[j] = sl[i]
+    for i, j in zip(lb, rb):
+        sr[j] = sl[i]
+    out = [sl[i] for i in lb] + [c for i, c in enumerate(sl) if i not in lc and i not in lb] \
+        + [c for j, c in enumerate(sr) if j not in rc and j not in rb]
+    sub = f"{''.join(sl)},{''.join(sr)}->{''.join(out)}"
+    if not _is(lhs) and not _is(rhs):
+        return np.einsum(sub, np.asarray(lhs), np.asarray(rhs))
+    return einsum(sub, lhs, rhs)
+
+
 def matmul(a, b):
-    """numpy.matmul semantics; two triplets go through ``rules.dot_two_rule`` (the dot_last
-    path of the reference, folx/wrapped_functions.py:294-309)."""
-    if _is(a) and not _is(b):
-        return dot(a, b)
-    if _is(a) and _is(b):
-        av, bv = a.ndim == 1, b.ndim == 1
-        if av:
-            a = expand_dims(a, 0)
-        if bv:
-            b = expand_dims(b, 1)
+    """numpy.matmul semantics (1-D operands are vectors, leading axes broadcast); either operand may
+    be a constant of any rank.  Two triplets with equal leading axes go through
+    ``rules.dot_two_rule`` (the dot_last path of the reference, folx/wrapped_functions.py:294-309);
+    everything else is the same contraction written as an einsum."""
+    if _is(a) and _is(b) and a.shape[:-2] == b.shape[:-2] and a.ndim >= 2 and b.ndim >= 2:
         Ja, Jb = _padJ(a, b)
-        lead = np.broadcast_shapes(a.x.shape[:-2], b.x.shape[:-2])
-        bc = lambda t, off: np.broadcast_to(t, (*t.shape[:off], *lead, *t.shape[-2:]))
-        out = OArr(*rules.dot_two_rule(bc(a.x, 0), bc(Ja, 1), bc(a.lap, 0), bc(b.x, 0), bc(Jb, 1), bc(b.lap, 0)))
-        if bv:
-            out = squeeze(out, -1)
-        if av:
-            out = squeeze(out, -1 if bv else -2)
-        return out
-    bt = swapaxes(b, -1, -2) if b.ndim > 1 else b
-    out = dot(bt, np.swapaxes(np.asarray(a), -1, -2) if np.ndim(a) > 1 else np.asarray(a))
-    return swapaxes(out, -1, -2) if out.ndim > 1 else out
+        return OArr(*rules.dot_two_rule(a.x, Ja, a.lap, b.x, Jb, b.lap))
+    sa = tuple(a.shape) if _is(a) else np.shape(a)
+    sb = tuple(b.shape) if _is(b) else np.shape(b)
+    av, bv = len(sa) == 1, len(sb) == 1
+    la, lb = ([] if av else list(sa[:-2])), ([] if bv else list(sb[:-2]))
+    L = max(len(la), len(lb))
+    lead = _letters(L)
+    # numpy's einsum broadcasts axes of size 1 that share a letter with a longer axis, as matmul does
+    sa_ = lead[L - len(la):] + ('' if av else 'y') + 'z'
+    sb_ = lead[L - len(lb):] + 'z' + ('' if bv else 'w')
+    out = lead + ('' if av else 'y') + ('' if bv else 'w')
+    return einsum(f'{sa_},{sb_}->{out}', a, b)
 
 
 def einsum(subscripts, a, b):

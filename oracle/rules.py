@@ -268,6 +268,15 @@ def dense_rule(x, J, lap, W, b=None):
     return y, J @ W, lap @ W
 
 
+def dot_const_rule(a, Ja, La, W):
+    """y = a @ W over the last two axes, ``a (.., Bt, I, Kc)`` with derivatives and ``W (Bt, Kc, J)`` a
+    constant with a batch axis (per-head weights): ``_dot_general_one_constant`` with batch
+    dimensions on the constant (folx/wrapped_functions.py:71-171); the product is linear in ``a``,
+    so it is applied to x, to every Jacobian row and to the Laplacian (:167-169).
+    Pinned by AD Hessian traces of per-head products in tests/test_oracle_rules.py."""
+    return a @ W, Ja @ W, La @ W
+
+
 def dot_two_rule(a, Ja, La, b, Jb, Lb):
     """y = a @ b over the last two axes with BOTH operands carrying derivatives (dense Jacobians
     on the same rows): the product is linear in each operand (JVP both ways,

@@ -175,6 +175,22 @@ class plain:
         return torch.einsum(subscripts, a, b)
 
     @staticmethod
+    def dot_general(lhs, rhs, dimension_numbers):
+        """jax.lax.dot_general: output axes are batch, lhs free, rhs free."""
+        a, b = plain._b(lhs, rhs)
+        (lc, rc), (lb, rb) = dimension_numbers
+        lc, lb = [i % a.ndim for i in lc], [i % a.ndim for i in lb]
+        rc, rb = [i % b.ndim for i in rc], [i % b.ndim for i in rb]
+        lf = [i for i in range(a.ndim) if i not in lc + lb]
+        rf = [i for i in range(b.ndim) if i not in rc + rb]
+        at = a.permute(*lb, *lf, *lc)
+        bt = b.permute(*rb, *rc, *rf)
+        bs = [a.shape[i] for i in lb]
+        y = at.reshape(*bs, int(np.prod([a.shape[i] for i in lf])), -1) @ bt.reshape(
+            *bs, -1, int(np.prod([b.shape[i] for i in rf])))
+        return y.reshape(*bs, *[a.shape[i] for i in lf], *[b.shape[i] for i in rf])
+
+    @staticmethod
     def softmax(a, axis=-1):
         return torch.softmax(a, dim=axis)
 

@@ -74,6 +74,10 @@ def dot_two(a, aj, al, b, bj, bl):
     return tuple(_t(t) for t in rules.dot_two_rule(_n(a), _n(aj), _n(al), _n(b), _n(bj), _n(bl)))
 
 
+def dot_const(a, aj, al, W):
+    return tuple(_t(t) for t in rules.dot_const_rule(_n(a), _n(aj), _n(al), _n(W)))
+
+
 def exp_envelope(d, dj, dl, sigma, pi):
     from oracle import backend as ob
 
@@ -182,8 +186,10 @@ def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
                 acc[ix[r, so], :, so] += d[r, :, so]
     res = _t(acc.reshape(k_out, B, S_outer * S_inner))
     if out is not None:
+        if OUT_DTYPE != np.float32:  # a float64 reference evaluation never writes into its arguments
+            return res.reshape(out.shape)
         out.reshape(k_out, B, S_outer * S_inner).copy_(res)
-        return out if OUT_DTYPE == np.float32 else res.reshape(out.shape)
+        return out
     return res
 
 
@@ -267,7 +273,7 @@ def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
                                                 _n(v), dense(vs), _n(vl)))
 
 
-KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
+KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'dot_const', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
                 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_reduce_rows', 'gather_cols', 'scatter_add_rows',
                 'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
 

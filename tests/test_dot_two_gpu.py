@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from bruteforce import brute_force, plain
+from one_constant_cases import ONE_CONSTANT_FNS
 from oracle import backend as ob
 from oracle import rules
 from tolerances import assert_lap, assert_triplet, assert_val
@@ -50,6 +51,78 @@ def test_dot_two_kernel(NB0, NB1, I, J, Kc, P):
         got = K.dot_two(va(qa(a, 0), 0), va(qa(aj, 1), 1), va(qa(al, 0), 0),
                         vb(qb(b, 0), 0), vb(qb(bj, 1), 1), vb(qb(bl, 0), 0))
         assert_triplet(got, ref, 'dot_two strided views')
+
+
+@pytest.mark.parametrize('B,Bt,I,J,Kc,P', [
+    (1, 1, 1, 1, 1, 1), (3, 4, 5, 7, 3, 4), (2, 4, 32, 64, 64, 12), (2, 1, 70, 45, 20, 3),
+    (2, 2, 33, 31, 100, 5), (4, 3, 8, 8, 16, 0),
+    # contracted axes longer than the kernel's tile depth: slices of the contracted axis, added
+    (2, 2, 9, 11, 130, 3), (1, 2, 16, 20, 300, 2),
+])
+def test_dot_const_kernel(B, Bt, I, J, Kc, P):
+    """Batched product with a constant that has a batch axis (per-head weights) vs the float64 rule;
+    the constant is read once per batch element (walker stride 0)."""
+    from folx_amd import kernels as K
+
+    print(f'case dot_const B={B} Bt={Bt} I={I} J={J} K={Kc} P={P}', flush=True)
+    rng = np.random.default_rng(43)
+    a, aj, al = rand(rng, B, Bt, I, Kc), rand(rng, P, B, Bt, I, Kc), rand(rng, B, Bt, I, Kc)
+    W = rand(rng, Bt, Kc, J)
+    f64 = lambda *t: [np.asarray(v, dtype=np.float64) for v in t]
+    ref = rules.dot_const_rule(*f64(a, aj, al, W))
+    got = K.dot_const(dev(a), dev(aj), dev(al), dev(W))
+    assert_triplet(got, ref, 'dot_const contiguous')
+    if P > 0:  # head-interleaved operand (walker, position, head, feature) viewed as (walker, head, position, feature)
+        q = lambda t, lead: dev(np.moveaxis(t, lead + 1, lead + 2)).transpose(lead + 1, lead + 2)
+        got = K.dot_const(q(a, 0), q(aj, 1), q(al, 0), dev(W))
+        assert_triplet(got, ref, 'dot_const strided views')
+
+
+@pytest.mark.parametrize('name', sorted(ONE_CONSTANT_FNS))
+@pytest.mark.parametrize('sparse', [False, True])
+def test_one_constant_products_in_models(name, sparse):
+    """One operand with derivatives against a constant of any rank on either side, any contracted and
+    batch axes (folx/wrapped_functions.py:71-171; test/test_layers.py:119-139, real half): oracle and
+    brute-force AD, dense (threshold 0) and sparse (threshold = number of inputs)."""
+    fn = ONE_CONSTANT_FNS[name]
+    x = (0.7 * np.random.default_rng(9).normal(size=(3, 4, 3))).astype(np.float32)
+    thr = 12 if sparse else 0
+    print(f'case one-constant {name} thr={thr}', flush=True)
+    out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fn(fnp, t), thr))(x)
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    J = out.jacobian.dense_array
+    assert tuple(out.x.shape) == tuple(ref.x.shape)
+    assert_val(out.x, ref.x, name + ' x')
+    assert_val(J, ref.J[: J.shape[0]], name + ' jacobian')
+    assert J.shape[0] == ref.J.shape[0] or np.abs(ref.J[J.shape[0]:]).max() == 0
+    assert_lap(out.laplacian, ref.lap, name + ' laplacian')
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    assert_val(out.x, by), assert_val(J, bJ[: J.shape[0]]), assert_lap(out.laplacian, bL)
+
+
+def test_per_head_weights_at_model_size():
+    """``einsum('nhd,hde->nhe')`` with per-head weights on a 32-electron, 4-head, 64-feature
+    activation behind a dense layer, 96 dense Jacobian rows: one launch of the batched product
+    with the constant operand, equal to the oracle."""
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(12)
+    W0 = rng.normal(size=(3, 256)).astype(np.float32) / 2
+    Wh = rng.normal(size=(4, 64, 64)).astype(np.float32) / 8
+
+    def fn(xp, x):
+        h = xp.reshape(xp.tanh(xp.dot(x, W0)), (32, 4, 64))
+        return xp.sum(xp.tanh(xp.einsum('nhd,hde->nhe', h, Wh)), axis=0)
+
+    x = (0.7 * rng.normal(size=(2, 32, 3))).astype(np.float32)
+    print('case per-head weights at model size', flush=True)
+    with K.LaunchTimer() as lt:
+        out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fn(fnp, t), 0))(x)
+    assert 'dot_const_fwdlap' in {entry for (entry, _key) in lt.summary()}
+    ref = fn(ob, ob.init_state(x, dtype=np.float64))
+    assert_val(out.x, ref.x, 'per-head x')
+    assert_val(out.jacobian.dense_array, ref.J, 'per-head jacobian')
+    assert_lap(out.laplacian, ref.lap, 'per-head laplacian')
 
 
 _ATT_W = [np.random.default_rng(40 + i).normal(size=(3, 8)).astype(np.float32) / 2 for i in range(3)]

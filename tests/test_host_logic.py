@@ -293,6 +293,37 @@ MATMUL_FNS = {
 _ATT_W = [np.random.default_rng(40 + i).normal(size=(3, 8)).astype(np.float32) / 2 for i in range(3)]
 
 
+from one_constant_cases import ONE_CONSTANT_FNS  # noqa: E402
+
+
+@pytest.mark.parametrize('name', sorted(ONE_CONSTANT_FNS))
+@pytest.mark.parametrize('thr', [0, 12])
+def test_dot_general_with_one_constant_operand(name, thr):
+    """One operand with derivatives against a constant of any rank, on either side, with any
+    contracted and batch axes (``_dot_general_one_constant``, folx/wrapped_functions.py:71-171; the
+    real half of test/test_layers.py:119-139 is 'matmul_vec' / 'vec_matmul' / the 2-D cases of
+    MATMUL_FNS): dense (threshold 0) and sparse (threshold = number of inputs)."""
+    x = np.random.default_rng(9).normal(size=(2, 4, 3)).astype(np.float32)
+    fn = ONE_CONSTANT_FNS[name]
+    got = check_against_oracle(fn, x, thr)
+    by, bJ, bL = brute_force(lambda t: fn(plain, t), x.astype(np.float64))
+    np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[1], bJ[: got[1].shape[0]], rtol=2e-4, atol=2e-5)
+    np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-5)
+
+
+def test_batched_constant_product_keeps_sparse_rows():
+    """Per-position weights applied to a node-wise feature keep one Jacobian row per input
+    coordinate of the node (the mask is constant along the contracted axis only after the union
+    over it: 3 rows), where a dense run has all 12."""
+    x = np.random.default_rng(9).normal(size=(2, 4, 3)).astype(np.float32)
+    out = run_product(ONE_CONSTANT_FNS['einsum_heads'], x, 12)
+    assert out.jacobian.weak and out.jacobian.x0_idx.shape[0] == 3
+    dense = run_product(ONE_CONSTANT_FNS['einsum_heads'], x, 0)
+    assert not dense.jacobian.weak
+    np.testing.assert_allclose(out.jacobian.dense_array.numpy(), dense.jacobian.dense_array.numpy(), rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize('name', sorted(MATMUL_FNS))
 @pytest.mark.parametrize('thr', [0, 12])
 def test_two_operand_matmul(name, thr):

@@ -509,6 +509,40 @@ def test_gather_and_scatter_rows():
     assert_val(got.reshape(k_out, B, So, Si), ref)
 
 
+@pytest.mark.parametrize('collide', [False, True])
+@pytest.mark.parametrize('k_in,B,So,Si,k_out', [(3, 4, 5, 6, 7), (3, 2, 32, 256, 96), (6, 3, 17, 1, 9)])
+def test_scatter_add_rows_into_existing(collide, k_in, B, So, Si, k_out):
+    """``scatter_add_rows(out=existing)``: a sparse Jacobian added in place into a dense row stack that
+    already holds values (the sparse skip connection added into a product's fresh output,
+    folx/api.py:230-249 through the dense branch).  Non-colliding: every (target row, position) is
+    named at most once; colliding: several stored rows of a position name the same target row."""
+    from folx_amd import kernels as K
+
+    rng = np.random.default_rng(70 + k_in + So)
+    if collide:
+        mask = rng.integers(-1, min(k_out, 2), size=(k_in, So))  # targets 0 / 1 only: collisions everywhere
+    else:
+        mask = np.stack([rng.permutation(k_out)[:k_in] for _ in range(So)], axis=1)  # distinct rows per position
+        mask[rng.random(mask.shape) < 0.2] = -1
+    data = rand(rng, k_in, B, So, Si)
+    base = rand(rng, k_out, B, So, Si)
+    ref = base.astype(np.float64) + ia.materialize(data.astype(np.float64),
+                                                   np.broadcast_to(mask[:, :, None], (k_in, So, Si)), k_out)
+    out = dev(base).reshape(k_out, B, So * Si)
+    keep = out.clone()
+    got = K.scatter_add_rows(dev(data).reshape(k_in, B, So * Si), dev(mask, torch.int32), k_out, B, So, Si, out=out)
+    assert got.data_ptr() == out.data_ptr(), 'accumulates in place'
+    assert_val(got.reshape(k_out, B, So, Si), ref)
+    # rows that no entry names keep their bits
+    named = np.zeros((k_out, So), dtype=bool)
+    for r in range(k_in):
+        for so in range(So):
+            if mask[r, so] >= 0:
+                named[mask[r, so], so] = True
+    untouched = torch.as_tensor(~named, device=out.device)[:, None, :, None].expand(k_out, B, So, Si)
+    assert torch.equal(got.reshape(k_out, B, So, Si)[untouched], keep.reshape(k_out, B, So, Si)[untouched])
+
+
 @pytest.mark.parametrize('n,P,lead', [(1, 3, (4,)), (2, 5, (3, 2)), (5, 7, (6,)), (8, 24, (4, 3)),
                                       (16, 96, (5, 4)), (32, 20, (3, 2)), (11, 4, (7,)),
                                       # two matrices per wavefront with an odd count; one matrix; a
