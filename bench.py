@@ -53,6 +53,8 @@ def parse():
                          'three-piece bf16 split on the bf16 matrix pipe')
     ap.add_argument('--no-split-leg', action='store_true',
                     help='skip the short second measurement with --gemm bf16x3 that a default run appends')
+    ap.add_argument('--no-other', action='store_true',
+                    help='skip the short measurements of the other workloads that a default run appends')
     ap.add_argument('--graph', action='store_true',
                     help='replay each chunk as a captured HIP graph (no per-kernel timing, no roofline)')
     ap.add_argument('--calibrate-copy', action='store_true',
@@ -63,7 +65,9 @@ def parse():
 def cpu_baseline(workload, budget_s, gpu_out=None, gpu_out_split=None):
     """The numpy oracle (fp32, dense Jacobians) on a bounded sample of the same workload: the first
     n walkers of the batch the GPU was timed on, whose GPU results (``gpu_out``) are compared with
-    the oracle's in the same run."""
+    the oracle's in the same run.  On the first walkers (at most 8) the oracle also runs in float64:
+    the GPU's distance from that result stands beside the float32 oracle's own distance from it, so
+    that a reader can tell the conditioning of the function from an error of the kernels."""
     from oracle import backend as ob
 
     from folx_amd import workloads as wl
@@ -76,10 +80,10 @@ def cpu_baseline(workload, budget_s, gpu_out=None, gpu_out_split=None):
     except Exception:
         threads = 1
 
-    def run(n):
+    def run(n, dtype=np.float32):
         x = wl.sample_inputs(workload, n, seed=2)  # the first n walkers of the GPU's batch (same seed, row-major draws)
         t0 = time.perf_counter()
-        out = forward(p, ob.init_state(x, dtype=np.float32), ob)
+        out = forward(p, ob.init_state(x, dtype=dtype), ob)
         dt = time.perf_counter() - t0
         assert np.isfinite(out.lap).all()
         return dt, out
@@ -94,28 +98,42 @@ def cpu_baseline(workload, budget_s, gpu_out=None, gpu_out_split=None):
         'value': n / dt,
         'unit': 'walkers/s',
         'cores': threads,
+        'host_cpu_count': os.cpu_count(),
         'kind': 'port',
-        'sample': f'{n} walkers of {workload}, numpy fp32 oracle with dense Jacobians, {dt:.1f} s',
+        'sample': f'{n} walkers of {workload}, numpy fp32 oracle with dense Jacobians, {dt:.1f} s '
+                  f'(BLAS threads {threads} of os.cpu_count() = {os.cpu_count()})',
     }
     if gpu_out is not None:
         # same walkers, GPU path against the CPU oracle: largest difference over the largest reference entry.
         # Both sides are float32; log|det| of the randomly initialised orbital matrices amplifies their
-        # rounding (the oracle's own float32 / float64 difference is 3e-4 on psiformer32), which is what
-        # these figures show -- the parity bars are enforced stage by stage in tests/.
-        rel = lambda g, r: float(np.abs(g[..., :n].astype(np.float64) - r).max() / max(np.abs(r).max(), 1e-30))
+        # rounding, which is what these figures show -- `against_fp64` below separates the two, and the
+        # parity bars are enforced stage by stage in tests/.
+        rel = lambda g, r, m: float(np.abs(g[..., :m].astype(np.float64) - r).max() / max(np.abs(r).max(), 1e-30))
+        parts = lambda o, m: (np.asarray(o.x, dtype=np.float64)[None, :m],
+                              np.asarray(o.J, dtype=np.float64).reshape(o.J.shape[0], -1)[:, :m],
+                              np.asarray(o.lap, dtype=np.float64)[None, :m])
 
-        def against_oracle(triplet):
+        def against(triplet, ref, m):
             gx, gJ, gl = triplet
-            return {
-                'value': rel(gx[None], np.asarray(out.x, dtype=np.float64)[None]),
-                'jacobian': rel(gJ, np.asarray(out.J, dtype=np.float64).reshape(out.J.shape[0], -1)[:, :n]),
-                'laplacian': rel(gl[None], np.asarray(out.lap, dtype=np.float64)[None]),
-                'walkers': n,
-            }
+            rx, rJ, rl = ref
+            return {'value': rel(gx[None], rx, m), 'jacobian': rel(gJ, rJ, m), 'laplacian': rel(gl[None], rl, m),
+                    'walkers': m}
 
-        res['gpu_vs_oracle_max_rel'] = against_oracle(gpu_out)
+        res['gpu_vs_oracle_max_rel'] = against(gpu_out, parts(out, n), n)
         if gpu_out_split is not None:  # the run with the bf16x3 products, same walkers
-            res['bf16x3_vs_oracle_max_rel'] = against_oracle(gpu_out_split)
+            res['bf16x3_vs_oracle_max_rel'] = against(gpu_out_split, parts(out, n), n)
+        m = min(n, 8)
+        _, out64 = run(m, np.float64)
+        ref64 = parts(out64, m)
+        o32 = parts(out, m)
+        res['against_fp64'] = {
+            'what': f'first {m} walkers: max |result - float64 oracle| / max |float64 oracle|; the float32 oracle\'s own '
+                    'distance is the rounding floor of this function in float32',
+            'gpu_vs_fp64': against(gpu_out, ref64, m),
+            'oracle_fp32_vs_fp64': against((o32[0][0], o32[1], o32[2][0]), ref64, m),
+        }
+        if gpu_out_split is not None:
+            res['against_fp64']['bf16x3_vs_fp64'] = against(gpu_out_split, ref64, m)
     return res
 
 
@@ -130,34 +148,86 @@ def describe(cfg):
             f'width {cfg.w1}, two-electron width {cfg.w2}, {cfg.n_det} determinants')
 
 
-def main():
-    args = parse()
-    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
-        print('bench.py measures one GPU: walkers are independent, every GPU would run this same '
-              'path on its share of the batch; run with --gpus 1', file=sys.stderr)
-        sys.exit(2)
+def roofline_of(dname, dkey, dn, dms, gemm):
+    """Roofline record of one entry point and shape: algorithmic flops or bytes of the rule (the per-unit
+    figures of the kernels' own headers) over the average duration of its launches."""
+    avg_s = dms / dn * 1e-3
+    mfma = lambda flops, kernel: {'bound': 'mfma', 'achieved': flops / avg_s / 1e12, 'peak': PEAK_FP32_MFMA_TFLOPS,
+                                  'unit': 'TFLOP/s', 'frac': flops / avg_s / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                                  'traffic': MEASURED_TRAFFIC_BYTES.get((dname, dkey)), 'kernel': kernel,
+                                  'launches': dn, 'avg_launch_ms': dms / dn}
+    hbm = lambda nbytes, kernel: {'bound': 'hbm', 'achieved': nbytes / avg_s / 1e9, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                                  'frac': nbytes / avg_s / 1e9 / PEAK_HBM_GBS, 'traffic': None, 'kernel': kernel,
+                                  'launches': dn, 'avg_launch_ms': dms / dn}
+    if dname == 'dense_fwdlap':
+        R, P, Kd, N, has_res = dkey
+        if N == 1:  # matrix-vector form
+            return hbm(4.0 * (P + 2) * R * (Kd + 1), f'dense_n1 kernels R={R} P={P} K={Kd}')
+        kern = (('dense_split_kernel' if gemm == 'bf16x3' and N > 128 else 'dense_dma_kernel')
+                if Kd % 16 == 0 and N % 4 == 0 else 'dense_kernel')
+        return mfma(2.0 * (P + 2) * R * Kd * N, kern + f' R={R} P={P} K={Kd} N={N} residual={has_res}')
+    if dname == 'mhsa_fwdlap':
+        Bc, n, H, d, P = dkey
+        return mfma((7.0 * P + 6) * 2 * n * n * d * Bc * H, f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}')
+    if dname == 'norm_dense_fwdlap' or (dname == 'dense_act_fwdlap' and dkey[4] > 128):
+        # the wide fused rules: one GEMM over the Jacobian rows (tiles cut across Jacobian rows)
+        # plus short launches for the x / lap rows; the events bracket the whole entry point
+        act, R, P, Kd, N = dkey
+        norm = dname == 'norm_dense_fwdlap'
+        return mfma(2.0 * (P + 2) * R * Kd * N,
+                    f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}, '
+                    f'{"32, false" if norm else "16 | 32, parts"}> + the short launches of its entry point '
+                    f'({dname}: x / lap rows GEMM, finish; with LayerNorm also weight fold and per-position rows), '
+                    f'act={act} R={R} P={P} K={Kd} N={N}')
+    if dname == 'dense_act_fwdlap':
+        act, R, P, Kd, N = dkey
+        r = hbm(4.0 * ((P + 2) * R * (Kd + N) + Kd * N), f'dense_act_kernel {act} R={R} P={P} K={Kd} N={N}')
+        r['mfma_tflops'] = 2.0 * (P + 2) * R * Kd * N / avg_s / 1e12
+        r['mfma_frac'] = r['mfma_tflops'] / PEAK_FP32_MFMA_TFLOPS
+        return r
+    if dname == 'elementwise_fwdlap':
+        name, S, P = dkey
+        return hbm(8.0 * (P + 2) * S, f'elementwise_kernel<{name}> S={S} P={P}')
+    if dname == 'layernorm_fwdlap':
+        R, F, P = dkey
+        return hbm(8.0 * (P + 2) * R * F, f'layernorm_kernel R={R} F={F} P={P}')
+    if dname == 'reduce_sum':
+        rows, outer, red, inner = dkey
+        return hbm(4.0 * rows * outer * (red + 1) * inner, f'reduce kernels rows={rows} outer={outer} red={red} inner={inner}')
+    if dname == 'mhsa_sparse_fwdlap':
+        Bc, n, H, d, k, P = dkey
+        return hbm(4.0 * n * d * (P + 3 * k + 8) * Bc * H, f'mhsa_sparse_kernel B={Bc} n={n} H={H} d={d} k={k} P={P}')
+    if dname in ('slogdet_fwdlap', 'slogdet_scaled_fwdlap'):
+        NM, n, P = dkey[:3]
+        k = dkey[3] if len(dkey) > 3 else -2
+        return hbm(4.0 * NM * n * n * ((P + 2) + (k + 2)), f'slogdet kernels NM={NM} n={n} P={P}')
+    return {'bound': 'hbm', 'achieved': None, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': None,
+            'traffic': None, 'kernel': f'{dname} {dkey}', 'launches': dn, 'avg_launch_ms': dms / dn}
 
+
+def measure(workload, steps, warmup, walkers=0, chunk=1024, gemm='f32', graph=False, calibrate_copy=False):
+    """Times ``steps`` steps of one workload after ``warmup`` untimed ones (inputs resident on the device, host clock
+    around device synchronisations) and finds the entry point with the largest total time, whose launches carry HIP
+    events on the launch stream inside the timed region.  Returns the pieces of the output line."""
     import torch
 
     import folx_amd
     from folx_amd import kernels as K
     from folx_amd import workloads as wl
 
-    K.set_gemm_mode(args.gemm)
-    forward, params_np, cfg, B, sigma, thr = wl.build(args.workload)
-    if args.walkers:
-        B = args.walkers
+    forward, params_np, cfg, B, sigma, thr = wl.build(workload)
+    if walkers:
+        B = walkers
     dev = torch.device('cuda', 0)
-    torch.cuda.set_device(dev)
     params = wl.to_device(params_np, dev)
-    x = torch.as_tensor(wl.sample_inputs(args.workload, B, seed=2)).to(dev)
+    x = torch.as_tensor(wl.sample_inputs(workload, B, seed=2)).to(dev)
     fl = folx_amd.forward_laplacian(lambda r: forward(params, r), thr)
-    step = folx_amd.batched_vmap(folx_amd.jit(folx_amd.vmap(fl)) if args.graph else fl, args.chunk)
+    step = folx_amd.batched_vmap(folx_amd.jit(folx_amd.vmap(fl)) if graph else fl, chunk)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         out = step(x)
     torch.cuda.synchronize()
-    if args.calibrate_copy:
+    if calibrate_copy:
         n = 1 << 28  # 2^28 floats = 1 GiB read + 1 GiB written by rows_affine_kernel
         src = torch.empty(n, device=dev, dtype=torch.float32).fill_(1.0)
         K.rows_affine(src, 1, (n,), (n,), None, None, 1.0, 0.0)
@@ -175,17 +245,49 @@ def main():
     with K.LaunchTimer(only=() if dominant is None else (dominant,)) as lt:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             out = step(x)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
     assert torch.isfinite(out.x).all() and torch.isfinite(out.laplacian).all()
+    summ = lt.summary()
+    roof = None
+    if summ:
+        (dname, dkey), (dn, dms) = max(summ.items(), key=lambda kv: kv[1][1])
+        roof = roofline_of(dname, dkey, dn, dms, gemm)
+        roof['entry_point'] = dname
+        roof['share_of_gpu_time'] = dms / steps / max(sum(ms for (_n, ms) in summ_all.values()), 1e-30)
+    per_kernel = {}
+    for (name, key), (n, ms) in summ_all.items():
+        per_kernel[name] = per_kernel.get(name, 0.0) + ms
+    return {'B': B, 'cfg': cfg, 'thr': thr, 'out': out, 'x': x, 'step': step, 'dt': dt, 'roof': roof,
+            'per_kernel': per_kernel, 'graph_mode': not summ}
+
+
+# the other BASELINE.json configurations, measured briefly after the headline: (steps, warm-up steps, chunk)
+OTHER_WORKLOADS = {'mlp_dense': (20, 5, 1024), 'mlp_sparse': (20, 5, 1024), 'ferminet16': (8, 4, 1024),
+                   'psiformer64': (2, 1, 1024)}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py measures one GPU: walkers are independent, every GPU would run this same '
+              'path on its share of the batch; run with --gpus 1', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from folx_amd import kernels as K
+
+    torch.cuda.set_device(0)
+    K.set_gemm_mode(args.gemm)
+    m = measure(args.workload, args.steps, args.warmup, args.walkers, args.chunk, args.gemm, args.graph,
+                args.calibrate_copy)
+    B, cfg, thr, out, x, step, dt, roof = (m[k] for k in ('B', 'cfg', 'thr', 'out', 'x', 'step', 'dt', 'roof'))
     ms_per_step = 1e3 * dt / args.steps
     value = B * args.steps / dt
-
-    # dominant kernel: the launch shape with the largest total time inside the timed region
-    summ = lt.summary()
-    if not summ:
+    if m['graph_mode']:
         line = {'metric': 'walkers/s of full forward Laplacian at 1 GPU', 'value': value, 'unit': 'walkers/s',
                 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': ms_per_step,
                 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
@@ -194,56 +296,6 @@ def main():
                 'roofline': None}
         print(json.dumps(line))
         return
-    per_kernel = {}
-    for (name, key), (n, ms) in summ_all.items():
-        per_kernel[name] = per_kernel.get(name, 0.0) + ms
-    (dname, dkey), (dn, dms) = max(summ.items(), key=lambda kv: kv[1][1])
-    roof = None
-    traffic = MEASURED_TRAFFIC_BYTES.get((dname, dkey))
-    if dname == 'dense_fwdlap':
-        R, P, Kd, N, has_res = dkey
-        flops = 2.0 * (P + 2) * R * Kd * N
-        achieved = flops / (dms / dn * 1e-3) / 1e12
-        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': (('dense_split_kernel' if args.gemm == 'bf16x3' and N > 128 else 'dense_dma_kernel')
-                           if Kd % 16 == 0 and N % 4 == 0 else 'dense_kernel')
-                + f' R={R} P={P} K={Kd} N={N} residual={has_res}', 'launches': dn,
-                'avg_launch_ms': dms / dn}
-    elif dname == 'mhsa_fwdlap':
-        Bc, n, H, d, P = dkey
-        flops = (7.0 * P + 6) * 2 * n * n * d * Bc * H
-        achieved = flops / (dms / dn * 1e-3) / 1e12
-        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': f'mhsa_kernel B={Bc} n={n} H={H} d={d} P={P}', 'launches': dn,
-                'avg_launch_ms': dms / dn}
-    elif dname == 'norm_dense_fwdlap' or (dname == 'dense_act_fwdlap' and dkey[4] > 128):
-        # the wide fused rules: one GEMM over the Jacobian rows (tiles cut across Jacobian rows)
-        # plus short launches for the x / lap rows; the events bracket the whole entry point
-        act, R, P, Kd, N = dkey
-        flops = 2.0 * (P + 2) * R * Kd * N
-        achieved = flops / (dms / dn * 1e-3) / 1e12
-        norm = dname == 'norm_dense_fwdlap'
-        roof = {'bound': 'mfma', 'achieved': achieved, 'peak': PEAK_FP32_MFMA_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': achieved / PEAK_FP32_MFMA_TFLOPS, 'traffic': traffic,
-                'kernel': f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}, '
-                          f'{"32, false" if norm else "16 | 32, parts"}> + the short launches of its entry point '
-                          f'({dname}: x / lap rows GEMM, finish; with LayerNorm also weight fold and per-position rows), '
-                          f'act={act} R={R} P={P} K={Kd} N={N}',
-                'launches': dn, 'avg_launch_ms': dms / dn}
-    elif dname == 'dense_act_fwdlap':
-        act, R, P, Kd, N = dkey
-        nbytes = 4.0 * ((P + 2) * R * (Kd + N) + Kd * N)
-        achieved = nbytes / (dms / dn * 1e-3) / 1e9
-        roof = {'bound': 'hbm', 'achieved': achieved, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                'frac': achieved / PEAK_HBM_GBS, 'traffic': None,
-                'kernel': f'dense_act_kernel {act} R={R} P={P} K={Kd} N={N}', 'launches': dn,
-                'avg_launch_ms': dms / dn,
-                'mfma_tflops': 2.0 * (P + 2) * R * Kd * N / (dms / dn * 1e-3) / 1e12}
-    else:
-        roof = {'bound': 'hbm', 'achieved': None, 'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': None,
-                'traffic': None, 'kernel': f'{dname} {dkey}', 'launches': dn, 'avg_launch_ms': dms / dn}
 
     line = {
         'metric': 'walkers/s of full forward Laplacian at 1 GPU',
@@ -267,11 +319,12 @@ def main():
         },
         'roofline': roof,
         # from the one untimed step in which every entry point carried events
-        'kernel_ms_per_step': {k: v for k, v in sorted(per_kernel.items(), key=lambda kv: -kv[1])},
+        'kernel_ms_per_step': {k: v for k, v in sorted(m['per_kernel'].items(), key=lambda kv: -kv[1])},
     }
     if roof is not None and roof.get('traffic') is not None:
-        roof['traffic_source'] = ('profiles/psiformer32_forward_laplacian.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this '
-                                  'command in earlier runs (counters cannot be read inside the timed run)')
+        roof['traffic_source'] = ('profiles/psiformer32_forward_laplacian.txt, table "HBM counters": rocprofv3 --pmc FETCH_SIZE / '
+                                  'WRITE_SIZE of this command in earlier runs, summed over the launches of the entry point '
+                                  '(counters cannot be read inside the timed run)')
     if args.gemm == 'bf16x3' and roof is not None and roof['bound'] == 'mfma' and 'mhsa' not in roof['kernel']:
         # six bf16 piece products per fp32 product: the matrix pipe's bf16 peak over six
         roof['peak'] = PEAK_BF16_MFMA_TFLOPS / 6.0
@@ -301,6 +354,26 @@ def main():
             K.set_gemm_mode('f32')
     else:
         out2 = None
+    if not args.no_other and args.gemm == 'f32' and args.workload == 'psiformer32' and not args.walkers:
+        # the other configurations of the benchmark suite, a few steps each: walkers/s, the entry point with
+        # the largest total time and its roofline fraction.  The headline stays the line's `value`.
+        others = {}
+        for name, (k_steps, k_warm, k_chunk) in OTHER_WORKLOADS.items():
+            try:
+                o = measure(name, k_steps, k_warm, 0, k_chunk)
+                r = o['roof'] or {}
+                others[name] = {
+                    'value': o['B'] * k_steps / o['dt'], 'unit': 'walkers/s', 'walkers': o['B'], 'steps': k_steps,
+                    'warmup': k_warm, 'ms_per_step': 1e3 * o['dt'] / k_steps,
+                    'workload': f"{describe(o['cfg'])}, ForwardLaplacianOperator({o['thr']})",
+                    'dominant': {k: r.get(k) for k in ('entry_point', 'kernel', 'bound', 'achieved', 'unit', 'frac',
+                                                       'avg_launch_ms', 'share_of_gpu_time', 'mfma_frac') if k in r},
+                }
+                del o
+            except Exception as e:  # a side measurement must not take the headline line down with it
+                others[name] = {'error': f'{type(e).__name__}: {e}'}
+            torch.cuda.empty_cache()
+        line['other_workloads'] = others
     if not args.no_cpu:
         host = lambda o: (o.x.cpu().numpy(), o.jacobian.dense_array.reshape(-1, B).cpu().numpy(),  # noqa: E731
                           o.laplacian.cpu().numpy())

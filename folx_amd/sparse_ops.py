@@ -252,17 +252,21 @@ def add_sparse_rows_(dense: torch.Tensor, data: torch.Tensor, idx: np.ndarray) -
 _ROWS_CACHE: dict = {}
 
 
-def weight_rows(W: torch.Tensor, ranges: tuple) -> torch.Tensor:
+def weight_rows(W: torch.Tensor, ranges: tuple, cache: bool = False) -> torch.Tensor:
     """Rows ``[lo, hi)`` of a weight matrix for each range, concatenated (a contiguous copy unless one
-    range covers it).  Kept per (tensor object, version, ranges): torch bumps ``_version`` on every
-    in-place update of ``W``, so a changed weight is never served from the cache, and an entry only
-    counts while the tensor it was made from is alive; at most 64 entries are held."""
+    range covers it).  ``cache``: only for a ``W`` that this module made from a numpy constant
+    (``device_const``, never written again): the copy is then kept per (tensor object, ranges).  A
+    tensor the caller owns may be updated in place at any time -- also between the replays of a
+    captured graph, which would go on reading a cached copy -- so its rows are copied on every
+    call, and a capture records that copy."""
     import weakref
 
     if len(ranges) == 1:
         lo, hi = ranges[0]
         return W[lo:hi]  # consecutive rows of a row-major matrix are contiguous
-    key = (id(W), W._version, ranges)
+    if not cache:
+        return torch.cat([W[lo:hi] for lo, hi in ranges], dim=0)
+    key = (id(W), ranges)
     hit = _ROWS_CACHE.get(key)
     if hit is not None and hit[0]() is W:
         return hit[1]

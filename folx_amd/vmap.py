@@ -33,29 +33,59 @@ def _cat(parts):
     raise TypeError(type(first))
 
 
-def batched_vmap(fn, max_batch_size: int):
+def batched_vmap(fn, max_batch_size: int, in_axes=0, out_axes=0):
     """Run ``fn`` over chunks of at most ``max_batch_size`` walkers and concatenate, to
-    bound the size of the Jacobian tensors (folx/vmap.py:45-74: full chunks are taken from
+    bound the size of the Jacobian tensors (folx/vmap.py:11-83: full chunks are taken from
     the END of the batch, the remainder -- the first ``B % max`` walkers -- runs on its
-    own and is placed first)."""
+    own and is placed first).
+
+    ``in_axes`` as in the reference (and ``jax.vmap``): one entry for all positional arguments
+    or one per argument; an int names the walker axis of that argument (moved to the front),
+    ``None`` an argument without a walker axis, which is shown whole to every walker.  Nothing
+    is inferred from shapes: an array that merely has ``B`` leading entries is only cut when its
+    entry of ``in_axes`` says so.  ``out_axes`` must be 0: results keep the walker axis where the
+    data layout has it."""
+    import numpy as np
+
+    if out_axes != 0 and not (isinstance(out_axes, (tuple, list)) and all(a == 0 for a in out_axes)):
+        raise NotImplementedError('batched_vmap: out_axes other than 0')
     batched = vmap(fn)
 
-    def result(x, *args, **kwargs):
-        import numpy as np
+    def result(*args, **kwargs):
+        axes = tuple(in_axes) if isinstance(in_axes, (tuple, list)) else (in_axes,) * len(args)
+        assert len(axes) == len(args), f'batched_vmap: {len(axes)} in_axes for {len(args)} arguments'
+        is_arr = lambda a: isinstance(a, (torch.Tensor, np.ndarray))
+        lead = []
+        for a, ax in zip(args, axes):
+            if ax is None or not is_arr(a):
+                lead.append(a)
+            else:
+                lead.append(a if ax == 0 else (a.movedim(ax, 0) if isinstance(a, torch.Tensor) else np.moveaxis(a, ax, 0)))
+        mapped = [a for a, ax in zip(lead, axes) if ax is not None and is_arr(a)]
+        assert mapped, 'batched_vmap: no argument carries a walker axis'
+        B = mapped[0].shape[0]
+        assert all(a.shape[0] == B for a in mapped), 'batched_vmap: walker axes differ in length'
 
-        B = x.shape[0]
+        def cut(lo, hi):
+            out = []
+            for a, ax in zip(lead, axes):
+                if not is_arr(a):
+                    out.append(a)
+                elif ax is None:   # the same array for every walker of the chunk
+                    out.append(a[None].expand(hi - lo, *a.shape) if isinstance(a, torch.Tensor)
+                               else np.broadcast_to(a[None], (hi - lo, *a.shape)))
+                else:
+                    out.append(a[lo:hi])
+            return out
+
         if B <= max_batch_size:
-            return batched(x, *args, **kwargs)
-        # every further array argument with the same leading walker axis is chunked along with x
-        # (in_axes = 0 of the reference); anything else is passed to every chunk as it is
-        walker = [isinstance(a, (torch.Tensor, np.ndarray)) and a.ndim >= 1 and a.shape[0] == B for a in args]
-        cut = lambda lo, hi: [a[lo:hi] if w else a for a, w in zip(args, walker)]
+            return batched(*cut(0, B), **kwargs)
         rem = B % max_batch_size
         parts = []
         if rem > 0:
-            parts.append(batched(x[:rem], *cut(0, rem), **kwargs))
+            parts.append(batched(*cut(0, rem), **kwargs))
         for s in range(rem, B, max_batch_size):
-            parts.append(batched(x[s : s + max_batch_size], *cut(s, s + max_batch_size), **kwargs))
+            parts.append(batched(*cut(s, s + max_batch_size), **kwargs))
         return _cat(parts)
 
     return result

@@ -962,6 +962,7 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
             and tuple(residual.shape) == (*lead, np.shape(W)[1])):
         res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
     Wt = so.device_const(W, dev)
+    w_const = not isinstance(W, torch.Tensor)  # a numpy constant: its device copy is never written again
     bt = None if bias is None else so.device_const(bias, dev)
     is_b = [isinstance(t, LazyBroadcast) for t in lc.parts]
     wds = [u.shape[-1] for u in srcs]
@@ -974,10 +975,10 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
         # then only contracts the per-position parts -- for a FermiNet layer 320 of 832 features.
         for u, (lo, hi) in [(u, r) for u, r, b_ in zip(srcs, ranges, is_b) if b_]:
             # one product per broadcast part, each adding the sum so far in its epilogue (no concatenation)
-            pre = K.dense(u.x, so.pad_rows(u.jacobian.dense_array, P), u.laplacian, so.weight_rows(Wt, ((lo, hi),)), None,
+            pre = K.dense(u.x, so.pad_rows(u.jacobian.dense_array, P), u.laplacian, so.weight_rows(Wt, ((lo, hi),), cache=w_const), None,
                           pre)
         keep = [i for i, b_ in enumerate(is_b) if not b_]
-        Wt = so.weight_rows(Wt, tuple(ranges[i] for i in keep))
+        Wt = so.weight_rows(Wt, tuple(ranges[i] for i in keep), cache=w_const)
         parts_, srcs_ = [lc.parts[i] for i in keep], [srcs[i] for i in keep]
     else:
         parts_, srcs_ = list(lc.parts), srcs

@@ -28,3 +28,16 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if 'gpu' in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How many compared entries met the pure relative bounds and how many needed the absolute floors."""
+    try:
+        from tolerances import FLOOR_STATS
+    except Exception:
+        return
+    for kind, (total, pure, _) in FLOOR_STATS.items():
+        if total:
+            terminalreporter.write_line(
+                f'parity bars, {kind}s: {total} entries compared, {100.0 * pure / total:.3f} % within the relative bound alone, '
+                f'{total - pure} needed the absolute floor')

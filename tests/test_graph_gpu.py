@@ -63,3 +63,46 @@ def test_jit_weights_in_place_and_invalidate():
         out = jitted(x)
     assert torch.equal(out.laplacian, eager(x).laplacian)
     assert torch.equal(out.jacobian.dense_array, eager(x).jacobian.dense_array)
+
+
+def test_jit_in_place_weight_update_reaches_every_part_of_a_concatenated_layer():
+    """A layer that reads a concatenation part by part contracts its per-position parts with a copy of
+    their rows of ``W`` (two kept row ranges here) and its per-walker part with a view of its rows.  With
+    ``W`` a device tensor the caller updates in place, a replay must read the new rows in every part: the
+    copy is made on every call (and so recorded in the graph), never served from a cache."""
+    from folx_amd import numpy as fnp
+
+    from folx_amd import kernels as K
+
+    g = torch.Generator(device='cuda').manual_seed(4)
+    n = 16                                                           # 48 Jacobian rows: full groups of 16
+    W0 = torch.randn(3, 16, device='cuda', generator=g)
+    Wm = torch.randn(16, 32, device='cuda', generator=g) / 4
+    box = {'W': torch.randn(16 + 16 + 32, 136, device='cuda', generator=g) / 6}
+
+    def fn(r):
+        e = fnp.dot(r, W0)                                           # (n, 16)
+        m = fnp.mean(fnp.tanh(e), axis=0)                            # (16,) per walker
+        h = fnp.tanh(fnp.dot(fnp.add(e, m), Wm))                     # (n, 32)
+        f = fnp.concatenate([e, fnp.broadcast_to(m, (n, 16)), h], axis=-1)
+        return fnp.sum(fnp.tanh(fnp.dot(f, box['W'])))
+
+    eager = folx_amd.vmap(folx_amd.forward_laplacian(fn, 0))
+    jitted = folx_amd.jit(eager)
+    x = torch.randn(5, n, 3, device='cuda', generator=g)
+    print('case jit concat layer, in-place weight update', flush=True)
+    with K.LaunchTimer() as lt:
+        eager(x)
+    # the fused layer contracts the 16 + 32 per-position features only: its copy of two row ranges of W is in use
+    assert any(entry == 'dense_act_fwdlap' and key[3] == 48 for (entry, key) in lt.summary()), lt.summary()
+    for _ in range(3):
+        out = jitted(x)
+    assert torch.equal(out.laplacian, eager(x).laplacian)
+    before = out.laplacian.clone()
+    box['W'].mul_(1.5)                                               # same address, new values
+    for _ in range(2):
+        out = jitted(x)
+        ref = eager(x)
+        assert torch.equal(out.laplacian, ref.laplacian)
+        assert torch.equal(out.jacobian.dense_array, ref.jacobian.dense_array)
+    assert not torch.equal(out.laplacian, before)

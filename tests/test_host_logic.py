@@ -188,6 +188,32 @@ def test_batched_vmap_chunks():
         np.testing.assert_allclose(part.jacobian.data.numpy(), full.jacobian.data.numpy())
 
 
+def test_batched_vmap_in_axes():
+    """An argument is cut into chunks only when ``in_axes`` says it has a walker axis (folx/vmap.py:11-30):
+    an array with B leading entries under ``None`` is shown whole to every walker, whatever the chunk size;
+    an int other than 0 names the walker axis."""
+    rng = np.random.default_rng(8)
+    B = 5
+    x = rng.normal(size=(B, 4)).astype(np.float32)
+    c = rng.normal(size=(B, 4)).astype(np.float32)      # a second input that happens to have B rows, no walker axis
+    f = lambda u, v: fnp.sum(fnp.multiply(fnp.tanh(u), fnp.sum(fnp.sin(v), axis=0)))
+    fl = folx_amd.forward_laplacian(f, 0)
+    full = folx_amd.batched_vmap(fl, 100, in_axes=(0, None))(x, c)
+    ref = folx_amd.vmap(fl)(x, np.broadcast_to(c[None], (B, B, 4)))
+    np.testing.assert_allclose(full.laplacian.numpy(), ref.laplacian.numpy(), rtol=1e-6)
+    for mb in (2, 3):
+        part = folx_amd.batched_vmap(fl, mb, in_axes=(0, None))(x, c)
+        np.testing.assert_allclose(part.x.numpy(), full.x.numpy(), rtol=1e-6)
+        np.testing.assert_allclose(part.laplacian.numpy(), full.laplacian.numpy(), rtol=1e-6)
+        np.testing.assert_allclose(part.jacobian.dense_array.numpy(), full.jacobian.dense_array.numpy(), rtol=1e-6)
+    g = folx_amd.forward_laplacian(lambda u: fnp.sum(fnp.tanh(u)), 0)
+    a = folx_amd.batched_vmap(g, 2, in_axes=1)(np.ascontiguousarray(x.T))
+    b = folx_amd.vmap(g)(x)
+    np.testing.assert_allclose(a.laplacian.numpy(), b.laplacian.numpy(), rtol=1e-6)
+    with pytest.raises(NotImplementedError):
+        folx_amd.batched_vmap(g, 2, out_axes=1)
+
+
 def test_register_function_plugs_in():
     calls = []
 

@@ -149,6 +149,43 @@ def test_psiformer_full_architecture_two_walkers(name):
         assert err <= max(2.0 * floor, 1e-5 * scale), (nm, err, floor)
 
 
+PER_WALKER_C = 4.0  # head-room over a walker's own float32 floor (two float32 evaluations differ by their summation order)
+
+
+def test_psiformer32_thirty_two_walkers_each_within_its_own_float32_floor():
+    """The headline configuration at full width on the first 32 walkers of the benchmark batch, walker by walker.
+    log|det| of a walker's random 16 x 16 orbital matrices amplifies float32 rounding by that walker's
+    condition number, so each walker has its own floor: the distance of the numpy oracle run in float32 from
+    its float64 run.  The HIP result of EVERY walker must be within PER_WALKER_C = 4 x that walker's floor (or
+    within the strict bars where the floor is below them), so the worst-conditioned walkers of the batch are
+    compared too, not only a well-conditioned pair."""
+    forward, p, cfg, _, sigma, thr = wl.build('psiformer32')
+    n = 32
+    x = wl.sample_inputs('psiformer32', n, seed=2)   # the first walkers of the batch bench.py times
+    fn = lambda xp, t: forward(p, t, xp)
+    print('case psiformer32, 32 walkers, per-walker bar', flush=True)
+    out = run(fn, x, thr)
+    r64 = fn(ob, ob.init_state(x, dtype=np.float64))
+    r32 = fn(ob, ob.init_state(x, dtype=np.float32))
+    got = (out.x.cpu().numpy().astype(np.float64)[None], out.jacobian.dense_array.cpu().numpy().astype(np.float64),
+           out.laplacian.cpu().numpy().astype(np.float64)[None])
+    worst = {}
+    for g, a64, a32, nm, strict in zip(got, (r64.x[None], r64.J, r64.lap[None]), (r32.x[None], r32.J, r32.lap[None]),
+                                       ('x', 'jacobian', 'laplacian'), (1e-5, 1e-5, 1e-4)):
+        a32 = np.asarray(a32, dtype=np.float64)
+        assert g.shape == a64.shape == (a64.shape[0], n)
+        scale = np.abs(a64).max(axis=0)                       # per walker
+        err = np.abs(g - a64).max(axis=0) / scale
+        floor = np.abs(a32 - a64).max(axis=0) / scale
+        ratio = err / np.maximum(PER_WALKER_C * floor, strict)
+        w = int(np.argmax(ratio))
+        worst[nm] = float(ratio[w])
+        print(f'psiformer32 {nm}: worst walker {w}: |hip - fp64| = {err[w]:.2e}, its float32 floor {floor[w]:.2e}; '
+              f'largest floor of the 32 walkers {floor.max():.2e}, median {np.median(floor):.2e}; '
+              f'median |hip - fp64| / floor = {np.median(err / np.maximum(floor, 1e-12)):.2f}', flush=True)
+        assert (ratio <= 1.0).all(), (nm, w, err[w], floor[w])
+
+
 def test_psiformer32_full_batch_properties():
     """At the full benchmark size (4096 walkers): walkers are independent, so any walker
     evaluated inside the big batch equals the same walker evaluated in a batch of 4; the
