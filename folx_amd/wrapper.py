@@ -58,6 +58,36 @@ def _dense_rows(t: FwdLaplArray, P: int) -> torch.Tensor:
     return J
 
 
+class _HookJacobian:
+    """What a ``custom_jac_hessian_jac`` hook sees of one argument's Jacobian: dense rows ``data (P, ...)``."""
+
+    __slots__ = ('data', 'x0_idx')
+
+    def __init__(self, data):
+        self.data, self.x0_idx = data, None
+
+    @property
+    def weak(self):
+        return False
+
+    @property
+    def dense_array(self):
+        return self.data
+
+
+class _HookArgs:
+    """Per-position view of the derivative-carrying arguments handed to a ``custom_jac_hessian_jac`` hook
+    (the fields of folx/api.py:348-409 that such hooks read)."""
+
+    def __init__(self, xs, Js, laps):
+        self.x = tuple(xs)
+        self.jacobian = tuple(_HookJacobian(j) for j in Js)
+        self.laplacian = tuple(laps)
+
+    def __len__(self):
+        return len(self.x)
+
+
 def _tree_map(f, tree, *rest):
     if isinstance(tree, (tuple, list)):
         return type(tree)(_tree_map(f, t, *[r[i] for r in rest]) for i, t in enumerate(tree))
@@ -80,14 +110,23 @@ def wrap_forward_laplacian(
     ``flags``: ``LINEAR`` skips the second-order term, as in the reference; the other flags
     choose cheaper forms of the same term there and change nothing here.  ``in_axes`` and
     ``index_static_args`` (which axes / arguments the reference may leave out of the Hessian) do
-    not change the result and are accepted for compatibility.  ``custom_jac_hessian_jac`` is the
-    reference's hook for a hand-written second-order term; a hand-written rule registered with
-    ``register_function`` takes its place here, so anything but ``None`` raises."""
-    if custom_jac_hessian_jac is not None:
-        raise NotImplementedError(
-            'custom_jac_hessian_jac: write the whole rule by hand and register it with register_function'
-        )
-    linear = (flags & FunctionFlags.LINEAR) == FunctionFlags.LINEAR
+    not change the result and are accepted for compatibility -- except that ``in_axes`` decides what
+    the hook below sees.
+
+    ``custom_jac_hessian_jac(args, extra_args, merge, materialize_idx)`` is the reference's hook for
+    a hand-written second-order term ``tr(J^T H_f J)`` (folx/api.py:434-441, called at
+    folx/hessian.py:516-517): when given, the automatic ``t^T H_f t`` is not formed and the hook's
+    result is added to ``J_f lap`` instead.  It is called as in the reference, once per position
+    that ``in_axes`` maps over: ``in_axes=None`` shows it whole per-walker arrays, ``in_axes=()`` one
+    element at a time, an int or tuple of axes the slices along those axes.  ``args`` has ``.x``,
+    ``.jacobian`` (objects with ``.data`` of shape ``(P, ...)`` and ``.x0_idx = None``: the Jacobians
+    are dense here) and ``.laplacian``, one entry per argument that carries derivatives;
+    ``extra_args`` are the other arguments, ``merge(xs, extra_args)`` puts both back in call
+    order; ``materialize_idx`` is always ``None`` (dense rows).  The result is a tensor, or a tree
+    of tensors, with as many entries as the function's output has at those positions."""
+    linear = (flags & FunctionFlags.LINEAR) == FunctionFlags.LINEAR or custom_jac_hessian_jac is not None
+    if isinstance(in_axes, int):
+        in_axes = (in_axes,)
     label = name or getattr(fn, '__name__', 'wrapped')
 
     def new_fn(args: tuple, kwargs: dict[str, Any], sparsity_threshold: int):
@@ -127,13 +166,63 @@ def wrap_forward_laplacian(
         Js = tuple(_dense_rows(t, P).transpose(0, 1) for t in ts)     # (B, P, *shape)
         laps = tuple(t.laplacian for t in ts)
 
+        extra_pos = [i for i in range(len(args)) if i not in lapl_pos]
+
+        def hook_term(xw, Jw, lw, bw, y):
+            """the caller's tr(J^T H_f J), evaluated position by position as ``in_axes`` says"""
+            extra = tuple(bw[bat_pos.index(i)] if i in bat_pos else consts[i] for i in extra_pos)
+
+            def merge(xs, ex):
+                full = [None] * len(args)
+                for i, v in zip(lapl_pos, xs):
+                    full[i] = v
+                for i, v in zip(extra_pos, ex):
+                    full[i] = v
+                return tuple(full)
+
+            def at_position(xs, Js, ls):
+                res = custom_jac_hessian_jac(_HookArgs(xs, Js, ls), extra, merge, None)
+                leaves = []
+                _tree_map(lambda t: leaves.append(torch.as_tensor(t).reshape(-1)), res)
+                return torch.cat(leaves) if len(leaves) != 1 else leaves[0]
+
+            Js = tuple(Jw)   # (P, *shape) per walker
+            if in_axes is None:
+                flat = at_position(xw, Js, lw)
+            else:
+                # positions = the axes NOT named by in_axes, the same for every argument; the hook is mapped over them
+                nd = xw[0].dim()
+                keep = sorted(a % nd for a in in_axes) if nd else []
+                other = [a for a in range(nd) if a not in keep]
+                mv = lambda t, lead: t.permute(*range(lead), *[lead + a for a in other], *[lead + a for a in keep]).reshape(
+                    *t.shape[:lead], -1, *[t.shape[lead + a] for a in keep])
+                xs_ = tuple(mv(t, 0) for t in xw)
+                Js_ = tuple(mv(t, 1) for t in Js)
+                ls_ = tuple(mv(t, 0) for t in lw)
+                flat = vmap(at_position, in_dims=(0, 1, 0))(xs_, Js_, ls_).reshape(-1)
+            leaves = []
+            _tree_map(lambda t: leaves.append(t), y)
+            total = sum(t.numel() for t in leaves)
+            if flat.numel() == 1 and total != 1:       # one number for every output entry (e.g. a term that is zero)
+                flat = flat.expand(total)
+            assert flat.numel() == total, (f'custom_jac_hessian_jac returned {flat.numel()} values for an output of '
+                                           f'{total} entries')
+            outs, off = [], 0
+            for t in leaves:
+                outs.append(flat[off:off + t.numel()].reshape(t.shape))
+                off += t.numel()
+            it = iter(outs)
+            return _tree_map(lambda t: next(it), y)
+
         def per_walker(xw, Jw, lw, bw):
             g = lambda *z: call(z, bw)  # noqa: E731
             first = lambda tv: jvp(g, xw, tv)[1]  # noqa: E731   J_f t
             y = g(*xw)
             Jy = vmap(first)(Jw)
             lap = first(lw)
-            if not linear:
+            if custom_jac_hessian_jac is not None:
+                lap = _tree_map(lambda l, q: l + q, lap, hook_term(xw, Jw, lw, bw, y))
+            elif not linear:
                 second = lambda tv: jvp(lambda *z: jvp(g, z, tv)[1], xw, tv)[1]  # noqa: E731   t^T H_f t
                 quad = vmap(second)(Jw)
                 lap = _tree_map(lambda l, q: l + q.sum(0), lap, quad)

@@ -842,6 +842,62 @@ def test_generic_rule_built_from_a_torch_function(thr):
     np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize('thr', [0, 16])
+def test_custom_jac_hessian_jac_hook(thr):
+    """folx/wrapper.py:73-138 with ``custom_jac_hessian_jac`` (folx/api.py:434-441): the hook's result replaces
+    the automatic tr(J^T H J).  (i) test/test_layers.py:501-529: an identity whose hook returns 10 gives
+    Laplacian 10, value and Jacobian untouched.  (ii) hand-written second-order terms that ARE the Hessian
+    trace -- elementwise (``in_axes=()``: one element and its Jacobian column per call), along the last axis
+    (``in_axes=-1``: rows), and the division rule's own form with two arguments (folx/custom_hessian.py:35-59)
+    -- give what autodiff gives."""
+    rng = np.random.default_rng(45)
+    x = rng.normal(size=(2, 16)).astype(np.float32)
+
+    ten = folx_amd.wrap_forward_laplacian(
+        lambda a: 1.0 * a, custom_jac_hessian_jac=lambda args, extra, merge, idx: tuple(torch.full_like(t, 10.0) for t in args.x))
+    folx_amd.register_function('identity', ten)
+    try:
+        out = folx_amd.vmap(folx_amd.forward_laplacian(lambda r: fnp.call('identity', r), thr))(x)
+    finally:
+        folx_amd.deregister_function('identity')
+    np.testing.assert_allclose(out.x.numpy(), x)
+    np.testing.assert_allclose(out.jacobian.dense_array.numpy(), np.eye(16)[:, None, :].repeat(2, 1), atol=1e-7)
+    np.testing.assert_allclose(out.laplacian.numpy(), 10.0)
+
+    y = rng.normal(size=(3, 4, 5)).astype(np.float32)
+
+    def cube_hook(args, extra, merge, idx):       # f = a^3 elementwise: f'' = 6 a, tr = 6 a sum_p J_p^2
+        (a,), (J,) = args.x, args.jacobian
+        assert a.shape == () and J.data.dim() == 1
+        return 6.0 * a * (J.data * J.data).sum()
+
+    def sumsq_hook(args, extra, merge, idx):      # f = sum_k a_k^2 over the last axis: H = 2 I
+        (a,), (J,) = args.x, args.jacobian
+        assert a.dim() == 1 and J.data.dim() == 2
+        return 2.0 * (J.data * J.data).sum()
+
+    def div_hook(args, extra, merge, idx):        # f = a / b (folx/custom_hessian.py:35-59)
+        a, b = merge(args.x, extra)
+        Ja, Jb = (j.data for j in args.jacobian)
+        return -2.0 / b**2 * (Ja * Jb).sum() + 2.0 * a / b**3 * (Jb * Jb).sum()
+
+    cases = [
+        (folx_amd.wrap_forward_laplacian(lambda a: a**3, in_axes=(), custom_jac_hessian_jac=cube_hook),
+         lambda r, rule: fnp.sum(rule((fnp.sin(r),), {}, thr)), lambda t: (torch.sin(t) ** 3).sum()),
+        (folx_amd.wrap_forward_laplacian(lambda a: (a * a).sum(-1), in_axes=-1, custom_jac_hessian_jac=sumsq_hook),
+         lambda r, rule: fnp.sum(fnp.tanh(rule((fnp.sin(r),), {}, thr))), lambda t: torch.tanh((torch.sin(t) ** 2).sum(-1)).sum()),
+        (folx_amd.wrap_forward_laplacian(lambda a, b: a / b, in_axes=(), custom_jac_hessian_jac=div_hook),
+         lambda r, rule: fnp.sum(rule((fnp.sin(r), fnp.add(fnp.square(r), 1.0)), {}, thr)),
+         lambda t: (torch.sin(t) / (t * t + 1.0)).sum()),
+    ]
+    for rule, model, whole in cases:
+        got = triplet_np(folx_amd.vmap(folx_amd.forward_laplacian(lambda r: model(r, rule), thr))(y))
+        by, bJ, bL = brute_force(whole, y.astype(np.float64))
+        np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
+        np.testing.assert_allclose(got[1], bJ.reshape(got[1].shape), rtol=2e-4, atol=2e-5)
+        np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
+
+
 def test_rules_that_carry_no_derivatives_or_act_elementwise():
     """folx/wrapper.py:141-176."""
     from folx_amd.api import BatchedArray

@@ -39,3 +39,33 @@ def test_wrapped_torch_function_between_rules(thr):
     assert_val(out.x, by, 'value')
     assert_val(J, bJ.reshape(tuple(J.shape)), 'jacobian')
     assert_lap(out.laplacian, bL, 'laplacian')
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_custom_jac_hessian_jac_hook_on_the_gpu(thr):
+    """``wrap_forward_laplacian(..., custom_jac_hessian_jac=hook)`` (folx/wrapper.py:73-138, folx/api.py:434-441):
+    the division rule's hand-written second-order term (folx/custom_hessian.py:35-59), element by element
+    (``in_axes=()``), between hand-written rules; and the reference's own test of the hook
+    (test/test_layers.py:501-529): a constant 10 becomes the Laplacian of an identity."""
+    rng = np.random.default_rng(47)
+    x = rng.normal(size=(5, 4, 3)).astype(np.float32)
+
+    def div_hook(args, extra, merge, idx):
+        a, b = merge(args.x, extra)
+        Ja, Jb = (j.data for j in args.jacobian)
+        return -2.0 / b**2 * (Ja * Jb).sum() + 2.0 * a / b**3 * (Jb * Jb).sum()
+
+    rule = folx_amd.wrap_forward_laplacian(lambda a, b: a / b, in_axes=(), custom_jac_hessian_jac=div_hook)
+    model = lambda r: fnp.sum(fnp.tanh(rule((fnp.sin(r), fnp.add(fnp.square(r), 1.0)), {}, thr)))
+    out = folx_amd.vmap(folx_amd.forward_laplacian(model, thr))(torch.as_tensor(x).cuda())
+    by, bJ, bL = brute_force(lambda t: torch.tanh(torch.sin(t) / (t * t + 1.0)).sum(), x.astype(np.float64))
+    J = out.jacobian.dense_array
+    assert_val(out.x, by, 'value')
+    assert_val(J, bJ.reshape(tuple(J.shape)), 'jacobian')
+    assert_lap(out.laplacian, bL, 'laplacian')
+
+    ten = folx_amd.wrap_forward_laplacian(
+        lambda a: 1.0 * a, custom_jac_hessian_jac=lambda args, extra, merge, idx: tuple(torch.full_like(t, 10.0) for t in args.x))
+    out = folx_amd.vmap(folx_amd.forward_laplacian(lambda r: ten((r,), {}, thr), thr))(torch.as_tensor(x).cuda())
+    assert_val(out.x, x, 'identity value')
+    assert torch.equal(out.laplacian, torch.full_like(out.laplacian, 10.0))
