@@ -54,6 +54,8 @@ SIGNATURES = {
     'folx_hip_slogdet_scaled_fwdlap': (c_int, [_P] * 12 + [c_int64, c_int64, c_int32, c_int32] + [c_int64] * 5 + [c_int32]),
     'folx_hip_sparse_slogdet_fwdlap': (c_int, [_P] * 11 + [c_int64] + [c_int32] * 6),
     'folx_hip_inv_fwdlap': (c_int, [_P] * 7 + [c_int64, c_int32, c_int32]),
+    'folx_hip_inv_values': (c_int, [_P] * 5 + [c_int64, c_int32]),
+    'folx_hip_trace_pair': (c_int, [_P] * 4 + [c_int64, c_int32]),
     'folx_hip_solve_fwdlap': (c_int, [_P] * 10 + [c_int64, c_int32, c_int32, c_int32]),
     'folx_hip_mhsa_fwdlap': (c_int, [_P] * 15 + [c_int64, c_int32, c_int32, c_int32, c_int32]),
     'folx_hip_mhsa_sparse_fwdlap': (c_int, [_P] * 14 + [c_int64, c_int32, c_int32, c_int32, c_int32]),

@@ -33,6 +33,7 @@ SOURCES = [
     'mhsa_sparse.hip',
     'layernorm.hip',
     'linsolve.hip',
+    'anysize.hip',
 ]
 
 # Packed FP32 instructions are switched off for all device code (-packed-fp32-ops).

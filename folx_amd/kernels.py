@@ -339,16 +339,19 @@ def dot_two(a, aj, al, b, bj, bl):
 
 
 def dot_const(a, aj, al, W):
-    """Batched product of a triplet with a constant that has a batch axis: a (B, Bt, I, Kc), aj (P, B, Bt, I, Kc),
-    al like a, W (Bt, Kc, J) float32 on the GPU -> contiguous y (B, Bt, I, J), y_jac (P, B, Bt, I, J), y_lap.  The
-    operands may be views; W is read once per batch element (walker stride 0).  Contracted lengths beyond the
-    kernel's tile depth are cut into slices of the contracted axis (views) whose products are added."""
+    """Batched product of a triplet with an operand that carries no derivatives: a (B, Bt, I, Kc), aj (P, B, Bt, I, Kc),
+    al like a; W (Bt, Kc, J) -- a constant with a batch axis, read once per batch element (walker stride 0) -- or
+    W (B, Bt, Kc, J), one matrix per walker and batch element.  float32 on the GPU; all operands may be views.
+    Returns contiguous y (B, Bt, I, J), y_jac (P, B, Bt, I, J), y_lap.  Contracted lengths beyond the kernel's tile
+    depth are cut into slices of the contracted axis (views) whose products are added."""
     for t in (a, aj, al, W):
         assert t.is_cuda and t.dtype == torch.float32
     B, Bt, I, Kc = a.shape
     J = W.shape[-1]
     P = aj.shape[0]
-    assert tuple(W.shape) == (Bt, Kc, J) and tuple(aj.shape) == (P, *a.shape) and al.shape == a.shape
+    if W.dim() == 3:
+        W = W.unsqueeze(0).expand(B, *W.shape)   # stride 0 along the walkers
+    assert tuple(W.shape) == (B, Bt, Kc, J) and tuple(aj.shape) == (P, *a.shape) and al.shape == a.shape
 
     def same_layout(t, u_strides):
         return all(st == su for st, su, n in zip(t.stride(), u_strides, t.shape) if n > 1)
@@ -358,12 +361,11 @@ def dot_const(a, aj, al, W):
     out = None
     for k0 in range(0, max(Kc, 1), DOT_TWO_KMAX):
         k1 = min(Kc, k0 + DOT_TWO_KMAX)
-        ac, ajc, alc, Wc = a[..., k0:k1], aj[..., k0:k1], al[..., k0:k1], W[:, k0:k1, :]
+        ac, ajc, alc, Wc = a[..., k0:k1], aj[..., k0:k1], al[..., k0:k1], W[:, :, k0:k1, :]
         y = torch.empty((B, Bt, I, J), device=a.device, dtype=torch.float32)
         yj = torch.empty((P, B, Bt, I, J), device=a.device, dtype=torch.float32)
         yl = torch.empty_like(y)
-        strides = (ctypes.c_int64 * 10)(*ac.stride(), ajc.stride(0) if P else 0, 0, Wc.stride(0), Wc.stride(1),
-                                        Wc.stride(2), 0)
+        strides = (ctypes.c_int64 * 10)(*ac.stride(), ajc.stride(0) if P else 0, *Wc.stride(), 0)
         with _timed('dot_const_fwdlap', (B * Bt, I, J, k1 - k0, P)):
             check(
                 _lib.load().folx_hip_dot_two_fwdlap(
@@ -372,13 +374,95 @@ def dot_const(a, aj, al, W):
                 ),
                 'dot_two_fwdlap (constant operand)',
             )
-        if out is None:
-            out = (y, yj, yl)
-        else:
-            add = lambda o, n: o if o.numel() == 0 else rows_affine(o, 1, (o.numel(),), (o.numel(),), None,
-                                                                    n.reshape(-1), 1.0, 1.0).reshape(o.shape)
-            out = tuple(add(o, n) for o, n in zip(out, (y, yj, yl)))
+        out = (y, yj, yl) if out is None else tuple(_add_flat(o, n) for o, n in zip(out, (y, yj, yl)))
     return out
+
+
+def _add_flat(a, b, alpha=1.0, beta=1.0):
+    """alpha a + beta b for two equally shaped contiguous tensors (one flat affine launch)."""
+    n = a.numel()
+    if n == 0:
+        return a
+    return rows_affine(a.reshape(n), 1, (n,), (n,), None, b.reshape(n), alpha, beta).reshape(a.shape)
+
+
+def inv_values(A):
+    """A (NM, n, n) contiguous -> A^-1 (NM, n, n), sign (NM,), log|det| (NM,): Gauss-Jordan with partial pivoting,
+    any n."""
+    _chk(A)
+    NM, n, _ = A.shape
+    Ainv = torch.empty_like(A)
+    sign = torch.empty(NM, device=A.device, dtype=torch.float32)
+    ld = torch.empty_like(sign)
+    with _timed('inv_values', (NM, n)):
+        check(_lib.load().folx_hip_inv_values(_stream(), _p(A), _p(Ainv), _p(sign), _p(ld), NM, n), 'inv_values')
+    return Ainv, sign, ld
+
+
+def trace_pair(M):
+    """M (R, n, n) contiguous -> tr M (R,), tr(M M) (R,)."""
+    _chk(M)
+    R, n, _ = M.shape
+    tr = torch.empty(R, device=M.device, dtype=torch.float32)
+    trsq = torch.empty_like(tr)
+    with _timed('trace_pair', (R, n)):
+        check(_lib.load().folx_hip_trace_pair(_stream(), _p(M), _p(tr), _p(trsq), R, n), 'trace_pair')
+    return tr, trsq
+
+
+def _inverse_times_rows(A, AJ, AL):
+    """A^-1 and, TRANSPOSED, M_c = A^-1 dA_c and L = A^-1 lap_A for matrices of any size: the batched product
+    (dA_c)^T A^-T with the derivative-carrying operand on the left, both read as transposed views.
+    A (NM, n, n), AJ (P, NM, n, n), AL (NM, n, n) contiguous -> Ainv, sign, logdet, Mt (P, NM, n, n), Lt (NM, n, n)."""
+    Ainv, sign, ld = inv_values(A)
+    t = lambda v: v.unsqueeze(-3).transpose(-1, -2)     # (.., NM, 1, n, n), matrices transposed
+    _, Mt, Lt = dot_const(t(A), t(AJ), t(AL), t(Ainv))
+    return Ainv, sign, ld, Mt.squeeze(-3), Lt.squeeze(-3)
+
+
+def slogdet_any(A, AJ, AL):
+    """The slogdet rule for matrices of any size, composed (folx/slogdet.py:296-317): A (.., n, n), AJ (P, .., n, n),
+    AL like A -> sign (..), logdet (..), jac (P, ..), lap (..).  jac_c = tr M_c and
+    lap = tr(A^-1 lap_A) - sum_c tr(M_c M_c) with M_c = A^-1 dA_c from the batched product kernel."""
+    _chk(A, AJ, AL)
+    n, P, lead = A.shape[-1], AJ.shape[0], tuple(A.shape[:-2])
+    NM = int(np.prod(lead, dtype=np.int64))
+    _, sign, ld, Mt, Lt = _inverse_times_rows(A.contiguous().reshape(NM, n, n), AJ.contiguous().reshape(P, NM, n, n),
+                                              AL.contiguous().reshape(NM, n, n))
+    trl, _ = trace_pair(Lt)
+    if P > 0:
+        trj, sqj = trace_pair(Mt.reshape(P * NM, n, n))
+        lap = _add_flat(trl, reduce_sum(sqj, 1, 1, P, NM).reshape(NM), 1.0, -1.0)
+    else:
+        trj, lap = torch.empty(0, device=A.device, dtype=torch.float32), trl
+    return sign.reshape(lead), ld.reshape(lead), trj.reshape(P, *lead), lap.reshape(lead)
+
+
+def inv_any(A, AJ, AL):
+    """The inverse rule for matrices of any size, composed (folx/linear_solve.py:114-145): C = A^-1,
+    C_jac[c] = -M_c C, C_lap = (2 sum_c M_c M_c - C lap_A) C with M_c = C dA_c.  Same shapes as ``inv``."""
+    _chk(A, AJ, AL)
+    n, P, lead = A.shape[-1], AJ.shape[0], tuple(A.shape[:-2])
+    NM = int(np.prod(lead, dtype=np.int64))
+    C, _, _, Mt, Lt = _inverse_times_rows(A.contiguous().reshape(NM, n, n), AJ.contiguous().reshape(P, NM, n, n),
+                                          AL.contiguous().reshape(NM, n, n))
+    four = lambda v: v.unsqueeze(-3)                     # (.., NM, 1, n, n)
+    if P > 0:
+        # 2 sum_c (M_c M_c)^T = 2 sum_c Mt_c Mt_c: the second-order term of the two-operand product rule
+        zero = torch.zeros_like(Lt)
+        S2t = None
+        for k0 in range(0, n, DOT_TWO_KMAX):   # contracted axis in slices the product kernel takes
+            k1 = min(n, k0 + DOT_TWO_KMAX)
+            _, _, part = dot_two(four(zero)[..., k0:k1], four(Mt)[..., k0:k1], four(zero)[..., k0:k1],
+                                 four(zero)[..., k0:k1, :], four(Mt)[..., k0:k1, :], four(zero)[..., k0:k1, :])
+            S2t = part if S2t is None else _add_flat(S2t, part)
+        Zt = _add_flat(Lt, S2t.reshape(Lt.shape), 1.0, -1.0)   # (L - 2 sum_c M_c M_c)^T
+    else:
+        Zt = Lt
+    negC = _add_flat(C, C, -1.0, 0.0)
+    t = lambda v: four(v).transpose(-1, -2)
+    _, CJ, CL = dot_const(t(Zt), t(Mt), t(Zt), four(negC))   # M_c (-C),  (L - 2 sum M M) (-C)
+    return C.reshape(A.shape), CJ.reshape(AJ.shape), CL.reshape(AL.shape)
 
 
 def elementwise(name, x, jac, lap, param=0.0, inplace=False):
@@ -663,6 +747,9 @@ def scatter_add_rows(data, idx, k_out, B, S_outer, S_inner, out=None):
         'scatter_add_rows',
     )
     return out
+
+
+SMALL_MATRIX_MAX = 32  # largest n (and number of right-hand sides) of the one-matrix-per-wavefront kernels
 
 
 def slogdet_scaled_supported(n, k_rows):

@@ -590,16 +590,20 @@ def cumsum(a, axis=-1):
 
 
 def _fold(op, a, axis):
+    """Reduction of one axis by a binary rule, as a tree: the two halves of the axis are combined element
+    by element (one launch of the binary rule per level, log2(n) levels), a leftover middle entry rides
+    along -- any length of the axis."""
     nd = len(_shape(a))
     ax = axis % nd
+    part = lambda t, lo, hi: getitem(t, tuple(slice(lo, hi) if d == ax else slice(None) for d in range(nd)))
     n = _shape(a)[ax]
-    if n > 64:
-        raise NotImplementedError('derivative-carrying max / min / prod reductions fold pairwise: axis too long')
-    take = lambda i: getitem(a, tuple(i if d == ax else slice(None) for d in range(nd)))
-    out = take(0)
-    for i in range(1, n):
-        out = op(out, take(i))
-    return out
+    assert n >= 1, 'reduction of an empty axis'
+    while n > 1:
+        h = n // 2
+        folded = op(part(a, 0, h), part(a, h, 2 * h))
+        a = folded if n == 2 * h else concatenate([folded, part(a, 2 * h, n)], axis=ax)
+        n = h + (n - 2 * h)
+    return squeeze(a, ax)
 
 
 def amax(a, axis=-1):
@@ -775,16 +779,17 @@ def logaddexp(a, b):
 
 
 def _scan(op, a, axis):
+    """Inclusive scan of one axis by an associative binary rule in log2(n) levels: at level s every entry
+    i >= s is combined with entry i - s (one launch of the binary rule per level) -- any length of the axis."""
     nd = len(_shape(a))
     ax = axis % nd
     n = _shape(a)[ax]
-    if n > 64:
-        raise NotImplementedError('cumulative max / min / prod fold pairwise: axis too long')
-    take = lambda i: getitem(a, tuple(slice(i, i + 1) if d == ax else slice(None) for d in range(nd)))
-    outs = [take(0)]
-    for i in range(1, n):
-        outs.append(op(outs[-1], take(i)))
-    return concatenate(outs, axis=ax)
+    part = lambda t, lo, hi: getitem(t, tuple(slice(lo, hi) if d == ax else slice(None) for d in range(nd)))
+    s_ = 1
+    while s_ < n:
+        a = concatenate([part(a, 0, s_), op(part(a, 0, n - s_), part(a, s_, n))], axis=ax)
+        s_ *= 2
+    return a
 
 
 def cumprod(a, axis=-1):

@@ -1619,7 +1619,18 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
         raise NotImplementedError('slogdet of a constant: call numpy.linalg.slogdet')
     row_axis = kwargs.get('row_axis')
     factor = kwargs.get('factor')
-    _check_matrix_size('slogdet', A.shape[-1])
+    if A.shape[-1] > K.SMALL_MATRIX_MAX:
+        # beyond the one-matrix-per-wavefront kernels: the same rule composed from an any-size inverse
+        # and the batched product kernel (folx/slogdet.py:296-317); canonical layout, dense Jacobian
+        if factor is not None:
+            A = _LAPLACE_FN_REGISTRY['mul']((A, factor), {}, sparsity_threshold)
+        if row_axis is not None and row_axis % A.ndim != A.ndim - 2:
+            perm = [a for a in range(A.ndim) if a != row_axis % A.ndim]
+            perm.insert(A.ndim - 2, row_axis % A.ndim)
+            A = transpose_rule((A,), {'permutation': perm}, sparsity_threshold)
+        assert A.shape[-1] == A.shape[-2], 'slogdet needs square matrices'
+        sign, ld, ldj, ldl = K.slogdet_any(A.x, A.jacobian.dense_array, A.laplacian)
+        return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
     if factor is not None:
         # slogdet(A * factor): with a dense A and a sparse factor of the same shape the product is
         # formed inside the slogdet kernel; any other combination is the mul rule first
@@ -1661,22 +1672,16 @@ def slogdet_wrapper(args, kwargs, sparsity_threshold):
     return BatchedArray(sign), FwdLaplArray(ld, FwdJacobian(ldj, None), ldl)
 
 
-def _check_matrix_size(what: str, n: int, m: int = 1):
-    """The determinant / inverse / solve kernels keep one matrix per wavefront: n, m <= 32."""
-    if n > 32 or m > 32:
-        raise NotImplementedError(
-            f'{what}: the gfx950 kernels are built for matrices of at most 32 x 32 (and at most 32 right-hand sides); '
-            f'got n = {n}' + (f', m = {m}' if m > 1 else ''))
-
-
 def inv_wrapper(args, kwargs, sparsity_threshold):
     """Matrix inverse (``inv_wrapper``, folx/linear_solve.py:114-145); dense output."""
     (A,) = args
     if not _is(A):
         raise NotImplementedError('inverse of a constant: call numpy.linalg.inv')
     assert A.shape[-1] == A.shape[-2], 'inv needs square matrices'
-    _check_matrix_size('inv', A.shape[-1])
-    C, CJ, CL = K.inv(A.x.contiguous(), A.jacobian.dense_array.contiguous(), A.laplacian.contiguous())
+    # one matrix per wavefront up to 32 x 32; beyond, the rule composed from an any-size inverse and the
+    # batched product kernels
+    rule = K.inv if A.shape[-1] <= K.SMALL_MATRIX_MAX else K.inv_any
+    C, CJ, CL = rule(A.x.contiguous(), A.jacobian.dense_array.contiguous(), A.laplacian.contiguous())
     return FwdLaplArray(C, FwdJacobian(CJ, None), CL)
 
 
@@ -1691,6 +1696,20 @@ def solve_wrapper(args, kwargs, sparsity_threshold):
     if not _is(like):
         raise NotImplementedError('solve of two constants: call numpy.linalg.solve')
     B, dev = like.B, like.x.device
+    n_, m_ = _logical_shape(A)[-1], (1 if len(_logical_shape(b)) == 1 else _logical_shape(b)[-1])
+    if n_ > K.SMALL_MATRIX_MAX or m_ > K.SMALL_MATRIX_MAX:
+        # beyond the one-system-per-wavefront kernel: y = A^-1 b through the inverse rule (any size) and the
+        # product rules; b of rank 1 is a vector, as numpy.matmul has it
+        from . import numpy as fnp
+
+        with fnp.sparsity_threshold(sparsity_threshold):
+            if _is(A):
+                Ainv = inv_wrapper((A,), {}, sparsity_threshold)
+            elif isinstance(A, (BatchedArray, torch.Tensor)):
+                raise NotImplementedError('solve: a walker-varying constant matrix beyond 32 x 32')
+            else:
+                Ainv = np.linalg.inv(np.asarray(A, dtype=np.float64)).astype(np.float32)
+            return force(fnp.matmul(Ainv, b))
 
     def parts(v):
         if _is(v):
@@ -1727,7 +1746,6 @@ def solve_wrapper(args, kwargs, sparsity_threshold):
     P = (AJ if AJ is not None else bJ).shape[0]
     full_A, full_b = (B, *batch, n, n), (B, *batch, n, m)
     ex = lambda t, shape: None if t is None else t.expand(*shape).contiguous()
-    _check_matrix_size('solve', n, m)
     y, yJ, yL = K.solve(ex(Ax, full_A), ex(AJ, (P, *full_A)), ex(AL, full_A),
                         ex(bx, full_b), ex(bJ, (P, *full_b)), ex(bL, full_b), P)
     if vector:
@@ -1804,17 +1822,37 @@ def mhsa_forward_laplacian(args, kwargs, sparsity_threshold):
     if n > 64 or d > 64 or d % 4 != 0:
         # beyond what the attention kernels are built for: the same function from its primitives
         # (two products of derivative-carrying operands around a softmax), as the reference
-        # evaluates attention that is written with einsum (folx/wrapped_functions.py:205-309)
-        if mask is not None or input_mask is not None:
-            raise NotImplementedError(
-                f'multi_head_self_attention with masks is built for n <= 64 and d <= 64 with d % 4 == 0 (got n = {n}, '
-                f'd = {d}); without masks larger shapes run through the matmul and softmax rules')
+        # evaluates attention that is written with einsum (folx/wrapped_functions.py:205-309).
+        # Masks (reference_mhsa_kernel, folx/experimental/pallas/attention/mhsa.py:79-94): a score whose
+        # query or key is padding is replaced by -1e20 in front of the softmax; Jacobian rows of inactive
+        # input coordinates are zero (the kernel never forms them, .../forward_laplacian.py:483-485).
         from . import numpy as fnp
 
+        if input_mask is not None:
+            im = input_mask.data if isinstance(input_mask, BatchedArray) else input_mask
+            im = im.to(dev) if isinstance(im, torch.Tensor) else torch.as_tensor(np.asarray(im)).to(dev)
+            im = (im != 0).to(torch.float32)
+            im = im[:, None].expand(im.shape[0], B) if im.dim() == 1 else im
+
+            def drop_rows(t):
+                J = t.jacobian.dense_array
+                assert im.shape[0] >= J.shape[0], 'input_mask must have one entry per Jacobian row'
+                J = so.pad_rows(J, im.shape[0])
+                PB, S = J.shape[0] * B, int(np.prod(t.shape, dtype=np.int64))
+                Jz = K.rows_affine(J.contiguous().reshape(PB, S), 1, (PB, S), (PB, S), im.reshape(PB, 1).contiguous(), None)
+                return FwdLaplArray(t.x, FwdJacobian(Jz.reshape(J.shape), None), t.laplacian)
+
+            q, k, v = drop_rows(q), drop_rows(k), drop_rows(v)
+            if bias is not None:
+                bias = drop_rows(bias)
         with fnp.sparsity_threshold(sparsity_threshold):
             sc = fnp.einsum('nhd,mhd->hnm', q, k)
             if bias is not None:
                 sc = fnp.add(sc, fnp.transpose(bias, (1, 0, 2)))
+            if mask is not None:
+                m = _mask_tensor(mask, (B, n), dev).to(torch.float32)
+                pair = (m[:, None, :, None] * m[:, None, None, :]).expand(B, sc.shape[0], n, n).contiguous()
+                sc = fnp.add(fnp.multiply(sc, BatchedArray(pair)), BatchedArray((1.0 - pair) * -1e20))
             return force(fnp.einsum('hnm,mhd->nhd', fnp.softmax(sc, axis=-1), v))
     if bias is None and mask is None and input_mask is None:
         sparse = _position_sparse_index(q, k, v)

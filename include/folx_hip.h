@@ -505,6 +505,28 @@ int folx_hip_sparse_slogdet_fwdlap(void* stream, const float* A, const float* A_
                                    int32_t n_coords, int32_t rank, int32_t width, int32_t transposed);
 
 /*
+ * Building blocks of the slogdet / det / inverse / solve rules for matrices of ANY size n (the
+ * rule kernels below and above stop at 32 x 32; the reference reaches LAPACK through
+ * jnp.linalg.slogdet / inv for every size, folx/slogdet.py:311-312, folx/linear_solve.py:124).
+ * A, Ainv [NM][n][n] (different buffers), sign, logdet [NM]:
+ *   Ainv = A^-1 by Gauss-Jordan elimination with partial pivoting (the pivot sequence of an LU
+ *   factorisation with partial pivoting: same sign), sign = sign(det A), logdet = log|det A|.
+ * The caller composes the rules from it and the batched product kernels:
+ *   M_c = Ainv A_jac[c],  ld_jac[c] = tr M_c,  ld_lap = tr(Ainv A_lap) - sum_c tr(M_c M_c)
+ *   (folx/slogdet.py:313-316);  C_jac[c] = -M_c Ainv,  C_lap = (2 sum_c M_c M_c - Ainv A_lap) Ainv
+ *   (folx/linear_solve.py:125-140).
+ */
+int folx_hip_inv_values(void* stream, const float* A, float* Ainv, float* sign, float* logdet,
+                        int64_t NM, int32_t n);
+
+/*
+ * tr[r] = tr M_r and trsq[r] = tr(M_r M_r) = sum_ij M_r[i][j] M_r[j][i] for a stack M [R][n][n]: the
+ * two contractions the slogdet rule takes of M_c = A^-1 d_c A, any n
+ * (jnp.einsum('k...ii->k...') and ('k...id,k...di->...'), folx/slogdet.py:314-316).
+ */
+int folx_hip_trace_pair(void* stream, const float* M, float* tr, float* trsq, int64_t R, int32_t n);
+
+/*
  * Inverse rule for NM matrices of size n x n (n <= 32) with dense Jacobians.
  *   A, A_lap, C, C_lap [NM][n][n]   A_jac, C_jac [P][NM][n][n]
  * C = A^-1;  M_p = C A_jac[p];  C_jac[p] = -M_p C;  C_lap = (2 sum_p M_p M_p - C A_lap) C.

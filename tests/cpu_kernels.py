@@ -241,6 +241,14 @@ def sparse_slogdet(A, AJ, AL, take, cols, rows, transposed):
     return _t(sign), _t(ld), _t(jac), _t(lap)
 
 
+def slogdet_any(A, AJ, AL):
+    return slogdet(A, AJ, AL)
+
+
+def inv_any(A, AJ, AL):
+    return inv(A, AJ, AL)
+
+
 def inv(A, AJ, AL):
     return tuple(_t(v) for v in rules.inv_rule(_n(A), _n(AJ), _n(AL)))
 
@@ -275,7 +283,7 @@ def mhsa_sparse(q, qs, ql, k, ks, kl, v, vs, vl, index, P, all_rows_named):
 
 KERNEL_NAMES = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'dot_const', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
                 'mul_sparse', 'rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_reduce_rows', 'gather_cols', 'scatter_add_rows',
-                'slogdet', 'sparse_slogdet', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
+                'slogdet', 'sparse_slogdet', 'slogdet_any', 'inv', 'inv_any', 'solve', 'mhsa', 'mhsa_sparse')
 
 
 def install(monkeypatch):

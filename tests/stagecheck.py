@@ -28,9 +28,9 @@ NOISE = 2.0 ** -22  # relative size of the input perturbation that measures a ru
 MAX_ALLOWANCE = 3.0  # largest widening of the bar accepted for a rule that is not a determinant
 
 _TRIPLETS = ('dense', 'dense_act', 'dense_act_parts', 'norm_dense', 'dot_two', 'dot_const', 'exp_envelope', 'layernorm', 'elementwise', 'binary',
-             'mul_sparse', 'inv', 'solve', 'mhsa', 'mhsa_sparse')
+             'mul_sparse', 'inv', 'inv_any', 'solve', 'mhsa', 'mhsa_sparse')
 _SINGLE = ('rows_affine', 'reduce_sum', 'reduce_max', 'gather_rows', 'gather_reduce_rows', 'gather_cols', 'scatter_add_rows')
-_DETS = ('slogdet', 'sparse_slogdet')
+_DETS = ('slogdet', 'sparse_slogdet', 'slogdet_any')
 
 
 def _snap(v):

@@ -320,6 +320,7 @@ _ATT_W = [np.random.default_rng(40 + i).normal(size=(3, 8)).astype(np.float32) /
 
 
 from one_constant_cases import ONE_CONSTANT_FNS  # noqa: E402
+from size_limit_cases import BIG_MATRIX_FNS  # noqa: E402
 
 
 @pytest.mark.parametrize('name', sorted(ONE_CONSTANT_FNS))
@@ -769,7 +770,7 @@ def test_forward_laplacian_of_several_arguments(thr):
 
 def test_attention_beyond_the_kernel_sizes_runs_through_matmul_and_softmax():
     """n > 64 or d > 64 (or d % 4 != 0): the attention rule evaluates the same function from the
-    two-operand product and softmax rules; with masks it says what the kernel is built for."""
+    two-operand product and softmax rules, masks included."""
     rng = np.random.default_rng(22)
     n, H, d = 5, 2, 6   # d % 4 != 0
     Wq, Wk, Wv = (rng.normal(size=(3, H * d)).astype(np.float32) / 2 for _ in range(3))
@@ -781,17 +782,43 @@ def test_attention_beyond_the_kernel_sizes_runs_through_matmul_and_softmax():
 
     check_against_oracle(fn, x, 0)
     check_against_oracle(fn, x, 6)
-    with pytest.raises(NotImplementedError, match='n <= 64'):
-        run_product(lambda xp, t: xp.sum(xp.multi_head_self_attention(
-            *(xp.reshape(xp.dot(t, w), (n, H, d)) for w in (Wq, Wk, Wv)), mask=np.ones(n, bool))), x, 0)
+    masked_attention_beyond_kernel_sizes(run_product, lambda o: triplet_np(o))
 
 
-def test_matrix_rules_name_their_size_limit():
-    x = np.random.default_rng(23).normal(size=(1, 33 * 33)).astype(np.float32)
-    with pytest.raises(NotImplementedError, match='32 x 32'):
-        run_product(lambda xp, t: xp.slogdet(xp.reshape(t, (33, 33)))[1], x, 0)
-    with pytest.raises(NotImplementedError, match='32 x 32'):
-        run_product(lambda xp, t: xp.sum(xp.inv(xp.reshape(t, (33, 33)))), x, 0)
+def masked_attention_beyond_kernel_sizes(run, to_np, n=5, H=2, d=6, valid=3, B=2):
+    """A padded sequence (``valid`` of n electrons, the coordinates of the others inactive) at a shape the
+    attention kernels do not take: scores of padding replaced by -1e20 in front of the softmax, Jacobian rows
+    of inactive coordinates dropped (test/experimental/pallas/test_attention.py:320-326, reference_mhsa_kernel
+    folx/experimental/pallas/attention/mhsa.py:79-94).  Rows of padding queries carry no meaning and are left
+    out of the comparison, as in the reference's test."""
+    rng = np.random.default_rng(24)
+    Wq, Wk, Wv = (rng.normal(size=(3, H * d)).astype(np.float32) / 2 for _ in range(3))
+    x = rng.normal(size=(B, n, 3)).astype(np.float32)
+    mask = np.zeros((B, n), dtype=bool)
+    mask[:, :valid] = True
+    imask = np.zeros((3 * n, B), dtype=bool)
+    imask[: 3 * valid] = True
+
+    def fn(xp, t, m, im):
+        q, k, v = (xp.reshape(xp.dot(t, w), (n, H, d)) for w in (Wq, Wk, Wv))
+        return xp.multi_head_self_attention(xp.multiply(q, 1.0 / np.sqrt(d)), k, v, mask=m, input_mask=im)
+
+    for thr in (0, 6):
+        got = to_np(run(lambda xp, t: fn(xp, t, mask, imask), x, thr))
+        ref = fn(ob, ob.init_state(x, dtype=np.float64), mask, imask)
+        np.testing.assert_allclose(got[0][:, :valid], ref.x[:, :valid], rtol=2e-4, atol=2e-5)
+        np.testing.assert_allclose(got[1][:, :, :valid], ref.J[:, :, :valid], rtol=2e-4, atol=2e-5)
+        np.testing.assert_allclose(got[2][:, :valid], ref.lap[:, :valid], rtol=2e-4, atol=2e-4)
+        assert np.isfinite(got[0]).all() and np.isfinite(got[1]).all() and np.isfinite(got[2]).all()
+        assert np.abs(got[1][3 * valid:]).max() == 0.0   # rows of inactive coordinates
+
+
+@pytest.mark.parametrize('name', sorted(BIG_MATRIX_FNS))
+def test_matrix_rules_beyond_the_small_matrix_kernels(name):
+    """slogdet / det / inv / solve of 34 x 34 matrices (the one-matrix-per-wavefront kernels stop at 32): the
+    rules dispatch to their any-size forms (folx/slogdet.py:296-344, folx/linear_solve.py:54-145 take any n)."""
+    x = (np.random.default_rng(23).normal(size=(2, 6)) * 0.3).astype(np.float32)
+    check_against_oracle(BIG_MATRIX_FNS[name], x, 0)
 
 
 @pytest.mark.parametrize('thr', [0, 6])
