@@ -39,6 +39,7 @@ __global__ __launch_bounds__(AS_NT) void inv_values_kernel(const float* __restri
   __syncthreads();
 
   float sgn = 1.0f, ldet = 0.0f;
+  bool singular = false;  // a zero (or non-finite) pivot: sign 0 and log|det| = -inf, as numpy.linalg.slogdet reports it
   for (int k = 0; k < n; ++k) {
     // pivot: the largest |W[i][k]|, i >= k, the first one among equals
     float best = -1.0f;
@@ -82,7 +83,8 @@ __global__ __launch_bounds__(AS_NT) void inv_values_kernel(const float* __restri
       }
     }
     __syncthreads();
-    sgn = piv == 0.0f ? 0.0f : sgn * ((piv < 0.0f) != (p != k) ? -1.0f : 1.0f);
+    if (!(fabsf(piv) > 0.0f) || !(fabsf(piv) < INFINITY)) singular = true;
+    sgn *= (piv < 0.0f) != (p != k) ? -1.0f : 1.0f;
     ldet += logf(fabsf(piv));
   }
   // the row swaps of the elimination are column swaps of the inverse, undone last to first
@@ -102,8 +104,8 @@ __global__ __launch_bounds__(AS_NT) void inv_values_kernel(const float* __restri
     for (int e = tid; e < nn; e += AS_NT) out[e] = W[(e / n) * ld + e % n];
   }
   if (tid == 0) {
-    sign[blockIdx.x] = sgn;
-    logdet[blockIdx.x] = ldet;
+    sign[blockIdx.x] = singular ? 0.0f : sgn;
+    logdet[blockIdx.x] = singular ? -INFINITY : ldet;
   }
 }
 

@@ -136,7 +136,7 @@ def test_floor_is_used_by_small_entries_only():
     rng = np.random.default_rng(21)
     rows, P, Kd, N = (4, 32), 96, 256, 256
     x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
-    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    W = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32)
     ref = rules.dense_rule(*f64(x, J, L, W))
     got = K.dense(dev(x), dev(J), dev(L), dev(W))
     gJ = got[1].cpu().numpy().astype(np.float64)

@@ -24,7 +24,8 @@ def dev(a):
 
 def _matrices(rng, lead, n, P):
     A = (np.eye(n) * 2.0 + rng.normal(size=(*lead, n, n)) / np.sqrt(n)).astype(np.float32)
-    A[..., [0, 1], :] = A[..., [1, 0], :]     # a row exchange: the pivot search has work to do, the sign is -1 times ...
+    if n >= 2:
+        A[..., [0, 1], :] = A[..., [1, 0], :]     # a row exchange: the pivot search has work to do and the sign flips
     J = rng.normal(size=(P, *lead, n, n)).astype(np.float32)
     L = rng.normal(size=(*lead, n, n)).astype(np.float32)
     return A, J, L
