@@ -265,6 +265,7 @@ def measure(workload, steps, warmup, walkers=0, chunk=1024, gemm='f32', graph=Fa
 
 
 # the other BASELINE.json configurations, measured briefly after the headline: (steps, warm-up steps, chunk)
+GRAPH_REPLAY_TOO = ('mlp_dense', 'mlp_sparse', 'ferminet16')
 OTHER_WORKLOADS = {'mlp_dense': (20, 5, 1024), 'mlp_sparse': (20, 5, 1024), 'ferminet16': (8, 4, 1024),
                    'psiformer64': (2, 1, 1024)}
 
@@ -370,8 +371,15 @@ def main():
                                                        'avg_launch_ms', 'share_of_gpu_time', 'mfma_frac') if k in r},
                 }
                 del o
+                if name in GRAPH_REPLAY_TOO:
+                    # the reference runs under jax.jit; its counterpart here is the replay of a captured HIP graph,
+                    # which takes the host's rule dispatch out of a step made of many short launches
+                    o = measure(name, k_steps, k_warm, 0, k_chunk, graph=True)
+                    others[name]['hip_graph_replay'] = {'value': o['B'] * k_steps / o['dt'], 'unit': 'walkers/s',
+                                                        'ms_per_step': 1e3 * o['dt'] / k_steps}
+                    del o
             except Exception as e:  # a side measurement must not take the headline line down with it
-                others[name] = {'error': f'{type(e).__name__}: {e}'}
+                others.setdefault(name, {})['error'] = f'{type(e).__name__}: {e}'
             torch.cuda.empty_cache()
         line['other_workloads'] = others
     if not args.no_cpu:

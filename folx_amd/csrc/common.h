@@ -33,6 +33,13 @@ struct Bcast3 {
   int64_t n1, n2;
   int64_t s0, s1, s2;
   __device__ __forceinline__ int64_t off(int64_t i) const {
+    if ((((uint64_t)i | (uint64_t)n1 | (uint64_t)n2) >> 32) == 0) {
+      // everything fits 32 bits (the usual case): a 64-bit division costs several times a 32-bit one
+      const uint32_t j = (uint32_t)i, m1 = (uint32_t)n1, m2 = (uint32_t)n2;
+      const uint32_t t = j / m2, i2 = j - t * m2;
+      const uint32_t i0 = t / m1, i1 = t - i0 * m1;
+      return i0 * s0 + i1 * s1 + i2 * s2;
+    }
     int64_t i2 = i % n2;
     int64_t t = i / n2;
     int64_t i1 = t % n1;

@@ -33,7 +33,10 @@ __device__ __forceinline__ float wave_sum1(float a) {
 
 constexpr int PSPLIT = 4;
 
-template <int NV>
+// PER_WAVE: for a few Jacobian rows (sparse storage, P <= 8) a whole workgroup per row of features would
+// mostly wait at its barrier: each WAVEFRONT owns a row of features then and walks all P Jacobian rows
+// itself (four in flight), no LDS and no barrier.
+template <int NV, bool PER_WAVE>
 __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
     const float* __restrict__ x, const float* __restrict__ jac, const float* __restrict__ lap,
     const float* __restrict__ gamma, const float* __restrict__ beta, float* __restrict__ y,
@@ -42,7 +45,9 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
   __shared__ float reds[PSPLIT][2];
   const int lane = threadIdx.x % FOLX_WAVE;
   const int w = threadIdx.x / FOLX_WAVE;
-  const int64_t row = blockIdx.x;
+  const int64_t row = PER_WAVE ? (int64_t)blockIdx.x * PSPLIT + w : (int64_t)blockIdx.x;
+  if (PER_WAVE && row >= R) return;
+  constexpr int PS = PER_WAVE ? 1 : PSPLIT;  // distance between the Jacobian rows of a wavefront
   const int F4 = F / 4;
   const float invF = 1.0f / (float)F;
   const int64_t S = R * (int64_t)F;  // elements per Jacobian row
@@ -117,13 +122,13 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
     }
   };
 
-  int p = w;
-  for (; p + 3 * PSPLIT < P; p += 4 * PSPLIT) {  // four Jacobian rows in flight per wavefront
+  int p = PER_WAVE ? 0 : w;
+  for (; p + 3 * PS < P; p += 4 * PS) {  // four Jacobian rows in flight per wavefront
     float4 u0[NV], u1[NV], u2[NV], u3[NV];
     load_row(p, u0);
-    load_row(p + PSPLIT, u1);
-    load_row(p + 2 * PSPLIT, u2);
-    load_row(p + 3 * PSPLIT, u3);
+    load_row(p + PS, u1);
+    load_row(p + 2 * PS, u2);
+    load_row(p + 3 * PS, u3);
     float a1, a2, a3, b1, b2, b3, c1, c2, c3, e1, e2, e3;
     partial(u0, a1, a2, a3);
     partial(u1, b1, b2, b3);
@@ -134,11 +139,11 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
     wave_sum3(c1, c2, c3);
     wave_sum3(e1, e2, e3);
     finish_row(p, u0, a1, a2, a3);
-    finish_row(p + PSPLIT, u1, b1, b2, b3);
-    finish_row(p + 2 * PSPLIT, u2, c1, c2, c3);
-    finish_row(p + 3 * PSPLIT, u3, e1, e2, e3);
+    finish_row(p + PS, u1, b1, b2, b3);
+    finish_row(p + 2 * PS, u2, c1, c2, c3);
+    finish_row(p + 3 * PS, u3, e1, e2, e3);
   }
-  for (; p < P; p += PSPLIT) {
+  for (; p < P; p += PS) {
     float4 u0[NV];
     load_row(p, u0);
     float a1, a2, a3;
@@ -149,19 +154,21 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void layernorm_kernel(
 
   // the sums over p of the four wavefronts meet in LDS (this barrier also orders every
   // wavefront's read of x before the write of y, which makes in-place use safe)
+  if constexpr (!PER_WAVE) {
 #pragma unroll
-  for (int v = 0; v < NV; ++v) redT[w][v * FOLX_WAVE + lane] = T[v];
-  if (lane == 0) { reds[w][0] = sb2; reds[w][1] = ss; }
-  __syncthreads();
-  if (w != 0) return;
-  sb2 = reds[0][0]; ss = reds[0][1];
+    for (int v = 0; v < NV; ++v) redT[w][v * FOLX_WAVE + lane] = T[v];
+    if (lane == 0) { reds[w][0] = sb2; reds[w][1] = ss; }
+    __syncthreads();
+    if (w != 0) return;
+    sb2 = reds[0][0]; ss = reds[0][1];
 #pragma unroll
-  for (int ww = 1; ww < PSPLIT; ++ww) {
-    sb2 += reds[ww][0]; ss += reds[ww][1];
+    for (int ww = 1; ww < PSPLIT; ++ww) {
+      sb2 += reds[ww][0]; ss += reds[ww][1];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-      const float4 t = redT[ww][v * FOLX_WAVE + lane];
-      T[v].x += t.x; T[v].y += t.y; T[v].z += t.z; T[v].w += t.w;
+      for (int v = 0; v < NV; ++v) {
+        const float4 t = redT[ww][v * FOLX_WAVE + lane];
+        T[v].x += t.x; T[v].y += t.y; T[v].z += t.z; T[v].w += t.w;
+      }
     }
   }
 
@@ -212,16 +219,21 @@ extern "C" int folx_hip_layernorm_fwdlap(void* stream, const float* x, const flo
   const void* ptrs[] = {x, jac, lap, gamma, beta, y, y_jac, y_lap};
   for (const void* p : ptrs)
     if (p && !folx_aligned16(p)) return FOLX_HIP_ENOTSUP;
-  const int64_t blocks = R;
+  const bool per_wave = P <= 8;
+  const int64_t blocks = per_wave ? (R + PSPLIT - 1) / PSPLIT : R;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)blocks), block(FOLX_WAVE * PSPLIT);
   const int nv = (F / 4 + FOLX_WAVE - 1) / FOLX_WAVE;
+#define FOLX_LN(NV)                                                                                               \
+  if (per_wave) layernorm_kernel<NV, true><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); \
+  else layernorm_kernel<NV, false><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps);
   switch (nv) {
-    case 1: layernorm_kernel<1><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); break;
-    case 2: layernorm_kernel<2><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); break;
-    case 3: layernorm_kernel<3><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); break;
-    default: layernorm_kernel<4><<<grid, block, 0, st>>>(x, jac, lap, gamma, beta, y, y_jac, y_lap, R, F, P, eps); break;
+    case 1: FOLX_LN(1) break;
+    case 2: FOLX_LN(2) break;
+    case 3: FOLX_LN(3) break;
+    default: FOLX_LN(4) break;
   }
+#undef FOLX_LN
   return folx_launch_status();
 }

@@ -82,44 +82,64 @@ __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void binary_kernel(
 //   y_lap = b a_lap + a b_lap + 2 sum_s a_jac[idx[s]] b_jac[s].
 // Same work split as binary_kernel; each lane keeps its k sparse rows and their indices in
 // registers, so the dense rows of the sparse operand are never built.
-template <int KMAX>
+// VEC = 4: a lane owns four consecutive elements (128-bit streaming accesses; S_w % 4 == 0, 16-byte aligned
+// operands), VEC = 1: one element.
+template <int KMAX, int VEC>
 __global__ __launch_bounds__(FOLX_WAVE * PSPLIT) void mul_sparse_kernel(
     const float* __restrict__ a, const float* __restrict__ aj, const float* __restrict__ al,
     const float* __restrict__ b, const float* __restrict__ bj, const float* __restrict__ bl,
     const int32_t* __restrict__ idx, float* __restrict__ y, float* __restrict__ yj, float* __restrict__ yl,
     int64_t S, int64_t S_w, int32_t P, int32_t k) {
-  __shared__ float red[PSPLIT][FOLX_WAVE];
+  __shared__ float red[PSPLIT][VEC][FOLX_WAVE];
   const int lane = threadIdx.x % FOLX_WAVE;
   const int w = threadIdx.x / FOLX_WAVE;
-  const int64_t i = (int64_t)blockIdx.x * FOLX_WAVE + lane;
+  const int64_t i = ((int64_t)blockIdx.x * FOLX_WAVE + lane) * VEC;
   const bool active = i < S;
-  float sab = 0.0f, av = 0.0f, bv = 0.0f;
+  float sab[VEC], av[VEC], bv[VEC];
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) sab[v] = av[v] = bv[v] = 0.0f;
   if (active) {
-    av = a[i];
-    bv = b[i];
-    const int64_t pos = i % S_w;
-    int32_t ix[KMAX];
-    float bs[KMAX];
+    const int64_t pos = (uint64_t)(i | S_w) >> 32 ? i % S_w : (int64_t)((uint32_t)i % (uint32_t)S_w);
+    int32_t ix[KMAX][VEC];
+    float bs[KMAX][VEC];
 #pragma unroll
-    for (int s = 0; s < KMAX; ++s) {
-      ix[s] = s < k ? idx[(int64_t)s * S_w + pos] : -1;
-      bs[s] = ix[s] >= 0 ? bj[(int64_t)s * S + i] : 0.0f;
-    }
+    for (int v = 0; v < VEC; ++v) { av[v] = a[i + v]; bv[v] = b[i + v]; }
+#pragma unroll
+    for (int s = 0; s < KMAX; ++s)
+#pragma unroll
+      for (int v = 0; v < VEC; ++v) {
+        ix[s][v] = s < k ? idx[(int64_t)s * S_w + pos + v] : -1;
+        bs[s][v] = ix[s][v] >= 0 ? bj[(int64_t)s * S + i + v] : 0.0f;
+      }
     for (int p = w; p < P; p += PSPLIT) {
-      const float ja = __builtin_nontemporal_load(&aj[(int64_t)p * S + i]);
-      float o = bv * ja;
+      float ja[VEC], o[VEC];
+      if constexpr (VEC == 4) {
+        const float4 t = folx_ld_stream4(aj + (int64_t)p * S + i);
+        ja[0] = t.x; ja[1] = t.y; ja[2] = t.z; ja[3] = t.w;
+      } else {
+        ja[0] = __builtin_nontemporal_load(&aj[(int64_t)p * S + i]);
+      }
 #pragma unroll
-      for (int s = 0; s < KMAX; ++s)
-        if (ix[s] == p) { o += av * bs[s]; sab += ja * bs[s]; }
-      __builtin_nontemporal_store(o, &yj[(int64_t)p * S + i]);
+      for (int v = 0; v < VEC; ++v) {
+        o[v] = bv[v] * ja[v];
+#pragma unroll
+        for (int s = 0; s < KMAX; ++s)
+          if (ix[s][v] == p) { o[v] += av[v] * bs[s][v]; sab[v] += ja[v] * bs[s][v]; }
+      }
+      if constexpr (VEC == 4) folx_st_stream4(yj + (int64_t)p * S + i, make_float4(o[0], o[1], o[2], o[3]));
+      else __builtin_nontemporal_store(o[0], &yj[(int64_t)p * S + i]);
     }
   }
-  red[w][lane] = sab;
+#pragma unroll
+  for (int v = 0; v < VEC; ++v) red[w][v][lane] = sab[v];
   __syncthreads();
   if (w == 0 && active) {
-    const float s = red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane];
-    y[i] = av * bv;
-    yl[i] = bv * al[i] + av * bl[i] + 2.0f * s;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+      const float s = red[0][v][lane] + red[1][v][lane] + red[2][v][lane] + red[3][v][lane];
+      y[i + v] = av[v] * bv[v];
+      yl[i + v] = bv[v] * al[i + v] + av[v] * bl[i + v] + 2.0f * s;
+    }
   }
 }
 
@@ -137,6 +157,49 @@ __global__ __launch_bounds__(256) void rows_affine_kernel(const float* __restric
   const float dv = d ? beta * d[id.off(i)] : 0.0f;
   // blockIdx.y strides over rows so that very tall stacks need no 64-bit grid
   for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) out[r * S + i] = in[r * in_S + oi] * cv + dv;
+}
+
+// The same map for index spaces whose inner extent is a multiple of 4 and whose operands are contiguous
+// (stride 1) or constant (stride 0) along it, all 16-byte aligned: a thread owns four consecutive
+// elements, one 128-bit streaming load and store per row, and its three offsets are computed once --
+// in 32-bit arithmetic (S < 2^31), without any division when the index space is flat.
+__global__ __launch_bounds__(256) void rows_affine_v4_kernel(const float* __restrict__ in,
+                                                             float* __restrict__ out, int64_t rows,
+                                                             int64_t in_S, int64_t S,
+                                                             const float* __restrict__ c,
+                                                             const float* __restrict__ d, float alpha,
+                                                             float beta, Bcast3 iin, Bcast3 ic,
+                                                             Bcast3 id) {
+  const uint32_t i = ((uint32_t)blockIdx.x * 256u + threadIdx.x) * 4u;
+  if (i >= (uint32_t)S) return;
+  const uint32_t n1 = (uint32_t)iin.n1, n2 = (uint32_t)iin.n2;
+  uint32_t i0 = 0, i1 = 0, i2 = i;
+  if (n2 < (uint32_t)S) {
+    i2 = i % n2;
+    const uint32_t t = i / n2;
+    i1 = t % n1;
+    i0 = t / n1;
+  }
+  const int64_t oi = i0 * iin.s0 + i1 * iin.s1 + i2 * iin.s2;
+  float4 cv = make_float4(alpha, alpha, alpha, alpha);
+  float4 dv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (c) {
+    const float* p = c + (i0 * ic.s0 + i1 * ic.s1 + i2 * ic.s2);
+    const float4 v = ic.s2 ? *reinterpret_cast<const float4*>(p) : make_float4(*p, *p, *p, *p);
+    cv = make_float4(alpha * v.x, alpha * v.y, alpha * v.z, alpha * v.w);
+  }
+  if (d) {
+    const float* p = d + (i0 * id.s0 + i1 * id.s1 + i2 * id.s2);
+    const float4 v = id.s2 ? *reinterpret_cast<const float4*>(p) : make_float4(*p, *p, *p, *p);
+    dv = make_float4(beta * v.x, beta * v.y, beta * v.z, beta * v.w);
+  }
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+    const float* p = in + r * in_S + oi;
+    float4 v;
+    if (iin.s2) v = folx_ld_stream4(p);
+    else v = make_float4(*p, *p, *p, *p);
+    folx_st_stream4(out + r * S + i, make_float4(v.x * cv.x + dv.x, v.y * cv.y + dv.y, v.z * cv.z + dv.z, v.w * cv.w + dv.w));
+  }
 }
 
 Bcast3 mk(const int64_t* dims, int k) {
@@ -188,8 +251,24 @@ extern "C" int folx_hip_rows_affine(void* stream, const float* in, float* out, i
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   Bcast3 iin = mk(dims, 1), ic = mk(dims, 2), id = mk(dims, 3);
   const unsigned gy = (unsigned)(rows < 1024 ? rows : 1024);
-  rows_affine_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
-      in, out, rows, in_S, S, c, d, alpha, beta, iin, ic, id);
+  // 128-bit form: inner extent a multiple of 4, every operand contiguous or constant along it, every other
+  // stride and the row pitch multiples of 4 floats, 16-byte aligned pointers, 32-bit element index
+  auto vec_ok = [&](const Bcast3& b, const float* p) {
+    if (!p) return true;
+    if (b.s2 != 0 && b.s2 != 1) return false;
+    if (b.s2 == 0) return true;
+    return folx_aligned16(p) && (dims[1] == 1 || b.s1 % 4 == 0) && (dims[0] == 1 || b.s0 % 4 == 0);
+  };
+  const bool v4 = dims[2] % 4 == 0 && S < 0x7fffffffLL && folx_aligned16(out) && vec_ok(iin, in) && vec_ok(ic, c) &&
+                  vec_ok(id, d) && (rows == 1 || iin.s2 == 0 || in_S % 4 == 0);
+  if (v4) {
+    const int64_t blocks4 = (S / 4 + 255) / 256;
+    rows_affine_v4_kernel<<<dim3((unsigned)blocks4, gy), dim3(256), 0, (hipStream_t)stream>>>(
+        in, out, rows, in_S, S, c, d, alpha, beta, iin, ic, id);
+  } else {
+    rows_affine_kernel<<<dim3((unsigned)blocks, gy), dim3(256), 0, (hipStream_t)stream>>>(
+        in, out, rows, in_S, S, c, d, alpha, beta, iin, ic, id);
+  }
   return folx_launch_status();
 }
 
@@ -204,15 +283,22 @@ extern "C" int folx_hip_mul_sparse_fwdlap(void* stream, const float* a, const fl
       (k_rows > 0 && (!b_jac || !index)))
     return FOLX_HIP_EINVAL;
   if (k_rows > 8) return FOLX_HIP_ENOTSUP;
-  const int64_t blocks = (S + FOLX_WAVE - 1) / FOLX_WAVE;
+  const bool vec4 = S_w % 4 == 0 && k_rows <= 4 && folx_aligned16(a) && folx_aligned16(a_jac) && folx_aligned16(a_lap) &&
+                    folx_aligned16(b) && folx_aligned16(b_jac) && folx_aligned16(b_lap) && folx_aligned16(y) &&
+                    folx_aligned16(y_jac) && folx_aligned16(y_lap);
+  const int64_t per_block = FOLX_WAVE * (vec4 ? 4 : 1);
+  const int64_t blocks = (S + per_block - 1) / per_block;
   if (blocks > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
   dim3 grid((unsigned)blocks), block(FOLX_WAVE * PSPLIT);
   hipStream_t st = (hipStream_t)stream;
-  if (k_rows <= 4)
-    mul_sparse_kernel<4><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
-                                                 k_rows);
+  if (vec4)
+    mul_sparse_kernel<4, 4><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
+                                                    k_rows);
+  else if (k_rows <= 4)
+    mul_sparse_kernel<4, 1><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
+                                                    k_rows);
   else
-    mul_sparse_kernel<8><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
-                                                 k_rows);
+    mul_sparse_kernel<8, 1><<<grid, block, 0, st>>>(a, a_jac, a_lap, b, b_jac, b_lap, index, y, y_jac, y_lap, S, S_w, P,
+                                                    k_rows);
   return folx_launch_status();
 }

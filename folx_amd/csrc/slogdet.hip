@@ -38,10 +38,11 @@ constexpr int TRB = 16;  // Jacobian rows whose traces are reduced together
 // 16 < n <= 32: one 32 x 32 tile (v_mfma_f32_32x32x2_f32) per wavefront.  Lane l holds, for step
 // t, the element (k = 2 t + l / 32, lr = l % 32) of an operand: as A operand that is row lr,
 // column k; as B operand row k, column lr.  With a[t] = Ainv[lr][k] and j[t] = J[k][lr]:
-//   mfma(a, j) accumulates M   = Ainv J      (A = Ainv,  B = J)
-//   mfma(j, a) accumulates M^T = J^T Ainv^T  (A = J^T,   B = Ainv^T) -- the SAME registers,
-// so the transpose that tr(M M) = sum_ab M[a][b] M^T[a][b] needs costs a second product and
-// no data movement, and tr M = sum over lanes and steps of a[t] j[t].
+//   mfma(a, j) accumulates M = Ainv J      (A = Ainv,  B = J)
+// and tr M = sum over lanes and steps of a[t] j[t].  The transpose that tr(M M) = sum_ab M[a][b] M[b][a]
+// needs comes back through LDS.  (It could be had as a second product of the SAME registers, mfma(j, a) =
+// J^T Ainv^T, without any data movement -- but then the kernel is bound by the matrix pipe: two 32 x 32 x 32
+// products per 4 KB row are 64 flop per byte, three times the ridge of the FP32 matrix peak over HBM.)
 __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet32_kernel(
     const float* __restrict__ A, const float* __restrict__ AJ, const float* __restrict__ AL,
     float* __restrict__ sign_out, float* __restrict__ logdet_out, float* __restrict__ jac_out,
@@ -49,8 +50,11 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet32_kernel(
     int64_t rstride, int64_t slice) {
   constexpr int NP = 32, STEPS = 16;
   constexpr int AUGS = smallmat::Aug<NP>::stride;  // row stride of the augmented matrix
-  __shared__ float aug[NP * AUGS];
+  constexpr int MTS = 36;  // row stride of the tile that hands M^T back
+  __shared__ __attribute__((aligned(16))) float aug[NP * AUGS];
   __shared__ float trs[TRB][FOLX_WAVE + 1];
+  static_assert(MTS <= AUGS, "the tile of M reuses the memory of the augmented matrix");
+  float* const mt = aug;  // the augmented matrix is dead once Ainv sits in registers
 
   const int lane = threadIdx.x;
   const int64_t m = blockIdx.x;
@@ -65,43 +69,66 @@ __global__ __launch_bounds__(FOLX_WAVE, 3) void slogdet32_kernel(
   const int lr = lane % 32;
   const int lq = lane / 32;
   float ainv[STEPS];
-  bool ok[STEPS];
-  int64_t eoff[STEPS];
+  int32_t eoff[STEPS];  // offsets inside one matrix fit 32 bits (checked by the launcher)
 #pragma unroll
   for (int t = 0; t < STEPS; ++t) {
     const int k = 2 * t + lq;
-    ok[t] = k < n && lr < n;
+    const bool ok = k < n && lr < n;
     // elements of the padding ask for element (0, 0): loads are never branched around, so
-    // that all of them are in flight before the first wait
-    eoff[t] = ok[t] ? (int64_t)k * rstride + lr : 0;
-    ainv[t] = ok[t] ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
+    // that all of them are in flight before the first wait.  What they bring in needs no masking:
+    // in M = Ainv J it meets the zero rows and columns of the padded Ainv, or lands in columns b >= n
+    // of M, which tr(M M) pairs with the zero rows M[b][.] and tr M never reads.
+    eoff[t] = ok ? (int32_t)(k * rstride) + lr : 0;
+    ainv[t] = ok ? aug[lr * AUGS + NP + k] : 0.0f;  // Ainv[lr][k]
   }
 
   float mm = 0.0f;
-  float raw[STEPS];
-  auto request = [&](int p) __attribute__((always_inline)) {
+  float raw0[STEPS], raw1[STEPS];  // two Jacobian rows on their way
+  auto request = [&](int p, float (&raw)[STEPS]) __attribute__((always_inline)) {
     const float* src = AJ + (int64_t)p * slice + base;
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) raw[t] = src[eoff[t]];  // A_jac[p][k][lr], padding masked when used
   };
-  if (P > 0) request(0);
-  for (int p = 0; p < P; ++p) {
-    float jv[STEPS];
+  // One product per row, M = Ainv J in accumulator layout (lane (b, h), register 4 g + j <-> M[8 g + 4 h + j][b]);
+  // tr(M M) = sum_ab M[a][b] M[b][a] takes M^T back from LDS: the tile is written row-major (row stride 36:
+  // the 128-bit reads of 16 lanes then fall on distinct banks) and lane (b, h) reads M[b][8 g + 4 h .. + 3].
+  // LDS serves a wavefront's accesses in issue order, so the round trip needs no barrier.
+  auto do_row = [&](int p, const float (&raw)[STEPS]) __attribute__((always_inline)) {
+    floatx16 c;
 #pragma unroll
-    for (int t = 0; t < STEPS; ++t) jv[t] = ok[t] ? raw[t] : 0.0f;
-    if (p + 1 < P) request(p + 1);  // the next row is on its way during the products
-    floatx16 c, ct;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) { c[r] = 0.0f; ct[r] = 0.0f; }
+    for (int r = 0; r < 16; ++r) c[r] = 0.0f;
     float tr = 0.0f;
 #pragma unroll
     for (int t = 0; t < STEPS; ++t) {
-      c = __builtin_amdgcn_mfma_f32_32x32x2f32(ainv[t], jv[t], c, 0, 0, 0);    // M   = Ainv J
-      ct = __builtin_amdgcn_mfma_f32_32x32x2f32(jv[t], ainv[t], ct, 0, 0, 0);  // M^T
-      tr = fmaf(ainv[t], jv[t], tr);                                          // this lane's part of tr M
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(ainv[t], raw[t], c, 0, 0, 0);  // M = Ainv J
+      tr = fmaf(ainv[t], raw[t], tr);                                        // this lane's part of tr M
     }
+    asm volatile("" ::: "memory");
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mm = fmaf(c[r], ct[r], mm);
+    for (int r = 0; r < 16; ++r) mt[(8 * (r / 4) + 4 * lq + r % 4) * MTS + lr] = c[r];
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 t4 = *reinterpret_cast<const float4*>(&mt[lr * MTS + 8 * g + 4 * lq]);
+      mm = fmaf(c[4 * g + 0], t4.x, mm);
+      mm = fmaf(c[4 * g + 1], t4.y, mm);
+      mm = fmaf(c[4 * g + 2], t4.z, mm);
+      mm = fmaf(c[4 * g + 3], t4.w, mm);
+    }
+    asm volatile("" ::: "memory");
+    return tr;
+  };
+  if (P > 0) request(0, raw0);
+  if (P > 1) request(1, raw1);
+  for (int p = 0; p < P; ++p) {
+    float tr;
+    if (p % 2 == 0) {
+      tr = do_row(p, raw0);
+      if (p + 2 < P) request(p + 2, raw0);
+    } else {
+      tr = do_row(p, raw1);
+      if (p + 2 < P) request(p + 2, raw1);
+    }
     trs[p % TRB][lane] = tr;
     if ((p + 1) % TRB == 0 || p + 1 == P) {
       // ld_jac of the last rows: four lanes per row add up 16 of its 64 parts each.
@@ -493,6 +520,7 @@ int launch_slogdet(hipStream_t st, const float* A, const float* A_jac, const flo
   dim3 block(FOLX_WAVE);
   if (n > 16) {
     if (fc) return FOLX_HIP_ENOTSUP;
+    if ((int64_t)(n - 1) * row_stride + n > 0x7fffffffLL) return FOLX_HIP_ENOTSUP;
     slogdet32_kernel<<<dim3((unsigned)NM), block, 0, st>>>(A, A_jac, A_lap, sign, logdet, ld_jac, ld_lap, NM, n, P, ND,
                                                            batch_stride, member_stride, row_stride, jac_stride);
     return folx_launch_status();

@@ -610,6 +610,15 @@ def _dot_then_act(h, W, kwargs, thr: int):
             h = layer_norm_rule((h, gamma, beta), {'eps': eps}, thr)
     if act is None:
         return dot_general((h, W), {**kwargs, 'residual': residual}, thr)
+    k_pad = 0
+    if (_is(h) and not _is(W) and not isinstance(W, torch.Tensor) and kwargs.get('row_slice') is None and np.ndim(W) == 2
+            and np.shape(W)[1] > 128 and np.shape(W)[0] % 16 != 0 and np.shape(W)[0] >= 16):
+        # a wide layer whose input width is no multiple of 16 (a first layer fed by raw features): the fused
+        # kernel takes it with the feature axis padded by zero columns against zero rows of W, which costs one
+        # copy of the input triplet and saves the pre-activation triplet's trip through memory
+        k_pad = -np.shape(W)[0] % 16
+        W = np.concatenate([np.asarray(W, dtype=np.float32), np.zeros((k_pad, np.shape(W)[1]), dtype=np.float32)], axis=0)
+    K_in = np.shape(W)[0] - k_pad
     fused = (
         _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
         and K.dense_act_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1))
@@ -630,11 +639,17 @@ def _dot_then_act(h, W, kwargs, thr: int):
                 new_mask = np.broadcast_to(proj, (proj.shape[0], *h.shape[:-1], N))
     if fused:  # the number of Jacobian rows decides whether the wide kernel's tiles are well filled
         fused = K.dense_act_supported(act, *np.shape(W), rows=h.x.numel() // max(h.x.shape[-1], 1), P=J.shape[0])
+    if not fused and k_pad:
+        W = W[:K_in]
     if fused:
         dev = h.x.device
         Wt = so.device_const(W, dev)
         bt = None if bias is None else so.device_const(bias, dev)
         res = None
+        hx, hl = h.x, h.laplacian
+        if k_pad:
+            padk = lambda t: torch.nn.functional.pad(t, (0, k_pad))
+            hx, J, hl = padk(hx), padk(J), padk(hl)
         if (_is(residual) and K.dense_act_residual_supported(*np.shape(W))
                 and tuple(residual.shape) == (*h.shape[:-1], np.shape(W)[1])
                 and residual.jacobian.data.shape[0] == J.shape[0]):
@@ -648,7 +663,7 @@ def _dot_then_act(h, W, kwargs, thr: int):
             if same:
                 res = (residual.x.contiguous(), residual.jacobian.data.contiguous(), residual.laplacian.contiguous())
                 residual = None
-        y, Jy, lapy = K.dense_act(act, h.x, J, h.laplacian, Wt, bt, param, res)
+        y, Jy, lapy = K.dense_act(act, hx, J, hl, Wt, bt, param, res)
         out = FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
     else:
         out = dot_general((h, W), kwargs, thr)
