@@ -55,6 +55,9 @@ def parse():
                     help='skip the short second measurement with --gemm bf16x3 that a default run appends')
     ap.add_argument('--no-other', action='store_true',
                     help='skip the short measurements of the other workloads that a default run appends')
+    ap.add_argument('--streaming-rules', action='store_true',
+                    help='instead of a workload: launch every HBM-bound rule at its largest workload shape (ten launches '
+                         'each, HIP events) and print one JSON line of achieved TB/s; the command profiles/ traces')
     ap.add_argument('--graph', action='store_true',
                     help='replay each chunk as a captured HIP graph (no per-kernel timing, no roofline)')
     ap.add_argument('--calibrate-copy', action='store_true',
@@ -270,6 +273,98 @@ OTHER_WORKLOADS = {'mlp_dense': (20, 5, 1024), 'mlp_sparse': (20, 5, 1024), 'fer
                    'psiformer64': (2, 1, 1024)}
 
 
+def streaming_rules():
+    """Every HBM-bound rule at the largest shape the benchmark workloads give it (a chunk of 1024 walkers): achieved
+    rate = the rule's algorithmic bytes (the per-unit figures of the kernels' headers) over the mean duration of ten
+    launches, HIP events on the launch stream.  One JSON line; `rocprofv3 --kernel-trace --stats` of this command gives
+    the same durations kernel by kernel."""
+    import torch
+
+    from folx_amd import kernels as K
+
+    dev = torch.device('cuda', 0)
+    g = torch.Generator(device='cuda').manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)  # noqa: E731
+    table = []
+
+    def run(name, kernel, fn, nbytes, reps=10):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        table.append({'rule': name, 'kernel': kernel, 'avg_us': 1e3 * ms, 'algorithmic_GB': nbytes / 1e9,
+                      'TB_per_s': nbytes / ms / 1e9, 'frac_of_8TBps': nbytes / ms / 1e9 / (PEAK_HBM_GBS / 1e3)})
+
+    n = 1 << 28
+    src = rn(n)
+    run('plain copy of 1 GiB (calibration of the HBM counters)', 'rows_affine_v4_kernel',
+        lambda: K.rows_affine(src, 1, (n,), (n,), None, None, 1.0, 0.0), 8.0 * n)
+    d2 = rn(n)
+    run('sum of two row stacks, 1 GiB each', 'rows_affine_v4_kernel',
+        lambda: K.rows_affine(src, 1, (n,), (n,), None, d2, 1.0, 1.0), 12.0 * n)
+    del src, d2
+    R, F, P = 32768, 256, 96                        # 1024 walkers x 32 electrons, width 256, dense Jacobian
+    x, J, L = rn(R, F), rn(P, R, F), rn(R, F)
+    run('tanh, P = 96 dense rows', 'elementwise_kernel', lambda: K.elementwise('tanh', x, J, L), 8.0 * (P + 2) * R * F)
+    gam, bet = rn(F), rn(F)
+    run('LayerNorm, P = 96 dense rows', 'layernorm_kernel<1, false>', lambda: K.layernorm(x, J, L, gam, bet, 1e-5),
+        8.0 * (P + 2) * R * F)
+    J3 = rn(3, R, F)
+    run('LayerNorm, k = 3 sparse rows (first layer)', 'layernorm_kernel<1, true>',
+        lambda: K.layernorm(x, J3, L, gam, bet, 1e-5), 8.0 * 5 * R * F, reps=30)
+    run('tanh, k = 3 sparse rows', 'elementwise_kernel', lambda: K.elementwise('tanh', x, J3, L), 8.0 * 5 * R * F, reps=30)
+    J2 = rn(P, R, F)
+    run('product of two triplets, P = 96', 'binary_kernel<mul>', lambda: K.binary('mul', x, J, L, x, J2, L),
+        12.0 * (P + 2) * R * F)
+    del J2
+    idx = torch.arange(3 * 32, device=dev, dtype=torch.int32).reshape(3, 32)
+    idxf = idx[:, :, None].expand(3, 32, 256).reshape(3, -1).contiguous()
+    v = lambda t, lead: t.view(*lead, 1024, -1)  # noqa: E731
+    run('dense x sparse product, P = 96, k = 3', 'mul_sparse_kernel<4, 4>',
+        lambda: K.mul_sparse(v(x, ()), v(J, (P,)), v(L, ()), v(x, ()), v(J3, (3,)), v(L, ()), idxf),
+        4.0 * (2 * P + 3 + 6) * R * F)
+    del J
+    data = rn(3, 1024, 32 * 256)
+    take = torch.full((96, 1, 32), -1, device=dev, dtype=torch.int32)
+    for so_ in range(32):
+        for r in range(3):
+            take[3 * so_ + r, 0, so_] = r
+    run('sparse -> dense hand-off, k = 3 rows to 96', 'gather_rows_flat_kernel<4>',
+        lambda: K.gather_rows(data, take, 96, 1, 1024, 32, 256), 4.0 * (3 + 96) * 1024 * 32 * 256)
+    out = rn(96, 1024, 32 * 256)
+    run('sparse skip connection added in place, k = 3 into 96 rows', 'scatter_add_rows_kernel<4>',
+        lambda: K.scatter_add_rows(data, idx, 96, 1024, 32, 256, out=out), 4.0 * 3 * 3 * 1024 * 32 * 256, reps=30)
+    del out, data
+    inp = rn(1, 49152, 16, 256)
+    run('sum over 16 electrons of a (48 x 1024, 16, 256) stack', 'reduce_mid_v4_kernel',
+        lambda: K.reduce_sum(inp, 1, 49152, 16, 256), 4.0 * 49152 * 17 * 256, reps=30)
+    del inp
+    A, AJ, AL = rn(16384, 16, 16), rn(96, 16384, 16, 16), rn(16384, 16, 16)
+    run('slogdet, 16384 matrices 16 x 16, P = 96', 'slogdet16_kernel<16, false, 4>', lambda: K.slogdet(A, AJ, AL),
+        4.0 * 98 * 256 * 16384)
+    A, AJ, AL = rn(16384, 8, 8), rn(48, 16384, 8, 8), rn(16384, 8, 8)
+    run('slogdet, 16384 matrices 8 x 8, P = 48', 'slogdet16_kernel<8, false, 4>', lambda: K.slogdet(A, AJ, AL),
+        4.0 * 50 * 64 * 16384, reps=30)
+    A, AJ, AL = rn(16384, 32, 32), rn(192, 16384, 32, 32), rn(16384, 32, 32)
+    run('slogdet, 16384 matrices 32 x 32, P = 192', 'slogdet32_kernel', lambda: K.slogdet(A, AJ, AL),
+        4.0 * 194 * 1024 * 16384, reps=5)
+    table[-1]['mfma_TFLOP_per_s'] = 2.0 * 192 * 32768 * 16384 / (table[-1]['avg_us'] * 1e-6) / 1e12
+    del A, AJ, AL
+    B, n_, H, d, k, Pd = 1024, 32, 4, 64, 3, 96
+    q, qs, ql = rn(B, n_, H, d) / 8, rn(k, B, n_, H, d) / 8, rn(B, n_, H, d) / 8
+    ix = torch.arange(k * n_, device=dev, dtype=torch.int32).reshape(n_, k).t().contiguous()
+    run('attention on position-sparse rows, k = 3 -> P = 96', 'mhsa_sparse_kernel',
+        lambda: K.mhsa_sparse(q, qs, ql, q, qs, ql, q, qs, ql, ix, Pd, True), 4.0 * n_ * d * (Pd + 3 * k + 8) * B * H)
+    print(json.dumps({'metric': 'achieved HBM rate of the streaming rules at their largest workload shapes',
+                      'peak_TB_per_s': PEAK_HBM_GBS / 1e3, 'rules': table}))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
@@ -283,6 +378,9 @@ def main():
 
     torch.cuda.set_device(0)
     K.set_gemm_mode(args.gemm)
+    if args.streaming_rules:
+        streaming_rules()
+        return
     m = measure(args.workload, args.steps, args.warmup, args.walkers, args.chunk, args.gemm, args.graph,
                 args.calibrate_copy)
     B, cfg, thr, out, x, step, dt, roof = (m[k] for k in ('B', 'cfg', 'thr', 'out', 'x', 'step', 'dt', 'roof'))

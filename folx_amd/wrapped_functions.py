@@ -611,13 +611,16 @@ def _dot_then_act(h, W, kwargs, thr: int):
     if act is None:
         return dot_general((h, W), {**kwargs, 'residual': residual}, thr)
     k_pad = 0
-    if (_is(h) and not _is(W) and not isinstance(W, torch.Tensor) and kwargs.get('row_slice') is None and np.ndim(W) == 2
+    if (_is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
             and np.shape(W)[1] > 128 and np.shape(W)[0] % 16 != 0 and np.shape(W)[0] >= 16):
         # a wide layer whose input width is no multiple of 16 (a first layer fed by raw features): the fused
         # kernel takes it with the feature axis padded by zero columns against zero rows of W, which costs one
         # copy of the input triplet and saves the pre-activation triplet's trip through memory
         k_pad = -np.shape(W)[0] % 16
-        W = np.concatenate([np.asarray(W, dtype=np.float32), np.zeros((k_pad, np.shape(W)[1]), dtype=np.float32)], axis=0)
+        if isinstance(W, torch.Tensor):  # a caller-owned device tensor: padded on every call (it may change in place)
+            W = torch.cat([W.to(torch.float32), W.new_zeros((k_pad, W.shape[1]), dtype=torch.float32)], dim=0)
+        else:
+            W = np.concatenate([np.asarray(W, dtype=np.float32), np.zeros((k_pad, np.shape(W)[1]), dtype=np.float32)], axis=0)
     K_in = np.shape(W)[0] - k_pad
     fused = (
         _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2

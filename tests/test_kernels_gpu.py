@@ -117,7 +117,7 @@ def test_dense(rows, P, Kd, N, bias):
     print(f'case dense rows={rows} P={P} K={Kd} N={N}', flush=True)
     rng = np.random.default_rng(2)
     x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
-    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    W = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32)
     b = rand(rng, N) if bias else None
     ref = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
     got = K.dense(dev(x), dev(J), dev(L), dev(W), None if b is None else dev(b))
@@ -193,7 +193,7 @@ def test_dense_act(rows, P, Kd, N, bias, act):
     print(f'case dense_act rows={rows} P={P} K={Kd} N={N} act={act}', flush=True)
     rng = np.random.default_rng(21)
     x, J, L = rand(rng, *rows, Kd), rand(rng, P, *rows, Kd), rand(rng, *rows, Kd)
-    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    W = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32)
     b = rand(rng, N) if bias else None
     z = rules.dense_rule(*f64(x, J, L, W), None if b is None else b.astype(np.float64))
     ref = rules.elementwise_rule(act, *z)
@@ -249,7 +249,7 @@ def test_norm_dense(rows, P, Kd, N, affine, bias, act):
     J = J + 0.3 * rand(rng, P, *rows, 1)  # rows with a mean of their own
     g = (1.0 + 0.3 * rand(rng, Kd)) if affine else None
     be = 0.2 * rand(rng, Kd) if affine else None
-    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    W = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32)
     b = rand(rng, N) if bias else None
     h = ob.layer_norm(ob.OArr(*f64(x, J, L)), None if g is None else g.astype(np.float64),
                       None if be is None else be.astype(np.float64), 1e-5)
@@ -310,7 +310,7 @@ def test_dense_act_parts(B, n, P, widths, bcast, N, act):
             xp_, lp_, Jp = (np.broadcast_to(np.expand_dims(t, -2), (*t.shape[:-1], n, w)) for t in (xp_, lp_, Jp))
         xs.append(xp_), ls.append(lp_), Jd.append(Jp)
     x, L, J = np.concatenate(xs, -1), np.concatenate(ls, -1), np.concatenate(Jd, -1)
-    W = rand(rng, Kd, N) / np.sqrt(Kd)
+    W = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32)
     b = rand(rng, N)
     ref = rules.elementwise_rule(act, *rules.dense_rule(*f64(x, J, L, W), b.astype(np.float64)))
     for rep in range(2):
@@ -430,7 +430,7 @@ def test_dense_row_slice(lead, n, lo, hi, P, Kd, N):
     print(f'case dense row_slice lead={lead} n={n} [{lo}:{hi}] P={P} K={Kd} N={N}', flush=True)
     rng = np.random.default_rng(20)
     x, J, L = rand(rng, *lead, n, Kd), rand(rng, P, *lead, n, Kd), rand(rng, *lead, n, Kd)
-    W, b = rand(rng, Kd, N) / np.sqrt(Kd), rand(rng, N)
+    W, b = (rand(rng, Kd, N) / np.sqrt(Kd)).astype(np.float32), rand(rng, N)
     ref = rules.dense_rule(*f64(x[..., lo:hi, :], J[..., lo:hi, :], L[..., lo:hi, :], W), b.astype(np.float64))
     got = K.dense(dev(x), dev(J), dev(L), dev(W), dev(b), None, (lo, hi))
     assert got[0].shape == (*lead, hi - lo, N)
