@@ -304,6 +304,30 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  if constexpr (PARTS) {
+    // The per-walker pre-activation term is what the accumulators START from (the products are added to it): its
+    // loads are in flight with the first chunk, where registers are plentiful, instead of in the epilogue.
+    // Register r of a block <-> Jacobian row p0 + 4 (lane / 32) + 8 ((r / 4) % GB) + r % 4 of position (r / 4) / GB.
+    if (a.pre_jac) {
+      constexpr int GB = PT / 8;
+      const int64_t pre_pstride = (R / a.pre_group) * N;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          int gc = col0 + wc + j * 32 + l32;
+          if (gc >= N) gc = N - 1;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int g = r / 4, b = g / GB;
+            int prow = p0 + 4 * lh + 8 * (g % GB) + r % 4;
+            if (prow >= P) prow = P - 1;  // rows past P of a ragged tile are neither stored nor summed
+            const int64_t pos = r0 + (wrow * TM + i) * PB + b;
+            acc[i][j][r] = a.pre_jac[(int64_t)prow * pre_pstride + (pos / a.pre_group) * N + gc];
+          }
+        }
+    }
+  }
   // LayerNorm's row sums are taken by ONE wavefront per tile row block and SIMD: block i of
   // tile row group wrow by the wavefront with column index i + 2 * wrow.  That wavefront runs
   // its own copy of the K loop; the others run the plain one.  Per tile row wr + 32 si + l32,
@@ -570,29 +594,15 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
 #pragma unroll
       for (int b = 0; b < PB; ++b) ss[b] = 0.0f;
       const float* resp = nullptr;
-      const float* prep[PB];
-      int64_t pre_pstride = 0;
-#pragma unroll
-      for (int b = 0; b < PB; ++b) prep[b] = nullptr;
-      if constexpr (PARTS) {
-        resp = a.res_jac ? a.res_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc : nullptr;
-        if (a.pre_jac) {
-          pre_pstride = (R / a.pre_group) * N;
-          const int gcc = gc < N ? gc : N - 1;
-#pragma unroll
-          for (int b = 0; b < PB; ++b)
-            prep[b] = a.pre_jac + ((pos + b) / a.pre_group) * N + gcc;
-        }
-      }
-      auto rows = [&](auto full, auto has_res, auto has_pre) __attribute__((always_inline)) {
+      if constexpr (PARTS) resp = a.res_jac ? a.res_jac + ((int64_t)(p0 + 4 * lh) * R + pos) * N + gc : nullptr;
+      auto rows = [&](auto full, auto has_res) __attribute__((always_inline)) {
         constexpr int GB = PT / 8;     // register groups per position
-        constexpr bool FULL = decltype(full)::value, RES = decltype(has_res)::value, PRE = decltype(has_pre)::value;
-        // What the epilogue reads from memory (skip connection, per-walker pre-activation term) is
-        // asked for one register group ahead of its use: the stores of a group cannot be told
-        // apart from these arrays, so a load written after them would wait for them to be issued,
-        // and every group would pay a round trip of its own.
-        float rbuf[2][4], pbuf[2][4];
-        auto fetch = [&](int g, float (&rb)[4], float (&pb)[4]) __attribute__((always_inline)) {
+        constexpr bool FULL = decltype(full)::value, RES = decltype(has_res)::value;
+        // What the epilogue reads from memory (the skip connection) is asked for one register group ahead
+        // of its use: the stores of a group cannot be told apart from that array, so a load written after
+        // them would wait for them to be issued, and every group would pay a round trip of its own.
+        float rbuf[2][4];
+        auto fetch = [&](int g, float (&rb)[4]) __attribute__((always_inline)) {
           const int b = g / GB;
 #pragma unroll
           for (int rr = 0; rr < 4; ++rr) {
@@ -600,24 +610,18 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
             const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
             const bool live = FULL || (p0 + 4 * lh + pl < P && gc < N);
             rb[rr] = 0.0f;
-            pb[rr] = 0.0f;
-            if constexpr (PRE) {
-              int prow = p0 + 4 * lh + pl;  // rows past P of a ragged tile are neither stored nor summed
-              if constexpr (!FULL) prow = prow < P ? prow : P - 1;
-              pb[rr] = prep[b][(int64_t)prow * pre_pstride];
-            }
             if constexpr (RES) {
               if constexpr (FULL) rb[rr] = __builtin_nontemporal_load(resp + off);
               else if (live) rb[rr] = resp[off];
             }
           }
         };
-        if constexpr (RES || PRE) fetch(0, rbuf[0], pbuf[0]);
+        if constexpr (RES) fetch(0, rbuf[0]);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int b = g / GB;          // position of this group inside the block
-          if constexpr (RES || PRE)
-            if (g + 1 < 4) fetch(g + 1, rbuf[(g + 1) & 1], pbuf[(g + 1) & 1]);
+          if constexpr (RES)
+            if (g + 1 < 4) fetch(g + 1, rbuf[(g + 1) & 1]);
           float ap[4] = {0.0f, 0.0f, 0.0f, 0.0f}, bp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
           if constexpr (NORM) {
             const float4* sp = reinterpret_cast<const float4*>(st + i * 32 + 8 * g + 4 * lh);
@@ -636,7 +640,6 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
             }
             const int64_t off = (int64_t)pl * pstride + (int64_t)b * N;
             float* o = out + off;
-            if constexpr (PRE) v += pbuf[g & 1][rr];
             if constexpr (FULL) {
               if constexpr (ACT) ss[b] = fmaf(v, v, ss[b]);
               float w = d1[b] * v;
@@ -649,20 +652,12 @@ __global__ __launch_bounds__(NT, 4) void dense_wide_kernel(WideParams a) {
           }
         }
       };
-      if (PARTS && prep[0] != nullptr) {
-        if (resp != nullptr) {
-          if (full_tile) rows(std::true_type{}, std::true_type{}, std::true_type{});
-          else rows(std::false_type{}, std::true_type{}, std::true_type{});
-        } else {
-          if (full_tile) rows(std::true_type{}, std::false_type{}, std::true_type{});
-          else rows(std::false_type{}, std::false_type{}, std::true_type{});
-        }
-      } else if (PARTS && resp != nullptr) {
-        if (full_tile) rows(std::true_type{}, std::true_type{}, std::false_type{});
-        else rows(std::false_type{}, std::true_type{}, std::false_type{});
+      if (PARTS && resp != nullptr) {
+        if (full_tile) rows(std::true_type{}, std::true_type{});
+        else rows(std::false_type{}, std::true_type{});
       } else {
-        if (full_tile) rows(std::true_type{}, std::false_type{}, std::false_type{});
-        else rows(std::false_type{}, std::false_type{}, std::false_type{});
+        if (full_tile) rows(std::true_type{}, std::false_type{});
+        else rows(std::false_type{}, std::false_type{});
       }
       const int64_t so = ((int64_t)pg * R + pos) * N + gc;
       if constexpr (ACT) {
