@@ -14,6 +14,10 @@ static inline int folx_launch_status() {
 static inline bool folx_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #ifdef __HIPCC__
+// Index of the wavefront inside its workgroup, in a scalar register: threadIdx.x / 64 is the same for the lanes of
+// a wavefront, but the compiler cannot know that; with the scalar, loops over "this wavefront's rows" have scalar trip
+// counts and row addresses take the scalar-base form instead of 64-bit vector arithmetic per access.
+__device__ __forceinline__ int folx_wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x / FOLX_WAVE)); }
 // Streaming accesses for data that is touched once per launch (Jacobian rows): non-temporal
 // loads and stores, which a row-strided copy on this GPU runs 12 % faster with.
 typedef float folx_vf4 __attribute__((ext_vector_type(4)));

@@ -191,7 +191,7 @@ __global__ __launch_bounds__(FOLX_WAVE * SLD_WPB, 4) void slogdet16_kernel(
   // one workgroup so that they start together and (with a barrier every D rows) stay together:
   // where members lie side by side along the matrix rows, the pieces of a row that the SLD_WPB
   // wavefronts ask for at about the same time are then one contiguous stretch of memory.
-  const int lane = threadIdx.x % FOLX_WAVE, wv = threadIdx.x / FOLX_WAVE;
+  const int lane = threadIdx.x % FOLX_WAVE, wv = folx_wave_id();
   float* aug = ws_all[wv];
   float* mt = ws_all[wv];
   float (*trs)[FOLX_WAVE + 1] = reinterpret_cast<float (*)[FOLX_WAVE + 1]>(ws_all[wv] + 16 * TS);
