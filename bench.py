@@ -180,7 +180,8 @@ def roofline_of(dname, dkey, dn, dms, gemm):
         norm = dname == 'norm_dense_fwdlap'
         return mfma(2.0 * (P + 2) * R * Kd * N,
                     f'dense_wide_kernel<{"true" if norm else "false"}, {"false" if act is None else "true"}, '
-                    f'{"32, false" if norm else "16 | 32, parts"}> + the short launches of its entry point '
+                    f'{"32, false" if norm else "16 | 32, parts"}, {"true" if gemm == "bf16x3" else "false"}> '
+                    f'+ the short launches of its entry point '
                     f'({dname}: x / lap rows GEMM, finish; with LayerNorm also weight fold and per-position rows), '
                     f'act={act} R={R} P={P} K={Kd} N={N}')
     if dname == 'dense_act_fwdlap':
