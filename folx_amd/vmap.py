@@ -44,7 +44,8 @@ def batched_vmap(fn, max_batch_size: int, in_axes=0, out_axes=0):
     ``None`` an argument without a walker axis, which is shown whole to every walker.  Nothing
     is inferred from shapes: an array that merely has ``B`` leading entries is only cut when its
     entry of ``in_axes`` says so.  ``out_axes`` must be 0: results keep the walker axis where the
-    data layout has it."""
+    data layout has it.  The returned function can itself be chunked again over another axis (nested use)
+    when it returns tensors."""
     import numpy as np
 
     if out_axes != 0 and not (isinstance(out_axes, (tuple, list)) and all(a == 0 for a in out_axes)):
@@ -88,4 +89,38 @@ def batched_vmap(fn, max_batch_size: int, in_axes=0, out_axes=0):
             parts.append(batched(*cut(s, s + max_batch_size), **kwargs))
         return _cat(parts)
 
+    def nested(*args, **kwargs):
+        """This chunked function under an OUTER ``vmap`` / ``batched_vmap`` (test/test_vmap.py:50-66): every
+        array argument arrives with the outer axis in front.  The two axes are flattened into one walker
+        axis (an argument that the inner level shows whole is repeated for the inner walkers), the
+        flattened batch runs in chunks, and the results get both axes back."""
+        axes = tuple(in_axes) if isinstance(in_axes, (tuple, list)) else (in_axes,) * len(args)
+        assert len(axes) == len(args), f'batched_vmap: {len(axes)} in_axes for {len(args)} arguments'
+        is_arr = lambda a: isinstance(a, (torch.Tensor, np.ndarray))
+        outer = [a.shape[0] for a in args if is_arr(a)]
+        inner = [a.shape[ax + 1] for a, ax in zip(args, axes) if is_arr(a) and ax is not None]
+        assert outer and inner, 'batched_vmap: no argument carries a walker axis'
+        Bo, Bi = outer[0], inner[0]
+        assert all(b == Bo for b in outer) and all(b == Bi for b in inner), 'batched_vmap: walker axes differ in length'
+        flat = []
+        for a, ax in zip(args, axes):
+            if not is_arr(a):
+                flat.append(a)
+                continue
+            t = a if isinstance(a, torch.Tensor) else torch.as_tensor(np.ascontiguousarray(a))
+            t = t[:, None].expand(Bo, Bi, *t.shape[1:]) if ax is None else t.movedim(ax + 1, 1)
+            t = t.reshape(Bo * Bi, *t.shape[2:])
+            flat.append(t if isinstance(a, torch.Tensor) else t.numpy())
+        out = batched_vmap(fn, max_batch_size)(*flat, **kwargs)
+
+        def unflatten(o):
+            if isinstance(o, (tuple, list)):
+                return type(o)(unflatten(v) for v in o)
+            if isinstance(o, torch.Tensor):
+                return o.reshape(Bo, Bi, *o.shape[1:])
+            raise NotImplementedError('nested batched_vmap: results must be tensors (apply an operator, or take .x / '
+                                      '.laplacian / .jacobian.dense_array inside the function)')
+        return unflatten(out)
+
+    result.batched = nested
     return result

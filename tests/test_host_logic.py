@@ -214,6 +214,41 @@ def test_batched_vmap_in_axes():
         folx_amd.batched_vmap(g, 2, out_axes=1)
 
 
+def test_batched_vmap_uneven_multiple_arguments_and_nested():
+    """The reference's own cases (test/test_vmap.py:23-66): a batch that the chunk size does not divide, two
+    mapped arguments, and two nested levels ``batched_vmap(batched_vmap(f, m, (0, None)), m, (None, 0))`` whose
+    result carries both axes, for chunk sizes 10, 5 and 1; here ``f`` is the Laplacian operator of
+    ``vdot(sin x, cos y)``, whose Laplacian is ``-2 vdot(sin x, cos y)``."""
+    rng = np.random.default_rng(42)
+    f = lambda u, v: fnp.sum(fnp.multiply(fnp.sin(u), fnp.cos(v)))
+    fl = folx_amd.forward_laplacian(f, 0)
+
+    class op:  # Laplacian and gradient as tensors with the walker axis in front (the operators take one argument)
+        @staticmethod
+        def batched(*args):
+            out = fl.batched(*args)
+            return out.laplacian, out.jacobian.dense_array.movedim(0, -1)
+    a21, b21 = rng.normal(size=(21, 3)).astype(np.float32), rng.normal(size=(21, 3)).astype(np.float32)
+    want = -2.0 * (np.sin(a21.astype(np.float64)) * np.cos(b21.astype(np.float64))).sum(-1)
+    for mb in (10, 5, 1):
+        lap, jac = folx_amd.batched_vmap(op, mb)(a21, b21)
+        assert tuple(lap.shape) == (21,) and tuple(jac.shape) == (21, 6)
+        np.testing.assert_allclose(lap.numpy(), want, rtol=1e-5, atol=1e-6)
+    a, b = a21[:10], b21[:7]
+    want2 = -2.0 * np.einsum('ik,jk->ji', np.sin(a.astype(np.float64)), np.cos(b.astype(np.float64)))  # [j over b][i over a]
+    for mb in (10, 5, 1):
+        lap, jac = folx_amd.batched_vmap(folx_amd.batched_vmap(op, mb, in_axes=(0, None)), mb, in_axes=(None, 0))(a, b)
+        assert tuple(lap.shape) == (7, 10) and tuple(jac.shape) == (7, 10, 6)
+        np.testing.assert_allclose(lap.numpy(), want2, rtol=1e-5, atol=1e-6)
+    # the outer level may also be the plain vmap
+    lap, _ = folx_amd.vmap(folx_amd.batched_vmap(op, 4, in_axes=(0, None)))(
+        np.broadcast_to(a[None], (7, 10, 3)).copy(), b)
+    np.testing.assert_allclose(lap.numpy(), want2, rtol=1e-5, atol=1e-6)
+    with pytest.raises(NotImplementedError):  # a triplet has one walker axis
+        folx_amd.vmap(folx_amd.batched_vmap(folx_amd.forward_laplacian(f, 0), 4, in_axes=(0, None)))(
+            np.broadcast_to(a[None], (7, 10, 3)).copy(), b)
+
+
 def test_register_function_plugs_in():
     calls = []
 
