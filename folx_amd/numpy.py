@@ -644,6 +644,36 @@ def pad(a, pad_width, constant_values=0.0):
     return out
 
 
+def lax_pad(operand, padding_value, padding_config):
+    """``jax.lax.pad`` (the ``pad_p`` primitive, folx/wrapped_functions.py:480-487): per axis ``(low, high, interior)``
+    with negative ``low`` / ``high`` cropping the (interior-padded) array, and a padding value that may itself carry
+    derivatives.  Every output element is an operand element or the padding value, so the result is one static
+    position gather from ``[operand elements..., padding value]``; sparse Jacobians stay sparse."""
+    shape = tuple(_shape(operand))
+    cfg = [tuple(int(v) for v in c) for c in padding_config]
+    assert len(cfg) == len(shape), 'lax_pad: one (low, high, interior) per axis'
+    n_total = int(np.prod(shape)) if shape else 1
+    per_axis = []
+    for n, (lo, hi, it) in zip(shape, cfg):
+        assert it >= 0, 'lax_pad: negative interior padding'
+        dil = n + max(n - 1, 0) * it
+        m = np.full(max(lo + dil + hi, 0), -1, dtype=np.int64)
+        pos = lo + np.arange(n) * (it + 1)
+        ok = (pos >= 0) & (pos < m.size)
+        m[pos[ok]] = np.arange(n)[ok]
+        per_axis.append(m)
+    grids = np.meshgrid(*per_axis, indexing='ij') if per_axis else []
+    valid = np.ones([m.size for m in per_axis], dtype=bool)
+    for g in grids:
+        valid &= g >= 0
+    table = np.full(valid.shape, n_total, dtype=np.int64)      # n_total: the slot of the padding value
+    if valid.any():
+        table[valid] = np.ravel_multi_index(tuple(g[valid] for g in grids), shape)
+    pv = padding_value if _is_triplet(padding_value) else np.full((1,), float(np.asarray(padding_value)), dtype=np.float32)
+    src = concatenate([reshape(operand, (n_total,)), reshape(pv, (1,))], axis=0)
+    return getitem(src, table)
+
+
 floor, ceil, round = (lambda a: _call('floor', (a,))), (lambda a: _call('ceil', (a,))), (lambda a: _call('round', (a,)))
 greater, greater_equal = (lambda a, b: _call('gt', (a, b))), (lambda a, b: _call('ge', (a, b)))
 less, less_equal = (lambda a, b: _call('lt', (a, b))), (lambda a, b: _call('le', (a, b)))
@@ -827,7 +857,8 @@ register_function('cumprod', _composed(cumprod, 'axis'))
 register_function('cummax', _composed(cummax, 'axis'))
 register_function('cummin', _composed(cummin, 'axis'))
 register_function('logaddexp', _composed(logaddexp))
-register_function('pad', _composed(pad, 'constant_values'))
+register_function('pad', lambda args, kw, thr: _composed(lax_pad, 'padding_config')(args, kw, thr) if 'padding_config' in kw
+                  else _composed(pad, 'constant_values')(args, kw, thr))   # lax.pad_p.bind(operand, value, padding_config=...)
 register_function('atan2', _composed(arctan2))                       # folx/wrapped_functions.py:419
 register_function('rem', _composed(remainder))                       # :438
 register_function('exp2', _composed(exp2))                           # :636

@@ -749,6 +749,35 @@ def pad(a: OArr, pad_width, constant_values=0.0):
                 np.pad(a.lap, [(0, 0)] + pw))
 
 
+def lax_pad(a: OArr, padding_value, padding_config):
+    """``jax.lax.pad`` semantics (what folx wraps as an indexing rule, folx/wrapped_functions.py:480-487), written
+    as array surgery: a canvas of the padding value, the operand laid out with strides ``interior + 1``, then the
+    low / high edges added or (negative) cut.  The padding value may carry derivatives."""
+    cfg = [tuple(int(v) for v in c) for c in padding_config]
+
+    def one(arr, lead, fill):          # arr (*lead_shape, *shape); fill broadcastable to lead_shape
+        shape = arr.shape[lead:]
+        dil = [n + max(n - 1, 0) * it for n, (_, _, it) in zip(shape, cfg)]
+        canvas = np.empty((*arr.shape[:lead], *dil), dtype=arr.dtype)
+        canvas[...] = np.asarray(fill).reshape(*np.shape(fill), *([1] * len(shape)))
+        canvas[(*[slice(None)] * lead, *[slice(None, None, it + 1) for (_, _, it) in cfg])] = arr
+        for ax, (lo, hi, _) in enumerate(cfg):
+            n = canvas.shape[lead + ax]
+            canvas = canvas[(*[slice(None)] * (lead + ax), slice(max(-lo, 0), n - max(-hi, 0)))]
+            edge = lambda w: np.broadcast_to(
+                np.asarray(fill).reshape(*np.shape(fill), *([1] * len(shape))),
+                (*canvas.shape[:lead + ax], w, *canvas.shape[lead + ax + 1:]))
+            canvas = np.concatenate([edge(max(lo, 0)), canvas, edge(max(hi, 0))], axis=lead + ax)
+        return canvas
+
+    B, P = a.x.shape[0], a.J.shape[0]
+    if _is(padding_value):
+        fx, fJ, fl = padding_value.x.reshape(B), padding_value.J.reshape(P, B), padding_value.lap.reshape(B)
+    else:
+        fx, fJ, fl = np.full(B, float(np.asarray(padding_value))), np.zeros((P, B)), np.zeros(B)
+    return OArr(one(a.x, 1, fx), one(a.J, 2, fJ), one(a.lap, 1, fl))
+
+
 def _cmp(fn):
     def f(a, b):
         av = a.x if _is(a) else np.asarray(a)

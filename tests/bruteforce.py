@@ -296,6 +296,22 @@ class plain:
         flat = [v for p in reversed(pw) for v in p]
         return torch.nn.functional.pad(a, flat, value=constant_values)
 
+    @staticmethod
+    def lax_pad(a, padding_value, padding_config):
+        """jax.lax.pad element by element: output position q of an axis holds operand entry j when
+        q = low + j (interior + 1), the padding value otherwise."""
+        cfg = [tuple(int(v) for v in c) for c in padding_config]
+        sizes = [max(lo + n + max(n - 1, 0) * it + hi, 0) for n, (lo, hi, it) in zip(a.shape, cfg)]
+        pv = padding_value if torch.is_tensor(padding_value) else torch.tensor(float(padding_value), dtype=a.dtype)
+        out = []
+        for q in np.ndindex(*sizes):
+            src = []
+            for qa, n, (lo, hi, it) in zip(q, a.shape, cfg):
+                j, r = divmod(qa - lo, it + 1)
+                src.append(j if r == 0 and 0 <= j < n else None)
+            out.append(pv.reshape(()) if any(v is None for v in src) else a[tuple(src)])
+        return torch.stack(out).reshape(sizes)
+
     arctan2 = staticmethod(lambda y, x: torch.atan2(y if torch.is_tensor(y) else plain._c(y, x), plain._c(x, y) if torch.is_tensor(y) else x))
     remainder = staticmethod(lambda a, b: torch.fmod(a, plain._c(b, a)))
     fmod = remainder

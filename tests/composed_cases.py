@@ -60,6 +60,13 @@ CASES = {
         xp.add(xp.multiply(xp.sin(_g(xp, xp.add(xp.tile(x, (6,)), _OFFS), slice(0, 65))), 0.2), 1.0), axis=-1),
     'cumprod_long_axis': lambda xp, x: xp.cumprod(xp.add(xp.multiply(xp.sin(xp.add(xp.tile(x, (6,)), _OFFS)), 0.2), 1.0)),
     'cummax_long_axis': lambda xp, x: xp.cummax(xp.tanh(xp.multiply(xp.add(xp.tile(x, (6,)), _SPREAD), 0.3))),
+    # jax.lax.pad as the reference's tests use it (test/test_layers.py:668-682): interior padding, a padding value
+    # that depends on the input, negative (cropping) edges
+    'lax_pad_interior': lambda xp, x: xp.lax_pad(xp.reshape(xp.sin(x), (4, 3)), 7.0, ((1, 0, 1), (0, 2, 0))),
+    'lax_pad_varying_value': lambda xp, x: xp.lax_pad(xp.tanh(_g(xp, x, slice(0, 11))),
+                                                       xp.square(xp.reshape(_g(xp, x, slice(11, 12)), ())), ((2, 1, 1),)),
+    'lax_pad_negative': lambda xp, x: xp.lax_pad(xp.multiply(xp.sin(x), x), 0.0, ((-1, -2, 0),)),
+    'lax_pad_negative_interior': lambda xp, x: xp.lax_pad(xp.reshape(xp.cos(x), (3, 4)), -1.5, ((-1, 2, 2), (1, -3, 1))),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }

@@ -49,6 +49,15 @@ def test_composed_rules(name, thr):
     check_against_oracle(composed_cases.CASES[name], X, thr)
 
 
+@pytest.mark.parametrize('name', ['lax_pad_interior', 'lax_pad_varying_value', 'lax_pad_negative', 'lax_pad_negative_interior',
+                                  'flip_pad'])
+def test_pad_keeps_the_jacobian_sparse(name):
+    """Padding is an indexing operation (folx/wrapped_functions.py:480-487; test/test_layers.py:668-682 asserts
+    ``is_jacobian_weak``, :763-776 one stored row): every output element is one operand element or the padding value."""
+    out = run_product(composed_cases.CASES[name], X, 12)
+    assert out.jacobian.weak and out.jacobian.data.shape[0] == 1
+
+
 @pytest.mark.parametrize('thr', [0, 12])
 def test_min_max(thr):
     check_against_oracle(min_max_elementwise, X, thr)
