@@ -846,6 +846,124 @@ def _composed(fn, *kw_names):
     return rule
 
 
+# jax.numpy / jax.nn names that trace to chains of the primitives above in the reference; the same chains here
+def relu(a):
+    return maximum(a, 0.0)
+
+
+def leaky_relu(a, negative_slope=0.01):
+    return where(greater_equal(a, 0.0), a, multiply(a, float(negative_slope)))
+
+
+def elu(a, alpha=1.0):
+    return where(greater(a, 0.0), a, multiply(expm1(minimum(a, 0.0)), float(alpha)))
+
+
+def gelu(a, approximate=True):
+    """``jax.nn.gelu``: the tanh form by default, ``approximate=False`` the erf form (test/test_layers.py:709)."""
+    if approximate:
+        inner = multiply(add(a, multiply(integer_pow(a, 3), 0.044715)), float(np.sqrt(2.0 / np.pi)))
+        return multiply(multiply(a, 0.5), add(tanh(inner), 1.0))
+    return multiply(multiply(a, 0.5), add(erf(multiply(a, float(1.0 / np.sqrt(2.0)))), 1.0))
+
+
+def log_softmax(a, axis=-1):
+    shifted = subtract(a, amax_const(a, axis, keepdims=True))
+    return subtract(shifted, log(sum(exp(shifted), axis, keepdims=True)))
+
+
+def var(a, axis=None, keepdims=False):
+    c = subtract(a, mean(a, axis, keepdims=True))
+    return mean(square(c), axis, keepdims)
+
+
+def std(a, axis=None, keepdims=False):
+    return sqrt(var(a, axis, keepdims))
+
+
+def norm(a, axis=None, keepdims=False):
+    """``jnp.linalg.norm`` (2-norm of a vector / Frobenius norm over ``axis``)."""
+    return sqrt(sum(square(a), axis, keepdims))
+
+
+def vdot(a, b):
+    """``jnp.vdot`` on real data: both arguments flattened, one number."""
+    n = int(np.prod(_shape(a), dtype=int))
+    return sum(multiply(reshape(a, (n,)), reshape(b, (n,))))
+
+
+def inner(a, b):
+    return tensordot(a, b, axes=((-1,), (-1,)))
+
+
+def outer(a, b):
+    na, nb = int(np.prod(_shape(a), dtype=int)), int(np.prod(_shape(b), dtype=int))
+    return multiply(reshape(a, (na, 1)), reshape(b, (1, nb)))
+
+
+def tensordot(a, b, axes=2):
+    """``jnp.tensordot``: a ``dot_general`` without batch axes."""
+    nda, ndb = len(_shape(a)), len(_shape(b))
+    if isinstance(axes, int):
+        ca, cb = tuple(range(nda - axes, nda)), tuple(range(axes))
+    else:
+        ca, cb = axes
+        ca = (ca,) if isinstance(ca, int) else tuple(ca)
+        cb = (cb,) if isinstance(cb, int) else tuple(cb)
+    return dot_general(a, b, ((tuple(i % nda for i in ca), tuple(i % ndb for i in cb)), ((), ())))
+
+
+def moveaxis(a, source, destination):
+    nd = len(_shape(a))
+    src = [s % nd for s in ((source,) if isinstance(source, int) else source)]
+    dst = [d % nd for d in ((destination,) if isinstance(destination, int) else destination)]
+    order = [i for i in range(nd) if i not in src]
+    for d, s_ in sorted(zip(dst, src)):
+        order.insert(d, s_)
+    return transpose(a, order)
+
+
+def take(a, indices, axis=None):
+    """``jnp.take`` with static integer indices (out-of-range entries are an error, as under ``mode='raise'``)."""
+    idx = np.asarray(indices)
+    if axis is None:
+        return getitem(reshape(a, (int(np.prod(_shape(a), dtype=int)),)), idx)
+    axis = axis % len(_shape(a))
+    return getitem(a, (*([slice(None)] * axis), idx))
+
+
+def diagonal(a, offset=0):
+    """Diagonal of the last two axes, as a new last axis (``jnp.diagonal(a, offset, -2, -1)``)."""
+    n, m = _shape(a)[-2:]
+    i = np.arange(max(min(n + min(offset, 0), m - max(offset, 0)), 0))
+    nd = len(_shape(a))
+    return getitem(a, (*([slice(None)] * (nd - 2)), i - min(offset, 0), i + max(offset, 0)))
+
+
+def trace(a, offset=0):
+    return sum(diagonal(a, offset), axis=-1)
+
+
+def roll(a, shift, axis):
+    n = _shape(a)[axis]
+    return take(a, (np.arange(n) - int(shift)) % n, axis)
+
+
+def repeat(a, repeats, axis):
+    return take(a, np.repeat(np.arange(_shape(a)[axis]), int(repeats)), axis)
+
+
+def zeros_like(a):
+    return np.zeros(tuple(_shape(a)), dtype=np.float32)
+
+
+def ones_like(a):
+    return np.ones(tuple(_shape(a)), dtype=np.float32)
+
+
+erfinv, gammaln = erf_inv, lgamma   # (jnp.max / jnp.min along one axis are amax / amin: the builtins keep their names here)
+
+
 # primitive names of jax.lax (folx/wrapped_functions.py:376-399, :468-513)
 register_function('clamp', lambda args, kw, thr: _composed(lambda lo, x, hi: clip(x, lo, hi))(args, kw, thr))
 register_function('select_n', lambda args, kw, thr: _composed(lambda c, b, a: where(c, a, b))(args, kw, thr))

@@ -826,3 +826,97 @@ def cummax(a: OArr, axis=-1):
 
 def cummin(a: OArr, axis=-1):
     return _cumarg(a, axis, amin)
+
+
+# jax.numpy / jax.nn names that the reference traces into chains of primitives -----------------------
+def _fields(a: OArr, fn):
+    """The same array surgery on the three fields; ``fn(t, lead)`` sees ``lead`` leading non-logical axes."""
+    return OArr(fn(a.x, 1), fn(a.J, 2), fn(a.lap, 1))
+
+
+def relu(a):
+    return maximum(a, 0.0)
+
+
+def leaky_relu(a, negative_slope=0.01):
+    return where(greater_equal(a, 0.0), a, multiply(a, float(negative_slope)))
+
+
+def elu(a, alpha=1.0):
+    return where(greater(a, 0.0), a, multiply(expm1(minimum(a, 0.0)), float(alpha)))
+
+
+def gelu(a, approximate=True):
+    if approximate:
+        u = multiply(add(a, multiply(integer_pow(a, 3), 0.044715)), float(np.sqrt(2.0 / np.pi)))
+        return multiply(multiply(a, 0.5), add(tanh(u), 1.0))
+    return multiply(multiply(a, 0.5), add(erf(multiply(a, float(1.0 / np.sqrt(2.0)))), 1.0))
+
+
+def log_softmax(a, axis=-1):
+    val, _ = logsumexp(a, axis)
+    return subtract(a, expand_dims(val, axis))
+
+
+def var(a, axis=None, keepdims=False):
+    m2 = mean(square(a), axis, keepdims)
+    return subtract(m2, square(mean(a, axis, keepdims)))
+
+
+def std(a, axis=None, keepdims=False):
+    return sqrt(var(a, axis, keepdims))
+
+
+def norm(a, axis=None, keepdims=False):
+    return sqrt(sum(square(a), axis, keepdims))
+
+
+def vdot(a, b):
+    return sum(multiply(reshape(a, (-1,)) if _is(a) else np.reshape(a, -1), reshape(b, (-1,)) if _is(b) else np.reshape(b, -1)))
+
+
+def tensordot(a, b, axes=2):
+    nda = a.ndim if _is(a) else np.ndim(a)
+    ndb = b.ndim if _is(b) else np.ndim(b)
+    if isinstance(axes, int):
+        ca, cb = tuple(range(nda - axes, nda)), tuple(range(axes))
+    else:
+        ca, cb = [(v,) if isinstance(v, int) else tuple(v) for v in axes]
+    return dot_general(a, b, ((tuple(i % nda for i in ca), tuple(i % ndb for i in cb)), ((), ())))
+
+
+def inner(a, b):
+    return tensordot(a, b, axes=((-1,), (-1,)))
+
+
+def outer(a, b):
+    return multiply(reshape(a, (-1, 1)), reshape(b, (1, -1)))
+
+
+def moveaxis(a: OArr, source, destination):
+    src = (source,) if isinstance(source, int) else tuple(source)
+    dst = (destination,) if isinstance(destination, int) else tuple(destination)
+    return _fields(a, lambda t, lead: np.moveaxis(t, [s % a.ndim + lead for s in src], [d % a.ndim + lead for d in dst]))
+
+
+def take(a: OArr, indices, axis=None):
+    idx = np.asarray(indices)
+    if axis is None:
+        return _fields(reshape(a, (-1,)), lambda t, lead: np.take(t, idx, axis=lead))
+    return _fields(a, lambda t, lead: np.take(t, idx, axis=axis % a.ndim + lead))
+
+
+def diagonal(a: OArr, offset=0):
+    return _fields(a, lambda t, lead: np.diagonal(t, offset, -2, -1))
+
+
+def trace(a: OArr, offset=0):
+    return _fields(a, lambda t, lead: np.trace(t, offset, -2, -1))
+
+
+def roll(a: OArr, shift, axis):
+    return _fields(a, lambda t, lead: np.roll(t, shift, axis % a.ndim + lead))
+
+
+def repeat(a: OArr, repeats, axis):
+    return _fields(a, lambda t, lead: np.repeat(t, repeats, axis % a.ndim + lead))

@@ -312,6 +312,30 @@ class plain:
             out.append(pv.reshape(()) if any(v is None for v in src) else a[tuple(src)])
         return torch.stack(out).reshape(sizes)
 
+    relu = staticmethod(torch.relu)
+    leaky_relu = staticmethod(lambda a, negative_slope=0.01: torch.nn.functional.leaky_relu(a, negative_slope))
+    elu = staticmethod(lambda a, alpha=1.0: torch.nn.functional.elu(a, alpha))
+    gelu = staticmethod(lambda a, approximate=True: torch.nn.functional.gelu(a, approximate='tanh' if approximate else 'none'))
+    log_softmax = staticmethod(lambda a, axis=-1: torch.log_softmax(a, dim=axis))
+    var = staticmethod(lambda a, axis=None, keepdims=False: torch.var(a, dim=axis, unbiased=False, keepdim=keepdims))
+    std = staticmethod(lambda a, axis=None, keepdims=False: torch.std(a, dim=axis, unbiased=False, keepdim=keepdims))
+    norm = staticmethod(lambda a, axis=None, keepdims=False: torch.linalg.vector_norm(a, dim=axis, keepdim=keepdims))
+    vdot = staticmethod(lambda a, b: torch.dot(plain._c(a, b).reshape(-1) if not torch.is_tensor(a) else a.reshape(-1),
+                                               plain._c(b, a).reshape(-1) if not torch.is_tensor(b) else b.reshape(-1)))
+    tensordot = staticmethod(lambda a, b, axes=2: torch.tensordot(
+        a if torch.is_tensor(a) else plain._c(a, b), b if torch.is_tensor(b) else plain._c(b, a),
+        dims=axes if isinstance(axes, int) else [list((v,) if isinstance(v, int) else v) for v in axes]))
+    inner = staticmethod(lambda a, b: torch.inner(a if torch.is_tensor(a) else plain._c(a, b), b if torch.is_tensor(b) else plain._c(b, a)))
+    outer = staticmethod(lambda a, b: torch.outer(a.reshape(-1), b.reshape(-1)))
+    moveaxis = staticmethod(torch.movedim)
+    take = staticmethod(lambda a, indices, axis=None: torch.take(a, torch.as_tensor(np.asarray(indices))) if axis is None
+                        else torch.index_select(a, axis, torch.as_tensor(np.asarray(indices)).reshape(-1)).reshape(
+                            *a.shape[:axis % a.ndim], *np.shape(indices), *a.shape[axis % a.ndim + 1:]))
+    diagonal = staticmethod(lambda a, offset=0: torch.diagonal(a, offset, -2, -1))
+    trace = staticmethod(lambda a, offset=0: torch.diagonal(a, offset, -2, -1).sum(-1))
+    roll = staticmethod(lambda a, shift, axis: torch.roll(a, shift, axis))
+    repeat = staticmethod(lambda a, repeats, axis: torch.repeat_interleave(a, repeats, dim=axis))
+
     arctan2 = staticmethod(lambda y, x: torch.atan2(y if torch.is_tensor(y) else plain._c(y, x), plain._c(x, y) if torch.is_tensor(y) else x))
     remainder = staticmethod(lambda a, b: torch.fmod(a, plain._c(b, a)))
     fmod = remainder

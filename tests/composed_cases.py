@@ -67,6 +67,27 @@ CASES = {
                                                        xp.square(xp.reshape(_g(xp, x, slice(11, 12)), ())), ((2, 1, 1),)),
     'lax_pad_negative': lambda xp, x: xp.lax_pad(xp.multiply(xp.sin(x), x), 0.0, ((-1, -2, 0),)),
     'lax_pad_negative_interior': lambda xp, x: xp.lax_pad(xp.reshape(xp.cos(x), (3, 4)), -1.5, ((-1, 2, 2), (1, -3, 1))),
+    # jax.numpy / jax.nn names that the reference reaches through its tracer (test/test_layers.py:695-716 uses the erf
+    # form of gelu); here they are compositions of the rules
+    'activations_by_name': lambda xp, x: xp.add(
+        xp.add(xp.gelu(_g(xp, x, slice(0, 4)), approximate=False), xp.gelu(_g(xp, x, slice(4, 8)))),
+        xp.add(xp.elu(xp.multiply(_g(xp, x, slice(8, 12)), 2.0), 1.3),
+               xp.add(xp.relu(xp.sin(xp.multiply(_g(xp, x, slice(0, 4)), 3.0))), xp.leaky_relu(_g(xp, x, slice(4, 8)), 0.2)))),
+    'log_softmax_var_std': lambda xp, x: xp.add(
+        xp.sum(xp.log_softmax(xp.reshape(xp.sin(x), (3, 4)), axis=-1), axis=0),
+        xp.add(xp.var(xp.reshape(xp.tanh(x), (3, 4)), axis=0),
+               xp.reshape(xp.std(xp.reshape(xp.multiply(x, x), (4, 3)), axis=-1, keepdims=True), (4,)))),
+    'norm_vdot_outer': lambda xp, x: xp.multiply(
+        xp.outer(xp.sin(_g(xp, x, slice(0, 3))), xp.tanh(_g(xp, x, slice(3, 7)))),
+        xp.add(xp.norm(xp.reshape(x, (3, 4)), axis=0), xp.vdot(xp.cos(x), xp.reshape(xp.square(x), (3, 4))))),
+    'tensordot_inner': lambda xp, x: xp.add(
+        xp.tensordot(xp.reshape(xp.sin(x), (2, 3, 2)), xp.reshape(xp.tanh(x), (3, 2, 2)), axes=2),
+        xp.inner(xp.reshape(xp.cos(x), (2, 6)), np.linspace(-1.0, 1.0, 12, dtype=np.float32).reshape(2, 6))),
+    'moveaxis_take_roll_repeat': lambda xp, x: xp.add(
+        xp.take(xp.moveaxis(xp.reshape(xp.sin(x), (2, 3, 2)), 0, -1), np.array([[2, 0], [1, 1]]), axis=0),
+        xp.reshape(xp.take(xp.roll(xp.repeat(xp.tanh(x), 2, axis=0), 5, axis=0), np.arange(0, 24, 3)), (2, 2, 2))),
+    'diagonal_trace': lambda xp, x: xp.add(
+        xp.diagonal(xp.reshape(xp.sin(x), (3, 2, 2))), xp.reshape(xp.trace(xp.reshape(xp.multiply(x, x), (3, 2, 2)), offset=1), (3, 1))),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }
