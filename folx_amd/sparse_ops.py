@@ -68,8 +68,10 @@ _MAX_TABLE_ENTRIES = 1 << 27  # beyond this the scatter-add kernel is used inste
 
 
 def _key(arr: np.ndarray, *extra):
-    a = np.ascontiguousarray(arr)
-    return (hashlib.blake2b(a.tobytes(), digest_size=16).digest(), a.shape, str(a.dtype), *extra)
+    a = np.asarray(arr)
+    # the shape is the ARGUMENT's: numpy.ascontiguousarray turns a 0-d array into shape (1,), and a scalar constant
+    # must not share its entry with a one-element vector of the same value
+    return (hashlib.blake2b(np.ascontiguousarray(a).tobytes(), digest_size=16).digest(), a.shape, str(a.dtype), *extra)
 
 
 def device_table(arr: np.ndarray, device) -> torch.Tensor:

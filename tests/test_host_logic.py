@@ -249,6 +249,20 @@ def test_batched_vmap_uneven_multiple_arguments_and_nested():
             np.broadcast_to(a[None], (7, 10, 3)).copy(), b)
 
 
+def test_constant_cache_keeps_scalars_and_one_element_vectors_apart():
+    """Constants are cached by content AND shape: a scalar 0.0 and ``zeros(1)`` have the same bytes (and
+    ``numpy.ascontiguousarray`` gives both the shape (1,)), but not the same entry."""
+    from folx_amd import sparse_ops as so
+
+    so.clear_caches()
+    cpu = torch.device('cpu')
+    s = so.device_const(np.float32(0.25), cpu)
+    v = so.device_const(np.full((1,), 0.25, dtype=np.float32), cpu)
+    m = so.device_const(np.full((1, 1), 0.25, dtype=np.float32), cpu)
+    assert tuple(s.shape) == () and tuple(v.shape) == (1,) and tuple(m.shape) == (1, 1)
+    assert so.device_const(np.float32(0.25), cpu) is s and so.device_const(np.full((1,), 0.25, dtype=np.float32), cpu) is v
+
+
 def test_register_function_plugs_in():
     calls = []
 
