@@ -313,15 +313,10 @@ def matmul(a, b):
     return _tr(y, [order.index(t) for t in want])
 
 
-def einsum(subscripts: str, a, b):
-    """Two-operand ``numpy.einsum`` (explicit ``->`` form, no repeated index inside an operand, no
-    ellipsis) as one ``dot_general``: indices shared by both operands and the output are batch
-    axes, shared ones missing from the output are contracted, the others are the free axes of
-    their operand -- the dimension numbers ``jnp.einsum`` hands to ``dot_general``
-    (folx/wrapped_functions.py:174-309)."""
-    ins, out = subscripts.replace(' ', '').split('->')
-    sa, sb = ins.split(',')
-    assert len(set(sa)) == len(sa) and len(set(sb)) == len(sb) and '.' not in subscripts, subscripts
+def _einsum_pair(sa: str, sb: str, out: str, a, b):
+    """One two-operand contraction as one ``dot_general``: indices shared by both operands and the output are
+    batch axes, shared ones missing from the output are contracted, the others are the free axes of their
+    operand -- the dimension numbers ``jnp.einsum`` hands to ``dot_general`` (folx/wrapped_functions.py:174-309)."""
     for idx, t in ((sa, a), (sb, b)):  # indices of one operand only that the output drops are summed first
         drop = [i for i, c in enumerate(idx) if c not in out and c not in (sb if idx is sa else sa)]
         if drop:
@@ -340,6 +335,40 @@ def einsum(subscripts: str, a, b):
     y = dot_general(a, b, dn)
     cur = batch + fa + fb
     return _tr(y, [cur.index(c) for c in out])
+
+
+def einsum(subscripts: str, *operands):
+    """``numpy.einsum`` for any number of operands, with or without ``->`` and with ``...`` (an ellipsis stands for
+    the same leading axes in every operand that has it): operands are contracted pairwise from the left, as
+    ``jnp.einsum`` lowers them to a chain of ``dot_general`` (test/test_layers.py:255-262 uses
+    ``'...i,...j,...ijk->...k'``).  No repeated index inside one operand."""
+    spec = subscripts.replace(' ', '')
+    ins, arrow, out = spec.partition('->')
+    terms = ins.split(',')
+    assert len(terms) == len(operands), f'einsum: {len(terms)} terms for {len(operands)} operands'
+    ranks = [len(_shape(t)) for t in operands]
+    n_ell = [r - (len(t) - 3) if '...' in t else 0 for t, r in zip(terms, ranks)]
+    pool = [c for c in 'ABCDEFGHIJKLMNOPQRSTUVWXYZ' if c not in spec]
+    width = max(n_ell) if n_ell else 0
+    ell = ''.join(pool[:width])
+    terms = [t.replace('...', ell[width - n:] if n else '') for t, n in zip(terms, n_ell)]
+    if arrow:
+        out = out.replace('...', ell)
+    else:           # implicit form: the ellipsis axes, then every index that appears exactly once, in alphabetical order
+        joined = ''.join(terms)
+        out = ell + ''.join(sorted(c for c in set(joined) if joined.count(c) == 1 and c not in ell))
+    for t, r in zip(terms, ranks):
+        assert len(t) == r and len(set(t)) == len(t), f'einsum: term {t!r} for an operand of rank {r}'
+    cur, scur = operands[0], terms[0]
+    for k in range(1, len(operands)):
+        later = set(out).union(*terms[k + 1:]) if k + 1 < len(terms) else set(out)
+        mid = ''.join(dict.fromkeys(c for c in scur + terms[k] if c in later))
+        cur, scur = _einsum_pair(scur, terms[k], mid, cur, operands[k]), mid
+    drop = tuple(i for i, c in enumerate(scur) if c not in out)
+    if drop:
+        cur = sum(cur, axis=drop) if _is_triplet(cur) else np.sum(np.asarray(cur), axis=drop)
+        scur = ''.join(c for c in scur if c in out)
+    return _tr(cur, [scur.index(c) for c in out])
 
 
 def softmax(a, axis=-1):

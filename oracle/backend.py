@@ -11,6 +11,7 @@ logical shape ``s``.  Every op applies the rule from ``oracle.rules``.
 from __future__ import annotations
 
 import numpy as np
+from builtins import sum as builtins_sum
 
 from . import rules
 
@@ -568,21 +569,52 @@ def matmul(a, b):
     return einsum(f'{sa_},{sb_}->{out}', a, b)
 
 
-def einsum(subscripts, a, b):
-    """Two-operand einsum of triplets, evaluated directly: linear in each operand, Hessian term
-    2 sum_p einsum(Ja_p, Jb_p) (folx/hessian.py:177-188)."""
-    ins, out = subscripts.replace(' ', '').split('->')
-    sa, sb = ins.split(',')
-    if not _is(a) or not _is(b):
-        t, c, tfirst = (a, np.asarray(b), True) if _is(a) else (b, np.asarray(a), False)
-        st, sc = (sa, sb) if tfirst else (sb, sa)
-        f = lambda v, lead: np.einsum(f'{lead}{st},{sc}->{lead}{out}', v, c)
-        return OArr(f(t.x, 'Z'), f(t.J, 'YZ'), f(t.lap, 'Z'))
-    Ja, Jb = _padJ(a, b)
-    e = lambda u, lu, v, lv, lo: np.einsum(f'{lu}{sa},{lv}{sb}->{lo}{out}', u, v)
-    x = e(a.x, 'Z', b.x, 'Z', 'Z')
-    J = e(Ja, 'YZ', b.x, 'Z', 'YZ') + e(a.x, 'Z', Jb, 'YZ', 'YZ')
-    lap = e(a.lap, 'Z', b.x, 'Z', 'Z') + e(a.x, 'Z', b.lap, 'Z', 'Z') + 2.0 * e(Ja, 'YZ', Jb, 'YZ', 'Z')
+def _einsum_terms(subscripts, ranks):
+    """Ellipsis and implicit-output forms of numpy.einsum written out with explicit letters."""
+    spec = subscripts.replace(' ', '')
+    ins, arrow, out = spec.partition('->')
+    terms = ins.split(',')
+    n_ell = [r - (len(t) - 3) if '...' in t else 0 for t, r in zip(terms, ranks)]
+    width = max(n_ell) if n_ell else 0
+    ell = ''.join([c for c in 'ABCDEFGHIJKLMNOPQRSTUVWX' if c not in spec][:width])
+    terms = [t.replace('...', ell[width - n:] if n else '') for t, n in zip(terms, n_ell)]
+    if arrow:
+        out = out.replace('...', ell)
+    else:
+        joined = ''.join(terms)
+        out = ell + ''.join(sorted(c for c in set(joined) if joined.count(c) == 1 and c not in ell))
+    return terms, out
+
+
+def einsum(subscripts, *ops):
+    """einsum of any number of triplets and constants, evaluated directly: the function is linear in every operand,
+    so J = sum_k f(.., J_k, ..), lap = sum_k f(.., lap_k, ..) + 2 sum_{k<l} sum_p f(.., J_k,p, .., J_l,p, ..)
+    (folx/hessian.py:177-188 for two operands)."""
+    terms, out = _einsum_terms(subscripts, [o.ndim if _is(o) else np.ndim(o) for o in ops])
+    trip = [k for k, o in enumerate(ops) if _is(o)]
+    assert trip, 'einsum: no triplet among the operands'
+    P = max(ops[k].P for k in trip)
+    padJ = {k: np.concatenate([ops[k].J, np.zeros((P - ops[k].P, *ops[k].J.shape[1:]), ops[k].J.dtype)], 0) for k in trip}
+
+    def ev(subst, lead_out):          # subst: {operand index: (array, leading letters)}; the others contribute their value
+        arrs, subs = [], []
+        for k, (o, t) in enumerate(zip(ops, terms)):
+            if k in subst:
+                arr, lead = subst[k]
+            elif _is(o):
+                arr, lead = o.x, 'Z'
+            else:
+                arr, lead = np.asarray(o), ''
+            arrs.append(arr)
+            subs.append(lead + t)
+        return np.einsum(','.join(subs) + '->' + lead_out + out, *arrs)
+
+    x = ev({}, 'Z')
+    J = builtins_sum(ev({k: (padJ[k], 'YZ')}, 'YZ') for k in trip)
+    lap = builtins_sum(ev({k: (ops[k].lap, 'Z')}, 'Z') for k in trip)
+    for a_, k in enumerate(trip):
+        for l in trip[a_ + 1:]:
+            lap = lap + 2.0 * ev({k: (padJ[k], 'YZ'), l: (padJ[l], 'YZ')}, 'Z')
     return OArr(x, J, lap)
 
 

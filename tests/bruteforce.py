@@ -170,9 +170,9 @@ class plain:
         return a @ b
 
     @staticmethod
-    def einsum(subscripts, a, b):
-        a, b = plain._b(a, b)
-        return torch.einsum(subscripts, a, b)
+    def einsum(subscripts, *ops):
+        like = [o for o in ops if torch.is_tensor(o)][0]
+        return torch.einsum(subscripts, *[o if torch.is_tensor(o) else plain._c(o, like) for o in ops])
 
     @staticmethod
     def dot_general(lhs, rhs, dimension_numbers):

@@ -10,6 +10,11 @@ _OFFS = ((0.37 * np.arange(72)) % 2.9).astype(np.float32)
 _SPREAD = np.random.default_rng(72).uniform(-2.0, 2.0, size=72).astype(np.float32)
 
 
+_W1 = np.cos(np.arange(32, dtype=np.float32)).reshape(4, 8)
+_W2 = np.sin(0.7 * np.arange(128, dtype=np.float32)).reshape(4, 4, 8)
+_W3 = np.cos(1.3 * np.arange(16, dtype=np.float32)).reshape(4, 4)
+
+
 def _g(xp, x, sl):
     return xp.getitem(x, (sl,))
 
@@ -88,6 +93,14 @@ CASES = {
         xp.reshape(xp.take(xp.roll(xp.repeat(xp.tanh(x), 2, axis=0), 5, axis=0), np.arange(0, 24, 3)), (2, 2, 2))),
     'diagonal_trace': lambda xp, x: xp.add(
         xp.diagonal(xp.reshape(xp.sin(x), (3, 2, 2))), xp.reshape(xp.trace(xp.reshape(xp.multiply(x, x), (3, 2, 2)), offset=1), (3, 1))),
+    # einsum with three operands, an ellipsis and the implicit output form (test/test_layers.py:255-262:
+    # dot(x, w1) + einsum('...i,...j,...ijk->...k', x, x, w2)); constants and triplets mixed
+    'einsum_three_operands': lambda xp, x: xp.add(
+        xp.dot(xp.reshape(x, (3, 4)), _W1),
+        xp.einsum('...i,...j,...ijk->...k', xp.reshape(xp.sin(x), (3, 4)), xp.reshape(x, (3, 4)), _W2)),
+    'einsum_implicit_and_chain': lambda xp, x: xp.add(
+        xp.einsum('ij,jk', xp.reshape(xp.sin(x), (3, 4)), xp.reshape(xp.tanh(x), (4, 3))),
+        xp.einsum('ai,ij,bj->ab', xp.reshape(xp.cos(x), (3, 4)), _W3, xp.reshape(xp.multiply(x, x), (3, 4)))),
     'inverse_trig': lambda xp, x: xp.add(xp.arcsin(xp.multiply(xp.tanh(x), 0.9)),
                                          xp.arccosh(xp.add(xp.square(x), 1.2))),
 }
