@@ -35,7 +35,8 @@ def generate(seed: int, n_steps: int = 7):
             i = int(rng.integers(1, len(shapes)))
             s = shapes[i]
             kind = rng.choice(['unary', 'binary', 'reshape', 'transpose', 'slice', 'sum', 'dot', 'concat', 'broadcast',
-                               'flip', 'where', 'cumsum', 'amax', 'take', 'binary_const', 'mean_keep', 'pad'])
+                               'flip', 'where', 'cumsum', 'amax', 'take', 'binary_const', 'mean_keep', 'pad',
+                               'matmul_t', 'softmax', 'logsumexp', 'logdet_spd'])
             size = int(np.prod(s, dtype=int))
             if kind == 'unary':
                 steps.append((str(rng.choice(_UNARY)), (i,), ())); shapes.append(s)
@@ -134,6 +135,26 @@ def generate(seed: int, n_steps: int = 7):
                 if min(out) < 1:
                     continue
                 steps.append(('lax_pad', (i,), (float(rng.normal()), cfg))); shapes.append(out)
+            elif kind == 'matmul_t':
+                # product of two derivative-carrying operands: v (..., m, k) times the transposed partner (..., k, m)
+                if len(s) < 2:
+                    continue
+                cands = [j for j in range(1, len(shapes)) if shapes[j] == s]
+                j = int(rng.choice(cands))
+                steps.append(('matmul_t', (i, j), ())); shapes.append((*s[:-1], s[-2]))
+            elif kind == 'softmax':
+                if not s or s[-1] < 2:
+                    continue
+                steps.append(('softmax', (i,), ())); shapes.append(s)
+            elif kind == 'logsumexp':
+                if not s or s[-1] < 2:
+                    continue
+                steps.append(('logsumexp', (i,), ())); shapes.append(s[:-1])
+            elif kind == 'logdet_spd':
+                # log det (v v^T + 2 I): symmetric positive definite, eigenvalues >= 2
+                if len(s) < 2 or s[-2] > 6:
+                    continue
+                steps.append(('logdet_spd', (i,), ())); shapes.append(s[:-2])
             if int(np.prod(shapes[-1], dtype=int)) > 400:     # keep the values small
                 steps.pop(); shapes.pop()
                 continue
@@ -178,10 +199,23 @@ def run(steps, xp, x):
             v = xp.take(a[0], static[0], axis=static[1])
         elif op == 'lax_pad':
             v = xp.lax_pad(a[0], static[0], static[1])
+        elif op == 'matmul_t':
+            v = xp.matmul(a[0], xp.swapaxes(xp.tanh(a[1]), -1, -2))
+        elif op == 'softmax':
+            v = xp.softmax(xp.tanh(a[0]), axis=-1)
+        elif op == 'logsumexp':
+            v = xp.logsumexp(xp.tanh(a[0]), axis=-1)[0]
+        elif op == 'logdet_spd':
+            t = xp.tanh(a[0])
+            m = t.shape[-2]
+            v = xp.slogdet(xp.add(xp.matmul(t, xp.swapaxes(t, -1, -2)), 2.0 * np.eye(m, dtype=np.float32)))[1]
         else:
             raise KeyError(op)
         vals.append(v)
     return vals[-1]
+
+
+USES_DETERMINANT = lambda steps: any(op == 'logdet_spd' for op, _, _ in steps)
 
 
 def describe(steps):
