@@ -23,13 +23,14 @@ def _factorizations(n):
     return out
 
 
-def generate(seed: int, n_steps: int = 7):
+def generate(seed: int, n_steps: int = 7, n_in: int = N_IN):
     """Returns a list of steps ``(op, operand indices, static arguments)``; shapes are tracked while drawing
-    so that every step is valid.  Value 0 is the input reshaped."""
+    so that every step is valid.  Value 0 is the input (``n_in`` entries), value 1 the input reshaped."""
     rng = np.random.default_rng(seed)
-    first = _SHAPES[rng.integers(len(_SHAPES))]
+    first_shapes = _SHAPES if n_in == N_IN else _factorizations(n_in)
+    first = first_shapes[rng.integers(len(first_shapes))]
     steps = [('reshape', (0,), (first,))]
-    shapes = [(N_IN,), first]          # value 0: the raw input; value 1: reshaped
+    shapes = [(n_in,), first]          # value 0: the raw input; value 1: reshaped
     for _ in range(n_steps):
         for _attempt in range(20):
             i = int(rng.integers(1, len(shapes)))
@@ -155,7 +156,7 @@ def generate(seed: int, n_steps: int = 7):
                 if len(s) < 2 or s[-2] > 6:
                     continue
                 steps.append(('logdet_spd', (i,), ())); shapes.append(s[:-2])
-            if int(np.prod(shapes[-1], dtype=int)) > 400:     # keep the values small
+            if int(np.prod(shapes[-1], dtype=int)) > 400 * max(n_in // N_IN, 1):     # keep the values small
                 steps.pop(); shapes.pop()
                 continue
             break
