@@ -74,3 +74,22 @@ def test_hip_path_against_the_oracle(block):
             print(f'random program seed {seed} thr {thr}: {rp.describe(steps)}', flush=True)
             out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: rp.run(steps, fnp, t), thr))(torch.as_tensor(x).cuda())
             _compare(out, ref, f'seed {seed} thr {thr}: {rp.describe(steps)}')
+
+
+@pytest.mark.gpu
+def test_graph_replay_of_random_programs_equals_eager_bit_for_bit():
+    """``folx_amd.jit``: the first call runs eagerly, the second is captured, later ones replay; every call returns the
+    bits of the eager run on the same input (fresh inputs per call)."""
+    for seed in range(24):
+        steps = rp.generate(seed, 8, 64 if seed % 3 == 0 else rp.N_IN)
+        n_in = 64 if seed % 3 == 0 else rp.N_IN
+        thr = (0, 3, 12)[seed % 3]
+        print(f'graph replay, random program seed {seed} thr {thr}: {rp.describe(steps)}', flush=True)
+        eager = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: rp.run(steps, fnp, t), thr))
+        fast = folx_amd.jit(folx_amd.vmap(folx_amd.forward_laplacian(lambda t: rp.run(steps, fnp, t), thr)))
+        for call in range(4):
+            x = torch.as_tensor(np.random.default_rng(7000 + seed + call).normal(size=(4, n_in)).astype(np.float32)).cuda()
+            a, b = eager(x), fast(x)
+            torch.cuda.synchronize()
+            assert torch.equal(a.x, b.x) and torch.equal(a.laplacian, b.laplacian), f'seed {seed} call {call}'
+            assert torch.equal(a.jacobian.dense_array, b.jacobian.dense_array), f'seed {seed} call {call}'
