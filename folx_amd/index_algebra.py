@@ -23,12 +23,26 @@ _MEMO_MAX = 1024
 
 
 def _freeze(v):
+    """Results of the memoized functions are values: read-only, and so is the memory they are views of (masks
+    are never written in place anywhere in this package)."""
     if isinstance(v, np.ndarray):
-        v.flags.writeable = False
+        b = v
+        while isinstance(b, np.ndarray):
+            b.flags.writeable = False
+            b = b.base
     elif isinstance(v, tuple):
         for t in v:
             _freeze(t)
     return v
+
+
+def _stable(v: np.ndarray) -> bool:
+    """Nobody can write to the memory of ``v``: the array and everything it is a view of are read-only."""
+    while isinstance(v, np.ndarray):
+        if v.flags.writeable:
+            return False
+        v = v.base
+    return v is None
 
 
 def _key_of(v):
@@ -41,18 +55,56 @@ def _key_of(v):
     return v
 
 
+_BY_IDENTITY: dict = {}
+
+
+def _identity_key(args):
+    """Key of an argument list by the MEMORY of its read-only arrays (address, shape, strides, type: two views of
+    one cached mask with the same layout are the same value), or None when some array could still be written to
+    (its address says nothing about its contents then) or an argument has no cheap key."""
+    key = []
+    for v in args:
+        if isinstance(v, np.ndarray):
+            if not _stable(v):
+                return None
+            key.append(('m', v.__array_interface__['data'][0], v.shape, v.strides, v.dtype.str))
+        elif isinstance(v, (list, tuple)):
+            sub = _identity_key(v)
+            if sub is None:
+                return None
+            key.append(sub)
+        elif v is None or isinstance(v, (bool, int, float, str, np.generic)):
+            key.append(v.item() if isinstance(v, np.generic) else v)
+        else:
+            return None
+    return tuple(key)
+
+
 def _memo(fn):
-    """Keeps results of a pure function of integer arrays and plain values by content."""
+    """Keeps results of a pure function of integer arrays and plain values by content.  Results are read-only
+    arrays that the next rule receives as they are, so from the second evaluation of a model on its masks ARE the
+    cached objects or views of them: a first look-up by the memory of read-only arguments (an entry keeps its arguments
+    alive, so an address cannot be reused while it is a key) saves building and hashing a key of the contents."""
     import functools
 
     @functools.wraps(fn)
     def wrapped(*args):
+        ikey = _identity_key(args)
+        if ikey is not None:
+            hit = _BY_IDENTITY.get((fn.__name__, ikey))
+            if hit is not None:
+                return hit[1]
         key = (fn.__name__, _key_of(args))
         hit = _MEMO.get(key)
         if hit is None:
             if len(_MEMO) >= _MEMO_MAX:
                 _MEMO.clear()
+                _BY_IDENTITY.clear()
             hit = _MEMO[key] = _freeze(fn(*args))
+        if ikey is not None:
+            if len(_BY_IDENTITY) >= 4 * _MEMO_MAX:
+                _BY_IDENTITY.clear()
+            _BY_IDENTITY[(fn.__name__, ikey)] = (args, hit)
         return hit
 
     return wrapped
@@ -63,10 +115,16 @@ def _memo(fn):
 # --------------------------------------------------------------------------------------
 
 
-def init_mask(shape) -> np.ndarray:
-    """Initial sparse mask: one row, entry i <- flat input i (folx/interpreter.py:283-293)."""
+def init_mask(shape, offset: int = 0) -> np.ndarray:
+    """Initial sparse mask: one row, entry i <- flat input ``offset + i`` (folx/interpreter.py:283-293).  The same
+    read-only array for the same shape, so that everything derived from it is found by identity."""
+    return _init_mask(tuple(int(n) for n in shape), int(offset))
+
+
+@_memo
+def _init_mask(shape, offset):
     n = int(np.prod(shape, dtype=int))
-    return np.arange(n, dtype=np.int32).reshape(1, *shape)
+    return (np.arange(n, dtype=np.int32) + np.int32(offset)).reshape(1, *shape)
 
 
 @_memo
@@ -285,6 +343,7 @@ def find_out_idx(masks, x_shapes, in_axes, linear_in_one: bool, threshold: int):
     return idx, dense_out
 
 
+@_memo
 def dot_projection(mask: np.ndarray, contract_axis: int, threshold: int):
     """Mask of ``h @ W`` for sparse ``h`` with one contracted axis
     (folx/wrapped_functions.py:113-157).  Returns ``(proj, aligned)``: ``proj`` is

@@ -45,7 +45,7 @@ def init_forward_laplacian_state(x: torch.Tensor, sparsity: bool, weights=None, 
     lap = so.zeros(x.shape, dev)
     if sparsity:
         data = so.device_const(np.ascontiguousarray(w), dev).reshape(1, 1, *shape).expand(1, B, *shape).contiguous()
-        return FwdLaplArray(x, FwdJacobian(data, ia.init_mask(shape) + np.int32(offset)), lap)
+        return FwdLaplArray(x, FwdJacobian(data, ia.init_mask(shape, offset)), lap)
     eye = np.zeros((total, n), dtype=np.float32)
     eye[offset:offset + n] = np.eye(n, dtype=np.float32) * w.reshape(-1)
     data = so.device_const(eye.reshape(total, 1, *shape), dev).expand(total, B, *shape).contiguous()

@@ -114,6 +114,7 @@ def clear_caches():
     _CONST_CACHE.clear()
     _ROWS_CACHE.clear()
     index_algebra._MEMO.clear()
+    index_algebra._BY_IDENTITY.clear()
 
 
 def zeros(shape, device) -> torch.Tensor:
