@@ -13,6 +13,7 @@ with ``torch.func``, since nothing else defines its derivatives.)
 from .api import BatchedArray, FunctionFlags, FwdJacobian, FwdLaplArray
 from .graph import jit
 from .interpreter import forward_laplacian, init_forward_laplacian_state
+from .fx import forward_laplacian_torch
 from .operators import (
     ForwardLaplacianOperator,
     Laplacian,
