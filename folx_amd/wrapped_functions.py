@@ -572,6 +572,13 @@ def _dot_batched_const(h: FwdLaplArray, W, thr: int) -> FwdLaplArray:
     return FwdLaplArray(y, FwdJacobian(Jy, new_mask), lapy)
 
 
+def _zero_rows_below(W, k_pad: int):
+    """``W`` with ``k_pad`` zero rows appended (the partner of zero feature columns appended to the input)."""
+    if isinstance(W, torch.Tensor):  # a caller-owned device tensor: padded on every call (it may change in place)
+        return torch.cat([W.to(torch.float32), W.new_zeros((k_pad, W.shape[1]), dtype=torch.float32)], dim=0)
+    return np.concatenate([np.asarray(W, dtype=np.float32), np.zeros((k_pad, np.shape(W)[1]), dtype=np.float32)], axis=0)
+
+
 def _dot_then_act(h, W, kwargs, thr: int):
     """``residual + act(layer_norm(h) @ W + bias)`` with ``act`` and ``layer_norm`` optional.
     A Dense + activation layer is ONE rule when the fused kernels take its shape
@@ -617,10 +624,7 @@ def _dot_then_act(h, W, kwargs, thr: int):
         # kernel takes it with the feature axis padded by zero columns against zero rows of W, which costs one
         # copy of the input triplet and saves the pre-activation triplet's trip through memory
         k_pad = -np.shape(W)[0] % 16
-        if isinstance(W, torch.Tensor):  # a caller-owned device tensor: padded on every call (it may change in place)
-            W = torch.cat([W.to(torch.float32), W.new_zeros((k_pad, W.shape[1]), dtype=torch.float32)], dim=0)
-        else:
-            W = np.concatenate([np.asarray(W, dtype=np.float32), np.zeros((k_pad, np.shape(W)[1]), dtype=np.float32)], axis=0)
+        W = _zero_rows_below(W, k_pad)
     K_in = np.shape(W)[0] - k_pad
     fused = (
         _is(h) and not _is(W) and kwargs.get('row_slice') is None and np.ndim(W) == 2
@@ -973,6 +977,15 @@ def _dot_parts(lc: LazyConcat, W, kwargs, thr: int):
               and K.dense_act_supported(act, Ktot, np.shape(W)[1], rows=B * group, P=P))
     if not ok:
         kw = dict(kwargs)
+        Kin = np.shape(W)[0] if np.ndim(W) == 2 else 0
+        if (act is not None and kwargs.get('norm') is None and kwargs.get('row_slice') is None and not _is(W)
+                and np.ndim(W) == 2 and np.shape(W)[1] > 128 and Kin % 16 != 0 and Kin >= 16 and Kin == lc.shape[-1]):
+            # a wide layer over a concatenation whose width is no multiple of 16: the zero columns that the fused
+            # kernel needs (see _dot_then_act) join the concatenation as one more part instead of a second copy
+            k_pad = -Kin % 16
+            zero = np.zeros((*lc.shape[:-1], k_pad), dtype=np.float32)
+            h = concatenate_rule(tuple(force(t) for t in lc.parts) + (zero,), {'dimension': -1}, thr)
+            return dot_general((h, _zero_rows_below(W, k_pad)), kw, thr)
         return dot_general((lc.value(thr), W), kw, thr)
     bias = kwargs.get('bias')
     res = None  # a skip connection with the same dense rows goes into the kernel's epilogue
