@@ -25,6 +25,33 @@ from .interpreter import ForwardLaplacianFn
 
 aten = torch.ops.aten
 
+# Named functions: the reference reaches its attention kernel through the NAME of a jitted function
+# (``register_function('_multi_head_self_attention', ...)``, folx/experimental/pallas/attention/__init__.py:45, looked
+# up by ``eval_pjit``, folx/interpreter.py:186-200).  The torch counterpart is a library operation: while a model is
+# being traced the function below records ONE node, which the graph evaluation hands to the rule registered under the
+# same key; outside a trace it is the plain differentiable arithmetic.
+_LIB = torch.library.Library('folx_amd', 'DEF')
+_LIB.define('multi_head_self_attention(Tensor q, Tensor k, Tensor v) -> Tensor')
+_TRACING = [False]
+
+
+def _mhsa_math(q, k, v):
+    p = torch.softmax(torch.einsum('ihd,jhd->hij', q, k), dim=-1)
+    return torch.einsum('hij,jhd->ihd', p, v)
+
+
+_LIB.impl('multi_head_self_attention', _mhsa_math, 'CompositeExplicitAutograd')
+
+
+def multi_head_self_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """``softmax(q k^T) v`` for per-sample tensors ``(n, heads, d)`` (no ``1 / sqrt(d)`` inside, as in the reference's
+    ``folx.experimental.pallas.attention.multi_head_self_attention``): in a model traced by
+    ``forward_laplacian_torch`` this is one equation and runs on the attention rule's kernel."""
+    if _TRACING[0]:
+        return torch.ops.folx_amd.multi_head_self_attention(q, k, v)
+    return _mhsa_math(q, k, v)
+
+
 
 def _is_t(v):
     from .wrapped_functions import Deferred
@@ -213,6 +240,8 @@ RULES = {
     aten.linalg_inv_ex.default: lambda A, check_errors=False: (fnp.inv(A), None),
     aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
     operator.getitem: lambda a, i: a[i],
+    aten._safe_softmax.default: lambda a, dim, dtype=None: fnp.softmax(a, axis=int(dim)),
+    torch.ops.folx_amd.multi_head_self_attention.default: fnp.multi_head_self_attention,
 }
 
 
@@ -312,7 +341,11 @@ class TracedForwardLaplacian(ForwardLaplacianFn):
 
             with torch.no_grad():
                 examples = [torch.zeros(s, dtype=torch.float32) + 0.5 for s in shapes]
-                gm = self.graphs[shapes] = make_fx(self.torch_fn)(*examples)
+                _TRACING[0] = True
+                try:
+                    gm = self.graphs[shapes] = make_fx(self.torch_fn)(*examples)
+                finally:
+                    _TRACING[0] = False
         return gm
 
     def _run(self, *lapl_args):

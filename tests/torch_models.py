@@ -71,4 +71,29 @@ def indexing_and_piecewise():
     return make, x
 
 
-MODELS = {'readme_mlp': readme_mlp, 'transformer_block': transformer_block, 'indexing_and_piecewise': indexing_and_piecewise}
+def attention_by_name():
+    """Attention through the named function (one equation in the trace, the attention rule's kernel) next to
+    ``scaled_dot_product_attention`` (traced into products and a softmax), both behind linear maps."""
+    from folx_amd.fx import multi_head_self_attention
+
+    n, H, d = 8, 2, 8
+    mods = _module(lambda: nn.ModuleDict(dict(emb=nn.Linear(3, H * d), q=nn.Linear(H * d, H * d), k=nn.Linear(H * d, H * d),
+                                              v=nn.Linear(H * d, H * d), o=nn.Linear(H * d, 4))), 4)
+
+    def make(dt):
+        m = mods[dt]
+
+        def f(x):  # x (n, 3)
+            h = torch.tanh(m['emb'](x))
+            q, k, v = (m[t](h).view(n, H, d) for t in ('q', 'k', 'v'))
+            a = multi_head_self_attention(q * d ** -0.5, k, v).reshape(n, H * d)
+            b = torch.nn.functional.scaled_dot_product_attention(q.permute(1, 0, 2), k.permute(1, 0, 2), v.permute(1, 0, 2))
+            return m['o'](a + b.permute(1, 0, 2).reshape(n, H * d)).sum(dim=0)
+
+        return f
+
+    x = (0.7 * np.random.default_rng(4).normal(size=(2, n, 3))).astype(np.float32)
+    return make, x
+
+
+MODELS = {'attention_by_name': attention_by_name, 'readme_mlp': readme_mlp, 'transformer_block': transformer_block, 'indexing_and_piecewise': indexing_and_piecewise}
