@@ -59,6 +59,10 @@ def parse():
     ap.add_argument('--streaming-rules', action='store_true',
                     help='instead of a workload: launch every HBM-bound rule at its largest workload shape (ten launches '
                          'each, HIP events) and print one JSON line of achieved TB/s; the command profiles/ traces')
+    ap.add_argument('--front-door', choices=('calls', 'torch'), default='calls',
+                    help="'torch': the workload's model as plain torch code, traced with torch.fx and evaluated through "
+                         'the same rules (folx_amd.forward_laplacian_torch); the default is the model written with '
+                         'folx_amd.numpy calls')
     ap.add_argument('--graph', action='store_true',
                     help='replay each chunk as a captured HIP graph (no per-kernel timing, no roofline)')
     ap.add_argument('--calibrate-copy', action='store_true',
@@ -210,7 +214,8 @@ def roofline_of(dname, dkey, dn, dms, gemm):
             'traffic': None, 'kernel': f'{dname} {dkey}', 'launches': dn, 'avg_launch_ms': dms / dn}
 
 
-def measure(workload, steps, warmup, walkers=0, chunk=1024, gemm='f32', graph=False, calibrate_copy=False):
+def measure(workload, steps, warmup, walkers=0, chunk=1024, gemm='f32', graph=False, calibrate_copy=False,
+            front_door='calls'):
     """Times ``steps`` steps of one workload after ``warmup`` untimed ones (inputs resident on the device, host clock
     around device synchronisations) and finds the entry point with the largest total time, whose launches carry HIP
     events on the launch stream inside the timed region.  Returns the pieces of the output line."""
@@ -226,7 +231,13 @@ def measure(workload, steps, warmup, walkers=0, chunk=1024, gemm='f32', graph=Fa
     dev = torch.device('cuda', 0)
     params = wl.to_device(params_np, dev)
     x = torch.as_tensor(wl.sample_inputs(workload, B, seed=2)).to(dev)
-    fl = folx_amd.forward_laplacian(lambda r: forward(params, r), thr)
+    if front_door == 'torch':
+        # the same model as plain torch code, traced once (torch.fx) and evaluated through the rules
+        from folx_amd import torch_namespace as txp
+
+        fl = folx_amd.forward_laplacian_torch(lambda r: forward(params_np, r, xp=txp), thr)
+    else:
+        fl = folx_amd.forward_laplacian(lambda r: forward(params, r), thr)
     step = folx_amd.batched_vmap(folx_amd.jit(folx_amd.vmap(fl)) if graph else fl, chunk)
 
     for _ in range(warmup):
@@ -387,7 +398,7 @@ def main():
         streaming_rules()
         return
     m = measure(args.workload, args.steps, args.warmup, args.walkers, args.chunk, args.gemm, args.graph,
-                args.calibrate_copy)
+                args.calibrate_copy, args.front_door)
     B, cfg, thr, out, x, step, dt, roof = (m[k] for k in ('B', 'cfg', 'thr', 'out', 'x', 'step', 'dt', 'roof'))
     ms_per_step = 1e3 * dt / args.steps
     value = B * args.steps / dt
@@ -420,6 +431,7 @@ def main():
             'chunk': args.chunk,
             'jacobian_rows': int(out.jacobian.dense_array.shape[0]),
             'gemm': args.gemm,
+            'front_door': args.front_door,
         },
         'roofline': roof,
         # from the one untimed step in which every entry point carried events

@@ -240,6 +240,7 @@ RULES = {
     aten.linalg_inv_ex.default: lambda A, check_errors=False: (fnp.inv(A), None),
     aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
     operator.getitem: lambda a, i: a[i],
+    aten.sign.default: fnp.sign, aten.sgn.default: fnp.sign,
     aten._safe_softmax.default: lambda a, dim, dtype=None: fnp.softmax(a, axis=int(dim)),
     torch.ops.folx_amd.multi_head_self_attention.default: fnp.multi_head_self_attention,
 }
@@ -290,27 +291,51 @@ def _any_triplet(v):
     return _is_t(v)
 
 
-def evaluate_graph(gm: torch.fx.GraphModule, inputs):
-    """One pass over the equations of a traced graph (folx/interpreter.py:218-264): an equation whose inputs are
-    all constants is evaluated eagerly by torch itself, the others through ``RULES``."""
+def fold_constants(gm: torch.fx.GraphModule):
+    """Every equation whose inputs are all constants, evaluated once by torch itself on the host (the reference binds
+    such equations eagerly while it interprets, folx/interpreter.py:222-245): node -> numpy array / scalar / tuple."""
     env = {}
-    it = iter(inputs)
     look = lambda a: env[a] if isinstance(a, torch.fx.Node) else a
+    is_const = lambda a: not isinstance(a, torch.fx.Node) or a in env
+
+    def all_const(v):
+        if isinstance(v, (list, tuple)):
+            return all(all_const(t) for t in v)
+        if isinstance(v, dict):
+            return all(all_const(t) for t in v.values())
+        return is_const(v)
+
     for node in gm.graph.nodes:
-        if node.op == 'placeholder':
-            env[node] = next(it)
-        elif node.op == 'get_attr':
+        if node.op == 'get_attr':
             obj = gm
             for part in node.target.split('.'):
                 obj = getattr(obj, part)
-            env[node] = _const(obj)
+            env[node] = obj.detach() if isinstance(obj, torch.Tensor) else obj
+        elif node.op == 'call_function' and all_const(node.args) and all_const(node.kwargs):
+            args = torch.fx.node.map_arg(node.args, look)
+            kwargs = torch.fx.node.map_arg(node.kwargs, look)
+            with torch.no_grad():
+                env[node] = node.target(*args, **kwargs)
+    return {n: _tree(v, _const) for n, v in env.items()}
+
+
+_DEVICE_CONST_MIN = 256   # constants of at least this many floats live on the device between evaluations
+
+
+def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
+    """One pass over the equations of a traced graph (folx/interpreter.py:218-264): constant equations come from
+    ``fold_constants``, the others go through ``RULES``."""
+    env = dict(fold_constants(gm) if consts is None else consts)
+    it = iter(inputs)
+    look = lambda a: env[a] if isinstance(a, torch.fx.Node) else a
+    for node in gm.graph.nodes:
+        if node in env:
+            continue
+        if node.op == 'placeholder':
+            env[node] = next(it)
         elif node.op == 'call_function':
             args = torch.fx.node.map_arg(node.args, look)
             kwargs = torch.fx.node.map_arg(node.kwargs, look)
-            if not _any_triplet(args) and not _any_triplet(kwargs) and node.target is not operator.getitem:
-                to_t = lambda v: torch.as_tensor(v) if isinstance(v, np.ndarray) else v
-                env[node] = _tree(node.target(*_tree(args, to_t), **_tree(kwargs, to_t)), _const)
-                continue
             kwargs = {k: v for k, v in kwargs.items() if k not in ('dtype', 'device', 'layout', 'pin_memory', 'memory_format')}
             rule = RULES.get(node.target) or _generic(node.target)
             try:
@@ -327,11 +352,13 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs):
 
 class TracedForwardLaplacian(ForwardLaplacianFn):
     """``forward_laplacian_torch(fn, thr)``: ``f(x)`` takes one sample, ``f.batched(x)`` walkers, as for
-    ``forward_laplacian``; the torch function is traced once per combination of input shapes."""
+    ``forward_laplacian``; the torch function is traced once per combination of input shapes, its constant
+    equations are evaluated then, and the larger constants (weights) are uploaded once per device."""
 
     def __init__(self, fn, sparsity_threshold):
         self.torch_fn = fn
         self.graphs = {}
+        self.constants = {}
         super().__init__(self._run, sparsity_threshold)
 
     def _graph(self, shapes):
@@ -346,11 +373,31 @@ class TracedForwardLaplacian(ForwardLaplacianFn):
                     gm = self.graphs[shapes] = make_fx(self.torch_fn)(*examples)
                 finally:
                     _TRACING[0] = False
+            self.constants[shapes] = fold_constants(gm)
         return gm
+
+    def _constants(self, shapes, device):
+        key = (shapes, str(device))
+        hit = self.constants.get(key)
+        if hit is None:
+            def place(v):
+                if (isinstance(v, np.ndarray) and v.dtype == np.float32 and v.size >= _DEVICE_CONST_MIN
+                        and device.type != 'cpu'):
+                    return torch.as_tensor(np.ascontiguousarray(v)).to(device)
+                return v
+            hit = self.constants[key] = {n: _tree(v, place) for n, v in self.constants[shapes].items()}
+        return hit
 
     def _run(self, *lapl_args):
         shapes = tuple(tuple(a.shape) for a in lapl_args)
-        return evaluate_graph(self._graph(shapes), lapl_args)
+        gm = self._graph(shapes)
+        return evaluate_graph(gm, lapl_args, self._constants(shapes, lapl_args[0].x.device))
+
+    def invalidate(self):
+        """Forget the traces (and the constants folded from them): the next call traces again, e.g. after the
+        parameters of a traced module have changed."""
+        self.graphs.clear()
+        self.constants.clear()
 
 
 def forward_laplacian_torch(fn, sparsity_threshold: int | float = 0) -> TracedForwardLaplacian:

@@ -68,3 +68,45 @@ def test_unknown_operation_gets_the_generic_rule(monkeypatch, caplog):
 def test_torch_models_on_the_gpu(name, thr):
     print(f'traced torch model {name} thr={thr}', flush=True)
     _check(name, thr, 'cuda')
+
+
+def _both_front_doors(forward, params, x, thr, device):
+    from folx_amd import torch_namespace as txp
+
+    by_calls = folx_amd.vmap(folx_amd.forward_laplacian(lambda r: forward(params, r), thr))(torch.as_tensor(x).to(device))
+    traced = folx_amd.vmap(folx_amd.forward_laplacian_torch(lambda r: forward(params, r, xp=txp), thr))(torch.as_tensor(x).to(device))
+    J1, J2 = by_calls.jacobian.dense_array.cpu().numpy(), traced.jacobian.dense_array.cpu().numpy()
+    scale = lambda a: max(1.0, float(np.abs(a).max()))
+    np.testing.assert_allclose(traced.x.cpu().numpy(), by_calls.x.cpu().numpy(), rtol=2e-4, atol=2e-5 * scale(J1))
+    np.testing.assert_allclose(J2, J1, rtol=5e-4, atol=1e-4 * scale(J1))
+    np.testing.assert_allclose(traced.laplacian.cpu().numpy(), by_calls.laplacian.cpu().numpy(), rtol=5e-4,
+                               atol=2e-4 * scale(by_calls.laplacian.cpu().numpy()))
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_benchmark_models_through_the_traced_front_door(thr, monkeypatch):
+    """The benchmark architectures (small widths) as plain torch code (``folx_amd.torch_namespace``), traced, against the
+    same models written with ``folx_amd.numpy`` calls."""
+    from folx_amd import workloads as wl
+
+    cpu_kernels.install(monkeypatch)
+    psi = wl.PsiFormerConfig(n_elec=4, n_nuc=2, n_layers=2, n_heads=2, head_dim=4, width=8, mlp_width=8, n_det=2, orb_shift=1.5)
+    fermi = wl.FermiNetConfig(n_elec=4, n_nuc=2, n_layers=3, w1=8, w2=4, n_det=2, orb_shift=1.5)
+    for cfg, forward, make in ((psi, wl.psiformer_forward, wl.psiformer_params), (fermi, wl.ferminet_forward, wl.ferminet_params)):
+        x = wl.sample_electrons(3, cfg.n_elec, 1.0, seed=5)
+        _both_front_doors(forward, make(cfg), x, thr, 'cpu')
+    params = wl.mlp_params(seed=0, in_dim=4, width=8, n_hidden=3)
+    _both_front_doors(wl.mlp_forward, params, np.random.default_rng(0).normal(size=(3, 6, 4)).astype(np.float32), thr, 'cpu')
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('thr', [0, 6])
+def test_benchmark_models_through_the_traced_front_door_on_the_gpu(thr):
+    from folx_amd import workloads as wl
+
+    print(f'benchmark architectures through both front doors, thr={thr}', flush=True)
+    psi = wl.PsiFormerConfig(n_elec=6, n_nuc=2, n_layers=2, n_heads=2, head_dim=8, width=16, mlp_width=16, n_det=3, orb_shift=1.5)
+    fermi = wl.FermiNetConfig(n_elec=6, n_nuc=2, n_layers=3, w1=16, w2=8, n_det=3, orb_shift=1.5)
+    for cfg, forward, make in ((psi, wl.psiformer_forward, wl.psiformer_params), (fermi, wl.ferminet_forward, wl.ferminet_params)):
+        x = wl.sample_electrons(5, cfg.n_elec, 1.0, seed=5)
+        _both_front_doors(forward, make(cfg), x, thr, 'cuda')
