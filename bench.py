@@ -470,6 +470,38 @@ def main():
             K.set_gemm_mode('f32')
     else:
         out2 = None
+    if (not args.no_other and args.gemm == 'f32' and args.workload == 'psiformer32' and not args.walkers
+            and args.front_door == 'calls' and not args.graph):
+        # the same model as plain torch code through the traced front door (torch.fx graph evaluated through the
+        # rules): reported beside the headline, never as `value`
+        try:
+            import folx_amd
+            from folx_amd import torch_namespace as txp
+            from folx_amd import workloads as wl
+
+            forward, params_np = wl.build(args.workload)[:2]
+            traced = folx_amd.batched_vmap(
+                folx_amd.forward_laplacian_torch(lambda r: forward(params_np, r, xp=txp), thr), args.chunk)
+            out3 = traced(x)
+            torch.cuda.synchronize()
+            n3 = max(1, min(args.steps, 3))
+            t0 = time.perf_counter()
+            for _ in range(n3):
+                out3 = traced(x)
+            torch.cuda.synchronize()
+            dt3 = time.perf_counter() - t0
+            rel = (out3.laplacian - out.laplacian).abs() / out.laplacian.abs().clamp_min(1e-30)
+            line['traced_torch_front_door'] = {
+                'value': B * n3 / dt3, 'unit': 'walkers/s', 'steps': n3, 'ms_per_step': 1e3 * dt3 / n3,
+                # per walker |difference| / |Laplacian| against the headline run (a different order of float32
+                # operations; the few walkers with near-singular orbital matrices carry the tail)
+                'laplacian_relative_difference_to_headline': {'median': float(rel.median()),
+                                                              'p99': float(rel.quantile(0.99))},
+                'how': 'folx_amd.forward_laplacian_torch: the model as plain torch code, traced once with torch.fx, '
+                       'every equation evaluated through the rule registry'}
+            del out3, traced
+        except Exception as e:  # the side measurement must not take the headline line down with it
+            line['traced_torch_front_door'] = {'error': f'{type(e).__name__}: {e}'}
     if not args.no_other and args.gemm == 'f32' and args.workload == 'psiformer32' and not args.walkers:
         # the other configurations of the benchmark suite, a few steps each: walkers/s, the entry point with
         # the largest total time and its roofline fraction.  The headline stays the line's `value`.
