@@ -110,3 +110,17 @@ def test_benchmark_models_through_the_traced_front_door_on_the_gpu(thr):
     for cfg, forward, make in ((psi, wl.psiformer_forward, wl.psiformer_params), (fermi, wl.ferminet_forward, wl.ferminet_params)):
         x = wl.sample_electrons(5, cfg.n_elec, 1.0, seed=5)
         _both_front_doors(forward, make(cfg), x, thr, 'cuda')
+
+
+@pytest.mark.gpu
+def test_traced_model_under_graph_replay():
+    """``folx_amd.jit`` around a traced model: replays return the bits of the eager evaluation."""
+    make, x = MODELS['transformer_block']()
+    fl = folx_amd.forward_laplacian_torch(make(torch.float32), 3)
+    eager, fast = folx_amd.vmap(fl), folx_amd.jit(folx_amd.vmap(fl))
+    for call in range(4):
+        xin = torch.as_tensor(x + 0.01 * call).cuda()
+        a, b = eager(xin), fast(xin)
+        torch.cuda.synchronize()
+        assert torch.equal(a.x, b.x) and torch.equal(a.laplacian, b.laplacian), f'call {call}'
+        assert torch.equal(a.jacobian.dense_array, b.jacobian.dense_array), f'call {call}'
