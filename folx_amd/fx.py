@@ -241,6 +241,9 @@ RULES = {
     aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
     operator.getitem: lambda a, i: a[i],
     aten.sign.default: fnp.sign, aten.sgn.default: fnp.sign,
+    aten.index_select.default: lambda a, dim, index: fnp.take(a, np.asarray(index), axis=int(dim)),
+    aten.take.default: lambda a, index: fnp.take(a, np.asarray(index)),
+    aten.squeeze_.dim: lambda a, dim: _squeeze(a, (dim,)), aten.unsqueeze_.default: lambda a, dim: fnp.expand_dims(a, int(dim)),
     aten._safe_softmax.default: lambda a, dim, dtype=None: fnp.softmax(a, axis=int(dim)),
     torch.ops.folx_amd.multi_head_self_attention.default: fnp.multi_head_self_attention,
 }

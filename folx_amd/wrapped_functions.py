@@ -1525,7 +1525,14 @@ def concatenate_rule(args, kwargs, sparsity_threshold):
     axis = kwargs.get('dimension', kwargs.get('axis', -1))
     trip = [t for t in args if _is(t)]
     if not trip:
-        return np.concatenate([np.asarray(t) for t in args], axis=axis)
+        walker = [t for t in args if isinstance(t, BatchedArray)]
+        if not walker:
+            return np.concatenate([np.asarray(t) for t in args], axis=axis)
+        # derivative-free values that differ from walker to walker (and constants among them)
+        Bw, devw, ndw = walker[0].data.shape[0], walker[0].data.device, walker[0].ndim
+        parts = [t.data if isinstance(t, BatchedArray) else
+                 so.device_const(t, devw).reshape(1, *np.shape(t)).expand(Bw, *np.shape(t)) for t in args]
+        return BatchedArray(torch.cat(parts, dim=axis % ndw + 1))
     first = trip[0]
     nd, B, dev = first.ndim, first.B, first.x.device
     axis = axis % nd

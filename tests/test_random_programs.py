@@ -93,3 +93,30 @@ def test_graph_replay_of_random_programs_equals_eager_bit_for_bit():
             torch.cuda.synchronize()
             assert torch.equal(a.x, b.x) and torch.equal(a.laplacian, b.laplacian), f'seed {seed} call {call}'
             assert torch.equal(a.jacobian.dense_array, b.jacobian.dense_array), f'seed {seed} call {call}'
+
+
+def test_traced_front_door_on_random_programs(monkeypatch, caplog):
+    """The same programs written with torch (``bruteforce.plain``), traced by ``forward_laplacian_torch`` and evaluated
+    through the rules, against the oracle; no equation may fall back to the generic rule."""
+    cpu_kernels.install(monkeypatch)
+    with caplog.at_level('WARNING'):
+        for seed in range(60):
+            steps = rp.generate(seed, 8 if seed < 40 else 14)
+            x = _inputs(seed)
+            ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
+            for thr in (0, 3, 12):
+                out = folx_amd.vmap(folx_amd.forward_laplacian_torch(lambda t: rp.run(steps, plain, t), thr))(x)
+                _compare(out, ref, f'traced, seed {seed} thr {thr}: {rp.describe(steps)}')
+    assert not [r for r in caplog.records if 'no forward-Laplacian rule' in r.message]
+
+
+@pytest.mark.gpu
+def test_traced_front_door_on_random_programs_on_the_gpu():
+    for seed in range(30):
+        steps = rp.generate(seed, 8)
+        x = _inputs(seed, walkers=5)
+        ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
+        for thr in (0, 12):
+            print(f'traced random program seed {seed} thr {thr}: {rp.describe(steps)}', flush=True)
+            out = folx_amd.vmap(folx_amd.forward_laplacian_torch(lambda t: rp.run(steps, plain, t), thr))(torch.as_tensor(x).cuda())
+            _compare(out, ref, f'traced, seed {seed} thr {thr}: {rp.describe(steps)}')
