@@ -993,6 +993,15 @@ def ones_like(a):
 erfinv, gammaln = erf_inv, lgamma   # (jnp.max / jnp.min along one axis are amax / amin: the builtins keep their names here)
 
 
+# jnp.linalg / jax.nn / jax.scipy.special spellings of the functions above
+import types as _types
+
+linalg = _types.SimpleNamespace(slogdet=slogdet, det=det, inv=inv, solve=solve, norm=norm)
+nn = _types.SimpleNamespace(softmax=softmax, log_softmax=log_softmax, logsumexp=logsumexp, gelu=gelu, silu=silu, relu=relu,
+                            elu=elu, leaky_relu=leaky_relu, sigmoid=sigmoid, softplus=softplus, tanh=tanh)
+special = _types.SimpleNamespace(erf=erf, erfc=erfc, erfinv=erf_inv, gammaln=lgamma, digamma=digamma, logsumexp=logsumexp)
+
+
 # primitive names of jax.lax (folx/wrapped_functions.py:376-399, :468-513)
 register_function('clamp', lambda args, kw, thr: _composed(lambda lo, x, hi: clip(x, lo, hi))(args, kw, thr))
 register_function('select_n', lambda args, kw, thr: _composed(lambda c, b, a: where(c, a, b))(args, kw, thr))
