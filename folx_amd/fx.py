@@ -249,6 +249,12 @@ RULES = {
 }
 
 
+def _amax_values(a, dims=(), keepdim=False):
+    s = _shape(a)
+    axes = _dims(dims, len(s))
+    return fnp.amax_const(a, axes, keepdims=bool(keepdim))
+
+
 def _fold_axes(fn, a, dims, keepdim):
     s = _shape(a)
     axes = sorted(_dims(dims, len(s)), reverse=True)
@@ -341,6 +347,8 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
             kwargs = torch.fx.node.map_arg(node.kwargs, look)
             kwargs = {k: v for k, v in kwargs.items() if k not in ('dtype', 'device', 'layout', 'pin_memory', 'memory_format')}
             rule = RULES.get(node.target) or _generic(node.target)
+            if node.target is aten.amax.default and node.users and all(u.target is aten.detach.default for u in node.users):
+                rule = _amax_values   # max(...).detach(): the shift of a softmax / logsumexp carries no derivatives
             try:
                 env[node] = rule(*args, **kwargs)
             except Exception:
