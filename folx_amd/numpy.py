@@ -506,6 +506,14 @@ def reshape(a, shape):
         tot = int(np.prod(_shape(a), dtype=int))
         rest = -int(np.prod(shape, dtype=int))
         shape = tuple(tot // rest if s == -1 else s for s in shape)
+    from .wrapped_functions import LazyDot
+
+    if (isinstance(a, LazyDot) and a._value is None and len(shape) >= 1 and shape[-1] == a.shape[-1]
+            and isinstance(a.h, FwdLaplArray) and a.kwargs.get('row_slice') is None and a.kwargs.get('norm') is None):
+        # only the leading axes change: the same product on the input with those leading axes, its epilogue
+        # (bias, activation, skip connection) still open -- e.g. `(h.reshape(-1, K) @ W).reshape(n, n, N) + b`
+        h = _call('reshape', (a.h,), {'new_sizes': (*shape[:-1], a.h.shape[-1])})
+        return LazyDot(h, a.W, a.kwargs, shape, a.thr)
     return _call('reshape', (a,), {'new_sizes': shape})
 
 
