@@ -167,6 +167,39 @@ def _max_dim(arg_fn, val_fn):
     return rule
 
 
+class _OnDemand:
+    """An output of a multi-output operation that is only computed when the graph reads it."""
+
+    def __init__(self, make):
+        self.make = make
+
+
+def _scan_with_indices(scan_fn, arg_fn):
+    """``cummax`` / ``cummin``: values from the scan; indices (no derivatives) = the arg-extremum over each prefix,
+    from an (n, n) masked copy, built only if the graph reads them."""
+    def rule(a, dim):
+        s = _shape(a)
+        ax = int(dim) % len(s)
+        n = s[ax]
+
+        def indices():
+            v = fnp.stop_gradient(a)
+            big = np.float32(np.finfo(np.float32).max) * (1.0 if arg_fn is fnp.argmin else -1.0)
+            keep = np.tril(np.ones((n, n), dtype=bool)).reshape((n,) + (1,) * (len(s) - 1 - ax) + (n,))
+            rows = fnp.expand_dims(fnp.moveaxis(v, ax, -1), ax)            # (..., 1, ..., n): prefix i reads entries <= i
+            full = fnp.where(keep, rows, big)
+            return arg_fn(full, axis=-1)
+
+        return scan_fn(a, axis=ax), _OnDemand(indices)
+
+    return rule
+
+
+def _item(a, i):
+    v = a[i]
+    return v.make() if isinstance(v, _OnDemand) else v
+
+
 def _clamp(a, lo=None, hi=None):
     return fnp.clip(a, lo, hi)
 
@@ -220,6 +253,8 @@ RULES = {
     aten.prod.dim_int: lambda a, dim, keepdim=False, dtype=None: _fold_axes(fnp.prod, a, (dim,), keepdim),
     aten.cumsum.default: lambda a, dim, dtype=None: fnp.cumsum(a, axis=int(dim)),
     aten.cumprod.default: lambda a, dim, dtype=None: fnp.cumprod(a, axis=int(dim)),
+    aten.cummax.default: _scan_with_indices(fnp.cummax, fnp.argmax), aten.cummin.default: _scan_with_indices(fnp.cummin, fnp.argmin),
+    aten.unbind.int: lambda a, dim=0: tuple(_select(a, dim, i) for i in range(_shape(a)[int(dim) % len(_shape(a))])),
     aten._softmax.default: lambda a, dim, half=False: fnp.softmax(a, axis=int(dim)),
     aten._log_softmax.default: lambda a, dim, half=False: fnp.log_softmax(a, axis=int(dim)),
     aten.logsumexp.default: lambda a, dim, keepdim=False: _logsumexp(a, dim, keepdim),
@@ -239,7 +274,7 @@ RULES = {
     aten._linalg_det.default: lambda A: (fnp.det(A), None, None),
     aten.linalg_inv_ex.default: lambda A, check_errors=False: (fnp.inv(A), None),
     aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
-    operator.getitem: lambda a, i: a[i],
+    operator.getitem: _item,
     aten.sign.default: fnp.sign, aten.sgn.default: fnp.sign,
     aten.index_select.default: lambda a, dim, index: fnp.take(a, np.asarray(index), axis=int(dim)),
     aten.take.default: lambda a, index: fnp.take(a, np.asarray(index)),

@@ -79,7 +79,8 @@ def device_table(arr: np.ndarray, device) -> torch.Tensor:
     key = _key(arr, 'i32', str(device))
     t = _TABLE_CACHE.get(key)
     if t is None:
-        t = torch.as_tensor(np.ascontiguousarray(arr, dtype=np.int32)).to(device)
+        # a copy: the source may be one of the read-only masks, which torch would warn about wrapping
+        t = torch.from_numpy(np.array(arr, dtype=np.int32, order='C')).to(device)
         _TABLE_CACHE[key] = t
     return t
 

@@ -10,6 +10,8 @@ N_IN = 12
 _SHAPES = [(12,), (3, 4), (4, 3), (2, 6), (6, 2), (2, 3, 2), (2, 2, 3), (3, 2, 2)]
 _UNARY = ['sin', 'cos', 'tanh', 'square', 'sigmoid']
 _BINARY = ['add', 'subtract', 'multiply', 'divide']
+_MORE = ['inv_spd', 'solve_spd', 'attention', 'scatter', 'cumprod', 'cummax', 'prod', 'amin', 'minimum', 'maximum', 'clip',
+         'layer_norm', 'where_data', 'abs_sqrt']
 
 
 def _factorizations(n):
@@ -23,9 +25,11 @@ def _factorizations(n):
     return out
 
 
-def generate(seed: int, n_steps: int = 7, n_in: int = N_IN):
+def generate(seed: int, n_steps: int = 7, n_in: int = N_IN, more: bool = False):
     """Returns a list of steps ``(op, operand indices, static arguments)``; shapes are tracked while drawing
-    so that every step is valid.  Value 0 is the input (``n_in`` entries), value 1 the input reshaped."""
+    so that every step is valid.  Value 0 is the input (``n_in`` entries), value 1 the input reshaped.  ``more``: also
+    the second family of steps (inverse / solve, attention, scatter, scans, min / max, clip, LayerNorm, a ``where`` whose
+    condition depends on the data)."""
     rng = np.random.default_rng(seed)
     first_shapes = _SHAPES if n_in == N_IN else _factorizations(n_in)
     first = first_shapes[rng.integers(len(first_shapes))]
@@ -37,7 +41,7 @@ def generate(seed: int, n_steps: int = 7, n_in: int = N_IN):
             s = shapes[i]
             kind = rng.choice(['unary', 'binary', 'reshape', 'transpose', 'slice', 'sum', 'dot', 'concat', 'broadcast',
                                'flip', 'where', 'cumsum', 'amax', 'take', 'binary_const', 'mean_keep', 'pad',
-                               'matmul_t', 'softmax', 'logsumexp', 'logdet_spd'])
+                               'matmul_t', 'softmax', 'logsumexp', 'logdet_spd'] + (_MORE if more else []))
             size = int(np.prod(s, dtype=int))
             if kind == 'unary':
                 steps.append((str(rng.choice(_UNARY)), (i,), ())); shapes.append(s)
@@ -156,6 +160,45 @@ def generate(seed: int, n_steps: int = 7, n_in: int = N_IN):
                 if len(s) < 2 or s[-2] > 6:
                     continue
                 steps.append(('logdet_spd', (i,), ())); shapes.append(s[:-2])
+            elif kind in ('inv_spd', 'solve_spd'):
+                if len(s) < 2 or s[-2] > 5 or s[-2] < 2:
+                    continue
+                steps.append((kind, (i,), ())); shapes.append((*s[:-2], s[-2], s[-2]) if kind == 'inv_spd' else (*s[:-1], s[-1]))
+            elif kind == 'attention':
+                # value (n, H d) with H in {1, 2}: q = tanh(v), k = sin(v), v = v reshaped to (n, H, d)
+                if len(s) != 2 or s[-1] % 2 != 0 or s[0] < 2:
+                    continue
+                H = int(rng.choice([1, 2]))
+                steps.append(('attention', (i,), (H,))); shapes.append(s)
+            elif kind == 'scatter':
+                if len(s) != 1 or s[0] < 3:
+                    continue
+                n_upd = int(rng.integers(1, 4))
+                cands = [j for j in range(1, len(shapes)) if len(shapes[j]) == 1 and shapes[j][0] >= n_upd]
+                j = int(rng.choice(cands))
+                idx = rng.integers(0, s[0], size=n_upd)
+                steps.append(('scatter', (i, j), (idx, str(rng.choice(['set', 'add'])) if len(set(idx.tolist())) == n_upd else 'add')))
+                shapes.append(s)
+            elif kind in ('cumprod', 'cummax', 'prod', 'amin'):
+                if not s or s[-1] < 2 or s[-1] > 8:
+                    continue
+                steps.append((kind, (i,), ())); shapes.append(s if kind in ('cumprod', 'cummax') else s[:-1])
+            elif kind in ('minimum', 'maximum'):
+                cands = [j for j in range(1, len(shapes)) if shapes[j] == s and j != i]
+                if not cands:
+                    continue
+                steps.append((kind, (i, int(rng.choice(cands))), ())); shapes.append(s)
+            elif kind == 'clip':
+                steps.append(('clip', (i,), (-0.45, 0.7))); shapes.append(s)
+            elif kind == 'layer_norm':
+                if not s or s[-1] < 3:
+                    continue
+                steps.append(('layer_norm', (i,), ())); shapes.append(s)
+            elif kind == 'where_data':
+                cands = [j for j in range(1, len(shapes)) if shapes[j] == s]
+                steps.append(('where_data', (i, int(rng.choice(cands))), ())); shapes.append(s)
+            elif kind == 'abs_sqrt':
+                steps.append(('abs_sqrt', (i,), ())); shapes.append(s)
             if int(np.prod(shapes[-1], dtype=int)) > 400 * max(n_in // N_IN, 1):     # keep the values small
                 steps.pop(); shapes.pop()
                 continue
@@ -206,6 +249,32 @@ def run(steps, xp, x):
             v = xp.softmax(xp.tanh(a[0]), axis=-1)
         elif op == 'logsumexp':
             v = xp.logsumexp(xp.tanh(a[0]), axis=-1)[0]
+        elif op in ('inv_spd', 'solve_spd'):
+            t = xp.tanh(a[0])
+            m = t.shape[-2]
+            A = xp.add(xp.matmul(t, xp.swapaxes(t, -1, -2)), 2.0 * np.eye(m, dtype=np.float32))
+            v = xp.inv(A) if op == 'inv_spd' else xp.solve(A, xp.sin(a[0]))
+        elif op == 'attention':
+            n, w = a[0].shape
+            H = static[0]
+            q, k, vv = (xp.reshape(f(a[0]), (n, H, w // H)) for f in (xp.tanh, xp.sin, lambda z: z))
+            v = xp.reshape(xp.multi_head_self_attention(q, k, vv), (n, w))
+        elif op == 'scatter':
+            v = xp.scatter(a[0], static[0], xp.getitem(xp.sin(a[1]), (slice(0, len(static[0])),)), static[1])
+        elif op in ('cumprod', 'prod'):
+            v = getattr(xp, op)(xp.add(xp.multiply(xp.tanh(a[0]), 0.5), 1.2), axis=-1)
+        elif op in ('cummax', 'amin'):
+            v = getattr(xp, op)(xp.sin(xp.multiply(a[0], 1.7)), axis=-1)
+        elif op in ('minimum', 'maximum'):
+            v = getattr(xp, op)(xp.sin(a[0]), xp.cos(a[1]))
+        elif op == 'clip':
+            v = xp.clip(xp.sin(a[0]), static[0], static[1])
+        elif op == 'layer_norm':
+            v = xp.layer_norm(xp.sin(a[0]), None, None, 1e-3)
+        elif op == 'where_data':
+            v = xp.where(xp.greater(xp.sin(xp.multiply(a[0], 2.3)), 0.05), xp.tanh(a[0]), xp.multiply(xp.cos(a[1]), 0.3))
+        elif op == 'abs_sqrt':
+            v = xp.sqrt(xp.add(xp.abs(xp.sin(xp.multiply(a[0], 1.3))), 0.3))
         elif op == 'logdet_spd':
             t = xp.tanh(a[0])
             m = t.shape[-2]

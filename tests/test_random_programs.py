@@ -30,16 +30,17 @@ def _compare(out, ref, what):
     np.testing.assert_allclose(gl, ref.lap, rtol=2e-4, atol=10 * floor(ref.lap), err_msg=what)
 
 
-@pytest.mark.parametrize('block', range(6))
+@pytest.mark.parametrize('block', range(8))
 def test_product_host_logic_against_the_oracle(block, monkeypatch):
-    """50 programs per block (blocks 0-3: 7 steps, 4-5: 14 steps), thresholds 0 (dense), 2, 3, 5 and 12; the caches
+    """50 programs per block (blocks 0-3: 7 steps, 4-5: 14 steps, 6-7: 9 steps with the second family of step
+    kinds), thresholds 0 (dense), 2, 3, 5 and 12; the caches
     are NOT cleared between programs, so entries of one program meet the lookups of the next."""
     cpu_kernels.install(monkeypatch)
     from folx_amd import sparse_ops
 
     sparse_ops.clear_caches()
     for seed in range(50 * block, 50 * block + 50):
-        steps = rp.generate(seed, 7 if block < 4 else 14)
+        steps = rp.generate(seed, (7, 7, 7, 7, 14, 14, 9, 9)[block], more=block >= 6)
         x = _inputs(seed)
         ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
         for thr in (0, 2, 3, 5, 12):
@@ -49,8 +50,8 @@ def test_product_host_logic_against_the_oracle(block, monkeypatch):
 
 def test_oracle_against_autograd_on_random_programs():
     """The oracle backend's rules in these combinations against the Hessian trace by torch AD in float64."""
-    for seed in range(40):
-        steps = rp.generate(seed)
+    for seed in range(80):
+        steps = rp.generate(seed, 7 if seed < 40 else 9, more=seed >= 40)
         x = _inputs(seed).astype(np.float64)
         ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
         by, bJ, bL = brute_force(lambda t: rp.run(steps, plain, t), x)
@@ -61,13 +62,14 @@ def test_oracle_against_autograd_on_random_programs():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize('block', range(3))
+@pytest.mark.parametrize('block', range(4))
 def test_hip_path_against_the_oracle(block):
     """The same programs on the GPU (5 walkers): every kernel the composed rules reach, in sequences nobody wrote by
-    hand.  Block 2 starts from 64 inputs: row extents that are multiples of 4 take the 128-bit forms of the kernels."""
+    hand.  Block 2 starts from 64 inputs: row extents that are multiples of 4 take the 128-bit forms of the kernels;
+    block 3 draws from the second family of step kinds too."""
     n_in = 64 if block == 2 else rp.N_IN
     for seed in range(30 * block, 30 * block + 30):
-        steps = rp.generate(seed, 14 if block == 1 else 7, n_in)
+        steps = rp.generate(seed, (7, 14, 7, 9)[block], n_in, more=block == 3)
         x = np.random.default_rng(1000 + seed).normal(size=(5, n_in)).astype(np.float32)
         ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
         for thr in (0, 3, 12, 64)[:4 if block == 2 else 3]:
@@ -80,8 +82,8 @@ def test_hip_path_against_the_oracle(block):
 def test_graph_replay_of_random_programs_equals_eager_bit_for_bit():
     """``folx_amd.jit``: the first call runs eagerly, the second is captured, later ones replay; every call returns the
     bits of the eager run on the same input (fresh inputs per call)."""
-    for seed in range(24):
-        steps = rp.generate(seed, 8, 64 if seed % 3 == 0 else rp.N_IN)
+    for seed in range(36):
+        steps = rp.generate(seed, 8, 64 if seed % 3 == 0 else rp.N_IN, more=seed >= 24)
         n_in = 64 if seed % 3 == 0 else rp.N_IN
         thr = (0, 3, 12)[seed % 3]
         print(f'graph replay, random program seed {seed} thr {thr}: {rp.describe(steps)}', flush=True)
@@ -100,8 +102,8 @@ def test_traced_front_door_on_random_programs(monkeypatch, caplog):
     through the rules, against the oracle; no equation may fall back to the generic rule."""
     cpu_kernels.install(monkeypatch)
     with caplog.at_level('WARNING'):
-        for seed in range(60):
-            steps = rp.generate(seed, 8 if seed < 40 else 14)
+        for seed in range(100):
+            steps = rp.generate(seed, (8, 14, 9)[(seed >= 40) + (seed >= 60)], more=seed >= 60)
             x = _inputs(seed)
             ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
             for thr in (0, 3, 12):
@@ -112,8 +114,8 @@ def test_traced_front_door_on_random_programs(monkeypatch, caplog):
 
 @pytest.mark.gpu
 def test_traced_front_door_on_random_programs_on_the_gpu():
-    for seed in range(30):
-        steps = rp.generate(seed, 8)
+    for seed in range(45):
+        steps = rp.generate(seed, 8, more=seed >= 30)
         x = _inputs(seed, walkers=5)
         ref = rp.run(steps, ob, ob.init_state(x, dtype=np.float64))
         for thr in (0, 12):
