@@ -23,7 +23,7 @@ from .operators import (
 )
 from .vmap import batched_vmap, vmap
 from .wrapped_functions import deregister_function, get_laplacian, is_registered, register_function
-from .wrapper import warp_without_fwd_laplacian, wrap_elementwise, wrap_forward_laplacian
+from .wrapper import custom_jvp, warp_without_fwd_laplacian, wrap_elementwise, wrap_forward_laplacian
 
 __all__ = [
     'BatchedArray',
@@ -47,4 +47,5 @@ __all__ = [
     'warp_without_fwd_laplacian',
     'wrap_elementwise',
     'wrap_forward_laplacian',
+    'custom_jvp',
 ]

@@ -27,7 +27,7 @@ import torch
 
 from .api import BatchedArray, FunctionFlags, FwdJacobian, FwdLaplArray
 
-__all__ = ['wrap_forward_laplacian', 'warp_without_fwd_laplacian', 'wrap_elementwise']
+__all__ = ['wrap_forward_laplacian', 'warp_without_fwd_laplacian', 'wrap_elementwise', 'custom_jvp']
 
 
 def _is(a):
@@ -94,6 +94,49 @@ def _tree_map(f, tree, *rest):
     return f(tree, *rest)
 
 
+class custom_jvp:
+    """A torch function with a derivative rule of the caller's own, spelled like ``jax.custom_jvp``::
+
+        @folx_amd.custom_jvp
+        def f(x): ...
+        @f.defjvp
+        def f_jvp(primals, tangents): return f(*primals), <J_f tangents>
+
+    Called with forward-Laplacian triplets it is evaluated by the generic rule with ``f_jvp`` in place of the
+    automatic ``J_f t`` -- the Jacobian and ``J_f lap`` come from the rule, ``t^T H_f t`` from its forward-mode
+    derivative -- as the reference evaluates a ``custom_jvp_call`` equation (folx/interpreter.py:202-208,
+    test/test_customjvp.py).  ``tangents`` holds zeros for the arguments that carry no derivatives.  Called with
+    anything else it is the plain function; under the trace of ``forward_laplacian_torch`` it raises, because the
+    trace would keep the function's operations and drop the rule."""
+
+    def __init__(self, fn):
+        self.fn = fn
+        self.jvp_rule = None
+        self.__name__ = getattr(fn, '__name__', 'custom_jvp')
+        self._rule = None
+
+    def defjvp(self, rule):
+        self.jvp_rule = rule
+        return rule
+
+    def __call__(self, *args, **kwargs):
+        from .numpy import current_threshold
+        from .wrapped_functions import Deferred
+
+        if not any(isinstance(a, (FwdLaplArray, Deferred)) for a in args):
+            from .fx import _TRACING
+
+            if _TRACING[0]:   # the trace would record the function's own operations and lose the rule
+                raise NotImplementedError(f'{self.__name__}: a custom_jvp function cannot be traced by '
+                                          'forward_laplacian_torch; call it under forward_laplacian')
+            return self.fn(*args, **kwargs)
+        if self.jvp_rule is None:
+            raise AttributeError(f'no derivative rule was given for {self.__name__} (defjvp)')
+        if self._rule is None:
+            self._rule = wrap_forward_laplacian(self)
+        return self._rule(args, kwargs, current_threshold())
+
+
 def wrap_forward_laplacian(
     fn: Callable,
     in_axes=None,
@@ -144,13 +187,28 @@ def wrap_forward_laplacian(
 
         consts = [None if (i in lapl_pos or i in bat_pos) else const(a) for i, a in enumerate(args)]
 
-        def call(xs, bs):
+        def merged(xs, bs):
             full = list(consts)
             for i, x in zip(lapl_pos, xs):
                 full[i] = x
             for i, b in zip(bat_pos, bs):
                 full[i] = b
-            return fn(*full, **kwargs)
+            return full
+
+        plain = fn.fn if isinstance(fn, custom_jvp) else fn
+
+        def call(xs, bs):
+            return plain(*merged(xs, bs), **kwargs)
+
+        def pushforward(g, xw, tv, bw):
+            """``J_f t``: forward mode through ``g``, or the caller's rule for a ``custom_jvp`` function."""
+            if not isinstance(fn, custom_jvp):
+                return jvp(g, xw, tv)[1]
+            primals = merged(xw, bw)
+            tangents = [torch.zeros_like(v) if isinstance(v, torch.Tensor) else 0.0 for v in primals]
+            for i, t in zip(lapl_pos, tv):
+                tangents[i] = t
+            return fn.jvp_rule(tuple(primals), tuple(tangents), **kwargs)[1]
 
         bvals = tuple(args[i].data for i in bat_pos)
         if not lapl_pos:  # nothing carries derivatives: a plain forward pass (folx/wrapper.py:112-114)
@@ -216,14 +274,14 @@ def wrap_forward_laplacian(
 
         def per_walker(xw, Jw, lw, bw):
             g = lambda *z: call(z, bw)  # noqa: E731
-            first = lambda tv: jvp(g, xw, tv)[1]  # noqa: E731   J_f t
+            first = lambda tv: pushforward(g, xw, tv, bw)  # noqa: E731   J_f t
             y = g(*xw)
             Jy = vmap(first)(Jw)
             lap = first(lw)
             if custom_jac_hessian_jac is not None:
                 lap = _tree_map(lambda l, q: l + q, lap, hook_term(xw, Jw, lw, bw, y))
             elif not linear:
-                second = lambda tv: jvp(lambda *z: jvp(g, z, tv)[1], xw, tv)[1]  # noqa: E731   t^T H_f t
+                second = lambda tv: jvp(lambda *z: pushforward(g, z, tv, bw), xw, tv)[1]  # noqa: E731   t^T H_f t
                 quad = vmap(second)(Jw)
                 lap = _tree_map(lambda l, q: l + q.sum(0), lap, quad)
             return y, Jy, lap

@@ -995,3 +995,33 @@ def test_rules_that_carry_no_derivatives_or_act_elementwise():
     np.testing.assert_allclose(got[0], by, rtol=2e-4, atol=2e-5)
     np.testing.assert_allclose(got[1], bJ.reshape(got[1].shape), rtol=2e-4, atol=2e-5)
     np.testing.assert_allclose(got[2], bL, rtol=2e-4, atol=2e-4)
+
+
+def test_custom_jvp_rule_is_used_for_both_orders(monkeypatch):
+    """test/test_customjvp.py:10-28: the rule differs from the true derivative by a factor of 2; value from the
+    function, Jacobian from the rule, Laplacian from the rule's own derivative.  Without triplets the object is
+    the plain function, and a missing rule is an error."""
+    cpu_kernels.install(monkeypatch)
+
+    @folx_amd.custom_jvp
+    def fn(x):
+        return torch.sin(x)
+
+    with pytest.raises(AttributeError, match='defjvp'):
+        folx_amd.vmap(folx_amd.forward_laplacian(fn, 0))(np.zeros((2, 3), dtype=np.float32))
+
+    @fn.defjvp
+    def fn_jvp(primals, tangents):
+        (x,), (t,) = primals, tangents
+        return fn(x), 2 * t * torch.cos(x)
+
+    x = np.random.default_rng(3).normal(size=(3, 10)).astype(np.float32)
+    for thr in (0, 10):
+        out = folx_amd.vmap(folx_amd.forward_laplacian(fn, thr))(x)
+        np.testing.assert_allclose(out.x.numpy(), np.sin(x), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(out.jacobian.dense_array.numpy(), 2 * np.cos(x)[None] * np.eye(10)[:, None, :],
+                                   rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(out.laplacian.numpy(), -2 * np.sin(x), rtol=1e-5, atol=1e-6)
+    assert torch.equal(fn(torch.tensor([0.5])), torch.sin(torch.tensor([0.5])))
+    with pytest.raises(NotImplementedError, match='cannot be traced'):
+        folx_amd.vmap(folx_amd.forward_laplacian_torch(fn, 0))(x)

@@ -69,3 +69,40 @@ def test_custom_jac_hessian_jac_hook_on_the_gpu(thr):
     out = folx_amd.vmap(folx_amd.forward_laplacian(lambda r: ten((r,), {}, thr), thr))(torch.as_tensor(x).cuda())
     assert_val(out.x, x, 'identity value')
     assert torch.equal(out.laplacian, torch.full_like(out.laplacian, 10.0))
+
+
+def _custom_rule_model():
+    """A function whose derivative rule differs from its true derivative by a factor of 2
+    (test/test_customjvp.py:10-28), between hand-written rules and with a constant argument."""
+    @folx_amd.custom_jvp
+    def wave(a, scale):
+        return torch.sin(a * scale)
+
+    @wave.defjvp
+    def wave_jvp(primals, tangents):
+        (a, scale), (ta, _) = primals, tangents
+        return wave(a, scale), 2.0 * ta * scale * torch.cos(a * scale)
+
+    scale = np.linspace(0.5, 1.5, 3).astype(np.float32)
+    model = lambda r: fnp.sum(fnp.square(wave(fnp.tanh(r), scale)), axis=-1)      # noqa: E731
+    # what the rule defines: d wave = 2 scale cos(a scale) da  <=>  wave behaves like 2 sin(a scale) + const
+    surrogate = lambda t: ((2.0 * torch.sin(torch.tanh(t) * torch.as_tensor(scale, dtype=t.dtype))))  # noqa: E731
+    return model, surrogate, scale
+
+
+@pytest.mark.parametrize('thr', [0, 6])
+def test_custom_jvp_rule_is_the_derivative_that_is_used(thr):
+    model, surrogate, scale = _custom_rule_model()
+    x = np.random.default_rng(52).normal(size=(5, 4, 3)).astype(np.float32)
+    out = folx_amd.vmap(folx_amd.forward_laplacian(model, thr))(torch.as_tensor(x).cuda())
+    # value: sum wave^2 with the function's values; derivatives chained by hand with d(wave) := ds, s = the surrogate
+    x64 = x.astype(np.float64)
+    s_val, s_J, s_L = brute_force(surrogate, x64)                  # (5,4,3), (12, 5,4,3), (5,4,3)
+    sin_v = np.sin(np.tanh(x64) * scale)
+    dsin, lsin = s_J.reshape(12, 5, 4, 3), s_L
+    want_J = (2 * sin_v[None] * dsin).sum(-1)
+    want_L = (2 * sin_v * lsin + 2 * (dsin ** 2).sum(0)).sum(-1)
+    J = out.jacobian.dense_array
+    assert_val(out.x, (sin_v ** 2).sum(-1), 'value')
+    assert_val(J, want_J.reshape(tuple(J.shape)), 'jacobian')
+    assert_lap(out.laplacian, want_L, 'laplacian')
