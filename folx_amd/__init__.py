@@ -48,4 +48,5 @@ __all__ = [
     'wrap_elementwise',
     'wrap_forward_laplacian',
     'custom_jvp',
+    'forward_laplacian_torch',
 ]
