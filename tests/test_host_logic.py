@@ -1025,3 +1025,18 @@ def test_custom_jvp_rule_is_used_for_both_orders(monkeypatch):
     assert torch.equal(fn(torch.tensor([0.5])), torch.sin(torch.tensor([0.5])))
     with pytest.raises(NotImplementedError, match='cannot be traced'):
         folx_amd.vmap(folx_amd.forward_laplacian_torch(fn, 0))(x)
+
+
+def test_auto_batched_vmap_without_a_gpu_runs_the_batch_whole(monkeypatch):
+    """folx/experimental/vmap.py:14-73: with nothing to measure (host arrays) the batch is not cut; a cap still is."""
+    cpu_kernels.install(monkeypatch)
+    from folx_amd.experimental import auto_batched_vmap
+
+    fl = folx_amd.forward_laplacian(lambda t: fnp.sum(fnp.tanh(fnp.multiply(t, t))), 0)
+    x = np.random.default_rng(4).normal(size=(40, 6)).astype(np.float32)
+    auto = auto_batched_vmap(fl)
+    whole = folx_amd.vmap(fl)(x)
+    assert torch.equal(auto(x).laplacian, whole.laplacian) and list(auto.chosen.values()) == [40]
+    capped = auto_batched_vmap(fl, max_batch_size=7)
+    np.testing.assert_allclose(capped(x).laplacian.numpy(), whole.laplacian.numpy(), rtol=1e-6, atol=1e-6)
+    assert list(capped.chosen.values()) == [7]
