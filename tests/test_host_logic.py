@@ -1040,3 +1040,27 @@ def test_auto_batched_vmap_without_a_gpu_runs_the_batch_whole(monkeypatch):
     capped = auto_batched_vmap(fl, max_batch_size=7)
     np.testing.assert_allclose(capped(x).laplacian.numpy(), whole.laplacian.numpy(), rtol=1e-6, atol=1e-6)
     assert list(capped.chosen.values()) == [7]
+
+
+def test_ad_helpers_have_the_reference_shapes_and_values():
+    """test/test_ad.py:12-37: jacfwd flattens the input on the last axis, jacrev the output on the first, hessian is
+    forward over reverse; values against torch.autograd.functional."""
+    from folx_amd.ad import hessian, jacfwd, jacrev
+
+    f = lambda x: torch.sin(x * x.sum())    # noqa: E731
+    x = torch.as_tensor(np.random.default_rng(5).normal(size=(3, 4)))
+    full = torch.autograd.functional.jacobian(f, x)                      # (3, 4, 3, 4)
+    assert jacfwd(f)(x).shape == (3, 4, 12) and jacrev(f)(x).shape == (12, 3, 4)
+    np.testing.assert_allclose(jacfwd(f)(x), full.reshape(3, 4, 12), rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(jacrev(f)(x), full.reshape(12, 3, 4), rtol=1e-12, atol=1e-13)
+    v = x.reshape(12)
+    H = hessian(f)(v)
+    assert H.shape == (12, 12, 12)
+    want = torch.stack([torch.autograd.functional.hessian(lambda z, i=i: f(z)[i], v) for i in range(12)])
+    np.testing.assert_allclose(H, want, rtol=1e-11, atol=1e-12)
+    # two arguments: jacrev gives one array per argument, jacfwd concatenates their entries
+    g = lambda a, b: torch.tanh(a) * b.sum()    # noqa: E731
+    a, b = x[0], x[1, :2]
+    ra, rb = jacrev(g)(a, b)
+    assert ra.shape == (4, 4) and rb.shape == (4, 2)
+    np.testing.assert_allclose(jacfwd(g)(a, b), torch.cat([ra, rb], dim=1), rtol=1e-12, atol=1e-13)
