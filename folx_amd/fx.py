@@ -276,6 +276,13 @@ RULES = {
     aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
     operator.getitem: _item,
     aten.sign.default: fnp.sign, aten.sgn.default: fnp.sign,
+    # a constant that only borrows the SHAPE of a data tensor (the seed of a gradient taken inside the function, ...)
+    aten.ones_like.default: lambda a, **_: np.ones(_shape(a), np.float32),
+    aten.zeros_like.default: lambda a, **_: np.zeros(_shape(a), np.float32),
+    aten.full_like.default: lambda a, value, **_: np.full(_shape(a), float(value), np.float32),
+    aten.new_ones.default: lambda a, size, **_: np.ones(tuple(int(n) for n in size), np.float32),
+    aten.new_zeros.default: lambda a, size, **_: np.zeros(tuple(int(n) for n in size), np.float32),
+    aten.new_full.default: lambda a, size, value, **_: np.full(tuple(int(n) for n in size), float(value), np.float32),
     aten.index_select.default: lambda a, dim, index: fnp.take(a, np.asarray(index), axis=int(dim)),
     aten.take.default: lambda a, index: fnp.take(a, np.asarray(index)),
     aten.squeeze_.dim: lambda a, dim: _squeeze(a, (dim,)), aten.unsqueeze_.default: lambda a, dim: fnp.expand_dims(a, int(dim)),
