@@ -106,6 +106,20 @@ def test_matrix_rules_in_models_beyond_32(name):
     assert_lap(out.laplacian, ref.lap, name + ' laplacian')
 
 
+def test_attention_at_shapes_the_kernels_do_not_take():
+    """d = 6 (no multiple of 4) with a padded sequence, and the smallest shape of
+    test/experimental/pallas/test_attention.py:323 (one electron, one head of one feature)."""
+    from test_host_logic import masked_attention_beyond_kernel_sizes
+
+    run = lambda fn, x, thr: folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fn(fnp, t), thr))(torch.as_tensor(x).cuda())  # noqa: E731
+    to_np = lambda o: (o.x.cpu().numpy().astype(np.float64), o.jacobian.dense_array.cpu().numpy().astype(np.float64),  # noqa: E731
+                       o.laplacian.cpu().numpy().astype(np.float64))
+    print('case attention n=5 H=2 d=6 valid=3', flush=True)
+    masked_attention_beyond_kernel_sizes(run, to_np)
+    print('case attention n=1 H=1 d=1', flush=True)
+    masked_attention_beyond_kernel_sizes(run, to_np, n=1, H=1, d=1, valid=1, B=1)
+
+
 def test_masked_attention_on_more_than_64_positions():
     """70 electrons of which 50 are real (the coordinates of the others inactive), 2 heads of 8: beyond the attention
     kernels' n <= 64, so the rule runs through the product and softmax rules with the masks applied; valid rows equal
