@@ -238,6 +238,9 @@ class FwdLaplArray:
         return FwdLaplArray(self.x, self.jacobian.as_dense, self.laplacian)
 
     # ---- operator sugar (the reference gets this from tracing jnp code) ----------------
+    # numpy leaves `array <op> triplet` to the reflected methods below instead of broadcasting over the tuple
+    __array_ufunc__ = None
+
     def __add__(self, o):
         from . import numpy as fnp
 
@@ -293,6 +296,71 @@ class FwdLaplArray:
 
         return fnp.getitem(self, idx)
 
+    def __rmatmul__(self, W):
+        from . import numpy as fnp
+
+        return fnp.matmul(W, self)
+
+    def __pow__(self, e):
+        from . import numpy as fnp
+
+        if isinstance(e, (int, np.integer)) and not isinstance(e, bool):
+            return fnp.integer_pow(self, int(e))
+        return fnp.power(self, e)
+
+    def __rpow__(self, base):
+        from . import numpy as fnp
+
+        return fnp.power(base, self)
+
+    def __abs__(self):
+        from . import numpy as fnp
+
+        return fnp.abs(self)
+
+    # comparisons give values without derivatives (== and != stay the tuple's own)
+    def __gt__(self, o):
+        from . import numpy as fnp
+
+        return fnp.greater(self, o)
+
+    def __ge__(self, o):
+        from . import numpy as fnp
+
+        return fnp.greater_equal(self, o)
+
+    def __lt__(self, o):
+        from . import numpy as fnp
+
+        return fnp.less(self, o)
+
+    def __le__(self, o):
+        from . import numpy as fnp
+
+        return fnp.less_equal(self, o)
+
+    @property
+    def T(self):
+        from . import numpy as fnp
+
+        return fnp.transpose(self, tuple(reversed(range(len(self.shape)))))
+
+    def transpose(self, *axes):
+        from . import numpy as fnp
+
+        if len(axes) == 1 and isinstance(axes[0], (tuple, list)):
+            axes = tuple(axes[0])
+        return fnp.transpose(self, axes if axes else tuple(reversed(range(len(self.shape)))))
+
+    def swapaxes(self, a, b):
+        from . import numpy as fnp
+
+        return fnp.swapaxes(self, a, b)
+
+    def mean(self, axis=None, keepdims=False):
+        from . import numpy as fnp
+
+        return fnp.mean(self, axis=axis, keepdims=keepdims)
     def reshape(self, *shape):
         from . import numpy as fnp
 

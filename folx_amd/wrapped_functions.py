@@ -756,6 +756,7 @@ class Deferred:
     way the triplet is the one the ordinary rules define."""
 
     __slots__ = ('_value', 'thr')
+    __array_ufunc__ = None   # `array <op> handle` goes to the reflected methods
 
     def __init__(self, thr: int):
         self._value, self.thr = None, int(thr)
@@ -795,7 +796,8 @@ class Deferred:
 
 
 for _name in ('__add__', '__radd__', '__sub__', '__rsub__', '__mul__', '__rmul__', '__truediv__', '__rtruediv__',
-              '__neg__', '__matmul__', '__getitem__', 'reshape', 'sum'):
+              '__neg__', '__matmul__', '__getitem__', 'reshape', 'sum', '__rmatmul__', '__pow__', '__rpow__', '__abs__',
+              '__gt__', '__ge__', '__lt__', '__le__', 'T', 'transpose', 'swapaxes', 'mean'):
     setattr(Deferred, _name, getattr(FwdLaplArray, _name))  # the same sugar: everything goes through folx_amd.numpy
 
 

@@ -1066,3 +1066,39 @@ def test_ad_helpers_have_the_reference_shapes_and_values():
     ra, rb = jacrev(g)(a, b)
     assert ra.shape == (4, 4) and rb.shape == (4, 2)
     np.testing.assert_allclose(jacfwd(g)(a, b), torch.cat([ra, rb], dim=1), rtol=1e-12, atol=1e-13)
+
+
+def test_python_operators_on_triplets(monkeypatch):
+    """A model written with Python operators only (the reference gets these from tracing jnp code): numpy and torch
+    constants on either side (numpy defers to the reflected methods instead of broadcasting over the tuple), powers,
+    comparisons, ``.T`` / ``.swapaxes`` / ``.mean``; also on values that are still deferred."""
+    cpu_kernels.install(monkeypatch)
+    rng = np.random.default_rng(0)
+    W = rng.normal(size=(4, 5)).astype(np.float32)
+    V = rng.normal(size=(3, 3)).astype(np.float32)
+    c = rng.normal(size=(5,)).astype(np.float32)
+    Vt, ct = torch.as_tensor(V), torch.as_tensor(c)
+
+    def f(x):           # x (3, 4)
+        h = fnp.tanh(x @ W)
+        g = (V @ h) ** 2 + abs(h) ** 1.5 - 2.0 ** (h * 0.3) + c * h - c / (2.0 + h ** 2) + (Vt @ h) * ct
+        m = fnp.where(h > 0.1, g, -g.T.T)
+        lazy = fnp.dot(h, W.T.copy())                                   # a deferred product: the same sugar
+        return (m / (1.0 + h.mean(axis=-1, keepdims=True) ** 2)).swapaxes(0, 1).sum(axis=0) + (lazy ** 2).T.sum(axis=0)[:3]
+
+    def t(x):
+        Wd, Vd, cd = (torch.as_tensor(a, dtype=x.dtype) for a in (W, V, c))
+        h = torch.tanh(x @ Wd)
+        g = (Vd @ h) ** 2 + abs(h) ** 1.5 - 2.0 ** (h * 0.3) + cd * h - cd / (2.0 + h ** 2) + (Vd @ h) * cd
+        m = torch.where(h > 0.1, g, -g)
+        return (m / (1.0 + h.mean(-1, keepdim=True) ** 2)).swapaxes(0, 1).sum(0) + ((h @ Wd.T) ** 2).T.sum(0)[:3]
+
+    x = rng.normal(size=(2, 3, 4)).astype(np.float32)
+    y, J, L = brute_force(t, x.astype(np.float64))
+    for thr in (0, 4, 12):
+        out = folx_amd.vmap(folx_amd.forward_laplacian(f, thr))(x)
+        np.testing.assert_allclose(out.x.numpy(), y, rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(out.jacobian.dense_array.numpy(), J.reshape(tuple(out.jacobian.dense_array.shape)), rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(out.laplacian.numpy(), L, rtol=1e-4, atol=1e-4)
+    with pytest.raises(TypeError):
+        np.add(c, folx_amd.vmap(folx_amd.forward_laplacian(lambda z: z, 0))(x))   # numpy functions do not take triplets
