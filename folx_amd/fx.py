@@ -122,6 +122,8 @@ def _select(a, dim, index):
 
 
 def _index(a, indices):
+    if any(isinstance(i, BatchedArray) for i in indices):
+        return _index_dynamic(a, list(indices))
     idx = tuple(slice(None) if i is None else np.asarray(i) for i in indices)
     return fnp.getitem(a, idx)
 
@@ -200,6 +202,376 @@ def _item(a, i):
     return v.make() if isinstance(v, _OnDemand) else v
 
 
+def _vector_norm(a, ord=2, dim=None, keepdim=False, dtype=None):
+    nd = len(_shape(a))
+    axes = _dims(dim, nd)
+    o = float(ord)
+    if o == 2.0:
+        out = fnp.sqrt(fnp.sum(fnp.square(a), axis=axes, keepdims=bool(keepdim)))
+    elif o == 1.0:
+        out = fnp.sum(fnp.abs(a), axis=axes, keepdims=bool(keepdim))
+    elif o == float('inf'):
+        out = _fold_axes(fnp.amax, fnp.abs(a), axes, keepdim)
+    elif o == -float('inf'):
+        out = _fold_axes(fnp.amin, fnp.abs(a), axes, keepdim)
+    else:
+        out = fnp.power(fnp.sum(fnp.power(fnp.abs(a), o), axis=axes, keepdims=bool(keepdim)), 1.0 / o)
+    return out
+
+
+def _var(root):
+    def rule(a, dim=None, correction=1, keepdim=False):
+        nd = len(_shape(a))
+        axes = _dims(dim, nd)
+        n = int(np.prod([_shape(a)[i] for i in axes], dtype=int))
+        c = 1 if correction is None else correction
+        centred = fnp.subtract(a, fnp.mean(a, axis=axes, keepdims=True))
+        v = fnp.multiply(fnp.sum(fnp.square(centred), axis=axes, keepdims=bool(keepdim)), 1.0 / max(n - float(c), 1e-30))
+        return fnp.sqrt(v) if root else v
+
+    return rule
+
+
+def _split(a, size, dim=0):
+    s = _shape(a)
+    dim = int(dim) % len(s)
+    sizes = [int(n) for n in size] if isinstance(size, (list, tuple)) else \
+        [min(int(size), s[dim] - lo) for lo in range(0, s[dim], int(size))]
+    out, lo = [], 0
+    for n in sizes:
+        out.append(_slice(a, dim, lo, lo + n))
+        lo += n
+    return tuple(out)
+
+
+def _triangle(lower):
+    def rule(a, diagonal=0):
+        n, m = _shape(a)[-2:]
+        keep = (np.tril if lower else np.triu)(np.ones((n, m), dtype=np.float32), int(diagonal))
+        return fnp.multiply(a, keep)
+
+    return rule
+
+
+def _roll(a, shifts, dims=()):
+    if not dims:   # the flattened array is rolled
+        return fnp.reshape(fnp.roll(fnp.reshape(a, (-1,)), int(shifts[0]), 0), _shape(a))
+    for sh, ax in zip(shifts, dims):
+        a = fnp.roll(a, int(sh), int(ax) % len(_shape(a)))
+    return a
+
+
+def _masked_fill(a, mask, value):
+    return fnp.where(mask, value if _is_t(value) else np.float32(value), a)
+
+
+def _gather(a, dim, index, sparse_grad=False):
+    """``out[i][j][k] = a[i][index[i][j][k]][k]`` (for dim 1): integer-array indexing with the other axes' own positions."""
+    if isinstance(index, BatchedArray):
+        assert tuple(index.shape) == tuple(n if ax != int(dim) % len(_shape(a)) else index.shape[ax] for ax, n in enumerate(_shape(a))), \
+            'gather with walker-dependent indices: the index covers the other axes whole'
+        return _select_along(a, index, int(dim))
+    idx = np.asarray(index)
+    nd = idx.ndim
+    dim = int(dim) % nd
+    grids = np.meshgrid(*[np.arange(n) for n in idx.shape], indexing='ij') if nd else []
+    return fnp.getitem(a, tuple(idx if ax == dim else grids[ax] for ax in range(nd)))
+
+
+def _sdpa(q, k, v, dropout_p=0.0, is_causal=False, attn_mask=None, scale=None, **_):
+    """``softmax(q k^T scale (+ mask)) v`` with q, k, v ``(..., H, n, d)``: the attention rule when nothing is masked
+    (one leading batch axis of extent one at most), the product and softmax rules otherwise."""
+    assert float(dropout_p) == 0.0, 'scaled_dot_product_attention: dropout has no forward Laplacian'
+    sq, sk = _shape(q), _shape(k)
+    d, n, m = sq[-1], sq[-2], sk[-2]
+    sc = float(scale) if scale is not None else 1.0 / float(np.sqrt(d))
+    lead = sq[:-3]
+    if attn_mask is None and not is_causal and n == m and all(x == 1 for x in lead) and len(sq) >= 3 and sq == sk == _shape(v):
+        H = sq[-3]
+        to_nhd = lambda t: fnp.transpose(fnp.reshape(t, (H, n, d)), (1, 0, 2))    # noqa: E731
+        o = fnp.multi_head_self_attention(fnp.multiply(to_nhd(q), sc), to_nhd(k), to_nhd(v))
+        return fnp.reshape(fnp.transpose(o, (1, 0, 2)), sq)
+    scores = fnp.multiply(fnp.matmul(q, fnp.swapaxes(k, -1, -2)), sc)
+    if is_causal:
+        scores = fnp.where(np.tril(np.ones((n, m), dtype=bool)), scores, np.float32(-1e30))
+    if attn_mask is not None:
+        am = attn_mask
+        if not _is_t(am) and np.asarray(am).dtype == bool:
+            scores = fnp.where(np.asarray(am), scores, np.float32(-1e30))
+        else:
+            scores = fnp.add(scores, am)
+    return fnp.matmul(fnp.softmax(scores, axis=-1), v)
+
+
+def _cdist(a, b, p=2.0, compute_mode=None):
+    diff = fnp.subtract(fnp.expand_dims(a, -2), fnp.expand_dims(b, -3))
+    return _vector_norm(diff, p, (-1,), False)
+
+
+def _log_sigmoid(a):
+    out = fnp.negative(fnp.softplus(fnp.negative(a)))
+    return out, None
+
+
+def _elu(a, alpha=1.0, scale=1.0, input_scale=1.0):
+    """``scale * (x > 0 ? x : alpha * (exp(input_scale * x) - 1))`` (selu and celu arrive in this form)."""
+    if float(input_scale) == 1.0:
+        out = fnp.elu(a, float(alpha))
+    else:
+        out = fnp.where(fnp.greater(fnp.stop_gradient(a), 0.0), a,
+                        fnp.multiply(fnp.expm1(fnp.multiply(a, float(input_scale))), float(alpha)))
+    return out if float(scale) == 1.0 else fnp.multiply(out, float(scale))
+
+
+def _solve_ex(A, B, left=True, check_errors=False):
+    if left:
+        return fnp.solve(A, B), None, None, None
+    # X A = B  <=>  A^T X^T = B^T
+    vec = len(_shape(B)) == len(_shape(A)) - 1
+    Bt = B if vec else fnp.swapaxes(B, -1, -2)
+    X = fnp.solve(fnp.swapaxes(A, -1, -2), Bt)
+    return (X if vec else fnp.swapaxes(X, -1, -2)), None, None, None
+
+
+def _div_mode(a, b, rounding_mode=None):
+    q = fnp.divide(a, b)
+    if rounding_mode is None:
+        return q
+    return fnp.trunc(q) if rounding_mode == 'trunc' else fnp.floor(q)
+
+
+def _prod_all(a, dtype=None):
+    return fnp.prod(fnp.reshape(a, (-1,)), axis=0)
+
+
+def _index_tuple(nd, dim, item):
+    return (*([slice(None)] * (int(dim) % nd)), item)
+
+
+def _copy(dst, src, non_blocking=False):
+    """The functional form of ``dst.copy_(src)``: ``src`` with the shape of ``dst``."""
+    return _expand(src, _shape(dst)) if _shape(src) != _shape(dst) else src
+
+
+def _slice_scatter(a, src, dim=0, start=None, end=None, step=1):
+    n = _shape(a)[int(dim) % len(_shape(a))]
+    end = None if end is None or end >= n else end
+    return fnp.scatter(a, _index_tuple(len(_shape(a)), dim, slice(start, end, step)), src, 'set')
+
+
+def _select_scatter(a, src, dim, index):
+    return fnp.scatter(a, _index_tuple(len(_shape(a)), dim, int(index)), src, 'set')
+
+
+def _index_put(a, indices, values, accumulate=False):
+    idx = tuple(slice(None) if i is None else np.asarray(i) for i in indices)
+    return fnp.scatter(a, idx, values, 'add' if accumulate else 'set')
+
+
+def _repeat(a, repeats):
+    reps = [int(r) for r in repeats]
+    s = _shape(a)
+    if len(reps) > len(s):
+        a = fnp.reshape(a, (1,) * (len(reps) - len(s)) + s)
+    return fnp.tile(a, tuple(reps))
+
+
+def _constant_pad(a, pad, value=0.0):
+    nd = len(_shape(a))
+    cfg = [(0, 0, 0)] * nd
+    for i in range(len(pad) // 2):          # pairs run from the LAST axis backwards; negative widths crop
+        cfg[nd - 1 - i] = (int(pad[2 * i]), int(pad[2 * i + 1]), 0)
+    return fnp.lax_pad(a, np.float32(value), tuple(cfg))
+
+
+def _extreme_all(fn):
+    def rule(a):
+        return fn(fnp.reshape(a, (-1,)), axis=0)
+
+    return rule
+
+
+def _frac(a):
+    return fnp.subtract(a, fnp.trunc(a))
+
+
+def _py_mod(a, b):
+    """Python-style remainder ``a - b floor(a / b)`` (``torch.remainder``); the quotient is piecewise constant."""
+    return fnp.subtract(a, fnp.multiply(b, fnp.floor(fnp.divide(fnp.stop_gradient(a), fnp.stop_gradient(b) if _is_t(b) else b))))
+
+
+def _lerp(a, b, w):
+    return fnp.add(a, fnp.multiply(w, fnp.subtract(b, a)))
+
+
+def _xlogy(a, b):
+    return fnp.multiply(a, fnp.log(b))
+
+
+def _dist(a, b, p=2):
+    return _vector_norm(fnp.subtract(a, b), p, None, False)
+
+
+def _logcumsumexp(a, dim):
+    """Shifted by the (derivative-free) maximum along the axis, like ``logsumexp``."""
+    nd = len(_shape(a))
+    ax = int(dim) % nd
+    m = fnp.amax_const(a, (ax,), keepdims=True)
+    return fnp.add(fnp.log(fnp.cumsum(fnp.exp(fnp.subtract(a, m)), axis=ax)), m)
+
+
+def _loss(pointwise):
+    def rule(a, b, reduction=1, *extra):
+        v = pointwise(fnp.subtract(a, b), *extra)
+        return v if reduction == 0 else (fnp.mean(v) if reduction == 1 else fnp.sum(v))
+
+    return rule
+
+
+def _huber(diff, delta=1.0):
+    """``0.5 d^2`` for ``|d| < delta``, ``delta (|d| - 0.5 delta)`` beyond."""
+    delta = float(delta)
+    ad = fnp.abs(diff)
+    return fnp.where(fnp.less(fnp.stop_gradient(ad), delta), fnp.multiply(fnp.square(diff), 0.5),
+                     fnp.multiply(fnp.subtract(ad, 0.5 * delta), delta))
+
+
+def _smooth_l1(diff, beta=1.0):
+    beta = float(beta)
+    return fnp.abs(diff) if beta == 0.0 else fnp.multiply(_huber(diff, beta), 1.0 / beta)
+
+
+def _glu(a, dim=-1):
+    s = _shape(a)
+    ax = int(dim) % len(s)
+    h = s[ax] // 2
+    return fnp.multiply(_slice(a, ax, 0, h), fnp.sigmoid(_slice(a, ax, h, 2 * h)))
+
+
+def _hard(lo, hi, scale, times_x):
+    """``clip(x + 3, 0, 6) / 6`` family."""
+    def rule(a):
+        g = fnp.multiply(fnp.clip(fnp.add(a, 3.0), lo, hi), scale)
+        return fnp.multiply(a, g) if times_x else g
+
+    return rule
+
+
+def _shrink(soft):
+    def rule(a, lambd=0.5):
+        lam = float(lambd)
+        v = fnp.stop_gradient(a)
+        if soft:
+            return fnp.where(fnp.greater(v, lam), fnp.subtract(a, lam), fnp.where(fnp.less(v, -lam), fnp.add(a, lam), np.float32(0.0)))
+        return fnp.where(fnp.logical_or(fnp.greater(v, lam), fnp.less(v, -lam)), a, np.float32(0.0))
+
+    return rule
+
+
+def _trilinear(i1, i2, i3, expand1, expand2, expand3, sumdim, unroll_dim=1):
+    """``(i1.unsqueeze(expand1) * i2.unsqueeze(expand2) * i3.unsqueeze(expand3)).sum(sumdim)`` (what ``bilinear`` lowers to)."""
+    def grow(t, dims):
+        for dm in sorted(int(v) for v in dims):
+            t = fnp.expand_dims(t, dm) if _is_t(t) else (t.unsqueeze(dm) if isinstance(t, torch.Tensor) else np.expand_dims(t, dm))
+        return t
+
+    prod = fnp.multiply(fnp.multiply(grow(i1, expand1), grow(i2, expand2)), grow(i3, expand3))
+    return fnp.sum(prod, axis=tuple(int(v) for v in sumdim))
+
+
+def _values_of(a):
+    """The values of a triplet / walker-dependent array as a torch tensor (B, *shape), or None for a constant."""
+    from .wrapped_functions import force
+
+    a = force(a)
+    if isinstance(a, FwdLaplArray):
+        return a.x
+    if isinstance(a, BatchedArray):
+        return a.data
+    return None
+
+
+def _select_along(a, index: BatchedArray, axis: int):
+    """``take_along_axis(a, index, axis)`` for indices that differ per walker (the positions of a sort, an arg-maximum):
+    a 0 / 1 selection ``index == m`` over the ``n`` entries of the axis, multiplied in and summed -- linear in ``a``,
+    ``n`` times the work of a static gather."""
+    s = _shape(a)
+    ax = axis % len(s)
+    n = s[ax]
+    pick = index.data.unsqueeze(ax + 2) == torch.arange(n, device=index.data.device).reshape((n,) + (1,) * (len(s) - 1 - ax))
+    src = fnp.expand_dims(a, ax)                                       # (..., 1, n, ...): broadcast over the picked slot
+    return fnp.sum(fnp.where(BatchedArray(pick), src, np.float32(0.0)), axis=ax + 1)
+
+
+def _sort(a, dim=-1, descending=False, stable=False):
+    v = _values_of(a)
+    if v is None:
+        r = torch.sort(torch.as_tensor(a), dim=int(dim), descending=bool(descending))
+        return _const(r.values), _const(r.indices)
+    ax = int(dim) % (v.dim() - 1)
+    idx = BatchedArray(torch.argsort(v, dim=ax + 1, descending=bool(descending), stable=True))
+    return (_select_along(a, idx, ax) if _is_t(a) and not isinstance(a, BatchedArray) else
+            BatchedArray(torch.gather(v, ax + 1, idx.data))), idx
+
+
+def _topk(a, k, dim=-1, largest=True, sorted=True):
+    v = _values_of(a)
+    if v is None:
+        r = torch.topk(torch.as_tensor(a), int(k), dim=int(dim), largest=bool(largest))
+        return _const(r.values), _const(r.indices)
+    ax = int(dim) % (v.dim() - 1)
+    idx = BatchedArray(torch.topk(v, int(k), dim=ax + 1, largest=bool(largest)).indices)
+    return (_select_along(a, idx, ax) if not isinstance(a, BatchedArray) else BatchedArray(torch.gather(v, ax + 1, idx.data))), idx
+
+
+def _index_dynamic(a, indices):
+    """``a[i0, i1, ...]`` where some integer arrays differ per walker: the indexed axes (consecutive ones) are flattened
+    into one, the flat position ``sum_j i_j stride_j`` is formed per walker, and the entries are picked by
+    ``_select_along``."""
+    s = _shape(a)
+    where_ = [i for i, ix in enumerate(indices) if ix is not None]
+    assert where_ == list(range(where_[0], where_[-1] + 1)), 'index arrays on consecutive axes only'
+    lo, hi = where_[0], where_[-1] + 1
+    dims = s[lo:hi]
+    dev = next(ix.data.device for ix in indices if isinstance(ix, BatchedArray))
+    B = next(ix.data.shape[0] for ix in indices if isinstance(ix, BatchedArray))
+    flat, stride = 0, 1
+    for ix, n in zip(reversed(indices[lo:hi]), reversed(dims)):
+        t = ix.data.long() if isinstance(ix, BatchedArray) else torch.as_tensor(np.asarray(ix), device=dev).long()[None]
+        flat = flat + torch.where(t < 0, t + n, t) * stride
+        stride *= n
+    ishape = tuple(flat.shape[1:])
+    flat = flat.expand(B, *ishape)
+    # (lead..., N, tail...) -> pick along N for every index entry
+    src = fnp.reshape(a, (*s[:lo], int(np.prod(dims, dtype=int)), *s[hi:]))
+    lead, tail = s[:lo], s[hi:]
+    k = int(np.prod(ishape, dtype=int))
+    idx = flat.reshape(B, *([1] * len(lead)), k, *([1] * len(tail))).expand(B, *lead, k, *tail)
+    out = _select_along(src, BatchedArray(idx), lo)
+    return fnp.reshape(out, (*lead, *ishape, *tail))
+
+
+def _arg(fn, a, dim, keepdim):
+    if dim is None:
+        return fn(fnp.reshape(a, (-1,)), axis=0)
+    out = fn(a, axis=int(dim))
+    return fnp.expand_dims(out, int(dim)) if keepdim else out
+
+
+def _group_norm(a, weight, bias, N, C, HxW, group, eps):
+    """Normalisation over each group of ``C / group`` channels and all positions behind them; (out, mean, rstd)."""
+    s = _shape(a)
+    out = fnp.layer_norm(fnp.reshape(a, (int(N), int(group), -1)), None, None, float(eps))
+    out = fnp.reshape(out, s)
+    per_channel = (1, int(C)) + (1,) * (len(s) - 2)
+    shaped = lambda t: fnp.reshape(t, per_channel) if _is_t(t) else t.reshape(per_channel)    # noqa: E731  (numpy or torch constant)
+    if weight is not None:
+        out = fnp.multiply(out, shaped(weight))
+    if bias is not None:
+        out = fnp.add(out, shaped(bias))
+    return out, None, None
+
+
 def _clamp(a, lo=None, hi=None):
     return fnp.clip(a, lo, hi)
 
@@ -228,7 +600,7 @@ RULES = {
     aten.asin.default: fnp.arcsin, aten.acos.default: fnp.arccos, aten.asinh.default: fnp.arcsinh,
     aten.acosh.default: fnp.arccosh, aten.atanh.default: fnp.arctanh, aten.exp2.default: fnp.exp2,
     aten.lgamma.default: fnp.lgamma, aten.digamma.default: fnp.digamma, aten.atan2.default: fnp.arctan2,
-    aten.softplus.default: _softplus, aten.elu.default: lambda a, alpha=1.0, scale=1.0, input_scale=1.0: fnp.elu(a, alpha),
+    aten.softplus.default: _softplus, aten.elu.default: _elu,
     aten.leaky_relu.default: lambda a, negative_slope=0.01: fnp.leaky_relu(a, negative_slope),
     aten.pow.Tensor_Scalar: _pow_scalar, aten.pow.Tensor_Tensor: fnp.power, aten.pow.Scalar: lambda b, e: fnp.power(float(b), e),
     aten.square.default: fnp.square,
@@ -273,7 +645,7 @@ RULES = {
     aten._linalg_slogdet.default: lambda A: (*fnp.slogdet(A), None, None),
     aten._linalg_det.default: lambda A: (fnp.det(A), None, None),
     aten.linalg_inv_ex.default: lambda A, check_errors=False: (fnp.inv(A), None),
-    aten._linalg_solve_ex.default: lambda A, B, left=True, check_errors=False: (fnp.solve(A, B), None, None, None),
+    aten._linalg_solve_ex.default: _solve_ex,
     operator.getitem: _item,
     aten.sign.default: fnp.sign, aten.sgn.default: fnp.sign,
     # a constant that only borrows the SHAPE of a data tensor (the seed of a gradient taken inside the function, ...)
@@ -287,6 +659,65 @@ RULES = {
     aten.take.default: lambda a, index: fnp.take(a, np.asarray(index)),
     aten.squeeze_.dim: lambda a, dim: _squeeze(a, (dim,)), aten.unsqueeze_.default: lambda a, dim: fnp.expand_dims(a, int(dim)),
     aten._safe_softmax.default: lambda a, dim, dtype=None: fnp.softmax(a, axis=int(dim)),
+    aten.linalg_vector_norm.default: _vector_norm,
+    aten.var.correction: _var(False), aten.std.correction: _var(True),
+    aten.split.Tensor: _split, aten.split_with_sizes.default: _split,
+    aten.tril.default: _triangle(True), aten.triu.default: _triangle(False),
+    aten.diagonal.default: lambda a, offset=0, dim1=0, dim2=1: fnp.diagonal(fnp.moveaxis(a, (int(dim1), int(dim2)), (-2, -1)), int(offset)),
+    aten.trace.default: fnp.trace,
+    aten.baddbmm.default: _addmm, aten.addmv.default: _addmm, aten.addbmm.default:
+        lambda bias, a, b, beta=1, alpha=1: fnp.add(_scaled(fnp.sum(fnp.matmul(a, b), axis=0), alpha), _scaled(bias, beta)),
+    aten.addcmul.default: lambda a, t1, t2, value=1: fnp.add(a, _scaled(fnp.multiply(t1, t2), value)),
+    aten.addcdiv.default: lambda a, t1, t2, value=1: fnp.add(a, _scaled(fnp.divide(t1, t2), value)),
+    aten.masked_fill.Scalar: _masked_fill, aten.masked_fill.Tensor: _masked_fill,
+    aten.roll.default: _roll,
+    aten.gather.default: _gather,
+    aten._linalg_check_errors.default: lambda *a, **k: None,
+    aten.mish.default: lambda a: fnp.multiply(a, fnp.tanh(fnp.softplus(a))),
+    aten.sort.default: _sort, aten.sort.stable: lambda a, stable=False, dim=-1, descending=False: _sort(a, dim, descending),
+    aten.topk.default: _topk,
+    aten.norm.ScalarOpt_dim: lambda a, p=2, dim=None, keepdim=False: _vector_norm(a, 2 if p is None else p, dim, keepdim),
+    aten.norm.Scalar: lambda a, p=2: _vector_norm(a, p, None, False),
+    aten.native_group_norm.default: _group_norm,
+    aten.argmax.default: lambda a, dim=None, keepdim=False: _arg(fnp.argmax, a, dim, keepdim),
+    aten.argmin.default: lambda a, dim=None, keepdim=False: _arg(fnp.argmin, a, dim, keepdim),
+    aten.empty_like.default: lambda a, **_: np.zeros(_shape(a), np.float32),
+    aten.copy.default: _copy, aten.slice_scatter.default: _slice_scatter, aten.select_scatter.default: _select_scatter,
+    aten.index_put.default: _index_put,
+    aten.repeat.default: _repeat, aten.constant_pad_nd.default: _constant_pad,
+    aten.max.default: _extreme_all(fnp.amax), aten.min.default: _extreme_all(fnp.amin),
+    aten.floor.default: fnp.floor, aten.ceil.default: fnp.ceil, aten.round.default: fnp.round, aten.trunc.default: fnp.trunc,
+    aten.frac.default: _frac, aten.fmod.Scalar: fnp.remainder, aten.fmod.Tensor: fnp.remainder,
+    aten.remainder.Scalar: _py_mod, aten.remainder.Tensor: _py_mod,
+    aten.lerp.Scalar: _lerp, aten.lerp.Tensor: _lerp,
+    aten.hypot.default: lambda a, b: fnp.sqrt(fnp.add(fnp.square(a), fnp.square(b))),
+    aten.logaddexp.default: fnp.logaddexp, aten.xlogy.Tensor: _xlogy, aten.dist.default: _dist,
+    aten.logcumsumexp.default: _logcumsumexp,
+    aten.mse_loss.default: _loss(fnp.square), aten.l1_loss.default: _loss(fnp.abs),
+    aten.huber_loss.default: _loss(_huber), aten.smooth_l1_loss.default: _loss(_smooth_l1),
+    aten.glu.default: _glu,
+    aten.hardswish.default: _hard(0.0, 6.0, 1.0 / 6.0, True), aten.hardsigmoid.default: _hard(0.0, 6.0, 1.0 / 6.0, False),
+    aten.relu6.default: lambda a: fnp.clip(a, 0.0, 6.0),
+    aten.softshrink.default: _shrink(True), aten.hardshrink.default: _shrink(False),
+    aten.threshold.default: lambda a, threshold, value: fnp.where(fnp.greater(fnp.stop_gradient(a), float(threshold)), a, np.float32(value)),
+    aten.rrelu_with_noise.default: lambda a, noise, lower=0.125, upper=1.0 / 3.0, training=False, generator=None:
+        fnp.leaky_relu(a, (float(lower) + float(upper)) / 2.0),
+    aten._prelu_kernel.default: lambda a, w: fnp.where(fnp.greater(fnp.stop_gradient(a), 0.0), a, fnp.multiply(a, w)),
+    aten._trilinear.default: _trilinear,
+    aten.unsafe_split.Tensor: _split, aten.unsafe_split_with_sizes.default: _split, aten.unsafe_chunk.default:
+        lambda a, chunks, dim=0: _split(a, -(-_shape(a)[int(dim) % len(_shape(a))] // int(chunks)), dim),
+    aten.celu.default: lambda a, alpha=1.0: _elu(a, float(alpha), 1.0, 1.0 / float(alpha)),
+    aten.clamp.Tensor: _clamp, aten.clamp_min.Tensor: lambda a, lo: fnp.maximum(a, lo), aten.clamp_max.Tensor: lambda a, hi: fnp.minimum(a, hi),
+    aten.div.Tensor_mode: _div_mode, aten.div.Scalar_mode: _div_mode,
+    aten.prod.default: _prod_all,
+    aten.where.ScalarSelf: fnp.where, aten.where.ScalarOther: fnp.where, aten.where.Scalar: fnp.where,
+    aten.log_sigmoid_forward.default: _log_sigmoid,
+    aten.hardtanh.default: lambda a, lo=-1.0, hi=1.0: fnp.clip(a, float(lo), float(hi)),
+    aten._scaled_dot_product_flash_attention_for_cpu.default: lambda q, k, v, dropout_p=0.0, is_causal=False, attn_mask=None,
+        scale=None: (_sdpa(q, k, v, dropout_p, is_causal, attn_mask, scale), None),
+    aten._scaled_dot_product_attention_math.default: lambda q, k, v, attn_mask=None, dropout_p=0.0, is_causal=False,
+        dropout_mask=None, scale=None, enable_gqa=False: (_sdpa(q, k, v, dropout_p, is_causal, attn_mask, scale), None),
+    aten._cdist_forward.default: _cdist,
     torch.ops.folx_amd.multi_head_self_attention.default: fnp.multi_head_self_attention,
 }
 
@@ -316,11 +747,67 @@ def _logsumexp(a, dims, keepdim):
     return fnp.expand_dims(out, axes[0]) if keepdim else out
 
 
+def _functional_form(target):
+    """``aten.add_.Tensor`` -> ``aten.add.Tensor`` when that has a rule, else None."""
+    name = getattr(target, '_schema', None)
+    if name is None:
+        return None
+    base = target._schema.name.split('::')[-1]
+    if not base.endswith('_') or base.endswith('__'):
+        return None
+    packet = getattr(aten, base[:-1], None)
+    functional = getattr(packet, target._overloadname, None) if packet is not None else None
+    return functional if functional in RULES else None
+
+
+def _disjoint_part_of_a_dead_tensor(part, at, order):
+    """``part`` is one piece of a split / chunk / unbind whose source nobody reads any more (only the split itself
+    does): updating the piece in place touches nothing else that the graph still looks at (the gates of a GRU cell)."""
+    if part.target is not operator.getitem:
+        return False
+    split = part.args[0]
+    if not isinstance(split, torch.fx.Node) or split.target not in _SPLITS:
+        return False
+    source = split.args[0]
+    return isinstance(source, torch.fx.Node) and all(u is split or order[u] < order[at] for u in source.users)
+
+
+_SPLITS = {aten.split.Tensor, aten.split_with_sizes.default, aten.unbind.int, aten.unsafe_split.Tensor,
+           aten.unsafe_split_with_sizes.default, aten.unsafe_chunk.default}
+_VIEWS = {aten.slice.Tensor, aten.select.int, aten.view.default, aten._unsafe_view.default, aten.reshape.default,
+          aten.transpose.int, aten.permute.default, aten.t.default, aten.expand.default, aten.unsqueeze.default,
+          aten.squeeze.dim, aten.squeeze.dims, aten.squeeze.default, aten.diagonal.default, aten.alias.default,
+          aten.detach.default, aten.unbind.int, aten.split.Tensor, aten.split_with_sizes.default, operator.getitem}
+
+
 def _generic(target):
     """An ATen operation without an entry above: the generic rule built from the operation itself, with the warning
     the reference gives for a primitive outside its registry (folx/wrapped_functions.py:609-614)."""
     def rule(*args, **kwargs):
         logging.warning(f'{target} has no forward-Laplacian rule; the following call computes the full Hessian of the operation')
+        if any(isinstance(v, (list, tuple)) and _any_triplet(v) for v in args):
+            # a list of tensors (block_diag, ...): the wrapped function takes its entries one by one
+            spans, flat = [], []
+            for v in args:
+                if isinstance(v, (list, tuple)) and _any_triplet(v):
+                    spans.append((len(flat), len(v)))
+                    flat.extend(v)
+                else:
+                    spans.append(None)
+                    flat.append(v)
+
+            def packed(*a):
+                it, full = 0, []
+                for sp in spans:
+                    if sp is None:
+                        full.append(a[it])
+                        it += 1
+                    else:
+                        full.append(list(a[it:it + sp[1]]))
+                        it += sp[1]
+                return target(*full, **kwargs)
+
+            return fnp.call(packed, *flat)
         return fnp.call(lambda *a: target(*a, **kwargs), *args)
 
     return rule
@@ -370,6 +857,8 @@ def fold_constants(gm: torch.fx.GraphModule):
     return {n: _tree(v, _const) for n, v in env.items()}
 
 
+_WEIGHT_READERS = {aten.mm.default, aten.addmm.default, aten.bmm.default, aten.matmul.default, aten.mv.default,
+                   aten.native_layer_norm.default}
 _DEVICE_CONST_MIN = 256   # constants of at least this many floats live on the device between evaluations
 
 
@@ -379,6 +868,7 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
     env = dict(fold_constants(gm) if consts is None else consts)
     it = iter(inputs)
     look = lambda a: env[a] if isinstance(a, torch.fx.Node) else a
+    order = {n: i for i, n in enumerate(gm.graph.nodes)}
     for node in gm.graph.nodes:
         if node in env:
             continue
@@ -388,7 +878,20 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
             args = torch.fx.node.map_arg(node.args, look)
             kwargs = torch.fx.node.map_arg(node.kwargs, look)
             kwargs = {k: v for k, v in kwargs.items() if k not in ('dtype', 'device', 'layout', 'pin_memory', 'memory_format')}
-            rule = RULES.get(node.target) or _generic(node.target)
+            rule = RULES.get(node.target)
+            functional = _functional_form(node.target) if rule is None else None
+            if functional is not None:
+                # an in-place update of an intermediate (inside a library function: ``tmp.add_(eps)``): the functional
+                # operation, and the updated tensor is what its name means from here on.  Updates through views of the
+                # caller's own tensors never get here (the trace is functionalized); a view updated in place would
+                # leave its base behind, so that case raises.
+                target_node = node.args[0]
+                if not isinstance(target_node, torch.fx.Node) or target_node.op == 'placeholder' or \
+                        (target_node.target in _VIEWS and not _disjoint_part_of_a_dead_tensor(target_node, node, order)):
+                    raise NotImplementedError(f'{node.format_node()}: in-place update of an input or of a view')
+                env[node] = env[target_node] = RULES[functional](*args, **kwargs)
+                continue
+            rule = rule or _generic(node.target)
             if node.target is aten.amax.default and node.users and all(u.target is aten.detach.default for u in node.users):
                 rule = _amax_values   # max(...).detach(): the shift of a softmax / logsumexp carries no derivatives
             try:
@@ -423,7 +926,9 @@ class TracedForwardLaplacian(ForwardLaplacianFn):
                 examples = [torch.zeros(s, dtype=torch.float32) + 0.5 for s in shapes]
                 _TRACING[0] = True
                 try:
-                    gm = self.graphs[shapes] = make_fx(self.torch_fn)(*examples)
+                    # in-place updates and slice assignments of the function become their functional forms
+                    # (add_, copy_ into a view, index_put_ ... -> add, slice_scatter, index_put ...)
+                    gm = self.graphs[shapes] = make_fx(torch.func.functionalize(self.torch_fn))(*examples)
                 finally:
                     _TRACING[0] = False
             self.constants[shapes] = fold_constants(gm)
@@ -438,7 +943,10 @@ class TracedForwardLaplacian(ForwardLaplacianFn):
                         and device.type != 'cpu'):
                     return torch.as_tensor(np.ascontiguousarray(v)).to(device)
                 return v
-            hit = self.constants[key] = {n: _tree(v, place) for n, v in self.constants[shapes].items()}
+            # only what the product rules read (weights): they take device tensors as they are, and every other
+            # rule keeps seeing host arrays, whatever the size of its constants
+            hit = self.constants[key] = {n: (_tree(v, place) if n.users and all(u.target in _WEIGHT_READERS for u in n.users) else v)
+                                         for n, v in self.constants[shapes].items()}
         return hit
 
     def _run(self, *lapl_args):

@@ -643,6 +643,18 @@ def rows_affine(inp, rows, row_shape, out_shape, c=None, d=None, alpha=1.0, beta
                 c, d = c2, d2
                 break
     if col is None:
+        # the INPUT is broadcast along several separate groups of axes: spell the first group out in a pass of its own
+        # (a plain broadcast copy, three index dimensions), then come back with one group fewer
+        rs = (1,) * (len(out_shape) - len(row_shape)) + tuple(int(v) for v in row_shape)
+        grown = [i for i, (a_, o_) in enumerate(zip(rs, out_shape)) if a_ == 1 and o_ != 1]
+        if grown:
+            first = [grown[0]]
+            while first[-1] + 1 in grown:
+                first.append(first[-1] + 1)
+            mid = tuple(out_shape[i] if i in first else rs[i] for i in range(len(rs)))
+            if mid != rs and len(first) < len(grown):
+                step = rows_affine(inp, rows, rs, mid)
+                return rows_affine(step, rows, mid, out_shape, c, d, alpha, beta)
         raise NotImplementedError(
             f'rows_affine: the input of shape {tuple(row_shape)} broadcast to {tuple(out_shape)} needs more than '
             'three index dimensions; broadcast it with broadcast_to first')

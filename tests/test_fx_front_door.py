@@ -124,3 +124,43 @@ def test_traced_model_under_graph_replay():
         torch.cuda.synchronize()
         assert torch.equal(a.x, b.x) and torch.equal(a.laplacian, b.laplacian), f'call {call}'
         assert torch.equal(a.jacobian.dense_array, b.jacobian.dense_array), f'call {call}'
+
+
+def _check_construct(name, thr, device, caplog):
+    from torch_constructs import CONSTRUCTS, X
+
+    fn, _ = CONSTRUCTS[name](torch.float32)
+    _, fn_ad = CONSTRUCTS[name](torch.float64)
+    with caplog.at_level('WARNING'):
+        out = folx_amd.vmap(folx_amd.forward_laplacian_torch(fn, thr))(torch.as_tensor(X).to(device))
+    assert not [r for r in caplog.records if 'no forward-Laplacian rule' in r.message], 'fell back to the generic rule'
+    by, bJ, bL = brute_force(fn_ad, X.astype(np.float64))
+    J = out.jacobian.dense_array
+    if J.shape[0] < bJ.shape[0]:
+        assert not np.abs(bJ[J.shape[0]:]).any()
+        bJ = bJ[: J.shape[0]]
+    assert_val(out.x, by, f'{name} value')
+    assert_val(J, bJ.reshape(tuple(J.shape)), f'{name} jacobian')
+    assert_lap(out.laplacian, bL, f'{name} laplacian')
+
+
+def _construct_names():
+    from torch_constructs import CONSTRUCTS
+
+    return sorted(CONSTRUCTS)
+
+
+@pytest.mark.parametrize('name', _construct_names())
+@pytest.mark.parametrize('thr', [0, 6])
+def test_everyday_torch_constructs_have_rules(name, thr, monkeypatch, caplog):
+    """Functional calls, modules, linalg and indexing as they appear in ordinary torch code: every traced equation finds
+    a rule of its own (no generic fallback), results against AD in float64."""
+    cpu_kernels.install(monkeypatch)
+    _check_construct(name, thr, 'cpu', caplog)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('name', _construct_names())
+def test_everyday_torch_constructs_on_the_gpu(name, caplog):
+    print(f'torch construct {name}', flush=True)
+    _check_construct(name, 6, 'cuda', caplog)

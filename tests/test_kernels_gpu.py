@@ -504,6 +504,15 @@ def test_rows_affine():
     assert_val(got, inp4.astype(np.float64) + eye)
     got = K.rows_affine(dev(inp4[:, :, :, :1]), 2, (2, 5, 1, 5), shape4, dev(eye), None, alpha=2.0)
     assert_val(got, 2.0 * np.broadcast_to(inp4[:, :, :, :1], (2, *shape4)).astype(np.float64) * eye)
+    # the INPUT broadcast along two separate groups of axes (what an outer-product style multiply of (n, 1, d, 1) with
+    # (n, m, d, e) gives): more than three index dimensions, spelled out in two passes
+    shape5 = (2, 5, 4, 8, 8)
+    inp5 = rand(rng, 3, 2, 5, 1, 8, 1)
+    c5 = rand(rng, 1, 1, 4, 8, 8)
+    got = K.rows_affine(dev(inp5), 3, (2, 5, 1, 8, 1), shape5, dev(c5), None, alpha=1.5)
+    assert_val(got, 1.5 * np.broadcast_to(inp5, (3, *shape5)).astype(np.float64) * c5)
+    got = K.rows_affine(dev(inp5[:, :, :, :, :1]), 3, (2, 5, 1, 1, 1), shape5, None, dev(c5), alpha=1.0, beta=2.0)
+    assert_val(got, np.broadcast_to(inp5[:, :, :, :, :1], (3, *shape5)).astype(np.float64) + 2.0 * c5)
 
 
 @pytest.mark.parametrize('outer,red,inner', [(7, 5, 9), (6, 100, 1), (3, 4, 1), (1, 33, 70)])
