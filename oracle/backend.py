@@ -720,20 +720,32 @@ def clip(a: OArr, lo=None, hi=None):
 
 
 def where(cond, a, b):
+    """``numpy.where`` with numpy's broadcasting over the PER-SAMPLE shapes (operands of lower rank are aligned on the
+    right, behind the walker axis)."""
     c = np.asarray(cond.data if isinstance(cond, OConst) else cond).astype(bool)
+    per_walker_cond = isinstance(cond, OConst)
     like = a if _is(a) else b
-    c = np.broadcast_to(c if isinstance(cond, OConst) else c[None], like.x.shape)
+    B, dt = like.x.shape[0], like.x.dtype
+    shapes = [c.shape[1:] if per_walker_cond else c.shape] + [v.x.shape[1:] if _is(v) else np.shape(v) for v in (a, b)]
+    full = np.broadcast_shapes(*shapes)
+    nd = len(full)
+
+    def lift(t, lead):      # t has `lead` leading axes (rows, walkers) in front of its per-sample shape
+        t = t.reshape(*t.shape[:lead], *((1,) * (nd - (t.ndim - lead))), *t.shape[lead:])
+        return np.broadcast_to(t, (*t.shape[:lead], *full))
+
+    c = lift(c, 1) if per_walker_cond else np.broadcast_to(lift(c, 0)[None], (B, *full))
+    P = max([v.J.shape[0] for v in (a, b) if _is(v)])
 
     def trip(v):
         if _is(v):
-            return v.x, v.J, v.lap
-        cv = np.broadcast_to(np.asarray(v, dtype=like.x.dtype), like.x.shape)
-        return cv, np.zeros_like(like.J), np.zeros_like(like.lap)
+            J = np.concatenate([v.J, np.zeros((P - v.J.shape[0], *v.J.shape[1:]), v.J.dtype)], 0)
+            return lift(v.x, 1), lift(J, 2), lift(v.lap, 1)
+        cv = np.broadcast_to(lift(np.asarray(v, dtype=dt), 0)[None], (B, *full))
+        return cv, np.zeros((P, B, *full), dt), np.zeros((B, *full), dt)
 
     (ax, aJ, aL), (bx, bJ, bL) = trip(a), trip(b)
-    P = max(aJ.shape[0], bJ.shape[0])
-    ext = lambda J: np.concatenate([J, np.zeros((P - J.shape[0], *J.shape[1:]), J.dtype)], 0)
-    return OArr(np.where(c, ax, bx), np.where(c[None], ext(aJ), ext(bJ)), np.where(c, aL, bL))
+    return OArr(np.where(c, ax, bx), np.where(c[None], aJ, bJ), np.where(c, aL, bL))
 
 
 def cumsum(a: OArr, axis=-1):

@@ -345,3 +345,26 @@ def test_dot_two_rule_vs_autograd_and_mul_sum():
     want = tri(lambda t: u(t) @ v(t), (I, J))
     for g_, w_ in zip(got, want):
         np.testing.assert_allclose(g_, w_, rtol=1e-9, atol=1e-10)
+
+
+def test_where_broadcasts_operands_of_different_rank_like_numpy():
+    """The oracle backend's ``where`` with a condition of rank 5, one operand of rank 5 and one of rank 1 (aligned on the
+    right, behind the walker axis) against AD through ``torch.where``."""
+    from bruteforce import brute_force, plain
+    from oracle import backend as ob
+
+    cond = np.array([True, False]).reshape(2, 1, 1, 1, 1)
+
+    def f(xp, x):
+        a = xp.add(xp.tanh(xp.reshape(xp.getitem(x, slice(0, 2)), (2, 1, 1, 1, 1))), 2.0)
+        r = xp.add(xp.reshape(xp.cos(xp.getitem(x, slice(2, 5))), (3,)), 2.0)
+        return xp.where(cond, a, r), xp.where(cond, 0.5, r), xp.where(cond[:, 0], a, np.float64(1.5))
+
+    x = np.random.default_rng(0).normal(size=(2, 5))
+    got = f(ob, ob.init_state(x, dtype=np.float64))
+    for i, g in enumerate(got):
+        y, J, L = brute_force(lambda t, i=i: f(plain, t)[i], x)
+        assert g.x.shape == y.shape
+        np.testing.assert_allclose(g.x, y, rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(g.J, J.reshape(g.J.shape), rtol=1e-12, atol=1e-13)
+        np.testing.assert_allclose(g.lap, L, rtol=1e-12, atol=1e-13)
