@@ -731,7 +731,7 @@ def where(cond, a, b):
     nd = len(full)
 
     def lift(t, lead):      # t has `lead` leading axes (rows, walkers) in front of its per-sample shape
-        t = t.reshape(*t.shape[:lead], *((1,) * (nd - (t.ndim - lead))), *t.shape[lead:])
+        t = t.reshape((*t.shape[:lead], *((1,) * (nd - (t.ndim - lead))), *t.shape[lead:]))
         return np.broadcast_to(t, (*t.shape[:lead], *full))
 
     c = lift(c, 1) if per_walker_cond else np.broadcast_to(lift(c, 0)[None], (B, *full))
