@@ -69,6 +69,23 @@ def test_argument_checks_return_error_codes(lib):
     assert lib.folx_hip_mul_sparse_fwdlap(*([null] * 11), 9, 4, 2, 1) == _lib.EINVAL       # S not a multiple of S_w
     assert lib.folx_hip_exp_envelope_fwdlap(*([null] * 9), 4, 2, 8, 1) == _lib.EINVAL
     assert lib.folx_hip_slogdet_scaled_fwdlap(*([null] * 12), 1, 1, 4, 1, 16, 0, 4, 16, 16, 1) == _lib.EINVAL
+    assert lib.folx_hip_dense_rows_fwdlap(*([null] * 12), 4, 1, 8, 8, 1, 1) == _lib.EINVAL
+    assert lib.folx_hip_dot_two_fwdlap(*([null] * 10), 1, 1, 4, 4, 4, 1, null) == _lib.EINVAL
+    assert lib.folx_hip_reduce_max(null, null, null, 2, 3, 4) == _lib.EINVAL
+    assert lib.folx_hip_reduce_max(null, null, null, -2, 3, 4) == _lib.EINVAL
+    assert lib.folx_hip_gather_reduce_rows(null, null, null, null, 2, 2, 1, 1, 4, 4, 1, 1, 1.0) == _lib.EINVAL
+    assert lib.folx_hip_gather_cols(null, null, null, null, 2, 4, 4, 1, 1) == _lib.EINVAL
+    assert lib.folx_hip_gather_cols(null, null, null, null, -2, 4, 4, 1, 1) == _lib.EINVAL
+    assert lib.folx_hip_scatter_add_rows(null, null, null, null, 2, 4, 1, 4, 1) == _lib.EINVAL
+    assert lib.folx_hip_slogdet_strided_fwdlap(*([null] * 8), 1, 1, 4, 1, 16, 16, 4, 16) == _lib.EINVAL
+    assert lib.folx_hip_sparse_slogdet_fwdlap(*([null] * 11), 1, 4, 1, 1, 1, 1, 0) == _lib.EINVAL
+    assert lib.folx_hip_inv_values(null, null, null, null, null, 1, 4) == _lib.EINVAL
+    assert lib.folx_hip_trace_pair(null, null, null, null, 1, 4) == _lib.EINVAL
+    assert lib.folx_hip_trace_pair(null, null, null, null, -1, 4) == _lib.EINVAL
+    assert lib.folx_hip_inv_fwdlap(*([null] * 7), 1, 4, 1) == _lib.EINVAL
+    assert lib.folx_hip_inv_fwdlap(*([null] * 7), -1, 4, 1) == _lib.EINVAL
+    assert lib.folx_hip_solve_fwdlap(*([null] * 10), 1, 4, 1, 1) == _lib.EINVAL
+    assert lib.folx_hip_solve_fwdlap(*([null] * 10), 1, 0, 1, 1) == _lib.EINVAL
     # empty problems are fine and launch nothing
     assert lib.folx_hip_dense_fwdlap(*([null] * 12), 0, 1, 8, 8) == _lib.OK
     assert lib.folx_hip_elementwise_fwdlap(null, 0, 0.0, null, null, null, null, null, null, 0, 1) == _lib.OK
