@@ -173,6 +173,12 @@ DENSE_ACT_CASES = [
     ((5, 40), 64, 16, 128, True, 'cos'),
     ((2, 64), 31, 104, 100, False, 'square'),   # odd number of Jacobian rows
     ((1, 64), 100, 100, 100, True, 'tanh'),     # one row tile, many groups
+    # a short tail of columns behind full strips (the last strip is mostly padding), 16+ Jacobian rows
+    ((1, 70), 40, 100, 98, True, 'silu'),       # tail of 2 columns, last tile of 6 rows
+    ((3, 50), 17, 68, 33, True, 'tanh'),        # one strip + 1 column, K = 68
+    ((1, 200), 16, 96, 68, False, 'softplus'),  # two strips + 4 columns
+    ((1, 5), 20, 100, 97, True, 'exp'),         # fewer rows than a tile
+    ((2, 48), 24, 100, 100, True, 'sin'),
     # wide layers (N > 128): tiles of 4 positions x 32 Jacobian rows, activation in the GEMM's epilogue
     ((2, 32), 96, 256, 256, True, 'tanh'),      # transformer MLP: three full groups of 32 Jacobian rows
     ((3, 16), 48, 832, 256, True, 'tanh'),      # one-electron stream: three groups of 16 Jacobian rows
