@@ -1041,3 +1041,54 @@ register_function('convert_element_type', _composed(lambda a, new_dtype=np.float
 register_function('dynamic_slice', _composed(lambda a, *start, slice_sizes: dynamic_slice(a, start, slice_sizes),
                                              'slice_sizes'))          # :468
 register_function('dynamic_update_slice', _composed(lambda a, u, *start: dynamic_update_slice(a, u, start)))  # :488
+
+
+# constants, dtypes and tests on plain arrays are numpy's own (``jnp.zeros``, ``jnp.eye``, ``jnp.float32`` ...)
+zeros, ones, eye, full, arange, linspace, array, asarray = (np.zeros, np.ones, np.eye, np.full, np.arange, np.linspace,
+                                                            np.array, np.asarray)
+float16, float32, float64, int8, int16, int32, int64, uint8, uint16, uint32, uint64, bool_ = (
+    np.float16, np.float32, np.float64, np.int8, np.int16, np.int32, np.int64, np.uint8, np.uint16, np.uint32, np.uint64,
+    np.bool_)
+rem = remainder                                      # jax.lax.rem
+
+
+def full_like(a, fill_value, dtype=None):
+    return np.full(_shape(a), fill_value, dtype=dtype or np.float32)
+
+
+def convert_element_type(a, new_dtype):              # jax.lax.convert_element_type
+    return astype(a, new_dtype)
+
+
+def allclose(a, b, rtol=1e-5, atol=1e-8):
+    """``numpy.allclose`` on values (triplets contribute their ``x``)."""
+    from .wrapped_functions import force
+
+    val = lambda v: force(v).x.detach().cpu().numpy() if _is_triplet(v) else (  # noqa: E731
+        v.data.detach().cpu().numpy() if isinstance(v, BatchedArray) else np.asarray(v))
+    return bool(np.allclose(val(a), val(b), rtol=rtol, atol=atol))
+
+
+def _reduce_named(fold):
+    def fn(a, axis=None, keepdims=False):
+        shape = _shape(a)
+        axes = sorted(_axes(axis, len(shape)), reverse=True)
+        out = a
+        for ax in axes:
+            out = fold(out, axis=ax)
+        if keepdims:
+            out = reshape(out, tuple(1 if i in axes else n for i, n in enumerate(shape)))
+        return out
+
+    return fn
+
+
+_LATE = {'max': _reduce_named(amax), 'min': _reduce_named(amin)}
+
+
+def __getattr__(name):
+    # ``fnp.max`` / ``fnp.min`` (``jnp.max``: all axes by default) without shadowing the builtins this module uses
+    try:
+        return _LATE[name]
+    except KeyError:
+        raise AttributeError(f'module {__name__!r} has no attribute {name!r}') from None

@@ -1102,3 +1102,25 @@ def test_python_operators_on_triplets(monkeypatch):
         np.testing.assert_allclose(out.laplacian.numpy(), L, rtol=1e-4, atol=1e-4)
     with pytest.raises(TypeError):
         np.add(c, folx_amd.vmap(folx_amd.forward_laplacian(lambda z: z, 0))(x))   # numpy functions do not take triplets
+
+
+def test_numpy_style_constants_and_full_reductions(monkeypatch):
+    """The names the reference's tests take from jnp / lax around a model: constants and dtypes (numpy's own),
+    ``max`` / ``min`` over all or some axes (module attributes that do not shadow the builtins), ``rem``,
+    ``convert_element_type``, ``allclose``."""
+    cpu_kernels.install(monkeypatch)
+    x = np.random.default_rng(0).normal(size=(2, 3, 4)).astype(np.float32)
+
+    def f(xp, t):
+        return xp.add(xp.add(xp.max(xp.sin(t)), xp.sum(xp.min(t, axis=-1, keepdims=True))),
+                      xp.sum(xp.multiply(xp.remainder(t, 0.7), np.eye(3, 4, dtype=np.float32))))
+
+    check_against_oracle(lambda xp, t: f(xp if xp is not fnp else fnp, t) if xp is fnp else
+                         xp.add(xp.add(xp.amax(xp.amax(xp.sin(t), axis=-1), axis=-1), xp.sum(xp.amin(t, axis=-1))),
+                                xp.sum(xp.multiply(xp.remainder(t, 0.7), np.eye(3, 4, dtype=np.float32)))), x, 0)
+    assert fnp.rem is fnp.remainder and fnp.zeros((2, 3)).shape == (2, 3) and fnp.eye(3).dtype == np.float64
+    assert fnp.float32 is np.float32 and fnp.full_like(np.zeros((2, 2)), 3.0).tolist() == [[3.0, 3.0], [3.0, 3.0]]
+    out = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: fnp.convert_element_type(fnp.tanh(t), fnp.float64), 0))(x)
+    assert fnp.allclose(out, np.tanh(x), atol=1e-6) and not fnp.allclose(out, np.tanh(x) + 1e-3)
+    with pytest.raises(AttributeError):
+        fnp.no_such_function
