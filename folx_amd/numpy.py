@@ -1092,3 +1092,52 @@ def __getattr__(name):
         return _LATE[name]
     except KeyError:
         raise AttributeError(f'module {__name__!r} has no attribute {name!r}') from None
+
+
+def fori_loop(lower, upper, body_fun, init_val):
+    """``jax.lax.fori_loop`` with bounds known when the model is written: the loop simply runs (define-by-run), each
+    iteration through the ordinary rules."""
+    val = init_val
+    for i in range(int(lower), int(upper)):
+        val = body_fun(i, val)
+    return val
+
+
+def scan(f, init, xs=None, length=None, reverse=False):
+    """``jax.lax.scan(f, init, xs)``: ``carry, y = f(carry, x)`` over the leading axis of ``xs`` -- constants, as in the
+    reference (folx/interpreter.py:133-184 asserts that the scanned-over inputs carry no derivatives), or triplets
+    (sliced through the indexing rule).  ``xs`` may be a tuple / list / dict of arrays or None (then ``length``
+    iterations with ``x = None``).  The ``y`` of the iterations are stacked along a new leading axis; ``None`` stays None."""
+    def lead(v):
+        if isinstance(v, (tuple, list)):
+            return lead(v[0])
+        if isinstance(v, dict):
+            return lead(next(iter(v.values())))
+        return _shape(v)[0]
+
+    def item(v, i):
+        if isinstance(v, (tuple, list)):
+            return type(v)(item(t, i) for t in v)
+        if isinstance(v, dict):
+            return {k: item(t, i) for k, t in v.items()}
+        return getitem(v, i) if _is_triplet(v) or isinstance(v, BatchedArray) else np.asarray(v)[i]
+
+    n = int(length) if xs is None else lead(xs)
+    order = range(n - 1, -1, -1) if reverse else range(n)
+    carry, ys = init, [None] * n
+    for i in order:
+        carry, ys[i] = f(carry, None if xs is None else item(xs, i))
+
+    def pile(parts):
+        first = parts[0]
+        if first is None:
+            return None
+        if isinstance(first, (tuple, list)):
+            return type(first)(pile([p[k] for p in parts]) for k in range(len(first)))
+        if isinstance(first, dict):
+            return {k: pile([p[k] for p in parts]) for k in first}
+        if any(_is_triplet(p) or isinstance(p, BatchedArray) for p in parts):
+            return stack(parts, axis=0)
+        return np.stack([np.asarray(p) for p in parts], axis=0)
+
+    return carry, (pile(ys) if n > 0 else None)

@@ -1124,3 +1124,44 @@ def test_numpy_style_constants_and_full_reductions(monkeypatch):
     assert fnp.allclose(out, np.tanh(x), atol=1e-6) and not fnp.allclose(out, np.tanh(x) + 1e-3)
     with pytest.raises(AttributeError):
         fnp.no_such_function
+
+
+def test_scan_and_fori_loop_run_as_python_loops(monkeypatch):
+    """``jax.lax.scan`` over constants (what the reference supports, folx/interpreter.py:133-184) and over a triplet, and
+    ``fori_loop``: a small recurrent cell against the oracle running the same loop."""
+    cpu_kernels.install(monkeypatch)
+    rng = np.random.default_rng(6)
+    W, U = rng.normal(size=(5, 5)).astype(np.float32) / 2, rng.normal(size=(3, 5)).astype(np.float32) / 2
+    drive = rng.normal(size=(4, 3)).astype(np.float32)            # scanned-over constants
+    V = rng.normal(size=(4, 5)).astype(np.float32)
+    x = rng.normal(size=(2, 4, 5)).astype(np.float32)              # per walker: 4 time steps of 5 features (scanned triplet)
+
+    def model(xp, t, scan, fori):
+        cell = lambda h, u: (lambda hn: (hn, xp.sum(xp.square(hn))))(xp.tanh(xp.add(xp.dot(h, W), np.asarray(u) @ U)))
+        h, ys = scan(cell, xp.getitem(t, 0), drive)                                        # constants scanned
+        h2, ys2 = scan(lambda c, row: (xp.add(xp.multiply(c, 0.5), xp.sin(row)), None), h, t, reverse=True)   # a triplet scanned
+        h3 = fori(1, 4, lambda i, c: xp.add(c, xp.multiply(xp.tanh(c), V[i])), h2)
+        return xp.add(xp.sum(h3), xp.sum(ys)), ys2
+
+    def with_loops(xp, t):
+        if xp is fnp:
+            return model(fnp, t, fnp.scan, fnp.fori_loop)[0]
+
+        def py_scan(f, init, xs, reverse=False):
+            n = xs.shape[0]
+            carry, ys = init, [None] * n
+            for i in (range(n - 1, -1, -1) if reverse else range(n)):
+                carry, ys[i] = f(carry, xs[i] if isinstance(xs, np.ndarray) else xp.getitem(xs, i))
+            return carry, (None if ys[0] is None else xp.stack(ys, axis=0))
+
+        def py_fori(lo, hi, body, init):
+            for i in range(lo, hi):
+                init = body(i, init)
+            return init
+
+        return model(xp, t, py_scan, py_fori)[0]
+
+    for thr in (0, 5, 20):
+        check_against_oracle(with_loops, x, thr)
+    out, ys2 = folx_amd.vmap(folx_amd.forward_laplacian(lambda t: model(fnp, t, fnp.scan, fnp.fori_loop), 0))(x)
+    assert ys2 is None and tuple(out.shape) == ()
