@@ -906,6 +906,53 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
     raise RuntimeError('graph without an output')
 
 
+_NAMED = {}
+
+
+def named_function(name: str, fn):
+    """A torch function that the trace keeps as ONE equation, evaluated by the rule registered under ``name`` -- the
+    reference looks jitted functions up by name the same way (``eval_pjit``, folx/interpreter.py:186-200:
+    ``register_function('my_layer', rule)`` + ``jax.jit(my_layer)``).  Returns the function to call in the model: while
+    ``forward_laplacian_torch`` traces, the call is a library operation ``folx_amd::<name>`` over its tensor arguments;
+    otherwise it is ``fn`` itself.  Without a rule under ``name`` at evaluation time the function gets the generic
+    rule (``wrap_forward_laplacian(fn)``).  ``fn`` takes tensors and returns a tensor or a tuple of tensors."""
+    assert name.isidentifier(), 'the name becomes an operator name'
+    if name in _NAMED:
+        assert _NAMED[name][0] is fn, f'{name} already names another function'
+        return _NAMED[name][1]
+
+    single = [True]
+
+    def impl(inputs):
+        out = fn(*inputs)
+        single[0] = not isinstance(out, (tuple, list))     # known once the operation has run (it runs while tracing)
+        return [out] if single[0] else list(out)
+
+    _LIB.define(f'{name}(Tensor[] inputs) -> Tensor[]')
+    _LIB.impl(name, impl, 'CompositeExplicitAutograd')
+    op = getattr(torch.ops.folx_amd, name).default
+
+    def rule(inputs):
+        from .wrapped_functions import get_laplacian, is_registered
+        from .wrapper import wrap_forward_laplacian
+
+        r = get_laplacian(name) if is_registered(name) else wrap_forward_laplacian(fn, name=name)
+        out = r(tuple(inputs), {}, fnp.current_threshold())
+        return list(out) if isinstance(out, (tuple, list)) else [out]
+
+    RULES[op] = rule
+
+    def call(*tensors):
+        if not _TRACING[0]:
+            return fn(*tensors)
+        out = op(list(tensors))
+        return out[0] if single[0] else tuple(out)
+
+    call.__name__ = name
+    _NAMED[name] = (fn, call)
+    return call
+
+
 class TracedForwardLaplacian(ForwardLaplacianFn):
     """``forward_laplacian_torch(fn, thr)``: ``f(x)`` takes one sample, ``f.batched(x)`` walkers, as for
     ``forward_laplacian``; the torch function is traced once per combination of input shapes, its constant

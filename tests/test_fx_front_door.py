@@ -164,3 +164,62 @@ def test_everyday_torch_constructs_have_rules(name, thr, monkeypatch, caplog):
 def test_everyday_torch_constructs_on_the_gpu(name, caplog):
     print(f'torch construct {name}', flush=True)
     _check_construct(name, 6, 'cuda', caplog)
+
+
+def _named_function_model():
+    from folx_amd import fx
+
+    torch.manual_seed(3)
+    W = torch.randn(4, 6) / 2
+    layer = fx.named_function('test_gated_layer', lambda h, g: torch.tanh(h @ W.to(h.dtype)) * torch.sigmoid(g).sum())
+    pair = fx.named_function('test_sin_cos_pair', lambda h: (torch.sin(h), torch.cos(h).sum(-1)))
+
+    def model(x):
+        s, c = pair(layer(x, x[:, 0]))
+        return (s * c[:, None]).sum(0)
+
+    return model, W
+
+
+def _check_named_functions(device):
+    """A function kept as one equation of the trace and looked up by NAME when the graph is evaluated
+    (folx/interpreter.py:186-200): the generic rule without a registry entry, the registered rule with one."""
+    from folx_amd import numpy as fnp
+
+    model, W = _named_function_model()
+    x = np.random.default_rng(0).normal(size=(2, 3, 4)).astype(np.float32)
+    by, bJ, bL = brute_force(model, x.astype(np.float64))          # outside a trace the names are the plain functions
+    fl = folx_amd.forward_laplacian_torch(model, 0)
+    out = folx_amd.vmap(fl)(torch.as_tensor(x).to(device))
+    (gm,) = fl.graphs.values()
+    targets = [str(n.target) for n in gm.graph.nodes if n.op == 'call_function']
+    assert 'folx_amd.test_gated_layer.default' in targets and 'folx_amd.test_sin_cos_pair.default' in targets
+    assert not any('tanh' in t or 'sigmoid' in t for t in targets)          # the bodies are not in the trace
+    assert_val(out.x, by, 'value')
+    assert_val(out.jacobian.dense_array, bJ.reshape(tuple(out.jacobian.dense_array.shape)), 'jacobian')
+    assert_lap(out.laplacian, bL, 'laplacian')
+    seen = []
+
+    def rule(args, kwargs, thr):            # a rule of the caller's own under the same name
+        seen.append(len(args))
+        h, g = args
+        return fnp.multiply(fnp.tanh(fnp.dot(h, W.numpy())), fnp.sum(fnp.sigmoid(g)))
+
+    folx_amd.register_function('test_gated_layer', rule)
+    try:
+        out2 = folx_amd.vmap(fl)(torch.as_tensor(x).to(device))
+    finally:
+        folx_amd.deregister_function('test_gated_layer')
+    assert seen == [2]
+    assert_val(out2.x, by, 'value by the registered rule')
+    assert_lap(out2.laplacian, bL, 'laplacian by the registered rule')
+
+
+def test_named_functions_are_single_equations_looked_up_by_name(monkeypatch):
+    cpu_kernels.install(monkeypatch)
+    _check_named_functions('cpu')
+
+
+@pytest.mark.gpu
+def test_named_functions_on_the_gpu():
+    _check_named_functions('cuda')
