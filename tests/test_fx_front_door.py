@@ -171,7 +171,7 @@ def _named_function_model():
 
     torch.manual_seed(3)
     W = torch.randn(4, 6) / 2
-    layer = fx.named_function('test_gated_layer', lambda h, g: torch.tanh(h @ W.to(h.dtype)) * torch.sigmoid(g).sum())
+    layer = fx.named_function('test_gated_layer', lambda h, g: torch.tanh(h @ W.to(h)) * torch.sigmoid(g).sum())   # (the generic rule runs it where the data is)
     pair = fx.named_function('test_sin_cos_pair', lambda h: (torch.sin(h), torch.cos(h).sum(-1)))
 
     def model(x):
