@@ -889,6 +889,10 @@ def evaluate_graph(gm: torch.fx.GraphModule, inputs, consts=None):
                 if not isinstance(target_node, torch.fx.Node) or target_node.op == 'placeholder' or \
                         (target_node.target in _VIEWS and not _disjoint_part_of_a_dead_tensor(target_node, node, order)):
                     raise NotImplementedError(f'{node.format_node()}: in-place update of an input or of a view')
+                for view in target_node.users:   # a view taken BEFORE the update and read AFTER it would miss the update
+                    if view.target in _VIEWS and order[view] < order[node] and any(order[w] > order[node] for w in view.users):
+                        raise NotImplementedError(f'{node.format_node()}: in-place update of a tensor whose earlier '
+                                                  f'view {view.name} is read afterwards')
                 env[node] = env[target_node] = RULES[functional](*args, **kwargs)
                 continue
             rule = rule or _generic(node.target)
